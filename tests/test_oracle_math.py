@@ -1,0 +1,244 @@
+"""What the mathematics fixes about the oracle, independent of any fixture:
+library routines, closed forms, brute force on small inputs, invariants.
+Mirrors the known-answer checks of the reference's tests/test_rotation.py,
+test_codebook.py, test_qjl.py and test_utils.py."""
+import numpy as np
+import pytest
+import scipy.linalg
+
+import tq_oracle as O
+
+
+@pytest.mark.parametrize("n", [1, 2, 8, 64, 128])
+def test_fwht_is_scipy_hadamard(n):
+    x = np.random.default_rng(n).standard_normal((5, n))
+    ref = x @ (scipy.linalg.hadamard(n) / np.sqrt(n)).T
+    np.testing.assert_allclose(O.fwht(x), ref, atol=1e-12)
+    np.testing.assert_allclose(O.fwht(O.fwht(x)), x, atol=1e-12)
+
+
+def test_fwht_rejects_non_pow2():
+    with pytest.raises(ValueError, match="power of 2"):
+        O.fwht(np.zeros(12))
+
+
+def test_sylvester_matches_scipy():
+    for n in (1, 2, 4, 16, 128):
+        assert np.array_equal(O.sylvester_hadamard(n), scipy.linalg.hadamard(n))
+    with pytest.raises(ValueError):
+        O.sylvester_hadamard(6)
+
+
+def test_fast_rotation_is_explicit_matrix():
+    rng = np.random.default_rng(5)
+    s1, s2, pd = O.sign_diagonals(128, rng)
+    R = np.diag(s2) @ (scipy.linalg.hadamard(128) / np.sqrt(128)) @ np.diag(s1)
+    x = rng.standard_normal((7, 128))
+    np.testing.assert_allclose(O.rotate_fast(x, s1, s2, pd), x @ R.T, atol=1e-12)
+    np.testing.assert_allclose(O.rotate_fast(x, s1, s2, pd, transpose=True), x @ R, atol=1e-12)
+    # padded, truncated case: d = 100 inside 128
+    x = rng.standard_normal((3, 100))
+    full = np.zeros((3, 128)); full[:, :100] = x
+    np.testing.assert_allclose(O.rotate_fast(x, s1, s2, pd), (full @ R.T)[:, :100], atol=1e-12)
+
+
+@pytest.mark.parametrize("d", [1, 8, 64, 128])
+def test_haar_is_rotation(d):
+    q = O.haar_rotation(d, np.random.default_rng(d))
+    np.testing.assert_allclose(q @ q.T, np.eye(d), atol=1e-10)
+    assert np.linalg.slogdet(q)[0] > 0
+    with pytest.raises(ValueError):
+        O.haar_rotation(0, np.random.default_rng(0))
+
+
+def test_centroid_closed_forms():
+    for d in (64, 128, 256):
+        np.testing.assert_allclose(O.centroids_for(1, d), [-np.sqrt(2 / (np.pi * d)), np.sqrt(2 / (np.pi * d))], atol=1e-15)
+        np.testing.assert_allclose(O.centroids_for(2, d), np.array([-1.51, -0.453, 0.453, 1.51]) / np.sqrt(d), atol=1e-15)
+    # textbook Max (1960) 8-level unit-Gaussian quantiser
+    max8 = np.array([0.2451, 0.7560, 1.3439, 2.1520])
+    c = O.centroids_for(3, 128) * np.sqrt(128)
+    np.testing.assert_allclose(c[4:], max8, atol=2e-4)
+    np.testing.assert_allclose(c, -c[::-1], atol=1e-12)
+
+
+def test_cond_mean_closed_forms():
+    assert abs(O.gauss_cond_mean(1.0, 0.0, np.inf) - np.sqrt(2 / np.pi)) < 1e-12
+    assert abs(O.gauss_cond_mean(1.0, -1.0, 1.0)) < 1e-12
+    assert O.gauss_cond_mean(1.0, 40.0, np.inf) == 41.0
+    assert O.gauss_cond_mean(1.0, -np.inf, -40.0) == -41.0
+    assert O.gauss_cond_mean(1.0, 40.0, 41.0) == 40.5
+    # numeric integration of x*pdf over [a,b] / mass
+    xs = np.linspace(-0.3, 0.7, 200001)
+    pdf = np.exp(-xs ** 2 / (2 * 0.25)) / np.sqrt(2 * np.pi * 0.25)
+    num = np.trapezoid(xs * pdf, xs) / np.trapezoid(pdf, xs)
+    assert abs(O.gauss_cond_mean(0.5, -0.3, 0.7) - num) < 1e-9
+
+
+@pytest.mark.parametrize("b", [1, 2, 3, 4])
+def test_nearest_index_is_argmin(b):
+    c = O.centroids_for(b, 128)
+    v = np.random.default_rng(b).standard_normal(500) / np.sqrt(128)
+    brute = np.argmin(np.abs(v[:, None] - c[None, :]), axis=1)
+    assert np.array_equal(O.nearest_index(v, c), brute)
+    # tie rule: exactly on a midpoint -> lower index; far outside -> clamped
+    mid = O.midpoints(c)
+    assert np.array_equal(O.nearest_index(mid, c), np.arange(len(mid)))
+    assert O.nearest_index(np.array([-9.0, 9.0]), c).tolist() == [0, len(c) - 1]
+
+
+def test_qjl_orthogonal_and_unbiased():
+    for d in (64, 128):
+        q = O.QJLRef(d, seed=123)
+        assert np.linalg.norm(q.S @ q.S.T - np.eye(d), "fro") < 1e-12
+    q = O.QJLRef(128, seed=5)
+    rng = np.random.default_rng(0)
+    x, y = rng.standard_normal(128), rng.standard_normal(128)
+    # E||x_hat||^2 = (pi/2)||x||^2 holds exactly for orthogonal S and +-1 signs
+    z, n = q.quantize(x)
+    assert abs(np.linalg.norm(q.dequantize(z, n)) ** 2 - (np.pi / 2) * n ** 2) < 1e-9
+    # unbiasedness over many projection seeds
+    est = []
+    for s in range(300):
+        qq = O.QJLRef(128, seed=s)
+        z, n = qq.quantize(x)
+        est.append(qq.dequantize(z, n) @ y)
+    se = np.std(est) / np.sqrt(len(est))
+    assert abs(np.mean(est) - x @ y) < 4 * se
+    z, n = q.quantize(np.zeros(128))
+    assert n == 0 and set(np.unique(z)) == {1}
+
+
+def test_pack_literals():
+    # reference tests/test_utils.py literals: 8 signs -> one byte, MSB first
+    assert O.pack_sign_bits(np.array([1, -1, 1, 1, -1, -1, 1, -1], dtype=np.int8)).tolist() == [0b10110010]
+    assert O.pack_sign_bits(np.ones(128, dtype=np.int8)).shape == (16,)
+    assert O.pack_index_stream(np.array([3, 0, 1, 2]), 2).tolist() == [0b11000110]
+    assert O.pack_index_stream(np.array([5, 2]), 3).tolist() == [0b10101000]
+    with pytest.raises(ValueError, match="bit_width must be 1-8"):
+        O.pack_index_stream(np.array([0]), 9)
+    assert O.TurboRef(128, 3).compressed_size_bits(100) == 100 * (128 * 3 + 32)
+
+
+def test_polar_invariants():
+    pq = O.PolarRef(128, 3, seed=1)
+    x = np.random.default_rng(2).standard_normal((16, 128))
+    idx, n = pq.quantize(x)
+    assert idx.min() >= 0 and idx.max() < 8
+    np.testing.assert_allclose(pq.dequantize(*pq.quantize(3.0 * x)), 3.0 * pq.dequantize(idx, n), rtol=1e-12)
+    assert np.all(pq.dequantize(*pq.quantize(np.zeros((2, 128)))) == 0)
+    xu = x / np.linalg.norm(x, axis=1, keepdims=True)
+    mse = np.mean(np.sum((pq.dequantize(*pq.quantize(xu)) - xu) ** 2, axis=1))
+    assert mse < 2 * 0.03
+    # wht mode: same contract, different rotation
+    pw = O.PolarRef(128, 3, seed=1, rotation="wht")
+    mse = np.mean(np.sum((pw.dequantize(*pw.quantize(xu)) - xu) ** 2, axis=1))
+    assert mse < 2 * 0.03
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_device_layout_roundtrip_and_placement(bits, kind):
+    rng = np.random.default_rng(bits)
+    T = 256
+    idx = rng.integers(0, 1 << bits, size=(T, 128)).astype(np.uint8)
+    g = rng.standard_normal(T).astype(np.float16)
+    buf = O.layout_pack(idx, g, bits, kind)
+    assert buf.dtype == np.uint8 and buf.size == 2 * O.block_bytes(bits) == T * (16 * bits + 2)
+    i2, g2 = O.layout_unpack(buf, bits, kind)
+    assert np.array_equal(i2, idx) and np.array_equal(g2.view(np.uint16), g.view(np.uint16))
+    # one-hot placement: a single non-zero code lands where the layout says
+    one = np.zeros((128, 128), dtype=np.uint8)
+    tok, dim = 77, 45
+    one[tok, dim] = (1 << bits) - 1
+    b = O.layout_pack(one, np.zeros(128, dtype=np.float16), bits, kind)
+    words = b[:128 * 16 * bits].view("<u4").reshape(bits, 128, 4)
+    if kind == "k":
+        row, pair, half = tok, dim // 2, dim % 2
+    else:
+        row, pair, half = 4 * (tok // 4) + dim % 4, 2 * (dim // 4) + (tok % 4) // 2, tok % 2
+    value = ((1 << bits) - 1) << (bits * half)
+    rowwords = words[:, row, :].reshape(-1)
+    expect = np.zeros(4 * bits, dtype=np.uint64)
+    if bits == 4:
+        expect[pair // 4] = value << (8 * (pair % 4))
+    elif bits == 2:
+        expect[pair // 8] = value << (4 * (pair % 8))
+    elif pair < 60:
+        expect[pair // 5] = value << (6 * (pair % 5))
+    else:
+        for part in range(3):
+            expect[3 * (pair - 60) + part] = ((value >> (2 * part)) & 3) << 30
+    assert np.array_equal(rowwords.astype(np.uint64), expect)
+    assert np.count_nonzero(words) == np.count_nonzero(expect)
+
+
+def test_turbo_encode_consistency():
+    rng = np.random.default_rng(3)
+    s1, s2, _ = O.sign_diagonals(128, rng)
+    cent = O.centroids_for(4, 128)
+    x = rng.standard_normal((64, 128))
+    x[3] = 0
+    idx, g, y = O.turbo_encode(x, s1, s2, cent)
+    assert g.dtype == np.float16 and g[3] == 0
+    # corrected norm: reconstruction has the original norm up to fp16 rounding
+    rec = O.turbo_decode(idx, g, cent, s1, s2)
+    np.testing.assert_allclose(np.linalg.norm(rec, axis=1), np.linalg.norm(x, axis=1), rtol=1e-3)
+    assert np.all(rec[3] == 0)
+    # same indices as the class in wht mode built from the same signs
+    n_bad, n_inadm = O.boundary_band_mismatches(y, idx, cent)
+    assert (n_bad, n_inadm) == (0, 0)
+    bad = idx.copy(); bad[0, 0] ^= 1
+    assert O.boundary_band_mismatches(y, bad, cent)[1] == 1
+
+
+def test_q8_0_textbook():
+    x = np.random.default_rng(4).standard_normal((5, 128)).astype(np.float32)
+    x[0, :32] = 0
+    q, s = O.q8_0_quantize(x)
+    assert q.dtype == np.int8 and s.shape == (5, 4) and s.dtype == np.float16
+    assert np.all(q[0, :32] == 0) and s[0, 0] == 0
+    assert np.abs(q).max() == 127
+    err = np.abs(O.q8_0_dequantize(q, s) - x)
+    assert err.max() <= np.abs(x).reshape(5, 4, 32).max(-1).max() / 127 * 0.51 + 1e-3
+
+
+def test_decode_attention_closed_forms():
+    rng = np.random.default_rng(6)
+    q = rng.standard_normal((4, 128))
+    v = rng.standard_normal((256, 128))
+    # identical keys -> uniform weights -> mean of V
+    k = np.tile(rng.standard_normal((1, 128)), (256, 1))
+    out, _, _ = O.decode_attention(q, k, v, 0.1)
+    np.testing.assert_allclose(out, np.tile(v.mean(0), (4, 1)), atol=1e-12)
+    # one dominant key -> its V row
+    k = rng.standard_normal((256, 128)) * 1e-3
+    k[17] = 50 * q[0]
+    out, _, _ = O.decode_attention(q[:1], k, v, 1.0)
+    np.testing.assert_allclose(out[0], v[17], atol=1e-9)
+    # brute force softmax, and tau = 0 == dense, tau > 0 with splits close to dense
+    k = rng.standard_normal((256, 128))
+    s = 0.2 * q @ k.T
+    p = np.exp(s - s.max(1, keepdims=True)); p /= p.sum(1, keepdims=True)
+    dense, _, _ = O.decode_attention(q, k, v, 0.2)
+    np.testing.assert_allclose(dense, p @ v, atol=1e-12)
+    sp, skip, frac = O.decode_attention(q, k, v, 0.2, n_splits=4, sparse_v_tau=1e-6)
+    assert 0 <= skip <= 1 and np.abs(sp - dense).max() < 1e-3
+    sp0, skip0, _ = O.decode_attention(q, k, v, 0.2, n_splits=4, sparse_v_tau=0.0)
+    assert skip0 == 0 and np.array_equal(sp0, dense)
+
+
+def test_score_tile_is_dequantised_inner_product():
+    rng = np.random.default_rng(8)
+    tq = O.TurboRef(128, 4, seed=42, rotation="wht")
+    keys = rng.standard_normal((32, 128))
+    qs = rng.standard_normal((5, 128))
+    c = tq.quantize(keys)
+    direct = qs @ tq.dequantize(c).T
+    pq = tq.polar_quant
+    cent = pq.centroids
+    cn = np.linalg.norm(cent[c.mse_indices], axis=1)
+    g = c.vector_norms / cn
+    tile = O.score_tile(qs, c.mse_indices, g, cent, lambda a: O.rotate_fast(a, pq.s1, pq.s2, pq.pd),
+                        tq.qjl.S, c.qjl_signs, c.residual_norms, tq.qjl.scale)
+    np.testing.assert_allclose(tile, direct, atol=1e-11)
