@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-codec hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over one batch of synthetic input:
+  * store leg (BASELINE config 2, the `value` of the JSON line): quantise+pack
+    one Llama-3-8B-shaped layer, K and V fp16 [8, 32768, 128], 4 outlier
+    channels x15 in K, into the turbo4 block format (one launch per tensor);
+  * the same leg in turbo3 (the bit width the 70 % target is stated for);
+  * decode leg (BASELINE config 3): fused decode attention over turbo3 K/V,
+    batch 16, 32 query heads on 8 KV heads, context 32768.
+Inputs are resident in HBM before the timed region; every step cycles through
+several distinct buffer sets so that the 256 MB Infinity Cache cannot serve
+the reads.  Kernel durations come from HIP events recorded on the stream the
+kernels are launched on (torch's current stream).
+
+Prints ONE JSON line.  `roofline` prices the store kernel against 8 TB/s with
+the algorithmic bytes per launch (322 B per vector for turbo4: 256 B fp16 in,
+64 B codes, 2 B norm); `cpu_baseline` is the NumPy oracle timed on this box's
+host cores over a stated sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+D = 128
+METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
+
+
+def synth_kv(torch, heads, tokens, seed, outliers):
+    """N(0,1) fp16 [heads, tokens, 128]; `outliers` fixed channels per head scaled x15."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn((heads, tokens, D), generator=g, device="cuda", dtype=torch.float32)
+    if outliers:
+        for h in range(heads):
+            ch = np.random.default_rng(1000 + h).choice(D, size=outliers, replace=False)
+            x[h][:, torch.as_tensor(ch, device="cuda")] *= 15.0
+    return x.to(torch.float16)
+
+
+def time_steps(torch, step, steps, warmup):
+    """(wall ms per step with sync brackets, event ms per step on the launch stream)."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        step(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, e0.elapsed_time(e1) / steps
+
+
+def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
+    heads, tokens = 8, 32768
+    codec_k, codec_v = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
+    sets = []
+    for s in range(n_sets):
+        k = synth_kv(torch, heads, tokens, 10 + s, outliers=4)
+        v = synth_kv(torch, heads, tokens, 20 + s, outliers=0)
+        kp = torch.empty(tqa.packed_bytes(bits, heads, tokens), dtype=torch.uint8, device="cuda")
+        vp = torch.empty_like(kp)
+        sets.append((k, v, kp, vp))
+
+    def step(i):
+        k, v, kp, vp = sets[i % n_sets]
+        codec_k.store(k, kind="k", out=kp)
+        codec_v.store(v, kind="v", out=vp)
+
+    wall_ms, ev_ms = time_steps(torch, step, steps, warmup)
+    n_vec = 2 * heads * tokens
+    bytes_per_vec = 256 + 16 * bits + 2
+    algo = n_vec * bytes_per_vec
+    launch_us = ev_ms * 1e3 / 2                      # two launches (K, V) per step
+    gbs = (algo / 2) / (launch_us * 1e-6) / 1e9      # per launch
+    # round-trip error of the last set
+    k, v, kp, vp = sets[0]
+    rec = codec_k.load(kp, heads, tokens, kind="k", domain="original")
+    rel = float((((rec - k.float()) ** 2).sum(-1) / (k.float() ** 2).sum(-1)).mean())
+    return {
+        "workload": f"turbo{bits} store, K+V fp16 [8,32768,128], 4 K outlier channels x15, block 128",
+        "ms_per_step": wall_ms, "event_ms_per_step": ev_ms, "kernel_us": launch_us,
+        "algorithmic_bytes_per_launch": algo // 2, "gbs": gbs, "frac": gbs / HBM_PEAK_GBS,
+        "roundtrip_rel_mse_k": rel, "buffer_sets": n_sets,
+    }
+
+
+def decode_leg(torch, tqa, steps, warmup, n_sets=2):
+    B, Hq, Hkv, N, bits = 16, 32, 8, 32768, 3
+    kc, vc = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
+    sets = []
+    for s in range(n_sets):
+        kp = torch.empty(tqa.packed_bytes(bits, B * Hkv, N), dtype=torch.uint8, device="cuda")
+        vp = torch.empty_like(kp)
+        per = kp.numel() // B
+        for b in range(B):                            # generated as in the store config, per sequence
+            k = synth_kv(torch, Hkv, N, 100 + 16 * s + b, outliers=4)
+            v = synth_kv(torch, Hkv, N, 200 + 16 * s + b, outliers=0)
+            kc.store(k, kind="k", out=kp[b * per:(b + 1) * per])
+            vc.store(v, kind="v", out=vp[b * per:(b + 1) * per])
+        g = torch.Generator(device="cuda").manual_seed(300 + s)
+        q = torch.randn((B, Hq, D), generator=g, device="cuda").to(torch.float16)
+        sets.append((q, kp, vp))
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N)
+
+    def step(i):
+        q, kp, vp = sets[i % n_sets]
+        attn(q, kp, vp)
+
+    wall_ms, ev_ms = time_steps(torch, step, steps, warmup)
+    algo = 2 * B * Hkv * N * 50
+    us = ev_ms * 1e3
+    gbs = algo / (us * 1e-6) / 1e9
+    return {
+        "workload": "fused decode attention, turbo3 K/V, B16 Hq32 Hkv8 d128 ctx 32768, queries rotated in-step",
+        "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_step": algo},
+        "buffer_sets": n_sets,
+    }
+
+
+def cpu_baseline(bits):
+    """The NumPy oracle on a bounded sample of the store workload: one head of K
+    and one head of V (2 x 32768 vectors), encode + pack, float64."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import tq_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        blas_threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        blas_threads = None
+    rng = np.random.default_rng(0)
+    n = 32768
+    k = rng.standard_normal((n, D)).astype(np.float16)
+    v = rng.standard_normal((n, D)).astype(np.float16)
+    s1, s2, _ = O.sign_diagonals(D, np.random.default_rng(42))
+    cent = O.centroids_for(bits, D)
+    t0 = time.perf_counter()
+    for x, kind in ((k, "k"), (v, "v")):
+        idx, g, _ = O.turbo_encode(x, s1, s2, cent)
+        O.layout_pack(idx, g, bits, kind)
+    dt = time.perf_counter() - t0
+    algo = 2 * n * (256 + 16 * bits + 2)
+    # attention leg: one (batch, kv head) group of config 3, decompress -> softmax -> PV
+    q = rng.standard_normal((4, D))
+    idx, g, _ = O.turbo_encode(k, s1, s2, cent)
+    vi, vg, _ = O.turbo_encode(v, s1, s2, cent)
+    t0 = time.perf_counter()
+    kr = O.turbo_decode_rotated(idx, g, cent)
+    vr = O.turbo_decode_rotated(vi, vg, cent)
+    O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
+    dta = time.perf_counter() - t0
+    return ({"value": algo / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+             "sample": f"NumPy oracle turbo{bits} encode+pack of 2 x 32768 fp16 vectors (1 of 8 heads of K and of V), "
+                       f"{dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
+             "host_cpus": os.cpu_count()},
+            {"value": dta * 128 * 1e6, "unit": "µs/step", "cores": blas_threads or 1, "kind": "port",
+             "sample": f"NumPy oracle decompress->softmax->PV for 1 of 128 (batch, kv-head) groups at ctx 32768 "
+                       f"({dta * 1e3:.1f} ms), extrapolated x128", "host_cpus": os.cpu_count()})
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; every (batch, kv-head) group and every vector is an "
+              "independent unit, so more GPUs only replicate this number. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import turboquant_plus_amd as tqa
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the codec has no CPU path", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+
+    s4 = store_leg(torch, tqa, 4, args.steps, args.warmup)
+    s3 = store_leg(torch, tqa, 3, args.steps, args.warmup)
+    dec = decode_leg(torch, tqa, args.steps, args.warmup)
+    if args.skip_cpu:
+        cpu_store = cpu_attn = None
+    else:
+        cpu_store, cpu_attn = cpu_baseline(4)
+    dec["cpu_baseline"] = cpu_attn
+
+    line = {
+        "metric": METRIC, "value": s4["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": s4["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": s4["workload"], "global_batch": 2 * 8 * 32768, "io": "fp16 in, 4-bit codes + fp16 norm out",
+                   "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": s4["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s4["frac"],
+                     "traffic": None, "kernel": "k_store<4,half>", "kernel_us": s4["kernel_us"],
+                     "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
+        "cpu_baseline": cpu_store,
+        "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec,
+    }
+    print(json.dumps(line, ensure_ascii=False))
+
+
+if __name__ == "__main__":
+    main()

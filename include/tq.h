@@ -1,0 +1,194 @@
+/*
+ * tq.h - C ABI of the MI355X (gfx950) TurboQuant+ KV-codec library.
+ *
+ * The reference (TheTom/turboquant_plus) has no FFI for this path: it is plain
+ * Python over NumPy.  Each entry point below names the reference function whose
+ * per-vector arithmetic it replaces (file:line in the reference tree); the
+ * Python classes of the same names call these through ctypes.
+ *
+ * Conventions
+ *   - every data pointer is DEVICE memory unless the comment says "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - all entry points enqueue work and return without synchronising;
+ *   - return value 0 = TQ_OK, negative = error (tq_last_error() has the text);
+ *   - a handle is immutable after tq_create and may be shared across threads;
+ *   - the library allocates device memory only in tq_create (small constant
+ *     tables) and frees it in tq_destroy.
+ */
+#ifndef TQ_H
+#define TQ_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TQ_OK 0
+#define TQ_ERR_ARG (-1)         /* null pointer, negative size, bad enum          */
+#define TQ_ERR_UNSUPPORTED (-2) /* shape / mode the kernels do not cover           */
+#define TQ_ERR_ALIGN (-3)       /* pointer not aligned as the entry point requires */
+#define TQ_ERR_HIP (-4)         /* HIP runtime error (no device, launch failure)   */
+
+enum { TQ_F16 = 0, TQ_F32 = 1, TQ_F64 = 2 };
+enum { TQ_ROT_DENSE = 0, TQ_ROT_WHT = 1 };
+enum { TQ_KIND_K = 0, TQ_KIND_V = 1 };
+enum { TQ_DOMAIN_ROTATED = 0, TQ_DOMAIN_ORIGINAL = 1 };
+enum { TQ_KFMT_TURBO = 0, TQ_KFMT_Q8_0 = 1 };
+
+typedef struct tq_handle tq_handle;
+
+/* All pointers in tq_config are HOST pointers, copied at tq_create. */
+typedef struct tq_config {
+    int32_t d;                /* vector dimension (1..1024; fused kernels need 128)   */
+    int32_t bits;             /* codebook bits, 1..8                                  */
+    int32_t rotation;         /* TQ_ROT_DENSE | TQ_ROT_WHT                            */
+    int32_t norm_correction;  /* polar_quant.py:109-112                               */
+    const double *centroids;  /* [1<<bits], sorted (codebook.py:29-49)                */
+    const double *signs1;     /* [padded_d], WHT mode (rotation.py:94)                */
+    const double *signs2;     /* [padded_d], WHT mode (rotation.py:95)                */
+    const double *rotation_matrix; /* [d*d] row-major, dense mode (rotation.py:25-50) */
+    const double *projection; /* [d*d] row-major QJL matrix S or NULL (qjl.py:57-62)  */
+    double projection_scale;  /* sqrt(pi/2)/sqrt(d) (qjl.py:131) or sqrt(pi/2)/d      */
+} tq_config;
+
+int tq_version(void);
+const char *tq_last_error(void);           /* thread-local text of the last failure  */
+int tq_device_count(void);                 /* 0 when no GPU is visible               */
+
+int tq_create(tq_handle **out, const tq_config *cfg);
+void tq_destroy(tq_handle *h);
+
+/* ---- reference-API kernels: float64 arithmetic, any d <= 1024 ---------------- */
+
+/* rotation.py:99-121 fast_walsh_hadamard_transform on each of n rows of length
+ * len (power of two <= 1024); normalised by 1/sqrt(len). */
+int tq_fwht(const void *x, void *y, int64_t n, int32_t len, int in_dtype, int out_dtype, void *stream);
+
+/* The handle's rotation applied to n rows of length d: dense Pi x (polar_quant.py:78)
+ * or D2 H D1 x with zero padding (rotation.py:124-185); transpose != 0 applies the
+ * transpose (polar_quant.py:114, rotation.py:148-160).  With d == 128, WHT mode and
+ * no float64 on either side the one-wavefront-per-vector fp32 butterfly runs. */
+int tq_rotate(const tq_handle *h, const void *x, void *y, int64_t n, int in_dtype, int out_dtype,
+              int transpose, void *stream);
+
+/* codebook.py:121-134 nearest_centroid_indices: idx = #{midpoints < value}.
+ * centroids: host pointer, n_centroids <= 256. */
+int tq_nearest_centroid(const double *values, int64_t n, const double *centroids_host, int32_t n_centroids,
+                        int32_t *idx, void *stream);
+
+/* polar_quant.py:56-85 PolarQuant.quantize: idx [n,d] uint8, norms [n] float64.
+ * rotated (optional, may be NULL) receives the rotated unit vectors [n,d] float64. */
+int tq_quantize_indices(const tq_handle *h, const void *x, int64_t n, int in_dtype, uint8_t *idx, double *norms,
+                        double *rotated, void *stream);
+
+/* polar_quant.py:87-119 PolarQuant.dequantize -> out [n,d] float64.  When x is not
+ * NULL also writes residual = x - out (polar_quant.py:121-132). */
+int tq_dequantize_indices(const tq_handle *h, const uint8_t *idx, const double *norms, int64_t n, double *out,
+                          const void *x, int x_dtype, double *residual, void *stream);
+
+/* qjl.py:72-94 QJL.quantize: signs [n,d] int8 in {+1,-1} (0 -> +1), norms [n] float64. */
+int tq_qjl_quantize(const tq_handle *h, const void *r, int64_t n, int in_dtype, int8_t *signs, double *norms,
+                    void *stream);
+
+/* qjl.py:96-134 QJL.dequantize: out = S^T z * (projection_scale * norm * shrinkage). */
+int tq_qjl_dequantize(const tq_handle *h, const int8_t *signs, const double *norms, double shrinkage, int64_t n,
+                      double *out, void *stream);
+
+/* utils.py:20-49 pack_bits / utils.py:52-68 unpack_bits on [n,d] int8 signs. */
+int tq_pack_bits(const int8_t *signs, int64_t n, int32_t d, uint8_t *packed, void *stream);
+int tq_unpack_bits(const uint8_t *packed, int64_t n, int32_t d, int8_t *signs, void *stream);
+
+/* utils.py:71-98 pack_indices: one MSB-first bit stream over count indices (bits 1..4);
+ * packed must hold ceil(count*bits/8) bytes. */
+int tq_pack_indices(const uint8_t *idx, int64_t count, int32_t bits, uint8_t *packed, void *stream);
+
+/* ---- production format ("turbo2/3/4"): d = 128, WHT rotation, fp32 arithmetic,
+ *      corrected fp16 norm, 128-token blocks ----------------------------------- */
+
+/* Bytes of the packed buffer for n_seqs sequences of `tokens` tokens each
+ * (blocks never straddle sequences): n_seqs * ceil(tokens/128) * 128*(16*bits+2). */
+int64_t tq_packed_bytes(int32_t bits, int64_t n_seqs, int64_t tokens);
+
+/* Norm -> normalise -> D2 H D1 -> nearest centroid -> corrected fp16 norm -> pack.
+ * Replaces the per-vector work of KVCacheCompressor.compress (kv_cache.py:98-141)
+ * for the MSE-only ("turboN") format; arithmetic of polar_quant.py:56-85 with the
+ * rotation of rotation.py:163-185 and the write-side norm correction of
+ * benchmarks/temporal_decay_prototype.py:58-90.  x is [n_seqs, tokens, 128];
+ * x and packed must be 16-byte aligned. */
+int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind,
+             void *packed, void *stream);
+
+/* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
+ * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
+ * original domain (transpose rotation applied). */
+int tq_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
+            int out_dtype, int domain, void *stream);
+
+/* Codebook indices [n_seqs, tokens, 128] uint8 and stored norms [n_seqs, tokens]
+ * float32 of a packed buffer (test and interop aid; no reference counterpart). */
+int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind,
+                    uint8_t *idx, float *norms, void *stream);
+
+/* tq_store (kind K) plus the QJL sketch of the residual against the stored
+ * reconstruction: TurboQuant.quantize (turboquant.py:79-100) in device format.
+ * sign_bits [n,16] uint8: bit j%8 of byte j/8 is set when (S r)_j >= 0 (zero maps
+ * to +1 as in qjl.py:89-90); rnorms [n] fp16 = ||residual||.  The handle needs a
+ * projection.  n = n_seqs*tokens rows; sign_bits / rnorms are in token order.
+ * The k argument of TQ_KFMT_Q8_0 attention is a tq_q8_0_store buffer. */
+int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed,
+                 uint8_t *sign_bits, void *rnorms_f16, void *stream);
+
+/* q8_0-style K rows (textbook ggml block_q8_0 arithmetic: per 32 values
+ * scale = max|x|/127 as fp16, q = roundf(x/scale); the reference tree has no
+ * code for it).  x [n_seqs, tokens, 128] -> 128-token blocks of
+ * [8 chunks][128 rows][16 B] int8 followed by [128][4] fp16 scales
+ * (136 bytes per token); tq_q8_0_bytes gives the buffer size. */
+int64_t tq_q8_0_bytes(int64_t n_seqs, int64_t tokens);
+int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream);
+/* q [n_seqs, tokens, 128] int8 and scales [n_seqs, tokens, 4] fp32 of such a buffer. */
+int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream);
+
+/* ---- attention over packed KV ------------------------------------------------ */
+
+typedef struct tq_attn_params {
+    int32_t batch, n_q_heads, n_kv_heads;  /* GQA group = n_q_heads / n_kv_heads, must be 4 */
+    int64_t tokens;                        /* context length per sequence                    */
+    int32_t n_splits;                      /* context splits per (batch, kv head), >= 1      */
+    int32_t k_format;                      /* TQ_KFMT_TURBO | TQ_KFMT_Q8_0                   */
+    float scale;                           /* logit scale, e.g. 1/sqrt(128)                  */
+    float sparse_v_tau;                    /* 0 = dense; skip V rows with weight < tau       */
+} tq_attn_params;
+
+/* Bytes of workspace tq_decode_attention needs (split partials). */
+int64_t tq_attn_workspace_bytes(const tq_attn_params *p);
+
+/* softmax(scale * q k^T) v over packed K/V (tests/test_kv_cache.py:73-89,128-131
+ * evaluated on stored codes; no reference kernel exists).
+ *   q      [batch, n_q_heads, 128] q_dtype, in the ORIGINAL domain; the kernel
+ *          rotates it with the K handle's rotation (or leaves it for q8_0 K);
+ *   k/v    packed buffers of [batch*n_kv_heads] sequences (tq_store), or for
+ *          TQ_KFMT_Q8_0: k = int8 [batch*n_kv_heads, tokens, 128], k_aux = fp16
+ *          scales [.., tokens, 4];
+ *   bias   optional additive logit bias [batch, n_q_heads, tokens] fp32 or NULL;
+ *   out    [batch, n_q_heads, 128] fp32, original domain;
+ *   skip_count optional uint64[2]: {skipped (query, position) pairs, total pairs}. */
+int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q,
+                        int q_dtype, const void *k, const void *k_aux, const void *v, const float *bias,
+                        float *out, unsigned long long *skip_count, void *workspace, int64_t workspace_bytes,
+                        void *stream);
+
+/* TurboQuant inner-product estimate for nq queries x nk keys (turboquant.py:102-124
+ * moved to the rotated/projected domain): logits[i,j] = <R q_i, g_j c[idx_j]> +
+ * projection_scale * rnorm_j * <S q_i, z_j>.  q [nq,128] q_dtype, packed/sign_bits/
+ * rnorms from tq_store_qjl with n_seqs = 1, logits [nq, nk] fp32 (or fp16 when
+ * out_dtype == TQ_F16).  workspace: nq*256*2 bytes. */
+int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
+                  const uint8_t *sign_bits, const void *rnorms_f16, int64_t nk, void *logits, int out_dtype,
+                  void *workspace, int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TQ_H */

@@ -633,15 +633,16 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
 
 def q8_0_quantize(x):
     """Per 32 consecutive values: scale = max|x|/127 stored as fp16,
-    q = round-half-even(x / scale) clipped to [-127,127] (scale 0 -> zeros).
-    The division uses the fp32 value of the unrounded scale, as ggml does."""
+    q = roundf(x * (1/scale)) (half away from zero, as ggml's quantize_row_q8_0
+    does; scale 0 -> zeros).  All arithmetic in fp32 with the unrounded scale."""
     x = np.asarray(x, dtype=np.float32)
     lead = x.shape[:-1]
     xb = x.reshape(lead + (x.shape[-1] // 32, 32))
     amax = np.abs(xb).max(axis=-1)
     scale = (amax / np.float32(127.0)).astype(np.float32)
     inv = np.where(scale > 0, np.float32(1.0) / np.where(scale > 0, scale, 1), 0).astype(np.float32)
-    q = np.rint(xb * inv[..., None]).clip(-127, 127).astype(np.int8)
+    t = (xb * inv[..., None]).astype(np.float32)
+    q = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).clip(-127, 127).astype(np.int8)
     return q.reshape(x.shape), scale.astype(np.float16)
 
 
@@ -673,8 +674,9 @@ def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
     transpose once), the fraction of (query, position) pairs whose V row was
     skipped, and the fraction with final softmax weight < tau.
 
+    Splits are runs of ceil(ceil(N/64) / n_splits) tiles of 64 positions.
     Sparse V: within split s the running maximum is the maximum over the
-    positions of that split seen so far in blocks of 64; a position's V row is
+    positions of that split seen so far in tiles of 64; a position's V row is
     skipped for query g when exp(s_i - m_running) < tau.  Softmax statistics
     always include every position.  tau = 0 reproduces the dense result.
     """
@@ -686,12 +688,16 @@ def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
     p_final = softmax_rows(s)
     if sparse_v_tau <= 0.0:
         return p_final @ v_rot, 0.0, 0.0
-    bounds = np.linspace(0, N, n_splits + 1).astype(int)
+    n_tiles = -(-N // 64)
+    tiles_per_split = -(-n_tiles // n_splits)
+    bounds = np.minimum(np.arange(n_splits + 1) * tiles_per_split * 64, N)
     num = np.zeros((G, v_rot.shape[1]))
     den = np.zeros(G)
     m_all = np.full(G, -np.inf)
     skipped = 0
     for a, b in zip(bounds[:-1], bounds[1:]):
+        if b <= a:
+            continue
         m = np.full(G, -np.inf)
         acc = np.zeros((G, v_rot.shape[1]))
         l = np.zeros(G)

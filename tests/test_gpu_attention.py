@@ -1,0 +1,192 @@
+"""GPU parity of attention over packed KV and of the score tile against the
+oracle.  The oracle consumes the codes the GPU stored (unpacked through the
+C ABI), so these tests isolate the attention arithmetic; the store itself is
+checked in test_gpu_turbo.py.
+
+Tolerance: queries, centroid pairs and softmax weights enter the MFMA as fp16
+(fp32 accumulation), so outputs are held to the fp16-I/O bar: max abs error
+<= 2e-3 * max|reference| per query row."""
+import numpy as np
+import pytest
+
+import tq_oracle as O
+import turboquant_plus_amd as tqa
+from turboquant_plus_amd import _lib as L
+
+pytestmark = pytest.mark.gpu
+D = 128
+
+
+def np_(t):
+    return t.detach().cpu().numpy()
+
+
+def reference_attention(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, n_splits=1, tau=0.0, bias=None,
+                        k_q8=None):
+    """Oracle attention on the GPU-stored codes -> (out [B,Hq,128], skip rate, final-weight rate)."""
+    G = Hq // Hkv
+    if k_q8 is None:
+        ki, kg = kc.unpack_codes(k_packed, B * Hkv, N, kind="k")
+        k_rot = O.turbo_decode_rotated(np_(ki), np_(kg).astype(np.float64), kc.centroids)
+        q_rot = O.rotate_fast(q.astype(np.float64), kc.signs1, kc.signs2, D)
+    else:
+        qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, N)
+        k_rot = O.q8_0_dequantize(np_(qq), np_(ss))
+        q_rot = q.astype(np.float64)
+    vi, vg = vc.unpack_codes(v_packed, B * Hkv, N, kind="v")
+    v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids)
+    out = np.zeros((B, Hq, D))
+    skipped = below = 0.0
+    for b in range(B):
+        for h in range(Hkv):
+            g = b * Hkv + h
+            qs = q_rot[b, h * G:(h + 1) * G]
+            bb = None if bias is None else bias[b, h * G:(h + 1) * G]
+            o, sk, fr = O.decode_attention(qs, k_rot[g], v_rot[g], scale, n_splits=n_splits, sparse_v_tau=tau,
+                                           logit_bias=bb)
+            out[b, h * G:(h + 1) * G] = O.rotate_fast(o, vc.signs1, vc.signs2, D, transpose=True)
+            skipped += sk
+            below += fr
+    return out, skipped / (B * Hkv), below / (B * Hkv)
+
+
+def assert_close(got, ref, rel=2e-3):
+    err = np.abs(got - ref).max(axis=-1)
+    bound = rel * np.abs(ref).max(axis=-1)
+    assert np.all(err <= bound), f"max err/bound = {(err / bound).max():.3f}"
+
+
+def make_kv(B, Hkv, N, seed, kbits=3, vbits=3):
+    rng = np.random.default_rng(seed)
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    kc = tqa.TurboCodec(kbits, seed=42)
+    vc = tqa.TurboCodec(vbits, seed=542)
+    return k, v, kc, vc, kc.store(k, kind="k"), vc.store(v, kind="v")
+
+
+@pytest.mark.parametrize("N,n_splits", [(64, 1), (128, 1), (100, 1), (1000, 3), (2048, 4), (4096 + 37, 8)])
+def test_decode_attention_turbo3(N, n_splits):
+    B, Hq, Hkv = 2, 8, 2
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=N)
+    q = np.random.default_rng(N + 1).standard_normal((B, Hq, D)).astype(np.float16)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits)
+    out = np_(attn(q, kp, vp))
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D))
+    assert_close(out, ref)
+    # the split count only moves the running maxima, i.e. the fp16 rounding of the weights
+    out1 = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=1)(q, kp, vp)).copy()
+    np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("kbits,vbits", [(4, 4), (2, 2), (4, 2), (3, 2)])
+def test_decode_attention_other_bit_widths(kbits, vbits):
+    B, Hq, Hkv, N = 1, 8, 2, 640
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=kbits * 10 + vbits, kbits=kbits, vbits=vbits)
+    q = np.random.default_rng(5).standard_normal((B, Hq, D)).astype(np.float32)
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=2)(q, kp, vp))
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D))
+    assert_close(out, ref)
+
+
+def test_decode_attention_closed_forms():
+    """Identical keys -> uniform weights -> mean of V; one dominant key -> its V row."""
+    tt = L.torch()
+    B, Hq, Hkv, N = 1, 4, 1, 512
+    rng = np.random.default_rng(0)
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    v = rng.standard_normal((1, N, D)).astype(np.float32)
+    vp = vc.store(v, kind="v")
+    v_hat = np_(vc.load(vp, 1, N, kind="v", domain="original"))[0].astype(np.float64)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    k = np.tile(rng.standard_normal((1, 1, D)).astype(np.float32), (1, N, 1))
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=2)(q, kc.store(k, kind="k"), vp))
+    assert_close(out[0], np.tile(v_hat.mean(0), (4, 1)), rel=3e-3)
+    k = (rng.standard_normal((1, N, D)) * 1e-3).astype(np.float32)
+    k[0, 300] = 40 * q[0, 2] / np.linalg.norm(q[0, 2])
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=2)(q, kc.store(k, kind="k"), vp))
+    assert_close(out[0, 2:3], v_hat[300:301], rel=3e-3)
+    assert tt.isfinite(tt.from_numpy(out)).all()
+
+
+def test_decode_attention_bias_and_sparse_v():
+    B, Hq, Hkv, N = 2, 8, 2, 4096
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=77)
+    rng = np.random.default_rng(78)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    for b in range(B):
+        for h in range(Hq):
+            bias[b, h, rng.choice(N, size=16, replace=False)] = 6.0
+    tt = L.torch()
+    bias_d = tt.from_numpy(bias).cuda()
+    dense = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=4)
+    out_d = np_(dense(q, kp, vp, bias=bias_d)).copy()
+    ref_d, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), bias=bias)
+    assert_close(out_d, ref_d)
+    for tau in (1e-6, 1e-3):
+        sparse = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=4, sparse_v_tau=tau)
+        out_s = np_(sparse(q, kp, vp, bias=bias_d)).copy()
+        ref_s, skip_o, below_o = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=4,
+                                                     tau=tau, bias=bias)
+        assert_close(out_s, ref_s)
+        rate = sparse.skip_rate()
+        # the kernel's predicate equals the oracle's up to fp16 logit error near the threshold
+        assert abs(rate - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4, (rate, skip_o)
+        assert rate <= below_o + 1e-4     # in-kernel test is never looser than the final-weight test
+        print(f"\nsparse V tau={tau}: kernel skip rate {rate:.4f}, oracle {skip_o:.4f}, final-weight rate {below_o:.4f}")
+        if tau == 1e-6:
+            np.testing.assert_allclose(out_s, out_d, rtol=0, atol=1e-4 * np.abs(ref_d).max())
+
+
+def test_decode_attention_q8_0_k_turbo2_v():
+    """BASELINE config 4 shape family: K q8_0-style (not rotated), V turbo2."""
+    B, Hq, Hkv, N = 1, 8, 2, 2048 + 64
+    rng = np.random.default_rng(4)
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    vc = tqa.TurboCodec(2, seed=542)
+    kq, _, _ = tqa.q8_0_store(k)
+    vp = vc.store(v, kind="v")
+    for tau in (0.0, 1e-6):
+        attn = tqa.DecodeAttention(None, vc, B, Hq, Hkv, N, n_splits=3, sparse_v_tau=tau)
+        out = np_(attn(q, kq, vp))
+        ref, skip_o, _ = reference_attention(q, None, vc, None, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=3, tau=tau,
+                                             k_q8=kq)
+        assert_close(out, ref)
+        if tau:
+            assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
+
+
+def test_decode_attention_rejects_unsupported_group():
+    kc, vc = tqa.TurboCodec(3), tqa.TurboCodec(3)
+    with pytest.raises(NotImplementedError, match="GQA"):
+        tqa.DecodeAttention(kc, vc, 1, 8, 1, 128)
+
+
+@pytest.mark.parametrize("projection", ["orthogonal", "gaussian"])
+def test_score_tile(projection):
+    """TurboQuant inner-product estimator (BASELINE config 5 family, reduced):
+    GPU logits against the oracle's on the stored codes, and the estimator's
+    bias against the exact inner products."""
+    tt = L.torch()
+    nk, nq = 1000, 200
+    rng = np.random.default_rng(12)
+    keys = rng.standard_normal((nk, D)).astype(np.float32)
+    qs = rng.standard_normal((nq, D)).astype(np.float16)
+    codec = tqa.TurboCodec(3, seed=42, projection=projection, projection_seed=2)
+    packed, sbits, rn = codec.store_qjl(keys)
+    logits = np_(codec.score_tile(qs, packed, sbits, rn, nk))
+    idx, g = codec.unpack_codes(packed, 1, nk)
+    z = np.unpackbits(np_(sbits), axis=1, bitorder="little")[:, :D].astype(np.float64) * 2 - 1
+    ref = O.score_tile(qs.astype(np.float64), np_(idx)[0], np_(g)[0].astype(np.float64), codec.centroids,
+                       lambda a: O.rotate_fast(a, codec.signs1, codec.signs2, D), codec.S, z,
+                       np_(rn).astype(np.float64), codec.projection_scale)
+    scale = np.linalg.norm(qs.astype(np.float64), axis=1)[:, None] * np.linalg.norm(keys.astype(np.float64), axis=1)[None, :]
+    assert np.abs(logits - ref).max() <= 2e-3 * scale.max() / np.sqrt(D) * 4
+    exact = qs.astype(np.float64) @ keys.astype(np.float64).T
+    err = logits - exact
+    assert abs(err.mean()) < 4 * err.std() / np.sqrt(err.size) + 1e-3       # unbiased
+    h = np_(codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=tt.float16)).astype(np.float64)
+    assert np.abs(h - ref).max() <= 4e-3 * np.abs(ref).max()

@@ -1,0 +1,253 @@
+"""GPU parity of the production ("turbo2/3/4") format against the oracle:
+rotation, fused quantise+pack, block layout bytes, load, the QJL store and
+q8_0-style K blocks.  All calls go through the C ABI (TurboCodec is ctypes
+plumbing).
+
+Bars: codebook indices and sign bits bit-exact except where the oracle's
+float64 decision value lies within 1e-6 * max(|b|, 1/sqrt(d)) of the boundary
+b (counted, asserted small); stored fp16 norms equal or one fp16 ulp apart when
+the float64 value sits within 1e-6 relative of a rounding midpoint (counted);
+fp32 outputs within 1e-5 relative."""
+import numpy as np
+import pytest
+
+import tq_oracle as O
+import turboquant_plus_amd as tqa
+from turboquant_plus_amd import _lib as L
+
+pytestmark = pytest.mark.gpu
+D = 128
+
+
+def np_(t):
+    return t.detach().cpu().numpy()
+
+
+def kv_like(seed, shape, outlier_channels=4):
+    """N(0,1) fp16 tensor; `outlier_channels` fixed channels per head scaled x15 (BASELINE config 2)."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(shape).astype(np.float32)
+    if outlier_channels:
+        H = shape[0]
+        for h in range(H):
+            ch = np.random.default_rng(1000 + h).choice(D, size=outlier_channels, replace=False)
+            x[h][:, ch] *= 15.0
+    return x.astype(np.float16)
+
+
+def check_codes(codec, x2d, idx_gpu, g_gpu, max_band_frac=2e-5):
+    """Indices / norms of the GPU against the oracle on the same rows."""
+    idx_o, g_o, y = O.turbo_encode(x2d, codec.signs1, codec.signs2, codec.centroids,
+                                   norm_correction=codec.norm_correction)
+    n_bad, n_inadm = O.boundary_band_mismatches(y, idx_gpu, codec.centroids, rel=1e-6)
+    assert n_inadm == 0, f"{n_inadm} index mismatches outside the 1e-6 boundary band"
+    assert n_bad <= max(2, max_band_frac * idx_gpu.size), f"{n_bad} in-band mismatches of {idx_gpu.size}"
+    # norms: compare as fp16 bit patterns; rows whose indices differ may differ in the corrected norm
+    same_rows = np.all(idx_gpu == idx_o, axis=1)
+    a = g_gpu.astype(np.float16)[same_rows].view(np.uint16).astype(np.int32)
+    b = g_o[same_rows].view(np.uint16).astype(np.int32)
+    off = np.abs(a - b)
+    assert off.max(initial=0) <= 1, "stored norm off by more than one fp16 ulp"
+    assert (off == 1).sum() <= max(2, 2e-3 * a.size), f"{(off == 1).sum()} norms off by one ulp of {a.size}"
+    return n_bad, int((off == 1).sum()), idx_o, g_o
+
+
+# ---- K1: rotation -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_rotate_wave_butterfly(dtype, transpose):
+    codec = tqa.TurboCodec(3, seed=11)
+    x = np.random.default_rng(0).standard_normal((1000, D)).astype(dtype)
+    y = np_(codec.rotate(x, transpose=transpose, dtype=L.torch().float32))
+    ref = O.rotate_fast(x.astype(np.float64), codec.signs1, codec.signs2, D, transpose=transpose)
+    # fp32 butterfly: absolute error <= 1e-6 * ||x|| / sqrt(d) per coordinate
+    tol = 1e-6 * np.linalg.norm(x.astype(np.float64), axis=1, keepdims=True) / np.sqrt(D) * 4
+    assert np.all(np.abs(y - ref) <= tol)
+    np.testing.assert_allclose(np.linalg.norm(y, axis=1), np.linalg.norm(x.astype(np.float64), axis=1), rtol=1e-5)
+
+
+def test_rotate_empty_and_roundtrip():
+    codec = tqa.TurboCodec(3, seed=11)
+    assert codec.rotate(np.zeros((0, D), dtype=np.float32)).shape == (0, D)
+    x = np.random.default_rng(1).standard_normal((7, D)).astype(np.float32)
+    back = np_(codec.rotate(codec.rotate(x), transpose=True))
+    np.testing.assert_allclose(back, x, atol=2e-6)
+
+
+# ---- K2/K3: store, layout, load ------------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_store_matches_oracle_bytes(bits, kind, dtype):
+    codec = tqa.TurboCodec(bits, seed=42)
+    x = kv_like(bits, (2, 256, D)).astype(dtype)
+    x[1, 17] = 0                                            # zero vector -> norm 0
+    packed = codec.store(x, kind=kind)
+    assert packed.numel() == tqa.packed_bytes(bits, 2, 256) == 2 * 2 * O.block_bytes(bits)
+    idx, g = codec.unpack_codes(packed, 2, 256, kind=kind)
+    idx, g = np_(idx).reshape(-1, D), np_(g).reshape(-1)
+    n_bad, n_ulp, idx_o, g_o = check_codes(codec, x.reshape(-1, D), idx, g)
+    assert g[256 + 17] == 0
+    # the packed bytes are exactly the oracle's layout of the GPU's own codes ...
+    mine = O.layout_pack(idx, g.astype(np.float16), bits, kind)
+    assert np.array_equal(np_(packed), mine)
+    # ... and of the oracle's codes when no boundary case occurred
+    if n_bad == 0 and n_ulp == 0:
+        assert np.array_equal(np_(packed), O.layout_pack(idx_o, g_o, bits, kind))
+    i2, g2 = O.layout_unpack(np_(packed), bits, kind)
+    assert np.array_equal(i2, idx) and np.array_equal(g2.astype(np.float32), g)
+
+
+@pytest.mark.parametrize("tokens", [1, 63, 128, 130, 257])
+def test_store_ragged_token_counts(tokens):
+    codec = tqa.TurboCodec(3, seed=5)
+    x = np.random.default_rng(tokens).standard_normal((3, tokens, D)).astype(np.float32)
+    for kind in ("k", "v"):
+        packed = codec.store(x, kind=kind)
+        nb = -(-tokens // 128)
+        assert packed.numel() == 3 * nb * 6400
+        idx, g = codec.unpack_codes(packed, 3, tokens, kind=kind)
+        check_codes(codec, x.reshape(-1, D), np_(idx).reshape(-1, D), np_(g).reshape(-1))
+        # padding rows of the last block hold the code of 0.0 and norm 0
+        full = np.zeros((3, nb * 128, D), dtype=np.float32)
+        full[:, :tokens] = x
+        assert np.array_equal(np_(packed), np_(codec.store(full, kind=kind)))
+
+
+def test_store_empty():
+    codec = tqa.TurboCodec(3)
+    assert codec.store(np.zeros((2, 0, D), dtype=np.float16)).numel() == 0
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_load_both_domains(bits, kind):
+    tt = L.torch()
+    codec = tqa.TurboCodec(bits, seed=42)
+    x = kv_like(7, (2, 200, D))
+    packed = codec.store(x, kind=kind)
+    idx, g = codec.unpack_codes(packed, 2, 200, kind=kind)
+    idx, g = np_(idx).reshape(-1, D), np_(g).reshape(-1)
+    rot = np_(codec.load(packed, 2, 200, kind=kind, domain="rotated")).reshape(-1, D)
+    ref_rot = O.turbo_decode_rotated(idx, g, codec.centroids)
+    np.testing.assert_allclose(rot, ref_rot, rtol=1e-6, atol=1e-12)     # one fp32 product
+    org = np_(codec.load(packed, 2, 200, kind=kind, domain="original")).reshape(-1, D)
+    ref = O.turbo_decode(idx, g, codec.centroids, codec.signs1, codec.signs2)
+    scale = np.linalg.norm(ref, axis=1, keepdims=True)
+    assert np.all(np.abs(org - ref) <= 1e-5 * scale / np.sqrt(D) * 4 + 1e-12)
+    # fp16 output: 2e-3 relative
+    h = np_(codec.load(packed, 2, 200, kind=kind, domain="original", dtype=tt.float16)).astype(np.float64).reshape(-1, D)
+    assert np.all(np.abs(h - ref) <= 2e-3 * np.abs(ref).max(axis=1, keepdims=True) + 1e-7)
+    # round trip error of the codec itself: cosine and the paper's MSE bound
+    xf = x.astype(np.float64).reshape(-1, D)
+    rel = np.sum((org - xf) ** 2, axis=1) / np.sum(xf ** 2, axis=1)
+    assert rel.mean() < 2 * {2: 0.117, 3: 0.03, 4: 0.009}[bits]
+
+
+def test_config1_polarquant_turbo3_roundtrip(golden):
+    """BASELINE config 1 end to end on the GPU: 4096 fp32 vectors, seed 0, one
+    seed-1 sign diagonal, 8-level codebook; indices against the fixture the
+    reference wrote, dequantised vectors and MSE against the oracle."""
+    X = np.random.default_rng(0).standard_normal((4096, D)).astype(np.float32)
+    codec = tqa.TurboCodec(3, seed=1, single_diagonal=True)
+    packed = codec.store(X, kind="k")
+    assert packed.numel() == 32 * 6400                     # 196 608 B codes + 8 192 B fp16 norms
+    idx, g = codec.unpack_codes(packed, 1, 4096)
+    idx, g = np_(idx)[0], np_(g)[0]
+    n_bad, n_ulp, idx_o, g_o = check_codes(codec, X, idx, g)
+    print(f"\nconfig 1: {n_bad} in-band index mismatches of {idx.size}, {n_ulp} norms off by one fp16 ulp")
+    if n_bad == 0:
+        assert np.array_equal(idx[:64], golden["c1_idx_first64"])
+        assert np.array_equal(np.bincount(idx.ravel(), minlength=8), golden["c1_idx_hist"])
+    deq = np_(codec.load(packed, 1, 4096, domain="original"))[0].astype(np.float64)
+    ref = O.turbo_decode(idx, g, codec.centroids, codec.signs1, codec.signs2)
+    err = np.linalg.norm(deq - ref, axis=1) / np.linalg.norm(ref, axis=1)
+    assert err.max() <= 1e-5
+    # fixture rows were dequantised with float64 norms; stored norms are fp16 (2^-11 relative)
+    np.testing.assert_allclose(deq[:64], golden["c1_deq_first64"], rtol=0, atol=1e-3 * np.abs(golden["c1_deq_first64"]).max())
+    mse = np.mean((deq - X.astype(np.float64)) ** 2)
+    assert abs(mse - float(golden["c1_mse"])) < 2e-3 * float(golden["c1_mse"])
+
+
+def test_config2_turbo4_store_full_size_properties():
+    """BASELINE config 2 at full size ([8, 32768, 128] fp16 K with 4 outlier
+    channels x15, and V): size-independent properties plus an oracle check on a
+    row sample."""
+    tt = L.torch()
+    for bits in (4, 3):
+        codec = tqa.TurboCodec(bits, seed=42)
+        for kind, seed, outl in (("k", 1, 4), ("v", 2, 0)):
+            x = kv_like(seed, (8, 32768, D), outlier_channels=outl)
+            xd = tt.from_numpy(x).cuda()
+            packed = codec.store(xd, kind=kind)
+            assert packed.numel() == 8 * 256 * O.block_bytes(bits)
+            idx, g = codec.unpack_codes(packed, 8, 32768, kind=kind)
+            assert int(idx.max()) < (1 << bits)
+            # determinism and sequence independence: head 3 alone gives the same bytes
+            one = codec.store(xd[3], kind=kind)
+            per_head = packed.numel() // 8
+            assert tt.equal(one, packed[3 * per_head:4 * per_head])
+            # reconstruction norm equals the input norm up to fp16 rounding of the stored norm
+            rec = codec.load(packed, 8, 32768, kind=kind, domain="rotated")
+            n_in = xd.float().norm(dim=-1)
+            n_out = rec.norm(dim=-1)
+            assert float(((n_out - n_in).abs() / n_in).max()) < 1.5e-3
+            # oracle on a sample of rows from several heads
+            rows = np.random.default_rng(5).choice(8 * 32768, size=2048, replace=False)
+            check_codes(codec, x.reshape(-1, D)[rows], np_(idx).reshape(-1, D)[rows], np_(g).reshape(-1)[rows],
+                        max_band_frac=5e-5)
+            org = codec.load(packed, 8, 32768, kind=kind, domain="original")
+            rel = float((((org - xd.float()) ** 2).sum(-1) / (xd.float() ** 2).sum(-1)).mean())
+            assert rel < 2 * {3: 0.03, 4: 0.009}[bits]
+            del x, xd, packed, idx, g, rec, org
+
+
+# ---- K4: QJL store ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("projection", ["orthogonal", "gaussian"])
+@pytest.mark.parametrize("bits", [2, 3])
+def test_store_qjl_matches_oracle(projection, bits):
+    codec = tqa.TurboCodec(bits, seed=42, projection=projection, projection_seed=2)
+    x = np.random.default_rng(9).standard_normal((300, D)).astype(np.float32)
+    x[4] = 0
+    packed, sbits, rn = codec.store_qjl(x)
+    idx, g = codec.unpack_codes(packed, 1, 300)
+    idx, g = np_(idx)[0], np_(g)[0]
+    # float64 kernel: indices equal the oracle's, norms bit-equal as fp16
+    idx_o, g_o, y = O.turbo_encode(x, codec.signs1, codec.signs2, codec.centroids)
+    n_bad, n_inadm = O.boundary_band_mismatches(y, idx, codec.centroids, rel=1e-12)
+    assert (n_bad, n_inadm) == (0, 0)
+    assert np.array_equal(g.astype(np.float16).view(np.uint16), g_o.view(np.uint16))
+    # residual against the stored reconstruction, sketched with S
+    resid = x.astype(np.float64) - O.turbo_decode(idx_o, g_o, codec.centroids, codec.signs1, codec.signs2)
+    proj = resid @ codec.S.T
+    z_o = np.where(proj >= 0, 1, -1)
+    z = np.unpackbits(np_(sbits), axis=1, bitorder="little")[:, :D].astype(np.int64) * 2 - 1
+    bad = z != z_o
+    band = 1e-6 * np.linalg.norm(resid, axis=1, keepdims=True) / np.sqrt(D) * np.ones_like(proj)
+    assert np.all(np.abs(proj)[bad] <= band[bad]), "sign mismatch outside the band"
+    assert bad.sum() <= 2
+    rn_o = np.linalg.norm(resid, axis=1).astype(np.float16)
+    off = np.abs(np_(rn).view(np.uint16).astype(np.int32) - rn_o.view(np.uint16).astype(np.int32))
+    assert off.max() <= 1 and (off == 1).sum() <= 2
+    assert np_(rn)[4] == 0 and g[4] == 0
+
+
+# ---- q8_0-style K blocks ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("tokens", [128, 200])
+def test_q8_0_store_bit_exact(tokens):
+    x = np.random.default_rng(3).standard_normal((2, tokens, D)).astype(np.float32)
+    x[0, 5, 32:64] = 0
+    packed, n_seqs, t = tqa.q8_0_store(x)
+    assert (n_seqs, t) == (2, tokens) and packed.numel() == 2 * (-(-tokens // 128)) * 128 * 136
+    q, s = tqa.q8_0_unpack(packed, 2, tokens)
+    q_o, s_o = O.q8_0_quantize(x)
+    assert np.array_equal(np_(q), q_o)
+    assert np.array_equal(np_(s).astype(np.float16).view(np.uint16), s_o.view(np.uint16))
+    x16 = x.astype(np.float16)
+    q2, s2 = tqa.q8_0_unpack(tqa.q8_0_store(x16)[0], 2, tokens)
+    q_o, s_o = O.q8_0_quantize(x16.astype(np.float32))
+    assert np.array_equal(np_(q2), q_o) and np.array_equal(np_(s2).astype(np.float16).view(np.uint16), s_o.view(np.uint16))

@@ -1,0 +1,635 @@
+// Attention over packed KV and the prefill-shaped score tile.
+//
+// k_decode_attn: split-K decode attention for one GQA group of 4 query heads.
+//   One 64-lane wavefront owns one context split and walks it in tiles of 64
+//   tokens.  Lane l holds packed row l of the tile (K: token l; V: token quad
+//   l/4, sub-row l%4), loaded as 16-byte chunks that are contiguous across
+//   lanes.  Pair codes are turned into fp16 pairs through a 4-byte-entry LUT
+//   in LDS (one ds_read per two values) and fed to the 4x4x4 fp16 MFMA with
+//   16 independent blocks: block b multiplies the 4 tokens 4b..4b+3 by the 4
+//   query heads, so all 64 lanes and all 16 blocks do useful work.
+//     QK: A_b = K[tokens 4b..4b+3][4 dims], B_b = q^T[4 dims][4 heads]
+//         -> lane (b,j) gets the logits of head j for tokens 4b..4b+3.
+//     PV: A_b = P[4 heads][tokens 4b..4b+3] (the same lane layout the QK output
+//         has), B_b = V[tokens 4b..4b+3][4 dims] -> D_b = partial out[4 heads][4 dims];
+//         the 16 blocks are summed across lanes once at the end of the split.
+//   Online softmax in base 2 (log2(e) folded into the query scale); accumulators
+//   are rescaled only when a running maximum moves.
+// k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
+//   the V rotation (one wavefront per query head).
+// k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
+//   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+#include "tq_device.h"
+
+namespace {
+
+using namespace tqd;
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RSQRT128 = 0.08838834764831845f;
+
+template <typename T> __device__ inline float ldf(const T *p) { return (float)*p; }
+template <> __device__ inline float ldf<__half>(const __half *p) { return __half2float(*p); }
+
+// runtime-p version of pair_lut_offset; p is a compile-time constant after unrolling
+template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t (&w)[4 * BITS], int p) {
+    if constexpr (BITS == 4) {
+        const int q = p >> 2, k = p & 3;
+        return k == 0 ? ((w[q] << 2) & 0x3FCu) : ((w[q] >> (8 * k - 2)) & 0x3FCu);
+    } else if constexpr (BITS == 2) {
+        const int q = p >> 3, k = p & 7;
+        return k == 0 ? ((w[q] << 2) & 0x3Cu) : ((w[q] >> (4 * k - 2)) & 0x3Cu);
+    } else {
+        if (p < 60) {
+            const int q = p / 5, k = p % 5;
+            return k == 0 ? ((w[q] << 2) & 0xFCu) : ((w[q] >> (6 * k - 2)) & 0xFCu);
+        }
+        const int t = p - 60;
+        return ((w[3 * t] >> 28) & 0xCu) | ((w[3 * t + 1] >> 26) & 0x30u) | ((w[3 * t + 2] >> 24) & 0xC0u);
+    }
+}
+
+template <int BITS> __device__ __forceinline__ void load_row(const uint8_t *block, int row, uint32_t (&w)[4 * BITS]) {
+#pragma unroll
+    for (int c = 0; c < BITS; ++c) {
+        const uint4 u = *reinterpret_cast<const uint4 *>(block + c * 2048 + row * 16);
+        w[4 * c] = u.x; w[4 * c + 1] = u.y; w[4 * c + 2] = u.z; w[4 * c + 3] = u.w;
+    }
+}
+
+__device__ __forceinline__ half4_t h4_from(uint32_t a, uint32_t b) {
+    const uint2 u = make_uint2(a, b);
+    return __builtin_bit_cast(half4_t, u);
+}
+
+__device__ __forceinline__ float4_t mfma4(half4_t a, half4_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 0, 0, 0);
+}
+
+// sum over the 16 lanes that share lane%4 (blocks b = 0..15)
+__device__ __forceinline__ float sum_over_blocks(float v) {
+    v += xor_lane<4>(v);
+    v += xor_lane<8>(v);
+    v += xor_lane<16>(v);
+    v += xor_lane<32>(v);
+    return v;
+}
+__device__ __forceinline__ float max_over_blocks(float v) {
+    v = fmaxf(v, xor_lane<4>(v));
+    v = fmaxf(v, xor_lane<8>(v));
+    v = fmaxf(v, xor_lane<16>(v));
+    v = fmaxf(v, xor_lane<32>(v));
+    return v;
+}
+
+struct AttnArgs {
+    const __half *qrot;  // [groups*4][128], rotated by the K rotation (turbo K), scaled by scale*log2(e)
+    const uint8_t *k, *v;
+    const uint32_t *klut, *vlut;  // pair LUTs (half2 per pair code)
+    const float *bias;            // [groups*4][tokens] natural-log units, or NULL
+    float *part_o;                // [groups][n_splits][4][128]
+    float *part_ml;               // [groups][n_splits][4][2]  (m in log2 units, l)
+    unsigned long long *skip;     // [0] += skipped (query, position) pairs
+    int64_t tokens, blocks_per_seq;
+    int n_groups, n_splits, tiles_per_split, n_tiles;
+    float tau;
+};
+
+constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
+
+template <int KFMT, int KBITS, int VBITS, bool SPARSE>
+__global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
+    constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
+    constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
+    constexpr int VBLOCK = TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
+    constexpr int KLUT_N = KFMT == KFMT_TURBO ? (1 << (2 * KBITS)) : 1;
+    constexpr int VLUT_N = 1 << (2 * VBITS);
+    __shared__ uint32_t klut_s[KLUT_N];
+    __shared__ uint32_t vlut_s[VLUT_N];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    if constexpr (KFMT == KFMT_TURBO)
+        for (int i = tid; i < KLUT_N; i += 256) klut_s[i] = a.klut[i];
+    for (int i = tid; i < VLUT_N; i += 256) vlut_s[i] = a.vlut[i];
+    __syncthreads();
+
+    const int64_t wid = (int64_t)blockIdx.x * 4 + (tid >> 6);
+    const int group = (int)(wid / a.n_splits), split = (int)(wid % a.n_splits);
+    if (group >= a.n_groups) return;
+    const int t_begin = split * a.tiles_per_split;
+    const int t_end = min(t_begin + a.tiles_per_split, a.n_tiles);
+    const int b4 = lane & ~3;  // 4 * block index
+    const int j = lane & 3;    // query head of the logits this lane holds; sub-row for V
+
+    float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
+    float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
+
+    // B operand of QK: q[head j][dims 4g..4g+3], g = 0..31
+    half4_t qreg[32];
+    {
+        const uint2 *qp = reinterpret_cast<const uint2 *>(a.qrot + ((int64_t)group * 4 + j) * 128);
+#pragma unroll
+        for (int g = 0; g < 32; ++g) qreg[g] = __builtin_bit_cast(half4_t, qp[g]);
+    }
+    float4_t acc_o[32];
+#pragma unroll
+    for (int g = 0; g < 32; ++g) acc_o[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+    unsigned nskip = 0;
+
+    const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
+    const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
+    const char *klut_b = reinterpret_cast<const char *>(klut_s);
+    const char *vlut_b = reinterpret_cast<const char *>(vlut_s);
+
+    uint32_t kw[KROW_DW];
+    if (t_begin < t_end) {
+        const uint8_t *kb = kbase + (int64_t)(t_begin >> 1) * KBLOCK;
+        const int row = (t_begin & 1) * 64 + lane;
+        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row, kw);
+        else load_row<8>(kb, row, kw);
+    }
+
+#pragma unroll 1
+    for (int tile = t_begin; tile < t_end; ++tile) {
+        const int64_t blk = tile >> 1;
+        const int half = tile & 1;
+        const int row = half * 64 + lane;
+        const int tok_in_block = half * 64 + b4;  // first of this lane's 4 tokens, inside the block
+        const uint8_t *kb = kbase + blk * KBLOCK;
+        const uint8_t *vb = vbase + blk * VBLOCK;
+
+        // ---- issue loads: K scales, V row (dense mode), next K row ----------------
+        float gk[4];
+        float kscale[4][4];
+        if constexpr (KFMT == KFMT_TURBO) {
+            const uint2 u = *reinterpret_cast<const uint2 *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS + 2 * tok_in_block);
+            gk[0] = __half2float(__ushort_as_half((unsigned short)(u.x & 0xffff)));
+            gk[1] = __half2float(__ushort_as_half((unsigned short)(u.x >> 16)));
+            gk[2] = __half2float(__ushort_as_half((unsigned short)(u.y & 0xffff)));
+            gk[3] = __half2float(__ushort_as_half((unsigned short)(u.y >> 16)));
+        } else {
+            const uint4 *sp = reinterpret_cast<const uint4 *>(kb + 8 * 2048 + 8 * tok_in_block);
+            const uint4 s0 = sp[0], s1 = sp[1];
+            const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                kscale[i][0] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i] & 0xffff)));
+                kscale[i][1] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i] >> 16)));
+                kscale[i][2] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i + 1] & 0xffff)));
+                kscale[i][3] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i + 1] >> 16)));
+            }
+        }
+        uint32_t vw[4 * VBITS];
+        if constexpr (!SPARSE) load_row<VBITS>(vb, row, vw);
+        const uint2 gvu = *reinterpret_cast<const uint2 *>(vb + TQ_ROWS_PER_BLOCK * 16 * VBITS + 2 * tok_in_block);
+        uint32_t kw_next[KROW_DW];
+        if (tile + 1 < t_end) {
+            const uint8_t *kbn = kbase + (int64_t)((tile + 1) >> 1) * KBLOCK;
+            const int rown = ((tile + 1) & 1) * 64 + lane;
+            if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, rown, kw_next);
+            else load_row<8>(kbn, rown, kw_next);
+        }
+        float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+        const int64_t tok0 = (int64_t)tile * 64 + b4;
+        if (a.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (tok0 + i < a.tokens) bias4[i] = a.bias[((int64_t)group * 4 + j) * a.tokens + tok0 + i] * LOG2E;
+        }
+
+        // ---- QK ------------------------------------------------------------------
+        float s[4];
+        if constexpr (KFMT == KFMT_TURBO) {
+            float4_t acc[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < 32; ++g) {
+                const uint32_t lo = *reinterpret_cast<const uint32_t *>(klut_b + pair_off<KBITS>(kw, 2 * g));
+                const uint32_t hi = *reinterpret_cast<const uint32_t *>(klut_b + pair_off<KBITS>(kw, 2 * g + 1));
+                acc[g & 3] = mfma4(h4_from(lo, hi), qreg[g], acc[g & 3]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] = ((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i])) * gk[i] + bias4[i];
+        } else {
+            float4_t acc[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < 32; ++g) {
+                const uint32_t w = kw[g];
+                half4_t kv;
+                kv[0] = (_Float16)(int)(int8_t)(w & 0xff);
+                kv[1] = (_Float16)(int)(int8_t)((w >> 8) & 0xff);
+                kv[2] = (_Float16)(int)(int8_t)((w >> 16) & 0xff);
+                kv[3] = (_Float16)(int)(int8_t)(w >> 24);
+                acc[g >> 3] = mfma4(kv, qreg[g], acc[g >> 3]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                s[i] = (acc[0][i] * kscale[i][0] + acc[1][i] * kscale[i][1]) +
+                       (acc[2][i] * kscale[i][2] + acc[3][i] * kscale[i][3]) + bias4[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (tok0 + i >= a.tokens) s[i] = -INFINITY;
+
+        // ---- online softmax (base 2) ------------------------------------------------
+        const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+        const float m_new = fmaxf(m_run, mx);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+            const float corr = exp2f(m_run - m_new);  // 0 on the first tile
+            l_run *= corr;
+            const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
+#pragma unroll
+            for (int g = 0; g < 32; ++g) {
+                acc_o[g][0] *= c0;
+                acc_o[g][1] *= c1;
+                acc_o[g][2] *= c2;
+                acc_o[g][3] *= c3;
+            }
+            m_run = m_new;
+        }
+        float p[4];
+        bool any_keep = false;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[i] = exp2f(s[i] - m_run);
+            l_run += p[i];
+            if constexpr (SPARSE) {
+                const bool in_range = tok0 + i < a.tokens;
+                const bool keep = p[i] >= a.tau;
+                if (in_range && !keep) ++nskip;
+                if (!keep) p[i] = 0.0f;
+                any_keep |= keep && in_range;
+            }
+        }
+        if constexpr (SPARSE) {
+            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {
+#pragma unroll
+                for (int q = 0; q < KROW_DW; ++q) kw[q] = kw_next[q];
+                continue;  // every V row of this tile is skipped: no V load, no dequant
+            }
+            load_row<VBITS>(vb, row, vw);
+        }
+
+        // ---- PV ------------------------------------------------------------------------
+        half4_t pv;
+        pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.x & 0xffff))));
+        pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
+        pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
+        pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
+#pragma unroll
+        for (int g = 0; g < 32; ++g) {
+            const uint32_t lo = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 2 * g));
+            const uint32_t hi = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 2 * g + 1));
+            acc_o[g] = mfma4(pv, h4_from(lo, hi), acc_o[g]);
+        }
+#pragma unroll
+        for (int q = 0; q < KROW_DW; ++q) kw[q] = kw_next[q];
+    }
+
+    // ---- end of split: sum the 16 blocks, write the partial ------------------------
+    const float l_tot = sum_over_blocks(l_run);
+#pragma unroll
+    for (int g = 0; g < 32; ++g) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float v = sum_over_blocks(acc_o[g][i]);
+            if (lane < 4) po[i * 128 + 4 * g + j] = v;
+        }
+    }
+    if (lane < 4) {
+        pml[2 * j] = m_run;
+        pml[2 * j + 1] = l_tot;
+    }
+    if constexpr (SPARSE) {
+        unsigned tot = nskip;
+        for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
+        if (lane == 0 && tot) atomicAdd(a.skip, (unsigned long long)tot);
+    }
+}
+
+// q -> rotated, scaled fp16 (one wavefront per query row); also clears the skip counter
+template <typename TI>
+__global__ __launch_bounds__(256) void k_prep_q(const TI *q, __half *qrot, int64_t n, const float *s1, const float *s2,
+                                                float scale_log2e, int rotate, unsigned long long *skip,
+                                                unsigned long long total_pairs) {
+    const int lane = threadIdx.x & 63;
+    const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (skip && blockIdx.x == 0 && threadIdx.x == 0) {
+        skip[0] = 0ull;
+        skip[1] = total_pairs;
+    }
+    if (v >= n) return;
+    float x0 = ldf(q + v * 128 + 2 * lane), x1 = ldf(q + v * 128 + 2 * lane + 1);
+    if (rotate) {
+        x0 *= s1[2 * lane];
+        x1 *= s1[2 * lane + 1];
+        wht128_wave(x0, x1, lane);
+        x0 *= s2[2 * lane] * RSQRT128;
+        x1 *= s2[2 * lane + 1] * RSQRT128;
+    }
+    qrot[v * 128 + 2 * lane] = __float2half_rn(x0 * scale_log2e);
+    qrot[v * 128 + 2 * lane + 1] = __float2half_rn(x1 * scale_log2e);
+}
+
+// merge split partials, un-rotate with the V rotation's transpose; one wavefront per query head
+__global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
+                                                      int64_t n_rows, int n_splits, const float *s1, const float *s2) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
+    if (r >= n_rows) return;
+    const int64_t group = r >> 2;
+    const int head = (int)(r & 3);
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) {
+        const float l = part_ml[((group * n_splits + s) * 4 + head) * 2 + 1];
+        if (l > 0.0f) M = fmaxf(M, part_ml[((group * n_splits + s) * 4 + head) * 2]);
+    }
+    float L = 0.0f, o0 = 0.0f, o1 = 0.0f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float *ml = part_ml + ((group * n_splits + s) * 4 + head) * 2;
+        if (!(ml[1] > 0.0f)) continue;
+        const float w = exp2f(ml[0] - M);
+        L += ml[1] * w;
+        const float *po = part_o + ((group * n_splits + s) * 4 + head) * 128;
+        o0 = fmaf(po[2 * lane], w, o0);
+        o1 = fmaf(po[2 * lane + 1], w, o1);
+    }
+    const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+    o0 *= invL * s2[2 * lane];
+    o1 *= invL * s2[2 * lane + 1];
+    wht128_wave(o0, o1, lane);
+    out[r * 128 + 2 * lane] = o0 * (s1[2 * lane] * RSQRT128);
+    out[r * 128 + 2 * lane + 1] = o1 * (s1[2 * lane + 1] * RSQRT128);
+}
+
+inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+struct WsLayout {
+    int64_t qrot, part_o, part_ml, total;
+};
+WsLayout ws_layout(const tq_attn_params *p) {
+    const int64_t rows = (int64_t)p->batch * p->n_q_heads;
+    const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
+    WsLayout w;
+    w.qrot = 0;
+    w.part_o = align256(rows * 128 * 2);
+    w.part_ml = w.part_o + align256(groups * p->n_splits * 4 * 128 * 4);
+    w.total = w.part_ml + align256(groups * p->n_splits * 4 * 2 * 4);
+    return w;
+}
+
+}  // namespace
+
+int64_t tqk_attn_workspace_bytes(const tq_attn_params *p) { return ws_layout(p).total; }
+
+int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q, int q_dtype,
+                         const void *k, const void *k_aux, const void *v, const float *bias, float *out,
+                         unsigned long long *skip_count, void *ws, int64_t ws_bytes, hipStream_t s) {
+    (void)k_aux;
+    const WsLayout w = ws_layout(p);
+    if (ws_bytes < w.total) {
+        tq_set_error("tq_decode_attention: workspace %lld < %lld bytes", (long long)ws_bytes, (long long)w.total);
+        return TQ_ERR_ARG;
+    }
+    const int64_t rows = (int64_t)p->batch * p->n_q_heads;
+    const int groups = p->batch * p->n_kv_heads;
+    __half *qrot = reinterpret_cast<__half *>((char *)ws + w.qrot);
+    float *part_o = reinterpret_cast<float *>((char *)ws + w.part_o);
+    float *part_ml = reinterpret_cast<float *>((char *)ws + w.part_ml);
+    const bool turbo_k = p->k_format == TQ_KFMT_TURBO;
+    const float sc = p->scale * LOG2E;
+    const unsigned long long total_pairs = (unsigned long long)rows * (unsigned long long)p->tokens;
+    const unsigned qgrid = (unsigned)((rows + 3) / 4);
+    const float *ks1 = turbo_k ? hk->s1_32 : nullptr, *ks2 = turbo_k ? hk->s2_32 : nullptr;
+    switch (q_dtype) {
+    case TQ_F16:
+        k_prep_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
+        break;
+    case TQ_F32:
+        k_prep_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
+        break;
+    case TQ_F64:
+        k_prep_q<double><<<qgrid, 256, 0, s>>>((const double *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
+        break;
+    default: tq_set_error("bad q dtype %d", q_dtype); return TQ_ERR_ARG;
+    }
+    int rc = tq_check_launch("prep_q");
+    if (rc) return rc;
+
+    AttnArgs a;
+    a.qrot = qrot;
+    a.k = (const uint8_t *)k;
+    a.v = (const uint8_t *)v;
+    a.klut = turbo_k ? (const uint32_t *)hk->pair_lut : nullptr;
+    a.vlut = (const uint32_t *)hv->pair_lut;
+    a.bias = bias;
+    a.part_o = part_o;
+    a.part_ml = part_ml;
+    a.skip = skip_count;
+    a.tokens = p->tokens;
+    a.blocks_per_seq = (p->tokens + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
+    a.n_groups = groups;
+    a.n_splits = p->n_splits;
+    a.n_tiles = (int)((p->tokens + 63) / 64);
+    a.tiles_per_split = (a.n_tiles + p->n_splits - 1) / p->n_splits;
+    a.tau = p->sparse_v_tau;
+    const bool sparse = p->sparse_v_tau > 0.0f;
+    if (sparse && !skip_count) {
+        tq_set_error("tq_decode_attention: sparse_v_tau > 0 needs skip_count");
+        return TQ_ERR_ARG;
+    }
+    const unsigned grid = (unsigned)(((int64_t)groups * p->n_splits + 3) / 4);
+    const int vb = hv->bits;
+    const int kb = turbo_k ? hk->bits : 8;
+#define TQ_ATTN(KF, KB, VB)                                                \
+    if (sparse) k_decode_attn<KF, KB, VB, true><<<grid, 256, 0, s>>>(a);  \
+    else k_decode_attn<KF, KB, VB, false><<<grid, 256, 0, s>>>(a)
+    if (turbo_k && kb == 3 && vb == 3) { TQ_ATTN(KFMT_TURBO, 3, 3); }
+    else if (turbo_k && kb == 4 && vb == 4) { TQ_ATTN(KFMT_TURBO, 4, 4); }
+    else if (turbo_k && kb == 2 && vb == 2) { TQ_ATTN(KFMT_TURBO, 2, 2); }
+    else if (turbo_k && kb == 4 && vb == 2) { TQ_ATTN(KFMT_TURBO, 4, 2); }
+    else if (turbo_k && kb == 3 && vb == 2) { TQ_ATTN(KFMT_TURBO, 3, 2); }
+    else if (!turbo_k && vb == 2) { TQ_ATTN(KFMT_Q8, 3, 2); }
+    else if (!turbo_k && vb == 3) { TQ_ATTN(KFMT_Q8, 3, 3); }
+    else if (!turbo_k && vb == 4) { TQ_ATTN(KFMT_Q8, 3, 4); }
+    else {
+        tq_set_error("tq_decode_attention: unsupported K/V format pair (k bits %d, v bits %d)", kb, vb);
+        return TQ_ERR_UNSUPPORTED;
+    }
+#undef TQ_ATTN
+    rc = tq_check_launch("decode_attn");
+    if (rc) return rc;
+    k_attn_combine<<<qgrid, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
+    return tq_check_launch("attn_combine");
+}
+
+// ---- prefill-shaped TurboQuant inner-product estimator --------------------------------
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+constexpr int KT_STRIDE = 264;  // halves per staged key row (256 + 8: 16-byte reads of 16 rows hit 64 distinct banks)
+
+// [R q | S q] as fp16, one wavefront per query
+template <typename TI>
+__global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, int64_t nq, const float *s1,
+                                                      const float *s2, const float *projT) {
+    __shared__ float qs[4][128];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t v = (int64_t)blockIdx.x * 4 + w;
+    float x0 = 0.f, x1 = 0.f;
+    if (v < nq) {
+        x0 = ldf(q + v * 128 + 2 * lane);
+        x1 = ldf(q + v * 128 + 2 * lane + 1);
+    }
+    qs[w][2 * lane] = x0;
+    qs[w][2 * lane + 1] = x1;
+    __syncthreads();
+    if (v >= nq) return;
+    float p0 = 0.f, p1 = 0.f;  // (S q)[2*lane], (S q)[2*lane+1]
+    for (int k = 0; k < 128; ++k) {
+        const float qk = qs[w][k];
+        p0 = fmaf(projT[k * 128 + 2 * lane], qk, p0);
+        p1 = fmaf(projT[k * 128 + 2 * lane + 1], qk, p1);
+    }
+    x0 *= s1[2 * lane];
+    x1 *= s1[2 * lane + 1];
+    wht128_wave(x0, x1, lane);
+    x0 *= s2[2 * lane] * RSQRT128;
+    x1 *= s2[2 * lane + 1] * RSQRT128;
+    qa[v * 256 + 2 * lane] = __float2half_rn(x0);
+    qa[v * 256 + 2 * lane + 1] = __float2half_rn(x1);
+    qa[v * 256 + 128 + 2 * lane] = __float2half_rn(p0);
+    qa[v * 256 + 128 + 2 * lane + 1] = __float2half_rn(p1);
+}
+
+template <typename T> __device__ inline void st_logit4(T *p, float4_t v, int n_ok);
+template <> __device__ inline void st_logit4<float>(float *p, float4_t v, int n_ok) {
+    if (n_ok >= 4 && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        for (int i = 0; i < 4 && i < n_ok; ++i) p[i] = v[i];
+    }
+}
+template <> __device__ inline void st_logit4<__half>(__half *p, float4_t v, int n_ok) {
+    for (int i = 0; i < 4 && i < n_ok; ++i) p[i] = __float2half_rn(v[i]);
+}
+
+// One workgroup per 128-key block: dequantise the block once into LDS as fp16
+// [g*c[idx] | scale*rnorm*z], then sweep all queries with 16x16x32 MFMA tiles
+// (keys on the M side so that each lane owns 4 consecutive keys of one query).
+template <int BITS, typename TO>
+__global__ __launch_bounds__(256) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
+                                                   const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
+                                                   const float *cent, float proj_scale) {
+    extern __shared__ _Float16 kt[];  // [128][KT_STRIDE]
+    __shared__ float cent_s[16];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int64_t key0 = (int64_t)blockIdx.x * 128;
+    const uint8_t *block = packed + (int64_t)blockIdx.x * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
+    if (tid < (1 << BITS)) cent_s[tid] = cent[tid];
+    __syncthreads();
+    {
+        const int key = tid & 127, part = tid >> 7;
+        _Float16 *row = kt + key * KT_STRIDE;
+        const bool valid = key0 + key < nk;
+        if (part == 0) {
+            uint32_t wv[4 * BITS];
+            load_row<BITS>(block, key, wv);
+            const float g = valid ? __half2float(reinterpret_cast<const __half *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key]) : 0.f;
+#pragma unroll
+            for (int p = 0; p < 64; ++p) {
+                const uint32_t pc = pair_off<BITS>(wv, p) >> 2;
+                row[2 * p] = (_Float16)(cent_s[pc & ((1u << BITS) - 1u)] * g);
+                row[2 * p + 1] = (_Float16)(cent_s[pc >> BITS] * g);
+            }
+        } else {
+            float rs = 0.f;
+            uint4 sb = make_uint4(0, 0, 0, 0);
+            if (valid) {
+                rs = proj_scale * __half2float(rnorms[key0 + key]);
+                sb = *reinterpret_cast<const uint4 *>(sign_bits + (key0 + key) * 16);
+            }
+            const uint32_t sw[4] = {sb.x, sb.y, sb.z, sb.w};
+            const _Float16 pos = (_Float16)rs, neg = (_Float16)(-rs);
+#pragma unroll
+            for (int jj = 0; jj < 128; ++jj) row[128 + jj] = ((sw[jj >> 5] >> (jj & 31)) & 1u) ? pos : neg;
+        }
+    }
+    __syncthreads();
+
+    const int kh = w & 1, qh = w >> 1;
+    const int r16 = lane & 15, kc = lane >> 4;
+    const int64_t n_qt = (nq + 127) / 128;
+    for (int64_t qt = 0; qt < n_qt; ++qt) {
+        float4_t acc[4][4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const int64_t qbase = qt * 128 + qh * 64;
+#pragma unroll 2
+        for (int ks = 0; ks < 8; ++ks) {
+            half8_t af[4], bf[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                af[a] = *reinterpret_cast<const half8_t *>(kt + (kh * 64 + a * 16 + r16) * KT_STRIDE + ks * 32 + 8 * kc);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int64_t qi = qbase + b * 16 + r16;
+                if (qi < nq) bf[b] = *reinterpret_cast<const half8_t *>(qa + qi * 256 + ks * 32 + 8 * kc);
+                else bf[b] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int64_t qi = qbase + b * 16 + r16;
+                const int64_t key = key0 + kh * 64 + a * 16 + 4 * kc;
+                if (qi < nq && key < nk) st_logit4(logits + qi * nk + key, acc[a][b], (int)min((int64_t)4, nk - key));
+            }
+    }
+}
+
+}  // namespace
+
+int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
+                   const uint8_t *sign_bits, const void *rnorms, int64_t nk, void *logits, int out_dtype, void *ws,
+                   int64_t ws_bytes, hipStream_t s) {
+    (void)ws_bytes;
+    __half *qa = reinterpret_cast<__half *>(ws);
+    const unsigned qgrid = (unsigned)((nq + 3) / 4);
+    switch (q_dtype) {
+    case TQ_F16: k_prep_score_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
+    case TQ_F32: k_prep_score_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
+    case TQ_F64: k_prep_score_q<double><<<qgrid, 256, 0, s>>>((const double *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
+    default: tq_set_error("bad q dtype %d", q_dtype); return TQ_ERR_ARG;
+    }
+    int rc = tq_check_launch("prep_score_q");
+    if (rc) return rc;
+    const unsigned grid = (unsigned)((nk + 127) / 128);
+    const size_t lds = (size_t)128 * KT_STRIDE * sizeof(_Float16);
+#define TQ_SCORE(B, T)                                                                                          \
+    {                                                                                                           \
+        (void)hipFuncSetAttribute((const void *)k_score_tile<B, T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                  (int)lds);                                                                    \
+        k_score_tile<B, T><<<grid, 256, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
+                                                  nq, nk, (T *)logits, h->centroids32, (float)h->proj_scale);   \
+    }
+    if (out_dtype == TQ_F32) {
+        if (h->bits == 2) TQ_SCORE(2, float) else if (h->bits == 3) TQ_SCORE(3, float) else TQ_SCORE(4, float)
+    } else {
+        if (h->bits == 2) TQ_SCORE(2, __half) else if (h->bits == 3) TQ_SCORE(3, __half) else TQ_SCORE(4, __half)
+    }
+#undef TQ_SCORE
+    return tq_check_launch("score_tile");
+}

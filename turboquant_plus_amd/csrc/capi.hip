@@ -1,0 +1,419 @@
+// extern "C" surface of the library: argument checks, handle lifetime, dispatch.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "tq_internal.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+// float64 -> fp16 bit pattern, one round-to-nearest-even
+uint16_t f64_to_f16_bits(double v) {
+    if (std::isnan(v)) return 0x7e00;
+    const uint16_t sign = std::signbit(v) ? 0x8000 : 0;
+    double a = std::fabs(v);
+    if (a >= 65520.0) return sign | 0x7c00;
+    if (a < 5.9604644775390625e-08 * 0.5) return sign;  // below half the smallest subnormal
+    int e;
+    double m = std::frexp(a, &e);  // a = m * 2^e, m in [0.5, 1)
+    int exp = e - 1;               // a = (2m) * 2^exp, 2m in [1, 2)
+    if (exp < -14) {               // subnormal: units of 2^-24
+        const double q = a / 5.9604644775390625e-08;
+        double r = std::nearbyint(q);
+        return sign | (uint16_t)r;
+    }
+    const double frac = (2.0 * m - 1.0) * 1024.0;
+    double r = std::nearbyint(frac);  // default rounding mode: nearest-even
+    uint32_t bits = ((uint32_t)(exp + 15) << 10) + (uint32_t)r;  // mantissa overflow carries into the exponent
+    return sign | (uint16_t)bits;
+}
+
+template <typename T> int upload(T **dst, const std::vector<T> &src) {
+    *dst = nullptr;
+    if (src.empty()) return TQ_OK;
+    hipError_t e = hipMalloc((void **)dst, src.size() * sizeof(T));
+    if (e != hipSuccess) {
+        tq_set_error("hipMalloc(%zu): %s", src.size() * sizeof(T), hipGetErrorString(e));
+        return TQ_ERR_HIP;
+    }
+    e = hipMemcpy(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        tq_set_error("hipMemcpy: %s", hipGetErrorString(e));
+        return TQ_ERR_HIP;
+    }
+    return TQ_OK;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+bool fast_ok(const tq_handle *h) { return h->d == 128 && h->rotation == TQ_ROT_WHT && h->s1_32; }
+
+}  // namespace
+
+void tq_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int tq_check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        tq_set_error("%s: %s", what, hipGetErrorString(e));
+        return TQ_ERR_HIP;
+    }
+    return TQ_OK;
+}
+
+extern "C" {
+
+int tq_version(void) { return 100; }
+
+const char *tq_last_error(void) { return g_err; }
+
+int tq_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int tq_create(tq_handle **out, const tq_config *cfg) {
+    if (!out || !cfg || !cfg->centroids) {
+        tq_set_error("tq_create: null argument");
+        return TQ_ERR_ARG;
+    }
+    *out = nullptr;
+    if (cfg->d < 1 || cfg->d > TQ_MAX_D) {
+        tq_set_error("tq_create: d must be in 1..%d (got %d)", TQ_MAX_D, cfg->d);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    if (cfg->bits < 1 || cfg->bits > 8) {
+        tq_set_error("tq_create: bits must be in 1..8 (got %d)", cfg->bits);
+        return TQ_ERR_ARG;
+    }
+    if (cfg->rotation == TQ_ROT_DENSE ? !cfg->rotation_matrix : (cfg->rotation != TQ_ROT_WHT || !cfg->signs1 || !cfg->signs2)) {
+        tq_set_error("tq_create: rotation tables missing for mode %d", cfg->rotation);
+        return TQ_ERR_ARG;
+    }
+    if (tq_device_count() < 1) {
+        tq_set_error("tq_create: no HIP device visible");
+        return TQ_ERR_HIP;
+    }
+    tq_handle *h = new tq_handle();
+    memset(h, 0, sizeof(*h));
+    h->d = cfg->d;
+    h->pd = tq_padded_dim(cfg->d);
+    h->bits = cfg->bits;
+    h->n_centroids = 1 << cfg->bits;
+    h->rotation = cfg->rotation;
+    h->norm_correction = cfg->norm_correction;
+    h->proj_scale = cfg->projection_scale;
+    h->has_proj = cfg->projection != nullptr;
+    (void)hipGetDevice(&h->device);
+
+    const int d = h->d, pd = h->pd, nc = h->n_centroids;
+    int rc = TQ_OK;
+    std::vector<double> cent(cfg->centroids, cfg->centroids + nc), bounds(nc - 1);
+    for (int k = 0; k + 1 < nc; ++k) bounds[k] = (cent[k] + cent[k + 1]) / 2.0;
+    rc = rc ? rc : upload(&h->centroids64, cent);
+    rc = rc ? rc : upload(&h->bounds64, bounds);
+    std::vector<double> s1, s2;
+    if (cfg->rotation == TQ_ROT_WHT) {
+        s1.assign(cfg->signs1, cfg->signs1 + pd);
+        s2.assign(cfg->signs2, cfg->signs2 + pd);
+        rc = rc ? rc : upload(&h->s1_64, s1);
+        rc = rc ? rc : upload(&h->s2_64, s2);
+    } else {
+        std::vector<double> m(cfg->rotation_matrix, cfg->rotation_matrix + (size_t)d * d), mt((size_t)d * d);
+        for (int i = 0; i < d; ++i)
+            for (int j = 0; j < d; ++j) mt[(size_t)j * d + i] = m[(size_t)i * d + j];
+        rc = rc ? rc : upload(&h->rot64, m);
+        rc = rc ? rc : upload(&h->rot64_t, mt);
+    }
+    std::vector<double> S;
+    if (cfg->projection) {
+        S.assign(cfg->projection, cfg->projection + (size_t)d * d);
+        std::vector<double> st((size_t)d * d);
+        for (int i = 0; i < d; ++i)
+            for (int j = 0; j < d; ++j) st[(size_t)j * d + i] = S[(size_t)i * d + j];
+        rc = rc ? rc : upload(&h->proj64, S);
+        rc = rc ? rc : upload(&h->proj64_t, st);
+    }
+    if (d == 128 && cfg->rotation == TQ_ROT_WHT && cfg->bits <= 4) {
+        std::vector<float> c32(cent.begin(), cent.end()), b32(bounds.begin(), bounds.end());
+        std::vector<float> s1f(s1.begin(), s1.end()), s2f(s2.begin(), s2.end());
+        rc = rc ? rc : upload(&h->centroids32, c32);
+        rc = rc ? rc : upload(&h->bounds32, b32);
+        rc = rc ? rc : upload(&h->s1_32, s1f);
+        rc = rc ? rc : upload(&h->s2_32, s2f);
+        // pair LUT: entry (hi << bits | lo) = half2(c[lo], c[hi])
+        const int b = cfg->bits;
+        std::vector<uint32_t> lut((size_t)1 << (2 * b));
+        for (int hi = 0; hi < nc; ++hi)
+            for (int lo = 0; lo < nc; ++lo)
+                lut[(size_t)(hi << b) | lo] = (uint32_t)f64_to_f16_bits(cent[lo]) | ((uint32_t)f64_to_f16_bits(cent[hi]) << 16);
+        uint32_t *dl = nullptr;
+        rc = rc ? rc : upload(&dl, lut);
+        h->pair_lut = dl;
+        if (cfg->projection) {
+            // M = S R^T with R[k][m] = s2[k] H[k][m] s1[m] / sqrt(128); stored as [k*128+j] = M[j][k]
+            std::vector<double> mt((size_t)128 * 128);
+            std::vector<float> pT((size_t)128 * 128);
+            const double rs = 1.0 / std::sqrt(128.0);
+            for (int j = 0; j < 128; ++j)
+                for (int k = 0; k < 128; ++k) {
+                    double acc = 0.0;
+                    for (int m = 0; m < 128; ++m) {
+                        const double hkm = (__builtin_popcount(k & m) & 1) ? -1.0 : 1.0;
+                        acc += S[(size_t)j * 128 + m] * (s2[k] * hkm * s1[m]);
+                    }
+                    mt[(size_t)k * 128 + j] = acc * rs;
+                    pT[(size_t)k * 128 + j] = (float)S[(size_t)j * 128 + k];
+                }
+            rc = rc ? rc : upload(&h->projrot64_t, mt);
+            rc = rc ? rc : upload(&h->projT32, pT);
+        }
+    }
+    if (rc) {
+        tq_destroy(h);
+        return rc;
+    }
+    *out = h;
+    return TQ_OK;
+}
+
+void tq_destroy(tq_handle *h) {
+    if (!h) return;
+    void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
+                    h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    delete h;
+}
+
+#define REQUIRE(cond, code, ...)      \
+    do {                              \
+        if (!(cond)) {                \
+            tq_set_error(__VA_ARGS__); \
+            return code;              \
+        }                             \
+    } while (0)
+
+int tq_fwht(const void *x, void *y, int64_t n, int32_t len, int in_dtype, int out_dtype, void *stream) {
+    REQUIRE(n >= 0 && (n == 0 || (x && y)), TQ_ERR_ARG, "tq_fwht: bad argument");
+    REQUIRE(len >= 1 && (len & (len - 1)) == 0, TQ_ERR_ARG, "Input length must be a positive power of 2, got %d", len);
+    REQUIRE(len <= TQ_MAX_D, TQ_ERR_UNSUPPORTED, "tq_fwht: length %d > %d", len, TQ_MAX_D);
+    if (n == 0) return TQ_OK;
+    return tqk_fwht(x, y, n, len, in_dtype, out_dtype, (hipStream_t)stream);
+}
+
+int tq_rotate(const tq_handle *h, const void *x, void *y, int64_t n, int in_dtype, int out_dtype, int transpose,
+              void *stream) {
+    REQUIRE(h && n >= 0 && (n == 0 || (x && y)), TQ_ERR_ARG, "tq_rotate: bad argument");
+    if (n == 0) return TQ_OK;
+    if (fast_ok(h) && in_dtype != TQ_F64 && out_dtype != TQ_F64)
+        return tqk_rotate128(h, x, y, n, in_dtype, out_dtype, transpose, (hipStream_t)stream);
+    return tqk_rotate64(h, x, y, n, in_dtype, out_dtype, transpose, (hipStream_t)stream);
+}
+
+int tq_nearest_centroid(const double *values, int64_t n, const double *centroids_host, int32_t n_centroids,
+                        int32_t *idx, void *stream) {
+    REQUIRE(values && centroids_host && idx && n >= 0, TQ_ERR_ARG, "tq_nearest_centroid: bad argument");
+    REQUIRE(n_centroids >= 1 && n_centroids <= 256, TQ_ERR_UNSUPPORTED, "tq_nearest_centroid: %d centroids (max 256)",
+            n_centroids);
+    if (n == 0) return TQ_OK;
+    double bounds[255];
+    for (int k = 0; k + 1 < n_centroids; ++k) bounds[k] = (centroids_host[k] + centroids_host[k + 1]) / 2.0;
+    return tqk_nearest(values, n, bounds, n_centroids - 1, idx, (hipStream_t)stream);
+}
+
+int tq_quantize_indices(const tq_handle *h, const void *x, int64_t n, int in_dtype, uint8_t *idx, double *norms,
+                        double *rotated, void *stream) {
+    REQUIRE(h && x && idx && norms && n >= 0, TQ_ERR_ARG, "tq_quantize_indices: bad argument");
+    if (n == 0) return TQ_OK;
+    return tqk_quantize_indices(h, x, n, in_dtype, idx, norms, rotated, (hipStream_t)stream);
+}
+
+int tq_dequantize_indices(const tq_handle *h, const uint8_t *idx, const double *norms, int64_t n, double *out,
+                          const void *x, int x_dtype, double *residual, void *stream) {
+    REQUIRE(h && idx && norms && out && n >= 0, TQ_ERR_ARG, "tq_dequantize_indices: bad argument");
+    REQUIRE(!residual || x, TQ_ERR_ARG, "tq_dequantize_indices: residual needs x");
+    if (n == 0) return TQ_OK;
+    return tqk_dequantize_indices(h, idx, norms, n, out, x, x_dtype, residual, (hipStream_t)stream);
+}
+
+int tq_qjl_quantize(const tq_handle *h, const void *r, int64_t n, int in_dtype, int8_t *signs, double *norms,
+                    void *stream) {
+    REQUIRE(h && r && signs && norms && n >= 0, TQ_ERR_ARG, "tq_qjl_quantize: bad argument");
+    REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_qjl_quantize: handle has no projection");
+    if (n == 0) return TQ_OK;
+    return tqk_qjl_quantize(h, r, n, in_dtype, signs, norms, (hipStream_t)stream);
+}
+
+int tq_qjl_dequantize(const tq_handle *h, const int8_t *signs, const double *norms, double shrinkage, int64_t n,
+                      double *out, void *stream) {
+    REQUIRE(h && signs && norms && out && n >= 0, TQ_ERR_ARG, "tq_qjl_dequantize: bad argument");
+    REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_qjl_dequantize: handle has no projection");
+    if (n == 0) return TQ_OK;
+    return tqk_qjl_dequantize(h, signs, norms, shrinkage, n, out, (hipStream_t)stream);
+}
+
+int tq_pack_bits(const int8_t *signs, int64_t n, int32_t d, uint8_t *packed, void *stream) {
+    REQUIRE(signs && packed && n >= 0 && d >= 1, TQ_ERR_ARG, "tq_pack_bits: bad argument");
+    if (n == 0) return TQ_OK;
+    return tqk_pack_bits(signs, n, d, packed, (hipStream_t)stream);
+}
+
+int tq_unpack_bits(const uint8_t *packed, int64_t n, int32_t d, int8_t *signs, void *stream) {
+    REQUIRE(signs && packed && n >= 0 && d >= 1, TQ_ERR_ARG, "tq_unpack_bits: bad argument");
+    if (n == 0) return TQ_OK;
+    return tqk_unpack_bits(packed, n, d, signs, (hipStream_t)stream);
+}
+
+int tq_pack_indices(const uint8_t *idx, int64_t count, int32_t bits, uint8_t *packed, void *stream) {
+    REQUIRE(bits >= 1 && bits <= 8, TQ_ERR_ARG, "bit_width must be 1-8, got %d", bits);
+    REQUIRE(idx && packed && count >= 0, TQ_ERR_ARG, "tq_pack_indices: bad argument");
+    if (count == 0) return TQ_OK;
+    return tqk_pack_indices(idx, count, bits, packed, (hipStream_t)stream);
+}
+
+int64_t tq_packed_bytes(int32_t bits, int64_t n_seqs, int64_t tokens) {
+    if (bits < 2 || bits > 4 || n_seqs < 0 || tokens < 0) return -1;
+    return n_seqs * ((tokens + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK) * (int64_t)(TQ_ROWS_PER_BLOCK * (16 * bits + 2));
+}
+
+int64_t tq_q8_0_bytes(int64_t n_seqs, int64_t tokens) {
+    if (n_seqs < 0 || tokens < 0) return -1;
+    return n_seqs * ((tokens + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK) * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
+}
+
+static int check_fast(const tq_handle *h, const char *who) {
+    REQUIRE(h, TQ_ERR_ARG, "%s: null handle", who);
+    REQUIRE(fast_ok(h), TQ_ERR_UNSUPPORTED, "%s: needs d == 128 and WHT rotation (handle has d=%d, rotation=%d)", who,
+            h->d, h->rotation);
+    REQUIRE(h->bits >= 2 && h->bits <= 4, TQ_ERR_UNSUPPORTED, "%s: bits must be 2, 3 or 4 (got %d)", who, h->bits);
+    return TQ_OK;
+}
+
+int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
+             void *stream) {
+    int rc = check_fast(h, "tq_store");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_store: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(x && packed, TQ_ERR_ARG, "tq_store: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_store: bad kind %d", kind);
+    REQUIRE(aligned16(x) && aligned16(packed), TQ_ERR_ALIGN, "tq_store: x and packed must be 16-byte aligned");
+    return tqk_store(h, x, n_seqs, tokens, in_dtype, kind, packed, nullptr, nullptr, (hipStream_t)stream);
+}
+
+int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed,
+                 uint8_t *sign_bits, void *rnorms_f16, void *stream) {
+    int rc = check_fast(h, "tq_store_qjl");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_store_qjl: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(x && packed && sign_bits && rnorms_f16, TQ_ERR_ARG, "tq_store_qjl: null pointer");
+    REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_store_qjl: handle has no projection");
+    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_store_qjl: packed must be 16-byte aligned");
+    return tqk_store(h, x, n_seqs, tokens, in_dtype, TQ_KIND_K, packed, sign_bits, rnorms_f16, (hipStream_t)stream);
+}
+
+int tq_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out, int out_dtype,
+            int domain, void *stream) {
+    int rc = check_fast(h, "tq_load");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_load: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(out && packed, TQ_ERR_ARG, "tq_load: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_load: bad kind %d", kind);
+    REQUIRE(domain == TQ_DOMAIN_ROTATED || domain == TQ_DOMAIN_ORIGINAL, TQ_ERR_ARG, "tq_load: bad domain %d", domain);
+    REQUIRE(aligned16(out) && aligned16(packed), TQ_ERR_ALIGN, "tq_load: out and packed must be 16-byte aligned");
+    return tqk_load(h, packed, n_seqs, tokens, kind, out, out_dtype, domain, (hipStream_t)stream);
+}
+
+int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
+                    float *norms, void *stream) {
+    int rc = check_fast(h, "tq_unpack_codes");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_unpack_codes: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(idx && norms && packed, TQ_ERR_ARG, "tq_unpack_codes: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_unpack_codes: bad kind %d", kind);
+    return tqk_unpack_codes(h, packed, n_seqs, tokens, kind, idx, norms, (hipStream_t)stream);
+}
+
+int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream) {
+    REQUIRE(x && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_store: bad argument");
+    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_store: packed must be 16-byte aligned");
+    return tqk_q8_0_store(x, n_seqs, tokens, in_dtype, packed, (hipStream_t)stream);
+}
+
+int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream) {
+    REQUIRE(q && scales && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_unpack: bad argument");
+    return tqk_q8_0_unpack(packed, n_seqs, tokens, q, scales, (hipStream_t)stream);
+}
+
+static int check_attn(const tq_attn_params *p) {
+    REQUIRE(p, TQ_ERR_ARG, "attention: null params");
+    REQUIRE(p->batch >= 1 && p->n_q_heads >= 1 && p->n_kv_heads >= 1 && p->tokens >= 1 && p->n_splits >= 1, TQ_ERR_ARG,
+            "attention: sizes must be positive");
+    REQUIRE(p->n_q_heads == 4 * p->n_kv_heads, TQ_ERR_UNSUPPORTED,
+            "attention: GQA group must be 4 query heads per KV head (got %d / %d)", p->n_q_heads, p->n_kv_heads);
+    REQUIRE(p->k_format == TQ_KFMT_TURBO || p->k_format == TQ_KFMT_Q8_0, TQ_ERR_ARG, "attention: bad k_format %d",
+            p->k_format);
+    REQUIRE(p->tokens < ((int64_t)1 << 36), TQ_ERR_UNSUPPORTED, "attention: context too long");
+    REQUIRE(p->sparse_v_tau >= 0.0f, TQ_ERR_ARG, "attention: sparse_v_tau must be >= 0");
+    return TQ_OK;
+}
+
+int64_t tq_attn_workspace_bytes(const tq_attn_params *p) {
+    if (check_attn(p)) return -1;
+    return tqk_attn_workspace_bytes(p);
+}
+
+int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q, int q_dtype,
+                        const void *k, const void *k_aux, const void *v, const float *bias, float *out,
+                        unsigned long long *skip_count, void *workspace, int64_t workspace_bytes, void *stream) {
+    int rc = check_attn(p);
+    if (rc) return rc;
+    rc = check_fast(hv, "tq_decode_attention (V)");
+    if (rc) return rc;
+    if (p->k_format == TQ_KFMT_TURBO) {
+        rc = check_fast(hk, "tq_decode_attention (K)");
+        if (rc) return rc;
+    }
+    REQUIRE(q && k && v && out && workspace, TQ_ERR_ARG, "tq_decode_attention: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v) && aligned16(workspace), TQ_ERR_ALIGN,
+            "tq_decode_attention: k, v and workspace must be 16-byte aligned");
+    return tqk_decode_attention(hk, hv, p, q, q_dtype, k, k_aux, v, bias, out, skip_count, workspace, workspace_bytes,
+                                (hipStream_t)stream);
+}
+
+int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
+                  const uint8_t *sign_bits, const void *rnorms_f16, int64_t nk, void *logits, int out_dtype,
+                  void *workspace, int64_t workspace_bytes, void *stream) {
+    int rc = check_fast(h, "tq_score_tile");
+    if (rc) return rc;
+    REQUIRE(q && packed && sign_bits && rnorms_f16 && logits && workspace && nq >= 0 && nk >= 0, TQ_ERR_ARG,
+            "tq_score_tile: bad argument");
+    REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_score_tile: handle has no projection");
+    REQUIRE(out_dtype == TQ_F32 || out_dtype == TQ_F16, TQ_ERR_ARG, "tq_score_tile: logits must be fp32 or fp16");
+    REQUIRE(workspace_bytes >= nq * 256 * 2, TQ_ERR_ARG, "tq_score_tile: workspace %lld < %lld bytes",
+            (long long)workspace_bytes, (long long)(nq * 256 * 2));
+    REQUIRE(aligned16(packed) && aligned16(workspace) && aligned16(logits), TQ_ERR_ALIGN,
+            "tq_score_tile: packed, workspace and logits must be 16-byte aligned");
+    if (nq == 0 || nk == 0) return TQ_OK;
+    return tqk_score_tile(h, q, q_dtype, nq, packed, sign_bits, rnorms_f16, nk, logits, out_dtype, workspace,
+                          workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

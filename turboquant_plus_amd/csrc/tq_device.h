@@ -1,0 +1,168 @@
+// Device-side helpers: cross-lane exchanges for wave64, Walsh-Hadamard
+// butterflies, and the packed "pair container" row format.
+#pragma once
+#include "tq_internal.h"
+
+namespace tqd {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// ---- cross-lane exchange ------------------------------------------------------
+// DPP control words (GCN3+/CDNA): quad_perm = 4 x 2-bit selectors, 0x12n =
+// row_ror:n, 0x141 = row_half_mirror.  Every pattern used here reads a valid
+// lane, so bound_ctrl / old are irrelevant.
+template <int CTRL> __device__ inline float dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> __device__ inline double dpp(double v) {
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, 0xF, 0xF, true);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xF, 0xF, true);
+    return __builtin_bit_cast(double, ((long long)hi << 32) | (unsigned)lo);
+}
+
+// value held by lane (lane ^ M); M in {1,2,4,8,16,32}
+template <int M, typename T> __device__ inline T xor_lane(T v) {
+    if constexpr (M == 1) return dpp<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (M == 4) return dpp<0x1B>(dpp<0x141>(v));  // half-mirror (^7) then quad reverse (^3)
+    else if constexpr (M == 8) return dpp<0x128>(v);  // row_ror:8
+    else if constexpr (M == 16) {
+        if constexpr (sizeof(T) == 4) {
+            return __builtin_bit_cast(T, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+        } else {
+            const long long b = __builtin_bit_cast(long long, v);
+            const int lo = __builtin_amdgcn_ds_swizzle((int)(b & 0xffffffffll), 0x401F);
+            const int hi = __builtin_amdgcn_ds_swizzle((int)(b >> 32), 0x401F);
+            return __builtin_bit_cast(T, ((long long)hi << 32) | (unsigned)lo);
+        }
+    } else {
+        static_assert(M == 32, "unsupported xor mask");
+        if constexpr (sizeof(T) == 4) {
+            const unsigned u = __builtin_bit_cast(unsigned, v);
+            // r[0] = lanes 0..31 duplicated into both halves, r[1] = lanes 32..63 duplicated
+            auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            const unsigned o = (__lane_id() < 32) ? r[1] : r[0];
+            return __builtin_bit_cast(T, o);
+        } else {
+            return __shfl_xor(v, 32);
+        }
+    }
+}
+
+// sum over the 16 lanes of a DPP row (result in every lane of the row)
+template <typename T> __device__ inline T row16_sum(T v) {
+    v += xor_lane<1>(v);
+    v += xor_lane<2>(v);
+    v += dpp<0x124>(v);  // row_ror:4
+    v += dpp<0x128>(v);  // row_ror:8
+    return v;
+}
+
+// ---- Walsh-Hadamard butterflies ------------------------------------------------
+// One cross-lane stage: lanes with bit M clear get own+partner, lanes with it
+// set get partner-own.  `sgn` is +1 / -1 accordingly (precomputed per lane).
+template <int M, typename T> __device__ inline T bfly(T v, T sgn) { return fma(sgn, v, xor_lane<M>(v)); }
+
+// 8 values per lane, 16 lanes per vector: element index e = 8*(lane&15) + m.
+// Unnormalised natural-order WHT of the 128 values held by a 16-lane row.
+template <typename T> __device__ inline void wht128_row16(T (&x)[8], int lane) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            if ((m & h) == 0) {
+                const T a = x[m], b = x[m + h];
+                x[m] = a + b;
+                x[m + h] = a - b;
+            }
+        }
+    }
+    const T s1 = (lane & 1) ? T(-1) : T(1), s2 = (lane & 2) ? T(-1) : T(1);
+    const T s4 = (lane & 4) ? T(-1) : T(1), s8 = (lane & 8) ? T(-1) : T(1);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) x[m] = bfly<1>(x[m], s1);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) x[m] = bfly<2>(x[m], s2);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) x[m] = bfly<4>(x[m], s4);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) x[m] = bfly<8>(x[m], s8);
+}
+
+// 2 values per lane, one 64-lane wavefront per vector: lane holds elements
+// (2*lane, 2*lane+1).  Stage h=1 is in-lane, h=2..64 are lane xor 1..32.
+__device__ inline void wht128_wave(float &a, float &b, int lane) {
+    const float t = a + b;
+    b = a - b;
+    a = t;
+#define TQ_STAGE(M)                                           \
+    {                                                         \
+        const float sg = (lane & M) ? -1.0f : 1.0f;           \
+        a = bfly<M>(a, sg);                                   \
+        b = bfly<M>(b, sg);                                   \
+    }
+    TQ_STAGE(1) TQ_STAGE(2) TQ_STAGE(4) TQ_STAGE(8) TQ_STAGE(16) TQ_STAGE(32)
+#undef TQ_STAGE
+}
+
+// ---- packed rows ----------------------------------------------------------------
+// A row holds 64 pair codes (128 values) in 4*BITS dwords; pair = lo | hi << BITS.
+//   BITS 4: pair p = byte p%4 of dword p/4
+//   BITS 2: pair p = nibble p%8 of dword p/8
+//   BITS 3: pairs 0..59 five to a dword at bit 6*(p%5); pair 60+t = bits 30..31 of
+//           dwords 3t, 3t+1, 3t+2 (low, middle, high two bits)
+// A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
+// norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows: row r = token
+// quad r/4, sub-row i = r%4; pair 2g+h = dim 4g+i of tokens 4*(r/4)+2h, +2h+1.
+__host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
+__host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
+__host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
+
+// byte offset (pair code * 4) into a 4-byte-entry LUT, P compile-time
+template <int BITS, int P> __device__ inline uint32_t pair_lut_offset(const uint32_t (&w)[4 * BITS]) {
+    if constexpr (BITS == 4) {
+        constexpr int q = P / 4, k = P % 4;
+        if constexpr (k == 0) return (w[q] << 2) & 0x3FCu;
+        else return (w[q] >> (8 * k - 2)) & 0x3FCu;
+    } else if constexpr (BITS == 2) {
+        constexpr int q = P / 8, k = P % 8;
+        if constexpr (k == 0) return (w[q] << 2) & 0x3Cu;
+        else return (w[q] >> (4 * k - 2)) & 0x3Cu;
+    } else {
+        static_assert(BITS == 3, "bits");
+        if constexpr (P < 60) {
+            constexpr int q = P / 5, k = P % 5;
+            if constexpr (k == 0) return (w[q] << 2) & 0xFCu;
+            else return (w[q] >> (6 * k - 2)) & 0xFCu;
+        } else {
+            constexpr int t = P - 60;
+            return ((w[3 * t] >> 28) & 0xCu) | ((w[3 * t + 1] >> 26) & 0x30u) | ((w[3 * t + 2] >> 24) & 0xC0u);
+        }
+    }
+}
+
+// runtime pair extraction (slow path: unpack / load kernels)
+__device__ inline uint32_t pair_code(const uint32_t *w, int bits, int p) {
+    if (bits == 4) return (w[p >> 2] >> (8 * (p & 3))) & 0xFFu;
+    if (bits == 2) return (w[p >> 3] >> (4 * (p & 7))) & 0xFu;
+    if (p < 60) return (w[p / 5] >> (6 * (p % 5))) & 0x3Fu;
+    const int t = p - 60;
+    return (w[3 * t] >> 30) | ((w[3 * t + 1] >> 30) << 2) | ((w[3 * t + 2] >> 30) << 4);
+}
+
+// (row, pair, half) of the code of (token, dim) inside its 128-token block
+__device__ inline void locate(int kind, int token, int dim, int &row, int &pair, int &half) {
+    if (kind == TQ_KIND_K) {
+        row = token;
+        pair = dim >> 1;
+        half = dim & 1;
+    } else {
+        row = (token & ~3) | (dim & 3);
+        pair = 2 * (dim >> 2) + ((token & 3) >> 1);
+        half = token & 1;
+    }
+}
+
+}  // namespace tqd

@@ -1,0 +1,78 @@
+// Internal declarations shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include "tq.h"
+
+#define TQ_MAX_D 1024
+#define TQ_ROWS_PER_BLOCK 128
+
+// Device-resident constant tables of a quantiser.  Everything the kernels read
+// through this struct is written once in tq_create.
+struct tq_handle {
+    int d, pd, bits, n_centroids, rotation, norm_correction;
+    int device;
+    // float64 tables (reference-API kernels)
+    double *centroids64;   // [n_centroids]
+    double *bounds64;      // [n_centroids-1] midpoints
+    double *s1_64, *s2_64; // [pd] (WHT)
+    double *rot64;         // [d*d]  Pi,   row-major          (dense)
+    double *rot64_t;       // [d*d]  Pi^T, row-major          (dense)
+    double *proj64;        // [d*d]  S
+    double *proj64_t;      // [d*d]  S^T
+    double proj_scale;
+    int has_proj;
+    // float32 tables (production kernels, d == 128, WHT)
+    float *centroids32;    // [n_centroids]
+    float *bounds32;       // [n_centroids-1]
+    float *s1_32, *s2_32;  // [128]
+    double *projrot64_t;   // [128*128] entry [k*128+j] = (S R^T)[j][k]   (d == 128, WHT, projection)
+    void *pair_lut;        // [4^bits] half2: (c[lo], c[hi]) for a pair code (bits <= 3), or [256] for 4
+    float *projT32;        // [128*128] entry [k*128+j] = S[j][k]  (query projection, score tile)
+};
+
+static inline int tq_padded_dim(int d) {
+    int p = 1;
+    while (p < d) p <<= 1;
+    return p;
+}
+
+// ---- launchers implemented in the kernel files -------------------------------
+int tqk_fwht(const void *x, void *y, int64_t n, int len, int in_dtype, int out_dtype, hipStream_t s);
+int tqk_rotate64(const tq_handle *h, const void *x, void *y, int64_t n, int in_dtype, int out_dtype, int transpose,
+                 hipStream_t s);
+int tqk_nearest(const double *values, int64_t n, const double *bounds_host, int nb, int32_t *idx, hipStream_t s);
+int tqk_quantize_indices(const tq_handle *h, const void *x, int64_t n, int in_dtype, uint8_t *idx, double *norms,
+                         double *rotated, hipStream_t s);
+int tqk_dequantize_indices(const tq_handle *h, const uint8_t *idx, const double *norms, int64_t n, double *out,
+                           const void *x, int x_dtype, double *residual, hipStream_t s);
+int tqk_qjl_quantize(const tq_handle *h, const void *r, int64_t n, int in_dtype, int8_t *signs, double *norms,
+                     hipStream_t s);
+int tqk_qjl_dequantize(const tq_handle *h, const int8_t *signs, const double *norms, double shrinkage, int64_t n,
+                       double *out, hipStream_t s);
+int tqk_pack_bits(const int8_t *signs, int64_t n, int d, uint8_t *packed, hipStream_t s);
+int tqk_unpack_bits(const uint8_t *packed, int64_t n, int d, int8_t *signs, hipStream_t s);
+int tqk_pack_indices(const uint8_t *idx, int64_t count, int bits, uint8_t *packed, hipStream_t s);
+
+int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_dtype, int out_dtype, int transpose,
+                  hipStream_t s);
+int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
+              uint8_t *sign_bits, void *rnorms, hipStream_t s);
+int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
+             int out_dtype, int domain, hipStream_t s);
+int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
+                     float *norms, hipStream_t s);
+int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
+int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, hipStream_t s);
+
+int64_t tqk_attn_workspace_bytes(const tq_attn_params *p);
+int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q, int q_dtype,
+                         const void *k, const void *k_aux, const void *v, const float *bias, float *out,
+                         unsigned long long *skip_count, void *ws, int64_t ws_bytes, hipStream_t s);
+int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
+                   const uint8_t *sign_bits, const void *rnorms, int64_t nk, void *logits, int out_dtype, void *ws,
+                   int64_t ws_bytes, hipStream_t s);
+
+void tq_set_error(const char *fmt, ...);
+int tq_check_launch(const char *what);

@@ -1,0 +1,547 @@
+// Production-format kernels (d = 128, sign-diagonal WHT rotation, fp32
+// arithmetic, corrected fp16 norm, 128-token blocks of packed pair codes).
+//
+//   k_wht128       one 64-lane wavefront per vector, two values per lane, the
+//                  seven butterfly stages in registers (one in-lane, six through
+//                  DPP / ds_swizzle / permlane32 exchanges).
+//   k_store        norm -> D2 H D1 -> nearest centroid -> corrected norm -> pack.
+//                  16 lanes per vector (8 values each): three in-lane stages and
+//                  four DPP row stages; a workgroup owns one 128-token block,
+//                  stages the codes in LDS and writes the block coalesced.
+//   k_store_qjl    float64 variant that also sketches the residual (1-bit QJL).
+//   k_load         packed block -> values (rotated or original domain).
+//   k_unpack_codes packed block -> uint8 indices + fp32 norms.
+//   k_q8_0_store   32-value int8 blocks with fp16 scale, 128-token block layout.
+#include "tq_device.h"
+#include "tq_device64.h"
+
+namespace {
+
+using namespace tqd;
+
+constexpr float RSQRT128 = 0.08838834764831845f;
+constexpr int CODE_STRIDE = 136;  // bytes per token in the LDS code stage (8-byte aligned, odd multiple of 8)
+
+// ---- typed 8-value loads / stores ---------------------------------------------
+template <typename T> __device__ inline void load8(const T *p, float (&v)[8]);
+template <> __device__ inline void load8<__half>(const __half *p, float (&v)[8]) {
+    const uint4 u = *reinterpret_cast<const uint4 *>(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __half2float(__ushort_as_half((unsigned short)(w[i] & 0xffffu)));
+        v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(w[i] >> 16)));
+    }
+}
+template <> __device__ inline void load8<float>(const float *p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float4 b = *reinterpret_cast<const float4 *>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <> __device__ inline void load8<double>(const double *p, float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)p[i];
+}
+template <typename T> __device__ inline void store8(T *p, const float (&v)[8]);
+template <> __device__ inline void store8<__half>(__half *p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        w[i] = (uint32_t)__half_as_ushort(__float2half_rn(v[2 * i])) |
+               ((uint32_t)__half_as_ushort(__float2half_rn(v[2 * i + 1])) << 16);
+    *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+template <> __device__ inline void store8<float>(float *p, const float (&v)[8]) {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+template <> __device__ inline void store8<double>(double *p, const float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = (double)v[i];
+}
+template <typename T> __device__ inline float ld1(const T *p) { return (float)*p; }
+template <> __device__ inline float ld1<__half>(const __half *p) { return __half2float(*p); }
+template <typename T> __device__ inline void st1(T *p, float v) { *p = (T)v; }
+template <> __device__ inline void st1<__half>(__half *p, float v) { *p = __float2half_rn(v); }
+
+// ---- K1: standalone rotation, one wavefront per vector -------------------------
+// y = sb * H(sa * x) / sqrt(128) with (sa, sb) = (s1, s2) forward, (s2, s1) transposed.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void k_wht128(const TI *x, TO *y, int64_t n, const float *sa, const float *sb) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    const float a0 = sa[2 * lane], a1 = sa[2 * lane + 1];
+    const float b0 = sb[2 * lane] * RSQRT128, b1 = sb[2 * lane + 1] * RSQRT128;
+    for (int64_t v = wave0; v < n; v += nwaves) {
+        float a = ld1(x + v * 128 + 2 * lane) * a0;
+        float b = ld1(x + v * 128 + 2 * lane + 1) * a1;
+        wht128_wave(a, b, lane);
+        st1(y + v * 128 + 2 * lane, a * b0);
+        st1(y + v * 128 + 2 * lane + 1, b * b1);
+    }
+}
+
+// ---- block packer ----------------------------------------------------------------
+// codes: LDS bytes [128 tokens][CODE_STRIDE]; norms: LDS float [128]; out: one block.
+template <int BITS> __device__ inline uint32_t pair_from_stage(const uint8_t *codes, int kind, int row, int p) {
+    uint32_t lo, hi;
+    if (kind == TQ_KIND_K) {
+        lo = codes[row * CODE_STRIDE + 2 * p];
+        hi = codes[row * CODE_STRIDE + 2 * p + 1];
+    } else {
+        const int tok = (row & ~3) + 2 * (p & 1);
+        const int dim = 4 * (p >> 1) + (row & 3);
+        lo = codes[tok * CODE_STRIDE + dim];
+        hi = codes[(tok + 1) * CODE_STRIDE + dim];
+    }
+    return lo | (hi << BITS);
+}
+
+template <int BITS, int NTHREADS>
+__device__ inline void pack_block(const uint8_t *codes, const float *norms, uint8_t *out_block, int kind) {
+    uint32_t *out = reinterpret_cast<uint32_t *>(out_block);
+    constexpr int NDW = TQ_ROWS_PER_BLOCK * 4 * BITS;
+    for (int o = threadIdx.x; o < NDW; o += NTHREADS) {
+        const int c = o >> 9, r = (o & 511) >> 2, k = o & 3;
+        const int q = 4 * c + k;
+        uint32_t word = 0;
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) word |= pair_from_stage<4>(codes, kind, r, 4 * q + t) << (8 * t);
+        } else if constexpr (BITS == 2) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) word |= pair_from_stage<2>(codes, kind, r, 8 * q + t) << (4 * t);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 5; ++t) word |= pair_from_stage<3>(codes, kind, r, 5 * q + t) << (6 * t);
+            const uint32_t tail = pair_from_stage<3>(codes, kind, r, 60 + q / 3);
+            word |= ((tail >> (2 * (q % 3))) & 3u) << 30;
+        }
+        out[o] = word;
+    }
+    for (int t = threadIdx.x; t < 64; t += NTHREADS) {
+        const uint32_t lo = __half_as_ushort(__float2half_rn(norms[2 * t]));
+        const uint32_t hi = __half_as_ushort(__float2half_rn(norms[2 * t + 1]));
+        out[NDW + t] = lo | (hi << 16);
+    }
+}
+
+struct StoreArgs {
+    const float *s1, *s2, *bounds, *cent;
+    int kind, norm_correction;
+    int64_t tokens;       // per sequence
+    int64_t blocks_per_seq;
+};
+
+// ---- K2: fused quantise + pack ---------------------------------------------------
+template <int BITS, typename TI>
+__global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, StoreArgs a) {
+    constexpr int NB = (1 << BITS) - 1;
+    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
+    __shared__ float csq_s[1 << BITS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int li = lane & 15, grp = tid >> 4;
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+
+    float bnd[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) bnd[k] = a.bounds[k];
+    if (tid < (1 << BITS)) {
+        const float c = a.cent[tid];
+        csq_s[tid] = c * c;
+    }
+    float s1v[8], s2v[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        s1v[m] = a.s1[8 * li + m];
+        s2v[m] = a.s2[8 * li + m] * RSQRT128;
+    }
+    __syncthreads();
+
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
+        const bool valid = tok0 + t < a.tokens;
+        float xv[8];
+        if (valid) {
+            load8(x + ((seq * a.tokens + tok0 + t) * 128 + 8 * li), xv);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) xv[m] = 0.0f;
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) ss = fmaf(xv[m], xv[m], ss);
+        ss = row16_sum(ss);
+        const float norm = sqrtf(ss);
+        const float inv = norm > 0.0f ? 1.0f / norm : 1.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) xv[m] *= s1v[m];
+        wht128_row16(xv, lane);
+        uint32_t w0 = 0, w1 = 0;
+        float cs = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const float yv = (xv[m] * s2v[m]) * inv;
+            uint32_t c = 0;
+#pragma unroll
+            for (int k = 0; k < NB; ++k) c += (bnd[k] < yv) ? 1u : 0u;
+            cs += csq_s[c];
+            if (m < 4) w0 |= c << (8 * m);
+            else w1 |= c << (8 * (m - 4));
+        }
+        cs = row16_sum(cs);
+        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(w0, w1);
+        if (li == 0) {
+            float g = norm;
+            if (a.norm_correction) {
+                const float cn = sqrtf(cs);
+                g = norm / (cn > 1e-10f ? cn : 1.0f);
+            }
+            norms_s[t] = g;
+        }
+    }
+    __syncthreads();
+    pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), a.kind);
+}
+
+// ---- K2 + K4 in float64: codes, corrected norm, residual sign sketch ---------------
+struct StoreQjlArgs {
+    const double *s1, *s2, *bounds, *cent;
+    const double *projrot_t;  // [128*128]: entry [k*128+j] = (S R^T)[j][k]
+    int norm_correction;
+    int64_t tokens, blocks_per_seq;
+};
+
+template <int BITS, typename TI>
+__global__ __launch_bounds__(128) void k_store_qjl(const TI *x, uint8_t *packed, uint8_t *sign_bits, __half *rnorms,
+                                                  StoreQjlArgs a) {
+    using namespace tq64;
+    constexpr int NB = (1 << BITS) - 1;
+    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
+    __shared__ double xs[VB * 128], ys[VB * 128];
+    __shared__ double nrm[VB], cn[VB], g16[VB];
+
+    const int tid = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const int64_t row0 = seq * a.tokens;  // first row of this sequence in x / sign_bits / rnorms
+
+    RotArgs rw;
+    rw.d = rw.pd = 128;
+    rw.mode = TQ_ROT_WHT;
+    rw.mat = nullptr;
+    rw.sa = a.s1;
+    rw.sb = a.s2;
+    RotArgs rp;
+    rp.d = rp.pd = 128;
+    rp.mode = TQ_ROT_DENSE;
+    rp.mat = a.projrot_t;
+    rp.sa = rp.sb = nullptr;
+
+    for (int sb = 0; sb < TQ_ROWS_PER_BLOCK / VB; ++sb) {
+        const int64_t t0 = tok0 + sb * VB;                // token index (in sequence) of staged vector 0
+        const int64_t nvalid = a.tokens - t0;             // vectors with v < nvalid exist
+        for (int i = tid; i < VB * 128; i += NT) {
+            const int v = i >> 7;
+            xs[i] = (v < nvalid) ? ldd(x, (row0 + t0 + v) * 128 + (i & 127)) : 0.0;
+        }
+        __syncthreads();
+        norms_block(xs, 128, 128, nrm);
+        for (int i = tid; i < VB * 128; i += NT) {
+            const double nv = nrm[i >> 7];
+            xs[i] = xs[i] / (nv > 0.0 ? nv : 1.0);
+        }
+        __syncthreads();
+        rotate_block(rw, xs, ys);  // ys = rotated unit vectors
+        for (int i = tid; i < VB * 128; i += NT) {
+            const int v = i >> 7, j = i & 127;
+            const double yv = ys[i];
+            int c = 0;
+#pragma unroll
+            for (int k = 0; k < NB; ++k) c += (a.bounds[k] < yv) ? 1 : 0;
+            codes[(sb * VB + v) * CODE_STRIDE + j] = (uint8_t)c;
+            xs[i] = a.cent[c];
+        }
+        __syncthreads();
+        norms_block(xs, 128, 128, cn);
+        if (tid < VB) {
+            double g = nrm[tid];
+            if (a.norm_correction) g = nrm[tid] / (cn[tid] > 1e-10 ? cn[tid] : 1.0);
+            const __half gh = double_to_half_rn(g);
+            g16[tid] = (double)__half2float(gh);
+            norms_s[sb * VB + tid] = __half2float(gh);
+        }
+        __syncthreads();
+        // residual in the rotated domain against the reconstruction the decoder will see
+        for (int i = tid; i < VB * 128; i += NT) {
+            const int v = i >> 7;
+            ys[i] = nrm[v] * ys[i] - g16[v] * xs[i];
+        }
+        __syncthreads();
+        norms_block(ys, 128, 128, cn);
+        if (tid < VB && tid < nvalid) rnorms[row0 + t0 + tid] = double_to_half_rn(cn[tid]);
+        rotate_block(rp, ys, xs);  // xs = (S R^T) e
+        for (int i = tid; i < VB * 16; i += NT) {
+            const int v = i >> 4, byte = i & 15;
+            if (v >= nvalid) continue;
+            unsigned bits = 0;
+#pragma unroll
+            for (int b = 0; b < 8; ++b) bits |= (xs[v * 128 + byte * 8 + b] >= 0.0 ? 1u : 0u) << b;
+            sign_bits[(row0 + t0 + v) * 16 + byte] = (uint8_t)bits;
+        }
+        __syncthreads();
+    }
+    pack_block<BITS, 128>(codes, norms_s, packed + blk * block_bytes(BITS), TQ_KIND_K);
+}
+
+// ---- K3: packed block -> values ----------------------------------------------------
+__device__ inline uint32_t row_dword(const uint8_t *block, int row, int q) {
+    return *reinterpret_cast<const uint32_t *>(block + (q >> 2) * 2048 + row * 16 + (q & 3) * 4);
+}
+
+__device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, int token, int dim) {
+    int row, p, half;
+    locate(kind, token, dim, row, p, half);
+    uint32_t pc;
+    if (bits == 4) pc = (row_dword(block, row, p >> 2) >> (8 * (p & 3))) & 0xFFu;
+    else if (bits == 2) pc = (row_dword(block, row, p >> 3) >> (4 * (p & 7))) & 0xFu;
+    else if (p < 60) pc = (row_dword(block, row, p / 5) >> (6 * (p % 5))) & 0x3Fu;
+    else {
+        const int t = p - 60;
+        pc = (row_dword(block, row, 3 * t) >> 30) | ((row_dword(block, row, 3 * t + 1) >> 30) << 2) |
+             ((row_dword(block, row, 3 * t + 2) >> 30) << 4);
+    }
+    return (pc >> (half * bits)) & ((1u << bits) - 1u);
+}
+
+__device__ inline float block_norm(const uint8_t *block, int bits, int token) {
+    const __half *nm = reinterpret_cast<const __half *>(block + block_code_bytes(bits));
+    return __half2float(nm[token]);
+}
+
+struct LoadArgs {
+    const float *s1, *s2, *cent;
+    int bits, kind, domain;
+    int64_t tokens, blocks_per_seq;
+};
+
+template <typename TO>
+__global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, LoadArgs a) {
+    __shared__ float cent_s[16];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int li = lane & 15, grp = tid >> 4;
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * (16 * a.bits + 2));
+    if (tid < (1 << a.bits)) cent_s[tid] = a.cent[tid];
+    float s1v[8], s2v[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        s1v[m] = a.s1[8 * li + m] * RSQRT128;
+        s2v[m] = a.s2[8 * li + m];
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
+        const bool valid = tok0 + t < a.tokens;
+        const float g = block_norm(block, a.bits, t);
+        float v[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) v[m] = cent_s[fetch_code(block, a.bits, a.kind, t, 8 * li + m)] * g;
+        if (a.domain == TQ_DOMAIN_ORIGINAL) {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) v[m] *= s2v[m];
+            wht128_row16(v, lane);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) v[m] *= s1v[m];
+        }
+        if (valid) store8(out + ((seq * a.tokens + tok0 + t) * 128 + 8 * li), v);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_unpack_codes(const uint8_t *packed, uint8_t *idx, float *norms, int bits,
+                                                      int kind, int64_t tokens, int64_t blocks_per_seq) {
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * (16 * bits + 2));
+    for (int e = threadIdx.x; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
+        const int t = e >> 7, dim = e & 127;
+        if (tok0 + t >= tokens) continue;
+        idx[(seq * tokens + tok0 + t) * 128 + dim] = (uint8_t)fetch_code(block, bits, kind, t, dim);
+    }
+    if (threadIdx.x < TQ_ROWS_PER_BLOCK && tok0 + threadIdx.x < tokens)
+        norms[seq * tokens + tok0 + threadIdx.x] = block_norm(block, bits, threadIdx.x);
+}
+
+// ---- q8_0-style K blocks ------------------------------------------------------------
+// Block of 128 tokens: [8 chunks][128 rows][16 B] int8 followed by [128][4] fp16 scales.
+// One thread per 32-value group: scale = max|x| / 127, q = roundf(x / scale) (ggml).
+template <typename TI>
+__global__ __launch_bounds__(256) void k_q8_0_store(const TI *x, uint8_t *packed, int64_t tokens, int64_t blocks_per_seq) {
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
+    for (int u = threadIdx.x; u < TQ_ROWS_PER_BLOCK * 4; u += 256) {
+        const int t = u >> 2, gq = u & 3;
+        const bool valid = tok0 + t < tokens;
+        float v[32];
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            v[j] = valid ? ld1(x + (seq * tokens + tok0 + t) * 128 + gq * 32 + j) : 0.0f;
+            amax = fmaxf(amax, fabsf(v[j]));
+        }
+        const float d = amax / 127.0f;
+        const float id = d > 0.0f ? 1.0f / d : 0.0f;
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = 0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const int qv = (int)roundf(v[j] * id);
+            w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
+        }
+        // 32 values = two 16-byte chunks (2*gq, 2*gq+1) of row t
+        *reinterpret_cast<uint4 *>(block + (2 * gq) * 2048 + t * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        *reinterpret_cast<uint4 *>(block + (2 * gq + 1) * 2048 + t * 16) = make_uint4(w[4], w[5], w[6], w[7]);
+        reinterpret_cast<__half *>(block + 8 * 2048)[t * 4 + gq] = __float2half_rn(d);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_q8_0_unpack(const uint8_t *packed, int8_t *q, float *scales, int64_t tokens,
+                                                     int64_t blocks_per_seq) {
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
+    for (int e = threadIdx.x; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
+        const int t = e >> 7, dim = e & 127;
+        if (tok0 + t >= tokens) continue;
+        q[(seq * tokens + tok0 + t) * 128 + dim] = (int8_t)block[(dim >> 4) * 2048 + t * 16 + (dim & 15)];
+    }
+    for (int e = threadIdx.x; e < TQ_ROWS_PER_BLOCK * 4; e += 256) {
+        const int t = e >> 2;
+        if (tok0 + t >= tokens) continue;
+        scales[(seq * tokens + tok0 + t) * 4 + (e & 3)] = __half2float(reinterpret_cast<const __half *>(block + 8 * 2048)[e]);
+    }
+}
+
+#define DISPATCH_T(dt, NAME, F)                      \
+    switch (dt) {                                    \
+    case TQ_F16: { using NAME = __half; F; } break;  \
+    case TQ_F32: { using NAME = float; F; } break;   \
+    case TQ_F64: { using NAME = double; F; } break;  \
+    default: tq_set_error("bad dtype %d", dt); return TQ_ERR_ARG; }
+
+inline int64_t blocks_for(int64_t tokens) { return (tokens + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK; }
+
+template <typename TI>
+int launch_wht128(const void *x, void *y, int64_t n, int out_dtype, const float *sa, const float *sb, hipStream_t s) {
+    const unsigned grid = (unsigned)((n + 3) / 4 < 8192 ? (n + 3) / 4 : 8192);
+    DISPATCH_T(out_dtype, TO, (k_wht128<TI, TO><<<grid, 256, 0, s>>>((const TI *)x, (TO *)y, n, sa, sb)));
+    return tq_check_launch("wht128");
+}
+
+}  // namespace
+
+int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_dtype, int out_dtype, int transpose,
+                  hipStream_t s) {
+    const float *sa = transpose ? h->s2_32 : h->s1_32;
+    const float *sb = transpose ? h->s1_32 : h->s2_32;
+    if (n == 0) return TQ_OK;
+    DISPATCH_T(in_dtype, TI, return launch_wht128<TI>(x, y, n, out_dtype, sa, sb, s));
+}
+
+int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
+              uint8_t *sign_bits, void *rnorms, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    if (sign_bits) {
+        if (!h->has_proj || !h->projrot64_t) {
+            tq_set_error("tq_store_qjl: handle has no projection");
+            return TQ_ERR_ARG;
+        }
+        StoreQjlArgs a;
+        a.s1 = h->s1_64; a.s2 = h->s2_64; a.bounds = h->bounds64; a.cent = h->centroids64;
+        a.projrot_t = h->projrot64_t;
+        a.norm_correction = h->norm_correction;
+        a.tokens = tokens; a.blocks_per_seq = bps;
+#define TQ_STOREQ_BITS(B)                                                                              \
+    DISPATCH_T(in_dtype, TI, (k_store_qjl<B, TI><<<grid, 128, 0, s>>>((const TI *)x, (uint8_t *)packed, \
+                                                                      sign_bits, (__half *)rnorms, a)))
+        switch (h->bits) {
+        case 2: TQ_STOREQ_BITS(2); break;
+        case 3: TQ_STOREQ_BITS(3); break;
+        case 4: TQ_STOREQ_BITS(4); break;
+        default: tq_set_error("tq_store_qjl: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+        }
+#undef TQ_STOREQ_BITS
+        return tq_check_launch("store_qjl");
+    }
+    StoreArgs a;
+    a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
+    a.kind = kind; a.norm_correction = h->norm_correction;
+    a.tokens = tokens; a.blocks_per_seq = bps;
+#define TQ_STORE_BITS(B) \
+    DISPATCH_T(in_dtype, TI, (k_store<B, TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, a)))
+    switch (h->bits) {
+    case 2: TQ_STORE_BITS(2); break;
+    case 3: TQ_STORE_BITS(3); break;
+    case 4: TQ_STORE_BITS(4); break;
+    default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+    }
+#undef TQ_STORE_BITS
+    return tq_check_launch("store");
+}
+
+int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
+             int out_dtype, int domain, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    LoadArgs a;
+    a.s1 = h->s1_32; a.s2 = h->s2_32; a.cent = h->centroids32;
+    a.bits = h->bits; a.kind = kind; a.domain = domain;
+    a.tokens = tokens; a.blocks_per_seq = bps;
+    DISPATCH_T(out_dtype, TO, (k_load<TO><<<grid, 256, 0, s>>>((const uint8_t *)packed, (TO *)out, a)));
+    return tq_check_launch("load");
+}
+
+int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
+                     float *norms, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    k_unpack_codes<<<grid, 256, 0, s>>>((const uint8_t *)packed, idx, norms, h->bits, kind, tokens, bps);
+    return tq_check_launch("unpack_codes");
+}
+
+int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    DISPATCH_T(in_dtype, TI, (k_q8_0_store<TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, tokens, bps)));
+    return tq_check_launch("q8_0_store");
+}
+
+int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    k_q8_0_unpack<<<grid, 256, 0, s>>>((const uint8_t *)packed, q, scales, tokens, bps);
+    return tq_check_launch("q8_0_unpack");
+}

@@ -1,0 +1,228 @@
+"""Production ("turbo2/3/4") KV format on the GPU: head_dim 128, sign-diagonal
+WHT rotation, Lloyd-Max codes packed in 128-token blocks with a corrected fp16
+norm per vector, and attention computed directly on the packed buffers.
+
+The reference describes this format only in its docs (block layout
+docs/papers/block-size-experiment.md:33-39, write-side norm correction
+benchmarks/temporal_decay_prototype.py:58-90, pre-rotated queries
+docs/pre-rotate-queries-plan.md:5-8, Sparse V docs/papers/sparse-v-dequant.md:66-78);
+its arithmetic is the MSE-only quantiser of turboquant/polar_quant.py:56-119
+with the rotation of turboquant/rotation.py:163-185.
+
+All tensors are torch CUDA tensors used as plain buffers; NumPy inputs are
+copied to the device first.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+
+from . import _lib as L
+from .codebook import optimal_centroids
+from .qjl import projection_matrix
+from .rotation import random_rotation_fast
+
+HEAD_DIM = 128
+BLOCK_TOKENS = 128
+
+
+def packed_bytes(bits: int, n_seqs: int, tokens: int) -> int:
+    n = L.lib().tq_packed_bytes(bits, n_seqs, tokens)
+    if n < 0:
+        raise ValueError("bits must be 2, 3 or 4 and sizes non-negative")
+    return int(n)
+
+
+class TurboCodec:
+    """One quantiser (rotation signs + codebook [+ QJL projection]) for K or V.
+
+    seed / single_diagonal: signs1, signs2 = the two `choice` draws of
+        random_rotation_fast(128, default_rng(seed)); single_diagonal forces
+        signs2 to ones (one sign diagonal, as in BASELINE config 1).
+    centroids: table override (default optimal_centroids(bits, 128)).
+    projection: None | "orthogonal" | "gaussian" with projection_seed: enables
+        store_qjl / score_tile.
+    """
+
+    def __init__(self, bits: int = 3, seed: int = 42, *, single_diagonal: bool = False, centroids=None,
+                 norm_correction: bool = True, projection: str | None = None, projection_seed: int | None = None,
+                 signs1=None, signs2=None):
+        if bits not in (2, 3, 4):
+            raise ValueError(f"turbo format supports 2, 3 or 4 bits, got {bits}")
+        self.bits = bits
+        self.d = HEAD_DIM
+        if signs1 is None:
+            signs1, s2, _ = random_rotation_fast(HEAD_DIM, np.random.default_rng(seed))
+            signs2 = np.ones(HEAD_DIM) if single_diagonal else s2
+        self.signs1 = np.asarray(signs1, dtype=np.float64)
+        self.signs2 = np.asarray(signs2, dtype=np.float64)
+        self.centroids = optimal_centroids(bits, HEAD_DIM) if centroids is None else np.asarray(centroids, np.float64)
+        if self.centroids.shape != (1 << bits,):
+            raise ValueError(f"centroids must have {1 << bits} entries")
+        self.norm_correction = norm_correction
+        self.S = None
+        self.projection_scale = 0.0
+        if projection is not None:
+            self.S, self.projection_scale = projection_matrix(
+                HEAD_DIM, seed + 1000 if projection_seed is None else projection_seed, projection)
+        self._handle = None
+
+    @property
+    def handle(self) -> L.Handle:
+        if self._handle is None:
+            self._handle = L.Handle(HEAD_DIM, self.bits, self.centroids, signs1=self.signs1, signs2=self.signs2,
+                                    projection=self.S, projection_scale=self.projection_scale,
+                                    norm_correction=self.norm_correction)
+        return self._handle
+
+    # ---- store / load ---------------------------------------------------------
+    @staticmethod
+    def _as_seqs(x):
+        xd = L.to_device(x)
+        if xd.shape[-1] != HEAD_DIM:
+            raise ValueError(f"last dimension must be {HEAD_DIM}, got {xd.shape[-1]}")
+        if xd.dim() == 2:
+            xd = xd[None]
+        tokens = xd.shape[-2]
+        n_seqs = xd.numel() // (tokens * HEAD_DIM) if tokens else 0
+        return xd.reshape(n_seqs, tokens, HEAD_DIM), n_seqs, tokens
+
+    def store(self, x, kind: str = "k", out=None):
+        """x [..., tokens, 128] (fp16/fp32/fp64) -> packed uint8 buffer; every
+        leading index is a sequence whose blocks do not mix with others."""
+        tt = L.torch()
+        xd, n_seqs, tokens = self._as_seqs(x)
+        nbytes = packed_bytes(self.bits, n_seqs, tokens)
+        if out is None:
+            out = tt.empty(nbytes, dtype=tt.uint8, device=xd.device)
+        elif out.numel() < nbytes:
+            raise ValueError(f"out holds {out.numel()} bytes, need {nbytes}")
+        L.check(L.lib().tq_store(self.handle.h, L.ptr(xd), n_seqs, tokens, L.dtype_code(xd),
+                                 L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        return out
+
+    def store_qjl(self, x):
+        """K-layout codes plus the residual sign sketch -> (packed, sign_bits [n,16] uint8, rnorms [n] fp16)."""
+        tt = L.torch()
+        xd, n_seqs, tokens = self._as_seqs(x)
+        n = n_seqs * tokens
+        packed = tt.empty(packed_bytes(self.bits, n_seqs, tokens), dtype=tt.uint8, device=xd.device)
+        bits = tt.empty((n, 16), dtype=tt.uint8, device=xd.device)
+        rn = tt.empty((n,), dtype=tt.float16, device=xd.device)
+        L.check(L.lib().tq_store_qjl(self.handle.h, L.ptr(xd), n_seqs, tokens, L.dtype_code(xd), L.ptr(packed),
+                                     L.ptr(bits), L.ptr(rn), L.stream_ptr()))
+        return packed, bits, rn
+
+    def load(self, packed, n_seqs: int, tokens: int, kind: str = "k", domain: str = "original", dtype=None):
+        """packed -> [n_seqs, tokens, 128] values in the original or the rotated domain."""
+        tt = L.torch()
+        dtype = tt.float32 if dtype is None else dtype
+        out = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=dtype, device=packed.device)
+        L.check(L.lib().tq_load(self.handle.h, L.ptr(packed), n_seqs, tokens, L.KIND_K if kind == "k" else L.KIND_V,
+                                L.ptr(out), L.dtype_code(out),
+                                L.DOMAIN_ORIGINAL if domain == "original" else L.DOMAIN_ROTATED, L.stream_ptr()))
+        return out
+
+    def unpack_codes(self, packed, n_seqs: int, tokens: int, kind: str = "k"):
+        """packed -> (indices uint8 [n_seqs, tokens, 128], stored norms fp32 [n_seqs, tokens])."""
+        tt = L.torch()
+        idx = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=tt.uint8, device=packed.device)
+        norms = tt.empty((n_seqs, tokens), dtype=tt.float32, device=packed.device)
+        L.check(L.lib().tq_unpack_codes(self.handle.h, L.ptr(packed), n_seqs, tokens,
+                                        L.KIND_K if kind == "k" else L.KIND_V, L.ptr(idx), L.ptr(norms),
+                                        L.stream_ptr()))
+        return idx, norms
+
+    def rotate(self, x, transpose: bool = False, dtype=None):
+        """R x (or R^T x) with the one-wavefront-per-vector fp32 butterfly."""
+        tt = L.torch()
+        xd = L.to_device(x)
+        if xd.dtype == tt.float64:
+            xd = xd.to(tt.float32)
+        flat = xd.reshape(-1, HEAD_DIM)
+        out = tt.empty(flat.shape, dtype=xd.dtype if dtype is None else dtype, device=xd.device)
+        L.check(L.lib().tq_rotate(self.handle.h, L.ptr(flat), L.ptr(out), flat.shape[0], L.dtype_code(flat),
+                                  L.dtype_code(out), int(transpose), L.stream_ptr()))
+        return out.reshape(xd.shape)
+
+    # ---- prefill-shaped inner-product estimator --------------------------------
+    def score_tile(self, q, packed, sign_bits, rnorms, n_keys: int, out_dtype=None):
+        """logits [nq, n_keys] = <R q, g c[idx]> + scale * rnorm * <S q, z>."""
+        tt = L.torch()
+        qd = L.to_device(q).reshape(-1, HEAD_DIM)
+        nq = qd.shape[0]
+        out_dtype = tt.float32 if out_dtype is None else out_dtype
+        logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device)
+        ws = tt.empty(max(nq * 256 * 2, 16), dtype=tt.uint8, device=qd.device)
+        L.check(L.lib().tq_score_tile(self.handle.h, L.ptr(qd), L.dtype_code(qd), nq, L.ptr(packed), L.ptr(sign_bits),
+                                      L.ptr(rnorms), n_keys, L.ptr(logits), L.dtype_code(logits), L.ptr(ws),
+                                      ws.numel(), L.stream_ptr()))
+        return logits
+
+
+def q8_0_store(x):
+    """x [..., tokens, 128] -> q8_0-style K buffer (uint8), n_seqs, tokens."""
+    tt = L.torch()
+    xd, n_seqs, tokens = TurboCodec._as_seqs(x)
+    out = tt.empty(int(L.lib().tq_q8_0_bytes(n_seqs, tokens)), dtype=tt.uint8, device=xd.device)
+    L.check(L.lib().tq_q8_0_store(L.ptr(xd), n_seqs, tokens, L.dtype_code(xd), L.ptr(out), L.stream_ptr()))
+    return out, n_seqs, tokens
+
+
+def q8_0_unpack(packed, n_seqs: int, tokens: int):
+    tt = L.torch()
+    q = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=tt.int8, device=packed.device)
+    s = tt.empty((n_seqs, tokens, 4), dtype=tt.float32, device=packed.device)
+    L.check(L.lib().tq_q8_0_unpack(L.ptr(packed), n_seqs, tokens, L.ptr(q), L.ptr(s), L.stream_ptr()))
+    return q, s
+
+
+class DecodeAttention:
+    """softmax(scale * q k^T) v over packed K/V for GQA groups of 4 query heads.
+
+    Holds the parameter block and the split workspace so that repeated steps
+    allocate nothing.  K is a turbo buffer (k_codec given) or a q8_0-style
+    buffer (k_codec None); V is always a turbo buffer written with kind="v".
+    """
+
+    def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec, batch: int, n_q_heads: int, n_kv_heads: int,
+                 tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0):
+        tt = L.torch()
+        dev = L.require_gpu()
+        self.k_codec, self.v_codec = k_codec, v_codec
+        if n_splits is None:
+            n_splits = default_splits(batch * n_kv_heads, tokens)
+        self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
+                                     n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
+                                     scale=(1.0 / math.sqrt(HEAD_DIM)) if scale is None else scale,
+                                     sparse_v_tau=sparse_v_tau)
+        nbytes = L.lib().tq_attn_workspace_bytes(C.byref(self.params))
+        if nbytes < 0:
+            L.check(L.ERR_UNSUPPORTED if n_q_heads != 4 * n_kv_heads else L.ERR_ARG)
+        self.workspace = tt.empty(int(nbytes), dtype=tt.uint8, device=dev)
+        self.skip = tt.zeros(2, dtype=tt.int64, device=dev)
+        self.out = tt.empty((batch, n_q_heads, HEAD_DIM), dtype=tt.float32, device=dev)
+
+    def __call__(self, q, k_packed, v_packed, bias=None):
+        """q [batch, n_q_heads, 128] in the original domain -> out fp32 [batch, n_q_heads, 128]."""
+        qd = L.to_device(q)
+        hk = self.k_codec.handle.h if self.k_codec is not None else None
+        L.check(L.lib().tq_decode_attention(hk, self.v_codec.handle.h, C.byref(self.params), L.ptr(qd),
+                                            L.dtype_code(qd), L.ptr(k_packed), None, L.ptr(v_packed), L.ptr(bias),
+                                            L.ptr(self.out), L.ptr(self.skip), L.ptr(self.workspace),
+                                            self.workspace.numel(), L.stream_ptr()))
+        return self.out
+
+    def skip_rate(self) -> float:
+        s = self.skip.cpu().numpy()
+        return float(s[0]) / float(s[1]) if s[1] else 0.0
+
+
+def default_splits(n_groups: int, tokens: int) -> int:
+    """Context splits per (batch, kv head): enough wavefronts to fill 256 CUs x 4
+    SIMDs twice over, at least 4 tiles of 64 tokens per split."""
+    tiles = max(1, (tokens + 63) // 64)
+    want = max(1, (2 * 1024 + n_groups - 1) // n_groups)
+    return int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
