@@ -516,8 +516,9 @@ def boundary_band_mismatches(y, idx_test, centroids, rel=1e-6):
 #           p//5); pair 60+q takes bits 30..31 of dwords 3q, 3q+1, 3q+2 as its
 #           low, middle and high two bits.           (48 B)
 # K rows: row = token, pair p = dims (2p, 2p+1).
-# V rows: row r of a block = token quad r//4, sub-row i = r%4; pair 2g+h =
-#         dim 4g+i of tokens 4*(r//4) + 2h and + 2h + 1.
+# V rows are dim-major inside each 64-token tile: row (token & 64) | (dim & 63)
+#         holds dims r and 64+r of the tile's 64 tokens; pair 32*(dim >> 6) + tp =
+#         tokens 2*tp and 2*tp+1 of the tile (lo, hi).
 # A BLOCK is 128 rows stored chunk-major: [16*b/16 chunks][128 rows][16 B],
 # followed by 128 fp16 norms (token order).  Block bytes = 128*(16*b + 2).
 
@@ -586,11 +587,10 @@ def layout_pack(idx: np.ndarray, g: np.ndarray, bits: int, kind: str) -> np.ndar
     if kind == "k":
         pairs = idx[:, 0::2] | (idx[:, 1::2] << np.uint32(bits))          # [T,64]
     else:
-        q = idx.reshape(T // 4, 4, 32, 4)                                  # quad, tok, g, i
-        q = q.transpose(0, 3, 2, 1)                                        # quad, i, g, tok
-        lo = q[..., 0::2]
-        hi = q[..., 1::2]
-        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row=(quad,i); pair=2g+h
+        q = idx.reshape(T // 64, 32, 2, 2, 64)                             # tile, token pair, parity, dim half, r
+        lo = q[:, :, 0].transpose(0, 3, 2, 1)                              # tile, r, dim half, token pair
+        hi = q[:, :, 1].transpose(0, 3, 2, 1)
+        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row = 64*tile + r; pair = 32*half + tp
     rows = _pairs_to_rows(pairs, bits)                                     # [T, 4*bits]
     rows = rows.reshape(nb, ROWS_PER_BLOCK, bits, 4).transpose(0, 2, 1, 3) # block, chunk, row, 4
     out = np.zeros((nb, block_bytes(bits)), dtype=np.uint8)
@@ -618,12 +618,10 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
         idx[:, 0::2] = lo
         idx[:, 1::2] = hi
     else:
-        q = np.zeros((T // 4, 4, 32, 4), dtype=np.uint8)                   # quad, i, g, tok
-        lo = lo.reshape(T // 4, 4, 32, 2)
-        hi = hi.reshape(T // 4, 4, 32, 2)
-        q[..., 0::2] = lo
-        q[..., 1::2] = hi
-        idx = q.transpose(0, 3, 2, 1).reshape(T, 128)                      # quad, tok, g, i
+        q = np.zeros((T // 64, 32, 2, 2, 64), dtype=np.uint8)              # tile, token pair, parity, dim half, r
+        q[:, :, 0] = lo.reshape(T // 64, 64, 2, 32).transpose(0, 3, 2, 1)
+        q[:, :, 1] = hi.reshape(T // 64, 64, 2, 32).transpose(0, 3, 2, 1)
+        idx = q.reshape(T, 128)
     return idx, g
 
 

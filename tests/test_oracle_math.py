@@ -156,7 +156,7 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
     if kind == "k":
         row, pair, half = tok, dim // 2, dim % 2
     else:
-        row, pair, half = 4 * (tok // 4) + dim % 4, 2 * (dim // 4) + (tok % 4) // 2, tok % 2
+        row, pair, half = (tok & 64) | (dim & 63), 32 * (dim >> 6) + (tok & 63) // 2, tok % 2
     value = ((1 << bits) - 1) << (bits * half)
     rowwords = words[:, row, :].reshape(-1)
     expect = np.zeros(4 * bits, dtype=np.uint64)

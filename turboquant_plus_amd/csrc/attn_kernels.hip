@@ -10,11 +10,13 @@
 //   query heads, so all 64 lanes and all 16 blocks do useful work.
 //     QK: A_b = K[tokens 4b..4b+3][4 dims], B_b = q^T[4 dims][4 heads]
 //         -> lane (b,j) gets the logits of head j for tokens 4b..4b+3.
-//     PV: A_b = P[4 heads][tokens 4b..4b+3] (the same lane layout the QK output
-//         has), B_b = V[tokens 4b..4b+3][4 dims] -> D_b = partial out[4 heads][4 dims];
-//         the 16 blocks are summed across lanes once at the end of the split.
-//   Online softmax in base 2 (log2(e) folded into the query scale); accumulators
-//   are rescaled only when a running maximum moves.
+//     PV: V rows are dim-major inside the tile (lane l holds dims l and 64+l of the
+//         64 tokens), so block b covers dims 4b..4b+3: A_b = P[4 heads][tokens
+//         4T..4T+3] (the fp16 weights, shared by all blocks through a 512-byte LDS
+//         exchange), B_b = V[tokens 4T..4T+3][dims 4b..4b+3] -> D_b = out[4 heads][4
+//         dims].  16 token groups x 2 dim halves = 32 MFMAs per tile into 16
+//         accumulator registers; no cross-lane reduction at the end of the split.
+//   Online softmax in base 2 (log2(e) folded into the query scale).
 // k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
 //   the V rotation (one wavefront per query head).
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
@@ -98,7 +100,7 @@ struct AttnArgs {
 constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
 
 template <int KFMT, int KBITS, int VBITS, bool SPARSE>
-__global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
     constexpr int VBLOCK = TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
@@ -106,6 +108,7 @@ __global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
     constexpr int VLUT_N = 1 << (2 * VBITS);
     __shared__ uint32_t klut_s[KLUT_N];
     __shared__ uint32_t vlut_s[VLUT_N];
+    __shared__ uint2 p_s[4][64];  // per wavefront: fp16 weights of the current tile, [token group][head]
 
     const int tid = threadIdx.x, lane = tid & 63;
     if constexpr (KFMT == KFMT_TURBO)
@@ -131,9 +134,11 @@ __global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
 #pragma unroll
         for (int g = 0; g < 32; ++g) qreg[g] = __builtin_bit_cast(half4_t, qp[g]);
     }
-    float4_t acc_o[32];
+    // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
+    float4_t acc_o[2][2];
 #pragma unroll
-    for (int g = 0; g < 32; ++g) acc_o[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
+    uint2 *p_w = p_s[tid >> 6];
     float m_run = -INFINITY, l_run = 0.0f;
     unsigned nskip = 0;
 
@@ -238,16 +243,17 @@ __global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
         // ---- online softmax (base 2) ------------------------------------------------
         const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
         const float m_new = fmaxf(m_run, mx);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-            const float corr = exp2f(m_run - m_new);  // 0 on the first tile
+        {
+            const float corr = exp2f(m_run - m_new);  // 0 on the first tile, 1 when the maximum stays
             l_run *= corr;
+            // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
             const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
 #pragma unroll
-            for (int g = 0; g < 32; ++g) {
-                acc_o[g][0] *= c0;
-                acc_o[g][1] *= c1;
-                acc_o[g][2] *= c2;
-                acc_o[g][3] *= c3;
+            for (int c = 0; c < 4; ++c) {
+                acc_o[c >> 1][c & 1][0] *= c0;
+                acc_o[c >> 1][c & 1][1] *= c1;
+                acc_o[c >> 1][c & 1][2] *= c2;
+                acc_o[c >> 1][c & 1][3] *= c3;
             }
             m_run = m_new;
         }
@@ -275,31 +281,40 @@ __global__ __launch_bounds__(256) void k_decode_attn(AttnArgs a) {
         }
 
         // ---- PV ------------------------------------------------------------------------
+        // weights (times the stored V norm) as fp16, published to the wavefront through LDS:
+        // entry 4*T + i = head i, tokens 4T..4T+3 of the tile (this lane is T = lane/4, i = lane%4)
         half4_t pv;
         pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.x & 0xffff))));
         pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
         pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
         pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
+        p_w[lane] = __builtin_bit_cast(uint2, pv);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; pair 32*hf + 2T (+1)
+        // = tokens 4T..4T+3.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf).
 #pragma unroll
-        for (int g = 0; g < 32; ++g) {
-            const uint32_t lo = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 2 * g));
-            const uint32_t hi = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 2 * g + 1));
-            acc_o[g] = mfma4(pv, h4_from(lo, hi), acc_o[g]);
+        for (int T = 0; T < 16; ++T) {
+            const half4_t pa = __builtin_bit_cast(half4_t, p_w[4 * T + j]);
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const uint32_t lo = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 32 * hf + 2 * T));
+                const uint32_t hi = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 32 * hf + 2 * T + 1));
+                acc_o[hf][T & 1] = mfma4(pa, h4_from(lo, hi), acc_o[hf][T & 1]);
+            }
         }
+        __builtin_amdgcn_wave_barrier();  // the next tile overwrites p_w
 #pragma unroll
         for (int q = 0; q < KROW_DW; ++q) kw[q] = kw_next[q];
     }
 
-    // ---- end of split: sum the 16 blocks, write the partial ------------------------
+    // ---- end of split: write the partial ---------------------------------------------
     const float l_tot = sum_over_blocks(l_run);
 #pragma unroll
-    for (int g = 0; g < 32; ++g) {
+    for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float v = sum_over_blocks(acc_o[g][i]);
-            if (lane < 4) po[i * 128 + 4 * g + j] = v;
-        }
-    }
+        for (int i = 0; i < 4; ++i) po[i * 128 + 64 * hf + lane] = acc_o[hf][0][i] + acc_o[hf][1][i];
     if (lane < 4) {
         pml[2 * j] = m_run;
         pml[2 * j + 1] = l_tot;

@@ -114,8 +114,9 @@ __device__ inline void wht128_wave(float &a, float &b, int lane) {
 //   BITS 3: pairs 0..59 five to a dword at bit 6*(p%5); pair 60+t = bits 30..31 of
 //           dwords 3t, 3t+1, 3t+2 (low, middle, high two bits)
 // A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
-// norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows: row r = token
-// quad r/4, sub-row i = r%4; pair 2g+h = dim 4g+i of tokens 4*(r/4)+2h, +2h+1.
+// norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows are dim-major
+// inside each 64-token tile: row (token & 64) | (dim & 63) holds dims r and 64+r
+// of the tile's tokens; pair 32*(dim >> 6) + tp = tokens 2tp, 2tp+1 of the tile.
 __host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
 __host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
 __host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
@@ -159,8 +160,8 @@ __device__ inline void locate(int kind, int token, int dim, int &row, int &pair,
         pair = dim >> 1;
         half = dim & 1;
     } else {
-        row = (token & ~3) | (dim & 3);
-        pair = 2 * (dim >> 2) + ((token & 3) >> 1);
+        row = (token & 64) | (dim & 63);
+        pair = ((dim >> 6) << 5) | ((token & 63) >> 1);
         half = token & 1;
     }
 }

@@ -91,8 +91,8 @@ template <int BITS> __device__ inline uint32_t pair_from_stage(const uint8_t *co
         lo = codes[row * CODE_STRIDE + 2 * p];
         hi = codes[row * CODE_STRIDE + 2 * p + 1];
     } else {
-        const int tok = (row & ~3) + 2 * (p & 1);
-        const int dim = 4 * (p >> 1) + (row & 3);
+        const int tok = (row & 64) + 2 * (p & 31);
+        const int dim = ((p >> 5) << 6) | (row & 63);
         lo = codes[tok * CODE_STRIDE + dim];
         hi = codes[(tok + 1) * CODE_STRIDE + dim];
     }
