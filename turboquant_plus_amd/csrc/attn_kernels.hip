@@ -2,25 +2,31 @@
 //
 // k_decode_attn: split-K decode attention for one GQA group of 4 query heads.
 //   One 64-lane wavefront owns one context split and walks it in tiles of 64
-//   tokens.  Lane l holds packed row l of the tile (K: token l; V: token quad
-//   l/4, sub-row l%4), loaded as 16-byte chunks that are contiguous across
+//   tokens.  Lane l holds packed row l of the tile (K: token l; V: dims l and
+//   64+l of all 64 tokens), loaded as 16-byte chunks that are contiguous across
 //   lanes.  Pair codes are turned into fp16 pairs through a 4-byte-entry LUT
 //   in LDS (one ds_read per two values) and fed to the 4x4x4 fp16 MFMA with
 //   16 independent blocks: block b multiplies the 4 tokens 4b..4b+3 by the 4
 //   query heads, so all 64 lanes and all 16 blocks do useful work.
-//     QK: A_b = K[tokens 4b..4b+3][4 dims], B_b = q^T[4 dims][4 heads]
-//         -> lane (b,j) gets the logits of head j for tokens 4b..4b+3.
+//   The MFMA's A-matrix broadcast (cbsz = 4, abid = source block) lets one block's
+//   A operand serve all 16 blocks:
+//     QK: A = q[4 heads][4 dims] read from block g%16 (each lane keeps only two
+//         4-dim slices of q), B_b = K^T[4 dims][tokens 4b..4b+3] -> lane l gets the 4
+//         heads' logits of token l; a 4x4 transpose inside each lane quad turns that
+//         into head l%4, tokens 4b..4b+3 for the softmax.
 //     PV: V rows are dim-major inside the tile (lane l holds dims l and 64+l of the
-//         64 tokens), so block b covers dims 4b..4b+3: A_b = P[4 heads][tokens
-//         4T..4T+3] (the fp16 weights, shared by all blocks through a 512-byte LDS
-//         exchange), B_b = V[tokens 4T..4T+3][dims 4b..4b+3] -> D_b = out[4 heads][4
-//         dims].  16 token groups x 2 dim halves = 32 MFMAs per tile into 16
-//         accumulator registers; no cross-lane reduction at the end of the split.
+//         64 tokens), so block b covers dims 4b..4b+3: A = P[4 heads][tokens 4T..4T+3],
+//         the fp16 weights held by block T and broadcast, B_b = V[tokens 4T..4T+3][dims
+//         4b..4b+3] -> D_b = out[4 heads][4 dims].  16 token groups x 2 dim halves = 32
+//         MFMAs per tile into 16 accumulator registers; no cross-lane reduction at the
+//         end of the split and no LDS traffic besides the LUT reads.
 //   Online softmax in base 2 (log2(e) folded into the query scale).
 // k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
 //   the V rotation (one wavefront per query head).
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+#include <utility>
+
 #include "tq_device.h"
 
 namespace {
@@ -68,6 +74,30 @@ __device__ __forceinline__ float4_t mfma4(half4_t a, half4_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 0, 0, 0);
 }
 
+// 4x4x4 MFMA whose A operand is taken from block ABID and broadcast to all 16 blocks
+template <int ABID> __device__ __forceinline__ float4_t mfma4_bcast(half4_t a, half4_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 4, ABID, 0);
+}
+
+// transpose the 4x4 matrix held by a quad of lanes (element [lane%4][register]), two exchange stages
+__device__ __forceinline__ void quad_transpose(float (&r)[4], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+#pragma unroll
+    for (int p = 0; p < 4; p += 2) {  // swap (even lane, odd reg) <-> (odd lane, even reg)
+        const float give = b0 ? r[p] : r[p + 1];
+        const float got = xor_lane<1>(give);
+        if (b0) r[p] = got;
+        else r[p + 1] = got;
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {     // swap (lane bit1 clear, reg p+2) <-> (lane bit1 set, reg p)
+        const float give = b1 ? r[p] : r[p + 2];
+        const float got = xor_lane<2>(give);
+        if (b1) r[p] = got;
+        else r[p + 2] = got;
+    }
+}
+
 // sum over the 16 lanes that share lane%4 (blocks b = 0..15)
 __device__ __forceinline__ float sum_over_blocks(float v) {
     v += xor_lane<4>(v);
@@ -99,6 +129,50 @@ struct AttnArgs {
 
 constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
 
+// QK over the 32 dim groups: B = this lane's K row (4 dims per group), A = q from block G % 16
+template <int BITS, int... G>
+__device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const uint32_t (&kw)[4 * BITS],
+                                         const char *lut, const half4_t (&qa)[2], float4_t (&acc)[4]) {
+    ((acc[G & 3] = mfma4_bcast<(G & 15)>(
+          qa[G >> 4],
+          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(kw, 2 * G)),
+                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(kw, 2 * G + 1))),
+          acc[G & 3])),
+     ...);
+}
+
+// q8_0-style K: one accumulator per 32-value block (dim groups 8*blk .. 8*blk+7), scaled afterwards
+template <int... G>
+__device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const uint32_t (&kw)[32],
+                                      const half4_t (&qa)[2], float4_t (&acc)[4]) {
+    auto cvt = [](uint32_t w) {
+        half4_t kv;
+        kv[0] = (_Float16)(int)(int8_t)(w & 0xff);
+        kv[1] = (_Float16)(int)(int8_t)((w >> 8) & 0xff);
+        kv[2] = (_Float16)(int)(int8_t)((w >> 16) & 0xff);
+        kv[3] = (_Float16)(int)(int8_t)(w >> 24);
+        return kv;
+    };
+    ((acc[G >> 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], cvt(kw[G]), acc[G >> 3])), ...);
+}
+
+// PV over the 16 token groups x 2 dim halves: A = weights of block T (broadcast), B = this lane's V row
+template <int BITS, int... T>
+__device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const uint32_t (&vw)[4 * BITS],
+                                       const char *lut, half4_t pv, float4_t (&acc_o)[2][2]) {
+    ((acc_o[0][T & 1] = mfma4_bcast<T>(
+          pv,
+          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 2 * T)),
+                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 2 * T + 1))),
+          acc_o[0][T & 1]),
+      acc_o[1][T & 1] = mfma4_bcast<T>(
+          pv,
+          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 32 + 2 * T)),
+                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 32 + 2 * T + 1))),
+          acc_o[1][T & 1])),
+     ...);
+}
+
 template <int KFMT, int KBITS, int VBITS, bool SPARSE>
 __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
@@ -108,7 +182,6 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     constexpr int VLUT_N = 1 << (2 * VBITS);
     __shared__ uint32_t klut_s[KLUT_N];
     __shared__ uint32_t vlut_s[VLUT_N];
-    __shared__ uint2 p_s[4][64];  // per wavefront: fp16 weights of the current tile, [token group][head]
 
     const int tid = threadIdx.x, lane = tid & 63;
     if constexpr (KFMT == KFMT_TURBO)
@@ -127,18 +200,18 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
     float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
 
-    // B operand of QK: q[head j][dims 4g..4g+3], g = 0..31
-    half4_t qreg[32];
+    // A operand of QK, broadcast from one block per MFMA: lane (b, i) keeps q[head i] for the
+    // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
+    half4_t qa[2];
     {
         const uint2 *qp = reinterpret_cast<const uint2 *>(a.qrot + ((int64_t)group * 4 + j) * 128);
-#pragma unroll
-        for (int g = 0; g < 32; ++g) qreg[g] = __builtin_bit_cast(half4_t, qp[g]);
+        qa[0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
+        qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[2][2];
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
-    uint2 *p_w = p_s[tid >> 6];
     float m_run = -INFINITY, l_run = 0.0f;
     unsigned nskip = 0;
 
@@ -147,12 +220,17 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     const char *klut_b = reinterpret_cast<const char *>(klut_s);
     const char *vlut_b = reinterpret_cast<const char *>(vlut_s);
 
+    // Rows are fetched one tile ahead into the same registers: the next K row right after QK has
+    // consumed the current one, the next V row right after PV (dense mode).  The index is clamped
+    // at the last tile, so the final prefetch re-reads a row instead of branching.
     uint32_t kw[KROW_DW];
+    uint32_t vw[4 * VBITS];
     if (t_begin < t_end) {
+        const int row0 = (t_begin & 1) * 64 + lane;
         const uint8_t *kb = kbase + (int64_t)(t_begin >> 1) * KBLOCK;
-        const int row = (t_begin & 1) * 64 + lane;
-        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row, kw);
-        else load_row<8>(kb, row, kw);
+        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row0, kw);
+        else load_row<8>(kb, row0, kw);
+        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(t_begin >> 1) * VBLOCK, row0, vw);
     }
 
 #pragma unroll 1
@@ -164,37 +242,9 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         const uint8_t *kb = kbase + blk * KBLOCK;
         const uint8_t *vb = vbase + blk * VBLOCK;
 
-        // ---- issue loads: K scales, V row (dense mode), next K row ----------------
-        float gk[4];
-        float kscale[4][4];
-        if constexpr (KFMT == KFMT_TURBO) {
-            const uint2 u = *reinterpret_cast<const uint2 *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS + 2 * tok_in_block);
-            gk[0] = __half2float(__ushort_as_half((unsigned short)(u.x & 0xffff)));
-            gk[1] = __half2float(__ushort_as_half((unsigned short)(u.x >> 16)));
-            gk[2] = __half2float(__ushort_as_half((unsigned short)(u.y & 0xffff)));
-            gk[3] = __half2float(__ushort_as_half((unsigned short)(u.y >> 16)));
-        } else {
-            const uint4 *sp = reinterpret_cast<const uint4 *>(kb + 8 * 2048 + 8 * tok_in_block);
-            const uint4 s0 = sp[0], s1 = sp[1];
-            const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                kscale[i][0] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i] & 0xffff)));
-                kscale[i][1] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i] >> 16)));
-                kscale[i][2] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i + 1] & 0xffff)));
-                kscale[i][3] = __half2float(__ushort_as_half((unsigned short)(sw[2 * i + 1] >> 16)));
-            }
-        }
-        uint32_t vw[4 * VBITS];
-        if constexpr (!SPARSE) load_row<VBITS>(vb, row, vw);
+        const int tile_n = min(tile + 1, t_end - 1);
+        const int row_n = (tile_n & 1) * 64 + lane;
         const uint2 gvu = *reinterpret_cast<const uint2 *>(vb + TQ_ROWS_PER_BLOCK * 16 * VBITS + 2 * tok_in_block);
-        uint32_t kw_next[KROW_DW];
-        if (tile + 1 < t_end) {
-            const uint8_t *kbn = kbase + (int64_t)((tile + 1) >> 1) * KBLOCK;
-            const int rown = ((tile + 1) & 1) * 64 + lane;
-            if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, rown, kw_next);
-            else load_row<8>(kbn, rown, kw_next);
-        }
         float bias4[4] = {0.f, 0.f, 0.f, 0.f};
         const int64_t tok0 = (int64_t)tile * 64 + b4;
         if (a.bias) {
@@ -204,38 +254,40 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         }
 
         // ---- QK ------------------------------------------------------------------
-        float s[4];
+        // D_b[head][token 4b + lane%4]: every lane gets the 4 heads' dot products of its own token
+        float sc[4];
         if constexpr (KFMT == KFMT_TURBO) {
             float4_t acc[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+            qk_turbo<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa, acc);
+            const float gk_own = __half2float(
+                reinterpret_cast<const __half *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS)[half * 64 + lane]);
 #pragma unroll
-            for (int g = 0; g < 32; ++g) {
-                const uint32_t lo = *reinterpret_cast<const uint32_t *>(klut_b + pair_off<KBITS>(kw, 2 * g));
-                const uint32_t hi = *reinterpret_cast<const uint32_t *>(klut_b + pair_off<KBITS>(kw, 2 * g + 1));
-                acc[g & 3] = mfma4(h4_from(lo, hi), qreg[g], acc[g & 3]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) s[i] = ((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i])) * gk[i] + bias4[i];
+            for (int i = 0; i < 4; ++i) sc[i] = ((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i])) * gk_own;
         } else {
             float4_t acc[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+            qk_q8(std::make_integer_sequence<int, 32>{}, kw, qa, acc);
+            const uint2 su = *reinterpret_cast<const uint2 *>(kb + 8 * 2048 + 8 * (half * 64 + lane));
+            const float d0 = __half2float(__ushort_as_half((unsigned short)(su.x & 0xffff)));
+            const float d1 = __half2float(__ushort_as_half((unsigned short)(su.x >> 16)));
+            const float d2 = __half2float(__ushort_as_half((unsigned short)(su.y & 0xffff)));
+            const float d3 = __half2float(__ushort_as_half((unsigned short)(su.y >> 16)));
 #pragma unroll
-            for (int g = 0; g < 32; ++g) {
-                const uint32_t w = kw[g];
-                half4_t kv;
-                kv[0] = (_Float16)(int)(int8_t)(w & 0xff);
-                kv[1] = (_Float16)(int)(int8_t)((w >> 8) & 0xff);
-                kv[2] = (_Float16)(int)(int8_t)((w >> 16) & 0xff);
-                kv[3] = (_Float16)(int)(int8_t)(w >> 24);
-                acc[g >> 3] = mfma4(kv, qreg[g], acc[g >> 3]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                s[i] = (acc[0][i] * kscale[i][0] + acc[1][i] * kscale[i][1]) +
-                       (acc[2][i] * kscale[i][2] + acc[3][i] * kscale[i][3]) + bias4[i];
+            for (int i = 0; i < 4; ++i) sc[i] = (acc[0][i] * d0 + acc[1][i] * d1) + (acc[2][i] * d2 + acc[3][i] * d3);
         }
+        {   // kw is dead now: fetch the next tile's K row into it
+            const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
+            if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, row_n, kw);
+            else load_row<8>(kbn, row_n, kw);
+        }
+        // -> lane (b, j): head j, tokens 4b..4b+3
+        quad_transpose(sc, lane);
+        float s[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = sc[i] + bias4[i];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             if (tok0 + i >= a.tokens) s[i] = -INFINITY;
@@ -272,41 +324,22 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
             }
         }
         if constexpr (SPARSE) {
-            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {
-#pragma unroll
-                for (int q = 0; q < KROW_DW; ++q) kw[q] = kw_next[q];
-                continue;  // every V row of this tile is skipped: no V load, no dequant
-            }
+            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) continue;  // every V row skipped: no V load, no dequant
             load_row<VBITS>(vb, row, vw);
         }
 
         // ---- PV ------------------------------------------------------------------------
-        // weights (times the stored V norm) as fp16, published to the wavefront through LDS:
-        // entry 4*T + i = head i, tokens 4T..4T+3 of the tile (this lane is T = lane/4, i = lane%4)
+        // weights (times the stored V norm) as fp16: this lane is token group T = lane/4, head lane%4
         half4_t pv;
         pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.x & 0xffff))));
         pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
         pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
         pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
-        p_w[lane] = __builtin_bit_cast(uint2, pv);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; pair 32*hf + 2T (+1)
-        // = tokens 4T..4T+3.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf).
-#pragma unroll
-        for (int T = 0; T < 16; ++T) {
-            const half4_t pa = __builtin_bit_cast(half4_t, p_w[4 * T + j]);
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
-                const uint32_t lo = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 32 * hf + 2 * T));
-                const uint32_t hi = *reinterpret_cast<const uint32_t *>(vlut_b + pair_off<VBITS>(vw, 32 * hf + 2 * T + 1));
-                acc_o[hf][T & 1] = mfma4(pa, h4_from(lo, hi), acc_o[hf][T & 1]);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();  // the next tile overwrites p_w
-#pragma unroll
-        for (int q = 0; q < KROW_DW; ++q) kw[q] = kw_next[q];
+        // = tokens 4T..4T+3.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
+        // weights of token group T sit in block T and are broadcast to every block.
+        pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
+        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
     }
 
     // ---- end of split: write the partial ---------------------------------------------
@@ -350,7 +383,9 @@ __global__ __launch_bounds__(256) void k_prep_q(const TI *q, __half *qrot, int64
     qrot[v * 128 + 2 * lane + 1] = __float2half_rn(x1 * scale_log2e);
 }
 
-// merge split partials, un-rotate with the V rotation's transpose; one wavefront per query head
+// merge split partials, un-rotate with the V rotation's transpose; one wavefront per query head.
+// Lane s first fetches (m, l) of split s (64 splits per pass), so the weights of all splits are
+// known after one round trip; the partial outputs are then streamed with independent loads.
 __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
                                                       int64_t n_rows, int n_splits, const float *s1, const float *s2) {
     const int lane = threadIdx.x & 63;
@@ -358,20 +393,35 @@ __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const
     if (r >= n_rows) return;
     const int64_t group = r >> 2;
     const int head = (int)(r & 3);
+    const float *ml = part_ml + (group * n_splits * 4 + head) * 2;   // + s*8
+    const float *po = part_o + (group * n_splits * 4 + head) * 128;  // + s*512
     float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) {
-        const float l = part_ml[((group * n_splits + s) * 4 + head) * 2 + 1];
-        if (l > 0.0f) M = fmaxf(M, part_ml[((group * n_splits + s) * 4 + head) * 2]);
+    for (int s0 = 0; s0 < n_splits; s0 += 64) {
+        const int s = s0 + lane;
+        float m = -INFINITY;
+        if (s < n_splits && ml[s * 8 + 1] > 0.0f) m = ml[s * 8];
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        M = fmaxf(M, m);
     }
     float L = 0.0f, o0 = 0.0f, o1 = 0.0f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float *ml = part_ml + ((group * n_splits + s) * 4 + head) * 2;
-        if (!(ml[1] > 0.0f)) continue;
-        const float w = exp2f(ml[0] - M);
-        L += ml[1] * w;
-        const float *po = part_o + ((group * n_splits + s) * 4 + head) * 128;
-        o0 = fmaf(po[2 * lane], w, o0);
-        o1 = fmaf(po[2 * lane + 1], w, o1);
+    for (int s0 = 0; s0 < n_splits; s0 += 64) {
+        const int s = s0 + lane;
+        float w = 0.0f, l = 0.0f;
+        if (s < n_splits) {
+            l = ml[s * 8 + 1];
+            w = l > 0.0f ? exp2f(ml[s * 8] - M) : 0.0f;
+        }
+        float lw = l * w;
+        for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
+        L += lw;
+        const int cnt = min(64, n_splits - s0);
+#pragma unroll 8
+        for (int t = 0; t < cnt; ++t) {
+            const float wt = __shfl(w, t);
+            const float2 v = *reinterpret_cast<const float2 *>(po + (int64_t)(s0 + t) * 512 + 2 * lane);
+            o0 = fmaf(v.x, wt, o0);
+            o1 = fmaf(v.y, wt, o1);
+        }
     }
     const float invL = L > 0.0f ? 1.0f / L : 0.0f;
     o0 *= invL * s2[2 * lane];

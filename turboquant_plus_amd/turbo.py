@@ -221,8 +221,8 @@ class DecodeAttention:
 
 
 def default_splits(n_groups: int, tokens: int) -> int:
-    """Context splits per (batch, kv head): enough wavefronts to fill 256 CUs x 4
-    SIMDs twice over, at least 4 tiles of 64 tokens per split."""
+    """Context splits per (batch, kv head): one wavefront per split, four
+    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each."""
     tiles = max(1, (tokens + 63) // 64)
-    want = max(1, (2 * 1024 + n_groups - 1) // n_groups)
+    want = max(1, (4 * 1024 + n_groups - 1) // n_groups)
     return int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
