@@ -30,6 +30,9 @@ struct tq_handle {
     double *projrot64_t;   // [128*128] entry [k*128+j] = (S R^T)[j][k]   (d == 128, WHT, projection)
     void *pair_lut;        // [4^bits] half2: (c[lo], c[hi]) for a pair code (bits <= 3), or [256] for 4
     float *projT32;        // [128*128] entry [k*128+j] = S[j][k]  (query projection, score tile)
+    void *rfrag16;         // [32][64][8] fp16 +-1: D2 H D1 in 16x16x32 MFMA A-fragment order
+    float *symthr32;       // [2^(bits-1)]: middle boundary, then the positive boundaries
+    int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };
 
 static inline int tq_padded_dim(int d) {
