@@ -33,6 +33,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 D = 128
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the reading of a
+# 1 GiB device copy (x2.000 and x1.000); figures and commands in profiles/bench_kernels_c2_c3.txt.
+TRAFFIC_BYTES = {"store4": 85.0e6, "store3": 80.8e6, "decode3": 429.8e6}
 METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
 
 
@@ -127,7 +130,8 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         "workload": "fused decode attention, turbo3 K/V, B16 Hq32 Hkv8 d128 ctx 32768, queries rotated in-step",
         "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes_per_step": algo},
+                     "traffic": TRAFFIC_BYTES["decode3"], "algorithmic_bytes_per_step": algo,
+                     "kernel": "k_decode_attn<turbo3,turbo3> (+ k_prep_q, k_attn_combine in the step time)"},
         "buffer_sets": n_sets,
     }
 
@@ -148,12 +152,14 @@ def cpu_baseline(bits):
     v = rng.standard_normal((n, D)).astype(np.float16)
     s1, s2, _ = O.sign_diagonals(D, np.random.default_rng(42))
     cent = O.centroids_for(bits, D)
+    reps = 8                                          # 8 x (one head of K + one head of V) = all of config 2
     t0 = time.perf_counter()
-    for x, kind in ((k, "k"), (v, "v")):
-        idx, g, _ = O.turbo_encode(x, s1, s2, cent)
-        O.layout_pack(idx, g, bits, kind)
+    for _ in range(reps):
+        for x, kind in ((k, "k"), (v, "v")):
+            idx, g, _ = O.turbo_encode(x, s1, s2, cent)
+            O.layout_pack(idx, g, bits, kind)
     dt = time.perf_counter() - t0
-    algo = 2 * n * (256 + 16 * bits + 2)
+    algo = reps * 2 * n * (256 + 16 * bits + 2)
     # attention leg: one (batch, kv head) group of config 3, decompress -> softmax -> PV
     q = rng.standard_normal((4, D))
     idx, g, _ = O.turbo_encode(k, s1, s2, cent)
@@ -164,8 +170,8 @@ def cpu_baseline(bits):
     O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
     dta = time.perf_counter() - t0
     return ({"value": algo / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"NumPy oracle turbo{bits} encode+pack of 2 x 32768 fp16 vectors (1 of 8 heads of K and of V), "
-                       f"{dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
+             "sample": f"NumPy oracle turbo{bits} encode+pack of all 2 x 262144 fp16 vectors of config 2 "
+                       f"(8 passes over one head of K and one of V), {dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
              "host_cpus": os.cpu_count()},
             {"value": dta * 128 * 1e6, "unit": "µs/step", "cores": blas_threads or 1, "kind": "port",
              "sample": f"NumPy oracle decompress->softmax->PV for 1 of 128 (batch, kv-head) groups at ctx 32768 "
@@ -178,6 +184,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 1 GiB device copy (5x) so that FETCH_SIZE / WRITE_SIZE counters can be calibrated")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; every (batch, kv-head) group and every vector is an "
@@ -190,6 +198,13 @@ def main():
         sys.exit(3)
     torch.cuda.set_device(0)
 
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     s4 = store_leg(torch, tqa, 4, args.steps, args.warmup)
     s3 = store_leg(torch, tqa, 3, args.steps, args.warmup)
     dec = decode_leg(torch, tqa, args.steps, args.warmup)
@@ -206,7 +221,8 @@ def main():
         "config": {"workload": s4["workload"], "global_batch": 2 * 8 * 32768, "io": "fp16 in, 4-bit codes + fp16 norm out",
                    "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": s4["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s4["frac"],
-                     "traffic": None, "kernel": "k_store<4,half>", "kernel_us": s4["kernel_us"],
+                     "traffic": TRAFFIC_BYTES["store4"], "kernel": "k_store_mfma<4> (K and V instances)",
+                     "kernel_us": s4["kernel_us"],
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
         "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec,
