@@ -136,6 +136,69 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
     }
 
 
+def asym_decode_leg(torch, tqa, steps, warmup):
+    """BASELINE config 4: K q8_0-style (not rotated), V turbo2, B4 Hq32 Hkv8 ctx 131072, +6 logit bias
+    on 64 random key positions per head (given as an additive fp32 bias input), Sparse V tau 1e-6."""
+    B, Hq, Hkv, N = 4, 32, 8, 131072
+    vc = tqa.TurboCodec(2, seed=542)
+    kq = torch.empty(B * Hkv * (N // 128) * 128 * 136, dtype=torch.uint8, device="cuda")
+    vp = torch.empty(tqa.packed_bytes(2, B * Hkv, N), dtype=torch.uint8, device="cuda")
+    perk, perv = kq.numel() // (B * Hkv), vp.numel() // (B * Hkv)
+    for s in range(B * Hkv):                         # one (sequence, kv head) at a time keeps peak memory low
+        k = synth_kv(torch, 1, N, 400 + s, outliers=4)
+        v = synth_kv(torch, 1, N, 500 + s, outliers=0)
+        kq[s * perk:(s + 1) * perk] = tqa.q8_0_store(k)[0]
+        vc.store(v, kind="v", out=vp[s * perv:(s + 1) * perv])
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn((B, Hq, D), generator=g, device="cuda").to(torch.float16)
+    bias = torch.zeros((B, Hq, N), dtype=torch.float32, device="cuda")
+    pos = torch.stack([torch.randperm(N, generator=g, device="cuda")[:64] for _ in range(B * Hq)]).view(B, Hq, 64)
+    bias.scatter_(2, pos, 6.0)
+    out = {}
+    for name, tau in (("dense", 0.0), ("sparse_v", 1e-6)):
+        attn = tqa.DecodeAttention(None, vc, B, Hq, Hkv, N, sparse_v_tau=tau)
+        wall_ms, ev_ms = time_steps(torch, lambda i: attn(q, kq, vp, bias=bias), steps, warmup)
+        skip = attn.skip_rate() if tau else 0.0
+        algo = B * Hkv * N * (136 + (1.0 - 0.0) * 34)  # dense bytes; Sparse V skips whole 64-token V tiles only
+        us = ev_ms * 1e3
+        out[name] = {"us_per_step": us, "skip_rate": skip, "n_splits": attn.params.n_splits,
+                     "achieved_gbs": algo / (us * 1e-6) / 1e9, "frac": algo / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    out["workload"] = ("decode attention, K q8_0-style + V turbo2, B4 Hq32 Hkv8 ctx 131072, +6 bias on 64 key "
+                       "positions per head as an fp32 bias input (67 MB, not counted), Sparse V tau 1e-6")
+    out["algorithmic_bytes_per_step"] = B * Hkv * N * 170
+    return out
+
+
+def score_tile_leg(torch, tqa, steps, warmup):
+    """BASELINE config 5: 65536 keys as 3-bit codes + QJL sketch (Gaussian projection, seed 2), 2048 fp16
+    queries -> 2048 x 65536 logits through the K=256 MFMA contraction."""
+    nk, nq = 65536, 2048
+    g = torch.Generator(device="cuda").manual_seed(11)
+    keys = torch.randn((nk, D), generator=g, device="cuda", dtype=torch.float32)
+    qs = torch.randn((nq, D), generator=g, device="cuda").to(torch.float16)
+    codec = tqa.TurboCodec(3, seed=42, projection="gaussian", projection_seed=2)
+    packed, sbits, rn = codec.store_qjl(keys)
+    out = {"workload": "TurboQuant estimator tile, 65536 keys (3-bit + QJL, gaussian S seed 2) x 2048 fp16 queries"}
+    flops = 2.0 * nq * nk * 256
+    for name, dt in (("fp32_logits", torch.float32), ("fp16_logits", torch.float16)):
+        logits = None
+
+        def step(i):
+            nonlocal logits
+            logits = codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt)
+        wall_ms, ev_ms = time_steps(torch, step, max(5, steps // 10), 2)
+        out[name] = {"us_per_call": ev_ms * 1e3, "mfma_tflops": flops / (ev_ms * 1e-3) / 1e12,
+                     "mfma_frac_of_2500": flops / (ev_ms * 1e-3) / 2.5e15,
+                     "logit_store_gbs": logits.numel() * logits.element_size() / (ev_ms * 1e-3) / 1e9}
+        if dt == torch.float32:
+            exact = qs[:256].float() @ keys.t()
+            err = logits[:256] - exact
+            out["estimator_bias"] = float(err.mean())
+            out["estimator_rms_error"] = float(err.pow(2).mean().sqrt())
+            out["exact_rms"] = float(exact.pow(2).mean().sqrt())
+    return out
+
+
 def cpu_baseline(bits):
     """The NumPy oracle on a bounded sample of the store workload: one head of K
     and one head of V (2 x 32768 vectors), encode + pack, float64."""
@@ -208,6 +271,10 @@ def main():
     s4 = store_leg(torch, tqa, 4, args.steps, args.warmup)
     s3 = store_leg(torch, tqa, 3, args.steps, args.warmup)
     dec = decode_leg(torch, tqa, args.steps, args.warmup)
+    torch.cuda.empty_cache()
+    asym = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+    torch.cuda.empty_cache()
+    tile = score_tile_leg(torch, tqa, args.steps, args.warmup)
     if args.skip_cpu:
         cpu_store = cpu_attn = None
     else:
@@ -225,7 +292,8 @@ def main():
                      "kernel_us": s4["kernel_us"],
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
-        "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec,
+        "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec, "asym_decode_q8k_turbo2v": asym,
+        "score_tile": tile,
     }
     print(json.dumps(line, ensure_ascii=False))
 

@@ -512,13 +512,13 @@ def boundary_band_mismatches(y, idx_test, centroids, rel=1e-6):
 # A ROW holds 64 pair codes (128 values) in 16*b bytes; pair p = (lo | hi << b).
 #   b = 4 : byte p of the row.                      (64 B, 4 pairs per dword)
 #   b = 2 : nibble p%8 of dword p//8.               (32 B, 8 pairs per dword)
-#   b = 3 : pairs 0..59 sit five to a dword (pair p in bits 6*(p%5).. of dword
-#           p//5); pair 60+q takes bits 30..31 of dwords 3q, 3q+1, 3q+2 as its
-#           low, middle and high two bits.           (48 B)
+#   b = 3 : four groups of 16 pairs, three dwords each: pair p = 16g + k sits for
+#           k < 15 in dword 3g + k//5 at bit 6*(k%5); pair 16g + 15 takes bits
+#           30..31 of dwords 3g, 3g+1, 3g+2 as its low, middle and high two bits. (48 B)
 # K rows: row = token, pair p = dims (2p, 2p+1).
 # V rows are dim-major inside each 64-token tile: row (token & 64) | (dim & 63)
-#         holds dims r and 64+r of the tile's 64 tokens; pair 32*(dim >> 6) + tp =
-#         tokens 2*tp and 2*tp+1 of the tile (lo, hi).
+#         holds dims r and 64+r of the tile's 64 tokens; tokens 2*tp and 2*tp+1 of
+#         the tile (lo, hi) of dim half hf = dim >> 6 are pair 16*(tp//8) + 2*(tp%8) + hf.
 # A BLOCK is 128 rows stored chunk-major: [16*b/16 chunks][128 rows][16 B],
 # followed by 128 fp16 norms (token order).  Block bytes = 128*(16*b + 2).
 
@@ -548,13 +548,12 @@ def _pairs_to_rows(pairs: np.ndarray, bits: int) -> np.ndarray:
         return out
     if bits == 3:
         out = np.zeros(lead + (12,), dtype=np.uint32)
-        body = pairs[..., :60].reshape(lead + (12, 5))
-        for k in range(5):
-            out |= body[..., k] << np.uint32(6 * k)
-        for q in range(4):
-            t = pairs[..., 60 + q]
+        grp = pairs.reshape(lead + (4, 16))
+        for g in range(4):
+            for k in range(15):
+                out[..., 3 * g + k // 5] |= grp[..., g, k] << np.uint32(6 * (k % 5))
             for part in range(3):
-                out[..., 3 * q + part] |= ((t >> np.uint32(2 * part)) & np.uint32(3)) << np.uint32(30)
+                out[..., 3 * g + part] |= ((grp[..., g, 15] >> np.uint32(2 * part)) & np.uint32(3)) << np.uint32(30)
         return out
     raise ValueError("bits must be 2, 3 or 4")
 
@@ -569,12 +568,13 @@ def _rows_to_pairs(rows: np.ndarray, bits: int) -> np.ndarray:
         return np.stack([(rows >> np.uint32(4 * k)) & np.uint32(0xF) for k in range(8)],
                         axis=-1).reshape(lead + (64,))
     if bits == 3:
-        body = np.stack([(rows >> np.uint32(6 * k)) & np.uint32(0x3F) for k in range(5)],
-                        axis=-1).reshape(lead + (60,))
+        cols = []
         top = (rows >> np.uint32(30)) & np.uint32(3)
-        tail = np.stack([top[..., 3 * q] | (top[..., 3 * q + 1] << 2) | (top[..., 3 * q + 2] << 4)
-                         for q in range(4)], axis=-1)
-        return np.concatenate([body, tail], axis=-1)
+        for g in range(4):
+            for k in range(15):
+                cols.append((rows[..., 3 * g + k // 5] >> np.uint32(6 * (k % 5))) & np.uint32(0x3F))
+            cols.append(top[..., 3 * g] | (top[..., 3 * g + 1] << 2) | (top[..., 3 * g + 2] << 4))
+        return np.stack(cols, axis=-1)
     raise ValueError("bits must be 2, 3 or 4")
 
 
@@ -588,9 +588,9 @@ def layout_pack(idx: np.ndarray, g: np.ndarray, bits: int, kind: str) -> np.ndar
         pairs = idx[:, 0::2] | (idx[:, 1::2] << np.uint32(bits))          # [T,64]
     else:
         q = idx.reshape(T // 64, 32, 2, 2, 64)                             # tile, token pair, parity, dim half, r
-        lo = q[:, :, 0].transpose(0, 3, 2, 1)                              # tile, r, dim half, token pair
-        hi = q[:, :, 1].transpose(0, 3, 2, 1)
-        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row = 64*tile + r; pair = 32*half + tp
+        lo = q[:, :, 0].transpose(0, 3, 1, 2)                              # tile, r, token pair, dim half
+        hi = q[:, :, 1].transpose(0, 3, 1, 2)
+        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row = 64*tile + r; pair = 2*tp + half
     rows = _pairs_to_rows(pairs, bits)                                     # [T, 4*bits]
     rows = rows.reshape(nb, ROWS_PER_BLOCK, bits, 4).transpose(0, 2, 1, 3) # block, chunk, row, 4
     out = np.zeros((nb, block_bytes(bits)), dtype=np.uint8)
@@ -619,8 +619,8 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
         idx[:, 1::2] = hi
     else:
         q = np.zeros((T // 64, 32, 2, 2, 64), dtype=np.uint8)              # tile, token pair, parity, dim half, r
-        q[:, :, 0] = lo.reshape(T // 64, 64, 2, 32).transpose(0, 3, 2, 1)
-        q[:, :, 1] = hi.reshape(T // 64, 64, 2, 32).transpose(0, 3, 2, 1)
+        q[:, :, 0] = lo.reshape(T // 64, 64, 32, 2).transpose(0, 2, 3, 1)
+        q[:, :, 1] = hi.reshape(T // 64, 64, 32, 2).transpose(0, 2, 3, 1)
         idx = q.reshape(T, 128)
     return idx, g
 

@@ -156,7 +156,7 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
     if kind == "k":
         row, pair, half = tok, dim // 2, dim % 2
     else:
-        row, pair, half = (tok & 64) | (dim & 63), 32 * (dim >> 6) + (tok & 63) // 2, tok % 2
+        row, pair, half = (tok & 64) | (dim & 63), 2 * ((tok & 63) // 2) + (dim >> 6), tok % 2
     value = ((1 << bits) - 1) << (bits * half)
     rowwords = words[:, row, :].reshape(-1)
     expect = np.zeros(4 * bits, dtype=np.uint64)
@@ -164,11 +164,11 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
         expect[pair // 4] = value << (8 * (pair % 4))
     elif bits == 2:
         expect[pair // 8] = value << (4 * (pair % 8))
-    elif pair < 60:
-        expect[pair // 5] = value << (6 * (pair % 5))
+    elif pair % 16 < 15:
+        expect[3 * (pair // 16) + (pair % 16) // 5] = value << (6 * ((pair % 16) % 5))
     else:
         for part in range(3):
-            expect[3 * (pair - 60) + part] = ((value >> (2 * part)) & 3) << 30
+            expect[3 * (pair // 16) + part] = ((value >> (2 * part)) & 3) << 30
     assert np.array_equal(rowwords.astype(np.uint64), expect)
     assert np.count_nonzero(words) == np.count_nonzero(expect)
 

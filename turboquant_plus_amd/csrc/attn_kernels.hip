@@ -22,7 +22,8 @@
 //         end of the split and no LDS traffic besides the LUT reads.
 //   Online softmax in base 2 (log2(e) folded into the query scale).
 // k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
-//   the V rotation (one wavefront per query head).
+//   the V rotation (one workgroup per query head).  Queries are rotated and scaled
+//   inside k_decode_attn by each wavefront, so a dense step is two launches.
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
 #include <utility>
@@ -48,12 +49,12 @@ template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t 
         const int q = p >> 3, k = p & 7;
         return k == 0 ? ((w[q] << 2) & 0x3Cu) : ((w[q] >> (4 * k - 2)) & 0x3Cu);
     } else {
-        if (p < 60) {
-            const int q = p / 5, k = p % 5;
+        const int g = p >> 4, kk = p & 15;
+        if (kk < 15) {
+            const int q = 3 * g + kk / 5, k = kk % 5;
             return k == 0 ? ((w[q] << 2) & 0xFCu) : ((w[q] >> (6 * k - 2)) & 0xFCu);
         }
-        const int t = p - 60;
-        return ((w[3 * t] >> 28) & 0xCu) | ((w[3 * t + 1] >> 26) & 0x30u) | ((w[3 * t + 2] >> 24) & 0xC0u);
+        return ((w[3 * g] >> 28) & 0xCu) | ((w[3 * g + 1] >> 26) & 0x30u) | ((w[3 * g + 2] >> 24) & 0xC0u);
     }
 }
 
@@ -115,7 +116,10 @@ __device__ __forceinline__ float max_over_blocks(float v) {
 }
 
 struct AttnArgs {
-    const __half *qrot;  // [groups*4][128], rotated by the K rotation (turbo K), scaled by scale*log2(e)
+    const void *q;       // [groups*4][128] queries in the original domain, q_dtype
+    int q_dtype;
+    const float *ks1, *ks2;  // K rotation signs (NULL: K is not rotated, q is only scaled)
+    float scale_log2e;       // logit scale * log2(e), folded into the fp16 query
     const uint8_t *k, *v;
     const uint32_t *klut, *vlut;  // pair LUTs (half2 per pair code)
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
@@ -160,15 +164,16 @@ __device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const ui
 template <int BITS, int... T>
 __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const uint32_t (&vw)[4 * BITS],
                                        const char *lut, half4_t pv, float4_t (&acc_o)[2][2]) {
+    // tokens 4T..4T+3 of dim half hf are pairs 4T + hf and 4T + 2 + hf of the row
     ((acc_o[0][T & 1] = mfma4_bcast<T>(
           pv,
-          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 2 * T)),
-                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 2 * T + 1))),
+          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T)),
+                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 2))),
           acc_o[0][T & 1]),
       acc_o[1][T & 1] = mfma4_bcast<T>(
           pv,
-          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 32 + 2 * T)),
-                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 32 + 2 * T + 1))),
+          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 1)),
+                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 3))),
           acc_o[1][T & 1])),
      ...);
 }
@@ -182,6 +187,7 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     constexpr int VLUT_N = 1 << (2 * VBITS);
     __shared__ uint32_t klut_s[KLUT_N];
     __shared__ uint32_t vlut_s[VLUT_N];
+    __shared__ __attribute__((aligned(16))) _Float16 q_s[4][4 * 128];  // per wavefront: its group's rotated queries
 
     const int tid = threadIdx.x, lane = tid & 63;
     if constexpr (KFMT == KFMT_TURBO)
@@ -202,9 +208,42 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
 
     // A operand of QK, broadcast from one block per MFMA: lane (b, i) keeps q[head i] for the
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
+    // The wavefront first rotates its group's four queries itself (four 128-point butterflies,
+    // two values per lane), scales them and parks them as fp16 in 1 KB of LDS.
     half4_t qa[2];
     {
-        const uint2 *qp = reinterpret_cast<const uint2 *>(a.qrot + ((int64_t)group * 4 + j) * 128);
+        _Float16 *qw = q_s[tid >> 6];
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const int64_t e = ((int64_t)group * 4 + h) * 128 + 2 * lane;
+            float x0, x1;
+            if (a.q_dtype == TQ_F16) {
+                const __half *qp = reinterpret_cast<const __half *>(a.q);
+                x0 = __half2float(qp[e]);
+                x1 = __half2float(qp[e + 1]);
+            } else if (a.q_dtype == TQ_F32) {
+                const float *qp = reinterpret_cast<const float *>(a.q);
+                x0 = qp[e];
+                x1 = qp[e + 1];
+            } else {
+                const double *qp = reinterpret_cast<const double *>(a.q);
+                x0 = (float)qp[e];
+                x1 = (float)qp[e + 1];
+            }
+            if (a.ks1) {
+                x0 *= a.ks1[2 * lane];
+                x1 *= a.ks1[2 * lane + 1];
+                wht128_wave(x0, x1, lane);
+                x0 *= a.ks2[2 * lane] * RSQRT128;
+                x1 *= a.ks2[2 * lane + 1] * RSQRT128;
+            }
+            qw[h * 128 + 2 * lane] = (_Float16)(x0 * a.scale_log2e);
+            qw[h * 128 + 2 * lane + 1] = (_Float16)(x1 * a.scale_log2e);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint2 *qp = reinterpret_cast<const uint2 *>(qw + j * 128);
         qa[0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
         qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
@@ -335,8 +374,8 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
         pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
         pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
-        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; pair 32*hf + 2T (+1)
-        // = tokens 4T..4T+3.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
+        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; pairs 4T + hf and
+        // 4T + 2 + hf = tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
         // weights of token group T sit in block T and are broadcast to every block.
         pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
         if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
@@ -359,38 +398,22 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     }
 }
 
-// q -> rotated, scaled fp16 (one wavefront per query row); also clears the skip counter
-template <typename TI>
-__global__ __launch_bounds__(256) void k_prep_q(const TI *q, __half *qrot, int64_t n, const float *s1, const float *s2,
-                                                float scale_log2e, int rotate, unsigned long long *skip,
-                                                unsigned long long total_pairs) {
-    const int lane = threadIdx.x & 63;
-    const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (skip && blockIdx.x == 0 && threadIdx.x == 0) {
-        skip[0] = 0ull;
-        skip[1] = total_pairs;
-    }
-    if (v >= n) return;
-    float x0 = ldf(q + v * 128 + 2 * lane), x1 = ldf(q + v * 128 + 2 * lane + 1);
-    if (rotate) {
-        x0 *= s1[2 * lane];
-        x1 *= s1[2 * lane + 1];
-        wht128_wave(x0, x1, lane);
-        x0 *= s2[2 * lane] * RSQRT128;
-        x1 *= s2[2 * lane + 1] * RSQRT128;
-    }
-    qrot[v * 128 + 2 * lane] = __float2half_rn(x0 * scale_log2e);
-    qrot[v * 128 + 2 * lane + 1] = __float2half_rn(x1 * scale_log2e);
+// Sparse-V bookkeeping: {skipped pairs, total pairs}; a fill kernel rather than a memset so that
+// the sequence stays safe to capture in a HIP graph.
+__global__ void k_clear_skip(unsigned long long *skip, unsigned long long total_pairs) {
+    skip[0] = 0ull;
+    skip[1] = total_pairs;
 }
 
-// merge split partials, un-rotate with the V rotation's transpose; one wavefront per query head.
-// Lane s first fetches (m, l) of split s (64 splits per pass), so the weights of all splits are
-// known after one round trip; the partial outputs are then streamed with independent loads.
+// merge split partials, un-rotate with the V rotation's transpose; one workgroup of four
+// wavefronts per query head.  Every wavefront fetches (m, l) of all splits (lane s <-> split s,
+// 64 per pass) so the weights are known after one round trip, streams the partial outputs of
+// its quarter of the splits with independent loads, and wavefront 0 adds the four quarters.
 __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
                                                       int64_t n_rows, int n_splits, const float *s1, const float *s2) {
-    const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
-    if (r >= n_rows) return;
+    __shared__ float red[4][130];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t r = blockIdx.x;  // row = group*4 + head
     const int64_t group = r >> 2;
     const int head = (int)(r & 3);
     const float *ml = part_ml + (group * n_splits * 4 + head) * 2;   // + s*8
@@ -416,13 +439,19 @@ __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const
         L += lw;
         const int cnt = min(64, n_splits - s0);
 #pragma unroll 8
-        for (int t = 0; t < cnt; ++t) {
+        for (int t = wv; t < cnt; t += 4) {
             const float wt = __shfl(w, t);
             const float2 v = *reinterpret_cast<const float2 *>(po + (int64_t)(s0 + t) * 512 + 2 * lane);
             o0 = fmaf(v.x, wt, o0);
             o1 = fmaf(v.y, wt, o1);
         }
     }
+    red[wv][2 * lane] = o0;
+    red[wv][2 * lane + 1] = o1;
+    __syncthreads();
+    if (wv != 0) return;
+    o0 = (red[0][2 * lane] + red[1][2 * lane]) + (red[2][2 * lane] + red[3][2 * lane]);
+    o1 = (red[0][2 * lane + 1] + red[1][2 * lane + 1]) + (red[2][2 * lane + 1] + red[3][2 * lane + 1]);
     const float invL = L > 0.0f ? 1.0f / L : 0.0f;
     o0 *= invL * s2[2 * lane];
     o1 *= invL * s2[2 * lane + 1];
@@ -462,31 +491,28 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     }
     const int64_t rows = (int64_t)p->batch * p->n_q_heads;
     const int groups = p->batch * p->n_kv_heads;
-    __half *qrot = reinterpret_cast<__half *>((char *)ws + w.qrot);
     float *part_o = reinterpret_cast<float *>((char *)ws + w.part_o);
     float *part_ml = reinterpret_cast<float *>((char *)ws + w.part_ml);
     const bool turbo_k = p->k_format == TQ_KFMT_TURBO;
     const float sc = p->scale * LOG2E;
     const unsigned long long total_pairs = (unsigned long long)rows * (unsigned long long)p->tokens;
-    const unsigned qgrid = (unsigned)((rows + 3) / 4);
-    const float *ks1 = turbo_k ? hk->s1_32 : nullptr, *ks2 = turbo_k ? hk->s2_32 : nullptr;
-    switch (q_dtype) {
-    case TQ_F16:
-        k_prep_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
-        break;
-    case TQ_F32:
-        k_prep_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
-        break;
-    case TQ_F64:
-        k_prep_q<double><<<qgrid, 256, 0, s>>>((const double *)q, qrot, rows, ks1, ks2, sc, turbo_k, skip_count, total_pairs);
-        break;
-    default: tq_set_error("bad q dtype %d", q_dtype); return TQ_ERR_ARG;
+    int rc = TQ_OK;
+    if (skip_count) {
+        k_clear_skip<<<1, 1, 0, s>>>(skip_count, total_pairs);
+        rc = tq_check_launch("clear_skip");
+        if (rc) return rc;
     }
-    int rc = tq_check_launch("prep_q");
-    if (rc) return rc;
+    if (q_dtype != TQ_F16 && q_dtype != TQ_F32 && q_dtype != TQ_F64) {
+        tq_set_error("bad q dtype %d", q_dtype);
+        return TQ_ERR_ARG;
+    }
 
     AttnArgs a;
-    a.qrot = qrot;
+    a.q = q;
+    a.q_dtype = q_dtype;
+    a.ks1 = turbo_k ? hk->s1_32 : nullptr;
+    a.ks2 = turbo_k ? hk->s2_32 : nullptr;
+    a.scale_log2e = sc;
     a.k = (const uint8_t *)k;
     a.v = (const uint8_t *)v;
     a.klut = turbo_k ? (const uint32_t *)hk->pair_lut : nullptr;
@@ -528,7 +554,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 #undef TQ_ATTN
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
-    k_attn_combine<<<qgrid, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
+    k_attn_combine<<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
     return tq_check_launch("attn_combine");
 }
 

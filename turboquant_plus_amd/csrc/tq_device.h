@@ -111,12 +111,13 @@ __device__ inline void wht128_wave(float &a, float &b, int lane) {
 // A row holds 64 pair codes (128 values) in 4*BITS dwords; pair = lo | hi << BITS.
 //   BITS 4: pair p = byte p%4 of dword p/4
 //   BITS 2: pair p = nibble p%8 of dword p/8
-//   BITS 3: pairs 0..59 five to a dword at bit 6*(p%5); pair 60+t = bits 30..31 of
-//           dwords 3t, 3t+1, 3t+2 (low, middle, high two bits)
+//   BITS 3: four groups of 16 pairs in three dwords each: pair 16g + k, k < 15, at bit
+//           6*(k%5) of dword 3g + k/5; pair 16g + 15 = bits 30..31 of dwords 3g, 3g+1,
+//           3g+2 (low, middle, high two bits)
 // A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
 // norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows are dim-major
 // inside each 64-token tile: row (token & 64) | (dim & 63) holds dims r and 64+r
-// of the tile's tokens; pair 32*(dim >> 6) + tp = tokens 2tp, 2tp+1 of the tile.
+// of the tile's tokens; pair 2*tp + (dim >> 6) = tokens 2tp, 2tp+1 of the tile.
 __host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
 __host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
 __host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
@@ -133,13 +134,13 @@ template <int BITS, int P> __device__ inline uint32_t pair_lut_offset(const uint
         else return (w[q] >> (4 * k - 2)) & 0x3Cu;
     } else {
         static_assert(BITS == 3, "bits");
-        if constexpr (P < 60) {
-            constexpr int q = P / 5, k = P % 5;
+        constexpr int g = P >> 4, kk = P & 15;
+        if constexpr (kk < 15) {
+            constexpr int q = 3 * g + kk / 5, k = kk % 5;
             if constexpr (k == 0) return (w[q] << 2) & 0xFCu;
             else return (w[q] >> (6 * k - 2)) & 0xFCu;
         } else {
-            constexpr int t = P - 60;
-            return ((w[3 * t] >> 28) & 0xCu) | ((w[3 * t + 1] >> 26) & 0x30u) | ((w[3 * t + 2] >> 24) & 0xC0u);
+            return ((w[3 * g] >> 28) & 0xCu) | ((w[3 * g + 1] >> 26) & 0x30u) | ((w[3 * g + 2] >> 24) & 0xC0u);
         }
     }
 }
@@ -148,9 +149,9 @@ template <int BITS, int P> __device__ inline uint32_t pair_lut_offset(const uint
 __device__ inline uint32_t pair_code(const uint32_t *w, int bits, int p) {
     if (bits == 4) return (w[p >> 2] >> (8 * (p & 3))) & 0xFFu;
     if (bits == 2) return (w[p >> 3] >> (4 * (p & 7))) & 0xFu;
-    if (p < 60) return (w[p / 5] >> (6 * (p % 5))) & 0x3Fu;
-    const int t = p - 60;
-    return (w[3 * t] >> 30) | ((w[3 * t + 1] >> 30) << 2) | ((w[3 * t + 2] >> 30) << 4);
+    const int g = p >> 4, k = p & 15;
+    if (k < 15) return (w[3 * g + k / 5] >> (6 * (k % 5))) & 0x3Fu;
+    return (w[3 * g] >> 30) | ((w[3 * g + 1] >> 30) << 2) | ((w[3 * g + 2] >> 30) << 4);
 }
 
 // (row, pair, half) of the code of (token, dim) inside its 128-token block
@@ -161,7 +162,7 @@ __device__ inline void locate(int kind, int token, int dim, int &row, int &pair,
         half = dim & 1;
     } else {
         row = (token & 64) | (dim & 63);
-        pair = ((dim >> 6) << 5) | ((token & 63) >> 1);
+        pair = (token & 62) | (dim >> 6);
         half = token & 1;
     }
 }

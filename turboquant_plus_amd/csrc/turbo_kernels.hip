@@ -94,8 +94,8 @@ template <int BITS> __device__ inline uint32_t pair_from_stage(const uint8_t *co
         lo = codes[row * CODE_STRIDE + 2 * p];
         hi = codes[row * CODE_STRIDE + 2 * p + 1];
     } else {
-        const int tok = (row & 64) + 2 * (p & 31);
-        const int dim = ((p >> 5) << 6) | (row & 63);
+        const int tok = (row & 64) + (p & 62);
+        const int dim = ((p & 1) << 6) | (row & 63);
         lo = codes[tok * CODE_STRIDE + dim];
         hi = codes[(tok + 1) * CODE_STRIDE + dim];
     }
@@ -117,10 +117,11 @@ __device__ inline void pack_block(const uint8_t *codes, const float *norms, uint
 #pragma unroll
             for (int t = 0; t < 8; ++t) word |= pair_from_stage<2>(codes, kind, r, 8 * q + t) << (4 * t);
         } else {
+            const int g = q / 3, j = q % 3;  // group of 16 pairs, dword inside the group
 #pragma unroll
-            for (int t = 0; t < 5; ++t) word |= pair_from_stage<3>(codes, kind, r, 5 * q + t) << (6 * t);
-            const uint32_t tail = pair_from_stage<3>(codes, kind, r, 60 + q / 3);
-            word |= ((tail >> (2 * (q % 3))) & 3u) << 30;
+            for (int t = 0; t < 5; ++t) word |= pair_from_stage<3>(codes, kind, r, 16 * g + 5 * j + t) << (6 * t);
+            const uint32_t tail = pair_from_stage<3>(codes, kind, r, 16 * g + 15);
+            word |= ((tail >> (2 * j)) & 3u) << 30;
         }
         out[o] = word;
     }
@@ -203,12 +204,12 @@ template <int BITS> __device__ __forceinline__ void pack_row_from_nibbles(const 
     } else {
         uint32_t tail[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) tail[t] = pair(60 + t);
+        for (int t = 0; t < 4; ++t) tail[t] = pair(16 * t + 15);
 #pragma unroll
         for (int q = 0; q < 12; ++q) {
             uint32_t w = ((tail[q / 3] >> (2 * (q % 3))) & 3u) << 30;
 #pragma unroll
-            for (int t = 0; t < 5; ++t) w |= pair(5 * q + t) << (6 * t);
+            for (int t = 0; t < 5; ++t) w |= pair(16 * (q / 3) + 5 * (q % 3) + t) << (6 * t);
             out[q] = w;
         }
     }
@@ -342,8 +343,7 @@ __global__ __launch_bounds__(256, 3) void k_store_mfma(const __half *x, uint8_t 
             }
             pack_row_from_nibbles<BITS>(nib, out);
         } else {
-            // row l = dims l and 64+l; nibble position of the row's code (hf, token): hf*64 + token,
-            // so that pair 32*hf + tp = tokens (2tp, 2tp+1) as the V layout wants
+            // row l = dims l and 64+l; the row's pair 2*tp + hf = tokens (2tp, 2tp+1) of dim half hf
             uint32_t nib[16];
 #pragma unroll
             for (int q = 0; q < 16; ++q) nib[q] = 0;
@@ -353,7 +353,8 @@ __global__ __launch_bounds__(256, 3) void k_store_mfma(const __half *x, uint8_t 
 #pragma unroll
                 for (int tok = 0; tok < 64; ++tok) {
                     const uint32_t c = (st[tok * STAGE_STRIDE + col] >> sh) & 0xFu;
-                    nib[(hf * 64 + tok) >> 3] |= c << (4 * (tok & 7));
+                    const int pos = 4 * (tok >> 1) + 2 * hf + (tok & 1);  // nibble of pair 2*tp + hf, half tok&1
+                    nib[pos >> 3] |= c << (4 * (pos & 7));
                 }
             }
             pack_row_from_nibbles<BITS>(nib, out);
@@ -545,11 +546,11 @@ __device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, 
     uint32_t pc;
     if (bits == 4) pc = (row_dword(block, row, p >> 2) >> (8 * (p & 3))) & 0xFFu;
     else if (bits == 2) pc = (row_dword(block, row, p >> 3) >> (4 * (p & 7))) & 0xFu;
-    else if (p < 60) pc = (row_dword(block, row, p / 5) >> (6 * (p % 5))) & 0x3Fu;
+    else if ((p & 15) < 15) pc = (row_dword(block, row, 3 * (p >> 4) + (p & 15) / 5) >> (6 * ((p & 15) % 5))) & 0x3Fu;
     else {
-        const int t = p - 60;
-        pc = (row_dword(block, row, 3 * t) >> 30) | ((row_dword(block, row, 3 * t + 1) >> 30) << 2) |
-             ((row_dword(block, row, 3 * t + 2) >> 30) << 4);
+        const int g = p >> 4;
+        pc = (row_dword(block, row, 3 * g) >> 30) | ((row_dword(block, row, 3 * g + 1) >> 30) << 2) |
+             ((row_dword(block, row, 3 * g + 2) >> 30) << 4);
     }
     return (pc >> (half * bits)) & ((1u << bits) - 1u);
 }

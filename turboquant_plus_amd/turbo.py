@@ -211,7 +211,9 @@ class DecodeAttention:
         hk = self.k_codec.handle.h if self.k_codec is not None else None
         L.check(L.lib().tq_decode_attention(hk, self.v_codec.handle.h, C.byref(self.params), L.ptr(qd),
                                             L.dtype_code(qd), L.ptr(k_packed), None, L.ptr(v_packed), L.ptr(bias),
-                                            L.ptr(self.out), L.ptr(self.skip), L.ptr(self.workspace),
+                                            L.ptr(self.out),
+                                            L.ptr(self.skip if self.params.sparse_v_tau > 0 else None),
+                                            L.ptr(self.workspace),
                                             self.workspace.numel(), L.stream_ptr()))
         return self.out
 
