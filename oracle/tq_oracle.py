@@ -510,15 +510,17 @@ def boundary_band_mismatches(y, idx_test, centroids, rel=1e-6):
 
 # ---- device layout: "pair containers" in 128-token blocks ------------------
 # A ROW holds 64 pair codes (128 values) in 16*b bytes; pair p = (lo | hi << b).
-#   b = 4 : byte p of the row.                      (64 B, 4 pairs per dword)
-#   b = 2 : nibble p%8 of dword p//8.               (32 B, 8 pairs per dword)
-#   b = 3 : four groups of 16 pairs, three dwords each: pair p = 16g + k sits for
-#           k < 15 in dword 3g + k//5 at bit 6*(k%5); pair 16g + 15 takes bits
-#           30..31 of dwords 3g, 3g+1, 3g+2 as its low, middle and high two bits. (48 B)
+# A row is four groups of 16 pairs (group g = pairs 16g..16g+15); a group owns b
+# dwords, and dword j of group g is row dword 4j + g, i.e. 16-byte chunk j of the row
+# holds dword j of the four groups.  Inside a group, pair k sits in
+#   b = 4 : byte k%4 of dword k//4
+#   b = 2 : nibble k%8 of dword k//8
+#   b = 3 : bits 6*(k%5).. of dword k//5 for k < 15; pair 15 takes bits 30..31 of
+#           dwords 0, 1, 2 as its low, middle and high two bits.
 # K rows: row = token, pair p = dims (2p, 2p+1).
 # V rows are dim-major inside each 64-token tile: row (token & 64) | (dim & 63)
 #         holds dims r and 64+r of the tile's 64 tokens; tokens 2*tp and 2*tp+1 of
-#         the tile (lo, hi) of dim half hf = dim >> 6 are pair 16*(tp//8) + 2*(tp%8) + hf.
+#         the tile (lo, hi) of dim half hf = dim >> 6 are pair 2*tp + hf.
 # A BLOCK is 128 rows stored chunk-major: [16*b/16 chunks][128 rows][16 B],
 # followed by 128 fp16 norms (token order).  Block bytes = 128*(16*b + 2).
 
@@ -534,48 +536,44 @@ def block_bytes(bits: int) -> int:
 
 
 def _pairs_to_rows(pairs: np.ndarray, bits: int) -> np.ndarray:
-    """pairs [..., 64] (values < 4**bits) -> row dwords [..., 4*bits] uint32."""
+    """pairs [..., 64] (values < 4**bits) -> row dwords [..., 4*bits] uint32.
+
+    A row is four groups of 16 pairs; group g owns `bits` dwords, and dword j
+    of group g is row dword 4*j + g (so 16-byte chunk j of the row holds dword
+    j of the four groups).  Inside a group: 4-bit pair k = byte k%4 of dword
+    k/4; 2-bit pair k = nibble k%8 of dword k/8; 3-bit pair k < 15 = bits
+    6*(k%5).. of dword k/5, pair 15 = bits 30..31 of dwords 0, 1, 2 (low,
+    middle, high two bits)."""
     pairs = pairs.astype(np.uint32)
     lead = pairs.shape[:-1]
-    if bits == 4:
-        p = pairs.reshape(lead + (16, 4))
-        return p[..., 0] | (p[..., 1] << 8) | (p[..., 2] << 16) | (p[..., 3] << 24)
-    if bits == 2:
-        p = pairs.reshape(lead + (8, 8))
-        out = np.zeros(lead + (8,), dtype=np.uint32)
-        for k in range(8):
-            out |= p[..., k] << np.uint32(4 * k)
-        return out
-    if bits == 3:
-        out = np.zeros(lead + (12,), dtype=np.uint32)
-        grp = pairs.reshape(lead + (4, 16))
-        for g in range(4):
-            for k in range(15):
-                out[..., 3 * g + k // 5] |= grp[..., g, k] << np.uint32(6 * (k % 5))
+    grp = pairs.reshape(lead + (4, 16))
+    out = np.zeros(lead + (4 * bits,), dtype=np.uint32)
+    if bits not in (2, 3, 4):
+        raise ValueError("bits must be 2, 3 or 4")
+    per, width = {4: (4, 8), 2: (8, 4), 3: (5, 6)}[bits]
+    for g in range(4):
+        for k in range(16 if bits != 3 else 15):
+            out[..., 4 * (k // per) + g] |= grp[..., g, k] << np.uint32(width * (k % per))
+        if bits == 3:
             for part in range(3):
-                out[..., 3 * g + part] |= ((grp[..., g, 15] >> np.uint32(2 * part)) & np.uint32(3)) << np.uint32(30)
-        return out
-    raise ValueError("bits must be 2, 3 or 4")
+                out[..., 4 * part + g] |= ((grp[..., g, 15] >> np.uint32(2 * part)) & np.uint32(3)) << np.uint32(30)
+    return out
 
 
 def _rows_to_pairs(rows: np.ndarray, bits: int) -> np.ndarray:
     rows = rows.astype(np.uint32)
-    lead = rows.shape[:-1]
-    if bits == 4:
-        return np.stack([(rows >> np.uint32(8 * k)) & np.uint32(0xFF) for k in range(4)],
-                        axis=-1).reshape(lead + (64,))
-    if bits == 2:
-        return np.stack([(rows >> np.uint32(4 * k)) & np.uint32(0xF) for k in range(8)],
-                        axis=-1).reshape(lead + (64,))
-    if bits == 3:
-        cols = []
-        top = (rows >> np.uint32(30)) & np.uint32(3)
-        for g in range(4):
-            for k in range(15):
-                cols.append((rows[..., 3 * g + k // 5] >> np.uint32(6 * (k % 5))) & np.uint32(0x3F))
-            cols.append(top[..., 3 * g] | (top[..., 3 * g + 1] << 2) | (top[..., 3 * g + 2] << 4))
-        return np.stack(cols, axis=-1)
-    raise ValueError("bits must be 2, 3 or 4")
+    if bits not in (2, 3, 4):
+        raise ValueError("bits must be 2, 3 or 4")
+    per, width = {4: (4, 8), 2: (8, 4), 3: (5, 6)}[bits]
+    mask = np.uint32((1 << width) - 1)
+    cols = []
+    for g in range(4):
+        for k in range(16 if bits != 3 else 15):
+            cols.append((rows[..., 4 * (k // per) + g] >> np.uint32(width * (k % per))) & mask)
+        if bits == 3:
+            top = [(rows[..., 4 * part + g] >> np.uint32(30)) & np.uint32(3) for part in range(3)]
+            cols.append(top[0] | (top[1] << np.uint32(2)) | (top[2] << np.uint32(4)))
+    return np.stack(cols, axis=-1)
 
 
 def layout_pack(idx: np.ndarray, g: np.ndarray, bits: int, kind: str) -> np.ndarray:

@@ -148,29 +148,30 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
     i2, g2 = O.layout_unpack(buf, bits, kind)
     assert np.array_equal(i2, idx) and np.array_equal(g2.view(np.uint16), g.view(np.uint16))
     # one-hot placement: a single non-zero code lands where the layout says
-    one = np.zeros((128, 128), dtype=np.uint8)
-    tok, dim = 77, 45
-    one[tok, dim] = (1 << bits) - 1
-    b = O.layout_pack(one, np.zeros(128, dtype=np.float16), bits, kind)
-    words = b[:128 * 16 * bits].view("<u4").reshape(bits, 128, 4)
-    if kind == "k":
-        row, pair, half = tok, dim // 2, dim % 2
-    else:
-        row, pair, half = (tok & 64) | (dim & 63), 2 * ((tok & 63) // 2) + (dim >> 6), tok % 2
-    value = ((1 << bits) - 1) << (bits * half)
-    rowwords = words[:, row, :].reshape(-1)
-    expect = np.zeros(4 * bits, dtype=np.uint64)
-    if bits == 4:
-        expect[pair // 4] = value << (8 * (pair % 4))
-    elif bits == 2:
-        expect[pair // 8] = value << (4 * (pair % 8))
-    elif pair % 16 < 15:
-        expect[3 * (pair // 16) + (pair % 16) // 5] = value << (6 * ((pair % 16) % 5))
-    else:
-        for part in range(3):
-            expect[3 * (pair // 16) + part] = ((value >> (2 * part)) & 3) << 30
-    assert np.array_equal(rowwords.astype(np.uint64), expect)
-    assert np.count_nonzero(words) == np.count_nonzero(expect)
+    for tok, dim in [(77, 45), (5, 31), (64, 127), (127, 94), (0, 0)]:
+        one = np.zeros((128, 128), dtype=np.uint8)
+        one[tok, dim] = (1 << bits) - 1
+        b = O.layout_pack(one, np.zeros(128, dtype=np.float16), bits, kind)
+        words = b[:128 * 16 * bits].view("<u4").reshape(bits, 128, 4)
+        if kind == "k":
+            row, pair, half = tok, dim // 2, dim % 2
+        else:
+            row, pair, half = (tok & 64) | (dim & 63), 2 * ((tok & 63) // 2) + (dim >> 6), tok % 2
+        value = ((1 << bits) - 1) << (bits * half)
+        rowwords = words[:, row, :].reshape(-1)
+        expect = np.zeros(4 * bits, dtype=np.uint64)
+        grp, k = pair // 16, pair % 16
+        if bits == 4:
+            expect[4 * (k // 4) + grp] = value << (8 * (k % 4))
+        elif bits == 2:
+            expect[4 * (k // 8) + grp] = value << (4 * (k % 8))
+        elif k < 15:
+            expect[4 * (k // 5) + grp] = value << (6 * (k % 5))
+        else:
+            for part in range(3):
+                expect[4 * part + grp] = ((value >> (2 * part)) & 3) << 30
+        assert np.array_equal(rowwords.astype(np.uint64), expect)
+        assert np.count_nonzero(words) == np.count_nonzero(expect)
 
 
 def test_turbo_encode_consistency():

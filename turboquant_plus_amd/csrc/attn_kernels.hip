@@ -40,22 +40,8 @@ constexpr float RSQRT128 = 0.08838834764831845f;
 template <typename T> __device__ inline float ldf(const T *p) { return (float)*p; }
 template <> __device__ inline float ldf<__half>(const __half *p) { return __half2float(*p); }
 
-// runtime-p version of pair_lut_offset; p is a compile-time constant after unrolling
 template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t (&w)[4 * BITS], int p) {
-    if constexpr (BITS == 4) {
-        const int q = p >> 2, k = p & 3;
-        return k == 0 ? ((w[q] << 2) & 0x3FCu) : ((w[q] >> (8 * k - 2)) & 0x3FCu);
-    } else if constexpr (BITS == 2) {
-        const int q = p >> 3, k = p & 7;
-        return k == 0 ? ((w[q] << 2) & 0x3Cu) : ((w[q] >> (4 * k - 2)) & 0x3Cu);
-    } else {
-        const int g = p >> 4, kk = p & 15;
-        if (kk < 15) {
-            const int q = 3 * g + kk / 5, k = kk % 5;
-            return k == 0 ? ((w[q] << 2) & 0xFCu) : ((w[q] >> (6 * k - 2)) & 0xFCu);
-        }
-        return ((w[3 * g] >> 28) & 0xCu) | ((w[3 * g + 1] >> 26) & 0x30u) | ((w[3 * g + 2] >> 24) & 0xC0u);
-    }
+    return pair_lut_offset<BITS>(w, p);
 }
 
 template <int BITS> __device__ __forceinline__ void load_row(const uint8_t *block, int row, uint32_t (&w)[4 * BITS]) {

@@ -109,11 +109,13 @@ __device__ inline void wht128_wave(float &a, float &b, int lane) {
 
 // ---- packed rows ----------------------------------------------------------------
 // A row holds 64 pair codes (128 values) in 4*BITS dwords; pair = lo | hi << BITS.
-//   BITS 4: pair p = byte p%4 of dword p/4
-//   BITS 2: pair p = nibble p%8 of dword p/8
-//   BITS 3: four groups of 16 pairs in three dwords each: pair 16g + k, k < 15, at bit
-//           6*(k%5) of dword 3g + k/5; pair 16g + 15 = bits 30..31 of dwords 3g, 3g+1,
-//           3g+2 (low, middle, high two bits)
+// The row is four groups of 16 pairs; a group owns BITS dwords and dword j of group g
+// is row dword 4j + g, so 16-byte chunk j of the row holds dword j of the four groups.
+// Inside a group, pair k sits in
+//   BITS 4: byte k%4 of dword k/4
+//   BITS 2: nibble k%8 of dword k/8
+//   BITS 3: bits 6*(k%5).. of dword k/5 for k < 15; pair 15 = bits 30..31 of dwords
+//           0, 1, 2 (low, middle, high two bits)
 // A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
 // norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows are dim-major
 // inside each 64-token tile: row (token & 64) | (dim & 63) holds dims r and 64+r
@@ -122,36 +124,30 @@ __host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
 __host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
 __host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
 
-// byte offset (pair code * 4) into a 4-byte-entry LUT, P compile-time
-template <int BITS, int P> __device__ inline uint32_t pair_lut_offset(const uint32_t (&w)[4 * BITS]) {
-    if constexpr (BITS == 4) {
-        constexpr int q = P / 4, k = P % 4;
-        if constexpr (k == 0) return (w[q] << 2) & 0x3FCu;
-        else return (w[q] >> (8 * k - 2)) & 0x3FCu;
-    } else if constexpr (BITS == 2) {
-        constexpr int q = P / 8, k = P % 8;
-        if constexpr (k == 0) return (w[q] << 2) & 0x3Cu;
-        else return (w[q] >> (4 * k - 2)) & 0x3Cu;
-    } else {
-        static_assert(BITS == 3, "bits");
-        constexpr int g = P >> 4, kk = P & 15;
-        if constexpr (kk < 15) {
-            constexpr int q = 3 * g + kk / 5, k = kk % 5;
-            if constexpr (k == 0) return (w[q] << 2) & 0xFCu;
-            else return (w[q] >> (6 * k - 2)) & 0xFCu;
-        } else {
-            return ((w[3 * g] >> 28) & 0xCu) | ((w[3 * g + 1] >> 26) & 0x30u) | ((w[3 * g + 2] >> 24) & 0xC0u);
-        }
+// pairs per dword and bits per pair
+__host__ __device__ constexpr int pairs_per_dword(int bits) { return bits == 4 ? 4 : bits == 2 ? 8 : 5; }
+// row dword and bit position of pair p (for BITS 3 not the tail pair, p % 16 == 15)
+__host__ __device__ constexpr int pair_dword(int bits, int p) { return 4 * ((p & 15) / pairs_per_dword(bits)) + (p >> 4); }
+__host__ __device__ constexpr int pair_shift(int bits, int p) { return 2 * bits * ((p & 15) % pairs_per_dword(bits)); }
+
+// byte offset (pair code * 4) into a 4-byte-entry LUT; p must fold to a constant
+template <int BITS> __device__ __forceinline__ uint32_t pair_lut_offset(const uint32_t (&w)[4 * BITS], int p) {
+    constexpr uint32_t MASK = ((1u << (2 * BITS)) - 1u) << 2;
+    if (BITS == 3 && (p & 15) == 15) {
+        const int g = p >> 4;
+        return ((w[g] >> 28) & 0xCu) | ((w[4 + g] >> 26) & 0x30u) | ((w[8 + g] >> 24) & 0xC0u);
     }
+    const int q = pair_dword(BITS, p), sh = pair_shift(BITS, p);
+    return sh == 0 ? ((w[q] << 2) & MASK) : ((w[q] >> (sh - 2)) & MASK);
 }
 
 // runtime pair extraction (slow path: unpack / load kernels)
 __device__ inline uint32_t pair_code(const uint32_t *w, int bits, int p) {
-    if (bits == 4) return (w[p >> 2] >> (8 * (p & 3))) & 0xFFu;
-    if (bits == 2) return (w[p >> 3] >> (4 * (p & 7))) & 0xFu;
-    const int g = p >> 4, k = p & 15;
-    if (k < 15) return (w[3 * g + k / 5] >> (6 * (k % 5))) & 0x3Fu;
-    return (w[3 * g] >> 30) | ((w[3 * g + 1] >> 30) << 2) | ((w[3 * g + 2] >> 30) << 4);
+    if (bits == 3 && (p & 15) == 15) {
+        const int g = p >> 4;
+        return (w[g] >> 30) | ((w[4 + g] >> 30) << 2) | ((w[8 + g] >> 30) << 4);
+    }
+    return (w[pair_dword(bits, p)] >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
 }
 
 // (row, pair, half) of the code of (token, dim) inside its 128-token block

@@ -108,18 +108,13 @@ __device__ inline void pack_block(const uint8_t *codes, const float *norms, uint
     constexpr int NDW = TQ_ROWS_PER_BLOCK * 4 * BITS;
     for (int o = threadIdx.x; o < NDW; o += NTHREADS) {
         const int c = o >> 9, r = (o & 511) >> 2, k = o & 3;
-        const int q = 4 * c + k;
+        // chunk c, dword k of the row = dword j = c of group g = k
+        constexpr int PER = pairs_per_dword(BITS);
+        const int g = k, j = c;
         uint32_t word = 0;
-        if constexpr (BITS == 4) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) word |= pair_from_stage<4>(codes, kind, r, 4 * q + t) << (8 * t);
-        } else if constexpr (BITS == 2) {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) word |= pair_from_stage<2>(codes, kind, r, 8 * q + t) << (4 * t);
-        } else {
-            const int g = q / 3, j = q % 3;  // group of 16 pairs, dword inside the group
-#pragma unroll
-            for (int t = 0; t < 5; ++t) word |= pair_from_stage<3>(codes, kind, r, 16 * g + 5 * j + t) << (6 * t);
+        for (int t = 0; t < PER; ++t) word |= pair_from_stage<BITS>(codes, kind, r, 16 * g + PER * j + t) << (2 * BITS * t);
+        if constexpr (BITS == 3) {
             const uint32_t tail = pair_from_stage<3>(codes, kind, r, 16 * g + 15);
             word |= ((tail >> (2 * j)) & 3u) << 30;
         }
@@ -190,27 +185,16 @@ template <int BITS> __device__ __forceinline__ void pack_row_from_nibbles(const 
         if constexpr (BITS == 4) return byte;
         else return (byte & ((1u << BITS) - 1u)) | ((byte >> 4) << BITS);
     };
-    if constexpr (BITS == 4) {
+    constexpr int PER = pairs_per_dword(BITS);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) out[q] = nib[q];
-    } else if constexpr (BITS == 2) {
+    for (int g = 0; g < 4; ++g) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
+        for (int j = 0; j < BITS; ++j) {
             uint32_t w = 0;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) w |= pair(8 * q + t) << (4 * t);
-            out[q] = w;
-        }
-    } else {
-        uint32_t tail[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) tail[t] = pair(16 * t + 15);
-#pragma unroll
-        for (int q = 0; q < 12; ++q) {
-            uint32_t w = ((tail[q / 3] >> (2 * (q % 3))) & 3u) << 30;
-#pragma unroll
-            for (int t = 0; t < 5; ++t) w |= pair(16 * (q / 3) + 5 * (q % 3) + t) << (6 * t);
-            out[q] = w;
+            for (int t = 0; t < PER; ++t) w |= pair(16 * g + PER * j + t) << (2 * BITS * t);
+            if constexpr (BITS == 3) w |= ((pair(16 * g + 15) >> (2 * j)) & 3u) << 30;
+            out[4 * j + g] = w;
         }
     }
 }
@@ -544,13 +528,12 @@ __device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, 
     int row, p, half;
     locate(kind, token, dim, row, p, half);
     uint32_t pc;
-    if (bits == 4) pc = (row_dword(block, row, p >> 2) >> (8 * (p & 3))) & 0xFFu;
-    else if (bits == 2) pc = (row_dword(block, row, p >> 3) >> (4 * (p & 7))) & 0xFu;
-    else if ((p & 15) < 15) pc = (row_dword(block, row, 3 * (p >> 4) + (p & 15) / 5) >> (6 * ((p & 15) % 5))) & 0x3Fu;
-    else {
+    if (bits == 3 && (p & 15) == 15) {
         const int g = p >> 4;
-        pc = (row_dword(block, row, 3 * g) >> 30) | ((row_dword(block, row, 3 * g + 1) >> 30) << 2) |
-             ((row_dword(block, row, 3 * g + 2) >> 30) << 4);
+        pc = (row_dword(block, row, g) >> 30) | ((row_dword(block, row, 4 + g) >> 30) << 2) |
+             ((row_dword(block, row, 8 + g) >> 30) << 4);
+    } else {
+        pc = (row_dword(block, row, pair_dword(bits, p)) >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
     }
     return (pc >> (half * bits)) & ((1u << bits) - 1u);
 }
