@@ -176,16 +176,57 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         uint16_t *drf = nullptr;
         rc = rc ? rc : upload(&drf, rf);
         h->rfrag16 = drf;
+        // factored transform for K rows: fragment f0*4+ks, row 4c+i, column 8kb+e
+        {
+            std::vector<uint16_t> rk((size_t)8 * 64 * 8);
+            for (int f = 0; f < 8; ++f)
+                for (int l = 0; l < 64; ++l)
+                    for (int e = 0; e < 8; ++e) {
+                        const int r = l & 15, f0 = f >> 2, ks = f & 3;
+                        const int m = 32 * (r >> 2) + 4 * f0 + (r & 3), k = 32 * (l >> 4) + 8 * ks + e;
+                        const double v = s1[k] * ((__builtin_popcount(m & k) & 1) ? -1.0 : 1.0);
+                        rk[((size_t)f * 64 + l) * 8 + e] = v < 0 ? 0xBC00 : 0x3C00;
+                    }
+            uint16_t *drk = nullptr;
+            rc = rc ? rc : upload(&drk, rk);
+            h->rfrag16k = drk;
+            // sign-field positions of the values with s2 = +1 inside a lane quarter's unfolded dwords: the
+            // kernel appends the sign bit of s2 * y' (1 = negative) and xors with this to get "positive"
+            std::vector<uint32_t> fl(16, 0u);
+            for (int c = 0; c < 4; ++c)
+                for (int v = 0; v < 32; ++v) {
+                    if (s2[32 * c + v] < 0) continue;
+                    if (b == 4) fl[c * 4 + v / 8] |= 1u << (4 * (v % 8) + 3);
+                    else if (b == 2) fl[c * 4 + v / 16] |= 1u << (2 * (v % 16) + 1);
+                    else if (b == 3 && v < 30) fl[c * 4 + v / 10] |= 1u << (3 * (v % 10) + 2);
+                    else if (b == 3) fl[c * 4 + 3] |= 1u << (3 * (v - 30) + 2);
+                }
+            rc = rc ? rc : upload(&h->s2flip, fl);
+        }
         // sign-symmetric boundaries (in fp32) allow the thermometer quantiser
         const int nb = nc - 1, mid = nb / 2;
         h->symmetric = 1;
         for (int j = 1; j <= mid; ++j)
             if (b32[mid + j] != -b32[mid - j] || !(b32[mid + j] > 0.0f)) h->symmetric = 0;
         if (std::fabs(b32[mid]) > 1e-12f) h->symmetric = 0;
+        for (int m = 0; m <= mid; ++m)
+            if (std::fabs(cent[mid + 1 + m] + cent[mid - m]) > 1e-9 * std::fabs(cent[mid + 1 + m])) h->symmetric = 0;
         std::vector<float> st((size_t)mid + 1);
         st[0] = b32[mid];
         for (int j = 1; j <= mid; ++j) st[j] = b32[mid + j];
         rc = rc ? rc : upload(&h->symthr32, st);
+        // squared centroid of magnitude level m as a multilinear form in the bits of m
+        // (Moebius transform over subsets), for counting-based sums of c^2
+        {
+            const int nl = mid + 1;  // levels 0..mid, a power of two
+            std::vector<double> f((size_t)nl);
+            for (int m = 0; m < nl; ++m) f[m] = cent[mid + 1 + m] * cent[mid + 1 + m];
+            for (int bit = 1; bit < nl; bit <<= 1)
+                for (int m = 0; m < nl; ++m)
+                    if (m & bit) f[m] -= f[m ^ bit];
+            std::vector<float> cf(f.begin(), f.end());
+            rc = rc ? rc : upload(&h->sqcoef32, cf);
+        }
         if (cfg->projection) {
             // M = S R^T with R[k][m] = s2[k] H[k][m] s1[m] / sqrt(128); stored as [k*128+j] = M[j][k]
             std::vector<double> mt((size_t)128 * 128);
@@ -217,7 +258,7 @@ void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
                     h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
-                    h->rfrag16,     h->symthr32};
+                    h->rfrag16,     h->symthr32, h->rfrag16k,    h->sqcoef32, h->s2flip};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete h;

@@ -31,7 +31,11 @@ struct tq_handle {
     void *pair_lut;        // [4^bits] half2: (c[lo], c[hi]) for a pair code (bits <= 3), or [256] for 4
     float *projT32;        // [128*128] entry [k*128+j] = S[j][k]  (query projection, score tile)
     void *rfrag16;         // [32][64][8] fp16 +-1: D2 H D1 in 16x16x32 MFMA A-fragment order
+    void *rfrag16k;        // [8][64][8] fp16 +-1: fragment f0*4+ks, lane l, element e = s1[k] H[m][k] with
+                           // m = 32(l%16/4) + 4 f0 + l%4, k = 32(l/16) + 8 ks + e (factored transform, K rows)
+    uint32_t *s2flip;      // [4][4]: per lane quarter and output dword, sign-field positions of dims with s2 = +1
     float *symthr32;       // [2^(bits-1)]: middle boundary, then the positive boundaries
+    float *sqcoef32;       // [2^(bits-1)]: c[mid+1+m]^2 = sum over subsets S of the set bits of m of sqcoef32[S]
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };
 

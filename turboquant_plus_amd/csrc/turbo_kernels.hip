@@ -351,6 +351,373 @@ __global__ __launch_bounds__(256, 3) void k_store_mfma(const __half *x, uint8_t 
     }
 }
 
+// ---- K2, fp16 input, K rows: codes packed in registers ---------------------------------
+// Index bits of H128[m][k] = (-1)^popcount(m & k) pair up, so the transform splits as
+//   m = 32c + 8fh + 4f0 + i  (c = lane quarter, fh/f0 = fragment, i = row in the lane)
+//   k = 32kb + 8ks + e       (kb = operand lane quarter, ks = input slice, e = element)
+//   y'[m] = s2[m] * sum_ks (-1)^popcount(fh & ks) * Q[f0][ks][4c + i],
+//   Q[f0][ks] = A[f0][ks] (16 x 32) * X[ks] (32 x 16 tokens),
+//   A[f0][ks][4c + i][8kb + e] = s1[k] * H[32c + 4f0 + i][k]:
+// eight MFMAs with +-1 operands (exact products, fp32 accumulation) and a four-point
+// butterfly over ks per (f0, i) replace a dense 128 x 128 product.  Lane quarter c of token
+// lane%16 ends up with dims 32c .. 32c+31 of that token, which is pair group c of the
+// token's row: BITS dwords that no other lane touches.  Code bits come from compares whose
+// lane masks are shifted into the dword with one add-with-carry each (w = 2w + bit, most
+// significant bit first) in unfolded form [sign, level bits]; one xor per dword turns the
+// appended sign bits into "positive after s2", sum c^2 comes from population counts on the
+// unfolded dwords and the final codes from one in-word fold (level bits are complemented
+// where the value is not positive).
+// Code bits are appended by hand-scheduled groups: every compare result (a lane mask in an
+// SGPR pair) is consumed at least three instructions after the compare that wrote it, which
+// is what the hardware needs between a vector instruction writing a scalar register and a
+// vector instruction reading it; the carry-out of each add goes to vcc and is never read.
+// The scalar registers named in the text are listed as clobbers.
+
+// The sign bit of the value itself is appended with one funnel shift (so the sign field of
+// the unfolded code is 1 for negative values).  t[0] is not used: the middle boundary is 0.
+
+// 3-bit: values y0..y4 in append order; t[1..3] magnitude boundaries
+__device__ __forceinline__ uint32_t append5_b3(uint32_t w, float y0, float y1, float y2, float y3, float y4, const float (&t)[4]) {
+    float u0, u1, u2, u3, u4;
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[68:69], |%[y4]|, %[t2]\n\t"
+        "v_cndmask_b32_e64 %[u0], %[t1], %[t3], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[u1], %[t1], %[t3], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[u2], %[t1], %[t3], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[u3], %[t1], %[t3], s[66:67]\n\t"
+        "v_cndmask_b32_e64 %[u4], %[t1], %[t3], s[68:69]\n\t"
+        "v_cmp_gt_f32_e64 s[70:71], |%[y0]|, %[u0]\n\t"
+        "v_cmp_gt_f32_e64 s[72:73], |%[y1]|, %[u1]\n\t"
+        "v_cmp_gt_f32_e64 s[74:75], |%[y2]|, %[u2]\n\t"
+        "v_cmp_gt_f32_e64 s[76:77], |%[y3]|, %[u3]\n\t"
+        "v_cmp_gt_f32_e64 s[78:79], |%[y4]|, %[u4]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[70:71]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[72:73]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[74:75]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[76:77]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y4], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[68:69]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[78:79]\n\t"
+        : [w] "+v"(w), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3), [u4] "=&v"(u4)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [y4] "v"(y4), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "vcc");
+    return w;
+}
+
+__device__ __forceinline__ uint32_t append2_b3(uint32_t w, float y0, float y1, const float (&t)[4]) {
+    float u0, u1;
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
+        "v_cndmask_b32_e64 %[u0], %[t1], %[t3], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[u1], %[t1], %[t3], s[62:63]\n\t"
+        "v_cmp_gt_f32_e64 s[70:71], |%[y0]|, %[u0]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
+        "v_cmp_gt_f32_e64 s[72:73], |%[y1]|, %[u1]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[70:71]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[72:73]\n\t"
+        : [w] "+v"(w), [u0] "=&v"(u0), [u1] "=&v"(u1)
+        : [y0] "v"(y0), [y1] "v"(y1), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "vcc");
+    return w;
+}
+
+// 4-bit: binary search over t[1..7] (t[4] first), values y0..y3 in append order
+__device__ __forceinline__ uint32_t append4_b4(uint32_t w, float y0, float y1, float y2, float y3, const float (&t)[8]) {
+    float a0, a1, a2, a3, b0, b1, b2, b3;
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t4]\n\t"
+        "v_cndmask_b32_e64 %[a0], %[t2], %[t6], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[a1], %[t2], %[t6], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[a2], %[t2], %[t6], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[a3], %[t2], %[t6], s[66:67]\n\t"
+        "v_cmp_gt_f32_e64 s[68:69], |%[y0]|, %[a0]\n\t"
+        "v_cmp_gt_f32_e64 s[70:71], |%[y1]|, %[a1]\n\t"
+        "v_cmp_gt_f32_e64 s[72:73], |%[y2]|, %[a2]\n\t"
+        "v_cmp_gt_f32_e64 s[74:75], |%[y3]|, %[a3]\n\t"
+        "v_cndmask_b32_e64 %[b0], %[t1], %[t5], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[b1], %[t1], %[t5], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[b2], %[t1], %[t5], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[b3], %[t1], %[t5], s[66:67]\n\t"
+        "v_cndmask_b32_e64 %[a0], %[t3], %[t7], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[a1], %[t3], %[t7], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[a2], %[t3], %[t7], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[a3], %[t3], %[t7], s[66:67]\n\t"
+        "v_cndmask_b32_e64 %[b0], %[b0], %[a0], s[68:69]\n\t"
+        "v_cndmask_b32_e64 %[b1], %[b1], %[a1], s[70:71]\n\t"
+        "v_cndmask_b32_e64 %[b2], %[b2], %[a2], s[72:73]\n\t"
+        "v_cndmask_b32_e64 %[b3], %[b3], %[a3], s[74:75]\n\t"
+        "v_cmp_gt_f32_e64 s[76:77], |%[y0]|, %[b0]\n\t"
+        "v_cmp_gt_f32_e64 s[78:79], |%[y1]|, %[b1]\n\t"
+        "v_cmp_gt_f32_e64 s[80:81], |%[y2]|, %[b2]\n\t"
+        "v_cmp_gt_f32_e64 s[82:83], |%[y3]|, %[b3]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[68:69]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[76:77]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[70:71]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[78:79]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[72:73]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[80:81]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[74:75]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[82:83]\n\t"
+        : [w] "+v"(w), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3), [b0] "=&v"(b0), [b1] "=&v"(b1),
+          [b2] "=&v"(b2), [b3] "=&v"(b3)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1]), [t2] "v"(t[2]),
+          [t3] "v"(t[3]), [t4] "v"(t[4]), [t5] "v"(t[5]), [t6] "v"(t[6]), [t7] "v"(t[7])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "vcc");
+    return w;
+}
+
+__device__ __forceinline__ uint32_t append4_b2(uint32_t w, float y0, float y1, float y2, float y3, const float (&t)[2]) {
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t1]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[62:63]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[64:65]\n\t"
+        "v_alignbit_b32 %[w], %[w], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[66:67]\n\t"
+        : [w] "+v"(w)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "vcc");
+    return w;
+}
+
+// n[S] += number of fields of the unfolded dword whose level bits include the set S
+template <int BITS> __device__ __forceinline__ void count_levels(uint32_t w, uint32_t (&n)[1 << (BITS - 1)]) {
+    if constexpr (BITS == 2) {
+        n[1] += __builtin_popcount(w & 0x55555555u);
+    } else if constexpr (BITS == 3) {
+        constexpr uint32_t K0 = 0x09249249u;  // bit 0 of the ten 3-bit fields
+        const uint32_t b0 = w & K0, b1 = (w >> 1) & K0;
+        n[1] += __builtin_popcount(b0);
+        n[2] += __builtin_popcount(b1);
+        n[3] += __builtin_popcount(b0 & b1);
+    } else {
+        constexpr uint32_t K0 = 0x11111111u;
+        const uint32_t b0 = w & K0, b1 = (w >> 1) & K0, b2 = (w >> 2) & K0;
+        const uint32_t b01 = b0 & b1;
+        n[1] += __builtin_popcount(b0);
+        n[2] += __builtin_popcount(b1);
+        n[3] += __builtin_popcount(b01);
+        n[4] += __builtin_popcount(b2);
+        n[5] += __builtin_popcount(b0 & b2);
+        n[6] += __builtin_popcount(b1 & b2);
+        n[7] += __builtin_popcount(b01 & b2);
+    }
+}
+
+// unfolded [sign, level] fields -> codes: level bits complemented where the sign bit is 0
+template <int BITS> __device__ __forceinline__ uint32_t fold_codes(uint32_t w) {
+    if constexpr (BITS == 2) {
+        return w ^ ((~w & 0xAAAAAAAAu) >> 1);
+    } else if constexpr (BITS == 3) {
+        const uint32_t np = ~w & 0x24924924u;  // sign bits of the ten fields
+        return w ^ (np - (np >> 2));
+    } else {
+        const uint32_t np = ~w & 0x88888888u;
+        return w ^ (np - (np >> 3));
+    }
+}
+
+struct StoreKArgs {
+    const uint4 *afrag;      // [8 fragments f0*4+ks][64 lanes] 8 halves (+-1)
+    const uint32_t *s2flip;  // [4 lane quarters][4]: sign-field positions of the dims with s2 = +1, per output dword
+                             // (3-bit: entry 3 is for the tail pair word): appended sign bit ^ this = "positive"
+    const float *symthr;     // [0] middle boundary, [1..] positive boundaries
+    const float *sqcoef;     // multilinear coefficients of c^2 over the level bits
+    int norm_correction;
+    int64_t tokens;
+    uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
+};
+
+// RAGGED: sequences whose token count is not a multiple of the block size (rows past the
+// end are quantised as zeros, and the block index needs a division by blocks per sequence).
+template <int BITS, bool RAGGED>
+__global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
+    constexpr int NT = 1 << (BITS - 1);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n16 = lane & 15, kc = lane >> 4;
+    float thr0[NT], coef[NT];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) {
+        thr0[k] = a.symthr[k];
+        coef[k] = a.sqcoef[k];
+    }
+    half8_t af[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, a.afrag[f * 64 + lane]);
+    uint32_t flip[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) flip[j] = a.s2flip[kc * 4 + j];
+
+    const uint32_t gw = blockIdx.x * 4 + wave, gstride = gridDim.x * 4;
+    const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
+    // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
+    // The address is always valid: units past the end and rows past a sequence's last token
+    // are clamped, and `valid` says whether the data is to be used.
+    auto fetch = [&](uint32_t unit, uint4 (&xb)[4], bool &valid) {
+        unit = unit < last_unit ? unit : last_unit;
+        const uint4 *p;
+        if constexpr (RAGGED) {
+            const uint32_t blk = unit >> 3, seq = blk / bps, bis = blk - seq * bps;
+            int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + (unit & 7) * 16 + n16;
+            valid = tok < a.tokens;
+            tok = valid ? tok : a.tokens - 1;
+            p = reinterpret_cast<const uint4 *>(x + ((int64_t)seq * a.tokens + tok) * 128 + 32 * kc);
+        } else {
+            valid = true;
+            p = reinterpret_cast<const uint4 *>(x + ((int64_t)unit * 16 + n16) * 128 + 32 * kc);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) xb[ks] = p[ks];
+    };
+
+    // an exact zero counts as positive only if the middle boundary is below zero
+    const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
+    const int diag_sel = n16 & 3;
+    const bool diag_here = kc == (n16 >> 2);
+
+    constexpr int DEPTH = 2;  // units of input in flight per wavefront
+    uint4 xq[DEPTH][4];
+    bool xvalid[DEPTH];
+#pragma unroll
+    for (int r = 0; r < DEPTH; ++r) fetch(gw + r * gstride, xq[r], xvalid[r]);
+
+#pragma unroll 1
+    for (uint32_t base = gw; base < a.n_units; base += DEPTH * gstride) {
+#pragma unroll
+        for (int r = 0; r < DEPTH; ++r) {
+            const uint32_t unit = base + r * gstride;
+            if (unit >= a.n_units) continue;
+            uint4 (&xb)[4] = xq[r];
+            if constexpr (RAGGED) {
+                if (!xvalid[r]) {
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
+                }
+            }
+
+            float4_t q[2][4];
+#pragma unroll
+            for (int f0 = 0; f0 < 2; ++f0)
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+                    q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], __builtin_bit_cast(half8_t, xb[ks]),
+                                                                       float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            // ||x||^2 on the matrix cores as well: the diagonal of X X^T (the same registers serve as
+            // both operands); token n16's entry is element n16 % 4 of lane quarter n16 / 4
+            float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+                gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
+                                                              gram, 0, 0, 0);
+            float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
+            ss = diag_here ? ss : 0.0f;
+            fetch(unit + DEPTH * gstride, xb, xvalid[r]);
+            ss += xor_lane<16>(ss);
+            ss += xor_lane<32>(ss);
+            const float norm = __builtin_amdgcn_sqrtf(ss);  // 1 ulp: scales boundaries (1e-7 relative) and the stored fp16 norm
+            const float scale = norm > 0.0f ? norm * 11.313708498984761f : 1.0f;  // y' = sqrt(128) ||x|| y
+            float thr[NT];
+#pragma unroll
+            for (int k = 0; k < NT; ++k) thr[k] = thr0[k] * scale;
+
+            // butterfly over the input slices: fragment 2*fh + f0 holds dims 32kc + 8fh + 4f0 + i
+            float4_t y[8];
+#pragma unroll
+            for (int f0 = 0; f0 < 2; ++f0) {
+                const float4_t s01 = q[f0][0] + q[f0][1], d01 = q[f0][0] - q[f0][1];
+                const float4_t s23 = q[f0][2] + q[f0][3], d23 = q[f0][2] - q[f0][3];
+                y[0 + f0] = s01 + s23;
+                y[2 + f0] = d01 + d23;
+                y[4 + f0] = s01 - s23;
+                y[6 + f0] = d01 - d23;
+            }
+            // value v = 0..31 of this lane (dim 32*kc + v) up to the sign s2
+            auto val = [&](int v) -> float { return y[v >> 2][v & 3]; };
+            const bool nonzero = norm > 0.0f;  // all-zero rows get the code of an exact 0 everywhere
+            uint32_t g[BITS];
+            uint32_t n[NT];
+#pragma unroll
+            for (int k = 0; k < NT; ++k) n[k] = 0;
+            if constexpr (BITS == 3) {
+                uint32_t tw = append2_b3(0u, val(31), val(30), thr);  // pair 15 = values 30 (low code), 31 (high code)
+                count_levels<3>(tw, n);
+                tw = fold_codes<3>(nonzero ? tw ^ flip[3] : (zero_word & 0x24u));
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    const int v = 10 * j;
+                    uint32_t w = append5_b3(0u, val(v + 9), val(v + 8), val(v + 7), val(v + 6), val(v + 5), thr);
+                    w = append5_b3(w, val(v + 4), val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+                    count_levels<3>(w, n);
+                    g[j] = fold_codes<3>(nonzero ? w ^ flip[j] : (zero_word & 0x24924924u)) | (((tw >> (2 * j)) & 3u) << 30);
+                }
+            } else if constexpr (BITS == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int v = 8 * j;
+                    uint32_t w = append4_b4(0u, val(v + 7), val(v + 6), val(v + 5), val(v + 4), thr);
+                    w = append4_b4(w, val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+                    count_levels<4>(w, n);
+                    g[j] = fold_codes<4>(nonzero ? w ^ flip[j] : (zero_word & 0x88888888u));
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int v = 16 * j + 12; v >= 16 * j; v -= 4) w = append4_b2(w, val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+                    count_levels<2>(w, n);
+                    g[j] = fold_codes<2>(nonzero ? w ^ flip[j] : (zero_word & 0xAAAAAAAAu));
+                }
+            }
+            const uint32_t blk = unit >> 3;
+            const int row = (int)(unit & 7) * 16 + n16;
+            uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
+#pragma unroll
+            for (int j = 0; j < BITS; ++j) *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kc * 4) = g[j];
+
+            float gn = norm;
+            if (a.norm_correction) {
+                float cs = 32.0f * coef[0];
+#pragma unroll
+                for (int k = 1; k < NT; ++k) cs = fmaf(coef[k], (float)n[k], cs);
+                cs += xor_lane<16>(cs);
+                cs += xor_lane<32>(cs);
+                gn = norm * __builtin_amdgcn_rsqf(cs);  // cs >= 128 min c^2 > 0
+            }
+            if (kc == 0) reinterpret_cast<__half *>(block + block_code_bytes(BITS))[row] = __float2half_rn(gn);
+        }
+    }
+}
+
 // ---- K2: fused quantise + pack ---------------------------------------------------
 template <int BITS, typename TI>
 __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, StoreArgs a) {
@@ -718,6 +1085,26 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
         m.rfrag = (const uint4 *)h->rfrag16; m.symthr = h->symthr32; m.cent = h->centroids32;
         m.kind = kind; m.norm_correction = h->norm_correction;
         m.tokens = tokens; m.blocks_per_seq = bps; m.n_blocks = n_seqs * bps;
+        if (kind == TQ_KIND_K && h->rfrag16k && h->s2flip && h->sqcoef32 && m.n_blocks < (1ll << 28)) {
+            StoreKArgs ka;
+            ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
+            ka.norm_correction = h->norm_correction; ka.tokens = tokens;
+            ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(m.n_blocks * 8);
+            // one wavefront per 16-token unit, four resident workgroups per CU
+            const unsigned kgrid = (unsigned)((ka.n_units + 3) / 4 < 1024 ? (ka.n_units + 3) / 4 : 1024);
+            const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
+#define TQ_STORE_K(B)                                                                                   \
+    if (ragged) k_store_k<B, true><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);       \
+    else k_store_k<B, false><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka)
+            switch (h->bits) {
+            case 2: TQ_STORE_K(2); break;
+            case 3: TQ_STORE_K(3); break;
+            case 4: TQ_STORE_K(4); break;
+            default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+            }
+#undef TQ_STORE_K
+            return tq_check_launch("store_k");
+        }
         // one wavefront per 64-token tile; at most 3 resident workgroups per CU, each with its own R' copy
         const int64_t units = 2 * m.n_blocks;
         const unsigned mgrid = (unsigned)((units + 3) / 4 < 768 ? (units + 3) / 4 : 768);
