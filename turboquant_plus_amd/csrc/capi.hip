@@ -190,6 +190,16 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
             uint16_t *drk = nullptr;
             rc = rc ? rc : upload(&drk, rk);
             h->rfrag16k = drk;
+            for (int f = 0; f < 8; ++f)
+                for (int l = 0; l < 64; ++l)
+                    for (int e = 0; e < 8; ++e) {
+                        const int m = 16 * (f >> 2) + (l & 15), k = 32 * (f & 3) + 8 * (l >> 4) + e;
+                        const double v = s1[k] * ((__builtin_popcount(m & k) & 1) ? -1.0 : 1.0);
+                        rk[((size_t)f * 64 + l) * 8 + e] = v < 0 ? 0xBC00 : 0x3C00;
+                    }
+            uint16_t *drv = nullptr;
+            rc = rc ? rc : upload(&drv, rk);
+            h->rfrag16v = drv;
             // sign-field positions of the values with s2 = +1 inside a lane quarter's unfolded dwords: the
             // kernel appends the sign bit of s2 * y' (1 = negative) and xors with this to get "positive"
             std::vector<uint32_t> fl(16, 0u);
@@ -258,7 +268,7 @@ void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
                     h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
-                    h->rfrag16,     h->symthr32, h->rfrag16k,    h->sqcoef32, h->s2flip};
+                    h->rfrag16,     h->symthr32, h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete h;

@@ -15,6 +15,9 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 template <int CTRL> __device__ inline float dpp(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
+template <int CTRL> __device__ inline uint32_t dpp(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
 template <int CTRL> __device__ inline double dpp(double v) {
     const long long b = __builtin_bit_cast(long long, v);
     const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, 0xF, 0xF, true);

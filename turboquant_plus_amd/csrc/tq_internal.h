@@ -33,6 +33,8 @@ struct tq_handle {
     void *rfrag16;         // [32][64][8] fp16 +-1: D2 H D1 in 16x16x32 MFMA A-fragment order
     void *rfrag16k;        // [8][64][8] fp16 +-1: fragment f0*4+ks, lane l, element e = s1[k] H[m][k] with
                            // m = 32(l%16/4) + 4 f0 + l%4, k = 32(l/16) + 8 ks + e (factored transform, K rows)
+    void *rfrag16v;        // [8][64][8] fp16 +-1: fragment d0*4+ks, lane l, element e = s1[k] H[16 d0 + l%16][k],
+                           // k = 32 ks + 8(l/16) + e (factored transform, V rows: B operand)
     uint32_t *s2flip;      // [4][4]: per lane quarter and output dword, sign-field positions of dims with s2 = +1
     float *symthr32;       // [2^(bits-1)]: middle boundary, then the positive boundaries
     float *sqcoef32;       // [2^(bits-1)]: c[mid+1+m]^2 = sum over subsets S of the set bits of m of sqcoef32[S]

@@ -718,6 +718,360 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
     }
 }
 
+// ---- K2, fp16 input, V rows ---------------------------------------------------------------
+// V rows are dim-major, so here the tokens are the MFMA rows (A = X, B = the +-1 factor): lane
+// quarter q, column n = lane mod 16 holds, per 16-token sub-tile u of a 64-token tile, tokens
+// 16q + 4u + i (i = 0..3) of dim 16*dd + 64*hf + n for the four rows dd and both dim halves.
+// A group of appends takes one token (u, i) and one dim half and adds its code to the current
+// dword of each of the four rows; sub-tiles run u = 3..0 so that pairs arrive in descending
+// order.  Values are normalised by the token's norm first (thresholds are shared).
+//   m = 64hf + 32d1 + 16d0 + n,  k = 32ks + 8kb + e,  dd = 2 d1 + d0
+//   y'[m] = s2[m] * sum_ks (-1)^popcount((d1 + 2hf) & ks) * Q[d0][ks],  Q[d0][ks] = X[ks] B[d0][ks],
+//   B[d0][ks][8kb + e][n] = s1[k] * H[16 d0 + n][k]
+
+// one 3-bit code per row: w_d = 8 w_d + [sign, level]; level counts of the token: n1 += bit 0,
+// n2 += bit 1, n3 += both
+__device__ __forceinline__ void append_rows_b3(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, uint32_t &n1, uint32_t &n2,
+                                               uint32_t &n3, float y0, float y1, float y2, float y3, const float (&t)[4]) {
+    float u0, u1, u2, u3;
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t2]\n\t"
+        "v_cndmask_b32_e64 %[u0], %[t1], %[t3], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[u1], %[t1], %[t3], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[u2], %[t1], %[t3], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[u3], %[t1], %[t3], s[66:67]\n\t"
+        "v_cmp_gt_f32_e64 s[68:69], |%[y0]|, %[u0]\n\t"
+        "v_cmp_gt_f32_e64 s[70:71], |%[y1]|, %[u1]\n\t"
+        "v_cmp_gt_f32_e64 s[72:73], |%[y2]|, %[u2]\n\t"
+        "v_cmp_gt_f32_e64 s[74:75], |%[y3]|, %[u3]\n\t"
+        "v_alignbit_b32 %[w0], %[w0], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[68:69]\n\t"
+        "v_alignbit_b32 %[w1], %[w1], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[70:71]\n\t"
+        "s_and_b64 s[76:77], s[60:61], s[68:69]\n\t"
+        "s_and_b64 s[78:79], s[62:63], s[70:71]\n\t"
+        "s_and_b64 s[80:81], s[64:65], s[72:73]\n\t"
+        "s_and_b64 s[82:83], s[66:67], s[74:75]\n\t"
+        "v_alignbit_b32 %[w2], %[w2], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[72:73]\n\t"
+        "v_alignbit_b32 %[w3], %[w3], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[74:75]\n\t"
+        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[68:69]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[70:71]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[72:73]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[74:75]\n\t"
+        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[76:77]\n\t"
+        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[78:79]\n\t"
+        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[80:81]\n\t"
+        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[82:83]\n\t"
+        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3), [n1] "+v"(n1), [n2] "+v"(n2), [n3] "+v"(n3),
+          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "vcc");
+}
+
+__device__ __forceinline__ void append_rows_b2(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, uint32_t &n1, float y0,
+                                               float y1, float y2, float y3, const float (&t)[2]) {
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t1]\n\t"
+        "v_alignbit_b32 %[w0], %[w0], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[60:61]\n\t"
+        "v_alignbit_b32 %[w1], %[w1], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[62:63]\n\t"
+        "v_alignbit_b32 %[w2], %[w2], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[64:65]\n\t"
+        "v_alignbit_b32 %[w3], %[w3], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[66:67]\n\t"
+        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3), [n1] "+v"(n1)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "vcc");
+}
+
+__device__ __forceinline__ void append_rows_b4(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, float y0, float y1, float y2,
+                                               float y3, const float (&t)[8]) {
+    float a0, a1, a2, a3, b0, b1, b2, b3;
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t4]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t4]\n\t"
+        "v_cndmask_b32_e64 %[a0], %[t2], %[t6], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[a1], %[t2], %[t6], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[a2], %[t2], %[t6], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[a3], %[t2], %[t6], s[66:67]\n\t"
+        "v_cmp_gt_f32_e64 s[68:69], |%[y0]|, %[a0]\n\t"
+        "v_cmp_gt_f32_e64 s[70:71], |%[y1]|, %[a1]\n\t"
+        "v_cmp_gt_f32_e64 s[72:73], |%[y2]|, %[a2]\n\t"
+        "v_cmp_gt_f32_e64 s[74:75], |%[y3]|, %[a3]\n\t"
+        "v_cndmask_b32_e64 %[b0], %[t1], %[t5], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[b1], %[t1], %[t5], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[b2], %[t1], %[t5], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[b3], %[t1], %[t5], s[66:67]\n\t"
+        "v_cndmask_b32_e64 %[a0], %[t3], %[t7], s[60:61]\n\t"
+        "v_cndmask_b32_e64 %[a1], %[t3], %[t7], s[62:63]\n\t"
+        "v_cndmask_b32_e64 %[a2], %[t3], %[t7], s[64:65]\n\t"
+        "v_cndmask_b32_e64 %[a3], %[t3], %[t7], s[66:67]\n\t"
+        "v_cndmask_b32_e64 %[b0], %[b0], %[a0], s[68:69]\n\t"
+        "v_cndmask_b32_e64 %[b1], %[b1], %[a1], s[70:71]\n\t"
+        "v_cndmask_b32_e64 %[b2], %[b2], %[a2], s[72:73]\n\t"
+        "v_cndmask_b32_e64 %[b3], %[b3], %[a3], s[74:75]\n\t"
+        "v_cmp_gt_f32_e64 s[76:77], |%[y0]|, %[b0]\n\t"
+        "v_cmp_gt_f32_e64 s[78:79], |%[y1]|, %[b1]\n\t"
+        "v_cmp_gt_f32_e64 s[80:81], |%[y2]|, %[b2]\n\t"
+        "v_cmp_gt_f32_e64 s[82:83], |%[y3]|, %[b3]\n\t"
+        "v_alignbit_b32 %[w0], %[w0], %[y0], 31\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[68:69]\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[w0], s[76:77]\n\t"
+        "v_alignbit_b32 %[w1], %[w1], %[y1], 31\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[70:71]\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[78:79]\n\t"
+        "v_alignbit_b32 %[w2], %[w2], %[y2], 31\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[72:73]\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[80:81]\n\t"
+        "v_alignbit_b32 %[w3], %[w3], %[y3], 31\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[66:67]\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[74:75]\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[82:83]\n\t"
+        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3), [b0] "=&v"(b0), [b1] "=&v"(b1),
+          [b2] "=&v"(b2), [b3] "=&v"(b3)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3]), [t4] "v"(t[4]), [t5] "v"(t[5]), [t6] "v"(t[6]), [t7] "v"(t[7])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "vcc");
+}
+
+// pair k = 0..15 of a 16-pair group -> dword inside the group (3-bit: 3 = the word of the tail pair) and shift
+__host__ __device__ constexpr int grp_word(int bits, int k) { return bits == 3 && k == 15 ? 3 : k / pairs_per_dword(bits); }
+__host__ __device__ constexpr int grp_shift(int bits, int k) { return bits == 3 && k == 15 ? 0 : 2 * bits * (k % pairs_per_dword(bits)); }
+// V rows: sign-field bits of group dword j that belong to dim half hf (pairs with k % 2 == hf) and to the tokens
+// of the 16-token group named by tokmask (pair k = tokens 2(k/2), 2(k/2)+1 as low and high code)
+__host__ __device__ constexpr uint32_t v_sign_mask(int bits, int j, int hf, uint32_t tokmask) {
+    uint32_t m = 0;
+    for (int k = 0; k < 16; ++k) {
+        if ((k & 1) != hf || grp_word(bits, k) != j) continue;
+        for (int h = 0; h < 2; ++h)
+            if ((tokmask >> (2 * (k >> 1) + h)) & 1) m |= 1u << (grp_shift(bits, k) + bits * h + bits - 1);
+    }
+    return m;
+}
+
+struct StoreVArgs {
+    const uint4 *bfrag;   // [8 fragments d0*4+ks][64 lanes] 8 halves (+-1)
+    const float *s2;      // [128] output signs
+    const float *symthr;  // [0] middle boundary, [1..] positive boundaries
+    const float *sqcoef;  // multilinear coefficients of c^2 over the level bits
+    int norm_correction;
+    int64_t tokens;
+    uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
+};
+
+template <int BITS, bool RAGGED>
+__global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
+    constexpr int NT = 1 << (BITS - 1);
+    constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail pair word)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n16 = lane & 15, kq = lane >> 4;
+    float thr0[NT], coef[NT];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) {
+        thr0[k] = a.symthr[k];
+        coef[k] = a.sqcoef[k];
+    }
+    half8_t bf[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, a.bfrag[f * 64 + lane]);
+    bool s2pos[4][2];
+#pragma unroll
+    for (int dd = 0; dd < 4; ++dd)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = a.s2[64 * hf + 16 * dd + n16] > 0.0f;
+    // an exact zero counts as positive only if the middle boundary is below zero
+    const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
+
+    const uint32_t gw = blockIdx.x * 4 + wave, gstride = gridDim.x * 4;
+    const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
+    // A operand of sub-tile u: row r = lane%16 is token 16(r/4) + 4u + r%4 of the tile, this lane
+    // supplies inputs 32ks + 8kq .. +7.  The address is always valid (clamped); `valid` says
+    // whether the row exists.
+    auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
+        unit = unit < last_unit ? unit : last_unit;
+        const uint32_t blk = unit >> 1;
+        const int tb = (int)(unit & 1) * 64 + 16 * (n16 >> 2) + 4 * u + (n16 & 3);
+        const uint4 *p;
+        if constexpr (RAGGED) {
+            const uint32_t seq = blk / bps, bis = blk - seq * bps;
+            int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + tb;
+            valid = tok < a.tokens;
+            tok = valid ? tok : a.tokens - 1;
+            p = reinterpret_cast<const uint4 *>(x + ((int64_t)seq * a.tokens + tok) * 128 + 8 * kq);
+        } else {
+            valid = true;
+            p = reinterpret_cast<const uint4 *>(x + ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) xb[ks] = p[4 * ks];
+    };
+
+    uint4 xq[2][4];
+    bool xvalid[2];
+    fetch(gw, 3, xq[0], xvalid[0]);
+    fetch(gw, 2, xq[1], xvalid[1]);
+
+#pragma unroll 1
+    for (uint32_t unit = gw; unit < a.n_units; unit += gstride) {
+        uint8_t *block = packed + (int64_t)(unit >> 1) * block_bytes(BITS);
+        const int half = (int)(unit & 1);
+        __half *norms_out = reinterpret_cast<__half *>(block + block_code_bytes(BITS)) + half * 64 + 16 * kq;
+        uint32_t w[4][NW];
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd)
+#pragma unroll
+            for (int j = 0; j < NW; ++j) w[dd][j] = 0;
+        uint32_t zbits = 0;  // bit 4u+i: token 16kq + 4u + i is all zero
+
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int u = 3 - q;
+            uint4 (&xb)[4] = xq[q & 1];
+            if constexpr (RAGGED) {
+                if (!xvalid[q & 1]) {
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            float4_t qq[2][4];
+#pragma unroll
+            for (int d0 = 0; d0 < 2; ++d0)
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+                    qq[d0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), bf[d0 * 4 + ks],
+                                                                        float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            // ||x||^2: diagonal of X X^T; element i of this lane is row 4kq + i, column n16
+            float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+                gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
+                                                              gram, 0, 0, 0);
+            if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
+            else fetch(unit + gstride, 5 - q, xb, xvalid[q & 1]);
+
+            float nrm[4];
+            float4_t inv;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float ss = row16_sum(n16 == 4 * kq + i ? gram[i] : 0.0f);
+                nrm[i] = __builtin_amdgcn_sqrtf(ss);
+                const bool nz = ss > 0.0f;
+                inv[i] = nz ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;  // 1 / (||x|| sqrt(128))
+                zbits |= nz ? 0u : 1u << (4 * u + i);
+            }
+            // butterfly over the input slices, then normalise: y[fh][d0] is row dd = 2(fh % 2) + d0, dim half fh / 2
+            float4_t y[4][2];
+#pragma unroll
+            for (int d0 = 0; d0 < 2; ++d0) {
+                const float4_t s01 = qq[d0][0] + qq[d0][1], d01 = qq[d0][0] - qq[d0][1];
+                const float4_t s23 = qq[d0][2] + qq[d0][3], d23 = qq[d0][2] - qq[d0][3];
+                y[0][d0] = (s01 + s23) * inv;
+                y[1][d0] = (d01 + d23) * inv;
+                y[2][d0] = (s01 - s23) * inv;
+                y[3][d0] = (d01 - d23) * inv;
+            }
+            uint32_t n1[4] = {0, 0, 0, 0}, n2[4] = {0, 0, 0, 0}, n3[4] = {0, 0, 0, 0};
+            // groups in descending pair order: pair 4u + 2(i/2) + hf, high code (odd i) first
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const int i = (g & 4 ? 0 : 2) + (g & 1 ? 0 : 1), hf = g & 2 ? 0 : 1;
+                const int j = grp_word(BITS, 4 * u + 2 * (i >> 1) + hf);
+                const float y0 = y[0 | (hf << 1)][0][i], y1 = y[0 | (hf << 1)][1][i];
+                const float y2 = y[1 | (hf << 1)][0][i], y3 = y[1 | (hf << 1)][1][i];
+                if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], n2[i], n3[i], y0, y1, y2, y3, thr0);
+                else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr0);
+                else append_rows_b4(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
+            }
+            // level counts of the four tokens, one byte per token, summed over the 16 columns
+            uint32_t cnt[NT];
+            if constexpr (BITS == 4) {
+                // dword u of every row is complete: vertical sums of the level-bit products over the rows
+                constexpr uint32_t K0 = 0x11111111u;
+                uint32_t sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int dd = 0; dd < 4; ++dd) {
+                    const uint32_t ww = w[dd][u];
+                    const uint32_t b0 = ww & K0, b1 = (ww >> 1) & K0, b2 = (ww >> 2) & K0, b01 = b0 & b1;
+                    sum[1] += b0; sum[2] += b1; sum[3] += b01; sum[4] += b2;
+                    sum[5] += b0 & b2; sum[6] += b1 & b2; sum[7] += b01 & b2;
+                }
+#pragma unroll
+                for (int p = 1; p < 8; ++p) {
+                    // token i sits at nibbles 4(i/2) + i%2 (hf 0) and two nibbles higher (hf 1)
+                    const uint32_t t = sum[p] + (sum[p] >> 8);
+                    cnt[p] = (t & 0x000F000Fu) | ((t & 0x00F000F0u) << 4);
+                }
+            } else {
+                cnt[1] = n1[0] | (n1[1] << 8) | (n1[2] << 16) | (n1[3] << 24);
+                if constexpr (BITS == 3) {
+                    cnt[2] = n2[0] | (n2[1] << 8) | (n2[2] << 16) | (n2[3] << 24);
+                    cnt[3] = n3[0] | (n3[1] << 8) | (n3[2] << 16) | (n3[3] << 24);
+                }
+            }
+            float cs = 128.0f * coef[0];
+            const int sh = 8 * (n16 & 3);
+#pragma unroll
+            for (int p = 1; p < NT; ++p) cs = fmaf(coef[p], (float)((row16_sum(cnt[p]) >> sh) & 0xFFu), cs);
+            const int isel = n16 & 3;
+            const float nsel = isel == 0 ? nrm[0] : isel == 1 ? nrm[1] : isel == 2 ? nrm[2] : nrm[3];
+            const float gn = a.norm_correction ? nsel * __builtin_amdgcn_rsqf(cs) : nsel;
+            if (n16 < 4) norms_out[4 * u + n16] = __float2half_rn(gn);
+        }
+
+        // sign fields: appended bit = "negative before s2"; xor makes it "positive after s2".  All-zero tokens
+        // (rare: padding rows, empty vectors) get the sign field of an exact zero.
+        const bool anyzero = __builtin_amdgcn_ballot_w64(zbits != 0) != 0;
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+            uint32_t zm = 0;
+            if (anyzero) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    zm |= (zbits >> t) & 1 ? (v_sign_mask(BITS, j, 0, 1u << t) | v_sign_mask(BITS, j, 1, 1u << t)) : 0u;
+            }
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                const uint32_t fm = (s2pos[dd][0] ? v_sign_mask(BITS, j, 0, 0xFFFFu) : 0u) | (s2pos[dd][1] ? v_sign_mask(BITS, j, 1, 0xFFFFu) : 0u);
+                uint32_t ww = w[dd][j] ^ fm;
+                ww = (ww & ~zm) | (zero_word & zm);
+                w[dd][j] = fold_codes<BITS>(ww);
+            }
+        }
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) {
+            const int row = half * 64 + 16 * dd + n16;
+#pragma unroll
+            for (int j = 0; j < BITS; ++j) {
+                uint32_t g = w[dd][j];
+                if constexpr (BITS == 3) g |= ((w[dd][3] >> (2 * j)) & 3u) << 30;
+                *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kq * 4) = g;
+            }
+        }
+    }
+}
+
 // ---- K2: fused quantise + pack ---------------------------------------------------
 template <int BITS, typename TI>
 __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, StoreArgs a) {
@@ -1104,6 +1458,26 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
             }
 #undef TQ_STORE_K
             return tq_check_launch("store_k");
+        }
+        if (kind == TQ_KIND_V && h->rfrag16v && h->sqcoef32 && m.n_blocks < (1ll << 28)) {
+            StoreVArgs va;
+            va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
+            va.norm_correction = h->norm_correction; va.tokens = tokens;
+            va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(m.n_blocks * 2);
+            // one wavefront per 64-token tile, three resident workgroups per CU
+            const unsigned vgrid = (unsigned)((va.n_units + 3) / 4 < 768 ? (va.n_units + 3) / 4 : 768);
+            const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
+#define TQ_STORE_V(B)                                                                                   \
+    if (ragged) k_store_v<B, true><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);       \
+    else k_store_v<B, false><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va)
+            switch (h->bits) {
+            case 2: TQ_STORE_V(2); break;
+            case 3: TQ_STORE_V(3); break;
+            case 4: TQ_STORE_V(4); break;
+            default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+            }
+#undef TQ_STORE_V
+            return tq_check_launch("store_v");
         }
         // one wavefront per 64-token tile; at most 3 resident workgroups per CU, each with its own R' copy
         const int64_t units = 2 * m.n_blocks;
