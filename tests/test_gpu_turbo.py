@@ -101,19 +101,24 @@ def test_store_matches_oracle_bytes(bits, kind, dtype):
 
 
 @pytest.mark.parametrize("tokens", [1, 63, 128, 130, 257])
-def test_store_ragged_token_counts(tokens):
-    codec = tqa.TurboCodec(3, seed=5)
-    x = np.random.default_rng(tokens).standard_normal((3, tokens, D)).astype(np.float32)
+@pytest.mark.parametrize("bits,dtype", [(3, np.float32), (2, np.float16), (3, np.float16), (4, np.float16)])
+def test_store_ragged_token_counts(tokens, bits, dtype):
+    codec = tqa.TurboCodec(bits, seed=5)
+    x = np.random.default_rng(tokens).standard_normal((3, tokens, D)).astype(dtype)
     for kind in ("k", "v"):
         packed = codec.store(x, kind=kind)
         nb = -(-tokens // 128)
-        assert packed.numel() == 3 * nb * 6400
+        assert packed.numel() == 3 * nb * O.block_bytes(bits)
         idx, g = codec.unpack_codes(packed, 3, tokens, kind=kind)
         check_codes(codec, x.reshape(-1, D), np_(idx).reshape(-1, D), np_(g).reshape(-1))
         # padding rows of the last block hold the code of 0.0 and norm 0
-        full = np.zeros((3, nb * 128, D), dtype=np.float32)
+        full = np.zeros((3, nb * 128, D), dtype=dtype)
         full[:, :tokens] = x
         assert np.array_equal(np_(packed), np_(codec.store(full, kind=kind)))
+        i_full, g_full = O.layout_unpack(np_(packed), bits, kind)
+        i_full = i_full.reshape(3, nb * 128, D)
+        zero_code = int(np.sum(O.midpoints(codec.centroids) < 0.0))
+        assert np.all(i_full[:, tokens:] == zero_code) and np.all(g_full.reshape(3, -1)[:, tokens:] == 0)
 
 
 def test_store_empty():

@@ -163,19 +163,6 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         uint32_t *dl = nullptr;
         rc = rc ? rc : upload(&dl, lut);
         h->pair_lut = dl;
-        // D2 H D1 (+-1) as fp16 in MFMA A-fragment order: fragment f = t*4 + ks, lane l, element e
-        // = R'[16t + l%16][32ks + 8(l/16) + e]
-        std::vector<uint16_t> rf((size_t)32 * 64 * 8);
-        for (int f = 0; f < 32; ++f)
-            for (int l = 0; l < 64; ++l)
-                for (int e = 0; e < 8; ++e) {
-                    const int m = 16 * (f >> 2) + (l & 15), k = 32 * (f & 3) + 8 * (l >> 4) + e;
-                    const double v = s2[m] * s1[k] * ((__builtin_popcount(m & k) & 1) ? -1.0 : 1.0);
-                    rf[((size_t)f * 64 + l) * 8 + e] = v < 0 ? 0xBC00 : 0x3C00;
-                }
-        uint16_t *drf = nullptr;
-        rc = rc ? rc : upload(&drf, rf);
-        h->rfrag16 = drf;
         // factored transform for K rows: fragment f0*4+ks, row 4c+i, column 8kb+e
         {
             std::vector<uint16_t> rk((size_t)8 * 64 * 8);
@@ -268,7 +255,7 @@ void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
                     h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
-                    h->rfrag16,     h->symthr32, h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v};
+                    h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete h;

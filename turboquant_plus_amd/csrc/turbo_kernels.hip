@@ -136,220 +136,11 @@ struct StoreArgs {
 
 // ---- K2, fp16 input: rotation on the matrix cores ------------------------------------
 // R' = D2 H D1 has entries +-1, so with fp16 inputs every product of X R'^T is exact and
-// only the fp32 accumulation rounds (same error class as the butterfly).  One 16x16x32
-// MFMA tile computes y'[16 dims][16 tokens] = R'[16 dims][32 k] x^T[32 k][16 tokens]:
-// lane l then holds dims 16t + 4(l/16) + 0..3 of token l%16, i.e. 32 of the 128 rotated
-// coordinates of one token, and the four lanes l%16 + {0,16,32,48} cover the token.
-// R' is kept in LDS in MFMA fragment order (32 KB); the +-1 table is an input of the
-// handle.  Quantisation uses the sign symmetry of the codebook (checked when the handle
-// is built): index = mid+1+m for y above the middle boundary, mid-m below it, with
-// m = #{positive boundaries < |y|}; thresholds are scaled by ||x|| sqrt(128) instead of
-// normalising the 128 coordinates.
+// only the fp32 accumulation rounds (same error class as the butterfly).  Quantisation uses
+// the sign symmetry of the codebook (checked when the handle is built): index = mid+1+m for
+// a positive rotated value, mid-m otherwise, with m = #{positive boundaries < |y|}.
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-struct StoreMfmaArgs {
-    const uint4 *rfrag;   // [32 fragments][64 lanes] 8 halves: R'[16t + l%16][32ks + 8(l/16) + e], fragment t*4+ks
-    const float *symthr;  // [0] middle boundary, [1..M] positive boundaries, M = 2^(bits-1) - 1
-    const float *cent;
-    int kind, norm_correction;
-    int64_t tokens, blocks_per_seq, n_blocks;
-};
-
-template <int BITS> __device__ __forceinline__ uint32_t quantize_sym(float y, const float (&thr)[1 << (BITS - 1)]) {
-    constexpr int M = (1 << (BITS - 1)) - 1;
-    const bool pos = y > thr[0];
-    const float a = fabsf(y);
-    if constexpr (BITS == 2) {
-        const bool g1 = a > thr[1];
-        return (pos ? 2u : 0u) | ((g1 == pos) ? 1u : 0u);
-    } else if constexpr (BITS == 3) {
-        const bool g1 = a > thr[1], g2 = a > thr[2], g3 = a > thr[3];
-        const bool m1 = g2, m0 = (g1 != g2) != g3;
-        return (pos ? 4u : 0u) | ((m1 == pos) ? 2u : 0u) | ((m0 == pos) ? 1u : 0u);
-    } else {
-        static_assert(BITS == 4 && M == 7, "bits");
-        const bool g1 = a > thr[1], g2 = a > thr[2], g3 = a > thr[3], g4 = a > thr[4];
-        const bool g5 = a > thr[5], g6 = a > thr[6], g7 = a > thr[7];
-        const bool m2 = g4, m1 = (g2 != g4) != g6;
-        const bool m0 = (((g1 != g2) != (g3 != g4)) != (g5 != g6)) != g7;
-        return (pos ? 8u : 0u) | ((m2 == pos) ? 4u : 0u) | ((m1 == pos) ? 2u : 0u) | ((m0 == pos) ? 1u : 0u);
-    }
-}
-
-// nibble codes of one staged row (16 dwords, 8 codes each) -> the row's 4*BITS packed dwords
-template <int BITS> __device__ __forceinline__ void pack_row_from_nibbles(const uint32_t (&nib)[16], uint32_t (&out)[4 * BITS]) {
-    // pair p = codes (2p, 2p+1) = nibbles (2p, 2p+1) = byte p of the staged row
-    auto pair = [&](int p) -> uint32_t {
-        const uint32_t byte = (nib[p >> 2] >> (8 * (p & 3))) & 0xFFu;
-        if constexpr (BITS == 4) return byte;
-        else return (byte & ((1u << BITS) - 1u)) | ((byte >> 4) << BITS);
-    };
-    constexpr int PER = pairs_per_dword(BITS);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-#pragma unroll
-        for (int j = 0; j < BITS; ++j) {
-            uint32_t w = 0;
-#pragma unroll
-            for (int t = 0; t < PER; ++t) w |= pair(16 * g + PER * j + t) << (2 * BITS * t);
-            if constexpr (BITS == 3) w |= ((pair(16 * g + 15) >> (2 * j)) & 3u) << 30;
-            out[4 * j + g] = w;
-        }
-    }
-}
-
-constexpr int STAGE_STRIDE = 80;  // bytes per staged token row: 64 B of nibble codes, padded to a 16-byte multiple
-
-// One wavefront owns one 64-token tile (half a block) from load to store; nothing is shared
-// between wavefronts except the read-only R' fragments, so the kernel has no barrier after the
-// prologue.  Per 16-token sub-tile: 32 MFMAs, ||x||^2 by fp16 dot products, scaled thresholds,
-// 32 codes per lane written as nibbles into the wavefront's LDS stage; the next sub-tile's
-// input is fetched into the operand registers as soon as the MFMAs have consumed them.  Then
-// every lane packs one row of the tile (K: its token; V: dims l and 64+l across the 64 tokens)
-// and the tile leaves as BITS coalesced 1 KB stores plus 128 B of norms.
-template <int BITS, int KIND>
-__global__ __launch_bounds__(256, 3) void k_store_mfma(const __half *x, uint8_t *packed, StoreMfmaArgs a) {
-    constexpr int NT = 1 << (BITS - 1);  // thresholds: middle + M positive
-    __shared__ uint4 rfrag_s[32 * 64];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_s[4][64 * STAGE_STRIDE];
-    __shared__ float csq_s[1 << BITS];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n16 = lane & 15, kc = lane >> 4;
-    for (int i = tid; i < 32 * 64; i += 256) rfrag_s[i] = a.rfrag[i];
-    if (tid < (1 << BITS)) {
-        const float c = a.cent[tid];
-        csq_s[tid] = c * c;
-    }
-    float thr0[NT];
-#pragma unroll
-    for (int k = 0; k < NT; ++k) thr0[k] = a.symthr[k];
-    __syncthreads();
-
-    uint8_t *st = stage_s[wave];
-    const int64_t n_units = a.n_blocks * 2;
-    const int64_t gw = (int64_t)blockIdx.x * 4 + wave, gstride = (int64_t)gridDim.x * 4;
-
-    // 32-bit index arithmetic (the launcher checks that the block count fits)
-    const uint32_t bps = (uint32_t)a.blocks_per_seq;
-    auto row_ptr = [&](int64_t unit, int tt) -> const uint4 * {
-        const uint32_t blk = (uint32_t)(unit >> 1);
-        const uint32_t seq = blk / bps, bis = blk - seq * bps;
-        const int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + (unit & 1) * 64 + tt * 16 + n16;
-        return tok < a.tokens ? reinterpret_cast<const uint4 *>(x + ((int64_t)seq * a.tokens + tok) * 128 + 8 * kc) : nullptr;
-    };
-    auto fetch = [&](const uint4 *p, uint4 (&xb)[4]) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = p ? p[4 * ks] : make_uint4(0, 0, 0, 0);
-    };
-
-    uint4 xb[4];
-    if (gw < n_units) fetch(row_ptr(gw, 0), xb);
-
-#pragma unroll 1
-    for (int64_t unit = gw; unit < n_units; unit += gstride) {
-        const int64_t blk = unit >> 1;
-        const int half = (int)(unit & 1);
-        uint8_t *block = packed + blk * block_bytes(BITS);
-        __half *norms_out = reinterpret_cast<__half *>(block + block_code_bytes(BITS)) + half * 64;
-
-#pragma unroll 1
-        for (int tt = 0; tt < 4; ++tt) {
-            asm volatile("" ::: "memory");  // keep the R' fragments in LDS: re-read per sub-tile, do not hoist 128 registers
-            float4_t acc[8];
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                acc[d] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
-                    acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        __builtin_bit_cast(half8_t, rfrag_s[(d * 4 + ks) * 64 + lane]),
-                        __builtin_bit_cast(half8_t, xb[ks]), acc[d], 0, 0, 0);
-            }
-            // ||x||^2 from the same registers: this lane holds 32 of the token's 128 inputs
-            float ss = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const uint32_t w[4] = {xb[ks].x, xb[ks].y, xb[ks].z, xb[ks].w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const half2_t h = __builtin_bit_cast(half2_t, w[e]);
-                    ss = __builtin_amdgcn_fdot2(h, h, ss, false);
-                }
-            }
-            {   // operand registers are free: fetch the next sub-tile (or the next unit's first)
-                const bool last = tt == 3;
-                const int64_t nu = last ? unit + gstride : unit;
-                fetch(nu < n_units ? row_ptr(nu, last ? 0 : tt + 1) : nullptr, xb);
-            }
-            ss += xor_lane<16>(ss);
-            ss += xor_lane<32>(ss);
-            const float norm = sqrtf(ss);
-            const float scale = norm > 0.0f ? norm * 11.313708498984761f : 1.0f;  // y' = sqrt(128) ||x|| y
-            float thr[NT];
-#pragma unroll
-            for (int k = 0; k < NT; ++k) thr[k] = thr0[k] * scale;
-            float cs = 0.0f;
-            const int t = tt * 16 + n16;
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                uint32_t w = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t c = quantize_sym<BITS>(acc[d][i], thr);
-                    cs += csq_s[c];
-                    w |= c << (4 * i);
-                }
-                *reinterpret_cast<uint16_t *>(st + t * STAGE_STRIDE + 8 * d + 2 * kc) = (uint16_t)w;
-            }
-            cs += xor_lane<16>(cs);
-            cs += xor_lane<32>(cs);
-            float g = norm;
-            if (a.norm_correction) {
-                const float cn = sqrtf(cs);
-                g = norm / (cn > 1e-10f ? cn : 1.0f);
-            }
-            if (kc == 0) norms_out[t] = __float2half_rn(g);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        uint32_t out[4 * BITS];
-        if constexpr (KIND == TQ_KIND_K) {
-            uint32_t nib[16];
-            const uint4 *rp = reinterpret_cast<const uint4 *>(st + lane * STAGE_STRIDE);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint4 u = rp[q];
-                nib[4 * q] = u.x; nib[4 * q + 1] = u.y; nib[4 * q + 2] = u.z; nib[4 * q + 3] = u.w;
-            }
-            pack_row_from_nibbles<BITS>(nib, out);
-        } else {
-            // row l = dims l and 64+l; the row's pair 2*tp + hf = tokens (2tp, 2tp+1) of dim half hf
-            uint32_t nib[16];
-#pragma unroll
-            for (int q = 0; q < 16; ++q) nib[q] = 0;
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
-                const int col = (64 * hf + lane) >> 1, sh = 4 * (lane & 1);
-#pragma unroll
-                for (int tok = 0; tok < 64; ++tok) {
-                    const uint32_t c = (st[tok * STAGE_STRIDE + col] >> sh) & 0xFu;
-                    const int pos = 4 * (tok >> 1) + 2 * hf + (tok & 1);  // nibble of pair 2*tp + hf, half tok&1
-                    nib[pos >> 3] |= c << (4 * (pos & 7));
-                }
-            }
-            pack_row_from_nibbles<BITS>(nib, out);
-        }
-#pragma unroll
-        for (int c = 0; c < BITS; ++c)
-            *reinterpret_cast<uint4 *>(block + c * 2048 + (half * 64 + lane) * 16) =
-                make_uint4(out[4 * c], out[4 * c + 1], out[4 * c + 2], out[4 * c + 3]);
-        __builtin_amdgcn_wave_barrier();  // the stage is rewritten by the next unit
-    }
-}
 
 // ---- K2, fp16 input, K rows: codes packed in registers ---------------------------------
 // Index bits of H128[m][k] = (-1)^popcount(m & k) pair up, so the transform splits as
@@ -1434,16 +1225,13 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
         const char *e = getenv("TQ_STORE_PATH");
         return e && strcmp(e, "butterfly") == 0;
     }();
-    if (in_dtype == TQ_F16 && h->symmetric && h->rfrag16 && !force_butterfly) {
-        StoreMfmaArgs m;
-        m.rfrag = (const uint4 *)h->rfrag16; m.symthr = h->symthr32; m.cent = h->centroids32;
-        m.kind = kind; m.norm_correction = h->norm_correction;
-        m.tokens = tokens; m.blocks_per_seq = bps; m.n_blocks = n_seqs * bps;
-        if (kind == TQ_KIND_K && h->rfrag16k && h->s2flip && h->sqcoef32 && m.n_blocks < (1ll << 28)) {
+    if (in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && n_seqs * bps < (1ll << 28) && !force_butterfly) {
+        const int64_t n_blocks = n_seqs * bps;
+        if (kind == TQ_KIND_K) {
             StoreKArgs ka;
             ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
             ka.norm_correction = h->norm_correction; ka.tokens = tokens;
-            ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(m.n_blocks * 8);
+            ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
             // one wavefront per 16-token unit, four resident workgroups per CU
             const unsigned kgrid = (unsigned)((ka.n_units + 3) / 4 < 1024 ? (ka.n_units + 3) / 4 : 1024);
             const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
@@ -1459,11 +1247,11 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 #undef TQ_STORE_K
             return tq_check_launch("store_k");
         }
-        if (kind == TQ_KIND_V && h->rfrag16v && h->sqcoef32 && m.n_blocks < (1ll << 28)) {
+        {
             StoreVArgs va;
             va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
             va.norm_correction = h->norm_correction; va.tokens = tokens;
-            va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(m.n_blocks * 2);
+            va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
             // one wavefront per 64-token tile, three resident workgroups per CU
             const unsigned vgrid = (unsigned)((va.n_units + 3) / 4 < 768 ? (va.n_units + 3) / 4 : 768);
             const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
@@ -1479,20 +1267,6 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 #undef TQ_STORE_V
             return tq_check_launch("store_v");
         }
-        // one wavefront per 64-token tile; at most 3 resident workgroups per CU, each with its own R' copy
-        const int64_t units = 2 * m.n_blocks;
-        const unsigned mgrid = (unsigned)((units + 3) / 4 < 768 ? (units + 3) / 4 : 768);
-#define TQ_STORE_MFMA(B)                                                                                   \
-    if (kind == TQ_KIND_K) k_store_mfma<B, TQ_KIND_K><<<mgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, m); \
-    else k_store_mfma<B, TQ_KIND_V><<<mgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, m)
-        switch (h->bits) {
-        case 2: TQ_STORE_MFMA(2); break;
-        case 3: TQ_STORE_MFMA(3); break;
-        case 4: TQ_STORE_MFMA(4); break;
-        default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
-        }
-#undef TQ_STORE_MFMA
-        return tq_check_launch("store_mfma");
     }
     StoreArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
