@@ -131,7 +131,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                      "traffic": TRAFFIC_BYTES["decode3"], "algorithmic_bytes_per_step": algo,
-                     "kernel": "k_decode_attn<turbo3,turbo3> (+ k_prep_q, k_attn_combine in the step time)"},
+                     "kernel": "k_decode_attn<turbo3,turbo3> (+ k_attn_combine in the step time)"},
         "buffer_sets": n_sets,
     }
 
@@ -288,7 +288,7 @@ def main():
         "config": {"workload": s4["workload"], "global_batch": 2 * 8 * 32768, "io": "fp16 in, 4-bit codes + fp16 norm out",
                    "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": s4["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s4["frac"],
-                     "traffic": TRAFFIC_BYTES["store4"], "kernel": "k_store_mfma<4> (K and V instances)",
+                     "traffic": TRAFFIC_BYTES["store4"], "kernel": "k_store_k<4> and k_store_v<4> (one launch each per step)",
                      "kernel_us": s4["kernel_us"],
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
