@@ -120,6 +120,14 @@ int64_t tq_packed_bytes(int32_t bits, int64_t n_seqs, int64_t tokens);
 int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind,
              void *packed, void *stream);
 
+/* K and V of one layer in one launch: the two tensors that KVCacheCompressor.compress
+ * (kv_cache.py:98-141) takes together.  Same results as tq_store(hk, k, .., TQ_KIND_K, ..)
+ * followed by tq_store(hv, v, .., TQ_KIND_V, ..); k and v are [n_seqs, tokens, 128] of the
+ * same dtype.  With fp16 input the two run as one kernel whose wavefronts are given equal
+ * shares of the combined work, so launch and pipeline-fill time is paid once. */
+int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
+                int64_t tokens, int in_dtype, void *packed_k, void *packed_v, void *stream);
+
 /* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
  * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
  * original domain (transpose rotation applied). */

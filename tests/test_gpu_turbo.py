@@ -121,6 +121,30 @@ def test_store_ragged_token_counts(tokens, bits, dtype):
         assert np.all(i_full[:, tokens:] == zero_code) and np.all(g_full.reshape(3, -1)[:, tokens:] == 0)
 
 
+@pytest.mark.parametrize("kbits,vbits", [(3, 3), (4, 4), (2, 2), (4, 2), (3, 4)])
+@pytest.mark.parametrize("shape,dtype", [((2, 1024, D), np.float16), ((3, 200, D), np.float16), ((5, 40, D), np.float16),
+                                         ((2, 130, D), np.float32)])
+def test_store_kv_equals_separate_stores(kbits, vbits, shape, dtype):
+    """One launch for K and V writes the same bytes as the two single-tensor stores
+    (reference: KVCacheCompressor.compress takes K and V together, kv_cache.py:98-141)."""
+    kc, vc = tqa.TurboCodec(kbits, seed=42), tqa.TurboCodec(vbits, seed=542)
+    rng = np.random.default_rng(kbits * 10 + vbits)
+    k = rng.standard_normal(shape).astype(dtype)
+    v = rng.standard_normal(shape).astype(dtype)
+    k[0, 3] = 0
+    pk, pv = kc.store_kv(vc, k, v)
+    assert np.array_equal(np_(pk), np_(kc.store(k, kind="k")))
+    assert np.array_equal(np_(pv), np_(vc.store(v, kind="v")))
+
+
+def test_store_kv_rejects_mismatched_shapes():
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    with pytest.raises(ValueError):
+        kc.store_kv(vc, np.zeros((2, 128, D), dtype=np.float16), np.zeros((2, 256, D), dtype=np.float16))
+    pk, pv = kc.store_kv(vc, np.zeros((2, 0, D), dtype=np.float16), np.zeros((2, 0, D), dtype=np.float16))
+    assert pk.numel() == 0 and pv.numel() == 0
+
+
 def test_store_empty():
     codec = tqa.TurboCodec(3)
     assert codec.store(np.zeros((2, 0, D), dtype=np.float16)).numel() == 0

@@ -54,6 +54,7 @@ PROTOTYPES = {
     "tq_pack_indices": (_I, [_P, _L, C.c_int32, _P, _P]),
     "tq_packed_bytes": (_L, [C.c_int32, _L, _L]),
     "tq_store": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
+    "tq_store_kv": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_load": (_I, [_P, _P, _L, _L, _I, _P, _I, _I, _P]),
     "tq_unpack_codes": (_I, [_P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_store_qjl": (_I, [_P, _P, _L, _L, _I, _P, _P, _P, _P]),

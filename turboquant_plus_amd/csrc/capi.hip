@@ -377,6 +377,19 @@ int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, 
     return tqk_store(h, x, n_seqs, tokens, in_dtype, kind, packed, nullptr, nullptr, (hipStream_t)stream);
 }
 
+int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
+                int in_dtype, void *packed_k, void *packed_v, void *stream) {
+    int rc = check_fast(hk, "tq_store_kv");
+    rc = rc ? rc : check_fast(hv, "tq_store_kv");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_store_kv: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(k && v && packed_k && packed_v, TQ_ERR_ARG, "tq_store_kv: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
+            "tq_store_kv: inputs and outputs must be 16-byte aligned");
+    return tqk_store_kv(hk, hv, k, v, n_seqs, tokens, in_dtype, packed_k, packed_v, (hipStream_t)stream);
+}
+
 int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed,
                  uint8_t *sign_bits, void *rnorms_f16, void *stream) {
     int rc = check_fast(h, "tq_store_qjl");

@@ -350,10 +350,22 @@ struct StoreKArgs {
 
 // RAGGED: sequences whose token count is not a multiple of the block size (rows past the
 // end are quantised as zeros, and the block index needs a division by blocks per sequence).
+// Units lo, lo + step, .. below end are handed out through a ticket counter in LDS (zero on
+// entry).  A counter shared by the wavefronts of a workgroup makes them a work queue (the
+// hardware favours the oldest wavefronts of a SIMD, and with a fixed share per wavefront the
+// youngest are left to finish alone at a fraction of the SIMD's issue rate); a counter per
+// wavefront gives a fixed strided share.
+__device__ __forceinline__ uint32_t take_ticket(uint32_t *counter, int lane) {
+    uint32_t t = 0;
+    if (lane == 0) t = atomicAdd(counter, 1u);
+    return __builtin_amdgcn_readfirstlane(t);
+}
+
 template <int BITS, bool RAGGED>
-__global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
+__device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
+                                              uint32_t end, uint32_t *counter) {
     constexpr int NT = 1 << (BITS - 1);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kc = lane >> 4;
     float thr0[NT], coef[NT];
 #pragma unroll
@@ -368,7 +380,6 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
 #pragma unroll
     for (int j = 0; j < 4; ++j) flip[j] = a.s2flip[kc * 4 + j];
 
-    const uint32_t gw = blockIdx.x * 4 + wave, gstride = gridDim.x * 4;
     const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
     // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
     // The address is always valid: units past the end and rows past a sequence's last token
@@ -398,15 +409,23 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
     constexpr int DEPTH = 2;  // units of input in flight per wavefront
     uint4 xq[DEPTH][4];
     bool xvalid[DEPTH];
+    uint32_t cur[DEPTH];
 #pragma unroll
-    for (int r = 0; r < DEPTH; ++r) fetch(gw + r * gstride, xq[r], xvalid[r]);
+    for (int r = 0; r < DEPTH; ++r) {
+        cur[r] = lo + step * take_ticket(counter, lane);
+        fetch(cur[r], xq[r], xvalid[r]);
+    }
 
 #pragma unroll 1
-    for (uint32_t base = gw; base < a.n_units; base += DEPTH * gstride) {
+    for (bool more = true; more;) {
 #pragma unroll
         for (int r = 0; r < DEPTH; ++r) {
-            const uint32_t unit = base + r * gstride;
-            if (unit >= a.n_units) continue;
+            const uint32_t unit = cur[r];
+            if (unit >= end) {  // tickets only grow: nothing is left for this wavefront
+                more = false;
+                break;
+            }
+            const uint32_t next = lo + step * take_ticket(counter, lane);
             uint4 (&xb)[4] = xq[r];
             if constexpr (RAGGED) {
                 if (!xvalid[r]) {
@@ -431,7 +450,8 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
                                                               gram, 0, 0, 0);
             float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
             ss = diag_here ? ss : 0.0f;
-            fetch(unit + DEPTH * gstride, xb, xvalid[r]);
+            cur[r] = next;
+            fetch(next, xb, xvalid[r]);
             ss += xor_lane<16>(ss);
             ss += xor_lane<32>(ss);
             const float norm = __builtin_amdgcn_sqrtf(ss);  // 1 ulp: scales boundaries (1e-7 relative) and the stored fp16 norm
@@ -672,11 +692,13 @@ struct StoreVArgs {
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
 };
 
+// Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.
 template <int BITS, bool RAGGED>
-__global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
+__device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
+                                              uint32_t end, uint32_t *counter) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail pair word)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kq = lane >> 4;
     float thr0[NT], coef[NT];
 #pragma unroll
@@ -695,7 +717,6 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
     // an exact zero counts as positive only if the middle boundary is below zero
     const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
 
-    const uint32_t gw = blockIdx.x * 4 + wave, gstride = gridDim.x * 4;
     const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
     // A operand of sub-tile u: row r = lane%16 is token 16(r/4) + 4u + r%4 of the tile, this lane
     // supplies inputs 32ks + 8kq .. +7.  The address is always valid (clamped); `valid` says
@@ -721,11 +742,13 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
 
     uint4 xq[2][4];
     bool xvalid[2];
-    fetch(gw, 3, xq[0], xvalid[0]);
-    fetch(gw, 2, xq[1], xvalid[1]);
+    uint32_t unit = lo + step * take_ticket(counter, lane);
+    fetch(unit, 3, xq[0], xvalid[0]);
+    fetch(unit, 2, xq[1], xvalid[1]);
 
 #pragma unroll 1
-    for (uint32_t unit = gw; unit < a.n_units; unit += gstride) {
+    for (; unit < end;) {
+        const uint32_t next = lo + step * take_ticket(counter, lane);
         uint8_t *block = packed + (int64_t)(unit >> 1) * block_bytes(BITS);
         const int half = (int)(unit & 1);
         __half *norms_out = reinterpret_cast<__half *>(block + block_code_bytes(BITS)) + half * 64 + 16 * kq;
@@ -760,7 +783,7 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
                 gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
                                                               gram, 0, 0, 0);
             if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-            else fetch(unit + gstride, 5 - q, xb, xvalid[q & 1]);
+            else fetch(next, 5 - q, xb, xvalid[q & 1]);
 
             float nrm[4];
             float4_t inv;
@@ -860,7 +883,45 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
                 *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kq * 4) = g;
             }
         }
+        unit = next;
     }
+}
+
+__device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g) { return (uint32_t)((uint64_t)n * b / g); }
+
+// single tensor: fixed strided share per wavefront (four workgroups of four wavefronts per CU for K, three for V)
+template <int BITS, bool RAGGED>
+__global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
+    __shared__ uint32_t counter[4];
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    __syncthreads();
+    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave]);
+}
+
+template <int BITS, bool RAGGED>
+__global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
+    __shared__ uint32_t counter[4];
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    __syncthreads();
+    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave]);
+}
+
+// K and V of one layer in one launch, one workgroup of 12 wavefronts per CU owning an equal
+// contiguous share of both tensors: every wavefront takes V tiles until the workgroup's share
+// is gone, then K units; the fine-grained K units level what the coarse V tiles leave uneven,
+// and the launch and pipeline-fill time is paid once.
+template <int KB, int VB, bool RAGGED>
+__global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk, StoreKArgs ka, const __half *xv, uint8_t *pv,
+                                                  StoreVArgs va) {
+    __shared__ uint32_t counter[2];
+    if (threadIdx.x < 2) counter[threadIdx.x] = 0;
+    __syncthreads();
+    store_v_units<VB, RAGGED>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
+                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0]);
+    store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
+                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1]);
 }
 
 // ---- K2: fused quantise + pack ---------------------------------------------------
@@ -1192,6 +1253,33 @@ int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_
     DISPATCH_T(in_dtype, TI, return launch_wht128<TI>(x, y, n, out_dtype, sa, sb, s));
 }
 
+// fp16 input with a sign-symmetric codebook: rotation on the matrix cores, codes packed in
+// registers.  The butterfly kernel serves every other case and can be forced with
+// TQ_STORE_PATH=butterfly.
+static bool store_fast_ok(const tq_handle *h, int in_dtype, int64_t n_blocks) {
+    static const bool force_butterfly = [] {
+        const char *e = getenv("TQ_STORE_PATH");
+        return e && strcmp(e, "butterfly") == 0;
+    }();
+    return in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && n_blocks < (1ll << 28) && !force_butterfly;
+}
+
+static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {
+    StoreKArgs ka;
+    ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
+    ka.norm_correction = h->norm_correction; ka.tokens = tokens;
+    ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
+    return ka;
+}
+
+static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {
+    StoreVArgs va;
+    va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
+    va.norm_correction = h->norm_correction; va.tokens = tokens;
+    va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
+    return va;
+}
+
 int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
               uint8_t *sign_bits, void *rnorms, hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
@@ -1219,54 +1307,37 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 #undef TQ_STOREQ_BITS
         return tq_check_launch("store_qjl");
     }
-    // fp16 input with a sign-symmetric codebook: rotation on the matrix cores.  The butterfly
-    // kernel serves every other case and can be forced with TQ_STORE_PATH=butterfly.
-    static const bool force_butterfly = [] {
-        const char *e = getenv("TQ_STORE_PATH");
-        return e && strcmp(e, "butterfly") == 0;
-    }();
-    if (in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && n_seqs * bps < (1ll << 28) && !force_butterfly) {
+    if (store_fast_ok(h, in_dtype, n_seqs * bps)) {
         const int64_t n_blocks = n_seqs * bps;
+        const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
         if (kind == TQ_KIND_K) {
-            StoreKArgs ka;
-            ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
-            ka.norm_correction = h->norm_correction; ka.tokens = tokens;
-            ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
-            // one wavefront per 16-token unit, four resident workgroups per CU
+            const StoreKArgs ka = make_k_args(h, tokens, bps, n_blocks);
+            // four workgroups of four wavefronts per CU
             const unsigned kgrid = (unsigned)((ka.n_units + 3) / 4 < 1024 ? (ka.n_units + 3) / 4 : 1024);
-            const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
 #define TQ_STORE_K(B)                                                                                   \
     if (ragged) k_store_k<B, true><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);       \
     else k_store_k<B, false><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka)
             switch (h->bits) {
             case 2: TQ_STORE_K(2); break;
             case 3: TQ_STORE_K(3); break;
-            case 4: TQ_STORE_K(4); break;
-            default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+            default: TQ_STORE_K(4); break;
             }
 #undef TQ_STORE_K
             return tq_check_launch("store_k");
         }
-        {
-            StoreVArgs va;
-            va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
-            va.norm_correction = h->norm_correction; va.tokens = tokens;
-            va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
-            // one wavefront per 64-token tile, three resident workgroups per CU
-            const unsigned vgrid = (unsigned)((va.n_units + 3) / 4 < 768 ? (va.n_units + 3) / 4 : 768);
-            const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
+        const StoreVArgs va = make_v_args(h, tokens, bps, n_blocks);
+        // three workgroups of four wavefronts per CU
+        const unsigned vgrid = (unsigned)((va.n_units + 3) / 4 < 768 ? (va.n_units + 3) / 4 : 768);
 #define TQ_STORE_V(B)                                                                                   \
     if (ragged) k_store_v<B, true><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);       \
     else k_store_v<B, false><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va)
-            switch (h->bits) {
-            case 2: TQ_STORE_V(2); break;
-            case 3: TQ_STORE_V(3); break;
-            case 4: TQ_STORE_V(4); break;
-            default: tq_set_error("tq_store: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
-            }
-#undef TQ_STORE_V
-            return tq_check_launch("store_v");
+        switch (h->bits) {
+        case 2: TQ_STORE_V(2); break;
+        case 3: TQ_STORE_V(3); break;
+        default: TQ_STORE_V(4); break;
         }
+#undef TQ_STORE_V
+        return tq_check_launch("store_v");
     }
     StoreArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
@@ -1282,6 +1353,41 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
     }
 #undef TQ_STORE_BITS
     return tq_check_launch("store");
+}
+
+int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
+                 int in_dtype, void *packed_k, void *packed_v, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens), n_blocks = n_seqs * bps;
+    if (n_blocks == 0) return TQ_OK;
+    if (!store_fast_ok(hk, in_dtype, n_blocks) || !store_fast_ok(hv, in_dtype, n_blocks)) {
+        const int rc = tqk_store(hk, k, n_seqs, tokens, in_dtype, TQ_KIND_K, packed_k, nullptr, nullptr, s);
+        return rc ? rc : tqk_store(hv, v, n_seqs, tokens, in_dtype, TQ_KIND_V, packed_v, nullptr, nullptr, s);
+    }
+    const StoreKArgs ka = make_k_args(hk, tokens, bps, n_blocks);
+    const StoreVArgs va = make_v_args(hv, tokens, bps, n_blocks);
+    const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
+    // one workgroup of 12 wavefronts per CU
+    const unsigned wg = 768;
+    const unsigned grid = (unsigned)((va.n_units + 11) / 12 < 256 ? (va.n_units + 11) / 12 : 256);
+#define TQ_KV(KB, VB)                                                                                                       \
+    if (ragged) k_store_kv<KB, VB, true><<<grid, wg, 0, s>>>((const __half *)k, (uint8_t *)packed_k, ka, (const __half *)v, \
+                                                              (uint8_t *)packed_v, va);                                      \
+    else k_store_kv<KB, VB, false><<<grid, wg, 0, s>>>((const __half *)k, (uint8_t *)packed_k, ka, (const __half *)v,        \
+                                                        (uint8_t *)packed_v, va)
+#define TQ_KV_V(KB)                      \
+    switch (hv->bits) {                  \
+    case 2: TQ_KV(KB, 2); break;         \
+    case 3: TQ_KV(KB, 3); break;         \
+    default: TQ_KV(KB, 4); break;        \
+    }
+    switch (hk->bits) {
+    case 2: TQ_KV_V(2); break;
+    case 3: TQ_KV_V(3); break;
+    default: TQ_KV_V(4); break;
+    }
+#undef TQ_KV_V
+#undef TQ_KV
+    return tq_check_launch("store_kv");
 }
 
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,

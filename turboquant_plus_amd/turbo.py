@@ -103,6 +103,20 @@ class TurboCodec:
                                  L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
 
+    def store_kv(self, v_codec: "TurboCodec", k, v):
+        """K with this codec and V with `v_codec` in one launch -> (packed_k, packed_v);
+        the same bytes as store(k, "k") and v_codec.store(v, "v")."""
+        tt = L.torch()
+        kd, n_seqs, tokens = self._as_seqs(k)
+        vd, n_seqs_v, tokens_v = v_codec._as_seqs(v)
+        if (n_seqs, tokens) != (n_seqs_v, tokens_v) or kd.dtype != vd.dtype:
+            raise ValueError("k and v must have the same shape and dtype")
+        pk = tt.empty(packed_bytes(self.bits, n_seqs, tokens), dtype=tt.uint8, device=kd.device)
+        pv = tt.empty(packed_bytes(v_codec.bits, n_seqs, tokens), dtype=tt.uint8, device=kd.device)
+        L.check(L.lib().tq_store_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, tokens,
+                                    L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
+        return pk, pv
+
     def store_qjl(self, x):
         """K-layout codes plus the residual sign sketch -> (packed, sign_bits [n,16] uint8, rnorms [n] fp16)."""
         tt = L.torch()
