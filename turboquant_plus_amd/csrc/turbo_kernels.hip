@@ -380,7 +380,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #pragma unroll
     for (int j = 0; j < 4; ++j) flip[j] = a.s2flip[kc * 4 + j];
 
-    const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
+    const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
     // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
     // The address is always valid: units past the end and rows past a sequence's last token
     // are clamped, and `valid` says whether the data is to be used.
@@ -717,7 +717,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // an exact zero counts as positive only if the middle boundary is below zero
     const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
 
-    const uint32_t bps = a.blocks_per_seq, last_unit = a.n_units - 1;
+    const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
     // A operand of sub-tile u: row r = lane%16 is token 16(r/4) + 4u + r%4 of the tile, this lane
     // supplies inputs 32ks + 8kq .. +7.  The address is always valid (clamped); `valid` says
     // whether the row exists.

@@ -103,7 +103,7 @@ class TurboCodec:
                                  L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
 
-    def store_kv(self, v_codec: "TurboCodec", k, v):
+    def store_kv(self, v_codec: "TurboCodec", k, v, out_k=None, out_v=None):
         """K with this codec and V with `v_codec` in one launch -> (packed_k, packed_v);
         the same bytes as store(k, "k") and v_codec.store(v, "v")."""
         tt = L.torch()
@@ -111,8 +111,11 @@ class TurboCodec:
         vd, n_seqs_v, tokens_v = v_codec._as_seqs(v)
         if (n_seqs, tokens) != (n_seqs_v, tokens_v) or kd.dtype != vd.dtype:
             raise ValueError("k and v must have the same shape and dtype")
-        pk = tt.empty(packed_bytes(self.bits, n_seqs, tokens), dtype=tt.uint8, device=kd.device)
-        pv = tt.empty(packed_bytes(v_codec.bits, n_seqs, tokens), dtype=tt.uint8, device=kd.device)
+        nk, nv = packed_bytes(self.bits, n_seqs, tokens), packed_bytes(v_codec.bits, n_seqs, tokens)
+        pk = tt.empty(nk, dtype=tt.uint8, device=kd.device) if out_k is None else out_k
+        pv = tt.empty(nv, dtype=tt.uint8, device=kd.device) if out_v is None else out_v
+        if pk.numel() < nk or pv.numel() < nv:
+            raise ValueError(f"output buffers hold {pk.numel()} and {pv.numel()} bytes, need {nk} and {nv}")
         L.check(L.lib().tq_store_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, tokens,
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
