@@ -128,6 +128,18 @@ int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, 
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                 int64_t tokens, int in_dtype, void *packed_k, void *packed_v, void *stream);
 
+/* Streaming append: n_new tokens per sequence at token positions pos .. pos+n_new-1 of a
+ * packed buffer laid out for `capacity` tokens per sequence (tq_packed_bytes(bits, n_seqs,
+ * capacity)); x is [n_seqs, n_new, 128].  The per-token compress step that kv_cache.py:65-66
+ * names ("compress_token") and PLAN.md:119-122 plans; the reference does not implement it.
+ * Same arithmetic as tq_store on fp32/fp64 input; the touched 128-token blocks are rebuilt:
+ * rows before pos are kept, rows from pos+n_new to the end of the last touched block get the
+ * code of 0.0 and norm 0 (what tq_store writes past the end of a sequence).  After appends
+ * covering tokens 0 .. T-1 in any chunking the touched blocks equal tq_store's of the first T
+ * tokens.  Appends to one buffer must be ordered (same stream). */
+int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity,
+              int in_dtype, int kind, void *packed, void *stream);
+
 /* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
  * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
  * original domain (transpose rotation applied). */
@@ -163,6 +175,8 @@ int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q
 typedef struct tq_attn_params {
     int32_t batch, n_q_heads, n_kv_heads;  /* GQA group = n_q_heads / n_kv_heads, must be 4 */
     int64_t tokens;                        /* context length per sequence                    */
+    int64_t capacity;                      /* tokens per sequence the K/V buffers are laid   */
+                                           /* out for (tq_append caches); 0 = tokens         */
     int32_t n_splits;                      /* context splits per (batch, kv head), >= 1      */
     int32_t k_format;                      /* TQ_KFMT_TURBO | TQ_KFMT_Q8_0                   */
     float scale;                           /* logit scale, e.g. 1/sqrt(128)                  */

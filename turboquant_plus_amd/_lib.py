@@ -30,7 +30,7 @@ class TQConfig(C.Structure):
 
 class TQAttnParams(C.Structure):
     _fields_ = [("batch", C.c_int32), ("n_q_heads", C.c_int32), ("n_kv_heads", C.c_int32), ("tokens", C.c_int64),
-                ("n_splits", C.c_int32), ("k_format", C.c_int32), ("scale", C.c_float), ("sparse_v_tau", C.c_float)]
+                ("capacity", C.c_int64), ("n_splits", C.c_int32), ("k_format", C.c_int32), ("scale", C.c_float), ("sparse_v_tau", C.c_float)]
 
 
 _P, _I, _L, _D = C.c_void_p, C.c_int, C.c_int64, C.c_double
@@ -55,6 +55,7 @@ PROTOTYPES = {
     "tq_packed_bytes": (_L, [C.c_int32, _L, _L]),
     "tq_store": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
     "tq_store_kv": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P]),
+    "tq_append": (_I, [_P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_load": (_I, [_P, _P, _L, _L, _I, _P, _I, _I, _P]),
     "tq_unpack_codes": (_I, [_P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_store_qjl": (_I, [_P, _P, _L, _L, _I, _P, _P, _P, _P]),

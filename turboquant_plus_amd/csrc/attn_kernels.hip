@@ -508,7 +508,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.part_ml = part_ml;
     a.skip = skip_count;
     a.tokens = p->tokens;
-    a.blocks_per_seq = (p->tokens + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
+    a.blocks_per_seq = ((p->capacity > 0 ? p->capacity : p->tokens) + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
     a.n_groups = groups;
     a.n_splits = p->n_splits;
     a.n_tiles = (int)((p->tokens + 63) / 64);

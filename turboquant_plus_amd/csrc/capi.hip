@@ -377,6 +377,20 @@ int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, 
     return tqk_store(h, x, n_seqs, tokens, in_dtype, kind, packed, nullptr, nullptr, (hipStream_t)stream);
 }
 
+int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
+              int kind, void *packed, void *stream) {
+    int rc = check_fast(h, "tq_append");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && pos >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_append: bad argument");
+    REQUIRE(pos + n_new <= capacity, TQ_ERR_ARG, "tq_append: tokens %lld..%lld do not fit a capacity of %lld", (long long)pos,
+            (long long)(pos + n_new), (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(x && packed, TQ_ERR_ARG, "tq_append: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_append: bad kind %d", kind);
+    REQUIRE(aligned16(x) && aligned16(packed), TQ_ERR_ALIGN, "tq_append: x and packed must be 16-byte aligned");
+    return tqk_append(h, x, n_seqs, pos, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream);
+}
+
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
                 int in_dtype, void *packed_k, void *packed_v, void *stream) {
     int rc = check_fast(hk, "tq_store_kv");
@@ -446,6 +460,8 @@ static int check_attn(const tq_attn_params *p) {
     REQUIRE(p->k_format == TQ_KFMT_TURBO || p->k_format == TQ_KFMT_Q8_0, TQ_ERR_ARG, "attention: bad k_format %d",
             p->k_format);
     REQUIRE(p->tokens < ((int64_t)1 << 36), TQ_ERR_UNSUPPORTED, "attention: context too long");
+    REQUIRE(p->capacity == 0 || p->capacity >= p->tokens, TQ_ERR_ARG, "attention: capacity %lld < tokens %lld",
+            (long long)p->capacity, (long long)p->tokens);
     REQUIRE(p->sparse_v_tau >= 0.0f, TQ_ERR_ARG, "attention: sparse_v_tau must be >= 0");
     return TQ_OK;
 }

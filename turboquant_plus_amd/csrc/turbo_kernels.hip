@@ -925,6 +925,44 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
 }
 
 // ---- K2: fused quantise + pack ---------------------------------------------------
+// One vector on the 16 lanes of a DPP row, 8 values per lane: norm, s1, 128-point butterfly,
+// s2/sqrt(128), normalise, compare-count against the boundaries, sum c^2.  Returns the
+// lane's 8 codes as bytes and (valid on every lane of the row) the norm to store.
+template <int BITS>
+__device__ __forceinline__ float quantize_vec16(float (&xv)[8], int lane, const float (&bnd)[(1 << BITS) - 1], const float (&s1v)[8],
+                                                const float (&s2v)[8], const float *csq_s, int norm_correction, uint2 &codes8) {
+    constexpr int NB = (1 << BITS) - 1;
+    float ss = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) ss = fmaf(xv[m], xv[m], ss);
+    ss = row16_sum(ss);
+    const float norm = sqrtf(ss);
+    const float inv = norm > 0.0f ? 1.0f / norm : 1.0f;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) xv[m] *= s1v[m];
+    wht128_row16(xv, lane);
+    uint32_t w0 = 0, w1 = 0;
+    float cs = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        const float yv = (xv[m] * s2v[m]) * inv;
+        uint32_t c = 0;
+#pragma unroll
+        for (int k = 0; k < NB; ++k) c += (bnd[k] < yv) ? 1u : 0u;
+        cs += csq_s[c];
+        if (m < 4) w0 |= c << (8 * m);
+        else w1 |= c << (8 * (m - 4));
+    }
+    cs = row16_sum(cs);
+    codes8 = make_uint2(w0, w1);
+    float g = norm;
+    if (norm_correction) {
+        const float cn = sqrtf(cs);
+        g = norm / (cn > 1e-10f ? cn : 1.0f);
+    }
+    return g;
+}
+
 template <int BITS, typename TI>
 __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, StoreArgs a) {
     constexpr int NB = (1 << BITS) - 1;
@@ -964,40 +1002,85 @@ __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, Sto
 #pragma unroll
             for (int m = 0; m < 8; ++m) xv[m] = 0.0f;
         }
-        float ss = 0.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) ss = fmaf(xv[m], xv[m], ss);
-        ss = row16_sum(ss);
-        const float norm = sqrtf(ss);
-        const float inv = norm > 0.0f ? 1.0f / norm : 1.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) xv[m] *= s1v[m];
-        wht128_row16(xv, lane);
-        uint32_t w0 = 0, w1 = 0;
-        float cs = 0.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            const float yv = (xv[m] * s2v[m]) * inv;
-            uint32_t c = 0;
-#pragma unroll
-            for (int k = 0; k < NB; ++k) c += (bnd[k] < yv) ? 1u : 0u;
-            cs += csq_s[c];
-            if (m < 4) w0 |= c << (8 * m);
-            else w1 |= c << (8 * (m - 4));
-        }
-        cs = row16_sum(cs);
-        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(w0, w1);
-        if (li == 0) {
-            float g = norm;
-            if (a.norm_correction) {
-                const float cn = sqrtf(cs);
-                g = norm / (cn > 1e-10f ? cn : 1.0f);
-            }
-            norms_s[t] = g;
-        }
+        uint2 c8;
+        const float g = quantize_vec16<BITS>(xv, lane, bnd, s1v, s2v, csq_s, a.norm_correction, c8);
+        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = c8;
+        if (li == 0) norms_s[t] = g;
     }
     __syncthreads();
     pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), a.kind);
+}
+
+// ---- K2, streaming append -------------------------------------------------------------
+// n_new tokens per sequence at positions pos .. pos+n_new-1 of a buffer laid out for
+// blocks_per_seq blocks per sequence.  One workgroup per touched block rebuilds the block:
+// rows before pos are unpacked from the block itself, the new rows are quantised exactly as
+// k_store does, the rest get the code of 0.0 and norm 0 (what k_store writes past the end of a
+// sequence), and pack_block writes the block back.  After any sequence of appends covering
+// tokens 0 .. T-1 the touched blocks equal those of k_store on the first T tokens.
+struct AppendArgs {
+    const float *s1, *s2, *bounds, *cent;
+    int kind, norm_correction;
+    int64_t pos, n_new, blocks_per_seq, first_block, n_touched;
+};
+
+__device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, int token, int dim);
+__device__ inline float block_norm(const uint8_t *block, int bits, int token);
+
+template <int BITS, typename TI>
+__global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, AppendArgs a) {
+    constexpr int NB = (1 << BITS) - 1;
+    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
+    __shared__ float csq_s[1 << BITS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int li = lane & 15, grp = tid >> 4;
+    const int64_t seq = blockIdx.x / a.n_touched, bis = a.first_block + blockIdx.x % a.n_touched;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    uint8_t *block = packed + (seq * a.blocks_per_seq + bis) * block_bytes(BITS);
+
+    float bnd[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) bnd[k] = a.bounds[k];
+    if (tid < (1 << BITS)) {
+        const float c = a.cent[tid];
+        csq_s[tid] = c * c;
+    }
+    float s1v[8], s2v[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        s1v[m] = a.s1[8 * li + m];
+        s2v[m] = a.s2[8 * li + m] * RSQRT128;
+    }
+    // rows already in the block
+    const int n_old = (int)(a.pos - tok0 < 0 ? 0 : (a.pos - tok0 > TQ_ROWS_PER_BLOCK ? TQ_ROWS_PER_BLOCK : a.pos - tok0));
+    for (int e = tid; e < n_old * 128; e += 256) {
+        const int t = e >> 7, dim = e & 127;
+        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(block, BITS, a.kind, t, dim);
+    }
+    for (int t = tid; t < n_old; t += 256) norms_s[t] = block_norm(block, BITS, t);
+    __syncthreads();
+
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
+        if (t < n_old) continue;  // whole 16-lane rows skip together
+        const int64_t rel = tok0 + t - a.pos;
+        float xv[8];
+        if (rel < a.n_new) {
+            load8(x + ((seq * a.n_new + rel) * 128 + 8 * li), xv);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) xv[m] = 0.0f;
+        }
+        uint2 c8;
+        const float g = quantize_vec16<BITS>(xv, lane, bnd, s1v, s2v, csq_s, a.norm_correction, c8);
+        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = c8;
+        if (li == 0) norms_s[t] = g;
+    }
+    __syncthreads();
+    pack_block<BITS, 256>(codes, norms_s, block, a.kind);
 }
 
 // ---- K2 + K4 in float64: codes, corrected norm, residual sign sketch ---------------
@@ -1353,6 +1436,28 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
     }
 #undef TQ_STORE_BITS
     return tq_check_launch("store");
+}
+
+int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
+               int kind, void *packed, hipStream_t s) {
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    AppendArgs a;
+    a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
+    a.kind = kind; a.norm_correction = h->norm_correction;
+    a.pos = pos; a.n_new = n_new; a.blocks_per_seq = blocks_for(capacity);
+    a.first_block = pos / TQ_ROWS_PER_BLOCK;
+    a.n_touched = (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
+    const unsigned grid = (unsigned)(n_seqs * a.n_touched);
+#define TQ_APPEND_BITS(B) \
+    DISPATCH_T(in_dtype, TI, (k_append<B, TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, a)))
+    switch (h->bits) {
+    case 2: TQ_APPEND_BITS(2); break;
+    case 3: TQ_APPEND_BITS(3); break;
+    case 4: TQ_APPEND_BITS(4); break;
+    default: tq_set_error("tq_append: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+    }
+#undef TQ_APPEND_BITS
+    return tq_check_launch("append");
 }
 
 int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,

@@ -120,6 +120,17 @@ class TurboCodec:
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
 
+    def append(self, x, packed, pos: int, capacity: int, kind: str = "k"):
+        """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of
+        `packed`, a buffer of packed_bytes(bits, n_seqs, capacity) bytes (tq_append)."""
+        xd, n_seqs, n_new = self._as_seqs(x)
+        need = packed_bytes(self.bits, n_seqs, capacity)
+        if packed.numel() < need:
+            raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
+        L.check(L.lib().tq_append(self.handle.h, L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
+                                  L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+        return packed
+
     def store_qjl(self, x):
         """K-layout codes plus the residual sign sketch -> (packed, sign_bits [n,16] uint8, rnorms [n] fp16)."""
         tt = L.torch()
@@ -205,14 +216,15 @@ class DecodeAttention:
     """
 
     def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec, batch: int, n_q_heads: int, n_kv_heads: int,
-                 tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0):
+                 tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0,
+                 capacity: int = 0):
         tt = L.torch()
         dev = L.require_gpu()
         self.k_codec, self.v_codec = k_codec, v_codec
         if n_splits is None:
             n_splits = default_splits(batch * n_kv_heads, tokens)
         self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
-                                     n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
+                                     capacity=capacity, n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
                                      scale=(1.0 / math.sqrt(HEAD_DIM)) if scale is None else scale,
                                      sparse_v_tau=sparse_v_tau)
         nbytes = L.lib().tq_attn_workspace_bytes(C.byref(self.params))
@@ -233,6 +245,13 @@ class DecodeAttention:
                                             L.ptr(self.workspace),
                                             self.workspace.numel(), L.stream_ptr()))
         return self.out
+
+    def set_tokens(self, tokens: int) -> None:
+        """Context length of the next calls (a cache that grows by append); the
+        buffers stay laid out for `capacity` tokens per sequence."""
+        if self.params.capacity and tokens > self.params.capacity:
+            raise ValueError(f"tokens {tokens} exceed the capacity {self.params.capacity}")
+        self.params.tokens = tokens
 
     def skip_rate(self) -> float:
         s = self.skip.cpu().numpy()
