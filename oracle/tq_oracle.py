@@ -344,6 +344,59 @@ class TurboMSERef:
         return self.polar_quant.dequantize(idx, norms)
 
 
+def channel_split(d: int, target_bits: float):
+    """outlier.py:45-67: (n_outlier, high_bits, n_normal, low_bits); the high-rate
+    channels are the first round(d * frac) ones."""
+    low = int(np.floor(target_bits))
+    n_out = int(round(d * (target_bits - low)))
+    return n_out, low + 1, d - n_out, low
+
+
+class OutlierRef:
+    """outlier.py:70-217: channels 0..n_outlier-1 through PolarQuant(high-1 bits, seed),
+    the rest through PolarQuant(low-1 bits, seed+500), QJL(seed+1000) on the full residual.
+    Returns plain tuples (outlier idx, outlier norms, normal idx, normal norms, signs,
+    residual norms)."""
+
+    def __init__(self, d, target_bits, seed=42):
+        self.d, self.target_bits = d, target_bits
+        self.n_outlier, self.high_bits, self.n_normal, self.low_bits = channel_split(d, target_bits)
+        self.effective_bits = (self.n_outlier * self.high_bits + self.n_normal * self.low_bits) / d
+        self.pq_outlier = PolarRef(self.n_outlier, self.high_bits - 1, seed) if self.n_outlier > 0 else None
+        self.pq_normal = PolarRef(self.n_normal, self.low_bits - 1, seed + 500) if self.n_normal > 0 else None
+        self.qjl = QJLRef(d, seed + 1000)
+
+    def quantize(self, x):
+        x = np.asarray(x, dtype=np.float64)
+        single = x.ndim == 1
+        xb = x[None] if single else x
+        parts, res = [], np.zeros_like(xb)
+        for pq, sl in ((self.pq_outlier, slice(0, self.n_outlier)), (self.pq_normal, slice(self.n_outlier, self.d))):
+            if pq is None:
+                parts += [np.array([]), np.array([])]
+                continue
+            sub = xb[:, np.arange(sl.start, sl.stop)]    # gathered as the reference does (outlier.py:119-120): the
+                                                         # memory order of the result decides the summation order of the norm
+            idx, n, r = pq.quantize_and_residual(sub if xb.shape[0] > 1 else sub[0])   # outlier.py:124,132
+            res[:, sl] = r
+            parts += [idx, n]
+        z, rn = self.qjl.quantize(res[0] if single else res)
+        return (*parts, z, rn)
+
+    def dequantize(self, c):
+        oi, on, ni, nn, z, rn = c
+        xq = self.qjl.dequantize(z, rn)
+        out = np.zeros_like(xq)
+        if self.pq_outlier is not None:
+            out[..., :self.n_outlier] = self.pq_outlier.dequantize(oi, on)
+        if self.pq_normal is not None:
+            out[..., self.n_outlier:] = self.pq_normal.dequantize(ni, nn)
+        return out + xq
+
+    def compression_ratio(self, original_bits=16):
+        return self.d * original_bits / (self.d * self.effective_bits + 32 + 64)   # outlier.py:209-217
+
+
 @dataclass
 class CompressedKVRef:
     k_compressed: list = field(default_factory=list)

@@ -126,6 +126,29 @@ fp = utils.memory_footprint_bytes(1000, 128, 3)
 out["footprint_1000_128_3"] = np.array([fp["mse_indices_bytes"], fp["qjl_signs_bytes"], fp["norms_bytes"],
                                         fp["total_bytes"], fp["original_fp16_bytes"]], dtype=np.int64)
 
+# ---- outlier-channel split (fractional bit rates) ----------------------------
+from turboquant.outlier import OutlierTurboQuant, _compute_channel_split  # noqa: E402
+
+out["outlier_split_args"] = np.array([[128, 2.5], [128, 3.5], [128, 3.25], [64, 2.5], [100, 3.5], [128, 3.0]])
+out["outlier_split_vals"] = np.array([_compute_channel_split(int(d_), b_) for d_, b_ in out["outlier_split_args"]],
+                                     dtype=np.int64)
+xo = np.random.default_rng(77).standard_normal((6, D))
+xo[2] = 0.0
+xo[4] *= 25.0
+out["outlier_x"] = xo
+for tb in (2.5, 3.5):
+    oq = OutlierTurboQuant(D, tb, seed=42)
+    tag = f"outlier_{str(tb).replace('.', 'p')}"
+    cv = oq.quantize(xo)
+    out[f"{tag}_oidx"], out[f"{tag}_onorm"] = cv.outlier_indices.astype(np.uint8), cv.outlier_norms
+    out[f"{tag}_nidx"], out[f"{tag}_nnorm"] = cv.normal_indices.astype(np.uint8), cv.normal_norms
+    out[f"{tag}_signs"], out[f"{tag}_rnorm"] = cv.qjl_signs, cv.residual_norms
+    out[f"{tag}_deq"] = oq.dequantize(cv)
+    c1 = oq.quantize(xo[1])
+    out[f"{tag}_single_deq"] = oq.dequantize(c1)
+    out[f"{tag}_meta"] = np.array([oq.n_outlier, oq.high_bits, oq.n_normal, oq.low_bits, oq.effective_bits,
+                                   oq.compression_ratio(), oq.compression_ratio(32)])
+
 # ---- BASELINE config 1: composition of reference functions ----------------
 X = np.random.default_rng(0).standard_normal((4096, D)).astype(np.float32)
 sd = np.random.default_rng(1).choice([-1.0, 1.0], size=D)

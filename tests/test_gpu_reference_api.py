@@ -201,6 +201,46 @@ def test_turboquant_golden(golden, b):
     np.testing.assert_allclose(tq.dequantize(single), golden[f"tq_deq_b{b}"][1], rtol=1e-10, atol=1e-12)
 
 
+@pytest.mark.parametrize("tb", [2.5, 3.5])
+def test_outlier_turboquant_golden(golden, tb):
+    """OutlierTurboQuant (turboquant/outlier.py:70-217) against vectors written from the reference; the
+    properties are those of the reference's tests/test_outlier.py."""
+    tag = f"outlier_{str(tb).replace('.', 'p')}"
+    oq = tqa.OutlierTurboQuant(D, tb, seed=42)
+    meta = golden[f"{tag}_meta"]
+    assert [oq.n_outlier, oq.high_bits, oq.n_normal, oq.low_bits] == [int(v) for v in meta[:4]]
+    assert oq.effective_bits == pytest.approx(tb, abs=0.01)
+    assert oq.compression_ratio() == meta[5] and oq.compression_ratio(32) == meta[6]
+    x = golden["outlier_x"]
+    c = oq.quantize(x)
+    assert c.effective_bits == oq.effective_bits
+    assert np.array_equal(c.outlier_indices, golden[f"{tag}_oidx"]) and np.array_equal(c.normal_indices, golden[f"{tag}_nidx"])
+    assert np.array_equal(c.qjl_signs, golden[f"{tag}_signs"])
+    np.testing.assert_allclose(c.outlier_norms, golden[f"{tag}_onorm"], rtol=1e-14)
+    np.testing.assert_allclose(c.normal_norms, golden[f"{tag}_nnorm"], rtol=1e-14)
+    np.testing.assert_allclose(c.residual_norms, golden[f"{tag}_rnorm"], rtol=1e-11, atol=1e-13)
+    deq = oq.dequantize(c)
+    np.testing.assert_allclose(deq, golden[f"{tag}_deq"], rtol=1e-11, atol=1e-12)
+    # batch == single, determinism (tests/test_outlier.py:81-112)
+    for i in (0, 1, 4):
+        np.testing.assert_allclose(oq.dequantize(oq.quantize(x[i])), deq[i], atol=1e-10)
+    np.testing.assert_allclose(oq.dequantize(oq.quantize(x[1])), golden[f"{tag}_single_deq"], rtol=1e-11, atol=1e-12)
+    assert np.array_equal(tqa.OutlierTurboQuant(D, tb, seed=42).dequantize(c), deq)
+
+
+def test_outlier_turboquant_quality_and_whole_bits():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((200, D))
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    oq = tqa.OutlierTurboQuant(D, 3.5, seed=42)
+    mse = np.mean(np.sum((oq.dequantize(oq.quantize(x)) - x) ** 2, axis=1))
+    assert mse < 0.03 * 2.0                                  # tests/test_outlier.py:30-48
+    whole = tqa.OutlierTurboQuant(D, 3.0, seed=42)           # no high-rate channels
+    assert whole.pq_outlier is None and whole.n_normal == D
+    assert whole.dequantize(whole.quantize(x[:3])).shape == (3, D)
+    assert tqa.OutlierTurboQuant(D, 2.5).compression_ratio() > 4.5 and tqa.OutlierTurboQuant(D, 3.5).compression_ratio() > 3.5
+
+
 @pytest.mark.parametrize("d", [96, 160, 192, 320])
 def test_turbo4_non_power_of_two_dims(d):
     x = np.random.default_rng(d).standard_normal((20, d))

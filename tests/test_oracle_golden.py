@@ -108,6 +108,34 @@ def test_turboquant(golden, b):
     assert tq.compression_ratio() == float(golden[f"tq_ratio_b{b}"])
 
 
+@pytest.mark.parametrize("tb", [2.5, 3.5])
+def test_outlier_split_quantiser(golden, tb):
+    """turboquant/outlier.py:45-217, fixtures written from the reference."""
+    tag = f"outlier_{str(tb).replace('.', 'p')}"
+    oq = O.OutlierRef(D, tb, seed=42)
+    meta = golden[f"{tag}_meta"]
+    assert [oq.n_outlier, oq.high_bits, oq.n_normal, oq.low_bits] == [int(v) for v in meta[:4]]
+    assert oq.effective_bits == meta[4] and oq.compression_ratio() == meta[5] and oq.compression_ratio(32) == meta[6]
+    c = oq.quantize(golden["outlier_x"])
+    assert np.array_equal(c[0], golden[f"{tag}_oidx"]) and np.array_equal(c[2], golden[f"{tag}_nidx"])
+    assert np.array_equal(c[1], golden[f"{tag}_onorm"]) and np.array_equal(c[3], golden[f"{tag}_nnorm"])
+    assert np.array_equal(c[4], golden[f"{tag}_signs"])
+    np.testing.assert_allclose(c[5], golden[f"{tag}_rnorm"], rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(oq.dequantize(c), golden[f"{tag}_deq"], rtol=1e-11, atol=1e-12)
+    single = oq.quantize(golden["outlier_x"][1])
+    np.testing.assert_allclose(oq.dequantize(single), golden[f"{tag}_single_deq"], rtol=1e-11, atol=1e-12)
+
+
+def test_outlier_channel_split(golden):
+    for (d, tb), want in zip(golden["outlier_split_args"], golden["outlier_split_vals"]):
+        assert list(O.channel_split(int(d), float(tb))) == [int(v) for v in want]
+    # a whole number of bits leaves no high-rate channels (one PolarQuant only)
+    oq = O.OutlierRef(D, 3.0, seed=42)
+    assert oq.pq_outlier is None and oq.n_normal == D
+    x = np.random.default_rng(0).standard_normal((4, D))
+    assert oq.dequantize(oq.quantize(x)).shape == (4, D)
+
+
 def test_kv_cache(golden):
     kv = O.KVRef(D, 3, 3, seed=42)
     c = kv.compress(golden["kv_k"], golden["kv_v"])

@@ -9,7 +9,9 @@ from .polar_quant import PolarQuant
 from .qjl import QJL
 from .turboquant import TurboQuant, TurboQuantMSE, CompressedVector
 from .kv_cache import KVCacheCompressor, CompressedKVCache
+from .outlier import OutlierTurboQuant, OutlierCompressedVector
 from .turbo import TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, packed_bytes
 
 __all__ = ["PolarQuant", "QJL", "TurboQuant", "TurboQuantMSE", "CompressedVector", "KVCacheCompressor",
+           "OutlierTurboQuant", "OutlierCompressedVector",
            "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "packed_bytes"]
