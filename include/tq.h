@@ -140,6 +140,15 @@ int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const v
 int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity,
               int in_dtype, int kind, void *packed, void *stream);
 
+/* Temporal decay: re-quantise a packed buffer to a narrower width without going back to the
+ * original vectors (`requantize_3to2`, benchmarks/temporal_decay_prototype.py:93-125): per row
+ * decode with the stored norm, renormalise, nearest centroid of `dst`'s codebook (a value equal
+ * to a midpoint takes the higher index, as np.digitize does there), corrected fp16 norm for the
+ * new codes.  src holds tq_packed_bytes(src bits, ..) bytes, dst tq_packed_bytes(dst bits, ..);
+ * width pairs 3->2, 4->3, 4->2; both handles must describe the same rotation. */
+int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs,
+                  int64_t tokens, int kind, void *packed_dst, void *stream);
+
 /* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
  * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
  * original domain (transpose rotation applied). */

@@ -534,6 +534,31 @@ def turbo_decode(idx, g, centroids, s1, s2):
     return rotate_fast(turbo_decode_rotated(idx, g, centroids), s1, s2, len(s1), transpose=True)
 
 
+def requantize(idx_src, g_src, cent_src, cent_dst, mid_dst=None):
+    """Temporal decay of a stored row to a narrower codebook, in the rotated domain
+    (benchmarks/temporal_decay_prototype.py:93-125, `requantize_3to2`): decode with the
+    stored (corrected) norm, renormalise, nearest narrower centroid by np.digitize over
+    the midpoints (a value equal to a midpoint takes the HIGHER index, unlike
+    nearest_index), corrected norm for the new codes.  Rows are independent."""
+    idx_src = np.asarray(idx_src)
+    g_src = np.asarray(g_src, dtype=np.float64)
+    mid = midpoints(cent_dst) if mid_dst is None else np.asarray(mid_dst, dtype=np.float64)
+    idx_out = np.zeros(idx_src.shape, dtype=np.uint8)
+    g_out = np.zeros(g_src.shape, dtype=np.float64)
+    for r in range(idx_src.shape[0]):
+        values = cent_src[idx_src[r]] * g_src[r]
+        recon = np.linalg.norm(values)
+        if recon > 1e-10:
+            normalized = values / recon
+        else:
+            normalized, recon = values, 0.0
+        i2 = np.digitize(normalized, mid)
+        cn = np.sqrt(np.sum(cent_dst[i2] ** 2))
+        idx_out[r] = i2
+        g_out[r] = recon / cn if cn > 1e-10 else recon
+    return idx_out, g_out
+
+
 def boundary_band_mismatches(y, idx_test, centroids, rel=1e-6):
     """Classify index mismatches against the fp64 decision values `y`.
 

@@ -149,6 +149,25 @@ for tb in (2.5, 3.5):
     out[f"{tag}_meta"] = np.array([oq.n_outlier, oq.high_bits, oq.n_normal, oq.low_bits, oq.effective_bits,
                                    oq.compression_ratio(), oq.compression_ratio(32)])
 
+# ---- temporal decay: 3-bit block -> 2-bit (benchmarks/temporal_decay_prototype.py:93-125) ----
+sys.path.insert(0, os.path.join(ref_root, "benchmarks"))
+import temporal_decay_prototype as tdp  # noqa: E402
+
+out["decay_c3"], out["decay_c2"] = tdp.CENTROIDS_3BIT, tdp.CENTROIDS_2BIT
+out["decay_mid3"], out["decay_mid2"] = tdp.MIDPOINTS_3BIT, tdp.MIDPOINTS_2BIT
+rd = np.random.default_rng(91)
+yd = rd.standard_normal((48, D))
+yd /= np.linalg.norm(yd, axis=1, keepdims=True)
+i3 = np.stack([tdp.quantize_3bit(r) for r in yd])
+n3 = np.abs(rd.standard_normal(48)) * 10.0
+n3[5] = 0.0
+out["decay_idx3"], out["decay_norm3"] = i3, n3
+rq = [tdp.requantize_3to2(i3[r], n3[r]) for r in range(48)]
+out["decay_idx2"] = np.stack([r_[0] for r_ in rq])
+out["decay_norm2"] = np.array([r_[1] for r_ in rq])
+out["decay_deq3"] = np.stack([tdp.dequantize_3bit(i3[r], n3[r]) for r in range(48)])
+out["decay_deq2"] = np.stack([tdp.dequantize_2bit(out["decay_idx2"][r], out["decay_norm2"][r]) for r in range(48)])
+
 # ---- BASELINE config 1: composition of reference functions ----------------
 X = np.random.default_rng(0).standard_normal((4096, D)).astype(np.float32)
 sd = np.random.default_rng(1).choice([-1.0, 1.0], size=D)

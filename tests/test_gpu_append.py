@@ -97,3 +97,68 @@ def test_decode_attention_over_a_growing_cache():
         assert np.array_equal(got, want), f"context {T}"
     with pytest.raises(ValueError):
         grow.set_tokens(capacity + 1)
+
+
+# ---- temporal decay: re-quantise packed rows to a narrower codebook ---------------------------
+
+def _check_requant(src, dst, packed_src, n_seqs, tokens, kind):
+    idx_s, g_s = src.unpack_codes(packed_src, n_seqs, tokens, kind=kind)
+    out = src.requantize_to(dst, packed_src, n_seqs, tokens, kind=kind)
+    assert out.numel() == tqa.packed_bytes(dst.bits, n_seqs, tokens)
+    idx_d, g_d = dst.unpack_codes(out, n_seqs, tokens, kind=kind)
+    idx_s, g_s = np_(idx_s).reshape(-1, D), np_(g_s).reshape(-1).astype(np.float64)
+    idx_d, g_d = np_(idx_d).reshape(-1, D), np_(g_d).reshape(-1)
+    want_idx, want_g = O.requantize(idx_s, g_s, src.centroids, dst.centroids)
+    # decision values of the oracle, for the boundary-band accounting of mismatching codes
+    vals = src.centroids[idx_s] * g_s[:, None]
+    nrm = np.linalg.norm(vals, axis=1, keepdims=True)
+    y = np.where(nrm > 1e-10, vals / np.where(nrm > 1e-10, nrm, 1.0), vals)
+    live = g_s != 0                                     # rows of all-zero vectors decode to 0 whatever their codes
+    n_bad, n_inadm = O.boundary_band_mismatches(y[live], idx_d[live], dst.centroids, rel=1e-6)
+    assert n_inadm == 0 and n_bad <= max(2, 2e-5 * idx_d.size)
+    same = np.all(idx_d == want_idx, axis=1)
+    a = g_d.astype(np.float16)[same].view(np.uint16).astype(np.int32)
+    b = want_g.astype(np.float16)[same].view(np.uint16).astype(np.int32)
+    assert np.abs(a - b).max(initial=0) <= 1 and (np.abs(a - b) == 1).sum() <= max(2, 2e-3 * a.size)
+    assert np.all(g_d[~live] == 0)
+    return out
+
+
+def test_requantize_3_to_2_prototype_presets(golden):
+    """The prototype's literal centroid presets, its rows, device format in between."""
+    c3, c2 = golden["decay_c3"], golden["decay_c2"]
+    src, dst = tqa.TurboCodec(3, seed=9, centroids=c3), tqa.TurboCodec(2, seed=9, centroids=c2)
+    idx3 = np.zeros((128, D), dtype=np.uint8)
+    idx3[:48] = golden["decay_idx3"]
+    g3 = np.zeros(128, dtype=np.float16)
+    g3[:48] = (golden["decay_norm3"] / np.sqrt(np.sum(c3[golden["decay_idx3"]] ** 2, axis=1))).astype(np.float16)
+    for kind in ("k", "v"):
+        packed = L.torch().from_numpy(O.layout_pack(idx3, g3, 3, kind)).cuda()
+        out = _check_requant(src, dst, packed, 1, 128, kind)
+        i2, g2 = O.layout_unpack(np_(out), 2, kind)
+        assert np.array_equal(i2[:48], golden["decay_idx2"])          # fp16 norms do not move these decisions
+
+
+@pytest.mark.parametrize("pair", [(3, 2), (4, 3), (4, 2)])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_requantize_stored_cache(pair, kind):
+    sb, db = pair
+    src, dst = tqa.TurboCodec(sb, seed=42), tqa.TurboCodec(db, seed=42)
+    x = np.random.default_rng(sb * 10 + db).standard_normal((3, 200, D)).astype(np.float16)
+    x[2, 7] = 0
+    packed = src.store(x, kind=kind)
+    out = _check_requant(src, dst, packed, 3, 200, kind)
+    # decayed rows still reconstruct the input: error between the two widths' own errors
+    rec_s = np_(src.load(packed, 3, 200, kind=kind, domain="original"))
+    rec_d = np_(dst.load(out, 3, 200, kind=kind, domain="original"))
+    direct = np_(dst.load(dst.store(x, kind=kind), 3, 200, kind=kind, domain="original"))
+    xf = x.astype(np.float64)
+    err = lambda r: float(np.mean(np.sum((r - xf) ** 2, -1)) / np.mean(np.sum(xf ** 2, -1)))
+    assert err(rec_s) < err(rec_d) < 1.6 * err(direct)
+
+
+def test_requantize_rejects_widening():
+    a, b = tqa.TurboCodec(2, seed=1), tqa.TurboCodec(3, seed=1)
+    buf = L.torch().zeros(tqa.packed_bytes(2, 1, 128), dtype=L.torch().uint8, device="cuda")
+    with pytest.raises(NotImplementedError):
+        a.requantize_to(b, buf, 1, 128)

@@ -136,6 +136,22 @@ def test_outlier_channel_split(golden):
     assert oq.dequantize(oq.quantize(x)).shape == (4, D)
 
 
+def test_temporal_decay_requantize(golden):
+    """3-bit rows -> 2-bit (benchmarks/temporal_decay_prototype.py:93-125); the prototype
+    takes the uncorrected norm and corrects at read time, the device format stores the corrected norm."""
+    c3, c2 = golden["decay_c3"], golden["decay_c2"]
+    idx3, n3 = golden["decay_idx3"], golden["decay_norm3"]
+    rn = np.sqrt(np.sum(c3[idx3] ** 2, axis=1))
+    g3 = n3 / rn                                        # corrected norm, as dequantize_3bit forms it
+    np.testing.assert_allclose(c3[idx3] * g3[:, None], golden["decay_deq3"], rtol=1e-15, atol=0)
+    idx2, g2 = O.requantize(idx3, g3, c3, c2, mid_dst=golden["decay_mid2"])
+    assert np.array_equal(idx2, golden["decay_idx2"])
+    np.testing.assert_allclose(g2, golden["decay_norm2"], rtol=1e-14, atol=0)
+    assert g2[5] == 0.0 and np.all(idx2[5] == 2)        # zero row: digitize(0.0) over (-m, 0, m)
+    # default midpoints are those of the preset centroids
+    np.testing.assert_allclose(O.midpoints(c2), golden["decay_mid2"], atol=1e-12)
+
+
 def test_kv_cache(golden):
     kv = O.KVRef(D, 3, 3, seed=42)
     c = kv.compress(golden["kv_k"], golden["kv_v"])

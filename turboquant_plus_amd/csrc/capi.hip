@@ -391,6 +391,21 @@ int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, in
     return tqk_append(h, x, n_seqs, pos, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream);
 }
 
+int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs, int64_t tokens,
+                  int kind, void *packed_dst, void *stream) {
+    int rc = check_fast(src_h, "tq_requantize");
+    rc = rc ? rc : check_fast(dst_h, "tq_requantize");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_requantize: bad argument");
+    REQUIRE(dst_h->bits < src_h->bits, TQ_ERR_UNSUPPORTED, "tq_requantize: destination must be narrower (%d -> %d bits)",
+            src_h->bits, dst_h->bits);
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(packed_src && packed_dst, TQ_ERR_ARG, "tq_requantize: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_requantize: bad kind %d", kind);
+    REQUIRE(aligned16(packed_src) && aligned16(packed_dst), TQ_ERR_ALIGN, "tq_requantize: buffers must be 16-byte aligned");
+    return tqk_requantize(src_h, dst_h, packed_src, n_seqs, tokens, kind, packed_dst, (hipStream_t)stream);
+}
+
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
                 int in_dtype, void *packed_k, void *packed_v, void *stream) {
     int rc = check_fast(hk, "tq_store_kv");

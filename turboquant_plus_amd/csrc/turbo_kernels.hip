@@ -1438,6 +1438,94 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
     return tq_check_launch("store");
 }
 
+// ---- temporal decay: re-quantise packed rows to a narrower codebook ------------------------
+// Per row in the rotated domain: values = c_src[idx] * g, renormalise, nearest centroid of the
+// destination codebook, corrected norm for the new codes.  One workgroup per block: unpack into
+// the LDS stage, 16 lanes per row, pack with the destination width.
+struct RequantArgs {
+    const float *cent_src, *cent_dst, *bounds_dst;
+    int kind;
+};
+
+template <int SB, int DB>
+__global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t *dst, RequantArgs a) {
+    constexpr int NB = (1 << DB) - 1;
+    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
+    __shared__ float csrc_s[1 << SB], cdst_s[1 << DB];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int li = lane & 15, grp = tid >> 4;
+    const uint8_t *sblock = src + (int64_t)blockIdx.x * block_bytes(SB);
+    if (tid < (1 << SB)) csrc_s[tid] = a.cent_src[tid];
+    if (tid < (1 << DB)) cdst_s[tid] = a.cent_dst[tid];
+    float bnd[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) bnd[k] = a.bounds_dst[k];
+    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
+        const int t = e >> 7, dim = e & 127;
+        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(sblock, SB, a.kind, t, dim);
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
+        const uint2 c8 = *reinterpret_cast<const uint2 *>(&codes[t * CODE_STRIDE + 8 * li]);
+        const float g = block_norm(sblock, SB, t);
+        float v[8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint32_t c = ((m < 4 ? c8.x : c8.y) >> (8 * (m & 3))) & 0xFFu;
+            v[m] = csrc_s[c] * g;
+            ss = fmaf(v[m], v[m], ss);
+        }
+        ss = row16_sum(ss);
+        float recon = sqrtf(ss);
+        const float inv = recon > 1e-10f ? 1.0f / recon : 1.0f;
+        if (!(recon > 1e-10f)) recon = 0.0f;
+        uint32_t w0 = 0, w1 = 0;
+        float cs = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const float yv = v[m] * inv;
+            uint32_t c = 0;
+#pragma unroll
+            for (int k = 0; k < NB; ++k) c += (bnd[k] <= yv) ? 1u : 0u;  // a value on a midpoint takes the higher index
+            const float cd = cdst_s[c];
+            cs = fmaf(cd, cd, cs);
+            if (m < 4) w0 |= c << (8 * m);
+            else w1 |= c << (8 * (m - 4));
+        }
+        cs = row16_sum(cs);
+        __builtin_amdgcn_wave_barrier();
+        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(w0, w1);
+        if (li == 0) {
+            const float cn = sqrtf(cs);
+            norms_s[t] = cn > 1e-10f ? recon / cn : recon;
+        }
+    }
+    __syncthreads();
+    pack_block<DB, 256>(codes, norms_s, dst + (int64_t)blockIdx.x * block_bytes(DB), a.kind);
+}
+
+int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
+                   hipStream_t s) {
+    const unsigned grid = (unsigned)(n_seqs * blocks_for(tokens));
+    if (grid == 0) return TQ_OK;
+    RequantArgs a;
+    a.cent_src = hs->centroids32; a.cent_dst = hd->centroids32; a.bounds_dst = hd->bounds32; a.kind = kind;
+    const int key = hs->bits * 10 + hd->bits;
+    switch (key) {
+    case 32: k_requantize<3, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
+    case 43: k_requantize<4, 3><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
+    case 42: k_requantize<4, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
+    default:
+        tq_set_error("tq_requantize: supported width pairs are 3->2, 4->3, 4->2 (got %d->%d)", hs->bits, hd->bits);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    return tq_check_launch("requantize");
+}
+
 int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
                int kind, void *packed, hipStream_t s) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;

@@ -131,6 +131,15 @@ class TurboCodec:
                                   L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
         return packed
 
+    def requantize_to(self, dst_codec: "TurboCodec", packed, n_seqs: int, tokens: int, kind: str = "k"):
+        """Temporal decay: re-quantise a buffer written with this codec to the narrower
+        `dst_codec` (same rotation) -> new packed buffer (tq_requantize)."""
+        tt = L.torch()
+        out = tt.empty(packed_bytes(dst_codec.bits, n_seqs, tokens), dtype=tt.uint8, device=packed.device)
+        L.check(L.lib().tq_requantize(self.handle.h, dst_codec.handle.h, L.ptr(packed), n_seqs, tokens,
+                                      L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        return out
+
     def store_qjl(self, x):
         """K-layout codes plus the residual sign sketch -> (packed, sign_bits [n,16] uint8, rnorms [n] fp16)."""
         tt = L.torch()
