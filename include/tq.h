@@ -149,6 +149,20 @@ int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, in
 int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs,
                   int64_t tokens, int kind, void *packed_dst, void *stream);
 
+/* Interchange with the llama.cpp fork's per-128 block layout, one block per vector in token
+ * order: norm fp16 | qs[32] | signs[16] (turbo3, 50 B: idx = low2 | hi1 << 2, low2 =
+ * (qs[j/4] >> ((j%4)*2)) & 3, hi1 = (signs[j/8] >> (j%8)) & 1; docs/papers/block-size-experiment.md:33-39,
+ * docs/papers/turbo4-resurrection.md:130-134), norm | qs[64] nibbles (turbo4, 66 B; :169), norm | qs[32]
+ * (turbo2, 34 B).  The norm is the corrected group norm in both formats, so codes and norms move
+ * unchanged; blocks is [n_seqs, tokens, tq_fork_block_bytes(bits)] bytes.  Import fills the rows
+ * past `tokens` of the last block like tq_store does.  The layout is known from the fork's
+ * documents only (the reference tree holds no code for it). */
+int64_t tq_fork_block_bytes(int32_t bits);
+int tq_export_fork_blocks(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind,
+                          void *blocks, void *stream);
+int tq_import_fork_blocks(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind,
+                          void *packed, void *stream);
+
 /* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
  * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
  * original domain (transpose rotation applied). */

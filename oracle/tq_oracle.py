@@ -15,6 +15,8 @@ step by step (citations are file:line in the reference tree):
   TurboQuant    turboquant/turboquant.py:33-171
   KV cache      turboquant/kv_cache.py:30-188
   bit packing   turboquant/utils.py:20-123
+  outlier split turboquant/outlier.py:45-217
+  temporal decay benchmarks/temporal_decay_prototype.py:93-125
 
 Pinned by (see tests/test_oracle_*.py): golden vectors written from the
 reference itself (tests/golden/), scipy.linalg.hadamard, brute-force argmin,
@@ -23,8 +25,10 @@ pack bytes and size arithmetic.
 
 Parity unpinned (no reference code exists for them; closed forms and brute
 force only): `q8_0_quantize`/`q8_0_dequantize` (textbook ggml block format),
-`decode_attention` (rotated-domain attention, Sparse-V predicate, split
-boundaries) and `score_tile` in its `gaussian` projection mode.
+`fork_blocks_pack`/`fork_blocks_unpack` (the llama.cpp fork's block layout,
+known from its documents only), `decode_attention` (rotated-domain attention,
+Sparse-V predicate, split boundaries) and `score_tile` in its `gaussian`
+projection mode.
 """
 from __future__ import annotations
 
@@ -699,6 +703,51 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
         q[:, :, 1] = hi.reshape(T // 64, 64, 32, 2).transpose(0, 2, 3, 1)
         idx = q.reshape(T, 128)
     return idx, g
+
+
+# --------------------------------------------------------------------------
+# Per-128 block layout of the llama.cpp fork, as its documents state it (no code for it exists in
+# the reference tree, so parity with the fork itself is unpinned): one block per 128-value vector,
+#   turbo3: norm fp16 | qs[32] | signs[16]  (50 B), idx = low2 | hi1 << 2,
+#           low2 = (qs[j/4] >> ((j%4)*2)) & 3, hi1 = (signs[j/8] >> (j%8)) & 1
+#           (docs/papers/block-size-experiment.md:33-39, docs/papers/turbo4-resurrection.md:130-134)
+#   turbo4: norm fp16 | qs[64]  (66 B), idx = (qs[j/2] >> ((j%2)*4)) & 0xF (turbo4-resurrection.md:169)
+#   turbo2: norm fp16 | qs[32]  (34 B), idx = (qs[j/4] >> ((j%4)*2)) & 3   (the 2-bit half of turbo3)
+# --------------------------------------------------------------------------
+
+def fork_block_bytes(bits: int) -> int:
+    return {2: 34, 3: 50, 4: 66}[bits]
+
+
+def fork_blocks_pack(idx: np.ndarray, g: np.ndarray, bits: int) -> np.ndarray:
+    """idx [T,128], g [T] fp16 -> uint8 [T, fork_block_bytes(bits)], token order."""
+    idx = np.asarray(idx).astype(np.uint8)
+    T = idx.shape[0]
+    out = np.zeros((T, fork_block_bytes(bits)), dtype=np.uint8)
+    out[:, 0:2] = np.asarray(g, dtype=np.float16).reshape(T, 1).view(np.uint8)
+    if bits == 4:
+        out[:, 2:66] = idx[:, 0::2] | (idx[:, 1::2] << 4)
+        return out
+    low = idx & 3
+    out[:, 2:34] = low[:, 0::4] | (low[:, 1::4] << 2) | (low[:, 2::4] << 4) | (low[:, 3::4] << 6)
+    if bits == 3:
+        hi = (idx >> 2) & 1
+        out[:, 34:50] = np.packbits(hi, axis=1, bitorder="little")
+    return out
+
+
+def fork_blocks_unpack(buf: np.ndarray, bits: int):
+    buf = np.asarray(buf, dtype=np.uint8).reshape(-1, fork_block_bytes(bits))
+    T = buf.shape[0]
+    g = np.ascontiguousarray(buf[:, 0:2]).view(np.float16).reshape(T)
+    j = np.arange(128)
+    if bits == 4:
+        idx = (buf[:, 2 + j // 2] >> ((j % 2) * 4)) & 0xF
+        return idx.astype(np.uint8), g
+    idx = (buf[:, 2 + j // 4] >> ((j % 4) * 2)) & 3
+    if bits == 3:
+        idx = idx | (((buf[:, 34 + j // 8] >> (j % 8)) & 1) << 2)
+    return idx.astype(np.uint8), g
 
 
 # --------------------------------------------------------------------------

@@ -162,3 +162,37 @@ def test_requantize_rejects_widening():
     buf = L.torch().zeros(tqa.packed_bytes(2, 1, 128), dtype=L.torch().uint8, device="cuda")
     with pytest.raises(NotImplementedError):
         a.requantize_to(b, buf, 1, 128)
+
+
+# ---- interchange with the fork's per-128 block layout ------------------------------------------
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_fork_blocks_export_import(bits, kind):
+    codec = tqa.TurboCodec(bits, seed=42, centroids=tqa.PRODUCTION_CENTROIDS[bits])
+    n_seqs, tokens = 3, 200
+    x = np.random.default_rng(bits).standard_normal((n_seqs, tokens, D)).astype(np.float16)
+    x[0, 9] = 0
+    packed = codec.store(x, kind=kind)
+    idx, g = codec.unpack_codes(packed, n_seqs, tokens, kind=kind)
+    idx, g = np_(idx).reshape(-1, D), np_(g).reshape(-1)
+    check_codes(codec, x.reshape(-1, D), idx, g)                      # the fork's centroid tables quantise like any other
+    blocks = codec.export_fork_blocks(packed, n_seqs, tokens, kind=kind)
+    assert tuple(blocks.shape) == (n_seqs, tokens, O.fork_block_bytes(bits))
+    want = O.fork_blocks_pack(idx, g.astype(np.float16), bits).reshape(n_seqs, tokens, -1)
+    assert np.array_equal(np_(blocks), want)
+    back = codec.import_fork_blocks(blocks, kind=kind)
+    assert np.array_equal(np_(back), np_(packed))                     # including the padding rows of the last block
+    # blocks written elsewhere (here: by the oracle from random codes) come in as the same codes
+    rng = np.random.default_rng(1)
+    ridx = rng.integers(0, 1 << bits, size=(2 * 128, D)).astype(np.uint8)
+    rg = np.abs(rng.standard_normal(2 * 128)).astype(np.float16)
+    ext = O.fork_blocks_pack(ridx, rg, bits).reshape(2, 128, -1)
+    i2, g2 = codec.unpack_codes(codec.import_fork_blocks(ext, kind=kind), 2, 128, kind=kind)
+    assert np.array_equal(np_(i2).reshape(-1, D), ridx) and np.array_equal(np_(g2).reshape(-1).astype(np.float16), rg)
+
+
+def test_fork_blocks_rejects_wrong_width():
+    codec = tqa.TurboCodec(3, seed=42)
+    with pytest.raises(ValueError):
+        codec.import_fork_blocks(np.zeros((1, 128, 66), dtype=np.uint8))

@@ -243,3 +243,30 @@ def test_score_tile_is_dequantised_inner_product():
     tile = O.score_tile(qs, c.mse_indices, g, cent, lambda a: O.rotate_fast(a, pq.s1, pq.s2, pq.pd),
                         tq.qjl.S, c.qjl_signs, c.residual_norms, tq.qjl.scale)
     np.testing.assert_allclose(tile, direct, atol=1e-11)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_fork_block_layout_formulas(bits):
+    """Per-128 block layout of the llama.cpp fork: the extraction formulas printed in
+    docs/papers/turbo4-resurrection.md:130-134,169 and the sizes of docs/papers/block-size-experiment.md:33-39,
+    applied element by element to what fork_blocks_pack wrote."""
+    rng = np.random.default_rng(bits)
+    idx = rng.integers(0, 1 << bits, size=(5, 128)).astype(np.uint8)
+    g = rng.standard_normal(5).astype(np.float16)
+    buf = O.fork_blocks_pack(idx, g, bits)
+    assert buf.shape == (5, {2: 34, 3: 50, 4: 66}[bits])
+    for t in range(5):
+        row = buf[t]
+        assert row[:2].view(np.float16)[0] == g[t]
+        qs = row[2:66] if bits == 4 else row[2:34]
+        signs = row[34:50] if bits == 3 else None
+        for j in range(128):
+            if bits == 4:
+                got = (qs[j // 2] >> ((j % 2) * 4)) & 0xF
+            else:
+                got = (qs[j // 4] >> ((j % 4) * 2)) & 0x3
+                if bits == 3 and signs[j // 8] & (1 << (j % 8)):
+                    got |= 4
+            assert got == idx[t, j]
+    i2, g2 = O.fork_blocks_unpack(buf, bits)
+    assert np.array_equal(i2, idx) and np.array_equal(g2.view(np.uint16), g.view(np.uint16))

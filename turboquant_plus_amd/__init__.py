@@ -10,8 +10,9 @@ from .qjl import QJL
 from .turboquant import TurboQuant, TurboQuantMSE, CompressedVector
 from .kv_cache import KVCacheCompressor, CompressedKVCache
 from .outlier import OutlierTurboQuant, OutlierCompressedVector
-from .turbo import TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, packed_bytes
+from .turbo import TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, packed_bytes, PRODUCTION_CENTROIDS
 
 __all__ = ["PolarQuant", "QJL", "TurboQuant", "TurboQuantMSE", "CompressedVector", "KVCacheCompressor",
            "OutlierTurboQuant", "OutlierCompressedVector",
-           "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "packed_bytes"]
+           "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "packed_bytes",
+           "PRODUCTION_CENTROIDS"]

@@ -57,6 +57,9 @@ PROTOTYPES = {
     "tq_store_kv": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_append": (_I, [_P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_requantize": (_I, [_P, _P, _P, _L, _L, _I, _P, _P]),
+    "tq_fork_block_bytes": (_L, [C.c_int32]),
+    "tq_export_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
+    "tq_import_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
     "tq_load": (_I, [_P, _P, _L, _L, _I, _P, _I, _I, _P]),
     "tq_unpack_codes": (_I, [_P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_store_qjl": (_I, [_P, _P, _L, _L, _I, _P, _P, _P, _P]),

@@ -123,6 +123,8 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
     int rc = TQ_OK;
     std::vector<double> cent(cfg->centroids, cfg->centroids + nc), bounds(nc - 1);
     for (int k = 0; k + 1 < nc; ++k) bounds[k] = (cent[k] + cent[k + 1]) / 2.0;
+    h->zero_code = 0;
+    for (int k = 0; k + 1 < nc; ++k) h->zero_code += bounds[k] < 0.0 ? 1 : 0;
     rc = rc ? rc : upload(&h->centroids64, cent);
     rc = rc ? rc : upload(&h->bounds64, bounds);
     std::vector<double> s1, s2;
@@ -404,6 +406,30 @@ int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *pa
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_requantize: bad kind %d", kind);
     REQUIRE(aligned16(packed_src) && aligned16(packed_dst), TQ_ERR_ALIGN, "tq_requantize: buffers must be 16-byte aligned");
     return tqk_requantize(src_h, dst_h, packed_src, n_seqs, tokens, kind, packed_dst, (hipStream_t)stream);
+}
+
+static int fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
+                       void *stream, const char *who) {
+    int rc = check_fast(h, who);
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "%s: bad argument", who);
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(src && dst, TQ_ERR_ARG, "%s: null pointer", who);
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "%s: bad kind %d", who, kind);
+    REQUIRE(aligned16(to_fork ? src : dst), TQ_ERR_ALIGN, "%s: the packed buffer must be 16-byte aligned", who);
+    return tqk_fork_blocks(h, to_fork, src, n_seqs, tokens, kind, dst, (hipStream_t)stream);
+}
+
+int64_t tq_fork_block_bytes(int32_t bits) { return bits == 3 ? 50 : bits == 4 ? 66 : bits == 2 ? 34 : -1; }
+
+int tq_export_fork_blocks(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *blocks,
+                          void *stream) {
+    return fork_blocks(h, 1, packed, n_seqs, tokens, kind, blocks, stream, "tq_export_fork_blocks");
+}
+
+int tq_import_fork_blocks(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind, void *packed,
+                          void *stream) {
+    return fork_blocks(h, 0, blocks, n_seqs, tokens, kind, packed, stream, "tq_import_fork_blocks");
 }
 
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,

@@ -37,6 +37,7 @@ struct tq_handle {
     uint32_t *s2flip;      // [4][4]: per lane quarter and output dword, sign-field positions of dims with s2 = +1
     float *symthr32;       // [2^(bits-1)]: middle boundary, then the positive boundaries
     float *sqcoef32;       // [2^(bits-1)]: c[mid+1+m]^2 = sum over subsets S of the set bits of m of sqcoef32[S]
+    int zero_code;         // codebook index of the value 0.0 (#boundaries below 0)
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };
 
@@ -71,6 +72,8 @@ int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, i
                int kind, void *packed, hipStream_t s);
 int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                    hipStream_t s);
+int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
+                    hipStream_t s);
 int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
                  int in_dtype, void *packed_k, void *packed_v, hipStream_t s);
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,

@@ -1526,6 +1526,105 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
     return tq_check_launch("requantize");
 }
 
+// ---- interchange with the per-128 block layout of the llama.cpp fork --------------------------
+// One block per vector, token order: norm fp16 | qs | signs (3-bit: two low bits of every index
+// in qs, the third in signs; 4-bit: nibbles; 2-bit: qs only) - 50 / 66 / 34 bytes.
+__host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 66 : 34; }
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_fork_export(const uint8_t *packed, uint8_t *out, int kind, int64_t tokens,
+                                                     int64_t blocks_per_seq) {
+    constexpr int FB = fork_block_bytes(BITS);
+    __shared__ uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    const int tid = threadIdx.x;
+    const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const uint8_t *block = packed + blk * block_bytes(BITS);
+    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
+        const int t = e >> 7, dim = e & 127;
+        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(block, BITS, kind, t, dim);
+    }
+    __syncthreads();
+    // one output byte per thread and step: byte b of the row of token t
+    for (int e = tid; e < TQ_ROWS_PER_BLOCK * FB; e += 256) {
+        const int t = e / FB, b = e % FB;
+        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
+        if (tok >= tokens) continue;
+        const uint8_t *c = codes + t * CODE_STRIDE;
+        uint32_t v;
+        if (b < 2) {
+            v = (reinterpret_cast<const uint16_t *>(block + block_code_bytes(BITS))[t] >> (8 * b)) & 0xFFu;
+        } else if (BITS == 4) {
+            const int j = 2 * (b - 2);
+            v = c[j] | (c[j + 1] << 4);
+        } else if (b < 34) {
+            const int j = 4 * (b - 2);
+            v = (c[j] & 3) | ((c[j + 1] & 3) << 2) | ((c[j + 2] & 3) << 4) | ((c[j + 3] & 3) << 6);
+        } else {
+            const int j = 8 * (b - 34);
+            v = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v |= ((c[j + k] >> 2) & 1u) << k;
+        }
+        out[(seq * tokens + tok) * FB + b] = (uint8_t)v;
+    }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_fork_import(const uint8_t *in, uint8_t *packed, int kind, int64_t tokens,
+                                                     int64_t blocks_per_seq, uint32_t zero_code) {
+    constexpr int FB = fork_block_bytes(BITS);
+    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
+    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
+    const int tid = threadIdx.x;
+    const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
+        const int t = e >> 7, j = e & 127;
+        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
+        uint32_t c = zero_code;  // rows past the end: what the store kernels write there
+        if (tok < tokens) {
+            const uint8_t *row = in + (seq * tokens + tok) * FB;
+            if (BITS == 4) c = (row[2 + j / 2] >> ((j % 2) * 4)) & 0xFu;
+            else {
+                c = (row[2 + j / 4] >> ((j % 4) * 2)) & 3u;
+                if (BITS == 3) c |= ((row[34 + j / 8] >> (j % 8)) & 1u) << 2;
+            }
+        }
+        codes[t * CODE_STRIDE + j] = (uint8_t)c;
+    }
+    for (int t = tid; t < TQ_ROWS_PER_BLOCK; t += 256) {
+        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
+        float g = 0.0f;
+        if (tok < tokens) {
+            const uint8_t *row = in + (seq * tokens + tok) * FB;
+            g = __half2float(__ushort_as_half((unsigned short)(row[0] | (row[1] << 8))));
+        }
+        norms_s[t] = g;
+    }
+    __syncthreads();
+    pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), kind);
+}
+
+int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
+                    hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    // index of 0.0: number of boundaries below it (a zero vector stores this code in every dim)
+    uint32_t zero_code = (uint32_t)(h->n_centroids / 2);
+    if (h->zero_code >= 0) zero_code = (uint32_t)h->zero_code;
+#define TQ_FORK(B)                                                                                                        \
+    if (to_fork) k_fork_export<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps);             \
+    else k_fork_import<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps, zero_code)
+    switch (h->bits) {
+    case 2: TQ_FORK(2); break;
+    case 3: TQ_FORK(3); break;
+    case 4: TQ_FORK(4); break;
+    default: tq_set_error("fork blocks: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+    }
+#undef TQ_FORK
+    return tq_check_launch("fork_blocks");
+}
+
 int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
                int kind, void *packed, hipStream_t s) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;

@@ -35,6 +35,17 @@ def packed_bytes(bits: int, n_seqs: int, tokens: int) -> int:
     return int(n)
 
 
+# Centroid tables the llama.cpp fork ships (d = 128), as printed in the reference's documents:
+# 2- and 3-bit benchmarks/temporal_decay_prototype.py:38-46, 4-bit docs/papers/turbo4-resurrection.md:163-166.
+# TurboCodec(bits, centroids=PRODUCTION_CENTROIDS[bits]) makes caches interchangeable with it.
+PRODUCTION_CENTROIDS = {
+    2: np.array([-0.133462, -0.039994, 0.039994, 0.133462]),
+    3: np.array([-0.190685, -0.117832, -0.065717, -0.021460, 0.021460, 0.065717, 0.117832, 0.190685]),
+    4: np.array([-0.1739, -0.1172, -0.0895, -0.0688, -0.0513, -0.0356, -0.0210, -0.0069,
+                 0.0069, 0.0210, 0.0356, 0.0513, 0.0688, 0.0895, 0.1172, 0.1739]),
+}
+
+
 class TurboCodec:
     """One quantiser (rotation signs + codebook [+ QJL projection]) for K or V.
 
@@ -138,6 +149,29 @@ class TurboCodec:
         out = tt.empty(packed_bytes(dst_codec.bits, n_seqs, tokens), dtype=tt.uint8, device=packed.device)
         L.check(L.lib().tq_requantize(self.handle.h, dst_codec.handle.h, L.ptr(packed), n_seqs, tokens,
                                       L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        return out
+
+    def export_fork_blocks(self, packed, n_seqs: int, tokens: int, kind: str = "k"):
+        """-> uint8 [n_seqs, tokens, 50 | 66 | 34]: the llama.cpp fork's per-128 block layout."""
+        tt = L.torch()
+        fb = int(L.lib().tq_fork_block_bytes(self.bits))
+        out = tt.empty((n_seqs, tokens, fb), dtype=tt.uint8, device=packed.device)
+        L.check(L.lib().tq_export_fork_blocks(self.handle.h, L.ptr(packed), n_seqs, tokens,
+                                              L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        return out
+
+    def import_fork_blocks(self, blocks, kind: str = "k"):
+        """Fork blocks [n_seqs, tokens, 50 | 66 | 34] -> packed buffer of this library."""
+        tt = L.torch()
+        dev = L.require_gpu()
+        bd = blocks if isinstance(blocks, tt.Tensor) else tt.from_numpy(np.ascontiguousarray(blocks))
+        if bd.dtype != tt.uint8 or bd.dim() != 3 or bd.shape[2] != int(L.lib().tq_fork_block_bytes(self.bits)):
+            raise ValueError("blocks must be uint8 [n_seqs, tokens, block bytes of this width]")
+        bd = bd.to(dev)
+        n_seqs, tokens = int(bd.shape[0]), int(bd.shape[1])
+        out = tt.empty(packed_bytes(self.bits, n_seqs, tokens), dtype=tt.uint8, device=bd.device)
+        L.check(L.lib().tq_import_fork_blocks(self.handle.h, L.ptr(bd.contiguous()), n_seqs, tokens,
+                                              L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
 
     def store_qjl(self, x):
