@@ -597,12 +597,15 @@ def boundary_band_mismatches(y, idx_test, centroids, rel=1e-6):
 # holds dword j of the four groups.  Inside a group, pair k sits in
 #   b = 4 : byte k%4 of dword k//4
 #   b = 2 : nibble k%8 of dword k//8
-#   b = 3 : bits 6*(k%5).. of dword k//5 for k < 15; pair 15 takes bits 30..31 of
-#           dwords 0, 1, 2 as its low, middle and high two bits.
+#   b = 3 : bits 6*(k%4).. of dword k//4 for k < 12; pairs 12..15 are a 24-bit tail (pair k at tail
+#           bit 6*(k-12)), byte j of which is the top byte of dword j.
+# Pairs 2q, 2q+1 ("quad" q: four values) are contiguous bits in every width, so a reader can index
+# a table by a whole quad.
 # K rows: row = token, pair p = dims (2p, 2p+1).
 # V rows are dim-major inside each 64-token tile: row (token & 64) | (dim & 63)
 #         holds dims r and 64+r of the tile's 64 tokens; tokens 2*tp and 2*tp+1 of
-#         the tile (lo, hi) of dim half hf = dim >> 6 are pair 2*tp + hf.
+#         the tile (lo, hi) of dim half hf = dim >> 6 are pair 4*(tp//2) + 2*hf + tp%2: a quad is four
+#         consecutive tokens of one dim.
 # A BLOCK is 128 rows stored chunk-major: [16*b/16 chunks][128 rows][16 B],
 # followed by 128 fp16 norms (token order).  Block bytes = 128*(16*b + 2).
 
@@ -623,22 +626,26 @@ def _pairs_to_rows(pairs: np.ndarray, bits: int) -> np.ndarray:
     A row is four groups of 16 pairs; group g owns `bits` dwords, and dword j
     of group g is row dword 4*j + g (so 16-byte chunk j of the row holds dword
     j of the four groups).  Inside a group: 4-bit pair k = byte k%4 of dword
-    k/4; 2-bit pair k = nibble k%8 of dword k/8; 3-bit pair k < 15 = bits
-    6*(k%5).. of dword k/5, pair 15 = bits 30..31 of dwords 0, 1, 2 (low,
-    middle, high two bits)."""
+    k/4; 2-bit pair k = nibble k%8 of dword k/8; 3-bit pair k < 12 = bits
+    6*(k%4).. of dword k/4, and pairs 12..15 form a 24-bit tail (pair k at tail
+    bit 6*(k-12)) whose byte j is the top byte of dword j.  Two adjacent pairs
+    2q, 2q+1 (a "quad" of four values) are contiguous bits in every width."""
     pairs = pairs.astype(np.uint32)
     lead = pairs.shape[:-1]
     grp = pairs.reshape(lead + (4, 16))
     out = np.zeros(lead + (4 * bits,), dtype=np.uint32)
     if bits not in (2, 3, 4):
         raise ValueError("bits must be 2, 3 or 4")
-    per, width = {4: (4, 8), 2: (8, 4), 3: (5, 6)}[bits]
+    per, width = {4: (4, 8), 2: (8, 4), 3: (4, 6)}[bits]
     for g in range(4):
-        for k in range(16 if bits != 3 else 15):
+        for k in range(16 if bits != 3 else 12):
             out[..., 4 * (k // per) + g] |= grp[..., g, k] << np.uint32(width * (k % per))
         if bits == 3:
-            for part in range(3):
-                out[..., 4 * part + g] |= ((grp[..., g, 15] >> np.uint32(2 * part)) & np.uint32(3)) << np.uint32(30)
+            tail = np.zeros(lead, dtype=np.uint32)
+            for k in range(12, 16):
+                tail |= grp[..., g, k] << np.uint32(6 * (k - 12))
+            for j in range(3):
+                out[..., 4 * j + g] |= ((tail >> np.uint32(8 * j)) & np.uint32(0xFF)) << np.uint32(24)
     return out
 
 
@@ -646,15 +653,17 @@ def _rows_to_pairs(rows: np.ndarray, bits: int) -> np.ndarray:
     rows = rows.astype(np.uint32)
     if bits not in (2, 3, 4):
         raise ValueError("bits must be 2, 3 or 4")
-    per, width = {4: (4, 8), 2: (8, 4), 3: (5, 6)}[bits]
+    per, width = {4: (4, 8), 2: (8, 4), 3: (4, 6)}[bits]
     mask = np.uint32((1 << width) - 1)
     cols = []
     for g in range(4):
-        for k in range(16 if bits != 3 else 15):
+        for k in range(16 if bits != 3 else 12):
             cols.append((rows[..., 4 * (k // per) + g] >> np.uint32(width * (k % per))) & mask)
         if bits == 3:
-            top = [(rows[..., 4 * part + g] >> np.uint32(30)) & np.uint32(3) for part in range(3)]
-            cols.append(top[0] | (top[1] << np.uint32(2)) | (top[2] << np.uint32(4)))
+            tail = ((rows[..., g] >> np.uint32(24)) | ((rows[..., 4 + g] >> np.uint32(24)) << np.uint32(8))
+                    | ((rows[..., 8 + g] >> np.uint32(24)) << np.uint32(16)))
+            for k in range(12, 16):
+                cols.append((tail >> np.uint32(6 * (k - 12))) & mask)
     return np.stack(cols, axis=-1)
 
 
@@ -667,10 +676,10 @@ def layout_pack(idx: np.ndarray, g: np.ndarray, bits: int, kind: str) -> np.ndar
     if kind == "k":
         pairs = idx[:, 0::2] | (idx[:, 1::2] << np.uint32(bits))          # [T,64]
     else:
-        q = idx.reshape(T // 64, 32, 2, 2, 64)                             # tile, token pair, parity, dim half, r
-        lo = q[:, :, 0].transpose(0, 3, 1, 2)                              # tile, r, token pair, dim half
-        hi = q[:, :, 1].transpose(0, 3, 1, 2)
-        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row = 64*tile + r; pair = 2*tp + half
+        q = idx.reshape(T // 64, 16, 2, 2, 2, 64)                          # tile, token quad, pair in quad, parity, dim half, r
+        lo = q[:, :, :, 0].transpose(0, 4, 1, 3, 2)                        # tile, r, token quad, dim half, pair in quad
+        hi = q[:, :, :, 1].transpose(0, 4, 1, 3, 2)
+        pairs = (lo | (hi << np.uint32(bits))).reshape(T, 64)              # row = 64*tile + r; pair = 4*tq + 2*half + tp%2
     rows = _pairs_to_rows(pairs, bits)                                     # [T, 4*bits]
     rows = rows.reshape(nb, ROWS_PER_BLOCK, bits, 4).transpose(0, 2, 1, 3) # block, chunk, row, 4
     out = np.zeros((nb, block_bytes(bits)), dtype=np.uint8)
@@ -698,9 +707,9 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
         idx[:, 0::2] = lo
         idx[:, 1::2] = hi
     else:
-        q = np.zeros((T // 64, 32, 2, 2, 64), dtype=np.uint8)              # tile, token pair, parity, dim half, r
-        q[:, :, 0] = lo.reshape(T // 64, 64, 32, 2).transpose(0, 2, 3, 1)
-        q[:, :, 1] = hi.reshape(T // 64, 64, 32, 2).transpose(0, 2, 3, 1)
+        q = np.zeros((T // 64, 16, 2, 2, 2, 64), dtype=np.uint8)           # tile, token quad, pair in quad, parity, dim half, r
+        q[:, :, :, 0] = lo.reshape(T // 64, 64, 16, 2, 2).transpose(0, 2, 4, 3, 1)
+        q[:, :, :, 1] = hi.reshape(T // 64, 64, 16, 2, 2).transpose(0, 2, 4, 3, 1)
         idx = q.reshape(T, 128)
     return idx, g
 

@@ -139,6 +139,23 @@ def test_decode_attention_bias_and_sparse_v():
             np.testing.assert_allclose(out_s, out_d, rtol=0, atol=1e-4 * np.abs(ref_d).max())
 
 
+def test_decode_attention_masked_prefix():
+    """-inf bias over a prefix: whole tiles and one whole split carry no weight; output stays finite and equals
+    attention over the remaining positions."""
+    B, Hq, Hkv, N = 1, 8, 2, 1024
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=91)
+    q = np.random.default_rng(92).standard_normal((B, Hq, D)).astype(np.float16)
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    bias[:, :, :300] = -np.inf          # split 0 of 4 (tokens 0..255) is masked completely
+    bias[:, 3, 300:700] = -np.inf       # one head loses two more splits' worth of tiles
+    tt = L.torch()
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=4)(q, kp, vp, bias=tt.from_numpy(bias).cuda()))
+    assert np.isfinite(out).all()
+    finite = np.where(np.isfinite(bias), bias, -1e30).astype(np.float32)   # same weights, no inf arithmetic in the oracle
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), bias=finite)
+    assert_close(out, ref)
+
+
 def test_decode_attention_q8_0_k_turbo2_v():
     """BASELINE config 4 shape family: K q8_0-style (not rotated), V turbo2."""
     B, Hq, Hkv, N = 1, 8, 2, 2048 + 64

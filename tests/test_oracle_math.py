@@ -156,7 +156,8 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
         if kind == "k":
             row, pair, half = tok, dim // 2, dim % 2
         else:
-            row, pair, half = (tok & 64) | (dim & 63), 2 * ((tok & 63) // 2) + (dim >> 6), tok % 2
+            tp = (tok & 63) // 2
+            row, pair, half = (tok & 64) | (dim & 63), 4 * (tp // 2) + 2 * (dim >> 6) + tp % 2, tok % 2
         value = ((1 << bits) - 1) << (bits * half)
         rowwords = words[:, row, :].reshape(-1)
         expect = np.zeros(4 * bits, dtype=np.uint64)
@@ -165,11 +166,12 @@ def test_device_layout_roundtrip_and_placement(bits, kind):
             expect[4 * (k // 4) + grp] = value << (8 * (k % 4))
         elif bits == 2:
             expect[4 * (k // 8) + grp] = value << (4 * (k % 8))
-        elif k < 15:
-            expect[4 * (k // 5) + grp] = value << (6 * (k % 5))
+        elif k < 12:
+            expect[4 * (k // 4) + grp] = value << (6 * (k % 4))
         else:
+            tail = value << (6 * (k - 12))
             for part in range(3):
-                expect[4 * part + grp] = ((value >> (2 * part)) & 3) << 30
+                expect[4 * part + grp] = ((tail >> (8 * part)) & 0xFF) << 24
         assert np.array_equal(rowwords.astype(np.uint64), expect)
         assert np.count_nonzero(words) == np.count_nonzero(expect)
 

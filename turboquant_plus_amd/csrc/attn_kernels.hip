@@ -4,8 +4,10 @@
 //   One 64-lane wavefront owns one context split and walks it in tiles of 64
 //   tokens.  Lane l holds packed row l of the tile (K: token l; V: dims l and
 //   64+l of all 64 tokens), loaded as 16-byte chunks that are contiguous across
-//   lanes.  Pair codes are turned into fp16 pairs through a 4-byte-entry LUT
-//   in LDS (one ds_read per two values) and fed to the 4x4x4 fp16 MFMA with
+//   lanes.  Codes are turned into fp16 values through a table in LDS: for 2- and
+//   3-bit codes a quad table (8-byte entries indexed by the 4*BITS bits of two
+//   adjacent pair codes, one ds_read_b64 per four values = one MFMA operand), for
+//   4-bit codes a pair table (4-byte entries).  They feed the 4x4x4 fp16 MFMA with
 //   16 independent blocks: block b multiplies the 4 tokens 4b..4b+3 by the 4
 //   query heads, so all 64 lanes and all 16 blocks do useful work.
 //   The MFMA's A-matrix broadcast (cbsz = 4, abid = source block) lets one block's
@@ -26,6 +28,7 @@
 //   inside k_decode_attn by each wavefront, so a dense step is two launches.
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+#include <cstring>
 #include <utility>
 
 #include "tq_device.h"
@@ -44,17 +47,48 @@ template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t 
     return pair_lut_offset<BITS>(w, p);
 }
 
+// bytes of the decode table of a codebook: quad entries for BITS <= 3, pair entries for 4
+__host__ __device__ constexpr int lut_bytes(int bits) { return bits <= 3 ? 8 << (4 * bits) : 4 << (2 * bits); }
+
+// the four values of quad Q (pairs 2Q, 2Q+1) of a row as an MFMA operand
+template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_t (&w)[4 * BITS], const char *lut, int Q) {
+    if constexpr (BITS <= 3) {
+        return __builtin_bit_cast(half4_t, *reinterpret_cast<const uint2 *>(lut + quad_lut_offset<BITS>(w, Q)));
+    } else {
+        const uint2 u = make_uint2(*reinterpret_cast<const uint32_t *>(lut + pair_lut_offset<BITS>(w, 2 * Q)),
+                                   *reinterpret_cast<const uint32_t *>(lut + pair_lut_offset<BITS>(w, 2 * Q + 1)));
+        return __builtin_bit_cast(half4_t, u);
+    }
+}
+
+// build a codebook's decode table in LDS from its pair table (half2 per pair code) in global memory
+// (256 threads); every global load is issued before the first LDS write
+template <int BITS> __device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, int tid) {
+    constexpr int NP = 1 << (2 * BITS);
+    if constexpr (BITS == 3) {
+        // lane l holds pair entry l; wavefront w writes the rows hi = w, w + 4, ..
+        uint2 *t = reinterpret_cast<uint2 *>(dst);
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t mine = pair_lut[lane];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int hi = wave + 4 * i;
+            t[hi * 64 + lane] = make_uint2(mine, (uint32_t)__builtin_amdgcn_readlane((int)mine, hi));
+        }
+    } else if constexpr (BITS == 2) {
+        reinterpret_cast<uint2 *>(dst)[tid] = make_uint2(pair_lut[tid & 15], pair_lut[tid >> 4]);
+    } else {
+        static_assert(NP == 256, "pair table of 256 entries");
+        reinterpret_cast<uint32_t *>(dst)[tid] = pair_lut[tid];
+    }
+}
+
 template <int BITS> __device__ __forceinline__ void load_row(const uint8_t *block, int row, uint32_t (&w)[4 * BITS]) {
 #pragma unroll
     for (int c = 0; c < BITS; ++c) {
         const uint4 u = *reinterpret_cast<const uint4 *>(block + c * 2048 + row * 16);
         w[4 * c] = u.x; w[4 * c + 1] = u.y; w[4 * c + 2] = u.z; w[4 * c + 3] = u.w;
     }
-}
-
-__device__ __forceinline__ half4_t h4_from(uint32_t a, uint32_t b) {
-    const uint2 u = make_uint2(a, b);
-    return __builtin_bit_cast(half4_t, u);
 }
 
 __device__ __forceinline__ float4_t mfma4(half4_t a, half4_t b, float4_t c) {
@@ -107,7 +141,7 @@ struct AttnArgs {
     const float *ks1, *ks2;  // K rotation signs (NULL: K is not rotated, q is only scaled)
     float scale_log2e;       // logit scale * log2(e), folded into the fp16 query
     const uint8_t *k, *v;
-    const uint32_t *klut, *vlut;  // pair LUTs (half2 per pair code)
+    const uint32_t *klut, *vlut;  // pair tables (half2 per pair code)
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
     float *part_o;                // [groups][n_splits][4][128]
     float *part_ml;               // [groups][n_splits][4][2]  (m in log2 units, l)
@@ -123,12 +157,7 @@ constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
 template <int BITS, int... G>
 __device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const uint32_t (&kw)[4 * BITS],
                                          const char *lut, const half4_t (&qa)[2], float4_t (&acc)[4]) {
-    ((acc[G & 3] = mfma4_bcast<(G & 15)>(
-          qa[G >> 4],
-          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(kw, 2 * G)),
-                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(kw, 2 * G + 1))),
-          acc[G & 3])),
-     ...);
+    ((acc[G & 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], quad_values<BITS>(kw, lut, G), acc[G & 3])), ...);
 }
 
 // q8_0-style K: one accumulator per 32-value block (dim groups 8*blk .. 8*blk+7), scaled afterwards
@@ -150,40 +179,35 @@ __device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const ui
 template <int BITS, int... T>
 __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const uint32_t (&vw)[4 * BITS],
                                        const char *lut, half4_t pv, float4_t (&acc_o)[2][2]) {
-    // tokens 4T..4T+3 of dim half hf are pairs 4T + hf and 4T + 2 + hf of the row
-    ((acc_o[0][T & 1] = mfma4_bcast<T>(
-          pv,
-          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T)),
-                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 2))),
-          acc_o[0][T & 1]),
-      acc_o[1][T & 1] = mfma4_bcast<T>(
-          pv,
-          h4_from(*reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 1)),
-                  *reinterpret_cast<const uint32_t *>(lut + pair_off<BITS>(vw, 4 * T + 3))),
-          acc_o[1][T & 1])),
+    // tokens 4T..4T+3 of dim half hf are quad 2T + hf of the row
+    ((acc_o[0][T & 1] = mfma4_bcast<T>(pv, quad_values<BITS>(vw, lut, 2 * T), acc_o[0][T & 1]),
+      acc_o[1][T & 1] = mfma4_bcast<T>(pv, quad_values<BITS>(vw, lut, 2 * T + 1), acc_o[1][T & 1])),
      ...);
 }
 
-template <int KFMT, int KBITS, int VBITS, bool SPARSE>
+// SHARE: K and V decode through one table (same width, same centroids); table positions are
+// compile-time constants so that they fold into the LDS instructions' offset fields.
+template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE>
 __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
     constexpr int VBLOCK = TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
-    constexpr int KLUT_N = KFMT == KFMT_TURBO ? (1 << (2 * KBITS)) : 1;
-    constexpr int VLUT_N = 1 << (2 * VBITS);
-    __shared__ uint32_t klut_s[KLUT_N];
-    __shared__ uint32_t vlut_s[VLUT_N];
-    __shared__ __attribute__((aligned(16))) _Float16 q_s[4][4 * 128];  // per wavefront: its group's rotated queries
+    constexpr int KLUT_BYTES = KFMT == KFMT_TURBO ? lut_bytes(KBITS) : 0;
+    static_assert(!SHARE || (KFMT == KFMT_TURBO && KBITS == VBITS), "a shared table needs equal code widths");
+    // static LDS (its address is a compile-time constant, so table positions fold into the LDS
+    // instructions): [K table][V table unless shared with K].  Before the tables are built the
+    // first 4 KB stage the rotated queries, 1 KB per wavefront.
+    constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
+    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 4096 ? LUT_TOTAL : 4096];
+    char *klut_s = smem;
+    char *vlut_s = SHARE ? klut_s : klut_s + KLUT_BYTES;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    if constexpr (KFMT == KFMT_TURBO)
-        for (int i = tid; i < KLUT_N; i += 256) klut_s[i] = a.klut[i];
-    for (int i = tid; i < VLUT_N; i += 256) vlut_s[i] = a.vlut[i];
-    __syncthreads();
-
     const int64_t wid = (int64_t)blockIdx.x * 4 + (tid >> 6);
-    const int group = (int)(wid / a.n_splits), split = (int)(wid % a.n_splits);
-    if (group >= a.n_groups) return;
+    // wave-uniform values in scalar registers: tile loop, block addresses and bounds become scalar work
+    const int group = __builtin_amdgcn_readfirstlane((int)(wid / a.n_splits));
+    const int split = __builtin_amdgcn_readfirstlane((int)(wid % a.n_splits));
+    const bool active = group < a.n_groups;  // a wavefront past the last group only helps to build the tables
     const int t_begin = split * a.tiles_per_split;
     const int t_end = min(t_begin + a.tiles_per_split, a.n_tiles);
     const int b4 = lane & ~3;  // 4 * block index
@@ -196,9 +220,9 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
     // The wavefront first rotates its group's four queries itself (four 128-point butterflies,
     // two values per lane), scales them and parks them as fp16 in 1 KB of LDS.
-    half4_t qa[2];
-    {
-        _Float16 *qw = q_s[tid >> 6];
+    half4_t qa[2] = {};
+    if (active) {
+        _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + (tid >> 6) * 512;
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int64_t e = ((int64_t)group * 4 + h) * 128 + 2 * lane;
@@ -233,6 +257,11 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         qa[0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
         qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
+    __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
+    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, tid);
+    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, tid);
+    __syncthreads();
+    if (!active) return;
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[2][2];
 #pragma unroll
@@ -242,8 +271,8 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
 
     const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
     const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
-    const char *klut_b = reinterpret_cast<const char *>(klut_s);
-    const char *vlut_b = reinterpret_cast<const char *>(vlut_s);
+    const char *klut_b = klut_s;
+    const char *vlut_b = vlut_s;
 
     // Rows are fetched one tile ahead into the same registers: the next K row right after QK has
     // consumed the current one, the next V row right after PV (dense mode).  The index is clamped
@@ -271,11 +300,12 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         const int row_n = (tile_n & 1) * 64 + lane;
         const uint2 gvu = *reinterpret_cast<const uint2 *>(vb + TQ_ROWS_PER_BLOCK * 16 * VBITS + 2 * tok_in_block);
         float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-        const int64_t tok0 = (int64_t)tile * 64 + b4;
+        const int tok0 = tile * 64 + b4;                 // the launcher checks tokens < 2^31
+        const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
         if (a.bias) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (tok0 + i < a.tokens) bias4[i] = a.bias[((int64_t)group * 4 + j) * a.tokens + tok0 + i] * LOG2E;
+                if (b4 + i < n_valid) bias4[i] = a.bias[((int64_t)group * 4 + j) * a.tokens + tok0 + i] * LOG2E;
         }
 
         // ---- QK ------------------------------------------------------------------
@@ -313,15 +343,18 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         float s[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) s[i] = sc[i] + bias4[i];
+        if (n_valid < 64) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (tok0 + i >= a.tokens) s[i] = -INFINITY;
+            for (int i = 0; i < 4; ++i)
+                if (b4 + i >= n_valid) s[i] = -INFINITY;
+        }
 
         // ---- online softmax (base 2) ------------------------------------------------
         const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
         const float m_new = fmaxf(m_run, mx);
         {
-            const float corr = exp2f(m_run - m_new);  // 0 on the first tile, 1 when the maximum stays
+            // 0 on the first tile, 1 when the maximum stays (also while every position so far is masked with -inf)
+            const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= corr;
             // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
             const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
@@ -335,13 +368,14 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
             m_run = m_new;
         }
         float p[4];
+        const float m_ref = m_run == -INFINITY ? 0.0f : m_run;  // all masked so far: weights are exp2(-inf) = 0, not NaN
         bool any_keep = false;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            p[i] = exp2f(s[i] - m_run);
+            p[i] = __builtin_amdgcn_exp2f(s[i] - m_ref);  // results below 2^-126 flush to zero
             l_run += p[i];
             if constexpr (SPARSE) {
-                const bool in_range = tok0 + i < a.tokens;
+                const bool in_range = b4 + i < n_valid;
                 const bool keep = p[i] >= a.tau;
                 if (in_range && !keep) ++nskip;
                 if (!keep) p[i] = 0.0f;
@@ -360,8 +394,8 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
         pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
         pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
-        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; pairs 4T + hf and
-        // 4T + 2 + hf = tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
+        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; quad 2T + hf =
+        // tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
         // weights of token group T sit in block T and are broadcast to every block.
         pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
         if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
@@ -503,10 +537,16 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.v = (const uint8_t *)v;
     a.klut = turbo_k ? (const uint32_t *)hk->pair_lut : nullptr;
     a.vlut = (const uint32_t *)hv->pair_lut;
+    const bool share = turbo_k && hk->bits == hv->bits &&
+                       std::memcmp(hk->pair_lut_host, hv->pair_lut_host, sizeof(hk->pair_lut_host)) == 0;
     a.bias = bias;
     a.part_o = part_o;
     a.part_ml = part_ml;
     a.skip = skip_count;
+    if (p->tokens >= ((int64_t)1 << 31)) {
+        tq_set_error("tq_decode_attention: tokens %lld beyond 2^31 - 1", (long long)p->tokens);
+        return TQ_ERR_UNSUPPORTED;
+    }
     a.tokens = p->tokens;
     a.blocks_per_seq = ((p->capacity > 0 ? p->capacity : p->tokens) + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
     a.n_groups = groups;
@@ -522,12 +562,19 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     const unsigned grid = (unsigned)(((int64_t)groups * p->n_splits + 3) / 4);
     const int vb = hv->bits;
     const int kb = turbo_k ? hk->bits : 8;
-#define TQ_ATTN(KF, KB, VB)                                                \
-    if (sparse) k_decode_attn<KF, KB, VB, true><<<grid, 256, 0, s>>>(a);  \
-    else k_decode_attn<KF, KB, VB, false><<<grid, 256, 0, s>>>(a)
-    if (turbo_k && kb == 3 && vb == 3) { TQ_ATTN(KFMT_TURBO, 3, 3); }
-    else if (turbo_k && kb == 4 && vb == 4) { TQ_ATTN(KFMT_TURBO, 4, 4); }
-    else if (turbo_k && kb == 2 && vb == 2) { TQ_ATTN(KFMT_TURBO, 2, 2); }
+#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, 256, 0, s>>>(a)
+#define TQ_ATTN(KF, KB, VB)                         \
+    if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
+    else TQ_ATTN_ONE(KF, KB, VB, false, false)
+    // same width and same centroids: one table
+#define TQ_ATTN_SAME(B)                                         \
+    if (share && sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, true);   \
+    else if (share) TQ_ATTN_ONE(KFMT_TURBO, B, B, false, true);       \
+    else if (sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, false);      \
+    else TQ_ATTN_ONE(KFMT_TURBO, B, B, false, false)
+    if (turbo_k && kb == 3 && vb == 3) { TQ_ATTN_SAME(3); }
+    else if (turbo_k && kb == 4 && vb == 4) { TQ_ATTN_SAME(4); }
+    else if (turbo_k && kb == 2 && vb == 2) { TQ_ATTN_SAME(2); }
     else if (turbo_k && kb == 4 && vb == 2) { TQ_ATTN(KFMT_TURBO, 4, 2); }
     else if (turbo_k && kb == 3 && vb == 2) { TQ_ATTN(KFMT_TURBO, 3, 2); }
     else if (!turbo_k && vb == 2) { TQ_ATTN(KFMT_Q8, 3, 2); }
@@ -538,6 +585,8 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         return TQ_ERR_UNSUPPORTED;
     }
 #undef TQ_ATTN
+#undef TQ_ATTN_SAME
+#undef TQ_ATTN_ONE
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
     k_attn_combine<<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);

@@ -165,6 +165,8 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         uint32_t *dl = nullptr;
         rc = rc ? rc : upload(&dl, lut);
         h->pair_lut = dl;
+        std::memset(h->pair_lut_host, 0, sizeof(h->pair_lut_host));
+        std::memcpy(h->pair_lut_host, lut.data(), lut.size() * sizeof(uint32_t));
         // factored transform for K rows: fragment f0*4+ks, row 4c+i, column 8kb+e
         {
             std::vector<uint16_t> rk((size_t)8 * 64 * 8);
@@ -197,8 +199,7 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                     if (s2[32 * c + v] < 0) continue;
                     if (b == 4) fl[c * 4 + v / 8] |= 1u << (4 * (v % 8) + 3);
                     else if (b == 2) fl[c * 4 + v / 16] |= 1u << (2 * (v % 16) + 1);
-                    else if (b == 3 && v < 30) fl[c * 4 + v / 10] |= 1u << (3 * (v % 10) + 2);
-                    else if (b == 3) fl[c * 4 + 3] |= 1u << (3 * (v - 30) + 2);
+                    else if (b == 3) fl[c * 4 + v / 8] |= 1u << (3 * (v % 8) + 2);  // entry 3: the tail word
                 }
             rc = rc ? rc : upload(&h->s2flip, fl);
         }

@@ -117,39 +117,55 @@ __device__ inline void wht128_wave(float &a, float &b, int lane) {
 // Inside a group, pair k sits in
 //   BITS 4: byte k%4 of dword k/4
 //   BITS 2: nibble k%8 of dword k/8
-//   BITS 3: bits 6*(k%5).. of dword k/5 for k < 15; pair 15 = bits 30..31 of dwords
-//           0, 1, 2 (low, middle, high two bits)
+//   BITS 3: bits 6*(k%4).. of dword k/4 for k < 12; pairs 12..15 form a 24-bit tail
+//           (pair k at tail bit 6*(k-12)) whose byte j is the top byte of dword j
+// Pairs 2q, 2q+1 ("quad" q, four values) are contiguous bits in every width, so a
+// reader can index a table by a whole quad with one field extract.
 // A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
 // norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows are dim-major
 // inside each 64-token tile: row (token & 64) | (dim & 63) holds dims r and 64+r
-// of the tile's tokens; pair 2*tp + (dim >> 6) = tokens 2tp, 2tp+1 of the tile.
+// of the tile's tokens; with tp = (token & 63) / 2 and hf = dim >> 6, tokens 2tp,
+// 2tp+1 are pair 4*(tp/2) + 2*hf + tp%2, so a quad is four consecutive tokens of
+// one dim.
 __host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
 __host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
 __host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
 
-// pairs per dword and bits per pair
-__host__ __device__ constexpr int pairs_per_dword(int bits) { return bits == 4 ? 4 : bits == 2 ? 8 : 5; }
-// row dword and bit position of pair p (for BITS 3 not the tail pair, p % 16 == 15)
+// pairs per dword (BITS 3: of the 12 pairs outside the tail)
+__host__ __device__ constexpr int pairs_per_dword(int bits) { return bits == 2 ? 8 : 4; }
+// true for the four pairs of a 3-bit group that live in the split tail
+__host__ __device__ constexpr bool pair_in_tail(int bits, int p) { return bits == 3 && (p & 15) >= 12; }
+// row dword and bit position of pair p (not for tail pairs)
 __host__ __device__ constexpr int pair_dword(int bits, int p) { return 4 * ((p & 15) / pairs_per_dword(bits)) + (p >> 4); }
 __host__ __device__ constexpr int pair_shift(int bits, int p) { return 2 * bits * ((p & 15) % pairs_per_dword(bits)); }
 
+// 24-bit tail (pairs 12..15) of group g of a 3-bit row
+__device__ __forceinline__ uint32_t tail24(const uint32_t *w, int g) {
+    return (w[g] >> 24) | ((w[4 + g] >> 24) << 8) | ((w[8 + g] >> 24) << 16);
+}
+
+// field `width` bits wide at bit `sh` of x, scaled by 2^SCALE (a table byte offset)
+template <int SCALE> __device__ __forceinline__ uint32_t field_offset(uint32_t x, int sh, int width) {
+    const uint32_t mask = ((1u << width) - 1u) << SCALE;
+    return sh >= SCALE ? ((x >> (sh - SCALE)) & mask) : ((x << (SCALE - sh)) & mask);
+}
+
 // byte offset (pair code * 4) into a 4-byte-entry LUT; p must fold to a constant
 template <int BITS> __device__ __forceinline__ uint32_t pair_lut_offset(const uint32_t (&w)[4 * BITS], int p) {
-    constexpr uint32_t MASK = ((1u << (2 * BITS)) - 1u) << 2;
-    if (BITS == 3 && (p & 15) == 15) {
-        const int g = p >> 4;
-        return ((w[g] >> 28) & 0xCu) | ((w[4 + g] >> 26) & 0x30u) | ((w[8 + g] >> 24) & 0xC0u);
-    }
-    const int q = pair_dword(BITS, p), sh = pair_shift(BITS, p);
-    return sh == 0 ? ((w[q] << 2) & MASK) : ((w[q] >> (sh - 2)) & MASK);
+    if (pair_in_tail(BITS, p)) return field_offset<2>(tail24(w, p >> 4), 6 * ((p & 15) - 12), 6);
+    return field_offset<2>(w[pair_dword(BITS, p)], pair_shift(BITS, p), 2 * BITS);
+}
+
+// byte offset (quad code * 8) into an 8-byte-entry LUT of quad Q = pairs 2Q, 2Q+1;
+// Q must fold to a constant
+template <int BITS> __device__ __forceinline__ uint32_t quad_lut_offset(const uint32_t (&w)[4 * BITS], int Q) {
+    if (pair_in_tail(BITS, 2 * Q)) return field_offset<3>(tail24(w, Q >> 3), 12 * ((Q & 7) - 6), 12);
+    return field_offset<3>(w[pair_dword(BITS, 2 * Q)], pair_shift(BITS, 2 * Q), 4 * BITS);
 }
 
 // runtime pair extraction (slow path: unpack / load kernels)
 __device__ inline uint32_t pair_code(const uint32_t *w, int bits, int p) {
-    if (bits == 3 && (p & 15) == 15) {
-        const int g = p >> 4;
-        return (w[g] >> 30) | ((w[4 + g] >> 30) << 2) | ((w[8 + g] >> 30) << 4);
-    }
+    if (pair_in_tail(bits, p)) return (tail24(w, p >> 4) >> (6 * ((p & 15) - 12))) & 63u;
     return (w[pair_dword(bits, p)] >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
 }
 
@@ -161,7 +177,7 @@ __device__ inline void locate(int kind, int token, int dim, int &row, int &pair,
         half = dim & 1;
     } else {
         row = (token & 64) | (dim & 63);
-        pair = (token & 62) | (dim >> 6);
+        pair = ((token & 60) | ((dim >> 6) << 1)) | ((token >> 1) & 1);
         half = token & 1;
     }
 }

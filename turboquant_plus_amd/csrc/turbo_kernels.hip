@@ -94,8 +94,8 @@ template <int BITS> __device__ inline uint32_t pair_from_stage(const uint8_t *co
         lo = codes[row * CODE_STRIDE + 2 * p];
         hi = codes[row * CODE_STRIDE + 2 * p + 1];
     } else {
-        const int tok = (row & 64) + (p & 62);
-        const int dim = ((p & 1) << 6) | (row & 63);
+        const int tok = (row & 64) + ((p & 60) | ((p & 1) << 1));
+        const int dim = ((p & 2) << 5) | (row & 63);
         lo = codes[tok * CODE_STRIDE + dim];
         hi = codes[(tok + 1) * CODE_STRIDE + dim];
     }
@@ -115,8 +115,10 @@ __device__ inline void pack_block(const uint8_t *codes, const float *norms, uint
 #pragma unroll
         for (int t = 0; t < PER; ++t) word |= pair_from_stage<BITS>(codes, kind, r, 16 * g + PER * j + t) << (2 * BITS * t);
         if constexpr (BITS == 3) {
-            const uint32_t tail = pair_from_stage<3>(codes, kind, r, 16 * g + 15);
-            word |= ((tail >> (2 * j)) & 3u) << 30;
+            uint32_t tail = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) tail |= pair_from_stage<3>(codes, kind, r, 16 * g + 12 + t) << (6 * t);
+            word |= ((tail >> (8 * j)) & 0xFFu) << 24;
         }
         out[o] = word;
     }
@@ -167,24 +169,21 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 // The sign bit of the value itself is appended with one funnel shift (so the sign field of
 // the unfolded code is 1 for negative values).  t[0] is not used: the middle boundary is 0.
 
-// 3-bit: values y0..y4 in append order; t[1..3] magnitude boundaries
-__device__ __forceinline__ uint32_t append5_b3(uint32_t w, float y0, float y1, float y2, float y3, float y4, const float (&t)[4]) {
-    float u0, u1, u2, u3, u4;
+// 3-bit: values y0..y3 in append order; t[1..3] magnitude boundaries
+__device__ __forceinline__ uint32_t append4_b3(uint32_t w, float y0, float y1, float y2, float y3, const float (&t)[4]) {
+    float u0, u1, u2, u3;
     asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
         "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
         "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t2]\n\t"
         "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t2]\n\t"
-        "v_cmp_gt_f32_e64 s[68:69], |%[y4]|, %[t2]\n\t"
         "v_cndmask_b32_e64 %[u0], %[t1], %[t3], s[60:61]\n\t"
         "v_cndmask_b32_e64 %[u1], %[t1], %[t3], s[62:63]\n\t"
         "v_cndmask_b32_e64 %[u2], %[t1], %[t3], s[64:65]\n\t"
         "v_cndmask_b32_e64 %[u3], %[t1], %[t3], s[66:67]\n\t"
-        "v_cndmask_b32_e64 %[u4], %[t1], %[t3], s[68:69]\n\t"
         "v_cmp_gt_f32_e64 s[70:71], |%[y0]|, %[u0]\n\t"
         "v_cmp_gt_f32_e64 s[72:73], |%[y1]|, %[u1]\n\t"
         "v_cmp_gt_f32_e64 s[74:75], |%[y2]|, %[u2]\n\t"
         "v_cmp_gt_f32_e64 s[76:77], |%[y3]|, %[u3]\n\t"
-        "v_cmp_gt_f32_e64 s[78:79], |%[y4]|, %[u4]\n\t"
         "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
         "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
         "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[70:71]\n\t"
@@ -197,32 +196,9 @@ __device__ __forceinline__ uint32_t append5_b3(uint32_t w, float y0, float y1, f
         "v_alignbit_b32 %[w], %[w], %[y3], 31\n\t"
         "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[66:67]\n\t"
         "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[76:77]\n\t"
-        "v_alignbit_b32 %[w], %[w], %[y4], 31\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[68:69]\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[78:79]\n\t"
-        : [w] "+v"(w), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3), [u4] "=&v"(u4)
-        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [y4] "v"(y4), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
-        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "vcc");
-    return w;
-}
-
-__device__ __forceinline__ uint32_t append2_b3(uint32_t w, float y0, float y1, const float (&t)[4]) {
-    float u0, u1;
-    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
-        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
-        "v_alignbit_b32 %[w], %[w], %[y0], 31\n\t"
-        "v_cndmask_b32_e64 %[u0], %[t1], %[t3], s[60:61]\n\t"
-        "v_cndmask_b32_e64 %[u1], %[t1], %[t3], s[62:63]\n\t"
-        "v_cmp_gt_f32_e64 s[70:71], |%[y0]|, %[u0]\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[60:61]\n\t"
-        "v_cmp_gt_f32_e64 s[72:73], |%[y1]|, %[u1]\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[70:71]\n\t"
-        "v_alignbit_b32 %[w], %[w], %[y1], 31\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[62:63]\n\t"
-        "v_addc_co_u32_e64 %[w], vcc, %[w], %[w], s[72:73]\n\t"
-        : [w] "+v"(w), [u0] "=&v"(u0), [u1] "=&v"(u1)
-        : [y0] "v"(y0), [y1] "v"(y1), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
-        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "vcc");
+        : [w] "+v"(w), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "vcc");
     return w;
 }
 
@@ -305,7 +281,7 @@ template <int BITS> __device__ __forceinline__ void count_levels(uint32_t w, uin
     if constexpr (BITS == 2) {
         n[1] += __builtin_popcount(w & 0x55555555u);
     } else if constexpr (BITS == 3) {
-        constexpr uint32_t K0 = 0x09249249u;  // bit 0 of the ten 3-bit fields
+        constexpr uint32_t K0 = 0x00249249u;  // bit 0 of the eight 3-bit fields
         const uint32_t b0 = w & K0, b1 = (w >> 1) & K0;
         n[1] += __builtin_popcount(b0);
         n[2] += __builtin_popcount(b1);
@@ -329,7 +305,7 @@ template <int BITS> __device__ __forceinline__ uint32_t fold_codes(uint32_t w) {
     if constexpr (BITS == 2) {
         return w ^ ((~w & 0xAAAAAAAAu) >> 1);
     } else if constexpr (BITS == 3) {
-        const uint32_t np = ~w & 0x24924924u;  // sign bits of the ten fields
+        const uint32_t np = ~w & 0x00924924u;  // sign bits of the eight fields
         return w ^ (np - (np >> 2));
     } else {
         const uint32_t np = ~w & 0x88888888u;
@@ -340,7 +316,7 @@ template <int BITS> __device__ __forceinline__ uint32_t fold_codes(uint32_t w) {
 struct StoreKArgs {
     const uint4 *afrag;      // [8 fragments f0*4+ks][64 lanes] 8 halves (+-1)
     const uint32_t *s2flip;  // [4 lane quarters][4]: sign-field positions of the dims with s2 = +1, per output dword
-                             // (3-bit: entry 3 is for the tail pair word): appended sign bit ^ this = "positive"
+                             // (3-bit: entry 3 is for the tail word): appended sign bit ^ this = "positive"
     const float *symthr;     // [0] middle boundary, [1..] positive boundaries
     const float *sqcoef;     // multilinear coefficients of c^2 over the level bits
     int norm_correction;
@@ -479,17 +455,19 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #pragma unroll
             for (int k = 0; k < NT; ++k) n[k] = 0;
             if constexpr (BITS == 3) {
-                uint32_t tw = append2_b3(0u, val(31), val(30), thr);  // pair 15 = values 30 (low code), 31 (high code)
-                count_levels<3>(tw, n);
-                tw = fold_codes<3>(nonzero ? tw ^ flip[3] : (zero_word & 0x24u));
+                // four words of eight values: dwords 0..2 and the tail, whose byte j rides on top of dword j
+                uint32_t w4[4];
 #pragma unroll
-                for (int j = 0; j < 3; ++j) {
-                    const int v = 10 * j;
-                    uint32_t w = append5_b3(0u, val(v + 9), val(v + 8), val(v + 7), val(v + 6), val(v + 5), thr);
-                    w = append5_b3(w, val(v + 4), val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+                for (int j = 3; j >= 0; --j) {
+                    const int v = 8 * j;
+                    uint32_t w = append4_b3(0u, val(v + 7), val(v + 6), val(v + 5), val(v + 4), thr);
+                    w = append4_b3(w, val(v + 3), val(v + 2), val(v + 1), val(v), thr);
                     count_levels<3>(w, n);
-                    g[j] = fold_codes<3>(nonzero ? w ^ flip[j] : (zero_word & 0x24924924u)) | (((tw >> (2 * j)) & 3u) << 30);
+                    w4[j] = fold_codes<3>(nonzero ? w ^ flip[j] : (zero_word & 0x00924924u));
                 }
+                g[0] = __builtin_amdgcn_perm(w4[3], w4[0], 0x04020100u);
+                g[1] = __builtin_amdgcn_perm(w4[3], w4[1], 0x05020100u);
+                g[2] = __builtin_amdgcn_perm(w4[3], w4[2], 0x06020100u);
             } else if constexpr (BITS == 4) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -667,17 +645,17 @@ __device__ __forceinline__ void append_rows_b4(uint32_t &w0, uint32_t &w1, uint3
         : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "vcc");
 }
 
-// pair k = 0..15 of a 16-pair group -> dword inside the group (3-bit: 3 = the word of the tail pair) and shift
-__host__ __device__ constexpr int grp_word(int bits, int k) { return bits == 3 && k == 15 ? 3 : k / pairs_per_dword(bits); }
-__host__ __device__ constexpr int grp_shift(int bits, int k) { return bits == 3 && k == 15 ? 0 : 2 * bits * (k % pairs_per_dword(bits)); }
-// V rows: sign-field bits of group dword j that belong to dim half hf (pairs with k % 2 == hf) and to the tokens
-// of the 16-token group named by tokmask (pair k = tokens 2(k/2), 2(k/2)+1 as low and high code)
+// pair k = 0..15 of a 16-pair group -> dword inside the group (3-bit: 3 = the tail word) and shift
+__host__ __device__ constexpr int grp_word(int bits, int k) { return k / pairs_per_dword(bits); }
+__host__ __device__ constexpr int grp_shift(int bits, int k) { return 2 * bits * (k % pairs_per_dword(bits)); }
+// V rows: sign-field bits of group dword j that belong to dim half hf (pairs with (k / 2) % 2 == hf) and to the
+// tokens of the 16-token group named by tokmask (pair k = tokens 4(k/4) + 2(k%2), +1 as low and high code)
 __host__ __device__ constexpr uint32_t v_sign_mask(int bits, int j, int hf, uint32_t tokmask) {
     uint32_t m = 0;
     for (int k = 0; k < 16; ++k) {
-        if ((k & 1) != hf || grp_word(bits, k) != j) continue;
+        if (((k >> 1) & 1) != hf || grp_word(bits, k) != j) continue;
         for (int h = 0; h < 2; ++h)
-            if ((tokmask >> (2 * (k >> 1) + h)) & 1) m |= 1u << (grp_shift(bits, k) + bits * h + bits - 1);
+            if ((tokmask >> (4 * (k >> 2) + 2 * (k & 1) + h)) & 1) m |= 1u << (grp_shift(bits, k) + bits * h + bits - 1);
     }
     return m;
 }
@@ -697,7 +675,7 @@ template <int BITS, bool RAGGED>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter) {
     constexpr int NT = 1 << (BITS - 1);
-    constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail pair word)
+    constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kq = lane >> 4;
     float thr0[NT], coef[NT];
@@ -807,11 +785,11 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 y[3][d0] = (d01 - d23) * inv;
             }
             uint32_t n1[4] = {0, 0, 0, 0}, n2[4] = {0, 0, 0, 0}, n3[4] = {0, 0, 0, 0};
-            // groups in descending pair order: pair 4u + 2(i/2) + hf, high code (odd i) first
+            // groups in descending pair order: pair 4u + 2hf + i/2, high code (odd i) first
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
-                const int i = (g & 4 ? 0 : 2) + (g & 1 ? 0 : 1), hf = g & 2 ? 0 : 1;
-                const int j = grp_word(BITS, 4 * u + 2 * (i >> 1) + hf);
+                const int i = 3 - (g & 3), hf = g & 4 ? 0 : 1;
+                const int j = grp_word(BITS, 4 * u);
                 const float y0 = y[0 | (hf << 1)][0][i], y1 = y[0 | (hf << 1)][1][i];
                 const float y2 = y[1 | (hf << 1)][0][i], y3 = y[1 | (hf << 1)][1][i];
                 if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], n2[i], n3[i], y0, y1, y2, y3, thr0);
@@ -833,9 +811,9 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 }
 #pragma unroll
                 for (int p = 1; p < 8; ++p) {
-                    // token i sits at nibbles 4(i/2) + i%2 (hf 0) and two nibbles higher (hf 1)
-                    const uint32_t t = sum[p] + (sum[p] >> 8);
-                    cnt[p] = (t & 0x000F000Fu) | ((t & 0x00F000F0u) << 4);
+                    // token i sits at nibble i (hf 0) and nibble 4 + i (hf 1); bytes of cnt: tokens 0, 2, 1, 3
+                    const uint32_t t = sum[p] + (sum[p] >> 16);
+                    cnt[p] = (t & 0x0F0Fu) | ((t & 0xF0F0u) << 12);
                 }
             } else {
                 cnt[1] = n1[0] | (n1[1] << 8) | (n1[2] << 16) | (n1[3] << 24);
@@ -845,7 +823,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 }
             }
             float cs = 128.0f * coef[0];
-            const int sh = 8 * (n16 & 3);
+            const int sh = BITS == 4 ? 8 * (((n16 & 1) << 1) | ((n16 >> 1) & 1)) : 8 * (n16 & 3);
 #pragma unroll
             for (int p = 1; p < NT; ++p) cs = fmaf(coef[p], (float)((row16_sum(cnt[p]) >> sh) & 0xFFu), cs);
             const int isel = n16 & 3;
@@ -879,7 +857,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #pragma unroll
             for (int j = 0; j < BITS; ++j) {
                 uint32_t g = w[dd][j];
-                if constexpr (BITS == 3) g |= ((w[dd][3] >> (2 * j)) & 3u) << 30;
+                if constexpr (BITS == 3) g = __builtin_amdgcn_perm(w[dd][3], g, 0x04020100u + ((uint32_t)j << 24));
                 *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kq * 4) = g;
             }
         }
@@ -1184,10 +1162,11 @@ __device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, 
     int row, p, half;
     locate(kind, token, dim, row, p, half);
     uint32_t pc;
-    if (bits == 3 && (p & 15) == 15) {
+    if (pair_in_tail(bits, p)) {
         const int g = p >> 4;
-        pc = (row_dword(block, row, g) >> 30) | ((row_dword(block, row, 4 + g) >> 30) << 2) |
-             ((row_dword(block, row, 8 + g) >> 30) << 4);
+        const uint32_t tail = (row_dword(block, row, g) >> 24) | ((row_dword(block, row, 4 + g) >> 24) << 8) |
+                              ((row_dword(block, row, 8 + g) >> 24) << 16);
+        pc = (tail >> (6 * ((p & 15) - 12))) & 63u;
     } else {
         pc = (row_dword(block, row, pair_dword(bits, p)) >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
     }
