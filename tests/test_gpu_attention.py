@@ -156,6 +156,34 @@ def test_decode_attention_masked_prefix():
     assert_close(out, ref)
 
 
+def test_decode_attention_many_groups_and_repeated_calls():
+    """Thousands of GQA groups with a short context against the oracle (spot-checked groups), and the same call
+    repeated many times on one workspace with identical results."""
+    B, Hq, Hkv, N = 4100, 4, 1, 128
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=93)
+    q = np.random.default_rng(94).standard_normal((B, Hq, D)).astype(np.float16)
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=2)(q, kp, vp))
+    sel = [0, 1, 2047, 4095, 4096, 4099]
+    ki, kg = kc.unpack_codes(kp, B, N, kind="k")
+    vi, vg = vc.unpack_codes(vp, B, N, kind="v")
+    k_rot = O.turbo_decode_rotated(np_(ki)[sel], np_(kg)[sel].astype(np.float64), kc.centroids)
+    v_rot = O.turbo_decode_rotated(np_(vi)[sel], np_(vg)[sel].astype(np.float64), vc.centroids)
+    q_rot = O.rotate_fast(q[sel].astype(np.float64), kc.signs1, kc.signs2, D)
+    for n, b in enumerate(sel):
+        o, _, _ = O.decode_attention(q_rot[n], k_rot[n], v_rot[n], 1 / np.sqrt(D))
+        assert_close(out[b], O.rotate_fast(o, vc.signs1, vc.signs2, D, transpose=True))
+    B, Hq, Hkv, N = 2, 8, 2, 1000
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=95)
+    q = np.random.default_rng(96).standard_normal((B, Hq, D)).astype(np.float16)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=5)
+    first = np_(attn(q, kp, vp)).copy()
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D))
+    assert_close(first, ref)
+    for _ in range(20):
+        again = np_(attn(q, kp, vp))
+        assert np.array_equal(again, first)
+
+
 def test_decode_attention_q8_0_k_turbo2_v():
     """BASELINE config 4 shape family: K q8_0-style (not rotated), V turbo2."""
     B, Hq, Hkv, N = 1, 8, 2, 2048 + 64

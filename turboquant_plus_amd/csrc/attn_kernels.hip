@@ -62,25 +62,30 @@ template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_
 }
 
 // build a codebook's decode table in LDS from its pair table (half2 per pair code) in global memory
-// (256 threads); every global load is issued before the first LDS write
-template <int BITS> __device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, int tid) {
+// with n_waves wavefronts; the global load is issued before the first LDS write
+template <int BITS> __device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, int tid, int n_waves) {
     constexpr int NP = 1 << (2 * BITS);
     if constexpr (BITS == 3) {
-        // lane l holds pair entry l; wavefront w writes the rows hi = w, w + 4, ..
+        // lane l holds pair entry l; wavefront w writes the rows hi = w, w + n_waves, ..
         uint2 *t = reinterpret_cast<uint2 *>(dst);
         const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t mine = pair_lut[lane];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int hi = wave + 4 * i;
+        for (int hi = wave; hi < 64; hi += n_waves)
             t[hi * 64 + lane] = make_uint2(mine, (uint32_t)__builtin_amdgcn_readlane((int)mine, hi));
-        }
     } else if constexpr (BITS == 2) {
-        reinterpret_cast<uint2 *>(dst)[tid] = make_uint2(pair_lut[tid & 15], pair_lut[tid >> 4]);
+        for (int e = tid; e < 256; e += 64 * n_waves)
+            reinterpret_cast<uint2 *>(dst)[e] = make_uint2(pair_lut[e & 15], pair_lut[e >> 4]);
     } else {
         static_assert(NP == 256, "pair table of 256 entries");
-        reinterpret_cast<uint32_t *>(dst)[tid] = pair_lut[tid];
+        for (int e = tid; e < 256; e += 64 * n_waves) reinterpret_cast<uint32_t *>(dst)[e] = pair_lut[e];
     }
+}
+
+// raise a progress mark in LDS to `mine` and return what it held before (one atomic per wavefront)
+__device__ __forceinline__ uint32_t lead_progress(uint32_t *mark, uint32_t mine, int lane) {
+    uint32_t t = 0;
+    if (lane == 0) t = atomicMax(mark, mine);
+    return __builtin_amdgcn_readfirstlane(t);
 }
 
 template <int BITS> __device__ __forceinline__ void load_row(const uint8_t *block, int row, uint32_t (&w)[4 * BITS]) {
@@ -187,8 +192,16 @@ __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const u
 
 // SHARE: K and V decode through one table (same width, same centroids); table positions are
 // compile-time constants so that they fold into the LDS instructions' offset fields.
+//
+// Work distribution: a workgroup of W wavefronts (W = blockDim / 64 divides n_splits) owns W
+// consecutive splits of one group, one split per wavefront (a fixed share, so results do not
+// depend on timing).  The hardware favours the oldest wavefronts of a SIMD, and left alone
+// the youngest finish late and alone on a memory system that needs every wavefront's loads
+// in flight to stay busy.  So the wavefronts of a workgroup publish their progress in LDS and
+// each sets its own issue priority to how many tiles it is behind the leader (at most 3):
+// they finish within a tile or two of each other.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE>
-__global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
     constexpr int VBLOCK = TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
@@ -196,72 +209,109 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     static_assert(!SHARE || (KFMT == KFMT_TURBO && KBITS == VBITS), "a shared table needs equal code widths");
     // static LDS (its address is a compile-time constant, so table positions fold into the LDS
     // instructions): [K table][V table unless shared with K].  Before the tables are built the
-    // first 4 KB stage the rotated queries, 1 KB per wavefront.
+    // first 1 KB stages the group's four rotated queries.
     constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
-    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 4096 ? LUT_TOTAL : 4096];
+    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 1024 ? LUT_TOTAL : 1024];
+    __shared__ uint32_t lead;  // tiles finished by the wavefront that is furthest ahead
     char *klut_s = smem;
     char *vlut_s = SHARE ? klut_s : klut_s + KLUT_BYTES;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int64_t wid = (int64_t)blockIdx.x * 4 + (tid >> 6);
-    // wave-uniform values in scalar registers: tile loop, block addresses and bounds become scalar work
-    const int group = __builtin_amdgcn_readfirstlane((int)(wid / a.n_splits));
-    const int split = __builtin_amdgcn_readfirstlane((int)(wid % a.n_splits));
-    const bool active = group < a.n_groups;  // a wavefront past the last group only helps to build the tables
+    // workgroup-uniform values in scalar registers: tile loop, block addresses and bounds become scalar work
+    const int n_waves = (int)(blockDim.x >> 6), wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wgs_per_group = a.n_splits / n_waves;
+    const int group = (int)(blockIdx.x / wgs_per_group), part = (int)(blockIdx.x % wgs_per_group);
+    const int split = part * n_waves + wave;  // index of this wavefront's partial
     const int t_begin = split * a.tiles_per_split;
     const int t_end = min(t_begin + a.tiles_per_split, a.n_tiles);
     const int b4 = lane & ~3;  // 4 * block index
     const int j = lane & 3;    // query head of the logits this lane holds; sub-row for V
+
+    const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
+    const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
+    const char *klut_b = klut_s;
+    const char *vlut_b = vlut_s;
+
+    // The first tile's rows are requested before anything else, so that the query rotation and
+    // the table build overlap the first trip to memory.  Afterwards rows are fetched one tile
+    // ahead into the same registers: the next K row right after QK has consumed the current
+    // one, the next V row right after PV (dense mode).  The index is clamped at the split's
+    // last tile, so the final prefetch re-reads a row instead of branching.  The norms
+    // travel with the rows, so no load is waited for in the tile that issued it.
+    uint32_t kw[KROW_DW];
+    uint32_t vw[4 * VBITS];
+    // K: this lane's token's fp16 norm (turbo) or its four fp16 block scales (q8_0-style)
+    auto load_knorm = [&](int tile) -> uint2 {
+        const uint8_t *kb = kbase + (int64_t)(tile >> 1) * KBLOCK;
+        const int r = (tile & 1) * 64 + lane;
+        if constexpr (KFMT == KFMT_TURBO)
+            return make_uint2(reinterpret_cast<const uint16_t *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS)[r], 0u);
+        else
+            return *reinterpret_cast<const uint2 *>(kb + 8 * 2048 + 8 * r);
+    };
+    // V: fp16 norms of this lane's four tokens 4b..4b+3
+    auto load_vnorm = [&](int tile) -> uint2 {
+        return *reinterpret_cast<const uint2 *>(vbase + (int64_t)(tile >> 1) * VBLOCK + TQ_ROWS_PER_BLOCK * 16 * VBITS +
+                                                2 * ((tile & 1) * 64 + b4));
+    };
+    uint2 kn = make_uint2(0u, 0u), gvu = make_uint2(0u, 0u);
+    int tile = t_begin;
+    if (tile < t_end) {
+        const int row0 = (tile & 1) * 64 + lane;
+        const uint8_t *kb = kbase + (int64_t)(tile >> 1) * KBLOCK;
+        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row0, kw);
+        else load_row<8>(kb, row0, kw);
+        kn = load_knorm(tile);
+        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile >> 1) * VBLOCK, row0, vw);
+        gvu = load_vnorm(tile);
+    }
+    if (tid == 0) lead = 0;
 
     float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
     float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
 
     // A operand of QK, broadcast from one block per MFMA: lane (b, i) keeps q[head i] for the
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
-    // The wavefront first rotates its group's four queries itself (four 128-point butterflies,
-    // two values per lane), scales them and parks them as fp16 in 1 KB of LDS.
-    half4_t qa[2] = {};
-    if (active) {
-        _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + (tid >> 6) * 512;
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-            const int64_t e = ((int64_t)group * 4 + h) * 128 + 2 * lane;
-            float x0, x1;
-            if (a.q_dtype == TQ_F16) {
-                const __half *qp = reinterpret_cast<const __half *>(a.q);
-                x0 = __half2float(qp[e]);
-                x1 = __half2float(qp[e + 1]);
-            } else if (a.q_dtype == TQ_F32) {
-                const float *qp = reinterpret_cast<const float *>(a.q);
-                x0 = qp[e];
-                x1 = qp[e + 1];
-            } else {
-                const double *qp = reinterpret_cast<const double *>(a.q);
-                x0 = (float)qp[e];
-                x1 = (float)qp[e + 1];
-            }
-            if (a.ks1) {
-                x0 *= a.ks1[2 * lane];
-                x1 *= a.ks1[2 * lane + 1];
-                wht128_wave(x0, x1, lane);
-                x0 *= a.ks2[2 * lane] * RSQRT128;
-                x1 *= a.ks2[2 * lane + 1] * RSQRT128;
-            }
-            qw[h * 128 + 2 * lane] = (_Float16)(x0 * a.scale_log2e);
-            qw[h * 128 + 2 * lane + 1] = (_Float16)(x1 * a.scale_log2e);
+    // The group's four queries are rotated by the first wavefronts (one 128-point butterfly per
+    // head, two values per lane), scaled and parked as fp16 in 1 KB of LDS for everybody.
+    for (int h = wave; h < 4; h += n_waves) {
+        _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + h * 128;
+        const int64_t e = ((int64_t)group * 4 + h) * 128 + 2 * lane;
+        float x0, x1;
+        if (a.q_dtype == TQ_F16) {
+            const __half *qp = reinterpret_cast<const __half *>(a.q);
+            x0 = __half2float(qp[e]);
+            x1 = __half2float(qp[e + 1]);
+        } else if (a.q_dtype == TQ_F32) {
+            const float *qp = reinterpret_cast<const float *>(a.q);
+            x0 = qp[e];
+            x1 = qp[e + 1];
+        } else {
+            const double *qp = reinterpret_cast<const double *>(a.q);
+            x0 = (float)qp[e];
+            x1 = (float)qp[e + 1];
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const uint2 *qp = reinterpret_cast<const uint2 *>(qw + j * 128);
+        if (a.ks1) {
+            x0 *= a.ks1[2 * lane];
+            x1 *= a.ks1[2 * lane + 1];
+            wht128_wave(x0, x1, lane);
+            x0 *= a.ks2[2 * lane] * RSQRT128;
+            x1 *= a.ks2[2 * lane + 1] * RSQRT128;
+        }
+        qw[2 * lane] = (_Float16)(x0 * a.scale_log2e);
+        qw[2 * lane + 1] = (_Float16)(x1 * a.scale_log2e);
+    }
+    __syncthreads();
+    half4_t qa[2];
+    {
+        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + j * 128);
         qa[0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
         qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
     __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
-    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, tid);
-    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, tid);
+    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, tid, n_waves);
+    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, tid, n_waves);
     __syncthreads();
-    if (!active) return;
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[2][2];
 #pragma unroll
@@ -269,36 +319,25 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
     float m_run = -INFINITY, l_run = 0.0f;
     unsigned nskip = 0;
 
-    const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
-    const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
-    const char *klut_b = klut_s;
-    const char *vlut_b = vlut_s;
-
-    // Rows are fetched one tile ahead into the same registers: the next K row right after QK has
-    // consumed the current one, the next V row right after PV (dense mode).  The index is clamped
-    // at the last tile, so the final prefetch re-reads a row instead of branching.
-    uint32_t kw[KROW_DW];
-    uint32_t vw[4 * VBITS];
-    if (t_begin < t_end) {
-        const int row0 = (t_begin & 1) * 64 + lane;
-        const uint8_t *kb = kbase + (int64_t)(t_begin >> 1) * KBLOCK;
-        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row0, kw);
-        else load_row<8>(kb, row0, kw);
-        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(t_begin >> 1) * VBLOCK, row0, vw);
-    }
-
 #pragma unroll 1
-    for (int tile = t_begin; tile < t_end; ++tile) {
+    while (tile < t_end) {
         const int64_t blk = tile >> 1;
         const int half = tile & 1;
         const int row = half * 64 + lane;
-        const int tok_in_block = half * 64 + b4;  // first of this lane's 4 tokens, inside the block
-        const uint8_t *kb = kbase + blk * KBLOCK;
         const uint8_t *vb = vbase + blk * VBLOCK;
 
-        const int tile_n = min(tile + 1, t_end - 1);
+        {   // issue priority = tiles behind the leader (wave-uniform, so the branches are scalar)
+            const uint32_t done = (uint32_t)(tile - t_begin);
+            const uint32_t behind = max(lead_progress(&lead, done, lane), done) - done;
+            if (behind == 0) __builtin_amdgcn_s_setprio(0);
+            else if (behind == 1) __builtin_amdgcn_s_setprio(1);
+            else if (behind == 2) __builtin_amdgcn_s_setprio(2);
+            else __builtin_amdgcn_s_setprio(3);
+        }
+        const int tile_next = tile + 1;
+        const int tile_n = min(tile_next, t_end - 1);
         const int row_n = (tile_n & 1) * 64 + lane;
-        const uint2 gvu = *reinterpret_cast<const uint2 *>(vb + TQ_ROWS_PER_BLOCK * 16 * VBITS + 2 * tok_in_block);
+        const uint2 gvu_next = load_vnorm(tile_n);
         float bias4[4] = {0.f, 0.f, 0.f, 0.f};
         const int tok0 = tile * 64 + b4;                 // the launcher checks tokens < 2^31
         const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
@@ -316,8 +355,7 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
             qk_turbo<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa, acc);
-            const float gk_own = __half2float(
-                reinterpret_cast<const __half *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS)[half * 64 + lane]);
+            const float gk_own = __half2float(__ushort_as_half((unsigned short)kn.x));
 #pragma unroll
             for (int i = 0; i < 4; ++i) sc[i] = ((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i])) * gk_own;
         } else {
@@ -325,7 +363,7 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
             qk_q8(std::make_integer_sequence<int, 32>{}, kw, qa, acc);
-            const uint2 su = *reinterpret_cast<const uint2 *>(kb + 8 * 2048 + 8 * (half * 64 + lane));
+            const uint2 su = kn;
             const float d0 = __half2float(__ushort_as_half((unsigned short)(su.x & 0xffff)));
             const float d1 = __half2float(__ushort_as_half((unsigned short)(su.x >> 16)));
             const float d2 = __half2float(__ushort_as_half((unsigned short)(su.y & 0xffff)));
@@ -337,6 +375,7 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
             const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
             if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, row_n, kw);
             else load_row<8>(kbn, row_n, kw);
+            kn = load_knorm(tile_n);
         }
         // -> lane (b, j): head j, tokens 4b..4b+3
         quad_transpose(sc, lane);
@@ -383,7 +422,11 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
             }
         }
         if constexpr (SPARSE) {
-            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) continue;  // every V row skipped: no V load, no dequant
+            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {  // every V row skipped: no V load, no dequant
+                gvu = gvu_next;
+                tile = tile_next;
+                continue;
+            }
             load_row<VBITS>(vb, row, vw);
         }
 
@@ -399,6 +442,8 @@ __global__ __launch_bounds__(256, 2) void k_decode_attn(AttnArgs a) {
         // weights of token group T sit in block T and are broadcast to every block.
         pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
         if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
+        gvu = gvu_next;
+        tile = tile_next;
     }
 
     // ---- end of split: write the partial ---------------------------------------------
@@ -559,10 +604,14 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: sparse_v_tau > 0 needs skip_count");
         return TQ_ERR_ARG;
     }
-    const unsigned grid = (unsigned)(((int64_t)groups * p->n_splits + 3) / 4);
+    // wavefronts per workgroup: the largest power of two up to 16 that divides the split count
+    int wpw = 16;
+    while (p->n_splits % wpw) wpw >>= 1;
+    const unsigned grid = (unsigned)((int64_t)groups * (p->n_splits / wpw));
+    const unsigned wg = 64u * (unsigned)wpw;
     const int vb = hv->bits;
     const int kb = turbo_k ? hk->bits : 8;
-#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, 256, 0, s>>>(a)
+#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, 0, s>>>(a)
 #define TQ_ATTN(KF, KB, VB)                         \
     if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
     else TQ_ATTN_ONE(KF, KB, VB, false, false)
