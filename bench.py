@@ -6,7 +6,7 @@
 A step is one pass of the hot path over one batch of synthetic input:
   * store leg (BASELINE config 2, the `value` of the JSON line): quantise+pack
     one Llama-3-8B-shaped layer, K and V fp16 [8, 32768, 128], 4 outlier
-    channels x15 in K, into the turbo4 block format (one launch per tensor);
+    channels x15 in K, into the turbo4 block format (K and V in one launch);
   * the same leg in turbo3 (the bit width the 70 % target is stated for);
   * decode leg (BASELINE config 3): fused decode attention over turbo3 K/V,
     batch 16, 32 query heads on 8 KV heads, context 32768.
@@ -14,6 +14,13 @@ Inputs are resident in HBM before the timed region; every step cycles through
 several distinct buffer sets so that the 256 MB Infinity Cache cannot serve
 the reads.  Kernel durations come from HIP events recorded on the stream the
 kernels are launched on (torch's current stream).
+
+The default warm-up is long on purpose (1000 steps, about 50-90 ms per leg):
+when a busy stretch starts after idle time the GPU's power management first
+drops the core clock from about 1.93 GHz to about 1.3 GHz and brings it back
+over the next 25-30 ms (read in-kernel from the cycle and wall-clock counters),
+and a 20-step warm-up times that transient (+15-20 % per step) instead of the
+sustained rate a serving loop sees.
 
 Prints ONE JSON line.  `roofline` prices the store kernel against 8 TB/s with
 the algorithmic bytes per launch (322 B per vector for turbo4: 256 B fp16 in,
@@ -185,7 +192,7 @@ def score_tile_leg(torch, tqa, steps, warmup):
         def step(i):
             nonlocal logits
             logits = codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt)
-        wall_ms, ev_ms = time_steps(torch, step, max(5, steps // 10), 2)
+        wall_ms, ev_ms = time_steps(torch, step, max(5, steps // 10), max(2, warmup // 10))
         out[name] = {"us_per_call": ev_ms * 1e3, "mfma_tflops": flops / (ev_ms * 1e-3) / 1e12,
                      "mfma_frac_of_2500": flops / (ev_ms * 1e-3) / 2.5e15,
                      "logit_store_gbs": logits.numel() * logits.element_size() / (ev_ms * 1e-3) / 1e9}
@@ -243,8 +250,8 @@ def cpu_baseline(bits):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (5x) so that FETCH_SIZE / WRITE_SIZE counters can be calibrated")
