@@ -200,7 +200,8 @@ typedef struct tq_attn_params {
     int64_t tokens;                        /* context length per sequence                    */
     int64_t capacity;                      /* tokens per sequence the K/V buffers are laid   */
                                            /* out for (tq_append caches); 0 = tokens         */
-    int32_t n_splits;                      /* context splits per (batch, kv head), >= 1      */
+    int32_t n_splits;                      /* context splits per (batch, kv head), >= 1; a   */
+                                           /* multiple of 16 lets 16 splits share a workgroup */
     int32_t k_format;                      /* TQ_KFMT_TURBO | TQ_KFMT_Q8_0                   */
     float scale;                           /* logit scale, e.g. 1/sqrt(128)                  */
     float sparse_v_tau;                    /* 0 = dense; skip V rows with weight < tau       */

@@ -25,7 +25,7 @@
 //   Online softmax in base 2 (log2(e) folded into the query scale).
 // k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
 //   the V rotation (one workgroup per query head).  Queries are rotated and scaled
-//   inside k_decode_attn by each wavefront, so a dense step is two launches.
+//   inside k_decode_attn, so a dense step is two launches.
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
 #include <cstring>
