@@ -229,7 +229,8 @@ int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_
  * moved to the rotated/projected domain): logits[i,j] = <R q_i, g_j c[idx_j]> +
  * projection_scale * rnorm_j * <S q_i, z_j>.  q [nq,128] q_dtype, packed/sign_bits/
  * rnorms from tq_store_qjl with n_seqs = 1, logits [nq, nk] fp32 (or fp16 when
- * out_dtype == TQ_F16).  workspace: nq*256*2 bytes. */
+ * out_dtype == TQ_F16).  workspace: 512 bytes per query, query count rounded up to a
+ * multiple of 32. */
 int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
                   const uint8_t *sign_bits, const void *rnorms_f16, int64_t nk, void *logits, int out_dtype,
                   void *workspace, int64_t workspace_bytes, void *stream);

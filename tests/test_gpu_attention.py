@@ -210,13 +210,13 @@ def test_decode_attention_rejects_unsupported_group():
         tqa.DecodeAttention(kc, vc, 1, 8, 1, 128)
 
 
-@pytest.mark.parametrize("projection", ["orthogonal", "gaussian"])
-def test_score_tile(projection):
+@pytest.mark.parametrize("projection,nk,nq", [("orthogonal", 1000, 200), ("gaussian", 1000, 200),
+                                              ("orthogonal", 333, 70), ("orthogonal", 2304, 513)])
+def test_score_tile(projection, nk, nq):
     """TurboQuant inner-product estimator (BASELINE config 5 family, reduced):
     GPU logits against the oracle's on the stored codes, and the estimator's
     bias against the exact inner products."""
     tt = L.torch()
-    nk, nq = 1000, 200
     rng = np.random.default_rng(12)
     keys = rng.standard_normal((nk, D)).astype(np.float32)
     qs = rng.standard_normal((nq, D)).astype(np.float16)

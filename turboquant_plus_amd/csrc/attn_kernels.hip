@@ -29,6 +29,7 @@
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
 #include <cstring>
+#include <type_traits>
 #include <utility>
 
 #include "tq_device.h"
@@ -646,6 +647,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 namespace {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int KT_STRIDE = 264;  // halves per staged key row (256 + 8: 16-byte reads of 16 rows hit 64 distinct banks)
 
 // [R q | S q] as fp16, one wavefront per query
@@ -675,51 +677,56 @@ __global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, i
     wht128_wave(x0, x1, lane);
     x0 *= s2[2 * lane] * RSQRT128;
     x1 *= s2[2 * lane + 1] * RSQRT128;
-    qa[v * 256 + 2 * lane] = __float2half_rn(x0);
-    qa[v * 256 + 2 * lane + 1] = __float2half_rn(x1);
-    qa[v * 256 + 128 + 2 * lane] = __float2half_rn(p0);
-    qa[v * 256 + 128 + 2 * lane + 1] = __float2half_rn(p1);
+    // operand-major layout: the 16-byte chunk (row r of query block v / 32, K values 16t + 8kb .. + 7) that
+    // lane r + 32kb of the score tile's MFMA reads in K step t sits at chunk index (block * 16 + t) * 64 + r + 32kb,
+    // so one wave-wide operand load is 1 KB of contiguous memory
+    __half2 *qa2 = reinterpret_cast<__half2 *>(qa);
+    const int64_t blk = v >> 5;
+    const int r = (int)(v & 31);
+    auto chunk_pair = [&](int k) {  // index of the half2 holding K values k, k + 1 (k even)
+        const int t = k >> 4, kb = (k >> 3) & 1, e = k & 7;
+        return (((blk * 16 + t) * 64 + r + 32 * kb) * 8 + e) >> 1;
+    };
+    qa2[chunk_pair(2 * lane)] = __halves2half2(__float2half_rn(x0), __float2half_rn(x1));
+    qa2[chunk_pair(128 + 2 * lane)] = __halves2half2(__float2half_rn(p0), __float2half_rn(p1));
 }
 
-template <typename T> __device__ inline void st_logit4(T *p, float4_t v, int n_ok);
-template <> __device__ inline void st_logit4<float>(float *p, float4_t v, int n_ok) {
-    if (n_ok >= 4 && ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)) {
-        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    } else {
-        for (int i = 0; i < 4 && i < n_ok; ++i) p[i] = v[i];
-    }
-}
-template <> __device__ inline void st_logit4<__half>(__half *p, float4_t v, int n_ok) {
-    for (int i = 0; i < 4 && i < n_ok; ++i) p[i] = __float2half_rn(v[i]);
-}
-
-// One workgroup per 128-key block: dequantise the block once into LDS as fp16
-// [g*c[idx] | scale*rnorm*z], then sweep all queries with 16x16x32 MFMA tiles
-// (keys on the M side so that each lane owns 4 consecutive keys of one query).
+// One workgroup of eight wavefronts per 256 keys: dequantise them once into LDS as fp16
+// [g*c[idx] | scale*rnorm*z], then sweep all queries with 32x32x16 MFMA tiles (queries on the M side,
+// keys on the N side).  A wavefront owns 64 queries of each 512-query tile: their operands (64 x 256
+// halves) live in registers, are used against the eight 32-key sub-blocks in turn, and are replaced,
+// step by step, with the next tile's while the last sub-block is being multiplied, so every query
+// operand crosses the vector memory path once per workgroup and a whole tile ahead of its use.
+constexpr int SCORE_KEYS = 256;  // keys per workgroup (two 128-row blocks)
 template <int BITS, typename TO>
-__global__ __launch_bounds__(256) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
-                                                   const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
-                                                   const float *cent, float proj_scale) {
-    extern __shared__ _Float16 kt[];  // [128][KT_STRIDE]
+__global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
+                                                      const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
+                                                      const float *cent, float proj_scale) {
+    extern __shared__ _Float16 kt[];  // [SCORE_KEYS][KT_STRIDE]
     __shared__ float cent_s[16];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int64_t key0 = (int64_t)blockIdx.x * 128;
-    const uint8_t *block = packed + (int64_t)blockIdx.x * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
+    const int64_t key0 = (int64_t)blockIdx.x * SCORE_KEYS;
     if (tid < (1 << BITS)) cent_s[tid] = cent[tid];
     __syncthreads();
     {
-        const int key = tid & 127, part = tid >> 7;
+        const int key = tid & (SCORE_KEYS - 1), part = tid >> 8;
         _Float16 *row = kt + key * KT_STRIDE;
         const bool valid = key0 + key < nk;
         if (part == 0) {
-            uint32_t wv[4 * BITS];
-            load_row<BITS>(block, key, wv);
-            const float g = valid ? __half2float(reinterpret_cast<const __half *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key]) : 0.f;
+            if (valid) {
+                const uint8_t *block = packed + (key0 + key) / TQ_ROWS_PER_BLOCK * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
+                uint32_t wv[4 * BITS];
+                load_row<BITS>(block, key & (TQ_ROWS_PER_BLOCK - 1), wv);
+                const float g = __half2float(reinterpret_cast<const __half *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key & (TQ_ROWS_PER_BLOCK - 1)]);
 #pragma unroll
-            for (int p = 0; p < 64; ++p) {
-                const uint32_t pc = pair_off<BITS>(wv, p) >> 2;
-                row[2 * p] = (_Float16)(cent_s[pc & ((1u << BITS) - 1u)] * g);
-                row[2 * p + 1] = (_Float16)(cent_s[pc >> BITS] * g);
+                for (int p = 0; p < 64; ++p) {
+                    const uint32_t pc = pair_off<BITS>(wv, p) >> 2;
+                    row[2 * p] = (_Float16)(cent_s[pc & ((1u << BITS) - 1u)] * g);
+                    row[2 * p + 1] = (_Float16)(cent_s[pc >> BITS] * g);
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 128; ++p) row[p] = (_Float16)0.0f;
             }
         } else {
             float rs = 0.f;
@@ -736,42 +743,109 @@ __global__ __launch_bounds__(256) void k_score_tile(const __half *qa, const uint
     }
     __syncthreads();
 
-    const int kh = w & 1, qh = w >> 1;
-    const int r16 = lane & 15, kc = lane >> 4;
-    const int64_t n_qt = (nq + 127) / 128;
-    for (int64_t qt = 0; qt < n_qt; ++qt) {
-        float4_t acc[4][4];
+    // two MFMA tiles of 32 x 32 per (64 queries, 32 keys): lane l of a result tile holds key column
+    // l % 32 for the query rows 8j + 4(l/32) + i, so a store instruction writes two runs of 32 consecutive
+    // logits (a whole 128-byte line for fp32).
+    const int qh = __builtin_amdgcn_readfirstlane(w);  // wave-uniform: row addresses of the stores stay scalar
+    const int c32 = lane & 31, kb = lane >> 5;
+    const uint32_t lane_off = (uint32_t)(4 * kb) * (uint32_t)nk + (uint32_t)c32;  // this lane's place relative to a row block
+    constexpr int QT = 512;
+    const int n_qt = (int)((nq + QT - 1) / QT);
+    const int nq_last = (int)nq - 1;  // the launcher checks the query count
+    half8_t qf[16][2];  // [K step of 16][32-query row block] of the current query tile
+    // rows past the last query are clamped (loaded, multiplied, never stored): no branch in the loop
+    const char *qrow[2];
+    auto point_queries = [&](int qt) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-            for (int b = 0; b < 4; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
-        const int64_t qbase = qt * 128 + qh * 64;
-#pragma unroll 2
-        for (int ks = 0; ks < 8; ++ks) {
-            half8_t af[4], bf[4];
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-                af[a] = *reinterpret_cast<const half8_t *>(kt + (kh * 64 + a * 16 + r16) * KT_STRIDE + ks * 32 + 8 * kc);
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int64_t qi = qbase + b * 16 + r16;
-                if (qi < nq) bf[b] = *reinterpret_cast<const half8_t *>(qa + qi * 256 + ks * 32 + 8 * kc);
-                else bf[b] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-#pragma unroll
-                for (int b = 0; b < 4; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        for (int mb = 0; mb < 2; ++mb) {
+            const int qi = min(qt * QT + qh * 64 + mb * 32 + c32, nq_last);
+            qrow[mb] = reinterpret_cast<const char *>(qa) + ((int64_t)(qi >> 5) * 16 * 64 + (qi & 31) + 32 * kb) * 16;
         }
+    };
+    auto load_queries = [&](int t) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+        for (int mb = 0; mb < 2; ++mb) qf[t][mb] = *reinterpret_cast<const half8_t *>(qrow[mb] + t * 1024);
+    };
+    point_queries(0);
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int64_t qi = qbase + b * 16 + r16;
-                const int64_t key = key0 + kh * 64 + a * 16 + 4 * kc;
-                if (qi < nq && key < nk) st_logit4(logits + qi * nk + key, acc[a][b], (int)min((int64_t)4, nk - key));
+    for (int t = 0; t < 16; ++t) load_queries(t);
+    const _Float16 *krow0 = kt + c32 * KT_STRIDE + 8 * kb;
+#pragma unroll 1
+    for (int qt = 0; qt < n_qt; ++qt) {
+        const int qbase = qt * QT + qh * 64;
+        point_queries(min(qt + 1, n_qt - 1));  // the last tile re-reads itself
+        // one 32-key sub-block against the resident query tile; the last one of a tile also fetches the next tile
+        auto sub_block = [&](const int ks, auto prefetch) {
+            float16_t acc[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[mb][e] = 0.0f;
+            const _Float16 *krow = krow0 + ks * 32 * KT_STRIDE;
+            // key operands come from LDS one step ahead; the scheduling fence after every step keeps the
+            // compiler from hoisting all sixteen steps' reads to the top
+            half8_t kf[2];
+            kf[0] = *reinterpret_cast<const half8_t *>(krow);
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                if (t + 1 < 16) kf[(t + 1) & 1] = *reinterpret_cast<const half8_t *>(krow + (t + 1) * 16);
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+                    acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[t][mb], kf[t & 1], acc[mb], 0, 0, 0);
+                if constexpr (decltype(prefetch)::value) load_queries(t);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            const bool full = key0 + ks * 32 + 32 <= nk && qbase + 64 <= (int)nq;
+            const int64_t key = key0 + ks * 32 + c32;
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                TO *ubase = logits + (int64_t)(qbase + mb * 32) * nk + (key0 + ks * 32);  // uniform: row 0 of the block
+                if constexpr (sizeof(TO) == 4) {
+                    if (full) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) (ubase + (int64_t)(8 * j + i) * nk)[lane_off] = (TO)acc[mb][4 * j + i];
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                const int qi = qbase + mb * 32 + 8 * j + 4 * kb + i;
+                                if (qi < (int)nq && key < nk) (ubase + (int64_t)(8 * j + i) * nk)[lane_off] = (TO)acc[mb][4 * j + i];
+                            }
+                    }
+                } else {
+                    // fp16: neighbouring lanes (keys c32, c32 ^ 1) trade two of their four rows so that every
+                    // lane stores two logits at once: even lanes rows i = 0, 1, odd lanes rows i = 2, 3
+                    const bool odd = lane & 1;
+                    const bool pair_ok = (nk & 1) == 0 && (reinterpret_cast<uintptr_t>(logits) & 3u) == 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
+                            const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
+                            const int i = odd ? 2 + h : h;
+                            const int qi = qbase + mb * 32 + 8 * j + 4 * kb + i;
+                            const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;  // keys (c32 & ~1), (c32 | 1)
+                            __half *p = reinterpret_cast<__half *>(ubase + (int64_t)(8 * j + h) * nk) + (lane_off + (odd ? 2u * (uint32_t)nk - 1u : 0u));
+                            const int64_t k0 = key - (odd ? 1 : 0);
+                            if (pair_ok && (full || (qi < (int)nq && k0 + 1 < nk))) {
+                                const uint32_t u = (uint32_t)__half_as_ushort(__float2half_rn(v0)) |
+                                                   ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
+                                *reinterpret_cast<uint32_t *>(p) = u;
+                            } else if (qi < (int)nq) {
+                                if (k0 < nk) p[0] = __float2half_rn(v0);
+                                if (k0 + 1 < nk) p[1] = __float2half_rn(v1);
+                            }
+                        }
+                }
+            }
+        };
+#pragma unroll 1
+        for (int ks = 0; ks < SCORE_KEYS / 32 - 1; ++ks) sub_block(ks, std::false_type{});
+        sub_block(SCORE_KEYS / 32 - 1, std::true_type{});
     }
 }
 
@@ -781,6 +855,10 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
                    const uint8_t *sign_bits, const void *rnorms, int64_t nk, void *logits, int out_dtype, void *ws,
                    int64_t ws_bytes, hipStream_t s) {
     (void)ws_bytes;
+    if (nq >= ((int64_t)1 << 31) / 128) {
+        tq_set_error("tq_score_tile: %lld queries beyond 2^24 - 1", (long long)nq);
+        return TQ_ERR_UNSUPPORTED;
+    }
     __half *qa = reinterpret_cast<__half *>(ws);
     const unsigned qgrid = (unsigned)((nq + 3) / 4);
     switch (q_dtype) {
@@ -791,13 +869,13 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
     }
     int rc = tq_check_launch("prep_score_q");
     if (rc) return rc;
-    const unsigned grid = (unsigned)((nk + 127) / 128);
-    const size_t lds = (size_t)128 * KT_STRIDE * sizeof(_Float16);
+    const unsigned grid = (unsigned)((nk + SCORE_KEYS - 1) / SCORE_KEYS);
+    const size_t lds = (size_t)SCORE_KEYS * KT_STRIDE * sizeof(_Float16);
 #define TQ_SCORE(B, T)                                                                                          \
     {                                                                                                           \
         (void)hipFuncSetAttribute((const void *)k_score_tile<B, T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                   (int)lds);                                                                    \
-        k_score_tile<B, T><<<grid, 256, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
+        k_score_tile<B, T><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
                                                   nq, nk, (T *)logits, h->centroids32, (float)h->proj_scale);   \
     }
     if (out_dtype == TQ_F32) {

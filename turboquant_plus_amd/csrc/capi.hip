@@ -540,7 +540,7 @@ int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, co
             "tq_score_tile: bad argument");
     REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_score_tile: handle has no projection");
     REQUIRE(out_dtype == TQ_F32 || out_dtype == TQ_F16, TQ_ERR_ARG, "tq_score_tile: logits must be fp32 or fp16");
-    REQUIRE(workspace_bytes >= nq * 256 * 2, TQ_ERR_ARG, "tq_score_tile: workspace %lld < %lld bytes",
+    REQUIRE(workspace_bytes >= (nq + 31) / 32 * 32 * 256 * 2, TQ_ERR_ARG, "tq_score_tile: workspace %lld < %lld bytes",
             (long long)workspace_bytes, (long long)(nq * 256 * 2));
     REQUIRE(aligned16(packed) && aligned16(workspace) && aligned16(logits), TQ_ERR_ALIGN,
             "tq_score_tile: packed, workspace and logits must be 16-byte aligned");

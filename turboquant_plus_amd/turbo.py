@@ -226,7 +226,7 @@ class TurboCodec:
         nq = qd.shape[0]
         out_dtype = tt.float32 if out_dtype is None else out_dtype
         logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device)
-        ws = tt.empty(max(nq * 256 * 2, 16), dtype=tt.uint8, device=qd.device)
+        ws = tt.empty(max((nq + 31) // 32 * 32 * 512, 16), dtype=tt.uint8, device=qd.device)
         L.check(L.lib().tq_score_tile(self.handle.h, L.ptr(qd), L.dtype_code(qd), nq, L.ptr(packed), L.ptr(sign_bits),
                                       L.ptr(rnorms), n_keys, L.ptr(logits), L.dtype_code(logits), L.ptr(ws),
                                       ws.numel(), L.stream_ptr()))
