@@ -214,6 +214,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
     __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 1024 ? LUT_TOTAL : 1024];
     __shared__ uint32_t lead;  // tiles finished by the wavefront that is furthest ahead
+    __shared__ uint32_t skipped;  // Sparse V: (query, position) pairs skipped by this workgroup
     char *klut_s = smem;
     char *vlut_s = SHARE ? klut_s : klut_s + KLUT_BYTES;
 
@@ -236,7 +237,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     // The first tile's rows are requested before anything else, so that the query rotation and
     // the table build overlap the first trip to memory.  Afterwards rows are fetched one tile
     // ahead into the same registers: the next K row right after QK has consumed the current
-    // one, the next V row right after PV (dense mode).  The index is clamped at the split's
+    // one, the next V row right after PV (with Sparse V only after a tile that used its V row).  The index is clamped at the split's
     // last tile, so the final prefetch re-reads a row instead of branching.  The norms
     // travel with the rows, so no load is waited for in the tile that issued it.
     uint32_t kw[KROW_DW];
@@ -263,10 +264,13 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row0, kw);
         else load_row<8>(kb, row0, kw);
         kn = load_knorm(tile);
-        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile >> 1) * VBLOCK, row0, vw);
+        load_row<VBITS>(vbase + (int64_t)(tile >> 1) * VBLOCK, row0, vw);
         gvu = load_vnorm(tile);
     }
-    if (tid == 0) lead = 0;
+    if (tid == 0) {
+        lead = 0;
+        skipped = 0;
+    }
 
     float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
     float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
@@ -319,6 +323,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
     unsigned nskip = 0;
+    bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
 #pragma unroll 1
     while (tile < t_end) {
@@ -423,12 +428,15 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
             }
         }
         if constexpr (SPARSE) {
-            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {  // every V row skipped: no V load, no dequant
+            // Every V row of the tile skipped: no dequant, and the next tile's V row is not requested in
+            // advance (negligible weights come in runs); a tile that then does need its row fetches it here.
+            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {
                 gvu = gvu_next;
                 tile = tile_next;
+                v_ahead = false;
                 continue;
             }
-            load_row<VBITS>(vb, row, vw);
+            if (!v_ahead) load_row<VBITS>(vb, row, vw);
         }
 
         // ---- PV ------------------------------------------------------------------------
@@ -442,7 +450,8 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         // tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
         // weights of token group T sit in block T and are broadcast to every block.
         pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
-        if constexpr (!SPARSE) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
+        load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
+        v_ahead = true;
         gvu = gvu_next;
         tile = tile_next;
     }
@@ -458,9 +467,13 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         pml[2 * j + 1] = l_tot;
     }
     if constexpr (SPARSE) {
+        // one device-wide atomic per workgroup: thousands of wavefronts finishing together on one address
+        // would queue for longer than the kernel's own tail
         unsigned tot = nskip;
         for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
-        if (lane == 0 && tot) atomicAdd(a.skip, (unsigned long long)tot);
+        if (lane == 0 && tot) atomicAdd(&skipped, tot);
+        __syncthreads();
+        if (tid == 0 && skipped) atomicAdd(a.skip, (unsigned long long)skipped);
     }
 }
 
