@@ -680,10 +680,12 @@ __global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, i
     __syncthreads();
     if (v >= nq) return;
     float p0 = 0.f, p1 = 0.f;  // (S q)[2*lane], (S q)[2*lane+1]
+#pragma unroll 16
     for (int k = 0; k < 128; ++k) {
         const float qk = qs[w][k];
-        p0 = fmaf(projT[k * 128 + 2 * lane], qk, p0);
-        p1 = fmaf(projT[k * 128 + 2 * lane + 1], qk, p1);
+        const float2 pt = *reinterpret_cast<const float2 *>(projT + k * 128 + 2 * lane);
+        p0 = fmaf(pt.x, qk, p0);
+        p1 = fmaf(pt.y, qk, p1);
     }
     x0 *= s1[2 * lane];
     x1 *= s1[2 * lane + 1];

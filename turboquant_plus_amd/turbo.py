@@ -303,7 +303,13 @@ class DecodeAttention:
 
 def default_splits(n_groups: int, tokens: int) -> int:
     """Context splits per (batch, kv head): one wavefront per split, four
-    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each."""
+    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each.
+    The kernel groups up to 16 splits (the largest power of two dividing the
+    count) into one workgroup, so the count is rounded down to a multiple of 16,
+    or to a power of two below 16."""
     tiles = max(1, (tokens + 63) // 64)
     want = max(1, (4 * 1024 + n_groups - 1) // n_groups)
-    return int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
+    n = int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
+    if n >= 16:
+        return n // 16 * 16
+    return 1 << (n.bit_length() - 1)
