@@ -1192,7 +1192,14 @@ __global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, Lo
     const int64_t blk = blockIdx.x;
     const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
-    const uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * (16 * a.bits + 2));
+    // the block (at most 8448 B) is copied into LDS with coalesced 16-byte loads; codes are picked from there
+    __shared__ __attribute__((aligned(16))) uint8_t block_s[TQ_ROWS_PER_BLOCK * (16 * 4 + 2)];
+    const int block_size = TQ_ROWS_PER_BLOCK * (16 * a.bits + 2);
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(packed + blk * (int64_t)block_size);
+        for (int e = tid; e < block_size / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = src[e];
+    }
+    const uint8_t *block = block_s;
     if (tid < (1 << a.bits)) cent_s[tid] = a.cent[tid];
     float s1v[8], s2v[8];
 #pragma unroll
