@@ -518,10 +518,10 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 //   y'[m] = s2[m] * sum_ks (-1)^popcount((d1 + 2hf) & ks) * Q[d0][ks],  Q[d0][ks] = X[ks] B[d0][ks],
 //   B[d0][ks][8kb + e][n] = s1[k] * H[16 d0 + n][k]
 
-// one 3-bit code per row: w_d = 8 w_d + [sign, level]; level counts of the token: n1 += bit 0,
-// n2 += bit 1, n3 += both
-__device__ __forceinline__ void append_rows_b3(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, uint32_t &n1, uint32_t &n2,
-                                               uint32_t &n3, float y0, float y1, float y2, float y3, const float (&t)[4]) {
+// one 3-bit code per row: w_d = 8 w_d + [sign, level]; the per-token level counts come from field-wise sums
+// over the rows afterwards
+__device__ __forceinline__ void append_rows_b3(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, float y0, float y1,
+                                                     float y2, float y3, const float (&t)[4]) {
     float u0, u1, u2, u3;
     asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t2]\n\t"
         "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t2]\n\t"
@@ -541,32 +541,15 @@ __device__ __forceinline__ void append_rows_b3(uint32_t &w0, uint32_t &w1, uint3
         "v_alignbit_b32 %[w1], %[w1], %[y1], 31\n\t"
         "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[62:63]\n\t"
         "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[w1], s[70:71]\n\t"
-        "s_and_b64 s[76:77], s[60:61], s[68:69]\n\t"
-        "s_and_b64 s[78:79], s[62:63], s[70:71]\n\t"
-        "s_and_b64 s[80:81], s[64:65], s[72:73]\n\t"
-        "s_and_b64 s[82:83], s[66:67], s[74:75]\n\t"
         "v_alignbit_b32 %[w2], %[w2], %[y2], 31\n\t"
         "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[64:65]\n\t"
         "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[w2], s[72:73]\n\t"
         "v_alignbit_b32 %[w3], %[w3], %[y3], 31\n\t"
         "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[66:67]\n\t"
         "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[w3], s[74:75]\n\t"
-        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[60:61]\n\t"
-        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[62:63]\n\t"
-        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[64:65]\n\t"
-        "v_addc_co_u32_e64 %[n2], vcc, %[n2], 0, s[66:67]\n\t"
-        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[68:69]\n\t"
-        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[70:71]\n\t"
-        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[72:73]\n\t"
-        "v_addc_co_u32_e64 %[n1], vcc, %[n1], 0, s[74:75]\n\t"
-        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[76:77]\n\t"
-        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[78:79]\n\t"
-        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[80:81]\n\t"
-        "v_addc_co_u32_e64 %[n3], vcc, %[n3], 0, s[82:83]\n\t"
-        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3), [n1] "+v"(n1), [n2] "+v"(n2), [n3] "+v"(n3),
-          [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3)
+        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3), [u0] "=&v"(u0), [u1] "=&v"(u1), [u2] "=&v"(u2), [u3] "=&v"(u3)
         : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t1] "v"(t[1]), [t2] "v"(t[2]), [t3] "v"(t[3])
-        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "vcc");
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "vcc");
 }
 
 __device__ __forceinline__ void append_rows_b2(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, uint32_t &n1, float y0,
@@ -784,7 +767,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 y[2][d0] = (s01 - s23) * inv;
                 y[3][d0] = (d01 - d23) * inv;
             }
-            uint32_t n1[4] = {0, 0, 0, 0}, n2[4] = {0, 0, 0, 0}, n3[4] = {0, 0, 0, 0};
+            uint32_t n1[4] = {0, 0, 0, 0};  // 2-bit: per-token count of the level bit
             // groups in descending pair order: pair 4u + 2hf + i/2, high code (odd i) first
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
@@ -792,7 +775,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 const int j = grp_word(BITS, 4 * u);
                 const float y0 = y[0 | (hf << 1)][0][i], y1 = y[0 | (hf << 1)][1][i];
                 const float y2 = y[1 | (hf << 1)][0][i], y3 = y[1 | (hf << 1)][1][i];
-                if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], n2[i], n3[i], y0, y1, y2, y3, thr0);
+                if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
                 else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr0);
                 else append_rows_b4(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
             }
@@ -815,12 +798,26 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                     const uint32_t t = sum[p] + (sum[p] >> 16);
                     cnt[p] = (t & 0x0F0Fu) | ((t & 0xF0F0u) << 12);
                 }
+            } else if constexpr (BITS == 3) {
+                // word u of every row (the tail word for u = 3) is complete: 3-bit fields 4hf + i hold token i's
+                // code; field-wise sums of the level-bit products over the four rows stay below 8
+                constexpr uint32_t K0 = 0x00249249u;
+                uint32_t sum[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int dd = 0; dd < 4; ++dd) {
+                    const uint32_t ww = w[dd][u];
+                    const uint32_t b0 = ww & K0, b1 = (ww >> 1) & K0;
+                    sum[1] += b0; sum[2] += b1; sum[3] += b0 & b1;
+                }
+#pragma unroll
+                for (int p = 1; p < 4; ++p) {
+                    // dim halves added in 6-bit lanes: e = tokens 0 and 2, o = tokens 1 and 3; then one byte per token
+                    const uint32_t lo = sum[p] & 0xFFFu, hi = sum[p] >> 12;
+                    const uint32_t e = (lo & 0x1C7u) + (hi & 0x1C7u), o = ((lo >> 3) & 0x1C7u) + ((hi >> 3) & 0x1C7u);
+                    cnt[p] = (e & 0x3Fu) | ((o & 0x3Fu) << 8) | ((e & 0xFC0u) << 10) | ((o & 0xFC0u) << 18);
+                }
             } else {
                 cnt[1] = n1[0] | (n1[1] << 8) | (n1[2] << 16) | (n1[3] << 24);
-                if constexpr (BITS == 3) {
-                    cnt[2] = n2[0] | (n2[1] << 8) | (n2[2] << 16) | (n2[3] << 24);
-                    cnt[3] = n3[0] | (n3[1] << 8) | (n3[2] << 16) | (n3[3] << 24);
-                }
             }
             float cs = 128.0f * coef[0];
             const int sh = BITS == 4 ? 8 * (((n16 & 1) << 1) | ((n16 >> 1) & 1)) : 8 * (n16 & 3);
