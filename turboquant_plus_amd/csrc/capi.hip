@@ -215,6 +215,31 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         st[0] = b32[mid];
         for (int j = 1; j <= mid; ++j) st[j] = b32[mid + j];
         rc = rc ? rc : upload(&h->symthr32, st);
+        // magnitude level by table: a bin of the value's top 12 bits holds at most one boundary, so
+        // level = (boundaries below the bin) + (|value| > the bin's boundary)
+        {
+            std::vector<uint2> ql(4096);
+            h->quant_lut_ok = 1;
+            for (uint32_t idx = 0; idx < 4096; ++idx) {
+                const uint32_t s = idx >> 11, e3 = idx & 2047u;
+                const uint32_t lo_bits = e3 << 20, hi_bits = (e3 + 1u) << 20;
+                float lo, hi;
+                std::memcpy(&lo, &lo_bits, 4);
+                std::memcpy(&hi, &hi_bits, 4);
+                const bool top = e3 >= 2040u;  // infinities and NaNs: the highest level
+                uint32_t below = 0, inside = 0, tbits = 0x7f800000u;
+                for (int j = 1; j <= mid; ++j) {
+                    if (top || st[j] < lo) ++below;
+                    else if (st[j] < hi) {
+                        ++inside;
+                        std::memcpy(&tbits, &st[j], 4);
+                    }
+                }
+                if (inside > 1) h->quant_lut_ok = 0;
+                ql[idx] = make_uint2((s << (b - 1)) | below, tbits);
+            }
+            rc = rc ? rc : upload(&h->quant_lut, ql);
+        }
         // squared centroid of magnitude level m as a multilinear form in the bits of m
         // (Moebius transform over subsets), for counting-based sums of c^2
         {
@@ -258,7 +283,7 @@ void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
                     h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
-                    h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v};
+                    h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v, h->quant_lut};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete h;

@@ -38,6 +38,10 @@ struct tq_handle {
     uint32_t *s2flip;      // [4][4]: per lane quarter and output dword, sign-field positions of dims with s2 = +1
     float *symthr32;       // [2^(bits-1)]: middle boundary, then the positive boundaries
     float *sqcoef32;       // [2^(bits-1)]: c[mid+1+m]^2 = sum over subsets S of the set bits of m of sqcoef32[S]
+    uint2 *quant_lut;      // [4096] indexed by the top 12 bits (sign, exponent, 3 mantissa bits) of a normalised
+                           // rotated value: .x = sign << (bits-1) | number of positive boundaries below the bin,
+                           // .y = fp32 bits of the one boundary inside the bin (+inf when there is none)
+    int quant_lut_ok;      // every bin holds at most one boundary (else the table cannot decide a level)
     int zero_code;         // codebook index of the value 0.0 (#boundaries below 0)
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };

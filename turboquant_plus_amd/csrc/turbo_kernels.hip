@@ -276,6 +276,53 @@ __device__ __forceinline__ uint32_t append4_b2(uint32_t w, float y0, float y1, f
     return w;
 }
 
+// 4-bit codes by table: entry e of a value (tq_handle::quant_lut, indexed by the value's top 12 bits) holds in
+// .x the unfolded field [sign, boundaries below the bin] and in .y the one boundary inside the bin, so
+// field = e.x + (|y| > e.y): one compare and one add-with-carry per value instead of a three-level search.
+__device__ __forceinline__ uint32_t quant_lut_offset(float y) { return (__float_as_uint(y) >> 17) & 0x7ff8u; }
+
+__device__ __forceinline__ uint32_t append4_lut(uint32_t w, float y0, float y1, float y2, float y3, uint2 e0, uint2 e1, uint2 e2,
+                                                uint2 e3) {
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t0]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t3]\n\t"
+        "v_lshlrev_b32_e32 %[w], 4, %[w]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[b0], s[60:61]\n\t"
+        "v_lshlrev_b32_e32 %[w], 4, %[w]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[b1], s[62:63]\n\t"
+        "v_lshlrev_b32_e32 %[w], 4, %[w]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[b2], s[64:65]\n\t"
+        "v_lshlrev_b32_e32 %[w], 4, %[w]\n\t"
+        "v_addc_co_u32_e64 %[w], vcc, %[w], %[b3], s[66:67]\n\t"
+        : [w] "+v"(w)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t0] "v"(e0.y), [t1] "v"(e1.y), [t2] "v"(e2.y), [t3] "v"(e3.y),
+          [b0] "v"(e0.x), [b1] "v"(e1.x), [b2] "v"(e2.x), [b3] "v"(e3.x)
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "vcc");
+    return w;
+}
+
+// the same for four rows at once (V kernel): w_d = 16 w_d + field_d
+__device__ __forceinline__ void append_rows_lut(uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3, float y0, float y1, float y2,
+                                                float y3, uint2 e0, uint2 e1, uint2 e2, uint2 e3) {
+    asm("v_cmp_gt_f32_e64 s[60:61], |%[y0]|, %[t0]\n\t"
+        "v_cmp_gt_f32_e64 s[62:63], |%[y1]|, %[t1]\n\t"
+        "v_cmp_gt_f32_e64 s[64:65], |%[y2]|, %[t2]\n\t"
+        "v_cmp_gt_f32_e64 s[66:67], |%[y3]|, %[t3]\n\t"
+        "v_lshlrev_b32_e32 %[w0], 4, %[w0]\n\t"
+        "v_lshlrev_b32_e32 %[w1], 4, %[w1]\n\t"
+        "v_lshlrev_b32_e32 %[w2], 4, %[w2]\n\t"
+        "v_lshlrev_b32_e32 %[w3], 4, %[w3]\n\t"
+        "v_addc_co_u32_e64 %[w0], vcc, %[w0], %[b0], s[60:61]\n\t"
+        "v_addc_co_u32_e64 %[w1], vcc, %[w1], %[b1], s[62:63]\n\t"
+        "v_addc_co_u32_e64 %[w2], vcc, %[w2], %[b2], s[64:65]\n\t"
+        "v_addc_co_u32_e64 %[w3], vcc, %[w3], %[b3], s[66:67]\n\t"
+        : [w0] "+v"(w0), [w1] "+v"(w1), [w2] "+v"(w2), [w3] "+v"(w3)
+        : [y0] "v"(y0), [y1] "v"(y1), [y2] "v"(y2), [y3] "v"(y3), [t0] "v"(e0.y), [t1] "v"(e1.y), [t2] "v"(e2.y), [t3] "v"(e3.y),
+          [b0] "v"(e0.x), [b1] "v"(e1.x), [b2] "v"(e2.x), [b3] "v"(e3.x)
+        : "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "vcc");
+}
+
 // n[S] += number of fields of the unfolded dword whose level bits include the set S
 template <int BITS> __device__ __forceinline__ void count_levels(uint32_t w, uint32_t (&n)[1 << (BITS - 1)]) {
     if constexpr (BITS == 2) {
@@ -319,10 +366,30 @@ struct StoreKArgs {
                              // (3-bit: entry 3 is for the tail word): appended sign bit ^ this = "positive"
     const float *symthr;     // [0] middle boundary, [1..] positive boundaries
     const float *sqcoef;     // multilinear coefficients of c^2 over the level bits
+    const uint2 *quant_lut;  // tq_handle::quant_lut (4-bit codes)
     int norm_correction;
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
 };
+
+// copy a handle's quantiser table (4096 x 8 B) into LDS with NT threads; every load is issued before the
+// first LDS write
+template <int NT> __device__ __forceinline__ void load_quant_lut(uint2 *dst, const uint2 *src) {
+    constexpr int N16 = 2048, PER = (N16 + NT - 1) / NT;  // 16-byte pieces
+    const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
+    uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+    uint4 v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = (int)threadIdx.x + i * NT;
+        v[i] = s4[e < N16 ? e : N16 - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = (int)threadIdx.x + i * NT;
+        if (e < N16) d4[e] = v[i];
+    }
+}
 
 // RAGGED: sequences whose token count is not a multiple of the block size (rows past the
 // end are quantised as zeros, and the block index needs a division by blocks per sequence).
@@ -339,7 +406,7 @@ __device__ __forceinline__ uint32_t take_ticket(uint32_t *counter, int lane) {
 
 template <int BITS, bool RAGGED>
 __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
-                                              uint32_t end, uint32_t *counter) {
+                                              uint32_t end, uint32_t *counter, const uint2 *qlut) {
     constexpr int NT = 1 << (BITS - 1);
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kc = lane >> 4;
@@ -435,6 +502,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             float thr[NT];
 #pragma unroll
             for (int k = 0; k < NT; ++k) thr[k] = thr0[k] * scale;
+            // table path (4 bits): values are normalised instead of the boundaries being scaled
+            const float inv = norm > 0.0f ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;
 
             // butterfly over the input slices: fragment 2*fh + f0 holds dims 32kc + 8fh + 4f0 + i
             float4_t y[8];
@@ -471,9 +540,17 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             } else if constexpr (BITS == 4) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
+                    // eight values into one unfolded dword through the table, highest value first
                     const int v = 8 * j;
-                    uint32_t w = append4_b4(0u, val(v + 7), val(v + 6), val(v + 5), val(v + 4), thr);
-                    w = append4_b4(w, val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+                    float yn[8];
+                    uint2 e[8];
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) {
+                        yn[m] = val(v + m) * inv;
+                        e[m] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(qlut) + quant_lut_offset(yn[m]));
+                    }
+                    uint32_t w = append4_lut(0u, yn[7], yn[6], yn[5], yn[4], e[7], e[6], e[5], e[4]);
+                    w = append4_lut(w, yn[3], yn[2], yn[1], yn[0], e[3], e[2], e[1], e[0]);
                     count_levels<4>(w, n);
                     g[j] = fold_codes<4>(nonzero ? w ^ flip[j] : (zero_word & 0x88888888u));
                 }
@@ -648,6 +725,7 @@ struct StoreVArgs {
     const float *s2;      // [128] output signs
     const float *symthr;  // [0] middle boundary, [1..] positive boundaries
     const float *sqcoef;  // multilinear coefficients of c^2 over the level bits
+    const uint2 *quant_lut;  // tq_handle::quant_lut (4-bit codes)
     int norm_correction;
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
@@ -656,7 +734,7 @@ struct StoreVArgs {
 // Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.
 template <int BITS, bool RAGGED>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
-                                              uint32_t end, uint32_t *counter) {
+                                              uint32_t end, uint32_t *counter, const uint2 *qlut) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
     const int tid = threadIdx.x, lane = tid & 63;
@@ -777,7 +855,14 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 const float y2 = y[1 | (hf << 1)][0][i], y3 = y[1 | (hf << 1)][1][i];
                 if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
                 else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr0);
-                else append_rows_b4(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
+                else {
+                    const char *ql = reinterpret_cast<const char *>(qlut);
+                    append_rows_lut(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3,
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y0)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y1)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y2)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y3)));
+                }
             }
             // level counts of the four tokens, one byte per token, summed over the 16 columns
             uint32_t cnt[NT];
@@ -868,19 +953,23 @@ __device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g)
 template <int BITS, bool RAGGED>
 __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
     __shared__ uint32_t counter[4];
+    __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
     __syncthreads();
-    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave]);
+    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut);
 }
 
 template <int BITS, bool RAGGED>
 __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
     __shared__ uint32_t counter[4];
+    __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
     __syncthreads();
-    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave]);
+    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut);
 }
 
 // K and V of one layer in one launch, one workgroup of 12 wavefronts per CU owning an equal
@@ -891,12 +980,16 @@ template <int KB, int VB, bool RAGGED>
 __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk, StoreKArgs ka, const __half *xv, uint8_t *pv,
                                                   StoreVArgs va) {
     __shared__ uint32_t counter[2];
+    __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 4096 : 2];
+    __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 4096 : 2];
     if (threadIdx.x < 2) counter[threadIdx.x] = 0;
+    if constexpr (KB == 4) load_quant_lut<768>(qlut_k, ka.quant_lut);
+    if constexpr (VB == 4) load_quant_lut<768>(qlut_v, va.quant_lut);
     __syncthreads();
     store_v_units<VB, RAGGED>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0]);
+                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v);
     store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1]);
+                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k);
 }
 
 // ---- K2: fused quantise + pack ---------------------------------------------------
@@ -1327,12 +1420,14 @@ static bool store_fast_ok(const tq_handle *h, int in_dtype, int64_t n_blocks) {
         const char *e = getenv("TQ_STORE_PATH");
         return e && strcmp(e, "butterfly") == 0;
     }();
-    return in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && n_blocks < (1ll << 28) && !force_butterfly;
+    return in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && (h->bits != 4 || h->quant_lut_ok) &&
+           n_blocks < (1ll << 28) && !force_butterfly;
 }
 
 static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {
     StoreKArgs ka;
     ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
+    ka.quant_lut = h->quant_lut;
     ka.norm_correction = h->norm_correction; ka.tokens = tokens;
     ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
     return ka;
@@ -1341,6 +1436,7 @@ static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, i
 static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {
     StoreVArgs va;
     va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
+    va.quant_lut = h->quant_lut;
     va.norm_correction = h->norm_correction; va.tokens = tokens;
     va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
     return va;
