@@ -110,7 +110,7 @@ def test_turboquant(golden, b):
 
 @pytest.mark.parametrize("tb", [2.5, 3.5])
 def test_outlier_split_quantiser(golden, tb):
-    """turboquant/outlier.py:45-217, fixtures written from the reference."""
+    """turboquant/outlier.py:45-217 : fractional bit rates by channel split; fixtures written from the reference."""
     tag = f"outlier_{str(tb).replace('.', 'p')}"
     oq = O.OutlierRef(D, tb, seed=42)
     meta = golden[f"{tag}_meta"]
@@ -137,7 +137,7 @@ def test_outlier_channel_split(golden):
 
 
 def test_temporal_decay_requantize(golden):
-    """3-bit rows -> 2-bit (benchmarks/temporal_decay_prototype.py:93-125, SURVEY 8(f) row 3); the prototype
+    """3-bit rows -> 2-bit (benchmarks/temporal_decay_prototype.py:93-125); the prototype
     takes the uncorrected norm and corrects at read time, the device format stores the corrected norm."""
     c3, c2 = golden["decay_c3"], golden["decay_c2"]
     idx3, n3 = golden["decay_idx3"], golden["decay_norm3"]
