@@ -484,13 +484,14 @@ __global__ void k_clear_skip(unsigned long long *skip, unsigned long long total_
     skip[1] = total_pairs;
 }
 
-// merge split partials, un-rotate with the V rotation's transpose; one workgroup of four
+// merge split partials, un-rotate with the V rotation's transpose; one workgroup of NW (4 or 16)
 // wavefronts per query head.  Every wavefront fetches (m, l) of all splits (lane s <-> split s,
 // 64 per pass) so the weights are known after one round trip, streams the partial outputs of
-// its quarter of the splits with independent loads, and wavefront 0 adds the four quarters.
-__global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
-                                                      int64_t n_rows, int n_splits, const float *s1, const float *s2) {
-    __shared__ float red[4][130];
+// its share of the splits with independent loads, and wavefront 0 adds the shares.
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
+                                                          int64_t n_rows, int n_splits, const float *s1, const float *s2) {
+    __shared__ float red[NW][130];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t r = blockIdx.x;  // row = group*4 + head
     const int64_t group = r >> 2;
@@ -518,7 +519,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const
         L += lw;
         const int cnt = min(64, n_splits - s0);
 #pragma unroll 8
-        for (int t = wv; t < cnt; t += 4) {
+        for (int t = wv; t < cnt; t += NW) {
             const float wt = __shfl(w, t);
             const float2 v = *reinterpret_cast<const float2 *>(po + (int64_t)(s0 + t) * 512 + 2 * lane);
             o0 = fmaf(v.x, wt, o0);
@@ -529,8 +530,13 @@ __global__ __launch_bounds__(256) void k_attn_combine(const float *part_o, const
     red[wv][2 * lane + 1] = o1;
     __syncthreads();
     if (wv != 0) return;
-    o0 = (red[0][2 * lane] + red[1][2 * lane]) + (red[2][2 * lane] + red[3][2 * lane]);
-    o1 = (red[0][2 * lane + 1] + red[1][2 * lane + 1]) + (red[2][2 * lane + 1] + red[3][2 * lane + 1]);
+    o0 = 0.0f;
+    o1 = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NW; q += 4) {
+        o0 += (red[q][2 * lane] + red[q + 1][2 * lane]) + (red[q + 2][2 * lane] + red[q + 3][2 * lane]);
+        o1 += (red[q][2 * lane + 1] + red[q + 1][2 * lane + 1]) + (red[q + 2][2 * lane + 1] + red[q + 3][2 * lane + 1]);
+    }
     const float invL = L > 0.0f ? 1.0f / L : 0.0f;
     o0 *= invL * s2[2 * lane];
     o1 *= invL * s2[2 * lane + 1];
@@ -652,7 +658,9 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 #undef TQ_ATTN_ONE
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
-    k_attn_combine<<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
+    // many splits: sixteen wavefronts share a row's partials
+    if (p->n_splits >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
+    else k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
     return tq_check_launch("attn_combine");
 }
 
