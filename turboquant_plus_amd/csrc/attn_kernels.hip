@@ -62,15 +62,15 @@ template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_
     }
 }
 
-// build a codebook's decode table in LDS from its pair table (half2 per pair code) in global memory
-// with n_waves wavefronts; the global load is issued before the first LDS write
-template <int BITS> __device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, int tid, int n_waves) {
+// build a codebook's decode table in LDS from its pair table (half2 per pair code) with n_waves wavefronts;
+// `mine` is pair entry tid % 64, fetched by the caller ahead of time (used by the 3-bit table only)
+template <int BITS>
+__device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, uint32_t mine, int tid, int n_waves) {
     constexpr int NP = 1 << (2 * BITS);
     if constexpr (BITS == 3) {
         // lane l holds pair entry l; wavefront w writes the rows hi = w, w + n_waves, ..
         uint2 *t = reinterpret_cast<uint2 *>(dst);
         const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const uint32_t mine = pair_lut[lane];
         for (int hi = wave; hi < 64; hi += n_waves)
             t[hi * 64 + lane] = make_uint2(mine, (uint32_t)__builtin_amdgcn_readlane((int)mine, hi));
     } else if constexpr (BITS == 2) {
@@ -271,6 +271,10 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         lead = 0;
         skipped = 0;
     }
+    // pair-table entries for the table build below: requested now, needed after the query rotation
+    uint32_t kpair = 0, vpair = 0;
+    if constexpr (KFMT == KFMT_TURBO && KBITS == 3) kpair = a.klut[lane];
+    if constexpr (!SHARE && VBITS == 3) vpair = a.vlut[lane];
 
     float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
     float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
@@ -314,8 +318,8 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
     __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
-    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, tid, n_waves);
-    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, tid, n_waves);
+    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
+    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
     __syncthreads();
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[2][2];
