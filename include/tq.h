@@ -140,6 +140,11 @@ int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const v
 int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity,
               int in_dtype, int kind, void *packed, void *stream);
 
+/* tq_append of the K and the V tokens of one decode step (same n_seqs, pos, n_new, capacity, dtype) in one
+ * launch: what a serving loop runs between two attention steps.  Same results as two tq_append calls. */
+int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
+                 int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, void *stream);
+
 /* Temporal decay: re-quantise a packed buffer to a narrower width without going back to the
  * original vectors (`requantize_3to2`, benchmarks/temporal_decay_prototype.py:93-125): per row
  * decode with the stored norm, renormalise, nearest centroid of `dst`'s codebook (a value equal

@@ -43,6 +43,30 @@ def test_append_in_chunks_equals_store(bits, kind):
     assert pos == 300
 
 
+@pytest.mark.parametrize("kbits,vbits", [(3, 3), (4, 4), (4, 2), (2, 4)])
+def test_append_kv_equals_two_appends(kbits, vbits):
+    """K and V of a step in one launch (tq_append_kv) write the bytes of two tq_append calls;
+    the (2, 4) pair has no fused kernel and takes the two-launch route inside the library."""
+    tt = L.torch()
+    kc, vc = tqa.TurboCodec(kbits, seed=7), tqa.TurboCodec(vbits, seed=507)
+    n_seqs, capacity = 5, 384
+    rng = np.random.default_rng(kbits * 10 + vbits)
+    k = rng.standard_normal((n_seqs, 200, D)).astype(np.float16)
+    v = rng.standard_normal((n_seqs, 200, D)).astype(np.float16)
+    ck = tt.zeros(tqa.packed_bytes(kbits, n_seqs, capacity), dtype=tt.uint8, device="cuda")
+    cv = tt.zeros(tqa.packed_bytes(vbits, n_seqs, capacity), dtype=tt.uint8, device="cuda")
+    rk, rv = tt.zeros_like(ck), tt.zeros_like(cv)
+    pos = 0
+    for n_new in [1, 1, 126, 1, 70, 1]:
+        kc.append_kv(vc, k[:, pos:pos + n_new], v[:, pos:pos + n_new], ck, cv, pos, capacity)
+        kc.append(k[:, pos:pos + n_new], rk, pos, capacity, kind="k")
+        vc.append(v[:, pos:pos + n_new], rv, pos, capacity, kind="v")
+        pos += n_new
+        assert tt.equal(ck, rk) and tt.equal(cv, rv), f"after {pos} tokens"
+    with pytest.raises(ValueError):
+        kc.append_kv(vc, k[:, :2], v[:, :3], ck, cv, 0, capacity)
+
+
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_append_codes_match_oracle(dtype):
     tt = L.torch()

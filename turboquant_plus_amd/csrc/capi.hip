@@ -419,6 +419,21 @@ int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, in
     return tqk_append(h, x, n_seqs, pos, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream);
 }
 
+int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
+                 int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, void *stream) {
+    int rc = check_fast(hk, "tq_append_kv");
+    rc = rc ? rc : check_fast(hv, "tq_append_kv");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && pos >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_append_kv: bad argument");
+    REQUIRE(pos + n_new <= capacity, TQ_ERR_ARG, "tq_append_kv: tokens %lld..%lld do not fit a capacity of %lld", (long long)pos,
+            (long long)(pos + n_new), (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(k && v && packed_k && packed_v, TQ_ERR_ARG, "tq_append_kv: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
+            "tq_append_kv: inputs and packed buffers must be 16-byte aligned");
+    return tqk_append_kv(hk, hv, k, v, n_seqs, pos, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream);
+}
+
 int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs, int64_t tokens,
                   int kind, void *packed_dst, void *stream) {
     int rc = check_fast(src_h, "tq_requantize");

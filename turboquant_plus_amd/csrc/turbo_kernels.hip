@@ -102,12 +102,14 @@ template <int BITS> __device__ inline uint32_t pair_from_stage(const uint8_t *co
     return lo | (hi << BITS);
 }
 
+// first_row > 0 (K rows only, where a row is a token): rows and norms below it are left as they are in memory.
 template <int BITS, int NTHREADS>
-__device__ inline void pack_block(const uint8_t *codes, const float *norms, uint8_t *out_block, int kind) {
+__device__ inline void pack_block(const uint8_t *codes, const float *norms, uint8_t *out_block, int kind, int first_row = 0) {
     uint32_t *out = reinterpret_cast<uint32_t *>(out_block);
     constexpr int NDW = TQ_ROWS_PER_BLOCK * 4 * BITS;
     for (int o = threadIdx.x; o < NDW; o += NTHREADS) {
         const int c = o >> 9, r = (o & 511) >> 2, k = o & 3;
+        if (r < first_row) continue;
         // chunk c, dword k of the row = dword j = c of group g = k
         constexpr int PER = pairs_per_dword(BITS);
         const int g = k, j = c;
@@ -122,10 +124,15 @@ __device__ inline void pack_block(const uint8_t *codes, const float *norms, uint
         }
         out[o] = word;
     }
-    for (int t = threadIdx.x; t < 64; t += NTHREADS) {
-        const uint32_t lo = __half_as_ushort(__float2half_rn(norms[2 * t]));
-        const uint32_t hi = __half_as_ushort(__float2half_rn(norms[2 * t + 1]));
-        out[NDW + t] = lo | (hi << 16);
+    if (first_row == 0) {
+        for (int t = threadIdx.x; t < 64; t += NTHREADS) {
+            const uint32_t lo = __half_as_ushort(__float2half_rn(norms[2 * t]));
+            const uint32_t hi = __half_as_ushort(__float2half_rn(norms[2 * t + 1]));
+            out[NDW + t] = lo | (hi << 16);
+        }
+    } else {
+        __half *nout = reinterpret_cast<__half *>(out + NDW);
+        for (int t = first_row + (int)threadIdx.x; t < TQ_ROWS_PER_BLOCK; t += NTHREADS) nout[t] = __float2half_rn(norms[t]);
     }
 }
 
@@ -1088,15 +1095,16 @@ __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, Sto
 // tokens 0 .. T-1 the touched blocks equal those of k_store on the first T tokens.
 struct AppendArgs {
     const float *s1, *s2, *bounds, *cent;
-    int kind, norm_correction;
+    int kind, norm_correction, zero_code;
     int64_t pos, n_new, blocks_per_seq, first_block, n_touched;
 };
 
 __device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, int token, int dim);
 __device__ inline float block_norm(const uint8_t *block, int bits, int token);
 
+// one workgroup rebuilds block `wg` (sequence wg / n_touched, touched block wg % n_touched)
 template <int BITS, typename TI>
-__global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, AppendArgs a) {
+__device__ __forceinline__ void append_block(const TI *x, uint8_t *packed, const AppendArgs &a, const int64_t wg) {
     constexpr int NB = (1 << BITS) - 1;
     __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
     __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
@@ -1104,7 +1112,7 @@ __global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, Ap
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int li = lane & 15, grp = tid >> 4;
-    const int64_t seq = blockIdx.x / a.n_touched, bis = a.first_block + blockIdx.x % a.n_touched;
+    const int64_t seq = wg / a.n_touched, bis = a.first_block + wg % a.n_touched;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
     uint8_t *block = packed + (seq * a.blocks_per_seq + bis) * block_bytes(BITS);
 
@@ -1121,34 +1129,57 @@ __global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, Ap
         s1v[m] = a.s1[8 * li + m];
         s2v[m] = a.s2[8 * li + m] * RSQRT128;
     }
-    // rows already in the block
+    // rows already in the block: the block is copied into LDS with coalesced loads and unpacked from there
     const int n_old = (int)(a.pos - tok0 < 0 ? 0 : (a.pos - tok0 > TQ_ROWS_PER_BLOCK ? TQ_ROWS_PER_BLOCK : a.pos - tok0));
-    for (int e = tid; e < n_old * 128; e += 256) {
-        const int t = e >> 7, dim = e & 127;
-        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(block, BITS, a.kind, t, dim);
+    const int n_end = (int)(a.pos + a.n_new - tok0 > TQ_ROWS_PER_BLOCK ? TQ_ROWS_PER_BLOCK : a.pos + a.n_new - tok0);  // first empty row
+    __shared__ __attribute__((aligned(16))) uint8_t old_s[block_bytes(BITS)];
+    // K rows are tokens: the rows already there stay untouched in memory and need not be unpacked
+    const bool keep_rows = a.kind == TQ_KIND_K;
+    if (n_old > 0 && !keep_rows) {
+        for (int e = tid; e < block_bytes(BITS) / 16; e += 256)
+            reinterpret_cast<uint4 *>(old_s)[e] = reinterpret_cast<const uint4 *>(block)[e];
+        __syncthreads();
+        for (int e = tid; e < n_old * 128; e += 256) {
+            const int t = e >> 7, dim = e & 127;
+            codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(old_s, BITS, a.kind, t, dim);
+        }
+        for (int t = tid; t < n_old; t += 256) norms_s[t] = block_norm(old_s, BITS, t);
     }
-    for (int t = tid; t < n_old; t += 256) norms_s[t] = block_norm(block, BITS, t);
+    // rows past the new tokens hold the code of 0.0 and norm 0 (what quantising a zero vector gives)
+    for (int e = tid; e < (TQ_ROWS_PER_BLOCK - n_end) * 32; e += 256) {
+        const int t = n_end + (e >> 5), q = e & 31;
+        *reinterpret_cast<uint32_t *>(&codes[t * CODE_STRIDE + 4 * q]) = 0x01010101u * (uint32_t)a.zero_code;
+    }
+    for (int t = n_end + tid; t < TQ_ROWS_PER_BLOCK; t += 256) norms_s[t] = 0.0f;
     __syncthreads();
 
 #pragma unroll 1
     for (int it = 0; it < 8; ++it) {
         const int t = it * 16 + grp;
-        if (t < n_old) continue;  // whole 16-lane rows skip together
+        if (t < n_old || t >= n_end) continue;  // whole 16-lane rows skip together
         const int64_t rel = tok0 + t - a.pos;
         float xv[8];
-        if (rel < a.n_new) {
-            load8(x + ((seq * a.n_new + rel) * 128 + 8 * li), xv);
-        } else {
-#pragma unroll
-            for (int m = 0; m < 8; ++m) xv[m] = 0.0f;
-        }
+        load8(x + ((seq * a.n_new + rel) * 128 + 8 * li), xv);
         uint2 c8;
         const float g = quantize_vec16<BITS>(xv, lane, bnd, s1v, s2v, csq_s, a.norm_correction, c8);
         *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = c8;
         if (li == 0) norms_s[t] = g;
     }
     __syncthreads();
-    pack_block<BITS, 256>(codes, norms_s, block, a.kind);
+    pack_block<BITS, 256>(codes, norms_s, block, a.kind, keep_rows ? n_old : 0);
+}
+
+template <int BITS, typename TI>
+__global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, AppendArgs a) {
+    append_block<BITS, TI>(x, packed, a, blockIdx.x);
+}
+
+// K and V of a decode step in one launch: the first half of the grid rebuilds K blocks, the second half V blocks
+template <int KB, int VB, typename TI>
+__global__ __launch_bounds__(256) void k_append_kv(const TI *xk, uint8_t *pk, AppendArgs ka, const TI *xv, uint8_t *pv, AppendArgs va) {
+    const unsigned half = gridDim.x >> 1;
+    if (blockIdx.x < half) append_block<KB, TI>(xk, pk, ka, blockIdx.x);
+    else append_block<VB, TI>(xv, pv, va, blockIdx.x - half);
 }
 
 // ---- K2 + K4 in float64: codes, corrected norm, residual sign sketch ---------------
@@ -1704,15 +1735,44 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
     return tq_check_launch("fork_blocks");
 }
 
-int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
-               int kind, void *packed, hipStream_t s) {
-    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+static AppendArgs make_append_args(const tq_handle *h, int64_t pos, int64_t n_new, int64_t capacity, int kind) {
     AppendArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
-    a.kind = kind; a.norm_correction = h->norm_correction;
+    a.kind = kind; a.norm_correction = h->norm_correction; a.zero_code = h->zero_code;
     a.pos = pos; a.n_new = n_new; a.blocks_per_seq = blocks_for(capacity);
     a.first_block = pos / TQ_ROWS_PER_BLOCK;
     a.n_touched = (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
+    return a;
+}
+
+int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
+                  int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s) {
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    const AppendArgs ka = make_append_args(hk, pos, n_new, capacity, TQ_KIND_K);
+    const AppendArgs va = make_append_args(hv, pos, n_new, capacity, TQ_KIND_V);
+    const unsigned grid = 2u * (unsigned)(n_seqs * ka.n_touched);
+    const int kb = hk->bits, vb = hv->bits;
+#define TQ_APPEND_KV(KB, VB)                                                                                                   \
+    DISPATCH_T(in_dtype, TI, (k_append_kv<KB, VB, TI><<<grid, 256, 0, s>>>((const TI *)k, (uint8_t *)packed_k, ka, (const TI *)v, \
+                                                                            (uint8_t *)packed_v, va)))
+    if (kb == 3 && vb == 3) { TQ_APPEND_KV(3, 3); }
+    else if (kb == 4 && vb == 4) { TQ_APPEND_KV(4, 4); }
+    else if (kb == 2 && vb == 2) { TQ_APPEND_KV(2, 2); }
+    else if (kb == 4 && vb == 2) { TQ_APPEND_KV(4, 2); }
+    else if (kb == 3 && vb == 2) { TQ_APPEND_KV(3, 2); }
+    else if (kb == 4 && vb == 3) { TQ_APPEND_KV(4, 3); }
+    else {  // other pairs: two launches
+        const int rc = tqk_append(hk, k, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_K, packed_k, s);
+        return rc ? rc : tqk_append(hv, v, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_V, packed_v, s);
+    }
+#undef TQ_APPEND_KV
+    return tq_check_launch("append_kv");
+}
+
+int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
+               int kind, void *packed, hipStream_t s) {
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    const AppendArgs a = make_append_args(h, pos, n_new, capacity, kind);
     const unsigned grid = (unsigned)(n_seqs * a.n_touched);
 #define TQ_APPEND_BITS(B) \
     DISPATCH_T(in_dtype, TI, (k_append<B, TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, a)))

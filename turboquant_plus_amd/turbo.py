@@ -142,6 +142,21 @@ class TurboCodec:
                                   L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
         return packed
 
+    def append_kv(self, v_codec: "TurboCodec", k, v, packed_k, packed_v, pos: int, capacity: int):
+        """append() of the K tokens (this codec) and the V tokens (`v_codec`) of one decode step
+        in one launch (tq_append_kv)."""
+        kd, n_seqs, n_new = self._as_seqs(k)
+        vd, vs, vn = self._as_seqs(v)
+        if (vs, vn) != (n_seqs, n_new) or vd.dtype != kd.dtype:
+            raise ValueError("k and v must have the same shape and dtype")
+        for codec, buf in ((self, packed_k), (v_codec, packed_v)):
+            need = packed_bytes(codec.bits, n_seqs, capacity)
+            if buf.numel() < need:
+                raise ValueError(f"packed holds {buf.numel()} bytes, need {need}")
+        L.check(L.lib().tq_append_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, pos, n_new, capacity,
+                                     L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
+        return packed_k, packed_v
+
     def requantize_to(self, dst_codec: "TurboCodec", packed, n_seqs: int, tokens: int, kind: str = "k"):
         """Temporal decay: re-quantise a buffer written with this codec to the narrower
         `dst_codec` (same rotation) -> new packed buffer (tq_requantize)."""
