@@ -132,6 +132,29 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
     algo = 2 * B * Hkv * N * 50
     us = ev_ms * 1e3
     gbs = algo / (us * 1e-6) / 1e9
+
+    # a whole serving step: append this step's K and V token of every sequence (the last position of the
+    # cache is rewritten each time), then attention; launched one by one and replayed from one HIP graph
+    g = torch.Generator(device="cuda").manual_seed(77)
+    k_new = torch.randn((B * Hkv, 1, D), generator=g, device="cuda").to(torch.float16)
+    v_new = torch.randn((B * Hkv, 1, D), generator=g, device="cuda").to(torch.float16)
+
+    def serving_step(i):
+        q, kp, vp = sets[i % n_sets]
+        kc.append_kv(vc, k_new, v_new, kp, vp, N - 1, N)
+        attn(q, kp, vp)
+
+    _, serve_ms = time_steps(torch, serving_step, steps, warmup)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        serving_step(0)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(n_sets):
+            serving_step(i)
+    _, graph_ms = time_steps(torch, lambda i: graph.replay(), max(1, steps // n_sets), max(1, warmup // n_sets))
     return {
         "workload": "fused decode attention, turbo3 K/V, B16 Hq32 Hkv8 d128 ctx 32768, queries rotated in-step",
         "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
@@ -139,6 +162,8 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
                      "traffic": TRAFFIC_BYTES["decode3"], "algorithmic_bytes_per_step": algo,
                      "kernel": "k_decode_attn<turbo3,turbo3> (+ k_attn_combine in the step time)"},
         "buffer_sets": n_sets,
+        "serving_step": {"workload": "tq_append_kv of one token per sequence + decode attention",
+                         "us_per_step": serve_ms * 1e3, "us_per_step_hip_graph": graph_ms * 1e3 / n_sets},
     }
 
 

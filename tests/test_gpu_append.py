@@ -148,6 +148,58 @@ def _check_requant(src, dst, packed_src, n_seqs, tokens, kind):
     return out
 
 
+def test_decode_step_replayed_from_a_hip_graph():
+    """append_kv + decode attention (dense and Sparse V) captured once in a HIP graph and replayed with new
+    inputs: every replay equals the eager result bit for bit, with eager work between the replays."""
+    tt = L.torch()
+    B, Hq, Hkv, cap, pos = 2, 8, 2, 512, 300
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    rng = np.random.default_rng(5)
+    k0 = rng.standard_normal((B * Hkv, pos, D)).astype(np.float16)
+    v0 = rng.standard_normal((B * Hkv, pos, D)).astype(np.float16)
+    ck = tt.zeros(tqa.packed_bytes(3, B * Hkv, cap), dtype=tt.uint8, device="cuda")
+    cv = tt.zeros_like(ck)
+    kc.append_kv(vc, k0, v0, ck, cv, 0, cap)
+    base_k, base_v = ck.clone(), cv.clone()
+    q_s = tt.zeros((B, Hq, D), dtype=tt.float16, device="cuda")
+    kn_s = tt.zeros((B * Hkv, 1, D), dtype=tt.float16, device="cuda")
+    vn_s = tt.zeros_like(kn_s)
+    for tau in (0.0, 1e-3):
+        attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, pos + 1, n_splits=4, capacity=cap, sparse_v_tau=tau)
+
+        def step():
+            kc.append_kv(vc, kn_s, vn_s, ck, cv, pos, cap)
+            return attn(q_s, ck, cv)
+
+        side = tt.cuda.Stream()
+        side.wait_stream(tt.cuda.current_stream())
+        with tt.cuda.stream(side):
+            step()                                   # warm-up outside the capture
+        tt.cuda.current_stream().wait_stream(side)
+        graph = tt.cuda.CUDAGraph()
+        with tt.cuda.graph(graph):
+            out_g = step()
+        for trial in range(4):
+            q = tt.from_numpy(rng.standard_normal((B, Hq, D)).astype(np.float16)).cuda()
+            kn = tt.from_numpy(rng.standard_normal((B * Hkv, 1, D)).astype(np.float16)).cuda()
+            vn = tt.from_numpy(rng.standard_normal((B * Hkv, 1, D)).astype(np.float16)).cuda()
+            ek, ev = base_k.clone(), base_v.clone()      # eager reference on private buffers
+            kc.append_kv(vc, kn, vn, ek, ev, pos, cap)
+            eager = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, pos + 1, n_splits=4, capacity=cap, sparse_v_tau=tau)
+            want = eager(q, ek, ev).clone()
+            want_skip = eager.skip_rate() if tau else 0.0
+            tt.cuda.synchronize()
+            q_s.copy_(q)
+            kn_s.copy_(kn)
+            vn_s.copy_(vn)
+            graph.replay()
+            tt.cuda.synchronize()
+            assert tt.equal(out_g, want), f"tau {tau}, replay {trial}"
+            assert tt.equal(ck, ek) and tt.equal(cv, ev)
+            if tau:
+                assert attn.skip_rate() == want_skip
+
+
 def test_requantize_3_to_2_prototype_presets(golden):
     """The prototype's literal centroid presets, its rows, device format in between."""
     c3, c2 = golden["decay_c3"], golden["decay_c2"]
