@@ -79,6 +79,33 @@ def test_decode_attention_turbo3(N, n_splits):
     np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
 
 
+@pytest.mark.parametrize("B,Hkv,N,n_splits,capacity", [
+    (1, 1, 64, 32, 0),        # one tile, 31 empty splits in a 16-wavefront workgroup
+    (1, 2, 200, 16, 0),       # 4 tiles over 16 splits: 12 empty, last tile ragged
+    (3, 1, 1000, 48, 1024),   # 48 = 3 workgroups of 16 splits; cache laid out for 1024 tokens
+    (2, 2, 1537, 32, 2048),   # ragged tail, capacity stride
+    (1, 3, 4000, 6, 0),       # 6 splits: workgroups of 2 wavefronts
+    (5, 1, 777, 7, 0),        # odd split count: one wavefront per workgroup
+])
+def test_decode_attention_split_and_capacity_shapes(B, Hkv, N, n_splits, capacity):
+    Hq = 4 * Hkv
+    rng = np.random.default_rng(N + n_splits)
+    cap = capacity or N
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    tt = L.torch()
+    ck = tt.zeros(tqa.packed_bytes(3, B * Hkv, cap), dtype=tt.uint8, device="cuda")
+    cv = tt.zeros_like(ck)
+    kc.append_kv(vc, k, v, ck, cv, 0, cap)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, capacity=capacity)(q, ck, cv))
+    kp, vp = kc.store(k, kind="k"), vc.store(v, kind="v")      # same codes without the capacity stride
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D))
+    assert np.isfinite(out).all()
+    assert_close(out, ref)
+
+
 @pytest.mark.parametrize("kbits,vbits", [(4, 4), (2, 2), (4, 2), (3, 2)])
 def test_decode_attention_other_bit_widths(kbits, vbits):
     B, Hq, Hkv, N = 1, 8, 2, 640
