@@ -22,10 +22,11 @@
 //         4b..4b+3] -> D_b = out[4 heads][4 dims].  16 token groups x 2 dim halves = 32
 //         MFMAs per tile into 16 accumulator registers; no cross-lane reduction at the
 //         end of the split and no LDS traffic besides the LUT reads.
-//   Online softmax in base 2 (log2(e) folded into the query scale).
-// k_attn_combine: log-sum-exp merge of the split partials, then the transpose of
-//   the V rotation (one workgroup per query head).  Queries are rotated and scaled
-//   inside k_decode_attn, so a dense step is two launches.
+//   Online softmax in base 2 (log2(e) folded into the query scale).  The wavefronts
+//   of a workgroup (up to 16 splits) merge their results in LDS and write one partial.
+// k_attn_combine / k_attn_combine_few: log-sum-exp merge of the workgroups' partials,
+//   then the transpose of the V rotation.  Queries are rotated and scaled inside
+//   k_decode_attn, so a dense step is two launches.
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
 #include <cstring>
@@ -149,8 +150,8 @@ struct AttnArgs {
     const uint8_t *k, *v;
     const uint32_t *klut, *vlut;  // pair tables (half2 per pair code)
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
-    float *part_o;                // [groups][n_splits][4][128]
-    float *part_ml;               // [groups][n_splits][4][2]  (m in log2 units, l)
+    float *part_o;                // [groups][workgroups per group][4][128]
+    float *part_ml;               // [groups][workgroups per group][4][2]  (m in log2 units, l)
     unsigned long long *skip;     // [0] += skipped (query, position) pairs
     int64_t tokens, blocks_per_seq;
     int n_groups, n_splits, tiles_per_split, n_tiles;
@@ -158,6 +159,7 @@ struct AttnArgs {
 };
 
 constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
+constexpr int MERGE_FLOATS = 520;  // LDS floats per wavefront for the end-of-kernel merge: out[4][128], m[4], l[4]
 
 // QK over the 32 dim groups: B = this lane's K row (4 dims per group), A = q from block G % 16
 template <int BITS, int... G>
@@ -276,8 +278,9 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     if constexpr (KFMT == KFMT_TURBO && KBITS == 3) kpair = a.klut[lane];
     if constexpr (!SHARE && VBITS == 3) vpair = a.vlut[lane];
 
-    float *po = a.part_o + ((int64_t)group * a.n_splits + split) * 4 * 128;
-    float *pml = a.part_ml + ((int64_t)group * a.n_splits + split) * 4 * 2;
+    // one partial per workgroup: index (group, part)
+    float *po = a.part_o + ((int64_t)group * wgs_per_group + part) * 4 * 128;
+    float *pml = a.part_ml + ((int64_t)group * wgs_per_group + part) * 4 * 2;
 
     // A operand of QK, broadcast from one block per MFMA: lane (b, i) keeps q[head i] for the
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
@@ -460,15 +463,52 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         tile = tile_next;
     }
 
-    // ---- end of split: write the partial ---------------------------------------------
+    // ---- end of split: the workgroup's wavefronts merge their partials in LDS and write one ------
     const float l_tot = sum_over_blocks(l_run);
+    if (n_waves == 1) {
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf)
+        for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) po[i * 128 + 64 * hf + lane] = acc_o[hf][0][i] + acc_o[hf][1][i];
-    if (lane < 4) {
-        pml[2 * j] = m_run;
-        pml[2 * j + 1] = l_tot;
+            for (int i = 0; i < 4; ++i) po[i * 128 + 64 * hf + lane] = acc_o[hf][0][i] + acc_o[hf][1][i];
+        if (lane < 4) {
+            pml[2 * j] = m_run;
+            pml[2 * j + 1] = l_tot;
+        }
+    } else {
+        // per wavefront: out[4][128], then m[4], l[4]
+        extern __shared__ float merge_s[];
+        constexpr int MS = MERGE_FLOATS;
+        float *mine = merge_s + wave * MS;
+        if (lane < 4) {
+            mine[512 + j] = m_run;
+            mine[516 + j] = l_tot;
+        }
+        __syncthreads();
+        // head j's maximum over the wavefronts that saw an unmasked position
+        float M = -INFINITY;
+        for (int w = 0; w < n_waves; ++w)
+            if (merge_s[w * MS + 516 + j] > 0.0f) M = fmaxf(M, merge_s[w * MS + 512 + j]);
+        const float f = l_tot > 0.0f ? __builtin_amdgcn_exp2f(m_run - M) : 0.0f;
+        const float f4[4] = {dpp<0x00>(f), dpp<0x55>(f), dpp<0xAA>(f), dpp<0xFF>(f)};
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[i * 128 + 64 * hf + lane] = (acc_o[hf][0][i] + acc_o[hf][1][i]) * f4[i];
+        __syncthreads();
+        for (int e = tid; e < 512; e += 64 * n_waves) {
+            float sum = 0.0f;
+            for (int w = 0; w < n_waves; ++w) sum += merge_s[w * MS + e];
+            po[e] = sum;
+        }
+        if (tid < 4) {  // lanes 0..3 of wavefront 0 hold heads 0..3
+            float L = 0.0f;
+            for (int w = 0; w < n_waves; ++w) {
+                const float lw = merge_s[w * MS + 516 + j];
+                if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(merge_s[w * MS + 512 + j] - M), L);
+            }
+            pml[2 * j] = M;
+            pml[2 * j + 1] = L;
+        }
     }
     if constexpr (SPARSE) {
         // one device-wide atomic per workgroup: thousands of wavefronts finishing together on one address
@@ -495,7 +535,6 @@ __global__ void k_clear_skip(unsigned long long *skip, unsigned long long total_
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
                                                           int64_t n_rows, int n_splits, const float *s1, const float *s2) {
-    __shared__ float red[NW][130];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t r = blockIdx.x;  // row = group*4 + head
     const int64_t group = r >> 2;
@@ -530,6 +569,7 @@ __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, c
             o1 = fmaf(v.y, wt, o1);
         }
     }
+    __shared__ float red[NW][130];
     red[wv][2 * lane] = o0;
     red[wv][2 * lane + 1] = o1;
     __syncthreads();
@@ -547,6 +587,47 @@ __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, c
     wht128_wave(o0, o1, lane);
     out[r * 128 + 2 * lane] = o0 * (s1[2 * lane] * RSQRT128);
     out[r * 128 + 2 * lane + 1] = o1 * (s1[2 * lane + 1] * RSQRT128);
+}
+
+// the same merge for at most four partials per row: one wavefront per row, every load issued before
+// anything is waited for (one trip to memory instead of three)
+__global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, const float *part_ml, float *out, int64_t n_rows,
+                                                          int n_parts, const float *s1, const float *s2) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
+    if (r >= n_rows) return;
+    const int64_t group = r >> 2;
+    const int head = (int)(r & 3);
+    const float *ml = part_ml + (group * n_parts * 4 + head) * 2;   // + p*8
+    const float *po = part_o + (group * n_parts * 4 + head) * 128;  // + p*512
+    float m[4], l[4];
+    float2 v[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int pc = p < n_parts ? p : 0;
+        m[p] = ml[pc * 8];
+        l[p] = p < n_parts ? ml[pc * 8 + 1] : 0.0f;
+        v[p] = *reinterpret_cast<const float2 *>(po + (int64_t)pc * 512 + 2 * lane);
+    }
+    const float2 s1v = *reinterpret_cast<const float2 *>(s1 + 2 * lane);
+    const float2 s2v = *reinterpret_cast<const float2 *>(s2 + 2 * lane);
+    float M = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+        if (l[p] > 0.0f) M = fmaxf(M, m[p]);
+    float L = 0.0f, o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const float w = l[p] > 0.0f ? exp2f(m[p] - M) : 0.0f;
+        L = fmaf(l[p], w, L);
+        o0 = fmaf(v[p].x, w, o0);
+        o1 = fmaf(v[p].y, w, o1);
+    }
+    const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+    o0 *= invL * s2v.x;
+    o1 *= invL * s2v.y;
+    wht128_wave(o0, o1, lane);
+    *reinterpret_cast<float2 *>(out + r * 128 + 2 * lane) = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
 }
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -633,9 +714,11 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     while (p->n_splits % wpw) wpw >>= 1;
     const unsigned grid = (unsigned)((int64_t)groups * (p->n_splits / wpw));
     const unsigned wg = 64u * (unsigned)wpw;
+    const int n_parts = p->n_splits / wpw;  // partials per group: the wavefronts of a workgroup merge theirs in LDS
+    const size_t merge_bytes = wpw > 1 ? (size_t)wpw * MERGE_FLOATS * sizeof(float) : 0;
     const int vb = hv->bits;
     const int kb = turbo_k ? hk->bits : 8;
-#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, 0, s>>>(a)
+#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, merge_bytes, s>>>(a)
 #define TQ_ATTN(KF, KB, VB)                         \
     if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
     else TQ_ATTN_ONE(KF, KB, VB, false, false)
@@ -662,9 +745,10 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 #undef TQ_ATTN_ONE
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
-    // many splits: sixteen wavefronts share a row's partials
-    if (p->n_splits >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
-    else k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, p->n_splits, hv->s1_32, hv->s2_32);
+    // many partials: sixteen wavefronts share a row's
+    if (n_parts >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
+    else if (n_parts > 4) k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
+    else k_attn_combine_few<<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
     return tq_check_launch("attn_combine");
 }
 
