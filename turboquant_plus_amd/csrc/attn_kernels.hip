@@ -152,7 +152,7 @@ struct AttnArgs {
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
     float *part_o;                // [groups][workgroups per group][4][128]
     float *part_ml;               // [groups][workgroups per group][4][2]  (m in log2 units, l)
-    unsigned long long *skip;     // [0] += skipped (query, position) pairs
+    unsigned long long *skip_slots;  // Sparse V: [workgroup] (query, position) pairs it skipped
     int64_t tokens, blocks_per_seq;
     int n_groups, n_splits, tiles_per_split, n_tiles;
     float tau;
@@ -511,21 +511,38 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         }
     }
     if constexpr (SPARSE) {
-        // one device-wide atomic per workgroup: thousands of wavefronts finishing together on one address
-        // would queue for longer than the kernel's own tail
+        // one slot per workgroup, added up by the merge kernel: thousands of wavefronts finishing together
+        // on one atomic would queue for longer than the kernel's own tail, and nothing needs clearing
         unsigned tot = nskip;
         for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
         if (lane == 0 && tot) atomicAdd(&skipped, tot);
         __syncthreads();
-        if (tid == 0 && skipped) atomicAdd(a.skip, (unsigned long long)skipped);
+        if (tid == 0) a.skip_slots[blockIdx.x] = skipped;
     }
 }
 
-// Sparse-V bookkeeping: {skipped pairs, total pairs}; a fill kernel rather than a memset so that
-// the sequence stays safe to capture in a HIP graph.
-__global__ void k_clear_skip(unsigned long long *skip, unsigned long long total_pairs) {
-    skip[0] = 0ull;
-    skip[1] = total_pairs;
+// Sparse-V bookkeeping, done by the first workgroup of the merge kernel: skip[0] = the sum of the decode
+// workgroups' slots (none for a dense step), skip[1] = all (query, position) pairs.
+struct SkipArgs {
+    const unsigned long long *slots;
+    int n_slots;
+    unsigned long long *skip;  // NULL: no bookkeeping asked for
+    unsigned long long total_pairs;
+};
+__device__ __forceinline__ void sum_skip_slots(const SkipArgs &k) {
+    if (!k.skip || blockIdx.x != 0) return;
+    __shared__ unsigned long long acc;
+    if (threadIdx.x == 0) acc = 0ull;
+    __syncthreads();
+    unsigned long long t = 0ull;
+    for (int i = (int)threadIdx.x; i < k.n_slots; i += (int)blockDim.x) t += k.slots[i];
+    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
+    if ((threadIdx.x & 63) == 0 && t) atomicAdd(&acc, t);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        k.skip[0] = acc;
+        k.skip[1] = k.total_pairs;
+    }
 }
 
 // merge split partials, un-rotate with the V rotation's transpose; one workgroup of NW (4 or 16)
@@ -534,7 +551,9 @@ __global__ void k_clear_skip(unsigned long long *skip, unsigned long long total_
 // its share of the splits with independent loads, and wavefront 0 adds the shares.
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
-                                                          int64_t n_rows, int n_splits, const float *s1, const float *s2) {
+                                                          int64_t n_rows, int n_splits, const float *s1, const float *s2,
+                                                          SkipArgs sk) {
+    sum_skip_slots(sk);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t r = blockIdx.x;  // row = group*4 + head
     const int64_t group = r >> 2;
@@ -592,7 +611,8 @@ __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, c
 // the same merge for at most four partials per row: one wavefront per row, every load issued before
 // anything is waited for (one trip to memory instead of three)
 __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, const float *part_ml, float *out, int64_t n_rows,
-                                                          int n_parts, const float *s1, const float *s2) {
+                                                          int n_parts, const float *s1, const float *s2, SkipArgs sk) {
+    sum_skip_slots(sk);
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
     if (r >= n_rows) return;
@@ -633,7 +653,7 @@ __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, c
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 struct WsLayout {
-    int64_t qrot, part_o, part_ml, total;
+    int64_t qrot, part_o, part_ml, skip_slots, total;
 };
 WsLayout ws_layout(const tq_attn_params *p) {
     const int64_t rows = (int64_t)p->batch * p->n_q_heads;
@@ -642,7 +662,8 @@ WsLayout ws_layout(const tq_attn_params *p) {
     w.qrot = 0;
     w.part_o = align256(rows * 128 * 2);
     w.part_ml = w.part_o + align256(groups * p->n_splits * 4 * 128 * 4);
-    w.total = w.part_ml + align256(groups * p->n_splits * 4 * 2 * 4);
+    w.skip_slots = w.part_ml + align256(groups * p->n_splits * 4 * 2 * 4);
+    w.total = w.skip_slots + align256(groups * p->n_splits * 8);
     return w;
 }
 
@@ -667,11 +688,6 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     const float sc = p->scale * LOG2E;
     const unsigned long long total_pairs = (unsigned long long)rows * (unsigned long long)p->tokens;
     int rc = TQ_OK;
-    if (skip_count) {
-        k_clear_skip<<<1, 1, 0, s>>>(skip_count, total_pairs);
-        rc = tq_check_launch("clear_skip");
-        if (rc) return rc;
-    }
     if (q_dtype != TQ_F16 && q_dtype != TQ_F32 && q_dtype != TQ_F64) {
         tq_set_error("bad q dtype %d", q_dtype);
         return TQ_ERR_ARG;
@@ -692,7 +708,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.bias = bias;
     a.part_o = part_o;
     a.part_ml = part_ml;
-    a.skip = skip_count;
+    a.skip_slots = reinterpret_cast<unsigned long long *>((char *)ws + w.skip_slots);
     if (p->tokens >= ((int64_t)1 << 31)) {
         tq_set_error("tq_decode_attention: tokens %lld beyond 2^31 - 1", (long long)p->tokens);
         return TQ_ERR_UNSUPPORTED;
@@ -746,9 +762,14 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
     // many partials: sixteen wavefronts share a row's
-    if (n_parts >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
-    else if (n_parts > 4) k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
-    else k_attn_combine_few<<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32);
+    SkipArgs sk;
+    sk.slots = a.skip_slots;
+    sk.n_slots = sparse ? (int)grid : 0;
+    sk.skip = skip_count;
+    sk.total_pairs = total_pairs;
+    if (n_parts >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
+    else if (n_parts > 4) k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
+    else k_attn_combine_few<<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
     return tq_check_launch("attn_combine");
 }
 
