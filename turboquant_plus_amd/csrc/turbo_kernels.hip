@@ -413,7 +413,8 @@ __device__ __forceinline__ uint32_t take_ticket(uint32_t *counter, int lane) {
 
 template <int BITS, bool RAGGED>
 __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
-                                              uint32_t end, uint32_t *counter, const uint2 *qlut) {
+                                              uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
+                                              const uint32_t *flips) {
     constexpr int NT = 1 << (BITS - 1);
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kc = lane >> 4;
@@ -425,10 +426,10 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     }
     half8_t af[8];
 #pragma unroll
-    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, a.afrag[f * 64 + lane]);
+    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
     uint32_t flip[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) flip[j] = a.s2flip[kc * 4 + j];
+    for (int j = 0; j < 4; ++j) flip[j] = flips[kc * 4 + j];
 
     const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
     // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
@@ -738,10 +739,14 @@ struct StoreVArgs {
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
 };
 
-// Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.
-template <int BITS, bool RAGGED>
+// Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.  The first
+// ticket is the caller's (the counter starts past the tickets given out this way), so the first tile's
+// input is requested before anything is waited for; `stage` then makes the workgroup's copy of the
+// constant operands (frag, s2: LDS) readable.
+template <int BITS, bool RAGGED, typename Stage>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
-                                              uint32_t end, uint32_t *counter, const uint2 *qlut) {
+                                              uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
+                                              const float *s2, uint32_t first_ticket, Stage &&stage) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
     const int tid = threadIdx.x, lane = tid & 63;
@@ -752,14 +757,6 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
         thr0[k] = a.symthr[k];
         coef[k] = a.sqcoef[k];
     }
-    half8_t bf[8];
-#pragma unroll
-    for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, a.bfrag[f * 64 + lane]);
-    bool s2pos[4][2];
-#pragma unroll
-    for (int dd = 0; dd < 4; ++dd)
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = a.s2[64 * hf + 16 * dd + n16] > 0.0f;
     // an exact zero counts as positive only if the middle boundary is below zero
     const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
 
@@ -788,9 +785,27 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 
     uint4 xq[2][4];
     bool xvalid[2];
-    uint32_t unit = lo + step * take_ticket(counter, lane);
-    fetch(unit, 3, xq[0], xvalid[0]);
-    fetch(unit, 2, xq[1], xvalid[1]);
+    uint32_t unit = lo + step * first_ticket;
+    // Only one wavefront per SIMD asks for its input before the constants: when every wavefront of the chip
+    // asks at once, the burst takes several microseconds to serve and nobody computes until it is through.
+    const bool early = first_ticket < 4;
+    if (early) {
+        fetch(unit, 3, xq[0], xvalid[0]);
+        fetch(unit, 2, xq[1], xvalid[1]);
+    }
+    stage();
+    if (!early) {
+        fetch(unit, 3, xq[0], xvalid[0]);
+        fetch(unit, 2, xq[1], xvalid[1]);
+    }
+    half8_t bf[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
+    bool s2pos[4][2];
+#pragma unroll
+    for (int dd = 0; dd < 4; ++dd)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = s2[64 * hf + 16 * dd + n16] > 0.0f;
 
 #pragma unroll 1
     for (; unit < end;) {
@@ -956,27 +971,47 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 
 __device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g) { return (uint32_t)((uint64_t)n * b / g); }
 
+// The +-1 operand fragments and sign tables are the same for every wavefront: a workgroup fetches them once
+// into LDS (thousands of wavefronts asking the L2 for the same 8 KB delayed the start by several microseconds).
+
 // single tensor: fixed strided share per wavefront (four workgroups of four wavefronts per CU for K, three for V)
 template <int BITS, bool RAGGED>
 __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
     __shared__ uint32_t counter[4];
     __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ uint32_t flip_s[16];
+    const int t = threadIdx.x, wave = t >> 6;
+    const uint4 c0 = a.afrag[t], c1 = a.afrag[256 + t];
+    const uint32_t c3 = a.s2flip[t & 15];
+    if ((t & 63) == 0) counter[wave] = 0;
     if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
+    frag_s[t] = c0;
+    frag_s[256 + t] = c1;
+    if (t < 16) flip_s[t] = c3;
     __syncthreads();
-    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut);
+    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, flip_s);
 }
 
 template <int BITS, bool RAGGED>
 __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
     __shared__ uint32_t counter[4];
     __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) counter[wave] = 0;
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ float s2_s[128];
+    const int t = threadIdx.x, wave = t >> 6;
+    const uint4 c0 = a.bfrag[t], c1 = a.bfrag[256 + t];
+    const float c2 = a.s2[t & 127];
+    if ((t & 63) == 0) counter[wave] = 1;  // ticket 0 is taken without asking
     if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
-    __syncthreads();
-    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut);
+    auto stage = [&] {
+        frag_s[t] = c0;
+        frag_s[256 + t] = c1;
+        if (t < 128) s2_s[t] = c2;
+        __syncthreads();
+    };
+    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
+                                stage);
 }
 
 // K and V of one layer in one launch, one workgroup of 12 wavefronts per CU owning an equal
@@ -989,14 +1024,29 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
     __shared__ uint32_t counter[2];
     __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 4096 : 2];
     __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 4096 : 2];
-    if (threadIdx.x < 2) counter[threadIdx.x] = 0;
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[1024];  // V fragments, then K fragments
+    __shared__ float s2_s[128];
+    __shared__ uint32_t flip_s[16];
+    const int t = threadIdx.x;
+    const uint4 c0 = t < 512 ? va.bfrag[t] : ka.afrag[t - 512];
+    const uint4 c1 = ka.afrag[256 + (t & 255)];
+    const float c2 = va.s2[t & 127];
+    const uint32_t c3 = ka.s2flip[t & 15];
+    if (t < 2) counter[t] = t == 0 ? 12u : 0u;  // V: the wavefronts' first tickets are their own numbers
     if constexpr (KB == 4) load_quant_lut<768>(qlut_k, ka.quant_lut);
     if constexpr (VB == 4) load_quant_lut<768>(qlut_v, va.quant_lut);
-    __syncthreads();
+    auto stage = [&] {
+        frag_s[t] = c0;
+        if (t < 256) frag_s[768 + t] = c1;
+        if (t < 128) s2_s[t] = c2;
+        if (t < 16) flip_s[t] = c3;
+        __syncthreads();
+    };
     store_v_units<VB, RAGGED>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v);
+                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v, frag_s, s2_s,
+                              (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
     store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k);
+                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s);
 }
 
 // ---- K2: fused quantise + pack ---------------------------------------------------
