@@ -411,10 +411,14 @@ __device__ __forceinline__ uint32_t take_ticket(uint32_t *counter, int lane) {
     return __builtin_amdgcn_readfirstlane(t);
 }
 
-template <int BITS, bool RAGGED>
+constexpr uint32_t DRAW_TICKET = 0xFFFFFFFFu;
+// first_ticket: the wavefront's first two tickets are first_ticket and first_ticket + 1 (the counter starts past
+// them), or DRAW_TICKET to draw them.  `stage` makes the workgroup's LDS copy of the constant operands (frag,
+// flips) readable; it runs after the first inputs have been requested.
+template <int BITS, bool RAGGED, typename Stage>
 __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
-                                              const uint32_t *flips) {
+                                              const uint32_t *flips, uint32_t first_ticket, Stage &&stage) {
     constexpr int NT = 1 << (BITS - 1);
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kc = lane >> 4;
@@ -424,12 +428,6 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
         thr0[k] = a.symthr[k];
         coef[k] = a.sqcoef[k];
     }
-    half8_t af[8];
-#pragma unroll
-    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
-    uint32_t flip[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) flip[j] = flips[kc * 4 + j];
 
     const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
     // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
@@ -463,9 +461,16 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     uint32_t cur[DEPTH];
 #pragma unroll
     for (int r = 0; r < DEPTH; ++r) {
-        cur[r] = lo + step * take_ticket(counter, lane);
+        cur[r] = lo + step * (first_ticket == DRAW_TICKET ? take_ticket(counter, lane) : first_ticket + r);
         fetch(cur[r], xq[r], xvalid[r]);
     }
+    stage();
+    half8_t af[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
+    uint32_t flip[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) flip[j] = flips[kc * 4 + j];
 
 #pragma unroll 1
     for (bool more = true; more;) {
@@ -977,20 +982,31 @@ __device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g)
 // single tensor: fixed strided share per wavefront (four workgroups of four wavefronts per CU for K, three for V)
 template <int BITS, bool RAGGED>
 __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
+    // measured at 262 144 vectors: the LDS copy of the constants gains 1.6 us with 4-bit codes and 0.3 us with
+    // 2-bit codes and loses 1.1 us with 3-bit codes, whose wavefronts then read them from memory themselves
+    constexpr bool STAGED = BITS != 3;
     __shared__ uint32_t counter[4];
     __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
-    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[STAGED ? 512 : 1];
     __shared__ uint32_t flip_s[16];
     const int t = threadIdx.x, wave = t >> 6;
-    const uint4 c0 = a.afrag[t], c1 = a.afrag[256 + t];
-    const uint32_t c3 = a.s2flip[t & 15];
-    if ((t & 63) == 0) counter[wave] = 0;
-    if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
-    frag_s[t] = c0;
-    frag_s[256 + t] = c1;
-    if (t < 16) flip_s[t] = c3;
-    __syncthreads();
-    store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, flip_s);
+    if ((t & 63) == 0) counter[wave] = 2;  // tickets 0 and 1 are taken without asking
+    if constexpr (STAGED) {
+        const uint4 c0 = a.afrag[t], c1 = a.afrag[256 + t];
+        const uint32_t c3 = a.s2flip[t & 15];
+        if constexpr (BITS == 4) load_quant_lut<256>(qlut, a.quant_lut);
+        auto stage = [&] {
+            frag_s[t] = c0;
+            frag_s[256 + t] = c1;
+            if (t < 16) flip_s[t] = c3;
+            __syncthreads();
+        };
+        store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s,
+                                    flip_s, 0u, stage);
+    } else {
+        store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, a.afrag,
+                                    a.s2flip, 0u, [] {});
+    }
 }
 
 template <int BITS, bool RAGGED>
@@ -1046,7 +1062,8 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
                               wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v, frag_s, s2_s,
                               (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
     store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s);
+                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s,
+                              DRAW_TICKET, [] {});
 }
 
 // ---- K2: fused quantise + pack ---------------------------------------------------
