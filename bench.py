@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0
 D = 128
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the reading of a
 # 1 GiB device copy (x2.000 and x1.000); figures and commands in profiles/bench_kernels_c2_c3.txt.
-TRAFFIC_BYTES = {"store4": 171.8e6, "store3": 163.0e6, "decode3": 432.9e6}
+TRAFFIC_BYTES = {"store4": 171.5e6, "store3": 161.8e6, "decode3": 423.5e6}
 METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
 
 
