@@ -29,6 +29,7 @@ host cores over a stated sample of the same workload.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -71,6 +72,37 @@ def time_steps(torch, step, steps, warmup):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
     return wall, e0.elapsed_time(e1) / steps
+
+
+def measured_peaks_leg(torch, tqa, steps, warmup):
+    """What this box sustains on plain streaming kernels (1 GiB, two buffer sets) and on back-to-back fp16
+    MFMAs, timed like the legs below; set beside the published peaks the fractions are quoted against."""
+    n = 1 << 30
+    bufs = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(4)]
+    for b in bufs:
+        b.zero_()
+    out = {"bytes_per_launch": n}
+    reps, warm = max(20, steps // 10), max(10, warmup // 10)
+    for mode in ("read", "write", "copy"):
+        best = 0.0
+        for chunked in (False, True):   # lanes striding over the whole buffer, or one contiguous slice per workgroup
+            def step(i):
+                src, dst = bufs[2 * (i % 2)], bufs[2 * (i % 2) + 1]
+                tqa.probe_stream(mode, None if mode == "write" else src, None if mode == "read" else dst, chunked)
+            _, ev_ms = time_steps(torch, step, reps, warm)
+            moved = n * (2 if mode == "copy" else 1)
+            best = max(best, moved / (ev_ms * 1e-3) / 1e9)
+        out[f"hbm_{mode}_gbs"] = best   # the better of the two access orders
+    del bufs
+    sink = torch.zeros(4, dtype=torch.float32, device="cuda")
+    flops = [0]
+
+    def mstep(i):
+        flops[0] = tqa.probe_mfma_f16(2000, sink)
+    _, ev_ms = time_steps(torch, mstep, reps, warm)
+    out["mfma_f16_tflops"] = flops[0] / (ev_ms * 1e-3) / 1e12
+    out["published"] = {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": 2500.0}
+    return out
 
 
 def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
@@ -185,17 +217,35 @@ def asym_decode_leg(torch, tqa, steps, warmup):
     bias = torch.zeros((B, Hq, N), dtype=torch.float32, device="cuda")
     pos = torch.stack([torch.randperm(N, generator=g, device="cuda")[:64] for _ in range(B * Hq)]).view(B, Hq, 64)
     bias.scatter_(2, pos, 6.0)
+    # fraction of (batch, q-head, position) whose final softmax weight is below tau (the definition of the
+    # reference's scripts/measure_skip_rate.py:69-74), from the stored K in fp32
+    below, scale = 0, 1.0 / math.sqrt(D)
+    for s in range(B * Hkv):
+        qi, sc = tqa.q8_0_unpack(kq[s * perk:(s + 1) * perk], 1, N)
+        kd = (qi.view(N, 4, 32).float() * sc.view(N, 4, 1)).view(N, D)
+        b, h = divmod(s, Hkv)
+        logit = q[b, 4 * h:4 * h + 4].float() @ kd.t() * scale + bias[b, 4 * h:4 * h + 4]
+        below += int((torch.softmax(logit, dim=-1) < 1e-6).sum())
+        del qi, sc, kd, logit
+    final_weight_skip = below / float(B * Hq * N)
     out = {}
-    for name, tau in (("dense", 0.0), ("sparse_v", 1e-6)):
+    q_peaked = (q.float() * 16.0).to(torch.float16)  # a second input for Sparse V: logits 16 x as spread, few tiles matter
+    for name, tau, qq in (("dense", 0.0, q), ("sparse_v", 1e-6, q), ("sparse_v_peaked_queries", 1e-6, q_peaked)):
         attn = tqa.DecodeAttention(None, vc, B, Hq, Hkv, N, sparse_v_tau=tau)
-        wall_ms, ev_ms = time_steps(torch, lambda i: attn(q, kq, vp, bias=bias), steps, warmup)
+        wall_ms, ev_ms = time_steps(torch, lambda i: attn(qq, kq, vp, bias=bias), steps, warmup)
         skip = attn.skip_rate() if tau else 0.0
         algo = B * Hkv * N * (136 + (1.0 - 0.0) * 34)  # dense bytes; Sparse V skips whole 64-token V tiles only
         us = ev_ms * 1e3
         out[name] = {"us_per_step": us, "skip_rate": skip, "n_splits": attn.params.n_splits,
                      "achieved_gbs": algo / (us * 1e-6) / 1e9, "frac": algo / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        if tau and qq is q:
+            # the kernel tests exp(logit - running maximum of its split), without the softmax denominator
+            out[name]["skip_rate_final_weight"] = final_weight_skip
+        if tau:
+            out[name]["bytes_required"] = B * Hkv * N * (136 + (1.0 - skip) * 34)
     out["workload"] = ("decode attention, K q8_0-style + V turbo2, B4 Hq32 Hkv8 ctx 131072, +6 bias on 64 key "
-                       "positions per head as an fp32 bias input (67 MB, not counted), Sparse V tau 1e-6")
+                       "positions per head as an fp32 bias input (67 MB, not counted), Sparse V tau 1e-6; "
+                       "sparse_v_peaked_queries: the same cache with the queries scaled x16")
     out["algorithmic_bytes_per_step"] = B * Hkv * N * 170
     return out
 
@@ -222,6 +272,10 @@ def score_tile_leg(torch, tqa, steps, warmup):
                      "mfma_frac_of_2500": flops / (ev_ms * 1e-3) / 2.5e15,
                      "logit_store_gbs": logits.numel() * logits.element_size() / (ev_ms * 1e-3) / 1e9}
         if dt == torch.float32:
+            _, dry_ms = time_steps(torch, lambda i: codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt, store=False),
+                                   max(5, steps // 10), max(2, warmup // 10))
+            out["no_store"] = {"us_per_call": dry_ms * 1e3, "mfma_tflops": flops / (dry_ms * 1e-3) / 1e12,
+                               "mfma_frac_of_2500": flops / (dry_ms * 1e-3) / 2.5e15}
             exact = qs[:256].float() @ keys.t()
             err = logits[:256] - exact
             out["estimator_bias"] = float(err.mean())
@@ -306,6 +360,8 @@ def main():
     asym = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
     torch.cuda.empty_cache()
     tile = score_tile_leg(torch, tqa, args.steps, args.warmup)
+    torch.cuda.empty_cache()
+    peaks = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
     if args.skip_cpu:
         cpu_store = cpu_attn = None
     else:
@@ -324,7 +380,7 @@ def main():
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
         "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec, "asym_decode_q8k_turbo2v": asym,
-        "score_tile": tile,
+        "score_tile": tile, "measured_peaks": peaks,
     }
     print(json.dumps(line, ensure_ascii=False))
 

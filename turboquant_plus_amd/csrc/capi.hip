@@ -576,7 +576,7 @@ int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, co
                   void *workspace, int64_t workspace_bytes, void *stream) {
     int rc = check_fast(h, "tq_score_tile");
     if (rc) return rc;
-    REQUIRE(q && packed && sign_bits && rnorms_f16 && logits && workspace && nq >= 0 && nk >= 0, TQ_ERR_ARG,
+    REQUIRE(q && packed && sign_bits && rnorms_f16 && workspace && nq >= 0 && nk >= 0, TQ_ERR_ARG,
             "tq_score_tile: bad argument");
     REQUIRE(h->has_proj, TQ_ERR_ARG, "tq_score_tile: handle has no projection");
     REQUIRE(out_dtype == TQ_F32 || out_dtype == TQ_F16, TQ_ERR_ARG, "tq_score_tile: logits must be fp32 or fp16");

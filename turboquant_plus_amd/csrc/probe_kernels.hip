@@ -1,0 +1,103 @@
+// Measurement probes: what this part sustains on plain streaming and on back-to-back MFMAs, so that
+// roofline fractions can be stated against measured figures as well as against the published peaks.
+// Not part of the codec; the callers time the launches themselves.
+#include "tq_device.h"
+#include "tq_internal.h"
+
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// mode 0: read, 1: write, 2: copy; 16 bytes per lane and step.  CHUNKED: every workgroup a contiguous slice,
+// else all lanes of the grid stride over the buffer.
+template <int MODE, bool CHUNKED>
+__global__ __launch_bounds__(512) void k_probe_stream(const uint4 *src, uint4 *dst, int64_t n16) {
+    const int64_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const int64_t lo = CHUNKED ? (int64_t)blockIdx.x * per : (int64_t)blockIdx.x * 512;
+    const int64_t hi = CHUNKED ? (lo + per < n16 ? lo + per : n16) : n16;
+    const int64_t step = CHUNKED ? 512 : (int64_t)gridDim.x * 512;
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    const uint4 fill = make_uint4(threadIdx.x, 1u, 2u, 3u);
+    for (int64_t i = lo + threadIdx.x; i < hi; i += step) {
+        if constexpr (MODE == 0) {
+            const uint4 v = src[i];
+            acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+        } else if constexpr (MODE == 1) {
+            dst[i] = fill;
+        } else {
+            dst[i] = src[i];
+        }
+    }
+    // keeps the reads alive; the condition does not hold for any data a caller would pass
+    if constexpr (MODE == 0) {
+        if ((acc.x & acc.y & acc.z & acc.w) == 0xFFFFFFFFu && dst) dst[0] = acc;
+    }
+}
+
+// 8 independent accumulator tiles per wavefront, `iters` rounds of one MFMA on each
+__global__ __launch_bounds__(256) void k_probe_mfma(int64_t iters, float *sink) {
+    const int lane = threadIdx.x & 63;
+    half8_t a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (_Float16)(0.001f * (float)((lane + e) & 7));
+        b[e] = (_Float16)(0.002f * (float)((lane * 3 + e) & 7));
+    }
+    float16_t acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.0f;
+    for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[t], 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[t][e];
+    if (s == -1.0f) sink[0] = s;  // sums of non-negative products: never taken, keeps the MFMAs alive
+}
+
+constexpr int PROBE_MFMA_WGS = 2048;  // 8 workgroups of 4 wavefronts per CU
+
+}  // namespace
+
+extern "C" int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (mode < 0 || mode > 2 || bytes < 16 || (bytes & 15) || (mode != 1 && !src) || (mode != 0 && !dst)) {
+        tq_set_error("tq_probe_stream: mode %d, %lld bytes (a multiple of 16), src %p, dst %p", mode, (long long)bytes, src, dst);
+        return TQ_ERR_ARG;
+    }
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) {
+        tq_set_error("tq_probe_stream: src and dst must be 16-byte aligned");
+        return TQ_ERR_ALIGN;
+    }
+    const int64_t n16 = bytes / 16;
+    const unsigned grid = 256 * 4;
+    const uint4 *s4 = (const uint4 *)src;
+    uint4 *d4 = (uint4 *)dst;
+    if (chunked) {
+        if (mode == 0) k_probe_stream<0, true><<<grid, 512, 0, s>>>(s4, d4, n16);
+        else if (mode == 1) k_probe_stream<1, true><<<grid, 512, 0, s>>>(nullptr, d4, n16);
+        else k_probe_stream<2, true><<<grid, 512, 0, s>>>(s4, d4, n16);
+    } else {
+        if (mode == 0) k_probe_stream<0, false><<<grid, 512, 0, s>>>(s4, d4, n16);
+        else if (mode == 1) k_probe_stream<1, false><<<grid, 512, 0, s>>>(nullptr, d4, n16);
+        else k_probe_stream<2, false><<<grid, 512, 0, s>>>(s4, d4, n16);
+    }
+    return tq_check_launch("probe_stream");
+}
+
+extern "C" int64_t tq_probe_mfma_f16(int64_t iters, float *sink, void *stream) {
+    if (iters < 1 || !sink) {
+        tq_set_error("tq_probe_mfma_f16: iters %lld, sink %p", (long long)iters, (void *)sink);
+        return (int64_t)TQ_ERR_ARG;
+    }
+    k_probe_mfma<<<PROBE_MFMA_WGS, 256, 0, (hipStream_t)stream>>>(iters, sink);
+    const int rc = tq_check_launch("probe_mfma");
+    if (rc) return (int64_t)rc;
+    return (int64_t)PROBE_MFMA_WGS * 4 * iters * 8 * (2ll * 32 * 32 * 16);
+}

@@ -234,17 +234,21 @@ class TurboCodec:
         return out.reshape(xd.shape)
 
     # ---- prefill-shaped inner-product estimator --------------------------------
-    def score_tile(self, q, packed, sign_bits, rnorms, n_keys: int, out_dtype=None):
-        """logits [nq, n_keys] = <R q, g c[idx]> + scale * rnorm * <S q, z>."""
+    def score_tile(self, q, packed, sign_bits, rnorms, n_keys: int, out_dtype=None, store: bool = True):
+        """logits [nq, n_keys] = <R q, g c[idx]> + scale * rnorm * <S q, z>.  store=False runs the
+        computation without writing the logits (a measurement aid) and returns None."""
         tt = L.torch()
         qd = L.to_device(q).reshape(-1, HEAD_DIM)
         nq = qd.shape[0]
         out_dtype = tt.float32 if out_dtype is None else out_dtype
-        logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device)
+        if out_dtype not in (tt.float32, tt.float16):
+            raise TypeError(f"logits must be float32 or float16, not {out_dtype}")
+        logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device) if store else None
         ws = tt.empty(max((nq + 31) // 32 * 32 * 512, 16), dtype=tt.uint8, device=qd.device)
         L.check(L.lib().tq_score_tile(self.handle.h, L.ptr(qd), L.dtype_code(qd), nq, L.ptr(packed), L.ptr(sign_bits),
-                                      L.ptr(rnorms), n_keys, L.ptr(logits), L.dtype_code(logits), L.ptr(ws),
-                                      ws.numel(), L.stream_ptr()))
+                                      L.ptr(rnorms), n_keys, L.ptr(logits) if store else None,
+                                      L.TQ_F16 if out_dtype == tt.float16 else L.TQ_F32,
+                                      L.ptr(ws), ws.numel(), L.stream_ptr()))
         return logits
 
 
@@ -263,6 +267,26 @@ def q8_0_unpack(packed, n_seqs: int, tokens: int):
     s = tt.empty((n_seqs, tokens, 4), dtype=tt.float32, device=packed.device)
     L.check(L.lib().tq_q8_0_unpack(L.ptr(packed), n_seqs, tokens, L.ptr(q), L.ptr(s), L.stream_ptr()))
     return q, s
+
+
+def probe_stream(mode: str, src, dst, chunked: bool = False):
+    """One launch of the streaming probe: "read" src, "write" dst or "copy" src to dst (uint8 device
+    tensors of equal size, a multiple of 16 bytes); chunked gives every workgroup one contiguous slice
+    instead of striding all lanes over the buffer.  The caller times it."""
+    code = {"read": 0, "write": 1, "copy": 2}[mode]
+    ref = dst if src is None else src
+    nbytes = 0 if ref is None else ref.numel()
+    L.check(L.lib().tq_probe_stream(code, int(chunked), None if src is None else L.ptr(src),
+                                    None if dst is None else L.ptr(dst), nbytes, L.stream_ptr()))
+
+
+def probe_mfma_f16(iters: int, sink) -> int:
+    """One launch of the MFMA probe (fp16 32x32x16, eight independent accumulators per wavefront on
+    every SIMD); returns the floating-point operations launched.  sink: a float32 device tensor."""
+    flops = int(L.lib().tq_probe_mfma_f16(iters, L.ptr(sink), L.stream_ptr()))
+    if flops < 0:
+        L.check(flops)
+    return flops
 
 
 class DecodeAttention:
