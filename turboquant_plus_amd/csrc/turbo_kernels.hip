@@ -1456,13 +1456,67 @@ __global__ __launch_bounds__(256) void k_q8_0_store(const TI *x, uint8_t *packed
         for (int j = 0; j < 8; ++j) w[j] = 0;
 #pragma unroll
         for (int j = 0; j < 32; ++j) {
-            const int qv = (int)roundf(v[j] * id);
+            const float tq = v[j] * id;
+            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
             w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
         }
         // 32 values = two 16-byte chunks (2*gq, 2*gq+1) of row t
         *reinterpret_cast<uint4 *>(block + (2 * gq) * 2048 + t * 16) = make_uint4(w[0], w[1], w[2], w[3]);
         *reinterpret_cast<uint4 *>(block + (2 * gq + 1) * 2048 + t * 16) = make_uint4(w[4], w[5], w[6], w[7]);
         reinterpret_cast<__half *>(block + 8 * 2048)[t * 4 + gq] = __float2half_rn(d);
+    }
+}
+
+// fp16 input: the block's 32 KB are read as 16-byte pieces that are contiguous across the lanes (four lanes
+// per 32-value group, whose maximum takes two lane exchanges), the block image is put together in LDS and
+// leaves as one contiguous copy.  Same arithmetic as k_q8_0_store: q = sign(t) floor(|t| + 0.5), t = x / scale.
+constexpr int Q8_LDS_CHUNK = 2048 + 16;  // chunk stride of the LDS image (padding spreads the 8-byte writes over the banks)
+__global__ __launch_bounds__(256) void k_q8_0_store_f16(const __half *x, uint8_t *packed, int64_t tokens, int64_t blocks_per_seq) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[8 * Q8_LDS_CHUNK + TQ_ROWS_PER_BLOCK * 8];
+    const int tid = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const int rows_here = (int)min((int64_t)TQ_ROWS_PER_BLOCK, tokens - tok0);
+    const uint4 *src = reinterpret_cast<const uint4 *>(x + (seq * tokens + tok0) * 128);
+    uint4 v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int i = tid + 256 * r;  // 16-byte piece of the block: row i / 16, values 8 (i % 16) .. + 7
+        v[r] = (i >> 4) < rows_here ? src[i] : make_uint4(0, 0, 0, 0);
+    }
+    __half *scales = reinterpret_cast<__half *>(img + 8 * Q8_LDS_CHUNK);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int i = tid + 256 * r, row = i >> 4, c8 = i & 15;
+        const uint32_t u[4] = {v[r].x, v[r].y, v[r].z, v[r].w};
+        float f[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f[2 * j] = __half2float(__ushort_as_half((unsigned short)(u[j] & 0xffffu)));
+            f[2 * j + 1] = __half2float(__ushort_as_half((unsigned short)(u[j] >> 16)));
+            amax = fmaxf(amax, fmaxf(fabsf(f[2 * j]), fabsf(f[2 * j + 1])));
+        }
+        amax = fmaxf(amax, xor_lane<1>(amax));
+        amax = fmaxf(amax, xor_lane<2>(amax));
+        const float d = amax / 127.0f;
+        const float id = d > 0.0f ? 1.0f / d : 0.0f;
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float t = f[j] * id;
+            const int qv = (int)copysignf(floorf(fabsf(t) + 0.5f), t);
+            w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
+        }
+        *reinterpret_cast<uint2 *>(img + (c8 >> 1) * Q8_LDS_CHUNK + row * 16 + (c8 & 1) * 8) = make_uint2(w[0], w[1]);
+        if ((c8 & 3) == 0) scales[row * 4 + (c8 >> 2)] = __float2half_rn(d);
+    }
+    __syncthreads();
+    uint4 *dst = reinterpret_cast<uint4 *>(packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136));
+    for (int i = tid; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) {
+        const int c = i >> 7;  // chunks 0..7 of 128 pieces each, then the scales
+        dst[i] = *reinterpret_cast<const uint4 *>(c < 8 ? img + c * Q8_LDS_CHUNK + (i & 127) * 16 : img + 8 * Q8_LDS_CHUNK + (i - 1024) * 16);
     }
 }
 
@@ -1914,6 +1968,10 @@ int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, 
     const int64_t bps = blocks_for(tokens);
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
+    if (in_dtype == TQ_F16 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed)) & 15u) == 0) {
+        k_q8_0_store_f16<<<grid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, tokens, bps);
+        return tq_check_launch("q8_0_store");
+    }
     DISPATCH_T(in_dtype, TI, (k_q8_0_store<TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, tokens, bps)));
     return tq_check_launch("q8_0_store");
 }
