@@ -1372,7 +1372,45 @@ struct LoadArgs {
     int64_t tokens, blocks_per_seq;
 };
 
-template <typename TO>
+// The eight codes of dims 8li .. 8li+7 of token t, code m at bit m*BITS.  K rows: the lane's four pairs are
+// one dword of a group (2-bit: half a dword; 3-bit: 24 bits of a dword, or the group's tail).  V rows: the same
+// pair position of eight consecutive rows.
+template <int BITS>
+__device__ __forceinline__ uint32_t load_codes8(const uint8_t *block, int kind, int t, int li) {
+    constexpr uint32_t CM = (1u << BITS) - 1u;
+    if (kind == TQ_KIND_K) {
+        const int g = li >> 2, q = li & 3;
+        if constexpr (BITS == 4) return row_dword(block, t, 4 * q + g);
+        if constexpr (BITS == 2) return (row_dword(block, t, 4 * (q >> 1) + g) >> (16 * (q & 1))) & 0xFFFFu;
+        if constexpr (BITS == 3) {
+            if (q < 3) return row_dword(block, t, 4 * q + g) & 0xFFFFFFu;
+            return (row_dword(block, t, g) >> 24) | ((row_dword(block, t, 4 + g) >> 24) << 8) | ((row_dword(block, t, 8 + g) >> 24) << 16);
+        }
+    }
+    const int r0 = (t & 64) | ((8 * li) & 63);
+    const int p = ((t & 60) | ((li >> 3) << 1)) | ((t >> 1) & 1);
+    const int g = p >> 4, k = p & 15;
+    const int hs = (t & 1) * BITS;
+    uint32_t w = 0;
+    if (BITS == 3 && k >= 12) {
+        const int sh = 6 * (k - 12) + hs;  // bit of the 24-bit tail; byte sh / 8 is the top byte of dword sh / 8
+        // a 3-bit code at tail bit sh may straddle two bytes: assemble the tail from the three top bytes
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint32_t tail = (row_dword(block, r0 + m, g) >> 24) | ((row_dword(block, r0 + m, 4 + g) >> 24) << 8) |
+                                  ((row_dword(block, r0 + m, 8 + g) >> 24) << 16);
+            w |= ((tail >> sh) & CM) << (m * BITS);
+        }
+    } else {
+        const int dw = 4 * (k / tqd::pairs_per_dword(BITS)) + g;
+        const int sh = 2 * BITS * (k % tqd::pairs_per_dword(BITS)) + hs;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) w |= ((row_dword(block, r0 + m, dw) >> sh) & CM) << (m * BITS);
+    }
+    return w;
+}
+
+template <typename TO, int BITS>
 __global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, LoadArgs a) {
     __shared__ float cent_s[16];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1380,15 +1418,15 @@ __global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, Lo
     const int64_t blk = blockIdx.x;
     const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
-    // the block (at most 8448 B) is copied into LDS with coalesced 16-byte loads; codes are picked from there
-    __shared__ __attribute__((aligned(16))) uint8_t block_s[TQ_ROWS_PER_BLOCK * (16 * 4 + 2)];
-    const int block_size = TQ_ROWS_PER_BLOCK * (16 * a.bits + 2);
+    // the block is copied into LDS with coalesced 16-byte loads; codes are picked from there
+    constexpr int block_size = TQ_ROWS_PER_BLOCK * (16 * BITS + 2);
+    __shared__ __attribute__((aligned(16))) uint8_t block_s[block_size];
     {
         const uint4 *src = reinterpret_cast<const uint4 *>(packed + blk * (int64_t)block_size);
         for (int e = tid; e < block_size / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = src[e];
     }
     const uint8_t *block = block_s;
-    if (tid < (1 << a.bits)) cent_s[tid] = a.cent[tid];
+    if (tid < (1 << BITS)) cent_s[tid] = a.cent[tid];
     float s1v[8], s2v[8];
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
@@ -1400,10 +1438,11 @@ __global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, Lo
     for (int it = 0; it < 8; ++it) {
         const int t = it * 16 + grp;
         const bool valid = tok0 + t < a.tokens;
-        const float g = block_norm(block, a.bits, t);
+        const float g = block_norm(block, BITS, t);
+        const uint32_t codes = load_codes8<BITS>(block, a.kind, t, li);
         float v[8];
 #pragma unroll
-        for (int m = 0; m < 8; ++m) v[m] = cent_s[fetch_code(block, a.bits, a.kind, t, 8 * li + m)] * g;
+        for (int m = 0; m < 8; ++m) v[m] = cent_s[(codes >> (m * BITS)) & ((1u << BITS) - 1u)] * g;
         if (a.domain == TQ_DOMAIN_ORIGINAL) {
 #pragma unroll
             for (int m = 0; m < 8; ++m) v[m] *= s2v[m];
@@ -1951,7 +1990,11 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.cent = h->centroids32;
     a.bits = h->bits; a.kind = kind; a.domain = domain;
     a.tokens = tokens; a.blocks_per_seq = bps;
-    DISPATCH_T(out_dtype, TO, (k_load<TO><<<grid, 256, 0, s>>>((const uint8_t *)packed, (TO *)out, a)));
+    switch (h->bits) {
+    case 2: DISPATCH_T(out_dtype, TO, (k_load<TO, 2><<<grid, 256, 0, s>>>((const uint8_t *)packed, (TO *)out, a))); break;
+    case 3: DISPATCH_T(out_dtype, TO, (k_load<TO, 3><<<grid, 256, 0, s>>>((const uint8_t *)packed, (TO *)out, a))); break;
+    default: DISPATCH_T(out_dtype, TO, (k_load<TO, 4><<<grid, 256, 0, s>>>((const uint8_t *)packed, (TO *)out, a))); break;
+    }
     return tq_check_launch("load");
 }
 
