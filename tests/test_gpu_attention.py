@@ -79,6 +79,26 @@ def test_decode_attention_turbo3(N, n_splits):
     np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("n_splits", [16, 3])
+def test_decode_attention_with_unequal_codebooks_of_one_width(bits, n_splits):
+    """K and V of the same width with different centroids cannot share a decode table: both tables and the
+    workgroup's merge space are in LDS at once."""
+    B, Hq, Hkv, N = 2, 8, 2, 2048 + 64
+    rng = np.random.default_rng(bits + n_splits)
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    kc = tqa.TurboCodec(bits, seed=42, centroids=tqa.PRODUCTION_CENTROIDS[bits])
+    vc = tqa.TurboCodec(bits, seed=542)
+    kp, vp = kc.store(k, kind="k"), vc.store(v, kind="v")
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    for tau in (0.0, 1e-4):
+        attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+        out = np_(attn(q, kp, vp))
+        ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau)
+        assert_close(out, ref)
+
+
 @pytest.mark.parametrize("B,Hkv,N,n_splits,capacity", [
     (1, 1, 64, 32, 0),        # one tile, 31 empty splits in a 16-wavefront workgroup
     (1, 2, 200, 16, 0),       # 4 tiles over 16 splits: 12 empty, last tile ragged

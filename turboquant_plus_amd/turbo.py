@@ -201,11 +201,14 @@ class TurboCodec:
                                      L.ptr(bits), L.ptr(rn), L.stream_ptr()))
         return packed, bits, rn
 
-    def load(self, packed, n_seqs: int, tokens: int, kind: str = "k", domain: str = "original", dtype=None):
-        """packed -> [n_seqs, tokens, 128] values in the original or the rotated domain."""
+    def load(self, packed, n_seqs: int, tokens: int, kind: str = "k", domain: str = "original", dtype=None, out=None):
+        """packed -> [n_seqs, tokens, 128] values in the original or the rotated domain (into `out` if given)."""
         tt = L.torch()
-        dtype = tt.float32 if dtype is None else dtype
-        out = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=dtype, device=packed.device)
+        if out is None:
+            dtype = tt.float32 if dtype is None else dtype
+            out = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=dtype, device=packed.device)
+        elif out.numel() != n_seqs * tokens * HEAD_DIM or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous tensor of {n_seqs * tokens * HEAD_DIM} elements")
         L.check(L.lib().tq_load(self.handle.h, L.ptr(packed), n_seqs, tokens, L.KIND_K if kind == "k" else L.KIND_V,
                                 L.ptr(out), L.dtype_code(out),
                                 L.DOMAIN_ORIGINAL if domain == "original" else L.DOMAIN_ROTATED, L.stream_ptr()))
