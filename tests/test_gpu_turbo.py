@@ -175,6 +175,29 @@ def test_load_both_domains(bits, kind):
     assert rel.mean() < 2 * {2: 0.117, 3: 0.03, 4: 0.009}[bits]
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (5, 64)])
+def test_load_fp16_matches_fp32_load(bits, kind, n_seqs, tokens):
+    """fp16 output in the original domain runs the transposed rotation on the matrix cores with fp16
+    centroids; the fp32 output keeps the fp32 butterfly.  Both decode the same codes: they agree to the
+    fp16 tolerance (2e-3 of the vector's largest component), ragged sequence ends included, and the
+    fp16 path writes nothing past its rows."""
+    tt = L.torch()
+    codec = tqa.TurboCodec(bits, seed=11 * bits)
+    x = kv_like(bits + tokens, (n_seqs, tokens, D))
+    x[0, min(3, tokens - 1)] = 0
+    packed = codec.store(x, kind=kind)
+    ref = np_(codec.load(packed, n_seqs, tokens, kind=kind, domain="original")).astype(np.float64)
+    out = tt.full((n_seqs * tokens * D + 64,), 7.0, dtype=tt.float16, device="cuda")
+    codec.load(packed, n_seqs, tokens, kind=kind, domain="original", out=out[:n_seqs * tokens * D])
+    got = np_(out).astype(np.float64)
+    assert (got[n_seqs * tokens * D:] == 7.0).all(), "wrote past the last row"
+    got = got[:n_seqs * tokens * D].reshape(n_seqs, tokens, D)
+    tol = 2e-3 * np.abs(ref).max(axis=-1, keepdims=True) + 1e-7
+    assert np.all(np.abs(got - ref) <= tol)
+
+
 def test_config1_polarquant_turbo3_roundtrip(golden):
     """BASELINE config 1 end to end on the GPU: 4096 fp32 vectors, seed 0, one
     seed-1 sign diagonal, 8-level codebook; indices against the fixture the

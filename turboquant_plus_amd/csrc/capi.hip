@@ -181,6 +181,18 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
             uint16_t *drk = nullptr;
             rc = rc ? rc : upload(&drk, rk);
             h->rfrag16k = drk;
+            // the same fragments for the way back (x = D1 H D2 y / sqrt(128)): the input-side signs are s2
+            for (int f = 0; f < 8; ++f)
+                for (int l = 0; l < 64; ++l)
+                    for (int e = 0; e < 8; ++e) {
+                        const int r = l & 15, f0 = f >> 2, ks = f & 3;
+                        const int m = 32 * (r >> 2) + 4 * f0 + (r & 3), k = 32 * (l >> 4) + 8 * ks + e;
+                        const double v = s2[k] * ((__builtin_popcount(m & k) & 1) ? -1.0 : 1.0);
+                        rk[((size_t)f * 64 + l) * 8 + e] = v < 0 ? 0xBC00 : 0x3C00;
+                    }
+            uint16_t *dri = nullptr;
+            rc = rc ? rc : upload(&dri, rk);
+            h->rfrag16k_inv = dri;
             for (int f = 0; f < 8; ++f)
                 for (int l = 0; l < 64; ++l)
                     for (int e = 0; e < 8; ++e) {
@@ -283,7 +295,8 @@ void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
                     h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
-                    h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v, h->quant_lut};
+                    h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v, h->quant_lut,
+                    h->rfrag16k_inv};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete h;

@@ -33,6 +33,7 @@ struct tq_handle {
     float *projT32;        // [128*128] entry [k*128+j] = S[j][k]  (query projection, score tile)
     void *rfrag16k;        // [8][64][8] fp16 +-1: fragment f0*4+ks, lane l, element e = s1[k] H[m][k] with
                            // m = 32(l%16/4) + 4 f0 + l%4, k = 32(l/16) + 8 ks + e (factored transform, K rows)
+    void *rfrag16k_inv;    // rfrag16k with s2 in place of s1: the transposed rotation of K-row-shaped data (tq_load)
     void *rfrag16v;        // [8][64][8] fp16 +-1: fragment d0*4+ks, lane l, element e = s1[k] H[16 d0 + l%16][k],
                            // k = 32 ks + 8(l/16) + e (factored transform, V rows: B operand)
     uint32_t *s2flip;      // [4][4]: per lane quarter and output dword, sign-field positions of dims with s2 = +1

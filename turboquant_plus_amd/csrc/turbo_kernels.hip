@@ -1454,6 +1454,211 @@ __global__ __launch_bounds__(256) void k_load(const uint8_t *packed, TO *out, Lo
     }
 }
 
+// ---- tq_load, K rows, fp16 output, original domain: the transposed rotation on the matrix cores ----------
+// The mirror image of store_k_units: a lane quarter's BITS dwords of a row are one pair group = 32 consecutive
+// rotated-domain values of one token, which is the B operand of the factored transform (fragments with s2
+// folded in); the 32 results of the lane are 32 consecutive output dims.  The centroids enter as fp16 (the pair
+// table), which the fp16 output's tolerance covers; fp32 and fp64 outputs keep the fp32 butterfly of k_load.
+struct LoadK16Args {
+    const uint4 *afrag;        // tq_handle::rfrag16k_inv
+    const float *s1;
+    const uint32_t *pair_lut;  // half2 per pair code
+    int64_t tokens;
+    uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
+};
+
+// byte offset (pair code * 4) of pair k = 0..15 of a group, from the group's dwords (3-bit: and its 24-bit tail)
+template <int BITS> __device__ __forceinline__ uint32_t group_pair_offset(const uint32_t (&cw)[BITS], uint32_t tail, int k) {
+    if constexpr (BITS == 4) return tqd::field_offset<2>(cw[k >> 2], 8 * (k & 3), 8);
+    else if constexpr (BITS == 2) return tqd::field_offset<2>(cw[k >> 3], 4 * (k & 7), 4);
+    else return k < 12 ? tqd::field_offset<2>(cw[k >> 2], 6 * (k & 3), 6) : tqd::field_offset<2>(tail, 6 * (k - 12), 6);
+}
+
+// 32 rotated-domain fp16 values of one token per lane (xb[ks] = values 8ks .. 8ks+7 of the lane quarter's 32)
+// -> the lane's 32 output dims as fp16 pairs: eight MFMAs, the butterfly over the slices, norm / sqrt(128), s1
+__device__ __forceinline__ void unrotate_unit16(const half8_t (&af)[8], const uint4 (&xb)[4], float g, const uint32_t (&smask)[16],
+                                                uint32_t (&o)[16]) {
+    float4_t q[2][4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int f0 = 0; f0 < 2; ++f0)
+            q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], __builtin_bit_cast(half8_t, xb[ks]),
+                                                               float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    // fragment 2*fh + f0 holds dims 32kc + 8fh + 4f0 + i
+    float4_t y[8];
+#pragma unroll
+    for (int f0 = 0; f0 < 2; ++f0) {
+        const float4_t s01 = q[f0][0] + q[f0][1], d01 = q[f0][0] - q[f0][1];
+        const float4_t s23 = q[f0][2] + q[f0][3], d23 = q[f0][2] - q[f0][3];
+        y[0 + f0] = s01 + s23;
+        y[2 + f0] = d01 + d23;
+        y[4 + f0] = s01 - s23;
+        y[6 + f0] = d01 - d23;
+    }
+    const float gs = g * RSQRT128;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const int v = 2 * w;
+        const uint32_t lo = __half_as_ushort(__float2half_rn(y[v >> 2][v & 3] * gs));
+        const uint32_t hi = __half_as_ushort(__float2half_rn(y[(v + 1) >> 2][(v + 1) & 3] * gs));
+        o[w] = (lo | (hi << 16)) ^ smask[w];
+    }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half *out, LoadK16Args a) {
+    __shared__ uint32_t lut_s[1 << (2 * BITS)];
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n16 = lane & 15, kc = lane >> 4;
+    for (int e = tid; e < (1 << (2 * BITS)); e += 256) lut_s[e] = a.pair_lut[e];
+    __shared__ float s1_s[128];
+    constexpr int XROW = 256 + 16;  // bytes per token row of the transposition space (padding spreads the banks)
+    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[4 * 16 * XROW];
+    frag_s[tid] = a.afrag[tid];
+    frag_s[256 + tid] = a.afrag[256 + tid];
+    if (tid < 128) s1_s[tid] = a.s1[tid];
+    __syncthreads();
+    uint32_t smask[16];  // sign bits of s1 for the lane's 32 output dims, two fp16 per dword
+#pragma unroll
+    for (int w = 0; w < 16; ++w)
+        smask[w] = (s1_s[32 * kc + 2 * w] < 0.0f ? 0x8000u : 0u) | (s1_s[32 * kc + 2 * w + 1] < 0.0f ? 0x80000000u : 0u);
+    half8_t af[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag_s[f * 64 + lane]);
+    const char *lut = reinterpret_cast<const char *>(lut_s);
+    const uint32_t bps = a.blocks_per_seq;
+#pragma unroll 1
+    for (uint32_t u = blockIdx.x * 4 + wave; u < a.n_units; u += gridDim.x * 4) {
+        const uint32_t blk = u >> 3, seq = blk / bps, bis = blk - seq * bps;
+        const int row = (int)(u & 7) * 16 + n16;
+        const uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
+        uint32_t cw[BITS];
+#pragma unroll
+        for (int j = 0; j < BITS; ++j) cw[j] = *reinterpret_cast<const uint32_t *>(block + j * 2048 + row * 16 + kc * 4);
+        const float g = __half2float(reinterpret_cast<const __half *>(block + block_code_bytes(BITS))[row]);
+        uint32_t tail = 0;
+        if constexpr (BITS == 3) tail = (cw[0] >> 24) | ((cw[1] >> 24) << 8) | ((cw[2] >> 24) << 16);
+        uint4 xb[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            xb[ks].x = *reinterpret_cast<const uint32_t *>(lut + group_pair_offset<BITS>(cw, tail, 4 * ks));
+            xb[ks].y = *reinterpret_cast<const uint32_t *>(lut + group_pair_offset<BITS>(cw, tail, 4 * ks + 1));
+            xb[ks].z = *reinterpret_cast<const uint32_t *>(lut + group_pair_offset<BITS>(cw, tail, 4 * ks + 2));
+            xb[ks].w = *reinterpret_cast<const uint32_t *>(lut + group_pair_offset<BITS>(cw, tail, 4 * ks + 3));
+        }
+        uint32_t o[16];
+        unrotate_unit16(af, xb, g, smask, o);
+        // through this wavefront's 4.25 KB of LDS, so that a store instruction writes four whole token rows
+        // (1 KB of contiguous memory) instead of sixty-four 16-byte pieces
+        uint8_t *mine = xpose_s + wave * (16 * XROW);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            *reinterpret_cast<uint4 *>(mine + n16 * XROW + kc * 64 + c * 16) = make_uint4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
+        const int64_t tok_base = (int64_t)bis * TQ_ROWS_PER_BLOCK + (int)(u & 7) * 16;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int tr = 4 * c + (lane >> 4);  // token of the unit this lane stores a piece of
+            const uint4 piece = *reinterpret_cast<const uint4 *>(mine + tr * XROW + (lane & 15) * 16);
+            if (tok_base + tr < a.tokens)
+                *reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok_base + tr) * 128 + 8 * (lane & 15))) = piece;
+        }
+    }
+}
+
+// The same for V rows (dim-major inside a 64-token tile): the tile's codes are staged in LDS and a lane gathers the
+// 32 codes of its token from 32 rows (same pair position in each).  Wavefront w takes tokens 16a + 4w + i of the
+// tile (a, i = 0..3), so that the dword a pair sits in - and for 3-bit codes whether it sits in the split tail -
+// is the same for the whole wavefront.  a.n_units counts 64-token tiles here.
+template <int BITS>
+__global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half *out, LoadK16Args a) {
+    constexpr int XROW = 256 + 16;
+    constexpr int PIECES = BITS * 64 + 8;  // 16-byte pieces of a tile: codes [BITS][64 rows][16 B], then 64 fp16 norms
+    __shared__ uint16_t cent_s[16];
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ float s1_s[128];
+    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[4 * 16 * XROW];
+    __shared__ __attribute__((aligned(16))) uint8_t tile_s[PIECES * 16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n16 = lane & 15, kc = lane >> 4;
+    if (tid < (1 << BITS)) cent_s[tid] = (uint16_t)(a.pair_lut[tid] & 0xffffu);  // pair (lo = code, hi = 0): low half = c[code]
+    frag_s[tid] = a.afrag[tid];
+    frag_s[256 + tid] = a.afrag[256 + tid];
+    if (tid < 128) s1_s[tid] = a.s1[tid];
+    __syncthreads();
+    uint32_t smask[16];
+#pragma unroll
+    for (int w = 0; w < 16; ++w)
+        smask[w] = (s1_s[32 * kc + 2 * w] < 0.0f ? 0x8000u : 0u) | (s1_s[32 * kc + 2 * w + 1] < 0.0f ? 0x80000000u : 0u);
+    half8_t af[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag_s[f * 64 + lane]);
+    const uint32_t bps = a.blocks_per_seq;
+    // this lane's token inside the tile and where its codes sit in a row
+    const int tl = 16 * (n16 >> 2) + 4 * wave + (n16 & 3);
+    const int hf = kc >> 1, r0 = 32 * (kc & 1);
+    const int p = ((tl & 60) | (hf << 1)) | ((tl >> 1) & 1);
+    const int grp = p >> 4, k = p & 15;  // k / pairs per dword depends on the wavefront only
+    const int hs = (tl & 1) * BITS;
+    constexpr uint32_t CM = (1u << BITS) - 1u;
+#pragma unroll 1
+    for (uint32_t tile = blockIdx.x; tile < a.n_units; tile += gridDim.x) {
+        const uint32_t blk = tile >> 1, half = tile & 1, seq = blk / bps, bis = blk - seq * bps;
+        const uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
+        __syncthreads();  // the previous tile's codes are no longer needed
+        for (int e = tid; e < PIECES; e += 256) {
+            const uint8_t *src = e < BITS * 64 ? block + (e >> 6) * 2048 + (64 * half + (e & 63)) * 16
+                                               : block + block_code_bytes(BITS) + 128 * half + (e - BITS * 64) * 16;
+            reinterpret_cast<uint4 *>(tile_s)[e] = *reinterpret_cast<const uint4 *>(src);
+        }
+        __syncthreads();
+        const float g = __half2float(reinterpret_cast<const __half *>(tile_s + BITS * 1024)[tl]);
+        uint32_t hv[32];  // fp16 bits of the lane's 32 values
+        if (BITS == 3 && wave == 3) {
+            const int sh = 6 * (k - 12) + hs;
+#pragma unroll
+            for (int v = 0; v < 32; ++v) {
+                const uint8_t *rowp = tile_s + (r0 + v) * 16 + grp * 4;
+                const uint32_t tail = (*reinterpret_cast<const uint32_t *>(rowp) >> 24) |
+                                      ((*reinterpret_cast<const uint32_t *>(rowp + 1024) >> 24) << 8) |
+                                      ((*reinterpret_cast<const uint32_t *>(rowp + 2048) >> 24) << 16);
+                hv[v] = cent_s[(tail >> sh) & CM];
+            }
+        } else {
+            const int dw = k / tqd::pairs_per_dword(BITS);
+            const int sh = 2 * BITS * (k % tqd::pairs_per_dword(BITS)) + hs;
+            const uint8_t *col = tile_s + dw * 1024 + grp * 4;
+#pragma unroll
+            for (int v = 0; v < 32; ++v) hv[v] = cent_s[(*reinterpret_cast<const uint32_t *>(col + (r0 + v) * 16) >> sh) & CM];
+        }
+        uint4 xb[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            xb[ks].x = hv[8 * ks] | (hv[8 * ks + 1] << 16);
+            xb[ks].y = hv[8 * ks + 2] | (hv[8 * ks + 3] << 16);
+            xb[ks].z = hv[8 * ks + 4] | (hv[8 * ks + 5] << 16);
+            xb[ks].w = hv[8 * ks + 6] | (hv[8 * ks + 7] << 16);
+        }
+        uint32_t o[16];
+        unrotate_unit16(af, xb, g, smask, o);
+        uint8_t *mine = xpose_s + wave * (16 * XROW);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            *reinterpret_cast<uint4 *>(mine + n16 * XROW + kc * 64 + c * 16) = make_uint4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
+        const int64_t tok_base = (int64_t)bis * TQ_ROWS_PER_BLOCK + 64 * half;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            // row 4c + lane/16 of the wavefront's space is token 16c + 4 wave + lane/16 of the tile
+            const int tr = 4 * c + (lane >> 4);
+            const int64_t tok = tok_base + 16 * c + 4 * wave + (lane >> 4);
+            const uint4 piece = *reinterpret_cast<const uint4 *>(mine + tr * XROW + (lane & 15) * 16);
+            if (tok < a.tokens)
+                *reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok) * 128 + 8 * (lane & 15))) = piece;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void k_unpack_codes(const uint8_t *packed, uint8_t *idx, float *norms, int bits,
                                                       int kind, int64_t tokens, int64_t blocks_per_seq) {
     const int64_t blk = blockIdx.x;
@@ -1986,6 +2191,30 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
     const int64_t bps = blocks_for(tokens);
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
+    if (out_dtype == TQ_F16 && kind == TQ_KIND_V && domain == TQ_DOMAIN_ORIGINAL && h->rfrag16k_inv) {
+        LoadK16Args k;
+        k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
+        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 2);
+        const unsigned g16 = (unsigned)std::min<int64_t>((int64_t)k.n_units, 256 * 4);
+        switch (h->bits) {
+        case 2: k_load_v16<2><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        case 3: k_load_v16<3><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        default: k_load_v16<4><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        }
+        return tq_check_launch("load_v16");
+    }
+    if (out_dtype == TQ_F16 && kind == TQ_KIND_K && domain == TQ_DOMAIN_ORIGINAL && h->rfrag16k_inv) {
+        LoadK16Args k;
+        k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
+        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 8);
+        const unsigned g16 = (unsigned)std::min<int64_t>(((int64_t)k.n_units + 3) / 4, 256 * 4);
+        switch (h->bits) {
+        case 2: k_load_k16<2><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        case 3: k_load_k16<3><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        default: k_load_k16<4><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
+        }
+        return tq_check_launch("load_k16");
+    }
     LoadArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.cent = h->centroids32;
     a.bits = h->bits; a.kind = kind; a.domain = domain;
