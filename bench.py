@@ -139,7 +139,7 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
         ok, ov = outs[i % 2]
         codec_k.load(kp_i, heads, tokens, kind="k", out=ok)
         codec_v.load(vp_i, heads, tokens, kind="v", out=ov)
-    _, lev_ms = time_steps(torch, lstep, max(20, steps // 4), max(10, warmup // 4))
+    _, lev_ms = time_steps(torch, lstep, steps, warmup)
     load_algo = n_vec * (16 * bits + 2 + 256)
     return {
         "workload": f"turbo{bits} store, K+V fp16 [8,32768,128], 4 K outlier channels x15, block 128",

@@ -780,47 +780,62 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int KT_STRIDE = 264;  // halves per staged key row (256 + 8: 16-byte reads of 16 rows hit 64 distinct banks)
 
-// [R q | S q] as fp16, one wavefront per query
+// [R q | S q] as fp16; a wavefront takes PREP_Q queries so that every row of the projection it fetches serves
+// all of them (one query per wavefront made the launch wait for 2048 x 64 KB of L2 reads)
+constexpr int PREP_Q = 4;
 template <typename TI>
 __global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, int64_t nq, const float *s1,
                                                       const float *s2, const float *projT) {
-    __shared__ float qs[4][128];
+    __shared__ float qs[4][PREP_Q][128];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int64_t v = (int64_t)blockIdx.x * 4 + w;
-    float x0 = 0.f, x1 = 0.f;
-    if (v < nq) {
-        x0 = ldf(q + v * 128 + 2 * lane);
-        x1 = ldf(q + v * 128 + 2 * lane + 1);
+    const int64_t v0 = ((int64_t)blockIdx.x * 4 + w) * PREP_Q;
+    float x0[PREP_Q], x1[PREP_Q];
+#pragma unroll
+    for (int i = 0; i < PREP_Q; ++i) {
+        const bool have = v0 + i < nq;
+        x0[i] = have ? ldf(q + (v0 + i) * 128 + 2 * lane) : 0.f;
+        x1[i] = have ? ldf(q + (v0 + i) * 128 + 2 * lane + 1) : 0.f;
+        qs[w][i][2 * lane] = x0[i];
+        qs[w][i][2 * lane + 1] = x1[i];
     }
-    qs[w][2 * lane] = x0;
-    qs[w][2 * lane + 1] = x1;
     __syncthreads();
-    if (v >= nq) return;
-    float p0 = 0.f, p1 = 0.f;  // (S q)[2*lane], (S q)[2*lane+1]
-#pragma unroll 16
+    if (v0 >= nq) return;
+    float p0[PREP_Q], p1[PREP_Q];  // (S q)[2*lane], (S q)[2*lane+1]
+#pragma unroll
+    for (int i = 0; i < PREP_Q; ++i) p0[i] = p1[i] = 0.f;
+#pragma unroll 8
     for (int k = 0; k < 128; ++k) {
-        const float qk = qs[w][k];
         const float2 pt = *reinterpret_cast<const float2 *>(projT + k * 128 + 2 * lane);
-        p0 = fmaf(pt.x, qk, p0);
-        p1 = fmaf(pt.y, qk, p1);
+#pragma unroll
+        for (int i = 0; i < PREP_Q; ++i) {
+            const float qk = qs[w][i][k];
+            p0[i] = fmaf(pt.x, qk, p0[i]);
+            p1[i] = fmaf(pt.y, qk, p1[i]);
+        }
     }
-    x0 *= s1[2 * lane];
-    x1 *= s1[2 * lane + 1];
-    wht128_wave(x0, x1, lane);
-    x0 *= s2[2 * lane] * RSQRT128;
-    x1 *= s2[2 * lane + 1] * RSQRT128;
-    // operand-major layout: the 16-byte chunk (row r of query block v / 32, K values 16t + 8kb .. + 7) that
-    // lane r + 32kb of the score tile's MFMA reads in K step t sits at chunk index (block * 16 + t) * 64 + r + 32kb,
-    // so one wave-wide operand load is 1 KB of contiguous memory
+    const float a0 = s1[2 * lane], a1 = s1[2 * lane + 1];
+    const float b0 = s2[2 * lane] * RSQRT128, b1 = s2[2 * lane + 1] * RSQRT128;
     __half2 *qa2 = reinterpret_cast<__half2 *>(qa);
-    const int64_t blk = v >> 5;
-    const int r = (int)(v & 31);
-    auto chunk_pair = [&](int k) {  // index of the half2 holding K values k, k + 1 (k even)
-        const int t = k >> 4, kb = (k >> 3) & 1, e = k & 7;
-        return (((blk * 16 + t) * 64 + r + 32 * kb) * 8 + e) >> 1;
-    };
-    qa2[chunk_pair(2 * lane)] = __halves2half2(__float2half_rn(x0), __float2half_rn(x1));
-    qa2[chunk_pair(128 + 2 * lane)] = __halves2half2(__float2half_rn(p0), __float2half_rn(p1));
+#pragma unroll
+    for (int i = 0; i < PREP_Q; ++i) {
+        const int64_t v = v0 + i;
+        if (v >= nq) break;
+        float y0 = x0[i] * a0, y1 = x1[i] * a1;
+        wht128_wave(y0, y1, lane);
+        y0 *= b0;
+        y1 *= b1;
+        // operand-major layout: the 16-byte chunk (row r of query block v / 32, K values 16t + 8kb .. + 7) that
+        // lane r + 32kb of the score tile's MFMA reads in K step t sits at chunk index (block * 16 + t) * 64 + r + 32kb,
+        // so one wave-wide operand load is 1 KB of contiguous memory
+        const int64_t blk = v >> 5;
+        const int r = (int)(v & 31);
+        auto chunk_pair = [&](int k) {  // index of the half2 holding K values k, k + 1 (k even)
+            const int t = k >> 4, kb = (k >> 3) & 1, e = k & 7;
+            return (((blk * 16 + t) * 64 + r + 32 * kb) * 8 + e) >> 1;
+        };
+        qa2[chunk_pair(2 * lane)] = __halves2half2(__float2half_rn(y0), __float2half_rn(y1));
+        qa2[chunk_pair(128 + 2 * lane)] = __halves2half2(__float2half_rn(p0[i]), __float2half_rn(p1[i]));
+    }
 }
 
 // One workgroup of eight wavefronts per 256 keys: dequantise them once into LDS as fp16
@@ -1001,7 +1016,7 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
         return TQ_ERR_UNSUPPORTED;
     }
     __half *qa = reinterpret_cast<__half *>(ws);
-    const unsigned qgrid = (unsigned)((nq + 3) / 4);
+    const unsigned qgrid = (unsigned)((nq + 4 * PREP_Q - 1) / (4 * PREP_Q));
     switch (q_dtype) {
     case TQ_F16: k_prep_score_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
     case TQ_F32: k_prep_score_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;

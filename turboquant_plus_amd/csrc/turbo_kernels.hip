@@ -1529,15 +1529,26 @@ __global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half 
     for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag_s[f * 64 + lane]);
     const char *lut = reinterpret_cast<const char *>(lut_s);
     const uint32_t bps = a.blocks_per_seq;
+    // the next unit's codes and norm are requested before the current one is worked on (the last fetch re-reads)
+    auto fetch = [&](uint32_t u, uint32_t (&cw)[BITS], __half &gh) {
+        u = u < a.n_units ? u : a.n_units - 1;
+        const uint8_t *block = packed + (int64_t)(u >> 3) * block_bytes(BITS);
+        const int row = (int)(u & 7) * 16 + n16;
+#pragma unroll
+        for (int j = 0; j < BITS; ++j) cw[j] = *reinterpret_cast<const uint32_t *>(block + j * 2048 + row * 16 + kc * 4);
+        gh = reinterpret_cast<const __half *>(block + block_code_bytes(BITS))[row];
+    };
+    uint32_t cw_next[BITS];
+    __half g_next;
+    fetch(blockIdx.x * 4 + wave, cw_next, g_next);
 #pragma unroll 1
     for (uint32_t u = blockIdx.x * 4 + wave; u < a.n_units; u += gridDim.x * 4) {
         const uint32_t blk = u >> 3, seq = blk / bps, bis = blk - seq * bps;
-        const int row = (int)(u & 7) * 16 + n16;
-        const uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
         uint32_t cw[BITS];
 #pragma unroll
-        for (int j = 0; j < BITS; ++j) cw[j] = *reinterpret_cast<const uint32_t *>(block + j * 2048 + row * 16 + kc * 4);
-        const float g = __half2float(reinterpret_cast<const __half *>(block + block_code_bytes(BITS))[row]);
+        for (int j = 0; j < BITS; ++j) cw[j] = cw_next[j];
+        const float g = __half2float(g_next);
+        fetch(u + gridDim.x * 4, cw_next, g_next);
         uint32_t tail = 0;
         if constexpr (BITS == 3) tail = (cw[0] >> 24) | ((cw[1] >> 24) << 8) | ((cw[2] >> 24) << 16);
         uint4 xb[4];
@@ -1602,17 +1613,32 @@ __global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half 
     const int grp = p >> 4, k = p & 15;  // k / pairs per dword depends on the wavefront only
     const int hs = (tl & 1) * BITS;
     constexpr uint32_t CM = (1u << BITS) - 1u;
+    static_assert(PIECES <= 512, "two pieces per thread at most");
+    uint4 pre0, pre1;  // pieces tid and tid + 256 of the next tile
+    auto fetch_tile = [&](uint32_t tile) {
+        tile = tile < a.n_units ? tile : a.n_units - 1;
+        const uint8_t *block = packed + (int64_t)(tile >> 1) * block_bytes(BITS);
+        const int half = (int)(tile & 1);
+        auto piece = [&](int e) {
+            e = min(e, PIECES - 1);
+            const uint8_t *src = e < BITS * 64 ? block + (e >> 6) * 2048 + (64 * half + (e & 63)) * 16
+                                               : block + block_code_bytes(BITS) + 128 * half + (e - BITS * 64) * 16;
+            return *reinterpret_cast<const uint4 *>(src);
+        };
+        pre0 = piece(tid);
+        if constexpr (PIECES > 256) pre1 = piece(tid + 256);
+    };
+    fetch_tile(blockIdx.x);
 #pragma unroll 1
     for (uint32_t tile = blockIdx.x; tile < a.n_units; tile += gridDim.x) {
         const uint32_t blk = tile >> 1, half = tile & 1, seq = blk / bps, bis = blk - seq * bps;
-        const uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
         __syncthreads();  // the previous tile's codes are no longer needed
-        for (int e = tid; e < PIECES; e += 256) {
-            const uint8_t *src = e < BITS * 64 ? block + (e >> 6) * 2048 + (64 * half + (e & 63)) * 16
-                                               : block + block_code_bytes(BITS) + 128 * half + (e - BITS * 64) * 16;
-            reinterpret_cast<uint4 *>(tile_s)[e] = *reinterpret_cast<const uint4 *>(src);
+        if (tid < PIECES) reinterpret_cast<uint4 *>(tile_s)[tid] = pre0;
+        if constexpr (PIECES > 256) {
+            if (tid + 256 < PIECES) reinterpret_cast<uint4 *>(tile_s)[tid + 256] = pre1;
         }
         __syncthreads();
+        fetch_tile(tile + gridDim.x);  // the next tile's pieces travel while this one is worked on
         const float g = __half2float(reinterpret_cast<const __half *>(tile_s + BITS * 1024)[tl]);
         uint32_t hv[32];  // fp16 bits of the lane's 32 values
         if (BITS == 3 && wave == 3) {
@@ -1838,6 +1864,17 @@ static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     return va;
 }
 
+// Workgroups of `kernel` (256 threads, static LDS only) that fit on the device at once: the persistent loops
+// below are launched with exactly that many, so that no workgroup waits for another one to finish.
+template <typename K> static unsigned resident_workgroups(K kernel) {
+    int per_cu = 0, dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1)
+        return 256u * 2u;
+    return (unsigned)prop.multiProcessorCount * (unsigned)per_cu;
+}
+
 int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
               uint8_t *sign_bits, void *rnorms, hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
@@ -1870,11 +1907,15 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
         const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
         if (kind == TQ_KIND_K) {
             const StoreKArgs ka = make_k_args(h, tokens, bps, n_blocks);
-            // four workgroups of four wavefronts per CU
-            const unsigned kgrid = (unsigned)((ka.n_units + 3) / 4 < 1024 ? (ka.n_units + 3) / 4 : 1024);
+            // as many workgroups of four wavefronts as are resident at once (registers and LDS decide: 2 to 4 per CU)
+            const unsigned kneed = (unsigned)((ka.n_units + 3) / 4);
 #define TQ_STORE_K(B)                                                                                   \
-    if (ragged) k_store_k<B, true><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);       \
-    else k_store_k<B, false><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka)
+    {                                                                                                   \
+        static const unsigned fit[2] = {resident_workgroups(k_store_k<B, false>), resident_workgroups(k_store_k<B, true>)}; \
+        const unsigned kgrid = kneed < fit[ragged] ? kneed : fit[ragged];                               \
+        if (ragged) k_store_k<B, true><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);   \
+        else k_store_k<B, false><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);         \
+    }
             switch (h->bits) {
             case 2: TQ_STORE_K(2); break;
             case 3: TQ_STORE_K(3); break;
@@ -1884,11 +1925,14 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
             return tq_check_launch("store_k");
         }
         const StoreVArgs va = make_v_args(h, tokens, bps, n_blocks);
-        // three workgroups of four wavefronts per CU
-        const unsigned vgrid = (unsigned)((va.n_units + 3) / 4 < 768 ? (va.n_units + 3) / 4 : 768);
+        const unsigned vneed = (unsigned)((va.n_units + 3) / 4);
 #define TQ_STORE_V(B)                                                                                   \
-    if (ragged) k_store_v<B, true><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);       \
-    else k_store_v<B, false><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va)
+    {                                                                                                   \
+        static const unsigned fit[2] = {resident_workgroups(k_store_v<B, false>), resident_workgroups(k_store_v<B, true>)}; \
+        const unsigned vgrid = vneed < fit[ragged] ? vneed : fit[ragged];                               \
+        if (ragged) k_store_v<B, true><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);   \
+        else k_store_v<B, false><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);         \
+    }
         switch (h->bits) {
         case 2: TQ_STORE_V(2); break;
         case 3: TQ_STORE_V(3); break;
@@ -2195,7 +2239,9 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
         LoadK16Args k;
         k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
         k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 2);
-        const unsigned g16 = (unsigned)std::min<int64_t>((int64_t)k.n_units, 256 * 4);
+        static const unsigned fit[3] = {resident_workgroups(k_load_v16<2>), resident_workgroups(k_load_v16<3>),
+                                        resident_workgroups(k_load_v16<4>)};
+        const unsigned g16 = (unsigned)std::min<int64_t>((int64_t)k.n_units, fit[h->bits - 2]);
         switch (h->bits) {
         case 2: k_load_v16<2><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
         case 3: k_load_v16<3><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
@@ -2207,7 +2253,9 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
         LoadK16Args k;
         k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
         k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 8);
-        const unsigned g16 = (unsigned)std::min<int64_t>(((int64_t)k.n_units + 3) / 4, 256 * 4);
+        static const unsigned fit[3] = {resident_workgroups(k_load_k16<2>), resident_workgroups(k_load_k16<3>),
+                                        resident_workgroups(k_load_k16<4>)};
+        const unsigned g16 = (unsigned)std::min<int64_t>(((int64_t)k.n_units + 3) / 4, fit[h->bits - 2]);
         switch (h->bits) {
         case 2: k_load_k16<2><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
         case 3: k_load_k16<3><<<g16, 256, 0, s>>>((const uint8_t *)packed, (__half *)out, k); break;
