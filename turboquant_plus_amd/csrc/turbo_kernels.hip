@@ -1155,11 +1155,12 @@ __global__ __launch_bounds__(256) void k_store(const TI *x, uint8_t *packed, Sto
 
 // ---- K2, streaming append -------------------------------------------------------------
 // n_new tokens per sequence at positions pos .. pos+n_new-1 of a buffer laid out for
-// blocks_per_seq blocks per sequence.  One workgroup per touched block rebuilds the block:
-// rows before pos are unpacked from the block itself, the new rows are quantised exactly as
-// k_store does, the rest get the code of 0.0 and norm 0 (what k_store writes past the end of a
-// sequence), and pack_block writes the block back.  After any sequence of appends covering
-// tokens 0 .. T-1 the touched blocks equal those of k_store on the first T tokens.
+// blocks_per_seq blocks per sequence, one workgroup per touched block.  The new rows are quantised
+// exactly as k_store does.  A block whose first token is among them is written whole: the rows
+// past the new tokens get the code of 0.0 and norm 0 (what k_store writes past the end of a
+// sequence).  A block that already holds tokens keeps them: K rows are tokens and are simply left
+// alone, V rows get the new tokens' codes put into their packed words.  After any sequence of
+// appends covering tokens 0 .. T-1 the touched blocks equal those of k_store on the first T tokens.
 struct AppendArgs {
     const float *s1, *s2, *bounds, *cent;
     int kind, norm_correction, zero_code;
@@ -1203,14 +1204,59 @@ __device__ __forceinline__ void append_block(const TI *x, uint8_t *packed, const
     // K rows are tokens: the rows already there stay untouched in memory and need not be unpacked
     const bool keep_rows = a.kind == TQ_KIND_K;
     if (n_old > 0 && !keep_rows) {
-        for (int e = tid; e < block_bytes(BITS) / 16; e += 256)
-            reinterpret_cast<uint4 *>(old_s)[e] = reinterpret_cast<const uint4 *>(block)[e];
-        __syncthreads();
-        for (int e = tid; e < n_old * 128; e += 256) {
-            const int t = e >> 7, dim = e & 127;
-            codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(old_s, BITS, a.kind, t, dim);
+        // V rows of a block that already holds tokens: the new tokens' codes are put into the packed rows in
+        // place (every row of the tile has one pair position per token), so nothing is unpacked or re-packed.
+        // Rows past the new tokens keep the code of 0.0 that the block's first append gave them.
+        constexpr int PIECES = block_bytes(BITS) / 16, NP = (PIECES + 255) / 256;
+        constexpr uint32_t CM = (1u << BITS) - 1u;
+        uint4 pre[NP];
+#pragma unroll
+        for (int i = 0; i < NP; ++i) pre[i] = reinterpret_cast<const uint4 *>(block)[min(tid + 256 * i, PIECES - 1)];
+        __syncthreads();  // csq_s is ready
+#pragma unroll 1
+        for (int it = 0; it < 8; ++it) {
+            const int t = it * 16 + grp;
+            if (t < n_old || t >= n_end) continue;
+            float xv[8];
+            load8(x + ((seq * a.n_new + (tok0 + t - a.pos)) * 128 + 8 * li), xv);
+            uint2 c8;
+            const float g = quantize_vec16<BITS>(xv, lane, bnd, s1v, s2v, csq_s, a.norm_correction, c8);
+            *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = c8;
+            if (li == 0) norms_s[t] = g;
         }
-        for (int t = tid; t < n_old; t += 256) norms_s[t] = block_norm(old_s, BITS, t);
+#pragma unroll
+        for (int i = 0; i < NP; ++i)
+            if (tid + 256 * i < PIECES) reinterpret_cast<uint4 *>(old_s)[tid + 256 * i] = pre[i];
+        __syncthreads();
+        if (tid < TQ_ROWS_PER_BLOCK) {
+            const int r = tid, rr = r & 63, t_lo = max(n_old, r & 64), t_hi = min(n_end, (r & 64) + 64);
+            for (int t = t_lo; t < t_hi; ++t) {
+                const int tl = t & 63, g = tl >> 4, k0 = (tl & 12) | ((tl >> 1) & 1), hs = (tl & 1) * BITS;
+                const uint32_t c0 = codes[t * CODE_STRIDE + rr], c1 = codes[t * CODE_STRIDE + 64 + rr];
+                uint8_t *rowp = old_s + r * 16 + g * 4;
+                if (BITS == 3 && k0 >= 12) {
+                    uint32_t *d0 = reinterpret_cast<uint32_t *>(rowp), *d1 = reinterpret_cast<uint32_t *>(rowp + 2048),
+                             *d2 = reinterpret_cast<uint32_t *>(rowp + 4096);
+                    uint32_t tail = (*d0 >> 24) | ((*d1 >> 24) << 8) | ((*d2 >> 24) << 16);
+                    const int s0 = 6 * (k0 - 12) + hs, s1 = s0 + 12;
+                    tail = (tail & ~((CM << s0) | (CM << s1))) | (c0 << s0) | (c1 << s1);
+                    *d0 = (*d0 & 0x00FFFFFFu) | (tail << 24);
+                    *d1 = (*d1 & 0x00FFFFFFu) | ((tail >> 8) << 24);
+                    *d2 = (*d2 & 0x00FFFFFFu) | ((tail >> 16) << 24);
+                } else {
+                    uint32_t *d = reinterpret_cast<uint32_t *>(rowp + (k0 / tqd::pairs_per_dword(BITS)) * 2048);
+                    const int s0 = 2 * BITS * (k0 % tqd::pairs_per_dword(BITS)) + hs, s1 = s0 + 4 * BITS;
+                    *d = (*d & ~((CM << s0) | (CM << s1))) | (c0 << s0) | (c1 << s1);
+                }
+            }
+        }
+        for (int t = n_old + tid; t < n_end; t += 256)
+            reinterpret_cast<__half *>(old_s + block_code_bytes(BITS))[t] = __float2half_rn(norms_s[t]);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NP; ++i)
+            if (tid + 256 * i < PIECES) reinterpret_cast<uint4 *>(block)[tid + 256 * i] = reinterpret_cast<const uint4 *>(old_s)[tid + 256 * i];
+        return;
     }
     // rows past the new tokens hold the code of 0.0 and norm 0 (what quantising a zero vector gives)
     for (int e = tid; e < (TQ_ROWS_PER_BLOCK - n_end) * 32; e += 256) {
