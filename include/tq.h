@@ -132,11 +132,12 @@ int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const v
  * packed buffer laid out for `capacity` tokens per sequence (tq_packed_bytes(bits, n_seqs,
  * capacity)); x is [n_seqs, n_new, 128].  The per-token compress step that kv_cache.py:65-66
  * names ("compress_token") and PLAN.md:119-122 plans; the reference does not implement it.
- * Same arithmetic as tq_store on fp32/fp64 input; the touched 128-token blocks are rebuilt:
- * rows before pos are kept, rows from pos+n_new to the end of the last touched block get the
- * code of 0.0 and norm 0 (what tq_store writes past the end of a sequence).  After appends
- * covering tokens 0 .. T-1 in any chunking the touched blocks equal tq_store's of the first T
- * tokens.  Appends to one buffer must be ordered (same stream). */
+ * Same arithmetic as tq_store on fp32/fp64 input.  In the touched 128-token blocks the tokens
+ * before pos are kept and the tokens from pos+n_new to the end of the last touched block get the
+ * code of 0.0 and norm 0 (what tq_store writes past the end of a sequence), so an append below
+ * the tokens already written truncates.  After appends covering tokens 0 .. T-1 in any chunking
+ * the touched blocks equal tq_store's of the first T tokens.  Appends to one buffer must be
+ * ordered (same stream). */
 int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity,
               int in_dtype, int kind, void *packed, void *stream);
 

@@ -43,6 +43,32 @@ def test_append_in_chunks_equals_store(bits, kind):
     assert pos == 300
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+@pytest.mark.parametrize("back_to,n_new", [(150, 1), (130, 17), (64, 3), (13, 1), (127, 2)])
+def test_append_after_a_rewind_truncates(bits, kind, back_to, n_new):
+    """Appending at a position below the tokens already written (a rolled-back speculative step) leaves
+    the touched blocks as tq_store writes them for the shortened sequence: the stale tokens behind the
+    new ones are gone from those blocks."""
+    tt = L.torch()
+    codec = tqa.TurboCodec(bits, seed=9)
+    n_seqs, capacity = 2, 384
+    rng = np.random.default_rng(bits * 100 + back_to)
+    x = rng.standard_normal((n_seqs, 230, D)).astype(np.float32)
+    y = rng.standard_normal((n_seqs, n_new, D)).astype(np.float32)
+    cache = tt.zeros(tqa.packed_bytes(bits, n_seqs, capacity), dtype=tt.uint8, device="cuda")
+    codec.append(x, cache, 0, capacity, kind=kind)
+    codec.append(y, cache, back_to, capacity, kind=kind)
+    now = np.concatenate([x[:, :back_to], y], axis=1)
+    want = np_(codec.store(now, kind=kind)).reshape(n_seqs, -1, O.block_bytes(bits))
+    got = blocks_of(cache, bits, n_seqs, capacity)
+    first, last = back_to // 128, (back_to + n_new - 1) // 128
+    for b in range(first, last + 1):      # the blocks the second append touched
+        assert np.array_equal(got[:, b], want[:, b]), f"block {b}"
+    for b in range(first):                # blocks before it are untouched
+        assert np.array_equal(got[:, b], want[:, b]), f"block {b}"
+
+
 @pytest.mark.parametrize("kbits,vbits", [(3, 3), (4, 4), (4, 2), (2, 4)])
 def test_append_kv_equals_two_appends(kbits, vbits):
     """K and V of a step in one launch (tq_append_kv) write the bytes of two tq_append calls;

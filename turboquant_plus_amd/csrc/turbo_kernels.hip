@@ -1229,10 +1229,15 @@ __device__ __forceinline__ void append_block(const TI *x, uint8_t *packed, const
             if (tid + 256 * i < PIECES) reinterpret_cast<uint4 *>(old_s)[tid + 256 * i] = pre[i];
         __syncthreads();
         if (tid < TQ_ROWS_PER_BLOCK) {
-            const int r = tid, rr = r & 63, t_lo = max(n_old, r & 64), t_hi = min(n_end, (r & 64) + 64);
+            // new tokens take their codes; tokens from n_end to the end of their 16-token group take the code of 0.0
+            // (as do the whole groups after it, below): what tq_store writes past the end of a sequence
+            const int r = tid, rr = r & 63, t_lo = max(n_old, r & 64), t_end = (r & 64) + 64;
+            const int t_hi = min(max((n_end + 15) & ~15, t_lo), t_end);
             for (int t = t_lo; t < t_hi; ++t) {
                 const int tl = t & 63, g = tl >> 4, k0 = (tl & 12) | ((tl >> 1) & 1), hs = (tl & 1) * BITS;
-                const uint32_t c0 = codes[t * CODE_STRIDE + rr], c1 = codes[t * CODE_STRIDE + 64 + rr];
+                const bool fresh = t < n_end;
+                const uint32_t c0 = fresh ? codes[t * CODE_STRIDE + rr] : (uint32_t)a.zero_code;
+                const uint32_t c1 = fresh ? codes[t * CODE_STRIDE + 64 + rr] : (uint32_t)a.zero_code;
                 uint8_t *rowp = old_s + r * 16 + g * 4;
                 if (BITS == 3 && k0 >= 12) {
                     uint32_t *d0 = reinterpret_cast<uint32_t *>(rowp), *d1 = reinterpret_cast<uint32_t *>(rowp + 2048),
@@ -1249,9 +1254,22 @@ __device__ __forceinline__ void append_block(const TI *x, uint8_t *packed, const
                     *d = (*d & ~((CM << s0) | (CM << s1))) | (c0 << s0) | (c1 << s1);
                 }
             }
+            // whole 16-token groups past the new tokens: every field the code of 0.0
+            uint32_t fill = 0;
+#pragma unroll
+            for (int f = 0; f < 32 / BITS; ++f) fill |= (uint32_t)a.zero_code << (f * BITS);
+            for (int t = max(t_hi, t_lo); t < t_end; t += 16) {
+                uint8_t *rowp = old_s + r * 16 + ((t & 63) >> 4) * 4;
+#pragma unroll
+                for (int j = 0; j < BITS; ++j) {
+                    uint32_t w = fill;
+                    if constexpr (BITS == 3) w = (fill & 0x00FFFFFFu) | (((fill & 0x00FFFFFFu) >> (8 * j)) << 24);
+                    *reinterpret_cast<uint32_t *>(rowp + j * 2048) = w;
+                }
+            }
         }
-        for (int t = n_old + tid; t < n_end; t += 256)
-            reinterpret_cast<__half *>(old_s + block_code_bytes(BITS))[t] = __float2half_rn(norms_s[t]);
+        for (int t = n_old + tid; t < TQ_ROWS_PER_BLOCK; t += 256)
+            reinterpret_cast<__half *>(old_s + block_code_bytes(BITS))[t] = __float2half_rn(t < n_end ? norms_s[t] : 0.0f);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NP; ++i)
