@@ -8,7 +8,7 @@
 //                  16 lanes per vector (8 values each): three in-lane stages and
 //                  four DPP row stages; a workgroup owns one 128-token block,
 //                  stages the codes in LDS and writes the block coalesced.
-//   k_store_qjl    float64 variant that also sketches the residual (1-bit QJL).
+//   k_store_qjl_mfma  float64 variant that also sketches the residual (1-bit QJL), projection on fp64 MFMAs.
 //   k_load         packed block -> values (rotated or original domain).
 //   k_unpack_codes packed block -> uint8 indices + fp32 norms.
 //   k_q8_0_store   32-value int8 blocks with fp16 scale, 128-token block layout.
@@ -1321,88 +1321,153 @@ struct StoreQjlArgs {
     int64_t tokens, blocks_per_seq;
 };
 
+// One workgroup of eight wavefronts per CU, looping over 128-token blocks, with the projection (S R^T, 128 KB
+// of doubles) resident in LDS; a wavefront takes 16 tokens of the block, lane (token n16, quarter kq) holding
+// the 32 dims d = 4 s + kq: norms and the first two butterfly stages (in the reference's stage order) exchange
+// across the lane quarters, the other five stages are in-lane, and the residual in the rotated domain, taken
+// against the reconstruction the decoder will see (stored fp16 norm), is at once the A operand of
+// v_mfma_f64_16x16x4_f64: 256 of them per 16 tokens against the matrix in LDS.  The sign bits of a token's 16
+// projections of one column block are one quarter of a ballot.
+typedef double double4_t __attribute__((ext_vector_type(4)));
 template <int BITS, typename TI>
-__global__ __launch_bounds__(128) void k_store_qjl(const TI *x, uint8_t *packed, uint8_t *sign_bits, __half *rnorms,
-                                                  StoreQjlArgs a) {
+__global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *packed, uint8_t *sign_bits, __half *rnorms,
+                                                       StoreQjlArgs a, int64_t n_blocks) {
     using namespace tq64;
     constexpr int NB = (1 << BITS) - 1;
+    extern __shared__ double mat_s[];  // [k][j] = (S R^T)[j][k]
     __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
     __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
-    __shared__ double xs[VB * 128], ys[VB * 128];
-    __shared__ double nrm[VB], cn[VB], g16[VB];
+    __shared__ double cent_s[1 << BITS], bnd_s[1 << BITS];
 
-    const int tid = threadIdx.x;
-    const int64_t blk = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n16 = lane & 15, kq = lane >> 4;
+
+    // the matrix is fetched once per workgroup, sixteen 16-byte pieces per thread, eight in flight at a time
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        double2 piece[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const double2 *>(a.projrot_t)[tid + 512 * (8 * b + i)];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) reinterpret_cast<double2 *>(mat_s)[tid + 512 * (8 * b + i)] = piece[i];
+    }
+    if (tid < (1 << BITS)) cent_s[tid] = a.cent[tid];
+    if (tid < NB) bnd_s[tid] = a.bounds[tid];
+    uint32_t neg1 = 0, neg2 = 0;  // bit s: s1 / s2 of dim 4 s + kq is -1
+#pragma unroll
+    for (int s = 0; s < 32; ++s) {
+        neg1 |= (a.s1[4 * s + kq] < 0.0 ? 1u : 0u) << s;
+        neg2 |= (a.s2[4 * s + kq] < 0.0 ? 1u : 0u) << s;
+    }
+    __syncthreads();
+    // one reciprocal instead of 32 divisions per token, and 1 / sqrt(128) as a factor: at most one unit in the
+    // last place away from the quotients, far inside the 1e-6 band the codes and signs are held to
+    const double inv_rn = 1.0 / sqrt(128.0);
+
+#pragma unroll 1
+    for (int64_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
     const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
-    const int64_t row0 = seq * a.tokens;  // first row of this sequence in x / sign_bits / rnorms
-
-    RotArgs rw;
-    rw.d = rw.pd = 128;
-    rw.mode = TQ_ROT_WHT;
-    rw.mat = nullptr;
-    rw.sa = a.s1;
-    rw.sb = a.s2;
-    RotArgs rp;
-    rp.d = rp.pd = 128;
-    rp.mode = TQ_ROT_DENSE;
-    rp.mat = a.projrot_t;
-    rp.sa = rp.sb = nullptr;
-
-    for (int sb = 0; sb < TQ_ROWS_PER_BLOCK / VB; ++sb) {
-        const int64_t t0 = tok0 + sb * VB;                // token index (in sequence) of staged vector 0
-        const int64_t nvalid = a.tokens - t0;             // vectors with v < nvalid exist
-        for (int i = tid; i < VB * 128; i += NT) {
-            const int v = i >> 7;
-            xs[i] = (v < nvalid) ? ldd(x, (row0 + t0 + v) * 128 + (i & 127)) : 0.0;
+    const int64_t row0 = seq * a.tokens;
+    {
+        const int u = wave;  // eight wavefronts, 16 tokens each
+        const int t = u * 16 + n16;
+        const bool valid = tok0 + t < a.tokens;
+        double e[32];
+#pragma unroll
+        for (int s = 0; s < 32; ++s) e[s] = valid ? ldd(x, (row0 + tok0 + t) * 128 + 4 * s + kq) : 0.0;
+        auto quarter_sum = [&](double v) {
+            v += xor_lane<16>(v);
+            v += xor_lane<32>(v);
+            return v;
+        };
+        double ss = 0.0;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) ss = fma(e[s], e[s], ss);
+        const double nrm = sqrt(quarter_sum(ss));
+        const double inv = nrm > 0.0 ? 1.0 / nrm : 1.0;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            e[s] = e[s] * inv;
+            if ((neg1 >> s) & 1u) e[s] = -e[s];
         }
-        __syncthreads();
-        norms_block(xs, 128, 128, nrm);
-        for (int i = tid; i < VB * 128; i += NT) {
-            const double nv = nrm[i >> 7];
-            xs[i] = xs[i] / (nv > 0.0 ? nv : 1.0);
+        // butterfly, strides 1 and 2 across the lane quarters, then 4 .. 64 in the lane
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const double p = xor_lane<16>(e[s]);
+            e[s] = (kq & 1) ? p - e[s] : e[s] + p;
         }
-        __syncthreads();
-        rotate_block(rw, xs, ys);  // ys = rotated unit vectors
-        for (int i = tid; i < VB * 128; i += NT) {
-            const int v = i >> 7, j = i & 127;
-            const double yv = ys[i];
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const double p = xor_lane<32>(e[s]);
+            e[s] = (kq & 2) ? p - e[s] : e[s] + p;
+        }
+#pragma unroll
+        for (int hb = 1; hb < 32; hb <<= 1)
+#pragma unroll
+            for (int s = 0; s < 32; ++s)
+                if (!(s & hb)) {
+                    const double p = e[s], q = e[s + hb];
+                    e[s] = p + q;
+                    e[s + hb] = p - q;
+                }
+        uint32_t cw[4] = {0u, 0u, 0u, 0u};  // the 32 codes, 4 bits each
+        double cs = 0.0;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            double yv = e[s] * inv_rn;
+            if ((neg2 >> s) & 1u) yv = -yv;
+            e[s] = yv;
             int c = 0;
 #pragma unroll
-            for (int k = 0; k < NB; ++k) c += (a.bounds[k] < yv) ? 1 : 0;
-            codes[(sb * VB + v) * CODE_STRIDE + j] = (uint8_t)c;
-            xs[i] = a.cent[c];
+            for (int k = 0; k < NB; ++k) c += (bnd_s[k] < yv) ? 1 : 0;
+            codes[t * CODE_STRIDE + 4 * s + kq] = (uint8_t)c;
+            cw[s >> 3] |= (uint32_t)c << (4 * (s & 7));
+            const double cv = cent_s[c];
+            cs = fma(cv, cv, cs);
         }
-        __syncthreads();
-        norms_block(xs, 128, 128, cn);
-        if (tid < VB) {
-            double g = nrm[tid];
-            if (a.norm_correction) g = nrm[tid] / (cn[tid] > 1e-10 ? cn[tid] : 1.0);
-            const __half gh = double_to_half_rn(g);
-            g16[tid] = (double)__half2float(gh);
-            norms_s[sb * VB + tid] = __half2float(gh);
-        }
-        __syncthreads();
+        const double cn = sqrt(quarter_sum(cs));
+        double g = nrm;
+        if (a.norm_correction) g = nrm / (cn > 1e-10 ? cn : 1.0);
+        const __half gh = double_to_half_rn(g);
+        const double g16 = (double)__half2float(gh);
+        if (kq == 0) norms_s[t] = __half2float(gh);
         // residual in the rotated domain against the reconstruction the decoder will see
-        for (int i = tid; i < VB * 128; i += NT) {
-            const int v = i >> 7;
-            ys[i] = nrm[v] * ys[i] - g16[v] * xs[i];
-        }
-        __syncthreads();
-        norms_block(ys, 128, 128, cn);
-        if (tid < VB && tid < nvalid) rnorms[row0 + t0 + tid] = double_to_half_rn(cn[tid]);
-        rotate_block(rp, ys, xs);  // xs = (S R^T) e
-        for (int i = tid; i < VB * 16; i += NT) {
-            const int v = i >> 4, byte = i & 15;
-            if (v >= nvalid) continue;
-            unsigned bits = 0;
+        double rs = 0.0;
 #pragma unroll
-            for (int b = 0; b < 8; ++b) bits |= (xs[v * 128 + byte * 8 + b] >= 0.0 ? 1u : 0u) << b;
-            sign_bits[(row0 + t0 + v) * 16 + byte] = (uint8_t)bits;
+        for (int s = 0; s < 32; ++s) {
+            e[s] = nrm * e[s] - g16 * cent_s[(cw[s >> 3] >> (4 * (s & 7))) & 15u];
+            rs = fma(e[s], e[s], rs);
         }
-        __syncthreads();
+        const double rnorm = sqrt(quarter_sum(rs));
+        if (valid && kq == 0) rnorms[row0 + tok0 + t] = double_to_half_rn(rnorm);
+        // (S R^T) e for the 16 tokens: D[token][j] += E[token][k] M[k][j], 8 column blocks x 32 steps of 4
+        double4_t acc[8];
+#pragma unroll
+        for (int jb = 0; jb < 8; ++jb) acc[jb] = double4_t{0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const double *mrow = mat_s + (4 * s + kq) * 128 + n16;
+#pragma unroll
+            for (int jb = 0; jb < 8; ++jb) acc[jb] = __builtin_amdgcn_mfma_f64_16x16x4f64(e[s], mrow[16 * jb], acc[jb], 0, 0, 0);
+        }
+        // lane (n16, kq) now holds the projections j = 16 jb + n16 of tokens 4 i + kq (register i of the result)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t piece = 0;
+#pragma unroll
+            for (int jb = 0; jb < 8; ++jb) {
+                const uint64_t m = __builtin_amdgcn_ballot_w64(acc[jb][i] >= 0.0);
+                if (n16 == jb) piece = (uint32_t)(m >> (16 * kq)) & 0xFFFFu;
+            }
+            const int64_t tk = tok0 + u * 16 + 4 * i + kq;
+            if (n16 < 8 && tk < a.tokens) reinterpret_cast<uint16_t *>(sign_bits)[(row0 + tk) * 8 + n16] = (uint16_t)piece;
+        }
     }
-    pack_block<BITS, 128>(codes, norms_s, packed + blk * block_bytes(BITS), TQ_KIND_K);
+    __syncthreads();
+    pack_block<BITS, 512>(codes, norms_s, packed + blk * block_bytes(BITS), TQ_KIND_K);
+    __syncthreads();  // the code stage is free for the next block
+    }
 }
 
 // ---- K3: packed block -> values ----------------------------------------------------
@@ -1954,9 +2019,14 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
         a.projrot_t = h->projrot64_t;
         a.norm_correction = h->norm_correction;
         a.tokens = tokens; a.blocks_per_seq = bps;
-#define TQ_STOREQ_BITS(B)                                                                              \
-    DISPATCH_T(in_dtype, TI, (k_store_qjl<B, TI><<<grid, 128, 0, s>>>((const TI *)x, (uint8_t *)packed, \
-                                                                      sign_bits, (__half *)rnorms, a)))
+        constexpr int MAT_BYTES = 128 * 128 * (int)sizeof(double);
+        const unsigned qgrid = grid < 256u ? grid : 256u;  // one workgroup per CU (the matrix fills its LDS), looping over blocks
+#define TQ_STOREQ_BITS(B)                                                                                          \
+    DISPATCH_T(in_dtype, TI,                                                                                       \
+               ((void)hipFuncSetAttribute((const void *)k_store_qjl_mfma<B, TI>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                          MAT_BYTES),                                                              \
+                k_store_qjl_mfma<B, TI><<<qgrid, 512, MAT_BYTES, s>>>((const TI *)x, (uint8_t *)packed, sign_bits,  \
+                                                                      (__half *)rnorms, a, (int64_t)grid)))
         switch (h->bits) {
         case 2: TQ_STOREQ_BITS(2); break;
         case 3: TQ_STOREQ_BITS(3); break;
