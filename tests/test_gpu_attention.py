@@ -186,6 +186,25 @@ def test_decode_attention_bias_and_sparse_v():
             np.testing.assert_allclose(out_s, out_d, rtol=0, atol=1e-4 * np.abs(ref_d).max())
 
 
+@pytest.mark.parametrize("N,misalign", [(1000, 0), (1001, 0), (999, 0), (1000, 1), (64, 0), (67, 1)])
+def test_decode_attention_dense_bias_every_position(N, misalign):
+    """A bias that differs at every position, for context lengths that are and are not multiples of four and
+    for a bias buffer that is not 16-byte aligned: the 16-byte and the element-wise reads give the same."""
+    B, Hq, Hkv = 2, 8, 2
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=N + misalign)
+    rng = np.random.default_rng(N)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = (2.0 * rng.standard_normal((B, Hq, N))).astype(np.float32)
+    tt = L.torch()
+    buf = tt.zeros(B * Hq * N + 4, dtype=tt.float32, device="cuda")
+    bias_d = buf[misalign:misalign + B * Hq * N].view(B, Hq, N)
+    bias_d.copy_(tt.from_numpy(bias))
+    for n_splits in (1, 3):
+        out = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits)(q, kp, vp, bias=bias_d))
+        ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, bias=bias)
+        assert_close(out, ref)
+
+
 def test_decode_attention_masked_prefix():
     """-inf bias over a prefix: whole tiles and one whole split carry no weight; output stays finite and equals
     attention over the remaining positions."""

@@ -329,6 +329,26 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
+    // additive logit bias of this lane's head and four tokens (natural-log units), one 16-byte load when the row
+    // allows it; positions past the context read as 0 (they are masked anyway)
+    const bool bias_vec = a.bias && (a.tokens & 3) == 0 && (reinterpret_cast<uintptr_t>(a.bias) & 15u) == 0;
+    auto load_bias = [&](int t, float (&bv)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[i] = 0.0f;
+        if (!a.bias) return;
+        const int tk = t * 64 + b4;  // the launcher checks tokens < 2^31
+        const float *row = a.bias + ((int64_t)group * 4 + j) * a.tokens;
+        if (bias_vec && tk + 3 < (int)a.tokens) {
+            const float4 v = *reinterpret_cast<const float4 *>(row + tk);
+            bv[0] = v.x; bv[1] = v.y; bv[2] = v.z; bv[3] = v.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (tk + i < (int)a.tokens) bv[i] = row[tk + i];
+        }
+    };
+    float bias_next[4];
+    load_bias(min(t_begin, max(t_end - 1, 0)), bias_next);
     unsigned nskip = 0;
     bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
@@ -351,14 +371,12 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         const int tile_n = min(tile_next, t_end - 1);
         const int row_n = (tile_n & 1) * 64 + lane;
         const uint2 gvu_next = load_vnorm(tile_n);
-        float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-        const int tok0 = tile * 64 + b4;                 // the launcher checks tokens < 2^31
         const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
-        if (a.bias) {
+        // the bias of this tile was requested a tile ago, like the rows; now the next tile's
+        float bias4[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (b4 + i < n_valid) bias4[i] = a.bias[((int64_t)group * 4 + j) * a.tokens + tok0 + i] * LOG2E;
-        }
+        for (int i = 0; i < 4; ++i) bias4[i] = bias_next[i] * LOG2E;
+        load_bias(tile_n, bias_next);
 
         // ---- QK ------------------------------------------------------------------
         // D_b[head][token 4b + lane%4]: every lane gets the 4 heads' dot products of its own token
