@@ -172,12 +172,20 @@ __device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const
 template <int... G>
 __device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const uint32_t (&kw)[32],
                                       const half4_t (&qa)[2], float4_t (&acc)[4]) {
+    // int8 -> fp16 without conversions: 0x6400 | (x + 128) is the fp16 number 1024 + (x + 128), exactly, so a byte
+    // permute builds two of them at once and one packed fp16 subtraction of 1152 leaves (x0, x2) and (x1, x3).  The
+    // values come out in the order 0, 2, 1, 3; the kernel parks its queries in the same order.
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     auto cvt = [](uint32_t w) {
+        const uint32_t u = w ^ 0x80808080u;
+        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const half2_t h02 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04020400u)) - bias;
+        const half2_t h13 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030401u)) - bias;
         half4_t kv;
-        kv[0] = (_Float16)(int)(int8_t)(w & 0xff);
-        kv[1] = (_Float16)(int)(int8_t)((w >> 8) & 0xff);
-        kv[2] = (_Float16)(int)(int8_t)((w >> 16) & 0xff);
-        kv[3] = (_Float16)(int)(int8_t)(w >> 24);
+        kv[0] = h02[0];
+        kv[1] = h02[1];
+        kv[2] = h13[0];
+        kv[3] = h13[1];
         return kv;
     };
     ((acc[G >> 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], cvt(kw[G]), acc[G >> 3])), ...);
@@ -310,8 +318,12 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
             x0 *= a.ks2[2 * lane] * RSQRT128;
             x1 *= a.ks2[2 * lane + 1] * RSQRT128;
         }
-        qw[2 * lane] = (_Float16)(x0 * a.scale_log2e);
-        qw[2 * lane + 1] = (_Float16)(x1 * a.scale_log2e);
+        // q8_0-style K rows hand their four values of a dim group over in the order 0, 2, 1, 3 (qk_q8)
+        const int d0 = 2 * lane, d1 = 2 * lane + 1;
+        const int p0 = KFMT == KFMT_Q8 ? (d0 & ~3) | ((d0 & 1) << 1) | ((d0 >> 1) & 1) : d0;
+        const int p1 = KFMT == KFMT_Q8 ? (d1 & ~3) | ((d1 & 1) << 1) | ((d1 >> 1) & 1) : d1;
+        qw[p0] = (_Float16)(x0 * a.scale_log2e);
+        qw[p1] = (_Float16)(x1 * a.scale_log2e);
     }
     __syncthreads();
     half4_t qa[2];
