@@ -202,7 +202,8 @@ int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q
 /* ---- attention over packed KV ------------------------------------------------ */
 
 typedef struct tq_attn_params {
-    int32_t batch, n_q_heads, n_kv_heads;  /* GQA group = n_q_heads / n_kv_heads, must be 4 */
+    int32_t batch, n_q_heads, n_kv_heads;  /* GQA group = n_q_heads / n_kv_heads; the kernels take */
+                                           /* four heads of a group per pass over K/V (4 is free) */
     int64_t tokens;                        /* context length per sequence                    */
     int64_t capacity;                      /* tokens per sequence the K/V buffers are laid   */
                                            /* out for (tq_append caches); 0 = tokens         */

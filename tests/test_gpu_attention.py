@@ -270,10 +270,46 @@ def test_decode_attention_q8_0_k_turbo2_v():
             assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
 
 
-def test_decode_attention_rejects_unsupported_group():
+def test_decode_attention_rejects_ragged_group():
     kc, vc = tqa.TurboCodec(3), tqa.TurboCodec(3)
-    with pytest.raises(NotImplementedError, match="GQA"):
-        tqa.DecodeAttention(kc, vc, 1, 8, 1, 128)
+    with pytest.raises(ValueError, match="multiple of the KV head count"):
+        tqa.DecodeAttention(kc, vc, 1, 7, 2, 128)
+
+
+@pytest.mark.parametrize("G,n_splits", [(1, 3), (2, 16), (3, 1), (5, 3), (7, 16), (8, 4), (12, 64)])
+def test_decode_attention_other_group_sizes(G, n_splits):
+    """Query-head groups other than four: passes of four heads over the same K/V, short last pass included,
+    with a logit bias per (head, position) and the Sparse V count summed over the passes."""
+    B, Hkv, N = 2, 3, 1500
+    Hq = G * Hkv
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=900 + G)
+    rng = np.random.default_rng(901 + G)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = (0.5 * rng.standard_normal((B, Hq, N))).astype(np.float32)
+    bias_d = L.torch().from_numpy(bias).cuda()
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits)
+    out = np_(attn(q, kp, vp, bias=bias_d)).copy()
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), bias=bias)
+    assert_close(out, ref)
+    # every head of a group against the same head served alone (G = 1 layout, same K/V): bitwise when the split
+    # count is the same, since a head's arithmetic does not depend on which row of the four it sits in
+    for h in (0, G - 1):
+        sel = [kv * G + h for kv in range(Hkv)]
+        one = tqa.DecodeAttention(kc, vc, B, Hkv, Hkv, N, n_splits=n_splits)
+        got = np_(one(np.ascontiguousarray(q[:, sel]), kp, vp, bias=L.torch().from_numpy(np.ascontiguousarray(bias[:, sel])).cuda()))
+        assert np.array_equal(got, out[:, sel])
+    tau = 1e-3
+    sparse = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+    out_s = np_(sparse(q, kp, vp, bias=bias_d)).copy()
+    ref_s, skip_o, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau,
+                                           bias=bias)
+    assert_close(out_s, ref_s)
+    rate = sparse.skip_rate()
+    assert abs(rate - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4, (rate, skip_o)
+    assert int(sparse.skip.cpu()[1]) == B * Hq * N
+    # a second call gives the same count (the passes add to a count that the first pass resets)
+    sparse(q, kp, vp, bias=bias_d)
+    assert sparse.skip_rate() == rate
 
 
 @pytest.mark.parametrize("projection,nk,nq", [("orthogonal", 1000, 200), ("gaussian", 1000, 200),

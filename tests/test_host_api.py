@@ -45,9 +45,11 @@ def test_size_entry_points_need_no_gpu():
     p = L.TQAttnParams(batch=16, n_q_heads=32, n_kv_heads=8, tokens=32768, n_splits=16,
                        k_format=L.KFMT_TURBO, scale=0.088, sparse_v_tau=0.0)
     assert lib.tq_attn_workspace_bytes(C.byref(p)) > 16 * 8 * 16 * 4 * 128 * 4
-    p.n_q_heads = 16
+    p.n_q_heads = 16                                       # groups of 2: two of the four head rows per pass idle
+    assert lib.tq_attn_workspace_bytes(C.byref(p)) > 16 * 8 * 16 * 4 * 128 * 4
+    p.n_q_heads = 20                                       # not a multiple of the KV head count
     assert lib.tq_attn_workspace_bytes(C.byref(p)) == -1
-    assert "GQA" in L.last_error()
+    assert "multiple of the KV head count" in L.last_error()
 
 
 def test_argument_errors_map_to_reference_exceptions():

@@ -155,6 +155,7 @@ struct AttnArgs {
     unsigned long long *skip_slots;  // Sparse V: [workgroup] (query, position) pairs it skipped
     int64_t tokens, blocks_per_seq;
     int n_groups, n_splits, tiles_per_split, n_tiles;
+    int q_group, head_off;  // query heads per KV head; first of the (up to) four heads this launch works on
     float tau;
 };
 
@@ -296,7 +297,8 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     // head, two values per lane), scaled and parked as fp16 in 1 KB of LDS for everybody.
     for (int h = wave; h < 4; h += n_waves) {
         _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + h * 128;
-        const int64_t e = ((int64_t)group * 4 + h) * 128 + 2 * lane;
+        // heads past the group's last one repeat it (their results are not written)
+        const int64_t e = ((int64_t)group * a.q_group + min(a.head_off + h, a.q_group - 1)) * 128 + 2 * lane;
         float x0, x1;
         if (a.q_dtype == TQ_F16) {
             const __half *qp = reinterpret_cast<const __half *>(a.q);
@@ -349,7 +351,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         for (int i = 0; i < 4; ++i) bv[i] = 0.0f;
         if (!a.bias) return;
         const int tk = t * 64 + b4;  // the launcher checks tokens < 2^31
-        const float *row = a.bias + ((int64_t)group * 4 + j) * a.tokens;
+        const float *row = a.bias + ((int64_t)group * a.q_group + min(a.head_off + j, a.q_group - 1)) * a.tokens;
         if (bias_vec && tk + 3 < (int)a.tokens) {
             const float4 v = *reinterpret_cast<const float4 *>(row + tk);
             bv[0] = v.x; bv[1] = v.y; bv[2] = v.z; bv[3] = v.w;
@@ -457,7 +459,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
             p[i] = __builtin_amdgcn_exp2f(s[i] - m_ref);  // results below 2^-126 flush to zero
             l_run += p[i];
             if constexpr (SPARSE) {
-                const bool in_range = b4 + i < n_valid;
+                const bool in_range = b4 + i < n_valid && a.head_off + j < a.q_group;
                 const bool keep = p[i] >= a.tau;
                 if (in_range && !keep) ++nskip;
                 if (!keep) p[i] = 0.0f;
@@ -558,6 +560,7 @@ struct SkipArgs {
     int n_slots;
     unsigned long long *skip;  // NULL: no bookkeeping asked for
     unsigned long long total_pairs;
+    int accumulate;            // a later launch of the same step: add to skip[0] instead of setting it
 };
 __device__ __forceinline__ void sum_skip_slots(const SkipArgs &k) {
     if (!k.skip || blockIdx.x != 0) return;
@@ -570,7 +573,7 @@ __device__ __forceinline__ void sum_skip_slots(const SkipArgs &k) {
     if ((threadIdx.x & 63) == 0 && t) atomicAdd(&acc, t);
     __syncthreads();
     if (threadIdx.x == 0) {
-        k.skip[0] = acc;
+        k.skip[0] = (k.accumulate ? k.skip[0] : 0ull) + acc;
         k.skip[1] = k.total_pairs;
     }
 }
@@ -582,12 +585,14 @@ __device__ __forceinline__ void sum_skip_slots(const SkipArgs &k) {
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
                                                           int64_t n_rows, int n_splits, const float *s1, const float *s2,
-                                                          SkipArgs sk) {
+                                                          SkipArgs sk, int q_group, int head_off) {
     sum_skip_slots(sk);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t r = blockIdx.x;  // row = group*4 + head
     const int64_t group = r >> 2;
     const int head = (int)(r & 3);
+    if (head_off + head >= q_group) return;  // a repeated head of a group with fewer than four left
+    const int64_t r_out = group * q_group + head_off + head;
     const float *ml = part_ml + (group * n_splits * 4 + head) * 2;   // + s*8
     const float *po = part_o + (group * n_splits * 4 + head) * 128;  // + s*512
     float M = -INFINITY;
@@ -634,20 +639,23 @@ __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, c
     o0 *= invL * s2[2 * lane];
     o1 *= invL * s2[2 * lane + 1];
     wht128_wave(o0, o1, lane);
-    out[r * 128 + 2 * lane] = o0 * (s1[2 * lane] * RSQRT128);
-    out[r * 128 + 2 * lane + 1] = o1 * (s1[2 * lane + 1] * RSQRT128);
+    out[r_out * 128 + 2 * lane] = o0 * (s1[2 * lane] * RSQRT128);
+    out[r_out * 128 + 2 * lane + 1] = o1 * (s1[2 * lane + 1] * RSQRT128);
 }
 
 // the same merge for at most four partials per row: one wavefront per row, every load issued before
 // anything is waited for (one trip to memory instead of three)
 __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, const float *part_ml, float *out, int64_t n_rows,
-                                                          int n_parts, const float *s1, const float *s2, SkipArgs sk) {
+                                                          int n_parts, const float *s1, const float *s2, SkipArgs sk, int q_group,
+                                                          int head_off) {
     sum_skip_slots(sk);
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
     if (r >= n_rows) return;
     const int64_t group = r >> 2;
     const int head = (int)(r & 3);
+    if (head_off + head >= q_group) return;
+    const int64_t r_out = group * q_group + head_off + head;
     const float *ml = part_ml + (group * n_parts * 4 + head) * 2;   // + p*8
     const float *po = part_o + (group * n_parts * 4 + head) * 128;  // + p*512
     float m[4], l[4];
@@ -677,7 +685,7 @@ __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, c
     o0 *= invL * s2v.x;
     o1 *= invL * s2v.y;
     wht128_wave(o0, o1, lane);
-    *reinterpret_cast<float2 *>(out + r * 128 + 2 * lane) = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
+    *reinterpret_cast<float2 *>(out + r_out * 128 + 2 * lane) = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
 }
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -764,6 +772,12 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     const size_t merge_bytes = wpw > 1 ? (size_t)wpw * MERGE_FLOATS * sizeof(float) : 0;
     const int vb = hv->bits;
     const int kb = turbo_k ? hk->bits : 8;
+    // The kernels work on four query heads of a KV head at a time (the 4-row MFMA block): a group of G heads takes
+    // ceil(G / 4) passes over the same K/V, each with its own merge launch; a last pass with fewer than four
+    // heads repeats the group's last head and does not write the repeats.
+    a.q_group = p->n_q_heads / p->n_kv_heads;
+    const int64_t rows4 = (int64_t)groups * 4;
+    for (a.head_off = 0; a.head_off < a.q_group; a.head_off += 4) {
 #define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, merge_bytes, s>>>(a)
 #define TQ_ATTN(KF, KB, VB)                         \
     if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
@@ -797,10 +811,18 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     sk.n_slots = sparse ? (int)grid : 0;
     sk.skip = skip_count;
     sk.total_pairs = total_pairs;
-    if (n_parts >= 64) k_attn_combine<16><<<(unsigned)rows, 1024, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
-    else if (n_parts > 4) k_attn_combine<4><<<(unsigned)rows, 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
-    else k_attn_combine_few<<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows, n_parts, hv->s1_32, hv->s2_32, sk);
-    return tq_check_launch("attn_combine");
+    sk.accumulate = a.head_off > 0;
+    if (n_parts >= 64)
+        k_attn_combine<16><<<(unsigned)rows4, 1024, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group, a.head_off);
+    else if (n_parts > 4)
+        k_attn_combine<4><<<(unsigned)rows4, 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group, a.head_off);
+    else
+        k_attn_combine_few<<<(unsigned)((rows4 + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group,
+                                                                      a.head_off);
+    rc = tq_check_launch("attn_combine");
+    if (rc) return rc;
+    }
+    return TQ_OK;
 }
 
 // ---- prefill-shaped TurboQuant inner-product estimator --------------------------------

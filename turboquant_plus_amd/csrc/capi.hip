@@ -550,8 +550,8 @@ static int check_attn(const tq_attn_params *p) {
     REQUIRE(p, TQ_ERR_ARG, "attention: null params");
     REQUIRE(p->batch >= 1 && p->n_q_heads >= 1 && p->n_kv_heads >= 1 && p->tokens >= 1 && p->n_splits >= 1, TQ_ERR_ARG,
             "attention: sizes must be positive");
-    REQUIRE(p->n_q_heads == 4 * p->n_kv_heads, TQ_ERR_UNSUPPORTED,
-            "attention: GQA group must be 4 query heads per KV head (got %d / %d)", p->n_q_heads, p->n_kv_heads);
+    REQUIRE(p->n_q_heads % p->n_kv_heads == 0, TQ_ERR_ARG,
+            "attention: the query head count must be a multiple of the KV head count (got %d / %d)", p->n_q_heads, p->n_kv_heads);
     REQUIRE(p->k_format == TQ_KFMT_TURBO || p->k_format == TQ_KFMT_Q8_0, TQ_ERR_ARG, "attention: bad k_format %d",
             p->k_format);
     REQUIRE(p->tokens < ((int64_t)1 << 36), TQ_ERR_UNSUPPORTED, "attention: context too long");

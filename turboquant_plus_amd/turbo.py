@@ -293,7 +293,10 @@ def probe_mfma_f16(iters: int, sink) -> int:
 
 
 class DecodeAttention:
-    """softmax(scale * q k^T) v over packed K/V for GQA groups of 4 query heads.
+    """softmax(scale * q k^T) v over packed K/V; n_q_heads a multiple of n_kv_heads.
+
+    The kernels take four query heads of a KV head per pass over its K/V, so a
+    group of 4 reads the cache once and a group of G reads it ceil(G / 4) times.
 
     Holds the parameter block and the split workspace so that repeated steps
     allocate nothing.  K is a turbo buffer (k_codec given) or a q8_0-style
@@ -314,7 +317,7 @@ class DecodeAttention:
                                      sparse_v_tau=sparse_v_tau)
         nbytes = L.lib().tq_attn_workspace_bytes(C.byref(self.params))
         if nbytes < 0:
-            L.check(L.ERR_UNSUPPORTED if n_q_heads != 4 * n_kv_heads else L.ERR_ARG)
+            L.check(L.ERR_ARG)
         self.workspace = tt.empty(int(nbytes), dtype=tt.uint8, device=dev)
         self.skip = tt.zeros(2, dtype=tt.int64, device=dev)
         self.out = tt.empty((batch, n_q_heads, HEAD_DIM), dtype=tt.float32, device=dev)
