@@ -198,6 +198,14 @@ int64_t tq_q8_0_bytes(int64_t n_seqs, int64_t tokens);
 int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream);
 /* q [n_seqs, tokens, 128] int8 and scales [n_seqs, tokens, 4] fp32 of such a buffer. */
 int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream);
+/* The same arithmetic for V rows (the boundary layers of the fork's Boundary V policy keep V as q8_0,
+ * docs/papers/layer-aware-v-compression.md:83-87; no reference code): blocks of the same size, values
+ * dim-major inside 64-token tiles as the decode kernel reads V (row 64*tile + dim % 64 of a block holds
+ * dims dim and dim + 64 of the tile's 64 tokens), then [2 tiles][4][64 tokens] fp16 scales.  Positions
+ * past `tokens` in the last block hold zeros.  tq_q8_0_unpack_v gives q and scales in token order as
+ * tq_q8_0_unpack does. */
+int tq_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream);
+int tq_q8_0_unpack_v(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream);
 
 /* ---- attention over packed KV ------------------------------------------------ */
 
@@ -210,6 +218,7 @@ typedef struct tq_attn_params {
     int32_t n_splits;                      /* context splits per (batch, kv head), >= 1; a   */
                                            /* multiple of 16 lets 16 splits share a workgroup */
     int32_t k_format;                      /* TQ_KFMT_TURBO | TQ_KFMT_Q8_0                   */
+    int32_t v_format;                      /* the same for V: TQ_KFMT_TURBO (0) | TQ_KFMT_Q8_0 */
     float scale;                           /* logit scale, e.g. 1/sqrt(128)                  */
     float sparse_v_tau;                    /* 0 = dense; skip V rows with weight < tau       */
 } tq_attn_params;
@@ -221,9 +230,9 @@ int64_t tq_attn_workspace_bytes(const tq_attn_params *p);
  * evaluated on stored codes; no reference kernel exists).
  *   q      [batch, n_q_heads, 128] q_dtype, in the ORIGINAL domain; the kernel
  *          rotates it with the K handle's rotation (or leaves it for q8_0 K);
- *   k/v    packed buffers of [batch*n_kv_heads] sequences (tq_store), or for
- *          TQ_KFMT_Q8_0: k = int8 [batch*n_kv_heads, tokens, 128], k_aux = fp16
- *          scales [.., tokens, 4];
+ *   k/v    packed buffers of [batch*n_kv_heads] sequences: tq_store (kind K / V) buffers for
+ *          TQ_KFMT_TURBO, tq_q8_0_store / tq_q8_0_store_v buffers for TQ_KFMT_Q8_0 (then the
+ *          handle of that side may be NULL; a q8_0 V is not rotated); k_aux is unused;
  *   bias   optional additive logit bias [batch, n_q_heads, tokens] fp32 or NULL;
  *   out    [batch, n_q_heads, 128] fp32, original domain;
  *   skip_count optional uint64[2]: {skipped (query, position) pairs, total pairs}. */

@@ -22,7 +22,7 @@ def np_(t):
 
 
 def reference_attention(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, n_splits=1, tau=0.0, bias=None,
-                        k_q8=None):
+                        k_q8=None, v_q8=None):
     """Oracle attention on the GPU-stored codes -> (out [B,Hq,128], skip rate, final-weight rate)."""
     G = Hq // Hkv
     if k_q8 is None:
@@ -33,8 +33,12 @@ def reference_attention(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, n_s
         qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, N)
         k_rot = O.q8_0_dequantize(np_(qq), np_(ss))
         q_rot = q.astype(np.float64)
-    vi, vg = vc.unpack_codes(v_packed, B * Hkv, N, kind="v")
-    v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids)
+    if v_q8 is None:
+        vi, vg = vc.unpack_codes(v_packed, B * Hkv, N, kind="v")
+        v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids)
+    else:  # q8_0-style V: stored unrotated
+        qq, ss = tqa.q8_0_unpack(v_q8, B * Hkv, N, kind="v")
+        v_rot = O.q8_0_dequantize(np_(qq), np_(ss))
     out = np.zeros((B, Hq, D))
     skipped = below = 0.0
     for b in range(B):
@@ -44,7 +48,7 @@ def reference_attention(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, n_s
             bb = None if bias is None else bias[b, h * G:(h + 1) * G]
             o, sk, fr = O.decode_attention(qs, k_rot[g], v_rot[g], scale, n_splits=n_splits, sparse_v_tau=tau,
                                            logit_bias=bb)
-            out[b, h * G:(h + 1) * G] = O.rotate_fast(o, vc.signs1, vc.signs2, D, transpose=True)
+            out[b, h * G:(h + 1) * G] = o if v_q8 is not None else O.rotate_fast(o, vc.signs1, vc.signs2, D, transpose=True)
             skipped += sk
             below += fr
     return out, skipped / (B * Hkv), below / (B * Hkv)
@@ -268,6 +272,46 @@ def test_decode_attention_q8_0_k_turbo2_v():
         assert_close(out, ref)
         if tau:
             assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
+
+
+@pytest.mark.parametrize("kbits,N,n_splits,G", [(None, 2048 + 64, 3, 4), (None, 1000, 16, 4), (3, 1500, 8, 4),
+                                                (4, 777, 1, 4), (None, 4096, 32, 2), (3, 300, 2, 6)])
+def test_decode_attention_q8_0_v(kbits, N, n_splits, G):
+    """V kept as q8_0-style rows (the boundary layers of a layer-adaptive policy), K q8_0-style or turbo.
+    The values differ a lot from block to block so that a scale taken from the wrong 32-dim block or the wrong
+    token shows."""
+    B, Hkv = 2, 2
+    Hq = G * Hkv
+    rng = np.random.default_rng(1000 + N)
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = (rng.standard_normal((B * Hkv, N, D)) * np.repeat([0.05, 1.0, 7.0, 0.4], 32) *
+         np.exp(rng.standard_normal((B * Hkv, N, 1)))).astype(np.float16)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    kc = tqa.TurboCodec(kbits, seed=42) if kbits else None
+    kp = kc.store(k, kind="k") if kbits else tqa.q8_0_store(k)[0]
+    vq, _, _ = tqa.q8_0_store(v, kind="v")
+    for tau in (0.0, 1e-3):
+        attn = tqa.DecodeAttention(kc, None, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+        out = np_(attn(q, kp, vq))
+        ref, skip_o, _ = reference_attention(q, kc, None, kp, None, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau,
+                                             k_q8=None if kbits else kp, v_q8=vq)
+        assert_close(out, ref)
+        if tau:
+            assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
+    # against the exact values: int8 rows keep V to about 1 % of each 32-value block's largest entry
+    if not kbits:
+        vt = tqa.TurboCodec(4, seed=542)
+        out_t = np_(tqa.DecodeAttention(None, vt, B, Hq, Hkv, N, n_splits=n_splits)(q, kp, vt.store(v, kind="v"))).copy()
+        qq, ss = tqa.q8_0_unpack(kp, B * Hkv, N)
+        k_hat = O.q8_0_dequantize(np_(qq), np_(ss))
+        exact = np.zeros((B, Hq, D))
+        for b in range(B):
+            for h in range(Hq):
+                g = b * Hkv + h // G
+                w = O.softmax_rows((q[b, h].astype(np.float64) @ k_hat[g].T / np.sqrt(D))[None])[0]
+                exact[b, h] = w @ v[g].astype(np.float64)
+        out8 = np_(tqa.DecodeAttention(None, None, B, Hq, Hkv, N, n_splits=n_splits)(q, kp, vq))
+        assert np.abs(out8 - exact).max() < 0.25 * np.abs(out_t - exact).max()
 
 
 def test_decode_attention_rejects_ragged_group():

@@ -303,3 +303,40 @@ def test_q8_0_store_bit_exact(tokens):
     q2, s2 = tqa.q8_0_unpack(tqa.q8_0_store(x16)[0], 2, tokens)
     q_o, s_o = O.q8_0_quantize(x16.astype(np.float32))
     assert np.array_equal(np_(q2), q_o) and np.array_equal(np_(s2).astype(np.float16).view(np.uint16), s_o.view(np.uint16))
+
+
+@pytest.mark.parametrize("tokens", [64, 128, 200, 1000])
+def test_q8_0_store_v_bit_exact_and_layout(tokens):
+    """V rows: the same values and scales as the K buffer holds, at the positions the decode kernel reads them
+    from (dim-major inside 64-token tiles), and zeros past the sequence's end."""
+    x = np.random.default_rng(5).standard_normal((2, tokens, D)).astype(np.float32)
+    x[1, 3, 64:96] = 0
+    q_o, s_o = O.q8_0_quantize(x)
+    for arr in (x, x.astype(np.float64)):
+        packed, n_seqs, t = tqa.q8_0_store(arr, kind="v")
+        assert (n_seqs, t) == (2, tokens) and packed.numel() == 2 * (-(-tokens // 128)) * 128 * 136
+        q, s = tqa.q8_0_unpack(packed, 2, tokens, kind="v")
+        assert np.array_equal(np_(q), q_o)
+        assert np.array_equal(np_(s).astype(np.float16).view(np.uint16), s_o.view(np.uint16))
+    x16 = x.astype(np.float16)
+    q2, s2 = tqa.q8_0_unpack(tqa.q8_0_store(x16, kind="v")[0], 2, tokens, kind="v")
+    q_o16, s_o16 = O.q8_0_quantize(x16.astype(np.float32))
+    assert np.array_equal(np_(q2), q_o16) and np.array_equal(np_(s2).astype(np.float16).view(np.uint16), s_o16.view(np.uint16))
+    # the layout, restated on the host: byte of (token t, dim) and scale of (t, 32-dim group)
+    raw = np_(packed).reshape(2, -1, 128 * 136)
+    tt, dd = np.meshgrid(np.arange(tokens), np.arange(D), indexing="ij")
+    tb = tt % 128
+    off = (4 * (dd // 64) + (tb % 64) // 16) * 2048 + (64 * (tb // 64) + dd % 64) * 16 + tb % 16
+    got = raw[:, tt // 128, off].view(np.int8)
+    assert np.array_equal(got, q_o)
+    sc = raw[:, :, 8 * 2048:].copy().view(np.float16).reshape(2, -1, 2, 4, 64)
+    tk, gq = np.meshgrid(np.arange(tokens), np.arange(4), indexing="ij")
+    assert np.array_equal(sc[:, tk // 128, (tk % 128) // 64, gq, tk % 64].view(np.uint16), s_o.view(np.uint16))
+    if tokens % 128:
+        pad = np.ones((raw.shape[1] * 128, D), dtype=bool)
+        pad[:tokens] = False
+        tp, dp = np.nonzero(pad)
+        tb = tp % 128
+        offp = (4 * (dp // 64) + (tb % 64) // 16) * 2048 + (64 * (tb // 64) + dp % 64) * 16 + tb % 16
+        assert not raw[:, tp // 128, offp].any()
+

@@ -30,7 +30,8 @@ class TQConfig(C.Structure):
 
 class TQAttnParams(C.Structure):
     _fields_ = [("batch", C.c_int32), ("n_q_heads", C.c_int32), ("n_kv_heads", C.c_int32), ("tokens", C.c_int64),
-                ("capacity", C.c_int64), ("n_splits", C.c_int32), ("k_format", C.c_int32), ("scale", C.c_float), ("sparse_v_tau", C.c_float)]
+                ("capacity", C.c_int64), ("n_splits", C.c_int32), ("k_format", C.c_int32), ("v_format", C.c_int32),
+                ("scale", C.c_float), ("sparse_v_tau", C.c_float)]
 
 
 _P, _I, _L, _D = C.c_void_p, C.c_int, C.c_int64, C.c_double
@@ -67,6 +68,8 @@ PROTOTYPES = {
     "tq_q8_0_bytes": (_L, [_L, _L]),
     "tq_q8_0_store": (_I, [_P, _L, _L, _I, _P, _P]),
     "tq_q8_0_unpack": (_I, [_P, _L, _L, _P, _P, _P]),
+    "tq_q8_0_store_v": (_I, [_P, _L, _L, _I, _P, _P]),
+    "tq_q8_0_unpack_v": (_I, [_P, _L, _L, _P, _P, _P]),
     "tq_attn_workspace_bytes": (_L, [C.POINTER(TQAttnParams)]),
     "tq_decode_attention": (_I, [_P, _P, C.POINTER(TQAttnParams), _P, _I, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
     "tq_score_tile": (_I, [_P, _P, _I, _L, _P, _P, _P, _L, _P, _I, _P, _L, _P]),

@@ -22,6 +22,10 @@
 //         4b..4b+3] -> D_b = out[4 heads][4 dims].  16 token groups x 2 dim halves = 32
 //         MFMAs per tile into 16 accumulator registers; no cross-lane reduction at the
 //         end of the split and no LDS traffic besides the LUT reads.
+//   q8_0-style V (VBITS = 8): the same dim-major rows hold int8 values, and the four fp16 scales of a token
+//   (one per 32 dims) go into the weights: block b covers dims of one 32-dim block per dim half, so the A
+//   operand is broadcast inside each half of the wavefront (cbsz = 3) from weights that were multiplied by that
+//   half's scales.
 //   Online softmax in base 2 (log2(e) folded into the query scale).  The wavefronts
 //   of a workgroup (up to 16 splits) merge their results in LDS and write one partial.
 // k_attn_combine / k_attn_combine_few: log-sum-exp merge of the workgroups' partials,
@@ -50,7 +54,9 @@ template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t 
 }
 
 // bytes of the decode table of a codebook: quad entries for BITS <= 3, pair entries for 4
-__host__ __device__ constexpr int lut_bytes(int bits) { return bits <= 3 ? 8 << (4 * bits) : 4 << (2 * bits); }
+__host__ __device__ constexpr int lut_bytes(int bits) {
+    return bits == 8 ? 0 : bits <= 3 ? 8 << (4 * bits) : 4 << (2 * bits);  // 8: int8 rows, no table
+}
 
 // the four values of quad Q (pairs 2Q, 2Q+1) of a row as an MFMA operand
 template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_t (&w)[4 * BITS], const char *lut, int Q) {
@@ -105,6 +111,28 @@ __device__ __forceinline__ float4_t mfma4(half4_t a, half4_t b, float4_t c) {
 // 4x4x4 MFMA whose A operand is taken from block ABID and broadcast to all 16 blocks
 template <int ABID> __device__ __forceinline__ float4_t mfma4_bcast(half4_t a, half4_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 4, ABID, 0);
+}
+
+// the same with the A operand taken from block ABID of each group of 8 blocks (lanes 0..31 and 32..63 apart)
+template <int ABID> __device__ __forceinline__ float4_t mfma4_bcast8(half4_t a, half4_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 3, ABID, 0);
+}
+
+// four int8 of a dword as fp16, in the order 0, 2, 1, 3: 0x6400 | (x + 128) is the fp16 number 1024 + (x + 128),
+// exactly, so a byte permute builds two of them at once and one packed fp16 subtraction of 1152 leaves (x0, x2)
+// and (x1, x3)
+__device__ __forceinline__ half4_t int8x4_to_half_0213(uint32_t w) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    const uint32_t u = w ^ 0x80808080u;
+    const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const half2_t h02 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04020400u)) - bias;
+    const half2_t h13 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030401u)) - bias;
+    half4_t kv;
+    kv[0] = h02[0];
+    kv[1] = h02[1];
+    kv[2] = h13[0];
+    kv[3] = h13[1];
+    return kv;
 }
 
 // transpose the 4x4 matrix held by a quad of lanes (element [lane%4][register]), two exchange stages
@@ -173,23 +201,8 @@ __device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const
 template <int... G>
 __device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const uint32_t (&kw)[32],
                                       const half4_t (&qa)[2], float4_t (&acc)[4]) {
-    // int8 -> fp16 without conversions: 0x6400 | (x + 128) is the fp16 number 1024 + (x + 128), exactly, so a byte
-    // permute builds two of them at once and one packed fp16 subtraction of 1152 leaves (x0, x2) and (x1, x3).  The
-    // values come out in the order 0, 2, 1, 3; the kernel parks its queries in the same order.
-    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-    auto cvt = [](uint32_t w) {
-        const uint32_t u = w ^ 0x80808080u;
-        const half2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-        const half2_t h02 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04020400u)) - bias;
-        const half2_t h13 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u, 0x04030401u)) - bias;
-        half4_t kv;
-        kv[0] = h02[0];
-        kv[1] = h02[1];
-        kv[2] = h13[0];
-        kv[3] = h13[1];
-        return kv;
-    };
-    ((acc[G >> 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], cvt(kw[G]), acc[G >> 3])), ...);
+    // the values of a dim group come out in the order 0, 2, 1, 3; the kernel parks its queries in the same order
+    ((acc[G >> 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], int8x4_to_half_0213(kw[G]), acc[G >> 3])), ...);
 }
 
 // PV over the 16 token groups x 2 dim halves: A = weights of block T (broadcast), B = this lane's V row
@@ -202,6 +215,24 @@ __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const u
      ...);
 }
 
+// q8_0-style V rows: dword 16*hf + T of the row = tokens 4T..4T+3 of dim half hf as int8.  a_lo / a_hi: the weights
+// (times the scales of this half-wavefront's 32-dim block of dim half hf) that token groups T < 8 / T >= 8 take
+// from block T % 8 of each half-wavefront.
+template <int... T>
+__device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, const uint32_t (&vw)[32],
+                                          const half4_t (&a_lo)[2], const half4_t (&a_hi)[2], float4_t (&acc_o)[2][2]) {
+    ((acc_o[0][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[0] : a_hi[0], int8x4_to_half_0213(vw[T]), acc_o[0][T & 1]),
+      acc_o[1][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[1] : a_hi[1], int8x4_to_half_0213(vw[16 + T]), acc_o[1][T & 1])),
+     ...);
+}
+
+// per-tile side data of the V rows: turbo = the fp16 norms of this lane's four tokens; q8_0-style = the fp16 scales
+// [2 * dim half + swapped]: of this lane's four tokens (0) and of the four tokens of lane ^ 32 (1), for the 32-dim
+// block that this lane's dims of that dim half lie in
+template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 1]; };
+
+constexpr float Q8V_PRESCALE = 64.0f;  // keeps weight * scale products out of fp16's subnormals; 65504 / 64 > any scale
+
 // SHARE: K and V decode through one table (same width, same centroids); table positions are
 // compile-time constants so that they fold into the LDS instructions' offset fields.
 //
@@ -212,11 +243,15 @@ __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const u
 // in flight to stay busy.  So the wavefronts of a workgroup publish their progress in LDS and
 // each sets its own issue priority to how many tiles it is behind the leader (at most 3):
 // they finish within a tile or two of each other.
+// int8 V rows take 32 registers instead of 8 to 16: those variants run with at most 8 wavefronts per workgroup,
+// which leaves each more than the 128 registers of a 16-wavefront workgroup.
+__host__ __device__ constexpr int max_waves_per_workgroup(int vbits) { return vbits == 8 ? 8 : 16; }
+
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE>
-__global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
-    constexpr int VBLOCK = TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
+    constexpr int VBLOCK = VBITS == 8 ? TQ_ROWS_PER_BLOCK * 136 : TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
     constexpr int KLUT_BYTES = KFMT == KFMT_TURBO ? lut_bytes(KBITS) : 0;
     static_assert(!SHARE || (KFMT == KFMT_TURBO && KBITS == VBITS), "a shared table needs equal code widths");
     // static LDS (its address is a compile-time constant, so table positions fold into the LDS
@@ -262,12 +297,25 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         else
             return *reinterpret_cast<const uint2 *>(kb + 8 * 2048 + 8 * r);
     };
-    // V: fp16 norms of this lane's four tokens 4b..4b+3
-    auto load_vnorm = [&](int tile) -> uint2 {
-        return *reinterpret_cast<const uint2 *>(vbase + (int64_t)(tile >> 1) * VBLOCK + TQ_ROWS_PER_BLOCK * 16 * VBITS +
-                                                2 * ((tile & 1) * 64 + b4));
+    // V: fp16 norms of this lane's four tokens 4b..4b+3, or their q8_0-style scales ([tile][32-dim block][token])
+    auto load_vnorm = [&](int tile) -> VSide<VBITS> {
+        VSide<VBITS> r;
+        const uint8_t *side = vbase + (int64_t)(tile >> 1) * VBLOCK + TQ_ROWS_PER_BLOCK * 16 * VBITS;
+        if constexpr (VBITS == 8) {
+            const int bh = lane >> 5;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                r.v[e] = *reinterpret_cast<const uint2 *>(side + 2 * ((((tile & 1) * 4 + 2 * (e >> 1) + bh) * 64) +
+                                                                      (e & 1 ? b4 ^ 32 : b4)));
+        } else {
+            r.v[0] = *reinterpret_cast<const uint2 *>(side + 2 * ((tile & 1) * 64 + b4));
+        }
+        return r;
     };
-    uint2 kn = make_uint2(0u, 0u), gvu = make_uint2(0u, 0u);
+    uint2 kn = make_uint2(0u, 0u);
+    VSide<VBITS> gvu;
+#pragma unroll
+    for (auto &e : gvu.v) e = make_uint2(0u, 0u);
     int tile = t_begin;
     if (tile < t_end) {
         const int row0 = (tile & 1) * 64 + lane;
@@ -336,7 +384,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     }
     __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
     if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
-    if constexpr (!SHARE) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
+    if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
     __syncthreads();
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[2][2];
@@ -384,7 +432,7 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
         const int tile_next = tile + 1;
         const int tile_n = min(tile_next, t_end - 1);
         const int row_n = (tile_n & 1) * 64 + lane;
-        const uint2 gvu_next = load_vnorm(tile_n);
+        const VSide<VBITS> gvu_next = load_vnorm(tile_n);
         const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
         float bias4[4];
@@ -480,15 +528,45 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
 
         // ---- PV ------------------------------------------------------------------------
         // weights (times the stored V norm) as fp16: this lane is token group T = lane/4, head lane%4
-        half4_t pv;
-        pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.x & 0xffff))));
-        pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.x >> 16))));
-        pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.y & 0xffff))));
-        pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.y >> 16))));
-        // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; quad 2T + hf =
-        // tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
-        // weights of token group T sit in block T and are broadcast to every block.
-        pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
+        if constexpr (VBITS == 8) {
+            // The dims of block b lie in 32-dim block b / 8 (+ 2 for the upper dim half), so the weights carry that
+            // block's scale and are broadcast inside each half of the wavefront: token group T is served by block
+            // T % 8 of both halves, which therefore also needs the weights of the lane 32 away.
+            float ps[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ps[i] = __shfl_xor(p[i], 32);
+            auto weights = [&](const float (&w)[4], uint2 sc) {
+                const float s0 = __half2float(__ushort_as_half((unsigned short)(sc.x & 0xffff))) * Q8V_PRESCALE;
+                const float s1 = __half2float(__ushort_as_half((unsigned short)(sc.x >> 16))) * Q8V_PRESCALE;
+                const float s2 = __half2float(__ushort_as_half((unsigned short)(sc.y & 0xffff))) * Q8V_PRESCALE;
+                const float s3 = __half2float(__ushort_as_half((unsigned short)(sc.y >> 16))) * Q8V_PRESCALE;
+                half4_t r;  // token order 0, 2, 1, 3, as int8x4_to_half_0213 hands the values over
+                r[0] = (_Float16)(w[0] * s0);
+                r[1] = (_Float16)(w[2] * s2);
+                r[2] = (_Float16)(w[1] * s1);
+                r[3] = (_Float16)(w[3] * s3);
+                return r;
+            };
+            const bool upper = lane >= 32;
+            half4_t a_lo[2], a_hi[2];
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const half4_t own = weights(p, gvu.v[2 * hf]), swp = weights(ps, gvu.v[2 * hf + 1]);
+                a_lo[hf] = upper ? swp : own;
+                a_hi[hf] = upper ? own : swp;
+            }
+            pv_all_q8(std::make_integer_sequence<int, 16>{}, vw, a_lo, a_hi, acc_o);
+        } else {
+            half4_t pv;
+            pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x & 0xffff))));
+            pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x >> 16))));
+            pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y & 0xffff))));
+            pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y >> 16))));
+            // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; quad 2T + hf =
+            // tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
+            // weights of token group T sit in block T and are broadcast to every block.
+            pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
+        }
         load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
         v_ahead = true;
         gvu = gvu_next;
@@ -496,6 +574,10 @@ __global__ __launch_bounds__(1024) void k_decode_attn(AttnArgs a) {
     }
 
     // ---- end of split: the workgroup's wavefronts merge their partials in LDS and write one ------
+    if constexpr (VBITS == 8) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] *= 1.0f / Q8V_PRESCALE;
+    }
     const float l_tot = sum_over_blocks(l_run);
     if (n_waves == 1) {
 #pragma unroll
@@ -636,6 +718,11 @@ __global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, c
         o1 += (red[q][2 * lane + 1] + red[q + 1][2 * lane + 1]) + (red[q + 2][2 * lane + 1] + red[q + 3][2 * lane + 1]);
     }
     const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+    if (!s1) {  // V rows were stored unrotated
+        out[r_out * 128 + 2 * lane] = o0 * invL;
+        out[r_out * 128 + 2 * lane + 1] = o1 * invL;
+        return;
+    }
     o0 *= invL * s2[2 * lane];
     o1 *= invL * s2[2 * lane + 1];
     wht128_wave(o0, o1, lane);
@@ -667,8 +754,8 @@ __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, c
         l[p] = p < n_parts ? ml[pc * 8 + 1] : 0.0f;
         v[p] = *reinterpret_cast<const float2 *>(po + (int64_t)pc * 512 + 2 * lane);
     }
-    const float2 s1v = *reinterpret_cast<const float2 *>(s1 + 2 * lane);
-    const float2 s2v = *reinterpret_cast<const float2 *>(s2 + 2 * lane);
+    const float2 s1v = s1 ? *reinterpret_cast<const float2 *>(s1 + 2 * lane) : make_float2(1.0f, 1.0f);
+    const float2 s2v = s1 ? *reinterpret_cast<const float2 *>(s2 + 2 * lane) : make_float2(1.0f, 1.0f);
     float M = -INFINITY;
 #pragma unroll
     for (int p = 0; p < 4; ++p)
@@ -682,6 +769,10 @@ __global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, c
         o1 = fmaf(v[p].y, w, o1);
     }
     const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+    if (!s1) {  // V rows were stored unrotated
+        *reinterpret_cast<float2 *>(out + r_out * 128 + 2 * lane) = make_float2(o0 * invL, o1 * invL);
+        return;
+    }
     o0 *= invL * s2v.x;
     o1 *= invL * s2v.y;
     wht128_wave(o0, o1, lane);
@@ -740,8 +831,10 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.k = (const uint8_t *)k;
     a.v = (const uint8_t *)v;
     a.klut = turbo_k ? (const uint32_t *)hk->pair_lut : nullptr;
-    a.vlut = (const uint32_t *)hv->pair_lut;
-    const bool share = turbo_k && hk->bits == hv->bits &&
+    const bool turbo_v = p->v_format == TQ_KFMT_TURBO;
+    a.vlut = turbo_v ? (const uint32_t *)hv->pair_lut : nullptr;
+    const float *vs1 = turbo_v ? hv->s1_32 : nullptr, *vs2 = turbo_v ? hv->s2_32 : nullptr;
+    const bool share = turbo_k && turbo_v && hk->bits == hv->bits &&
                        std::memcmp(hk->pair_lut_host, hv->pair_lut_host, sizeof(hk->pair_lut_host)) == 0;
     a.bias = bias;
     a.part_o = part_o;
@@ -763,14 +856,14 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: sparse_v_tau > 0 needs skip_count");
         return TQ_ERR_ARG;
     }
-    // wavefronts per workgroup: the largest power of two up to 16 that divides the split count
-    int wpw = 16;
+    // wavefronts per workgroup: the largest power of two up to 16 (8 for int8 V rows) that divides the split count
+    int wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? hv->bits : 8);
     while (p->n_splits % wpw) wpw >>= 1;
     const unsigned grid = (unsigned)((int64_t)groups * (p->n_splits / wpw));
     const unsigned wg = 64u * (unsigned)wpw;
     const int n_parts = p->n_splits / wpw;  // partials per group: the wavefronts of a workgroup merge theirs in LDS
     const size_t merge_bytes = wpw > 1 ? (size_t)wpw * MERGE_FLOATS * sizeof(float) : 0;
-    const int vb = hv->bits;
+    const int vb = turbo_v ? hv->bits : 8;
     const int kb = turbo_k ? hk->bits : 8;
     // The kernels work on four query heads of a KV head at a time (the 4-row MFMA block): a group of G heads takes
     // ceil(G / 4) passes over the same K/V, each with its own merge launch; a last pass with fewer than four
@@ -796,6 +889,9 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     else if (!turbo_k && vb == 2) { TQ_ATTN(KFMT_Q8, 3, 2); }
     else if (!turbo_k && vb == 3) { TQ_ATTN(KFMT_Q8, 3, 3); }
     else if (!turbo_k && vb == 4) { TQ_ATTN(KFMT_Q8, 3, 4); }
+    else if (!turbo_k && vb == 8) { TQ_ATTN(KFMT_Q8, 3, 8); }
+    else if (turbo_k && kb == 3 && vb == 8) { TQ_ATTN(KFMT_TURBO, 3, 8); }
+    else if (turbo_k && kb == 4 && vb == 8) { TQ_ATTN(KFMT_TURBO, 4, 8); }
     else {
         tq_set_error("tq_decode_attention: unsupported K/V format pair (k bits %d, v bits %d)", kb, vb);
         return TQ_ERR_UNSUPPORTED;
@@ -813,11 +909,11 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     sk.total_pairs = total_pairs;
     sk.accumulate = a.head_off > 0;
     if (n_parts >= 64)
-        k_attn_combine<16><<<(unsigned)rows4, 1024, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group, a.head_off);
+        k_attn_combine<16><<<(unsigned)rows4, 1024, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group, a.head_off);
     else if (n_parts > 4)
-        k_attn_combine<4><<<(unsigned)rows4, 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group, a.head_off);
+        k_attn_combine<4><<<(unsigned)rows4, 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group, a.head_off);
     else
-        k_attn_combine_few<<<(unsigned)((rows4 + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, hv->s1_32, hv->s2_32, sk, a.q_group,
+        k_attn_combine_few<<<(unsigned)((rows4 + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group,
                                                                       a.head_off);
     rc = tq_check_launch("attn_combine");
     if (rc) return rc;

@@ -543,7 +543,18 @@ int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, v
 
 int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream) {
     REQUIRE(q && scales && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_unpack: bad argument");
-    return tqk_q8_0_unpack(packed, n_seqs, tokens, q, scales, (hipStream_t)stream);
+    return tqk_q8_0_unpack(packed, n_seqs, tokens, q, scales, TQ_KIND_K, (hipStream_t)stream);
+}
+
+int tq_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream) {
+    REQUIRE(x && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_store_v: bad argument");
+    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_store_v: packed must be 16-byte aligned");
+    return tqk_q8_0_store_v(x, n_seqs, tokens, in_dtype, packed, (hipStream_t)stream);
+}
+
+int tq_q8_0_unpack_v(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream) {
+    REQUIRE(q && scales && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_unpack_v: bad argument");
+    return tqk_q8_0_unpack(packed, n_seqs, tokens, q, scales, TQ_KIND_V, (hipStream_t)stream);
 }
 
 static int check_attn(const tq_attn_params *p) {
@@ -554,6 +565,8 @@ static int check_attn(const tq_attn_params *p) {
             "attention: the query head count must be a multiple of the KV head count (got %d / %d)", p->n_q_heads, p->n_kv_heads);
     REQUIRE(p->k_format == TQ_KFMT_TURBO || p->k_format == TQ_KFMT_Q8_0, TQ_ERR_ARG, "attention: bad k_format %d",
             p->k_format);
+    REQUIRE(p->v_format == TQ_KFMT_TURBO || p->v_format == TQ_KFMT_Q8_0, TQ_ERR_ARG, "attention: bad v_format %d",
+            p->v_format);
     REQUIRE(p->tokens < ((int64_t)1 << 36), TQ_ERR_UNSUPPORTED, "attention: context too long");
     REQUIRE(p->capacity == 0 || p->capacity >= p->tokens, TQ_ERR_ARG, "attention: capacity %lld < tokens %lld",
             (long long)p->capacity, (long long)p->tokens);
@@ -571,8 +584,10 @@ int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_
                         unsigned long long *skip_count, void *workspace, int64_t workspace_bytes, void *stream) {
     int rc = check_attn(p);
     if (rc) return rc;
-    rc = check_fast(hv, "tq_decode_attention (V)");
-    if (rc) return rc;
+    if (p->v_format == TQ_KFMT_TURBO) {
+        rc = check_fast(hv, "tq_decode_attention (V)");
+        if (rc) return rc;
+    }
     if (p->k_format == TQ_KFMT_TURBO) {
         rc = check_fast(hk, "tq_decode_attention (K)");
         if (rc) return rc;

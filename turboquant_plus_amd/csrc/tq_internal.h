@@ -89,7 +89,8 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
 int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
                      float *norms, hipStream_t s);
 int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
-int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, hipStream_t s);
+int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
+int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, int kind, hipStream_t s);
 
 int64_t tqk_attn_workspace_bytes(const tq_attn_params *p);
 int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q, int q_dtype,

@@ -1919,8 +1919,50 @@ __global__ __launch_bounds__(256) void k_q8_0_store_f16(const __half *x, uint8_t
     }
 }
 
+// q8_0-style V blocks: the same 32-value groups and arithmetic, laid out as the decode kernel reads V rows.
+// Byte of (token t of the block, dim): 16-byte chunk 4 * (dim / 64) + (t % 64) / 16 of row 64 * (t / 64) + dim % 64,
+// byte t % 16; scale of (t, 32-dim group gq): fp16 [t / 64][gq][t % 64] behind the values.
+__device__ __forceinline__ int q8v_byte(int t, int dim) {
+    return (4 * (dim >> 6) + ((t & 63) >> 4)) * 2048 + (64 * (t >> 6) + (dim & 63)) * 16 + (t & 15);
+}
+__device__ __forceinline__ int q8v_scale(int t, int gq) { return ((t >> 6) * 4 + gq) * 64 + (t & 63); }
+
+// One thread per 32-value group; the block image is put together in LDS and leaves as one contiguous copy, with
+// zeros at the positions past the sequence's end.
+template <typename TI>
+__global__ __launch_bounds__(256) void k_q8_0_store_v(const TI *x, uint8_t *packed, int64_t tokens, int64_t blocks_per_seq) {
+    __shared__ __attribute__((aligned(16))) uint8_t img[TQ_ROWS_PER_BLOCK * 136];
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    for (int u = threadIdx.x; u < TQ_ROWS_PER_BLOCK * 4; u += 256) {
+        // consecutive threads take consecutive tokens of one group, so their bytes share LDS words rarely
+        const int t = u & 127, gq = u >> 7;
+        const bool valid = tok0 + t < tokens;
+        float v[32];
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            v[j] = valid ? ld1(x + (seq * tokens + tok0 + t) * 128 + gq * 32 + j) : 0.0f;
+            amax = fmaxf(amax, fabsf(v[j]));
+        }
+        const float d = amax / 127.0f;
+        const float id = d > 0.0f ? 1.0f / d : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const float tq = v[j] * id;
+            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            img[q8v_byte(t, gq * 32 + j)] = (uint8_t)(qv & 0xFF);
+        }
+        reinterpret_cast<__half *>(img + 8 * 2048)[q8v_scale(t, gq)] = __float2half_rn(d);
+    }
+    __syncthreads();
+    uint4 *dst = reinterpret_cast<uint4 *>(packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136));
+    for (int i = threadIdx.x; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) dst[i] = reinterpret_cast<const uint4 *>(img)[i];
+}
+
 __global__ __launch_bounds__(256) void k_q8_0_unpack(const uint8_t *packed, int8_t *q, float *scales, int64_t tokens,
-                                                     int64_t blocks_per_seq) {
+                                                     int64_t blocks_per_seq, int kind) {
     const int64_t blk = blockIdx.x;
     const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
@@ -1928,12 +1970,14 @@ __global__ __launch_bounds__(256) void k_q8_0_unpack(const uint8_t *packed, int8
     for (int e = threadIdx.x; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
         const int t = e >> 7, dim = e & 127;
         if (tok0 + t >= tokens) continue;
-        q[(seq * tokens + tok0 + t) * 128 + dim] = (int8_t)block[(dim >> 4) * 2048 + t * 16 + (dim & 15)];
+        q[(seq * tokens + tok0 + t) * 128 + dim] =
+            (int8_t)block[kind == TQ_KIND_V ? q8v_byte(t, dim) : (dim >> 4) * 2048 + t * 16 + (dim & 15)];
     }
     for (int e = threadIdx.x; e < TQ_ROWS_PER_BLOCK * 4; e += 256) {
         const int t = e >> 2;
         if (tok0 + t >= tokens) continue;
-        scales[(seq * tokens + tok0 + t) * 4 + (e & 3)] = __half2float(reinterpret_cast<const __half *>(block + 8 * 2048)[e]);
+        scales[(seq * tokens + tok0 + t) * 4 + (e & 3)] =
+            __half2float(reinterpret_cast<const __half *>(block + 8 * 2048)[kind == TQ_KIND_V ? q8v_scale(t, e & 3) : e]);
     }
 }
 
@@ -2430,10 +2474,18 @@ int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, 
     return tq_check_launch("q8_0_store");
 }
 
-int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, hipStream_t s) {
+int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
-    k_q8_0_unpack<<<grid, 256, 0, s>>>((const uint8_t *)packed, q, scales, tokens, bps);
+    DISPATCH_T(in_dtype, TI, (k_q8_0_store_v<TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, tokens, bps)));
+    return tq_check_launch("q8_0_store_v");
+}
+
+int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, int kind, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    const unsigned grid = (unsigned)(n_seqs * bps);
+    if (grid == 0) return TQ_OK;
+    k_q8_0_unpack<<<grid, 256, 0, s>>>((const uint8_t *)packed, q, scales, tokens, bps, kind);
     return tq_check_launch("q8_0_unpack");
 }

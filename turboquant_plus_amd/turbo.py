@@ -255,20 +255,30 @@ class TurboCodec:
         return logits
 
 
-def q8_0_store(x):
-    """x [..., tokens, 128] -> q8_0-style K buffer (uint8), n_seqs, tokens."""
+def _kind_name(kind: str) -> str:
+    if kind not in ("k", "v"):
+        raise ValueError(f"kind must be 'k' or 'v', got {kind!r}")
+    return kind
+
+
+def q8_0_store(x, kind: str = "k"):
+    """x [..., tokens, 128] -> q8_0-style buffer (uint8), n_seqs, tokens.  kind="v" lays the same int8
+    values and scales out as the decode kernel reads V rows (dim-major inside 64-token tiles)."""
     tt = L.torch()
     xd, n_seqs, tokens = TurboCodec._as_seqs(x)
     out = tt.empty(int(L.lib().tq_q8_0_bytes(n_seqs, tokens)), dtype=tt.uint8, device=xd.device)
-    L.check(L.lib().tq_q8_0_store(L.ptr(xd), n_seqs, tokens, L.dtype_code(xd), L.ptr(out), L.stream_ptr()))
+    fn = L.lib().tq_q8_0_store if _kind_name(kind) == "k" else L.lib().tq_q8_0_store_v
+    L.check(fn(L.ptr(xd), n_seqs, tokens, L.dtype_code(xd), L.ptr(out), L.stream_ptr()))
     return out, n_seqs, tokens
 
 
-def q8_0_unpack(packed, n_seqs: int, tokens: int):
+def q8_0_unpack(packed, n_seqs: int, tokens: int, kind: str = "k"):
+    """int8 values [n_seqs, tokens, 128] and fp32 scales [n_seqs, tokens, 4] of a q8_0_store buffer."""
     tt = L.torch()
     q = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=tt.int8, device=packed.device)
     s = tt.empty((n_seqs, tokens, 4), dtype=tt.float32, device=packed.device)
-    L.check(L.lib().tq_q8_0_unpack(L.ptr(packed), n_seqs, tokens, L.ptr(q), L.ptr(s), L.stream_ptr()))
+    fn = L.lib().tq_q8_0_unpack if _kind_name(kind) == "k" else L.lib().tq_q8_0_unpack_v
+    L.check(fn(L.ptr(packed), n_seqs, tokens, L.ptr(q), L.ptr(s), L.stream_ptr()))
     return q, s
 
 
@@ -300,10 +310,11 @@ class DecodeAttention:
 
     Holds the parameter block and the split workspace so that repeated steps
     allocate nothing.  K is a turbo buffer (k_codec given) or a q8_0-style
-    buffer (k_codec None); V is always a turbo buffer written with kind="v".
+    buffer (k_codec None); V is a turbo buffer written with kind="v" (v_codec
+    given) or a q8_0_store(x, kind="v") buffer (v_codec None).
     """
 
-    def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec, batch: int, n_q_heads: int, n_kv_heads: int,
+    def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec | None, batch: int, n_q_heads: int, n_kv_heads: int,
                  tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0,
                  capacity: int = 0):
         tt = L.torch()
@@ -313,6 +324,7 @@ class DecodeAttention:
             n_splits = default_splits(batch * n_kv_heads, tokens)
         self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
                                      capacity=capacity, n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
+                                     v_format=L.KFMT_TURBO if v_codec is not None else L.KFMT_Q8_0,
                                      scale=(1.0 / math.sqrt(HEAD_DIM)) if scale is None else scale,
                                      sparse_v_tau=sparse_v_tau)
         nbytes = L.lib().tq_attn_workspace_bytes(C.byref(self.params))
@@ -326,7 +338,8 @@ class DecodeAttention:
         """q [batch, n_q_heads, 128] in the original domain -> out fp32 [batch, n_q_heads, 128]."""
         qd = L.to_device(q)
         hk = self.k_codec.handle.h if self.k_codec is not None else None
-        L.check(L.lib().tq_decode_attention(hk, self.v_codec.handle.h, C.byref(self.params), L.ptr(qd),
+        hv = self.v_codec.handle.h if self.v_codec is not None else None
+        L.check(L.lib().tq_decode_attention(hk, hv, C.byref(self.params), L.ptr(qd),
                                             L.dtype_code(qd), L.ptr(k_packed), None, L.ptr(v_packed), L.ptr(bias),
                                             L.ptr(self.out),
                                             L.ptr(self.skip if self.params.sparse_v_tau > 0 else None),
