@@ -206,6 +206,13 @@ int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q
  * tq_q8_0_unpack does. */
 int tq_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream);
 int tq_q8_0_unpack_v(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream);
+/* tq_append for q8_0-style buffers of either kind (laid out for `capacity` tokens per sequence,
+ * tq_q8_0_bytes(n_seqs, capacity)): same positions, truncation and ordering rules; after appends
+ * covering tokens 0 .. T-1 the touched blocks equal tq_q8_0_store's / tq_q8_0_store_v's of the
+ * first T tokens.  The buffer must start out zeroed: blocks that no append has touched are read by
+ * the attention kernel's last tile and must hold finite scales. */
+int tq_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
+                   void *packed, void *stream);
 
 /* ---- attention over packed KV ------------------------------------------------ */
 

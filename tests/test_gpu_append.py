@@ -298,3 +298,62 @@ def test_fork_blocks_rejects_wrong_width():
     codec = tqa.TurboCodec(3, seed=42)
     with pytest.raises(ValueError):
         codec.import_fork_blocks(np.zeros((1, 128, 66), dtype=np.uint8))
+
+
+# ---- q8_0-style buffers (boundary layers of a layer-adaptive policy) ---------------------------------------
+
+@pytest.mark.parametrize("kind", ["k", "v"])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_q8_0_append_in_chunks_equals_store(kind, dtype):
+    tt = L.torch()
+    n_seqs, capacity = 3, 512
+    x = np.random.default_rng(11).standard_normal((n_seqs, 300, D)).astype(dtype)
+    x[1, 5] = 0
+    cache = tt.zeros(128 * 136 * n_seqs * 4, dtype=tt.uint8, device="cuda")
+    pos = 0
+    for n_new in [1, 1, 62, 64, 5, 130, 37]:
+        tqa.q8_0_append(x[:, pos:pos + n_new], cache, pos, capacity, kind=kind)
+        pos += n_new
+        want = np_(tqa.q8_0_store(x[:, :pos], kind=kind)[0]).reshape(n_seqs, -1, 128 * 136)
+        got = np_(cache).reshape(n_seqs, -1, 128 * 136)
+        nb = want.shape[1]
+        assert np.array_equal(got[:, :nb], want), f"after {pos} tokens"
+        assert not got[:, nb:].any()
+    # a rewind truncates: the touched block holds the tokens before pos, the new ones, then zeros
+    tqa.q8_0_append(x[:, 100:103], cache, 200, capacity, kind=kind)
+    y = np.concatenate([x[:, :200], x[:, 100:103]], axis=1)
+    want = np_(tqa.q8_0_store(y, kind=kind)[0]).reshape(n_seqs, -1, 128 * 136)
+    got = np_(cache).reshape(n_seqs, -1, 128 * 136)
+    assert np.array_equal(got[:, :2], want)
+    with pytest.raises(ValueError):
+        tqa.q8_0_append(x[:, :10], cache, 510, capacity, kind=kind)
+
+
+@pytest.mark.parametrize("fmt", [("q8_0", "q8_0"), ("q8_0", "turbo2"), ("turbo3", "q8_0"), ("turbo3", "turbo3")])
+def test_layer_decode_loop_over_a_growing_cache(fmt):
+    """A layer of a layer-adaptive policy in a serving loop: prefill by one append, then single-token appends with
+    attention after each, against attention over a cache stored in one go."""
+    from test_gpu_attention import assert_close, reference_attention
+    B, Hq, Hkv, capacity = 2, 8, 2, 400
+    layer = tqa.LayerKV(tqa.LayerFormat(*fmt), seed=3)
+    rng = np.random.default_rng(12)
+    # fp32 input: the append and the store of fp32 rows share one arithmetic (fp16 rows are stored through the
+    # matrix-core rotation, which may round a value at a code boundary the other way)
+    k = rng.standard_normal((B * Hkv, 260, D)).astype(np.float32)
+    v = rng.standard_normal((B * Hkv, 260, D)).astype(np.float32)
+    kc, vc = layer.new_cache(B * Hkv, capacity)
+    attn = layer.attention(B, Hq, Hkv, 1, n_splits=2, capacity=capacity)
+    layer.append(k[:, :250], v[:, :250], kc, vc, 0, capacity)
+    pos = 250
+    for step in range(10):
+        layer.append(k[:, pos:pos + 1], v[:, pos:pos + 1], kc, vc, pos, capacity)
+        pos += 1
+        q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+        attn.set_tokens(pos)
+        out = np_(attn(q, kc, vc)).copy()
+        kp, vp = layer.store(k[:, :pos], v[:, :pos])
+        once = np_(layer.attention(B, Hq, Hkv, pos, n_splits=2)(q, kp, vp))
+        assert np.array_equal(out, once), f"step {step}"
+    ref, _, _ = reference_attention(q, layer.k_codec, layer.v_codec, kp, vp, B, Hq, Hkv, pos, 1 / np.sqrt(D),
+                                    k_q8=kp if layer.k_codec is None else None, v_q8=vp if layer.v_codec is None else None)
+    assert_close(out, ref)

@@ -70,6 +70,7 @@ PROTOTYPES = {
     "tq_q8_0_unpack": (_I, [_P, _L, _L, _P, _P, _P]),
     "tq_q8_0_store_v": (_I, [_P, _L, _L, _I, _P, _P]),
     "tq_q8_0_unpack_v": (_I, [_P, _L, _L, _P, _P, _P]),
+    "tq_q8_0_append": (_I, [_P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_attn_workspace_bytes": (_L, [C.POINTER(TQAttnParams)]),
     "tq_decode_attention": (_I, [_P, _P, C.POINTER(TQAttnParams), _P, _I, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
     "tq_score_tile": (_I, [_P, _P, _I, _L, _P, _P, _P, _L, _P, _I, _P, _L, _P]),

@@ -552,6 +552,18 @@ int tq_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype,
     return tqk_q8_0_store_v(x, n_seqs, tokens, in_dtype, packed, (hipStream_t)stream);
 }
 
+int tq_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
+                   void *packed, void *stream) {
+    REQUIRE(n_seqs >= 0 && pos >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_q8_0_append: bad argument");
+    REQUIRE(pos + n_new <= capacity, TQ_ERR_ARG, "tq_q8_0_append: tokens %lld..%lld do not fit a capacity of %lld",
+            (long long)pos, (long long)(pos + n_new), (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(x && packed, TQ_ERR_ARG, "tq_q8_0_append: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_q8_0_append: bad kind %d", kind);
+    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_append: packed must be 16-byte aligned");
+    return tqk_q8_0_append(x, n_seqs, pos, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream);
+}
+
 int tq_q8_0_unpack_v(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, void *stream) {
     REQUIRE(q && scales && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_unpack_v: bad argument");
     return tqk_q8_0_unpack(packed, n_seqs, tokens, q, scales, TQ_KIND_V, (hipStream_t)stream);

@@ -1961,6 +1961,51 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v(const TI *x, uint8_t *pack
     for (int i = threadIdx.x; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) dst[i] = reinterpret_cast<const uint4 *>(img)[i];
 }
 
+// Streaming append for both layouts: one workgroup per (sequence, touched block).  Tokens before `pos` stay, the
+// n_new tokens from `pos` on are quantised from x [n_seqs, n_new, 128], and the rest of the last touched block
+// becomes zeros (what the store kernels write past a sequence's end).  Bytes of neighbouring tokens share words in
+// the V layout; byte stores keep them apart.
+template <typename TI, int KIND>
+__global__ __launch_bounds__(256) void k_q8_0_append(const TI *x, uint8_t *packed, int64_t pos, int64_t n_new,
+                                                     int64_t blocks_per_seq, int64_t first_block, int64_t n_touched) {
+    const int64_t seq = blockIdx.x / n_touched, bis = first_block + blockIdx.x % n_touched;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    uint8_t *block = packed + (seq * blocks_per_seq + bis) * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
+    __half *scales = reinterpret_cast<__half *>(block + 8 * 2048);
+    for (int u = threadIdx.x; u < TQ_ROWS_PER_BLOCK * 4; u += 256) {
+        const int t = KIND == TQ_KIND_V ? u & 127 : u >> 2, gq = KIND == TQ_KIND_V ? u >> 7 : u & 3;
+        const int64_t tok = tok0 + t;
+        if (tok < pos) continue;
+        const bool valid = tok < pos + n_new;
+        float v[32];
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            v[j] = valid ? ld1(x + (seq * n_new + (tok - pos)) * 128 + gq * 32 + j) : 0.0f;
+            amax = fmaxf(amax, fabsf(v[j]));
+        }
+        const float d = amax / 127.0f;
+        const float id = d > 0.0f ? 1.0f / d : 0.0f;
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = 0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const float tq = v[j] * id;
+            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            if constexpr (KIND == TQ_KIND_V) block[q8v_byte(t, gq * 32 + j)] = (uint8_t)(qv & 0xFF);
+            else w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
+        }
+        if constexpr (KIND == TQ_KIND_V) {
+            scales[q8v_scale(t, gq)] = __float2half_rn(d);
+        } else {
+            *reinterpret_cast<uint4 *>(block + (2 * gq) * 2048 + t * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+            *reinterpret_cast<uint4 *>(block + (2 * gq + 1) * 2048 + t * 16) = make_uint4(w[4], w[5], w[6], w[7]);
+            scales[t * 4 + gq] = __float2half_rn(d);
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void k_q8_0_unpack(const uint8_t *packed, int8_t *q, float *scales, int64_t tokens,
                                                      int64_t blocks_per_seq, int kind) {
     const int64_t blk = blockIdx.x;
@@ -2480,6 +2525,22 @@ int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype
     if (grid == 0) return TQ_OK;
     DISPATCH_T(in_dtype, TI, (k_q8_0_store_v<TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, tokens, bps)));
     return tq_check_launch("q8_0_store_v");
+}
+
+int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
+                    void *packed, hipStream_t s) {
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    const int64_t bps = blocks_for(capacity);
+    const int64_t first = pos / TQ_ROWS_PER_BLOCK, n_touched = (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - first + 1;
+    const unsigned grid = (unsigned)(n_seqs * n_touched);
+    if (kind == TQ_KIND_V) {
+        DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_V><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
+                                                                                   bps, first, n_touched)));
+    } else {
+        DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_K><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
+                                                                                   bps, first, n_touched)));
+    }
+    return tq_check_launch("q8_0_append");
 }
 
 int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, int kind, hipStream_t s) {

@@ -19,7 +19,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-from .turbo import DecodeAttention, TurboCodec, q8_0_store
+from . import _lib as L
+from .turbo import DecodeAttention, TurboCodec, packed_bytes, q8_0_append, q8_0_store
 
 FORMATS = ("q8_0", "turbo4", "turbo3", "turbo2")
 
@@ -101,6 +102,33 @@ class LayerKV:
         kp = q8_0_store(k, kind="k")[0] if self.k_codec is None else self.k_codec.store(k, kind="k")
         vp = q8_0_store(v, kind="v")[0] if self.v_codec is None else self.v_codec.store(v, kind="v")
         return kp, vp
+
+    def new_cache(self, n_seqs: int, capacity: int):
+        """Zeroed (k, v) buffers for `capacity` tokens per sequence, to be filled by append()."""
+        tt = L.torch()
+        dev = L.require_gpu()
+
+        def nbytes(codec):
+            if codec is None:
+                return int(L.lib().tq_q8_0_bytes(n_seqs, capacity))
+            return packed_bytes(codec.bits, n_seqs, capacity)
+        return (tt.zeros(nbytes(self.k_codec), dtype=tt.uint8, device=dev),
+                tt.zeros(nbytes(self.v_codec), dtype=tt.uint8, device=dev))
+
+    def append(self, k, v, k_cache, v_cache, pos: int, capacity: int):
+        """The K and V tokens [n_seqs, n_new, 128] of a decode step at positions pos .. pos+n_new-1."""
+        if self.k_codec is not None and self.v_codec is not None:
+            self.k_codec.append_kv(self.v_codec, k, v, k_cache, v_cache, pos, capacity)
+            return k_cache, v_cache
+        if self.k_codec is None:
+            q8_0_append(k, k_cache, pos, capacity, kind="k")
+        else:
+            self.k_codec.append(k, k_cache, pos, capacity, kind="k")
+        if self.v_codec is None:
+            q8_0_append(v, v_cache, pos, capacity, kind="v")
+        else:
+            self.v_codec.append(v, v_cache, pos, capacity, kind="v")
+        return k_cache, v_cache
 
     def attention(self, batch: int, n_q_heads: int, n_kv_heads: int, tokens: int, **kw) -> DecodeAttention:
         return DecodeAttention(self.k_codec, self.v_codec, batch, n_q_heads, n_kv_heads, tokens, **kw)

@@ -272,6 +272,18 @@ def q8_0_store(x, kind: str = "k"):
     return out, n_seqs, tokens
 
 
+def q8_0_append(x, packed, pos: int, capacity: int, kind: str = "k"):
+    """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of a q8_0-style buffer laid
+    out for `capacity` tokens per sequence (zero-initialised; tq_q8_0_append)."""
+    xd, n_seqs, n_new = TurboCodec._as_seqs(x)
+    need = int(L.lib().tq_q8_0_bytes(n_seqs, capacity))
+    if packed.numel() < need:
+        raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
+    L.check(L.lib().tq_q8_0_append(L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
+                                   L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+    return packed
+
+
 def q8_0_unpack(packed, n_seqs: int, tokens: int, kind: str = "k"):
     """int8 values [n_seqs, tokens, 128] and fp32 scales [n_seqs, tokens, 4] of a q8_0_store buffer."""
     tt = L.torch()
