@@ -322,6 +322,8 @@ def test_q8_0_store_v_bit_exact_and_layout(tokens):
     q2, s2 = tqa.q8_0_unpack(tqa.q8_0_store(x16, kind="v")[0], 2, tokens, kind="v")
     q_o16, s_o16 = O.q8_0_quantize(x16.astype(np.float32))
     assert np.array_equal(np_(q2), q_o16) and np.array_equal(np_(s2).astype(np.float16).view(np.uint16), s_o16.view(np.uint16))
+    # fp16 rows take a kernel of their own: the same bytes, padding included, as the general one writes
+    assert np.array_equal(np_(tqa.q8_0_store(x16, kind="v")[0]), np_(tqa.q8_0_store(x16.astype(np.float32), kind="v")[0]))
     # the layout, restated on the host: byte of (token t, dim) and scale of (t, 32-dim group)
     raw = np_(packed).reshape(2, -1, 128 * 136)
     tt, dd = np.meshgrid(np.arange(tokens), np.arange(D), indexing="ij")

@@ -1961,6 +1961,66 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v(const TI *x, uint8_t *pack
     for (int i = threadIdx.x; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) dst[i] = reinterpret_cast<const uint4 *>(img)[i];
 }
 
+// fp16 input, 16-byte aligned: the block's 32 KB come in as 16-byte pieces that are contiguous across the lanes and
+// are parked in LDS in token order; one thread per 32-value group finds the scale; then one thread per (dim, 16
+// tokens) reads its column, quantises and stores one 16-byte chunk, so that 64 lanes write 1 KB in one piece.
+// Same arithmetic as k_q8_0_store_v.
+constexpr int Q8V_ROW = 256 + 16;  // LDS bytes per token: the padding spreads the 16-byte row reads over the banks
+__global__ __launch_bounds__(256) void k_q8_0_store_v_f16(const __half *x, uint8_t *packed, int64_t tokens, int64_t blocks_per_seq) {
+    __shared__ __attribute__((aligned(16))) uint8_t raw[TQ_ROWS_PER_BLOCK * Q8V_ROW];
+    __shared__ float inv[TQ_ROWS_PER_BLOCK * 4];
+    const int64_t blk = blockIdx.x;
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    uint8_t *block = packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
+    const int n_valid = (int)min((int64_t)TQ_ROWS_PER_BLOCK, tokens - tok0);
+    const uint4 *src = reinterpret_cast<const uint4 *>(x + (seq * tokens + tok0) * 128);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int i = threadIdx.x + 256 * k, t = i >> 4;
+        const uint4 v = t < n_valid ? src[i] : make_uint4(0u, 0u, 0u, 0u);
+        *reinterpret_cast<uint4 *>(raw + t * Q8V_ROW + (i & 15) * 16) = v;
+    }
+    __syncthreads();
+    __half *scales = reinterpret_cast<__half *>(block + 8 * 2048);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int u = threadIdx.x + 256 * k, t = u >> 2, gq = u & 3;
+        float amax = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(raw + t * Q8V_ROW + gq * 64 + c * 16);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                amax = fmaxf(amax, fabsf(__half2float(__ushort_as_half((unsigned short)(w[e] & 0xffff)))));
+                amax = fmaxf(amax, fabsf(__half2float(__ushort_as_half((unsigned short)(w[e] >> 16)))));
+            }
+        }
+        const float d = amax / 127.0f;
+        inv[u] = d > 0.0f ? 1.0f / d : 0.0f;
+        scales[q8v_scale(t, gq)] = __float2half_rn(d);
+    }
+    __syncthreads();
+    // unit = (16-token group c16 of the block, dim): lanes along dim % 64, so a wavefront stores 64 consecutive rows
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int u = threadIdx.x + 256 * k;
+        const int l = u & 63, hf = (u >> 6) & 1, c16 = u >> 7;  // c16 = 0..7: tile c16 / 4, tokens 16 * (c16 % 4) ..
+        const int dim = 64 * hf + l, gq = dim >> 5;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int t = 16 * c16 + e;
+            const float v = __half2float(*reinterpret_cast<const __half *>(raw + t * Q8V_ROW + 2 * dim));
+            const float tq = v * inv[t * 4 + gq];
+            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            w[e >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (e & 3));
+        }
+        *reinterpret_cast<uint4 *>(block + (4 * hf + (c16 & 3)) * 2048 + (64 * (c16 >> 2) + l) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 // Streaming append for both layouts: one workgroup per (sequence, touched block).  Tokens before `pos` stay, the
 // n_new tokens from `pos` on are quantised from x [n_seqs, n_new, 128], and the rest of the last touched block
 // becomes zeros (what the store kernels write past a sequence's end).  Bytes of neighbouring tokens share words in
@@ -2523,6 +2583,10 @@ int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype
     const int64_t bps = blocks_for(tokens);
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
+    if (in_dtype == TQ_F16 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed)) & 15u) == 0) {
+        k_q8_0_store_v_f16<<<grid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, tokens, bps);
+        return tq_check_launch("q8_0_store_v");
+    }
     DISPATCH_T(in_dtype, TI, (k_q8_0_store_v<TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, tokens, bps)));
     return tq_check_launch("q8_0_store_v");
 }
