@@ -342,6 +342,36 @@ def cpu_baseline(bits):
                        f"({dta * 1e3:.1f} ms), extrapolated x128", "host_cpus": os.cpu_count()})
 
 
+def boundary_layer_leg(torch, tqa, steps, warmup):
+    """A boundary layer of the fork's layer-adaptive modes (K and V kept as q8_0-style rows) at the config-3
+    shape: the V store of a prefill and the decode step."""
+    B, Hq, Hkv, N = 16, 32, 8, 32768
+    per = N * 136
+    kq = torch.empty(B * Hkv * per, dtype=torch.uint8, device="cuda")
+    vq = torch.empty_like(kq)
+    vsets = []
+    for b in range(B):
+        k = synth_kv(torch, Hkv, N, 600 + b, outliers=4)
+        v = synth_kv(torch, Hkv, N, 700 + b, outliers=0)
+        kq[b * Hkv * per:(b + 1) * Hkv * per] = tqa.q8_0_store(k)[0]
+        vq[b * Hkv * per:(b + 1) * Hkv * per] = tqa.q8_0_store(v, kind="v")[0]
+        if b < 4:
+            vsets.append(v)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    q = torch.randn((B, Hq, D), generator=g, device="cuda").to(torch.float16)
+    attn = tqa.DecodeAttention(None, None, B, Hq, Hkv, N)
+    _, ev_ms = time_steps(torch, lambda i: attn(q, kq, vq), steps, warmup)
+    algo = 2 * B * Hkv * per
+    us = ev_ms * 1e3
+    _, st_ms = time_steps(torch, lambda i: tqa.q8_0_store(vsets[i % 4], kind="v"), steps, warmup)
+    st_bytes = Hkv * N * (256 + 136)
+    return {"workload": "decode attention, K and V q8_0-style (136 B per row), B16 Hq32 Hkv8 ctx 32768",
+            "us_per_step": us, "n_splits": attn.params.n_splits, "algorithmic_bytes_per_step": algo,
+            "achieved_gbs": algo / (us * 1e-6) / 1e9, "frac": algo / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "v_store": {"vectors": Hkv * N, "us_per_call": st_ms * 1e3, "gbs": st_bytes / (st_ms * 1e-3) / 1e9,
+                        "note": "includes the allocation of the output buffer by the host wrapper"}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -377,6 +407,8 @@ def main():
     torch.cuda.empty_cache()
     tile = score_tile_leg(torch, tqa, args.steps, args.warmup)
     torch.cuda.empty_cache()
+    boundary = boundary_layer_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+    torch.cuda.empty_cache()
     peaks = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
     if args.skip_cpu:
         cpu_store = cpu_attn = None
@@ -396,7 +428,7 @@ def main():
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
         "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec, "asym_decode_q8k_turbo2v": asym,
-        "score_tile": tile, "measured_peaks": peaks,
+        "score_tile": tile, "boundary_layer_q8k_q8v": boundary, "measured_peaks": peaks,
     }
     print(json.dumps(line, ensure_ascii=False))
 
