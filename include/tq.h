@@ -175,6 +175,15 @@ int tq_import_fork_blocks(const tq_handle *h, const void *blocks, int64_t n_seqs
 int tq_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
             int out_dtype, int domain, void *stream);
 
+/* K and V of one layer back to fp16 in the original domain, the two tensors that
+ * KVCacheCompressor.decompress (kv_cache.py:143-165) returns together.  Same results as
+ * tq_load(hk, packed_k, .., TQ_KIND_K, out_k, TQ_F16, TQ_DOMAIN_ORIGINAL, ..) followed by
+ * tq_load(hv, packed_v, .., TQ_KIND_V, out_v, ..); out_k and out_v are [n_seqs, tokens, 128]
+ * fp16.  The two run as one kernel whose workgroups are divided between the tensors, so launch
+ * and pipeline-fill time is paid once. */
+int tq_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, const void *packed_v,
+               int64_t n_seqs, int64_t tokens, void *out_k, void *out_v, void *stream);
+
 /* Codebook indices [n_seqs, tokens, 128] uint8 and stored norms [n_seqs, tokens]
  * float32 of a packed buffer (test and interop aid; no reference counterpart). */
 int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind,

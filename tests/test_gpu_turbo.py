@@ -198,6 +198,39 @@ def test_load_fp16_matches_fp32_load(bits, kind, n_seqs, tokens):
     assert np.all(np.abs(got - ref) <= tol)
 
 
+@pytest.mark.parametrize("kbits,vbits", [(2, 2), (3, 3), (4, 4), (4, 2), (3, 4), (2, 3)])
+@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (8, 4096)])
+def test_load_kv_equals_two_loads(kbits, vbits, n_seqs, tokens):
+    """tq_load_kv (K and V of a layer to fp16 in one launch) returns the bytes of the two tq_load calls it
+    replaces, for every width pair, ragged sequence ends and grids smaller than the device, and writes nothing
+    past either output."""
+    tt = L.torch()
+    kc, vc = tqa.TurboCodec(kbits, seed=5), tqa.TurboCodec(vbits, seed=6)
+    k = kv_like(kbits + tokens, (n_seqs, tokens, D))
+    v = kv_like(vbits + tokens + 1, (n_seqs, tokens, D), outlier_channels=0)
+    pk, pv = kc.store_kv(vc, k, v)
+    n = n_seqs * tokens * D
+    ref_k = kc.load(pk, n_seqs, tokens, kind="k", domain="original", dtype=tt.float16)
+    ref_v = vc.load(pv, n_seqs, tokens, kind="v", domain="original", dtype=tt.float16)
+    ok = tt.full((n + 64,), 7.0, dtype=tt.float16, device="cuda")
+    ov = tt.full((n + 64,), 7.0, dtype=tt.float16, device="cuda")
+    kc.load_kv(vc, pk, pv, n_seqs, tokens, out_k=ok[:n], out_v=ov[:n])
+    assert (np_(ok[n:]) == 7.0).all() and (np_(ov[n:]) == 7.0).all(), "wrote past the last row"
+    assert tt.equal(ok[:n].view(tt.int16), ref_k.reshape(-1).view(tt.int16))
+    assert tt.equal(ov[:n].view(tt.int16), ref_v.reshape(-1).view(tt.int16))
+
+
+def test_load_kv_argument_errors():
+    tt = L.torch()
+    kc, vc = tqa.TurboCodec(3, seed=5), tqa.TurboCodec(3, seed=6)
+    pk = tt.zeros(tqa.packed_bytes(3, 1, 128), dtype=tt.uint8, device="cuda")
+    with pytest.raises(ValueError):
+        kc.load_kv(vc, pk, pk[:100], 1, 128)
+    with pytest.raises(ValueError):
+        kc.load_kv(vc, pk, pk, 1, 128, out_k=tt.zeros(5, dtype=tt.float16, device="cuda"))
+    assert L.lib().tq_load_kv(kc.handle.h, vc.handle.h, None, None, 1, 128, None, None, None) == L.ERR_ARG
+
+
 def test_config1_polarquant_turbo3_roundtrip(golden):
     """BASELINE config 1 end to end on the GPU: 4096 fp32 vectors, seed 0, one
     seed-1 sign diagonal, 8-level codebook; indices against the fixture the

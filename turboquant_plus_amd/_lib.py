@@ -63,6 +63,7 @@ PROTOTYPES = {
     "tq_export_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
     "tq_import_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
     "tq_load": (_I, [_P, _P, _L, _L, _I, _P, _I, _I, _P]),
+    "tq_load_kv": (_I, [_P, _P, _P, _P, _L, _L, _P, _P, _P]),
     "tq_unpack_codes": (_I, [_P, _P, _L, _L, _I, _P, _P, _P]),
     "tq_store_qjl": (_I, [_P, _P, _L, _L, _I, _P, _P, _P, _P]),
     "tq_q8_0_bytes": (_L, [_L, _L]),

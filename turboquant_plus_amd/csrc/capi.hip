@@ -524,6 +524,19 @@ int tq_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t toke
     return tqk_load(h, packed, n_seqs, tokens, kind, out, out_dtype, domain, (hipStream_t)stream);
 }
 
+int tq_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, const void *packed_v, int64_t n_seqs,
+               int64_t tokens, void *out_k, void *out_v, void *stream) {
+    int rc = check_fast(hk, "tq_load_kv");
+    rc = rc ? rc : check_fast(hv, "tq_load_kv");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_load_kv: bad argument");
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(packed_k && packed_v && out_k && out_v, TQ_ERR_ARG, "tq_load_kv: null pointer");
+    REQUIRE(aligned16(packed_k) && aligned16(packed_v) && aligned16(out_k) && aligned16(out_v), TQ_ERR_ALIGN,
+            "tq_load_kv: inputs and outputs must be 16-byte aligned");
+    return tqk_load_kv(hk, hv, packed_k, packed_v, n_seqs, tokens, out_k, out_v, (hipStream_t)stream);
+}
+
 int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
                     float *norms, void *stream) {
     int rc = check_fast(h, "tq_unpack_codes");

@@ -86,6 +86,8 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
                  int in_dtype, void *packed_k, void *packed_v, hipStream_t s);
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
              int out_dtype, int domain, hipStream_t s);
+int tqk_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, const void *packed_v, int64_t n_seqs,
+                int64_t tokens, void *out_k, void *out_v, hipStream_t s);
 int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, uint8_t *idx,
                      float *norms, hipStream_t s);
 int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);

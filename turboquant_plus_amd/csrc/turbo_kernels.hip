@@ -1635,16 +1635,18 @@ __device__ __forceinline__ void unrotate_unit16(const half8_t (&af)[8], const ui
     }
 }
 
+constexpr int LOAD16_XROW = 256 + 16;  // bytes per token row of the transposition space (padding spreads the banks)
+constexpr int LOAD16_XPOSE_BYTES = 4 * 16 * LOAD16_XROW;
+
+// Workgroup `bid` of `nb` running the K-row loop; the LDS arrays belong to the calling kernel
+// (lut_s: 1 << 2 BITS dwords, frag_s: 512 uint4, s1_s: 128 floats, xpose_s: LOAD16_XPOSE_BYTES).
 template <int BITS>
-__global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half *out, LoadK16Args a) {
-    __shared__ uint32_t lut_s[1 << (2 * BITS)];
-    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+__device__ __forceinline__ void load_k16_body(const uint8_t *packed, __half *out, const LoadK16Args &a, uint32_t bid, uint32_t nb,
+                                              uint32_t *lut_s, uint4 *frag_s, float *s1_s, uint8_t *xpose_s) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kc = lane >> 4;
     for (int e = tid; e < (1 << (2 * BITS)); e += 256) lut_s[e] = a.pair_lut[e];
-    __shared__ float s1_s[128];
-    constexpr int XROW = 256 + 16;  // bytes per token row of the transposition space (padding spreads the banks)
-    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[4 * 16 * XROW];
+    constexpr int XROW = LOAD16_XROW;
     frag_s[tid] = a.afrag[tid];
     frag_s[256 + tid] = a.afrag[256 + tid];
     if (tid < 128) s1_s[tid] = a.s1[tid];
@@ -1669,15 +1671,15 @@ __global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half 
     };
     uint32_t cw_next[BITS];
     __half g_next;
-    fetch(blockIdx.x * 4 + wave, cw_next, g_next);
+    fetch(bid * 4 + wave, cw_next, g_next);
 #pragma unroll 1
-    for (uint32_t u = blockIdx.x * 4 + wave; u < a.n_units; u += gridDim.x * 4) {
+    for (uint32_t u = bid * 4 + wave; u < a.n_units; u += nb * 4) {
         const uint32_t blk = u >> 3, seq = blk / bps, bis = blk - seq * bps;
         uint32_t cw[BITS];
 #pragma unroll
         for (int j = 0; j < BITS; ++j) cw[j] = cw_next[j];
         const float g = __half2float(g_next);
-        fetch(u + gridDim.x * 4, cw_next, g_next);
+        fetch(u + nb * 4, cw_next, g_next);
         uint32_t tail = 0;
         if constexpr (BITS == 3) tail = (cw[0] >> 24) | ((cw[1] >> 24) << 8) | ((cw[2] >> 24) << 16);
         uint4 xb[4];
@@ -1707,19 +1709,25 @@ __global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half 
     }
 }
 
+template <int BITS>
+__global__ __launch_bounds__(256) void k_load_k16(const uint8_t *packed, __half *out, LoadK16Args a) {
+    __shared__ uint32_t lut_s[1 << (2 * BITS)];
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ float s1_s[128];
+    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[LOAD16_XPOSE_BYTES];
+    load_k16_body<BITS>(packed, out, a, blockIdx.x, gridDim.x, lut_s, frag_s, s1_s, xpose_s);
+}
+
 // The same for V rows (dim-major inside a 64-token tile): the tile's codes are staged in LDS and a lane gathers the
 // 32 codes of its token from 32 rows (same pair position in each).  Wavefront w takes tokens 16a + 4w + i of the
 // tile (a, i = 0..3), so that the dword a pair sits in - and for 3-bit codes whether it sits in the split tail -
 // is the same for the whole wavefront.  a.n_units counts 64-token tiles here.
+// (cent_s: 16 fp16 bit patterns, tile_s: (BITS * 64 + 8) * 16 bytes; the others as for K rows)
 template <int BITS>
-__global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half *out, LoadK16Args a) {
-    constexpr int XROW = 256 + 16;
+__device__ __forceinline__ void load_v16_body(const uint8_t *packed, __half *out, const LoadK16Args &a, uint32_t bid, uint32_t nb,
+                                              uint16_t *cent_s, uint4 *frag_s, float *s1_s, uint8_t *xpose_s, uint8_t *tile_s) {
+    constexpr int XROW = LOAD16_XROW;
     constexpr int PIECES = BITS * 64 + 8;  // 16-byte pieces of a tile: codes [BITS][64 rows][16 B], then 64 fp16 norms
-    __shared__ uint16_t cent_s[16];
-    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
-    __shared__ float s1_s[128];
-    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[4 * 16 * XROW];
-    __shared__ __attribute__((aligned(16))) uint8_t tile_s[PIECES * 16];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n16 = lane & 15, kc = lane >> 4;
     if (tid < (1 << BITS)) cent_s[tid] = (uint16_t)(a.pair_lut[tid] & 0xffffu);  // pair (lo = code, hi = 0): low half = c[code]
@@ -1757,9 +1765,9 @@ __global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half 
         pre0 = piece(tid);
         if constexpr (PIECES > 256) pre1 = piece(tid + 256);
     };
-    fetch_tile(blockIdx.x);
+    fetch_tile(bid);
 #pragma unroll 1
-    for (uint32_t tile = blockIdx.x; tile < a.n_units; tile += gridDim.x) {
+    for (uint32_t tile = bid; tile < a.n_units; tile += nb) {
         const uint32_t blk = tile >> 1, half = tile & 1, seq = blk / bps, bis = blk - seq * bps;
         __syncthreads();  // the previous tile's codes are no longer needed
         if (tid < PIECES) reinterpret_cast<uint4 *>(tile_s)[tid] = pre0;
@@ -1767,7 +1775,7 @@ __global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half 
             if (tid + 256 < PIECES) reinterpret_cast<uint4 *>(tile_s)[tid + 256] = pre1;
         }
         __syncthreads();
-        fetch_tile(tile + gridDim.x);  // the next tile's pieces travel while this one is worked on
+        fetch_tile(tile + nb);  // the next tile's pieces travel while this one is worked on
         const float g = __half2float(reinterpret_cast<const __half *>(tile_s + BITS * 1024)[tl]);
         uint32_t hv[32];  // fp16 bits of the lane's 32 values
         if (BITS == 3 && wave == 3) {
@@ -1812,6 +1820,34 @@ __global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half 
                 *reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok) * 128 + 8 * (lane & 15))) = piece;
         }
     }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half *out, LoadK16Args a) {
+    __shared__ uint16_t cent_s[16];
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ float s1_s[128];
+    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[LOAD16_XPOSE_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t tile_s[(BITS * 64 + 8) * 16];
+    load_v16_body<BITS>(packed, out, a, blockIdx.x, gridDim.x, cent_s, frag_s, s1_s, xpose_s, tile_s);
+}
+
+// K and V of a layer in one launch.  The V tiles and the K turns (four 16-token units, one per wavefront) form one
+// sequence of 64-token turns, V first, dealt round-robin to the workgroups: each runs the V-tile loop over its
+// tiles and then the K-row loop from its first K turn on, reloading the tables in between (the handles may differ).
+template <int KB, int VB>
+__global__ __launch_bounds__(256) void k_load_kv16(const uint8_t *packed_k, __half *out_k, LoadK16Args ak, const uint8_t *packed_v,
+                                                   __half *out_v, LoadK16Args av) {
+    constexpr int TILE_V = (VB * 64 + 8) * 16, AUX_K = 4 << (2 * KB), AUX_V = TILE_V + 32;
+    __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
+    __shared__ float s1_s[128];
+    __shared__ __attribute__((aligned(16))) uint8_t xpose_s[LOAD16_XPOSE_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t aux_s[AUX_K > AUX_V ? AUX_K : AUX_V];
+    const uint32_t bid = blockIdx.x, nb = gridDim.x, v_turns = av.n_units;
+    if (bid < v_turns) load_v16_body<VB>(packed_v, out_v, av, bid, nb, reinterpret_cast<uint16_t *>(aux_s + TILE_V), frag_s, s1_s, xpose_s, aux_s);
+    __syncthreads();  // every wavefront is done with the V tables and tiles
+    const uint32_t first = bid >= v_turns ? bid : bid + (v_turns - bid + nb - 1) / nb * nb;  // this workgroup's first turn past V
+    load_k16_body<KB>(packed_k, out_k, ak, first - v_turns, nb, reinterpret_cast<uint32_t *>(aux_s), frag_s, s1_s, xpose_s);
 }
 
 __global__ __launch_bounds__(256) void k_unpack_codes(const uint8_t *packed, uint8_t *idx, float *norms, int bits,
@@ -2511,6 +2547,54 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
 #undef TQ_KV_V
 #undef TQ_KV
     return tq_check_launch("store_kv");
+}
+
+// K and V of a layer to fp16 in the original domain.  One launch when both handles hold the fragments of the
+// inverse transform, else the two tq_load launches.
+int tqk_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, const void *packed_v, int64_t n_seqs,
+                int64_t tokens, void *out_k, void *out_v, hipStream_t s) {
+    const int64_t bps = blocks_for(tokens);
+    if (n_seqs * bps == 0) return TQ_OK;
+    if (!hk->rfrag16k_inv || !hv->rfrag16k_inv) {
+        const int rc = tqk_load(hk, packed_k, n_seqs, tokens, TQ_KIND_K, out_k, TQ_F16, TQ_DOMAIN_ORIGINAL, s);
+        return rc ? rc : tqk_load(hv, packed_v, n_seqs, tokens, TQ_KIND_V, out_v, TQ_F16, TQ_DOMAIN_ORIGINAL, s);
+    }
+    LoadK16Args ak, av;
+    ak.afrag = (const uint4 *)hk->rfrag16k_inv; ak.s1 = hk->s1_32; ak.pair_lut = (const uint32_t *)hk->pair_lut;
+    ak.tokens = tokens; ak.blocks_per_seq = (uint32_t)bps; ak.n_units = (uint32_t)(n_seqs * bps * 8);
+    av.afrag = (const uint4 *)hv->rfrag16k_inv; av.s1 = hv->s1_32; av.pair_lut = (const uint32_t *)hv->pair_lut;
+    av.tokens = tokens; av.blocks_per_seq = (uint32_t)bps; av.n_units = (uint32_t)(n_seqs * bps * 2);
+    unsigned fit = 0;
+#define TQ_LKV(KB, VB)                                                                                             \
+    {                                                                                                              \
+        static const unsigned f = resident_workgroups(k_load_kv16<KB, VB>);                                        \
+        fit = f;                                                                                                   \
+    }
+#define TQ_LKV_V(KB, M)        \
+    switch (hv->bits) {        \
+    case 2: M(KB, 2); break;   \
+    case 3: M(KB, 3); break;   \
+    default: M(KB, 4); break;  \
+    }
+#define TQ_LKV_K(M)                  \
+    switch (hk->bits) {              \
+    case 2: TQ_LKV_V(2, M); break;   \
+    case 3: TQ_LKV_V(3, M); break;   \
+    default: TQ_LKV_V(4, M); break;  \
+    }
+    TQ_LKV_K(TQ_LKV)
+    // a workgroup takes one V tile or four K units per turn: no more workgroups than turns
+    const int64_t turns = ((int64_t)ak.n_units + 3) / 4 + av.n_units;
+    const unsigned grid = (unsigned)std::min<int64_t>(fit, turns);
+#define TQ_LKV_GO(KB, VB)                                                                                                \
+    k_load_kv16<KB, VB><<<grid, 256, 0, s>>>((const uint8_t *)packed_k, (__half *)out_k, ak, (const uint8_t *)packed_v, \
+                                              (__half *)out_v, av)
+    TQ_LKV_K(TQ_LKV_GO)
+#undef TQ_LKV_GO
+#undef TQ_LKV_K
+#undef TQ_LKV_V
+#undef TQ_LKV
+    return tq_check_launch("load_kv16");
 }
 
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,

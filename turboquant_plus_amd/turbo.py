@@ -214,6 +214,24 @@ class TurboCodec:
                                 L.DOMAIN_ORIGINAL if domain == "original" else L.DOMAIN_ROTATED, L.stream_ptr()))
         return out
 
+    def load_kv(self, v_codec: "TurboCodec", packed_k, packed_v, n_seqs: int, tokens: int, out_k=None, out_v=None):
+        """(packed_k, packed_v) -> K and V [n_seqs, tokens, 128] fp16 in the original domain in one launch;
+        the same values as load(packed_k, .., "k", dtype=float16) and v_codec.load(packed_v, .., "v", dtype=float16)."""
+        tt = L.torch()
+        outs = []
+        for o in (out_k, out_v):
+            if o is None:
+                o = tt.empty((n_seqs, tokens, HEAD_DIM), dtype=tt.float16, device=packed_k.device)
+            elif o.dtype != tt.float16 or o.numel() != n_seqs * tokens * HEAD_DIM or not o.is_contiguous():
+                raise ValueError(f"outputs must be contiguous fp16 tensors of {n_seqs * tokens * HEAD_DIM} elements")
+            outs.append(o)
+        nk, nv = packed_bytes(self.bits, n_seqs, tokens), packed_bytes(v_codec.bits, n_seqs, tokens)
+        if packed_k.numel() < nk or packed_v.numel() < nv:
+            raise ValueError(f"packed buffers hold {packed_k.numel()} and {packed_v.numel()} bytes, need {nk} and {nv}")
+        L.check(L.lib().tq_load_kv(self.handle.h, v_codec.handle.h, L.ptr(packed_k), L.ptr(packed_v), n_seqs, tokens,
+                                   L.ptr(outs[0]), L.ptr(outs[1]), L.stream_ptr()))
+        return outs[0], outs[1]
+
     def unpack_codes(self, packed, n_seqs: int, tokens: int, kind: str = "k"):
         """packed -> (indices uint8 [n_seqs, tokens, 128], stored norms fp32 [n_seqs, tokens])."""
         tt = L.torch()
