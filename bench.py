@@ -315,7 +315,7 @@ def cpu_baseline(bits):
     v = rng.standard_normal((n, D)).astype(np.float16)
     s1, s2, _ = O.sign_diagonals(D, np.random.default_rng(42))
     cent = O.centroids_for(bits, D)
-    reps = 8                                          # 8 x (one head of K + one head of V) = all of config 2
+    reps = 32                                         # 8 x (one head of K + one head of V) = all of config 2; four times over
     t0 = time.perf_counter()
     for _ in range(reps):
         for x, kind in ((k, "k"), (v, "v")):
@@ -333,8 +333,8 @@ def cpu_baseline(bits):
     O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
     dta = time.perf_counter() - t0
     return ({"value": algo / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"NumPy oracle turbo{bits} encode+pack of all 2 x 262144 fp16 vectors of config 2 "
-                       f"(8 passes over one head of K and one of V), {dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
+             "sample": f"NumPy oracle turbo{bits} encode+pack of all 2 x 262144 fp16 vectors of config 2, four times over "
+                       f"(32 passes over one head of K and one of V), {dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
              "host_cpus": os.cpu_count()},
             {"value": dta * 128 * 1e6, "unit": "µs/step", "cores": blas_threads or 1, "kind": "port",
              "sample": f"NumPy oracle decompress->softmax->PV for 1 of 128 (batch, kv-head) groups at ctx 32768 "
