@@ -1836,7 +1836,7 @@ __global__ __launch_bounds__(256) void k_load_v16(const uint8_t *packed, __half 
 // sequence of 64-token turns, V first, dealt round-robin to the workgroups: each runs the V-tile loop over its
 // tiles and then the K-row loop from its first K turn on, reloading the tables in between (the handles may differ).
 template <int KB, int VB>
-__global__ __launch_bounds__(256) void k_load_kv16(const uint8_t *packed_k, __half *out_k, LoadK16Args ak, const uint8_t *packed_v,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_load_kv16(const uint8_t *packed_k, __half *out_k, LoadK16Args ak, const uint8_t *packed_v,
                                                    __half *out_v, LoadK16Args av) {
     constexpr int TILE_V = (VB * 64 + 8) * 16, AUX_K = 4 << (2 * KB), AUX_V = TILE_V + 32;
     __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
