@@ -766,7 +766,8 @@ def fork_blocks_unpack(buf: np.ndarray, bits: int):
 def q8_0_quantize(x):
     """Per 32 consecutive values: scale = max|x|/127 stored as fp16,
     q = roundf(x * (1/scale)) (half away from zero, as ggml's quantize_row_q8_0
-    does; scale 0 -> zeros).  All arithmetic in fp32 with the unrounded scale."""
+    does; scale 0 -> zeros).  All arithmetic in fp32 with the unrounded scale.
+    roundf is not floor(|t| + 0.5): for |t| = 0.5 - 2^-25 the sum rounds up to 1.0 in fp32."""
     x = np.asarray(x, dtype=np.float32)
     lead = x.shape[:-1]
     xb = x.reshape(lead + (x.shape[-1] // 32, 32))
@@ -774,7 +775,9 @@ def q8_0_quantize(x):
     scale = (amax / np.float32(127.0)).astype(np.float32)
     inv = np.where(scale > 0, np.float32(1.0) / np.where(scale > 0, scale, 1), 0).astype(np.float32)
     t = (xb * inv[..., None]).astype(np.float32)
-    q = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).clip(-127, 127).astype(np.int8)
+    a = np.abs(t)
+    f = np.floor(a)
+    q = (np.sign(t) * (f + (a - f >= np.float32(0.5)))).clip(-127, 127).astype(np.int8)  # roundf; a - f is exact
     return q.reshape(x.shape), scale.astype(np.float16)
 
 

@@ -381,3 +381,30 @@ def test_score_tile(projection, nk, nq):
     assert abs(err.mean()) < 4 * err.std() / np.sqrt(err.size) + 1e-3       # unbiased
     h = np_(codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=tt.float16)).astype(np.float64)
     assert np.abs(h - ref).max() <= 4e-3 * np.abs(ref).max()
+
+
+FORMATS = ["turbo2", "turbo3", "turbo4", "q8_0"]
+
+
+@pytest.mark.parametrize("vfmt", FORMATS)
+@pytest.mark.parametrize("kfmt", FORMATS)
+def test_decode_attention_every_format_pair(kfmt, vfmt):
+    """Every K format with every V format that a layer-adaptive policy can ask for (policy.layer_formats):
+    dense and Sparse V, a ragged context, two workgroups' worth of splits."""
+    B, Hq, Hkv, N, n_splits = 2, 8, 2, 1100, 4
+    rng = np.random.default_rng(FORMATS.index(kfmt) * 4 + FORMATS.index(vfmt))
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    kc = tqa.TurboCodec(int(kfmt[-1]), seed=42) if kfmt != "q8_0" else None
+    vc = tqa.TurboCodec(int(vfmt[-1]), seed=542) if vfmt != "q8_0" else None
+    kp = kc.store(k, kind="k") if kc else tqa.q8_0_store(k)[0]
+    vp = vc.store(v, kind="v") if vc else tqa.q8_0_store(v, kind="v")[0]
+    for tau in (0.0, 1e-3):
+        attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+        out = np_(attn(q, kp, vp))
+        ref, skip_o, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau,
+                                             k_q8=None if kc else kp, v_q8=None if vc else vp)
+        assert_close(out, ref)
+        if tau:
+            assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4

@@ -243,9 +243,14 @@ def test_config1_polarquant_turbo3_roundtrip(golden):
     idx, g = np_(idx)[0], np_(g)[0]
     n_bad, n_ulp, idx_o, g_o = check_codes(codec, X, idx, g)
     print(f"\nconfig 1: {n_bad} in-band index mismatches of {idx.size}, {n_ulp} norms off by one fp16 ulp")
-    if n_bad == 0:
-        assert np.array_equal(idx[:64], golden["c1_idx_first64"])
-        assert np.array_equal(np.bincount(idx.ravel(), minlength=8), golden["c1_idx_hist"])
+    # the fixture the reference wrote: every position where the GPU agrees with the oracle (all but the n_bad
+    # in-band ones) must carry the reference's index; the histogram may move by the in-band cases only
+    agree = idx[:64] == idx_o[:64]
+    assert (~agree).sum() <= n_bad
+    assert np.array_equal(idx[:64][agree], golden["c1_idx_first64"][agree])
+    assert np.array_equal(idx_o[:64], golden["c1_idx_first64"])
+    hist_gap = np.abs(np.bincount(idx.ravel(), minlength=8) - golden["c1_idx_hist"]).sum()
+    assert hist_gap <= 2 * n_bad
     deq = np_(codec.load(packed, 1, 4096, domain="original"))[0].astype(np.float64)
     ref = O.turbo_decode(idx, g, codec.centroids, codec.signs1, codec.signs2)
     err = np.linalg.norm(deq - ref, axis=1) / np.linalg.norm(ref, axis=1)

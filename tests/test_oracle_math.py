@@ -206,6 +206,35 @@ def test_q8_0_textbook():
     assert err.max() <= np.abs(x).reshape(5, 4, 32).max(-1).max() / 127 * 0.51 + 1e-3
 
 
+def test_q8_0_literal_blocks():
+    """ggml's quantize_row_q8_0 written out on four hand-made 32-value blocks: d = amax/127 kept in fp32 for
+    the division (id = 1/d, x*id), stored as fp16; q = roundf(x*id), i.e. halves go away from zero."""
+    x = np.zeros((1, 128), dtype=np.float32)
+    # block 0: amax 127 -> d = 1, q = roundf(x).  Ties at +-0.5, +-1.5, +-2.5 (banker's rounding would give
+    # 0, 2, 2), values just either side of a half, the extreme on the negative side.
+    b0 = [-127.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 0.49999997, -0.49999997, 0.50000006, 3.0, -0.0, 100.25, -100.75]
+    x[0, :len(b0)] = b0
+    q0 = [-127, 1, -1, 2, -2, 3, -3, 127, -127, 0, 0, 1, 3, 0, 100, -101]
+    # block 1: all zero -> d = 0, id = 0, q = 0
+    # block 2: amax = 127 * (1 + 2^-12): d = 1 + 2^-12 in fp32, which fp16 rounds to 1.0.  100.5 / d = 100.4755
+    # -> 100 (dividing by the fp16-rounded scale would give 100.5 -> 101); 0.5 / d < 0.5 -> 0 (1 with the
+    # rounded scale).
+    d2 = np.float32(1.0) + np.float32(2.0 ** -12)
+    x[0, 64:68] = [np.float32(127.0) * d2, 100.5, 0.5, -100.5]
+    q2 = [127, 100, 0, -100]
+    # block 3: amax 63.5 -> d = 0.5: -63.5 -> -127, 0.25 -> 0.5 -> 1, 0.75 -> 1.5 -> 2, -0.25 -> -1
+    x[0, 96:100] = [-63.5, 0.25, 0.75, -0.25]
+    q3 = [-127, 1, 2, -1]
+    q, s = O.q8_0_quantize(x)
+    assert q[0, :16].tolist() == q0 and not q[0, 16:64].any()
+    assert q[0, 64:68].tolist() == q2 and not q[0, 68:96].any()
+    assert q[0, 96:100].tolist() == q3 and not q[0, 100:].any()
+    assert s.dtype == np.float16 and s[0].tolist() == [1.0, 0.0, 1.0, 0.5]
+    # dequantised value = q * stored (fp16) scale
+    np.testing.assert_array_equal(O.q8_0_dequantize(q, s)[0, 96:100], [-63.5, 0.5, 1.0, -0.5])
+    np.testing.assert_array_equal(O.q8_0_dequantize(q, s)[0, 64:66], [127.0, 100.0])
+
+
 def test_decode_attention_closed_forms():
     rng = np.random.default_rng(6)
     q = rng.standard_normal((4, 128))
@@ -229,6 +258,113 @@ def test_decode_attention_closed_forms():
     assert 0 <= skip <= 1 and np.abs(sp - dense).max() < 1e-3
     sp0, skip0, _ = O.decode_attention(q, k, v, 0.2, n_splits=4, sparse_v_tau=0.0)
     assert skip0 == 0 and np.array_equal(sp0, dense)
+
+
+def _sparse_v_case():
+    """Logits are written directly (zero queries, logits = bias) as multiples of ln 10, so every weight
+    is a power of ten and the Sparse-V bookkeeping can be done by hand.  N = 256 in 2 splits of two
+    64-position tiles each; tau = 1e-2.  Row 0 of the bias:
+
+      split 0, tile 0: pos 0 -> 0 (tile max, weight 1: kept), pos 1 -> -1 (0.1: kept), pos 2 -> -3 (1e-3: skipped)
+      split 0, tile 1: pos 64 -> +3 (new running max), pos 65 -> +2 (0.1: kept), pos 66 -> +0.5 (10^-2.5: skipped,
+                       although its logit is above that of pos 0, which was kept against the earlier maximum;
+                       against the split's final maximum pos 0 and pos 1 would be 1e-3 and 1e-4: skipped)
+      split 1, tile 2: pos 128 -> +1 (max of ITS split: kept), pos 129 -> -0.5 (10^-1.5 against the split's own
+                       maximum: kept; against a maximum carried over from split 0 it would be 10^-3.5)
+      split 1, tile 3: pos 192 -> +1 (equal to the running max: weight 1, kept), pos 193 -> -1.5 (10^-2.5: skipped)
+      every other position -> -30 (skipped)
+
+    Row 1 is all zeros: every weight is 1, nothing is skipped, the output is the mean of V."""
+    N, ln10 = 256, np.log(10.0)
+    e = np.full(N, -30.0)
+    for pos, val in {0: 0, 1: -1, 2: -3, 64: 3, 65: 2, 66: 0.5, 128: 1, 129: -0.5, 192: 1, 193: -1.5}.items():
+        e[pos] = val
+    bias = np.stack([e * ln10, np.zeros(N)])
+    kept = [0, 1, 64, 65, 128, 129, 192]
+    return N, e, bias, kept
+
+
+def test_sparse_v_hand_built_case():
+    N, e, bias, kept = _sparse_v_case()
+    rng = np.random.default_rng(0)
+    k = rng.standard_normal((N, 128))
+    v = np.zeros((N, 128))
+    v[:, 0] = 1.0                       # output[0] = kept weight / total weight
+    v[:, 1] = np.arange(N)              # output[1] = weighted mean position of the kept set
+    v[:, 2] = rng.standard_normal(N)
+    out, skip, below = O.decode_attention(np.zeros((2, 128)), k, v, 0.3, n_splits=2, sparse_v_tau=1e-2,
+                                          logit_bias=bias)
+    w = 10.0 ** e
+    Z = w.sum()
+    assert abs(Z - 1124.6111282027869) < 1e-9             # 1000+100+10+10+sqrt(10)+1+1/sqrt(10)+.1+10^-1.5+.001
+    assert abs(out[0, 0] - 1121.416227766017 / 1124.6111282027869) < 1e-12
+    pos_sum = 1 * 0.1 + 64 * 1000 + 65 * 100 + 128 * 10 + 129 * 10 ** -0.5 + 192 * 10
+    assert abs(out[0, 1] - pos_sum / Z) < 1e-9
+    assert abs(out[0, 2] - (w[kept] * v[kept, 2]).sum() / Z) < 1e-12
+    np.testing.assert_allclose(out[1], v.mean(0), atol=1e-12)
+    assert skip == (N - len(kept)) / (2 * N)               # 249 skipped pairs of 512
+    # final softmax weights >= tau: 1000/Z and 100/Z only; row 1 has 1/256 < 1e-2 everywhere
+    assert below == (254 + 256) / 512
+    # the three plausible mistakes give other numbers
+    final_max_kept = [64, 65]                              # weights against the split's final maximum
+    assert abs(out[0, 0] - w[final_max_kept + [128, 129, 192]].sum() / Z) > 1e-4
+    carried_max_kept = [0, 1, 64, 65]                      # one running maximum over both splits
+    assert abs(out[0, 0] - w[carried_max_kept].sum() / Z) > 1e-3
+
+
+def test_sparse_v_threshold_is_strict():
+    """weight < tau skips, weight == tau keeps (docs/papers/sparse-v-dequant.md:69-75 `if (attn_weight < 1e-6f)
+    continue`): with tau = 1 exactly the positions that hold the running maximum (weight exp(0) = 1) survive."""
+    N = 128
+    bias = np.zeros((1, N))
+    bias[0, [5, 70]] = [2.0, 2.0]       # tile 0: pos 5 is the max; tile 1: pos 70 ties the running max
+    bias[0, 100] = 1.0
+    v = np.zeros((N, 128)); v[:, 0] = np.arange(N)
+    out, skip, _ = O.decode_attention(np.zeros((1, 128)), np.zeros((N, 128)), v, 1.0, n_splits=1, sparse_v_tau=1.0,
+                                      logit_bias=bias)
+    Z = 2 * np.exp(2.0) + np.exp(1.0) + (N - 3)
+    assert abs(out[0, 0] - (5 + 70) * np.exp(2.0) / Z) < 1e-12
+    assert skip == (N - 2) / N
+
+
+def test_sparse_v_split_bounds():
+    """Splits are runs of ceil(n_tiles / n_splits) tiles: N = 320 (5 tiles) in 2 splits -> tiles {0,1,2} and {3,4}.
+    pos 130 (tile 2) -> +5, pos 190 (tile 2) -> 0, pos 200 (tile 3) -> 0, everything else -30.  Tiles 0 and 1 see
+    only -30: every weight there is 1 against the running maximum and is kept (128 positions of negligible
+    weight).  Tile 2: 130 kept, 190 (1e-5) and the rest skipped.  Tile 3 opens split 1 with a fresh maximum:
+    200 kept (with tiles {0,1} / {2,3,4}, or a carried maximum, it would be 1e-5 and skipped).  Tile 4: all skipped."""
+    N, ln10 = 320, np.log(10.0)
+    e = np.full(N, -30.0)
+    e[130], e[190], e[200] = 5, 0, 0
+    v = np.zeros((N, 128)); v[:, 0] = 1.0
+    out, skip, _ = O.decode_attention(np.zeros((1, 128)), np.zeros((N, 128)), v, 1.0, n_splits=2, sparse_v_tau=1e-3,
+                                      logit_bias=(e * ln10)[None])
+    assert skip == (N - 130) / N
+    assert abs(out[0, 0] - (1e5 + 1) / (1e5 + 2)) < 1e-12
+
+
+def test_gaussian_projection_scale_by_slope():
+    """QJL with a raw Gaussian matrix: E[S^T sign(S r)] = d sqrt(2/pi) r/|r|, so the reconstruction
+    scale * |r| * S^T sign(S r) has regression slope 1 on r only for scale = sqrt(pi/2)/d.  The slope
+    sum(<q,r_hat><q,r>) / sum(<q,r>^2) over many keys and queries is 1 within sampling error; the orthogonal
+    mode's constant sqrt(pi/2)/sqrt(d) would give sqrt(d) = 11.3."""
+    d = 128
+    rng = np.random.default_rng(11)
+    r = rng.standard_normal((4000, d))
+    qv = rng.standard_normal((64, d))
+    for mode in ("gaussian", "orthogonal"):
+        ql = O.QJLRef(d, seed=2, projection=mode)
+        z, n = ql.quantize(r)
+        r_hat = ql.dequantize(z, n)
+        a, b = qv @ r_hat.T, qv @ r.T
+        slope = (a * b).sum() / (b * b).sum()
+        assert abs(slope - 1.0) < 0.03, (mode, slope)
+    # and the score tile's correction term carries that same constant
+    ql = O.QJLRef(d, seed=2, projection="gaussian")
+    assert ql.scale == np.sqrt(np.pi / 2) / d
+    z, n = ql.quantize(r[:50])
+    tile = O.score_tile(qv, np.zeros((50, d), dtype=np.int64), np.zeros(50), np.zeros(8), lambda a: a, ql.S, z, n, ql.scale)
+    np.testing.assert_allclose(tile, qv @ ql.dequantize(z, n).T, atol=1e-10)
 
 
 def test_score_tile_is_dequantised_inner_product():

@@ -372,8 +372,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
         const int d0 = 2 * lane, d1 = 2 * lane + 1;
         const int p0 = KFMT == KFMT_Q8 ? (d0 & ~3) | ((d0 & 1) << 1) | ((d0 >> 1) & 1) : d0;
         const int p1 = KFMT == KFMT_Q8 ? (d1 & ~3) | ((d1 & 1) << 1) | ((d1 >> 1) & 1) : d1;
-        qw[p0] = (_Float16)(x0 * a.scale_log2e);
-        qw[p1] = (_Float16)(x1 * a.scale_log2e);
+        // turbo K: the rotated query is rounded to fp16 once, with the logit scale folded in.  q8_0-style K: an
+        // fp16 query goes in as it is, so that its products with the int8 values are exact, and the logit scale
+        // joins the rows' block scales in fp32 (rounding the scaled query would move logits of rows with large
+        // channels by several 1e-3, which a peaked softmax over a long context turns into output error)
+        const float qscale = KFMT == KFMT_Q8 ? 1.0f : a.scale_log2e;
+        qw[p0] = (_Float16)(x0 * qscale);
+        qw[p1] = (_Float16)(x1 * qscale);
     }
     __syncthreads();
     half4_t qa[2];
@@ -457,10 +462,10 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
             for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
             qk_q8(std::make_integer_sequence<int, 32>{}, kw, qa, acc);
             const uint2 su = kn;
-            const float d0 = __half2float(__ushort_as_half((unsigned short)(su.x & 0xffff)));
-            const float d1 = __half2float(__ushort_as_half((unsigned short)(su.x >> 16)));
-            const float d2 = __half2float(__ushort_as_half((unsigned short)(su.y & 0xffff)));
-            const float d3 = __half2float(__ushort_as_half((unsigned short)(su.y >> 16)));
+            const float d0 = __half2float(__ushort_as_half((unsigned short)(su.x & 0xffff))) * a.scale_log2e;
+            const float d1 = __half2float(__ushort_as_half((unsigned short)(su.x >> 16))) * a.scale_log2e;
+            const float d2 = __half2float(__ushort_as_half((unsigned short)(su.y & 0xffff))) * a.scale_log2e;
+            const float d3 = __half2float(__ushort_as_half((unsigned short)(su.y >> 16))) * a.scale_log2e;
 #pragma unroll
             for (int i = 0; i < 4; ++i) sc[i] = (acc[0][i] * d0 + acc[1][i] * d1) + (acc[2][i] * d2 + acc[3][i] * d3);
         }
@@ -886,6 +891,11 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     else if (turbo_k && kb == 2 && vb == 2) { TQ_ATTN_SAME(2); }
     else if (turbo_k && kb == 4 && vb == 2) { TQ_ATTN(KFMT_TURBO, 4, 2); }
     else if (turbo_k && kb == 3 && vb == 2) { TQ_ATTN(KFMT_TURBO, 3, 2); }
+    else if (turbo_k && kb == 3 && vb == 4) { TQ_ATTN(KFMT_TURBO, 3, 4); }
+    else if (turbo_k && kb == 4 && vb == 3) { TQ_ATTN(KFMT_TURBO, 4, 3); }
+    else if (turbo_k && kb == 2 && vb == 3) { TQ_ATTN(KFMT_TURBO, 2, 3); }
+    else if (turbo_k && kb == 2 && vb == 4) { TQ_ATTN(KFMT_TURBO, 2, 4); }
+    else if (turbo_k && kb == 2 && vb == 8) { TQ_ATTN(KFMT_TURBO, 2, 8); }
     else if (!turbo_k && vb == 2) { TQ_ATTN(KFMT_Q8, 3, 2); }
     else if (!turbo_k && vb == 3) { TQ_ATTN(KFMT_Q8, 3, 3); }
     else if (!turbo_k && vb == 4) { TQ_ATTN(KFMT_Q8, 3, 4); }

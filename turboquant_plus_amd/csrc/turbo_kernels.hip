@@ -1892,7 +1892,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store(const TI *x, uint8_t *packed
 #pragma unroll
         for (int j = 0; j < 32; ++j) {
             const float tq = v[j] * id;
-            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            const int qv = (int)roundf(tq);
             w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
         }
         // 32 values = two 16-byte chunks (2*gq, 2*gq+1) of row t
@@ -1941,7 +1941,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store_f16(const __half *x, uint8_t
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const float t = f[j] * id;
-            const int qv = (int)copysignf(floorf(fabsf(t) + 0.5f), t);
+            const int qv = (int)roundf(t);
             w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
         }
         *reinterpret_cast<uint2 *>(img + (c8 >> 1) * Q8_LDS_CHUNK + row * 16 + (c8 & 1) * 8) = make_uint2(w[0], w[1]);
@@ -1987,7 +1987,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v(const TI *x, uint8_t *pack
 #pragma unroll
         for (int j = 0; j < 32; ++j) {
             const float tq = v[j] * id;
-            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            const int qv = (int)roundf(tq);
             img[q8v_byte(t, gq * 32 + j)] = (uint8_t)(qv & 0xFF);
         }
         reinterpret_cast<__half *>(img + 8 * 2048)[q8v_scale(t, gq)] = __float2half_rn(d);
@@ -2050,7 +2050,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v_f16(const __half *x, uint8
             const int t = 16 * c16 + e;
             const float v = __half2float(*reinterpret_cast<const __half *>(raw + t * Q8V_ROW + 2 * dim));
             const float tq = v * inv[t * 4 + gq];
-            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            const int qv = (int)roundf(tq);
             w[e >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (e & 3));
         }
         *reinterpret_cast<uint4 *>(block + (4 * hf + (c16 & 3)) * 2048 + (64 * (c16 >> 2) + l) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
@@ -2088,7 +2088,7 @@ __global__ __launch_bounds__(256) void k_q8_0_append(const TI *x, uint8_t *packe
 #pragma unroll
         for (int j = 0; j < 32; ++j) {
             const float tq = v[j] * id;
-            const int qv = (int)copysignf(floorf(fabsf(tq) + 0.5f), tq);
+            const int qv = (int)roundf(tq);
             if constexpr (KIND == TQ_KIND_V) block[q8v_byte(t, gq * 32 + j)] = (uint8_t)(qv & 0xFF);
             else w[j >> 2] |= ((uint32_t)(qv & 0xFF)) << (8 * (j & 3));
         }
