@@ -257,6 +257,20 @@ int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_
                         float *out, unsigned long long *skip_count, void *workspace, int64_t workspace_bytes,
                         void *stream);
 
+/* tq_decode_attention for callers that cannot allocate device memory or pass a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and results as tq_decode_attention; the split partials go to a workspace of
+ * TQ_STATIC_WORKSPACE_BYTES that is built into the library's device code (every GPU the library runs on
+ * holds one copy until the process ends), so the call allocates nothing.  Parameter sets whose
+ * tq_attn_workspace_bytes() exceeds that size (about batch * n_kv_heads * n_splits > 7900) are rejected with
+ * TQ_ERR_UNSUPPORTED.  All calls on one GPU share the one workspace: calls that overlap in time on the same
+ * GPU (different streams or threads) race; order them.  The workspace's address is looked up once per
+ * device, in tq_create or in the first call on that device. */
+#define TQ_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)
+int tq_decode_attention_static(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q,
+                               int q_dtype, const void *k, const void *v, const float *bias, float *out,
+                               unsigned long long *skip_count, void *stream);
+
 /* TurboQuant inner-product estimate for nq queries x nk keys (turboquant.py:102-124
  * moved to the rotated/projected domain): logits[i,j] = <R q_i, g_j c[idx_j]> +
  * projection_scale * rnorm_j * <S q_i, z_j>.  q [nq,128] q_dtype, packed/sign_bits/

@@ -33,6 +33,7 @@
 //   k_decode_attn, so a dense step is two launches.
 // k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+#include <mutex>
 #include <cstring>
 #include <type_traits>
 #include <utility>
@@ -929,6 +930,59 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     if (rc) return rc;
     }
     return TQ_OK;
+}
+
+// ---- decode attention for callers that cannot allocate -----------------------------------
+// The split partials live in a file-scope device array instead of a caller's workspace.  Every
+// GPU the library runs on holds its own copy of the array, at its own address, until the process
+// ends; the address is looked up once per device (with that device current) and kept.  In host
+// code the array's name is only a handle for that lookup, never a device address.
+namespace {
+constexpr int64_t STATIC_WS_BYTES = TQ_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_WS_BYTES];
+constexpr int MAX_DEVICES = 64;
+void *g_scratch_ptr[MAX_DEVICES];  // per device: device address of that GPU's copy of `scratch`
+std::mutex g_scratch_mutex;
+}  // namespace
+
+// Device address of the current device's scratch array (looked up on the first call per device).
+int tqk_static_scratch(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        tq_set_error("static workspace: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+        return TQ_ERR_HIP;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            tq_set_error("static workspace: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return TQ_ERR_HIP;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return TQ_OK;
+}
+
+int tqk_decode_attention_static(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q,
+                                int q_dtype, const void *k, const void *v, const float *bias, float *out,
+                                unsigned long long *skip_count, hipStream_t s) {
+    const int64_t need = ws_layout(p).total;
+    if (need > STATIC_WS_BYTES) {
+        tq_set_error("tq_decode_attention_static: batch * n_kv_heads * n_splits = %lld needs %lld bytes of split "
+                     "partials, the built-in workspace holds %lld; lower n_splits or use tq_decode_attention",
+                     (long long)p->batch * p->n_kv_heads * p->n_splits, (long long)need, (long long)STATIC_WS_BYTES);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    void *ptr = nullptr;
+    const int rc = tqk_static_scratch(&ptr);
+    if (rc) return rc;
+    // every partial and every skip slot that the merge kernel reads is written by this call's main kernel first,
+    // so nothing of the previous call's contents needs clearing
+    return tqk_decode_attention(hk, hv, p, q, q_dtype, k, nullptr, v, bias, out, skip_count, ptr, STATIC_WS_BYTES, s);
 }
 
 // ---- prefill-shaped TurboQuant inner-product estimator --------------------------------

@@ -118,6 +118,14 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
     h->proj_scale = cfg->projection_scale;
     h->has_proj = cfg->projection != nullptr;
     (void)hipGetDevice(&h->device);
+    {   // look up this device's built-in attention workspace now, where set-up work is expected
+        void *ws = nullptr;
+        const int rcw = tqk_static_scratch(&ws);
+        if (rcw) {
+            delete h;
+            return rcw;
+        }
+    }
 
     const int d = h->d, pd = h->pd, nc = h->n_centroids;
     int rc = TQ_OK;
@@ -622,6 +630,24 @@ int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_
             "tq_decode_attention: k, v and workspace must be 16-byte aligned");
     return tqk_decode_attention(hk, hv, p, q, q_dtype, k, k_aux, v, bias, out, skip_count, workspace, workspace_bytes,
                                 (hipStream_t)stream);
+}
+
+int tq_decode_attention_static(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q,
+                               int q_dtype, const void *k, const void *v, const float *bias, float *out,
+                               unsigned long long *skip_count, void *stream) {
+    int rc = check_attn(p);
+    if (rc) return rc;
+    if (p->v_format == TQ_KFMT_TURBO) {
+        rc = check_fast(hv, "tq_decode_attention_static (V)");
+        if (rc) return rc;
+    }
+    if (p->k_format == TQ_KFMT_TURBO) {
+        rc = check_fast(hk, "tq_decode_attention_static (K)");
+        if (rc) return rc;
+    }
+    REQUIRE(q && k && v && out, TQ_ERR_ARG, "tq_decode_attention_static: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v), TQ_ERR_ALIGN, "tq_decode_attention_static: k and v must be 16-byte aligned");
+    return tqk_decode_attention_static(hk, hv, p, q, q_dtype, k, v, bias, out, skip_count, (hipStream_t)stream);
 }
 
 int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,

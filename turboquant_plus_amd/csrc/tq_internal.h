@@ -100,6 +100,10 @@ int64_t tqk_attn_workspace_bytes(const tq_attn_params *p);
 int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q, int q_dtype,
                          const void *k, const void *k_aux, const void *v, const float *bias, float *out,
                          unsigned long long *skip_count, void *ws, int64_t ws_bytes, hipStream_t s);
+int tqk_static_scratch(void **out);
+int tqk_decode_attention_static(const tq_handle *hk, const tq_handle *hv, const tq_attn_params *p, const void *q,
+                                int q_dtype, const void *k, const void *v, const float *bias, float *out,
+                                unsigned long long *skip_count, hipStream_t s);
 int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
                    const uint8_t *sign_bits, const void *rnorms, int64_t nk, void *logits, int out_dtype, void *ws,
                    int64_t ws_bytes, hipStream_t s);
