@@ -77,6 +77,7 @@ def time_steps(torch, step, steps, warmup):
 def measured_peaks_leg(torch, tqa, steps, warmup):
     """What this box sustains on plain streaming kernels (1 GiB, two buffer sets) and on back-to-back fp16
     MFMAs, timed like the legs below; set beside the published peaks the fractions are quoted against."""
+    from turboquant_plus_amd import probes
     n = 1 << 30
     bufs = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(4)]
     for b in bufs:
@@ -88,7 +89,7 @@ def measured_peaks_leg(torch, tqa, steps, warmup):
         for chunked in (False, True):   # lanes striding over the whole buffer, or one contiguous slice per workgroup
             def step(i):
                 src, dst = bufs[2 * (i % 2)], bufs[2 * (i % 2) + 1]
-                tqa.probe_stream(mode, None if mode == "write" else src, None if mode == "read" else dst, chunked)
+                probes.probe_stream(mode, None if mode == "write" else src, None if mode == "read" else dst, chunked)
             _, ev_ms = time_steps(torch, step, reps, warm)
             moved = n * (2 if mode == "copy" else 1)
             best = max(best, moved / (ev_ms * 1e-3) / 1e9)
@@ -98,7 +99,7 @@ def measured_peaks_leg(torch, tqa, steps, warmup):
     flops = [0]
 
     def mstep(i):
-        flops[0] = tqa.probe_mfma_f16(2000, sink)
+        flops[0] = probes.probe_mfma_f16(2000, sink)
     _, ev_ms = time_steps(torch, mstep, reps, warm)
     out["mfma_f16_tflops"] = flops[0] / (ev_ms * 1e-3) / 1e12
     out["published"] = {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": 2500.0}

@@ -282,21 +282,6 @@ int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, co
                   const uint8_t *sign_bits, const void *rnorms_f16, int64_t nk, void *logits, int out_dtype,
                   void *workspace, int64_t workspace_bytes, void *stream);
 
-/* ---- measurement probes --------------------------------------------------------
- * No counterpart in the reference: plain streaming and back-to-back MFMA launches whose
- * sustained rates a benchmark can set beside the published peaks.  The caller times them. */
-
-/* One launch that reads `bytes` from src (mode 0; dst may be NULL), writes `bytes` to dst
- * (mode 1; src ignored) or copies src to dst (mode 2).  chunked = 0: the lanes of the whole
- * grid stride over the buffer; 1: every workgroup takes one contiguous slice (reads and
- * writes favour different orders on this part).  bytes: a multiple of 16. */
-int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream);
-
-/* One launch of `iters` rounds of eight independent v_mfma_f32_32x32x16_f16 per wavefront on
- * every SIMD of the chip.  Returns the floating-point operations launched (> 0) or an error
- * code (< 0).  sink: 4 bytes of device memory (never written for valid inputs). */
-int64_t tq_probe_mfma_f16(int64_t iters, float *sink, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -23,12 +23,20 @@ reference itself (tests/golden/), scipy.linalg.hadamard, brute-force argmin,
 closed-form centroids and conditional expectations, orthogonality, literal
 pack bytes and size arithmetic.
 
-Parity unpinned (no reference code exists for them; closed forms and brute
-force only): `q8_0_quantize`/`q8_0_dequantize` (textbook ggml block format),
-`fork_blocks_pack`/`fork_blocks_unpack` (the llama.cpp fork's block layout,
-known from its documents only), `decode_attention` (rotated-domain attention,
-Sparse-V predicate, split boundaries) and `score_tile` in its `gaussian`
-projection mode.
+Functions the reference holds no code for, and what pins them instead
+(tests/test_oracle_math.py):
+  `q8_0_quantize`/`q8_0_dequantize`  ggml's published quantize_row_q8_0 (d = amax/127
+      kept in fp32, id = 1/d, roundf(x*id), d stored as fp16), on literal blocks: ties at
+      +-0.5/1.5/2.5, the largest float below one half, a zero block, a scale that changes
+      when rounded to fp16;
+  `decode_attention`, Sparse-V branch  hand-built cases whose skipped set and output are
+      written down (running maximum vs the split's final one, a maximum not carried
+      across splits, weight == tau kept, split bounds for a ragged tile count);
+  `score_tile`, `gaussian` projection  regression slope of the reconstruction on the true
+      residual (1 only for the scale sqrt(pi/2)/d);
+  `fork_blocks_pack`/`fork_blocks_unpack`  the extraction formulas the reference's documents
+      print, applied element by element.  No block written by the fork itself is available:
+      parity with the fork's bytes stays unpinned.
 """
 from __future__ import annotations
 

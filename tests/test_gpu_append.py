@@ -357,3 +357,18 @@ def test_layer_decode_loop_over_a_growing_cache(fmt):
     ref, _, _ = reference_attention(q, layer.k_codec, layer.v_codec, kp, vp, B, Hq, Hkv, pos, 1 / np.sqrt(D),
                                     k_q8=kp if layer.k_codec is None else None, v_q8=vp if layer.v_codec is None else None)
     assert_close(out, ref)
+
+
+def test_store_into_a_capacity_buffer_is_rejected_for_several_sequences():
+    """tq_store lays sequences out ceil(tokens / 128) blocks apart; a buffer sized for a larger capacity has
+    another stride, so the host wrapper refuses it instead of mislaying every sequence after the first."""
+    tt = L.torch()
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    x = np.random.default_rng(0).standard_normal((2, 128, D)).astype(np.float16)
+    cache = tt.zeros(tqa.packed_bytes(3, 2, 512), dtype=tt.uint8, device="cuda")
+    with pytest.raises(ValueError, match="append"):
+        kc.store(x, kind="k", out=cache)
+    with pytest.raises(ValueError, match="append_kv"):
+        kc.store_kv(vc, x, x, out_k=cache, out_v=cache.clone())
+    one = kc.store(x[:1], kind="k", out=cache)           # a single sequence has no stride: allowed
+    assert one is cache

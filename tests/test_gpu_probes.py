@@ -1,11 +1,12 @@
-"""GPU tests of the measurement probes (tq_probe_stream, tq_probe_mfma_f16) and of the score tile's
-store-less mode.  They have no counterpart in the reference: the checks are that the streaming probe
+"""GPU tests of the benchmark's measurement probes (libtq_probe.so: tq_probe_stream, tq_probe_mfma_f16) and of
+the score tile's store-less mode.  They have no counterpart in the reference: the checks are that the streaming probe
 moves exactly the bytes it is asked to, in both access orders, and that the other two run and report."""
 import numpy as np
 import pytest
 
 import turboquant_plus_amd as tqa
 from turboquant_plus_amd import _lib as L
+from turboquant_plus_amd import probes
 from test_gpu_turbo import np_
 
 pytestmark = pytest.mark.gpu
@@ -17,17 +18,17 @@ def test_stream_probe_moves_the_bytes(chunked, nbytes):
     tt = L.torch()
     src = tt.randint(0, 256, (nbytes + 32,), dtype=tt.uint8, device="cuda")
     dst = tt.full((nbytes + 32,), 7, dtype=tt.uint8, device="cuda")
-    tqa.probe_stream("copy", src[:nbytes], dst[:nbytes], chunked)
+    probes.probe_stream("copy", src[:nbytes], dst[:nbytes], chunked)
     got = np_(dst)
     assert np.array_equal(got[:nbytes], np_(src)[:nbytes])
     assert (got[nbytes:] == 7).all(), "wrote past the end"
-    tqa.probe_stream("write", None, dst[:nbytes], chunked)
+    probes.probe_stream("write", None, dst[:nbytes], chunked)
     got = np_(dst).copy()
     assert (got[nbytes:] == 7).all(), "wrote past the end"
     words = got[:nbytes].view(np.uint32).reshape(-1, 4)
     assert (words[:, 1] == 1).all() and (words[:, 2] == 2).all() and (words[:, 3] == 3).all()
     before = np_(src).copy()
-    tqa.probe_stream("read", src[:nbytes], None, chunked)
+    probes.probe_stream("read", src[:nbytes], None, chunked)
     assert np.array_equal(np_(src), before)
 
 
@@ -35,20 +36,22 @@ def test_stream_probe_rejects_bad_sizes():
     tt = L.torch()
     buf = tt.zeros(64, dtype=tt.uint8, device="cuda")
     with pytest.raises(ValueError):
-        tqa.probe_stream("copy", buf[:24], buf[32:56])
+        probes.probe_stream("copy", buf[:24], buf[32:56])
     with pytest.raises(ValueError):
-        tqa.probe_stream("write", None, None)
+        probes.probe_stream("write", None, None)
 
 
 def test_mfma_probe_reports_its_work():
     tt = L.torch()
     sink = tt.zeros(4, dtype=tt.float32, device="cuda")
-    flops = tqa.probe_mfma_f16(3, sink)
+    flops = probes.probe_mfma_f16(3, sink)
     tt.cuda.synchronize()
     assert flops == 2048 * 4 * 3 * 8 * 2 * 32 * 32 * 16
     assert float(sink.abs().sum()) == 0.0
     with pytest.raises(ValueError):
-        tqa.probe_mfma_f16(0, sink)
+        probes.probe_mfma_f16(0, sink)
+    with pytest.raises(ValueError):
+        probes.probe_mfma_f16(probes.MAX_ITERS + 1, sink)      # a single launch is bounded
 
 
 def test_score_tile_without_stores_runs():

@@ -162,3 +162,20 @@ def test_kv_shape_asserts():
         kv.compress(np.zeros((1, 1, 4, 32)), np.zeros((1, 1, 4, 32)))
     with pytest.raises(AssertionError):
         kv.compress(np.zeros((1, 1, 4, 64)), np.zeros((1, 1, 5, 64)))
+
+
+def test_requantize_rejects_another_rotation():
+    """Codes written under one rotation mean nothing under another: the check is made on the host tables,
+    before any device work."""
+    a, b = tqa.TurboCodec(3, seed=1), tqa.TurboCodec(2, seed=501)
+    with pytest.raises(ValueError, match="same rotation"):
+        a.requantize_to(b, None, 1, 128)
+
+
+def test_probe_library_is_separate_from_the_codec_abi():
+    """The benchmark's probes live in their own library and header; the codec's header and library do not
+    carry them."""
+    from turboquant_plus_amd import probes
+    assert not any(n.startswith("tq_probe") for n in header_symbols())
+    assert not hasattr(L.lib(), "tq_probe_stream")
+    assert hasattr(probes.lib(), "tq_probe_stream") and hasattr(probes.lib(), "tq_probe_mfma_f16")

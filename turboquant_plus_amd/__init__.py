@@ -11,11 +11,10 @@ from .turboquant import TurboQuant, TurboQuantMSE, CompressedVector
 from .kv_cache import KVCacheCompressor, CompressedKVCache
 from .outlier import OutlierTurboQuant, OutlierCompressedVector
 from .policy import LayerFormat, LayerKV, layer_formats, effective_bits
-from .turbo import (TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, q8_0_append, packed_bytes, PRODUCTION_CENTROIDS,
-                    probe_stream, probe_mfma_f16)
+from .turbo import (TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, q8_0_append, packed_bytes, PRODUCTION_CENTROIDS)
 
 __all__ = ["PolarQuant", "QJL", "TurboQuant", "TurboQuantMSE", "CompressedVector", "KVCacheCompressor",
            "OutlierTurboQuant", "OutlierCompressedVector",
            "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "q8_0_append", "packed_bytes",
-           "PRODUCTION_CENTROIDS", "probe_stream", "probe_mfma_f16", "LayerFormat", "LayerKV", "layer_formats",
+           "PRODUCTION_CENTROIDS", "LayerFormat", "LayerKV", "layer_formats",
            "effective_bits"]

@@ -76,8 +76,6 @@ PROTOTYPES = {
     "tq_decode_attention": (_I, [_P, _P, C.POINTER(TQAttnParams), _P, _I, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
     "tq_decode_attention_static": (_I, [_P, _P, C.POINTER(TQAttnParams), _P, _I, _P, _P, _P, _P, _P, _P]),
     "tq_score_tile": (_I, [_P, _P, _I, _L, _P, _P, _P, _L, _P, _I, _P, _L, _P]),
-    "tq_probe_stream": (_I, [_I, _I, _P, _P, _L, _P]),
-    "tq_probe_mfma_f16": (_L, [_L, _P, _P]),
 }
 
 _lib = None

@@ -31,7 +31,7 @@
 // k_attn_combine / k_attn_combine_few: log-sum-exp merge of the workgroups' partials,
 //   then the transpose of the V rotation.  Queries are rotated and scaled inside
 //   k_decode_attn, so a dense step is two launches.
-// k_score_tile: TurboQuant inner-product estimate, 16x16x32 fp16 MFMA over a
+// k_score_tile: TurboQuant inner-product estimate, 32x32x16 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
 #include <mutex>
 #include <cstring>

@@ -1,8 +1,10 @@
 // Measurement probes: what this part sustains on plain streaming and on back-to-back MFMAs, so that
 // roofline fractions can be stated against measured figures as well as against the published peaks.
 // Not part of the codec; the callers time the launches themselves.
-#include "tq_device.h"
-#include "tq_internal.h"
+// Built into its own library (libtq_probe.so, header tq_probe.h): the codec's C ABI does not carry it.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "tq_probe.h"
 
 namespace {
 
@@ -67,14 +69,8 @@ constexpr int PROBE_MFMA_WGS = 2048;  // 8 workgroups of 4 wavefronts per CU
 
 extern "C" int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream) {
     hipStream_t s = (hipStream_t)stream;
-    if (mode < 0 || mode > 2 || bytes < 16 || (bytes & 15) || (mode != 1 && !src) || (mode != 0 && !dst)) {
-        tq_set_error("tq_probe_stream: mode %d, %lld bytes (a multiple of 16), src %p, dst %p", mode, (long long)bytes, src, dst);
-        return TQ_ERR_ARG;
-    }
-    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) {
-        tq_set_error("tq_probe_stream: src and dst must be 16-byte aligned");
-        return TQ_ERR_ALIGN;
-    }
+    if (mode < 0 || mode > 2 || bytes < 16 || (bytes & 15) || (mode != 1 && !src) || (mode != 0 && !dst)) return TQ_PROBE_ERR_ARG;
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) return TQ_PROBE_ERR_ARG;
     const int64_t n16 = bytes / 16;
     const unsigned grid = 256 * 4;
     const uint4 *s4 = (const uint4 *)src;
@@ -88,16 +84,13 @@ extern "C" int tq_probe_stream(int mode, int chunked, const void *src, void *dst
         else if (mode == 1) k_probe_stream<1, false><<<grid, 512, 0, s>>>(nullptr, d4, n16);
         else k_probe_stream<2, false><<<grid, 512, 0, s>>>(s4, d4, n16);
     }
-    return tq_check_launch("probe_stream");
+    return hipGetLastError() == hipSuccess ? 0 : TQ_PROBE_ERR_HIP;
 }
 
 extern "C" int64_t tq_probe_mfma_f16(int64_t iters, float *sink, void *stream) {
-    if (iters < 1 || !sink) {
-        tq_set_error("tq_probe_mfma_f16: iters %lld, sink %p", (long long)iters, (void *)sink);
-        return (int64_t)TQ_ERR_ARG;
-    }
+    // one launch keeps every CU busy for about iters * 0.13 us: the cap bounds a single launch at about 0.13 s
+    if (iters < 1 || iters > TQ_PROBE_MAX_ITERS || !sink) return (int64_t)TQ_PROBE_ERR_ARG;
     k_probe_mfma<<<PROBE_MFMA_WGS, 256, 0, (hipStream_t)stream>>>(iters, sink);
-    const int rc = tq_check_launch("probe_mfma");
-    if (rc) return (int64_t)rc;
+    if (hipGetLastError() != hipSuccess) return (int64_t)TQ_PROBE_ERR_HIP;
     return (int64_t)PROBE_MFMA_WGS * 4 * iters * 8 * (2ll * 32 * 32 * 16);
 }

@@ -2149,15 +2149,10 @@ int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_
 }
 
 // fp16 input with a sign-symmetric codebook: rotation on the matrix cores, codes packed in
-// registers.  The butterfly kernel serves every other case and can be forced with
-// TQ_STORE_PATH=butterfly.
+// registers.  The butterfly kernel serves every other case (fp32 / fp64 input, asymmetric codebooks).
 static bool store_fast_ok(const tq_handle *h, int in_dtype, int64_t n_blocks) {
-    static const bool force_butterfly = [] {
-        const char *e = getenv("TQ_STORE_PATH");
-        return e && strcmp(e, "butterfly") == 0;
-    }();
     return in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && (h->bits != 4 || h->quant_lut_ok) &&
-           n_blocks < (1ll << 28) && !force_butterfly;
+           n_blocks < (1ll << 28);
 }
 
 static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {

@@ -110,6 +110,11 @@ class TurboCodec:
             out = tt.empty(nbytes, dtype=tt.uint8, device=xd.device)
         elif out.numel() < nbytes:
             raise ValueError(f"out holds {out.numel()} bytes, need {nbytes}")
+        elif n_seqs > 1 and out.numel() != nbytes:
+            # sequences are laid out ceil(tokens / 128) blocks apart: a buffer sized for a larger capacity has
+            # another stride, and every sequence after the first would land in the wrong place
+            raise ValueError(f"out holds {out.numel()} bytes but {n_seqs} sequences of {tokens} tokens take exactly "
+                             f"{nbytes}; fill a cache laid out for a larger capacity with append()")
         L.check(L.lib().tq_store(self.handle.h, L.ptr(xd), n_seqs, tokens, L.dtype_code(xd),
                                  L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
@@ -127,6 +132,10 @@ class TurboCodec:
         pv = tt.empty(nv, dtype=tt.uint8, device=kd.device) if out_v is None else out_v
         if pk.numel() < nk or pv.numel() < nv:
             raise ValueError(f"output buffers hold {pk.numel()} and {pv.numel()} bytes, need {nk} and {nv}")
+        if n_seqs > 1 and (pk.numel() != nk or pv.numel() != nv):
+            raise ValueError(f"output buffers hold {pk.numel()} and {pv.numel()} bytes but {n_seqs} sequences of "
+                             f"{tokens} tokens take exactly {nk} and {nv}; fill a cache laid out for a larger "
+                             "capacity with append_kv()")
         L.check(L.lib().tq_store_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, tokens,
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
@@ -161,6 +170,9 @@ class TurboCodec:
         """Temporal decay: re-quantise a buffer written with this codec to the narrower
         `dst_codec` (same rotation) -> new packed buffer (tq_requantize)."""
         tt = L.torch()
+        if not (np.array_equal(self.signs1, dst_codec.signs1) and np.array_equal(self.signs2, dst_codec.signs2)):
+            raise ValueError("requantize_to: both codecs must use the same rotation (same sign diagonals); "
+                             "codes written under one rotation mean nothing under another")
         out = tt.empty(packed_bytes(dst_codec.bits, n_seqs, tokens), dtype=tt.uint8, device=packed.device)
         L.check(L.lib().tq_requantize(self.handle.h, dst_codec.handle.h, L.ptr(packed), n_seqs, tokens,
                                       L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
@@ -310,26 +322,6 @@ def q8_0_unpack(packed, n_seqs: int, tokens: int, kind: str = "k"):
     fn = L.lib().tq_q8_0_unpack if _kind_name(kind) == "k" else L.lib().tq_q8_0_unpack_v
     L.check(fn(L.ptr(packed), n_seqs, tokens, L.ptr(q), L.ptr(s), L.stream_ptr()))
     return q, s
-
-
-def probe_stream(mode: str, src, dst, chunked: bool = False):
-    """One launch of the streaming probe: "read" src, "write" dst or "copy" src to dst (uint8 device
-    tensors of equal size, a multiple of 16 bytes); chunked gives every workgroup one contiguous slice
-    instead of striding all lanes over the buffer.  The caller times it."""
-    code = {"read": 0, "write": 1, "copy": 2}[mode]
-    ref = dst if src is None else src
-    nbytes = 0 if ref is None else ref.numel()
-    L.check(L.lib().tq_probe_stream(code, int(chunked), None if src is None else L.ptr(src),
-                                    None if dst is None else L.ptr(dst), nbytes, L.stream_ptr()))
-
-
-def probe_mfma_f16(iters: int, sink) -> int:
-    """One launch of the MFMA probe (fp16 32x32x16, eight independent accumulators per wavefront on
-    every SIMD); returns the floating-point operations launched.  sink: a float32 device tensor."""
-    flops = int(L.lib().tq_probe_mfma_f16(iters, L.ptr(sink), L.stream_ptr()))
-    if flops < 0:
-        L.check(flops)
-    return flops
 
 
 class DecodeAttention:
