@@ -41,7 +41,7 @@ typedef struct tq_handle tq_handle;
 
 /* All pointers in tq_config are HOST pointers, copied at tq_create. */
 typedef struct tq_config {
-    int32_t d;                /* vector dimension (1..1024; fused kernels need 128)   */
+    int32_t d;                /* vector dimension (1..4096; fused kernels need 128)   */
     int32_t bits;             /* codebook bits, 1..8                                  */
     int32_t rotation;         /* TQ_ROT_DENSE | TQ_ROT_WHT                            */
     int32_t norm_correction;  /* polar_quant.py:109-112                               */
@@ -60,10 +60,10 @@ int tq_device_count(void);                 /* 0 when no GPU is visible          
 int tq_create(tq_handle **out, const tq_config *cfg);
 void tq_destroy(tq_handle *h);
 
-/* ---- reference-API kernels: float64 arithmetic, any d <= 1024 ---------------- */
+/* ---- reference-API kernels: float64 arithmetic, any d <= 4096 ---------------- */
 
 /* rotation.py:99-121 fast_walsh_hadamard_transform on each of n rows of length
- * len (power of two <= 1024); normalised by 1/sqrt(len). */
+ * len (power of two <= 4096); normalised by 1/sqrt(len). */
 int tq_fwht(const void *x, void *y, int64_t n, int32_t len, int in_dtype, int out_dtype, void *stream);
 
 /* The handle's rotation applied to n rows of length d: dense Pi x (polar_quant.py:78)
@@ -202,7 +202,8 @@ int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t toke
  * scale = max|x|/127 as fp16, q = roundf(x/scale); the reference tree has no
  * code for it).  x [n_seqs, tokens, 128] -> 128-token blocks of
  * [8 chunks][128 rows][16 B] int8 followed by [128][4] fp16 scales
- * (136 bytes per token); tq_q8_0_bytes gives the buffer size. */
+ * (136 bytes per token); tq_q8_0_bytes gives the buffer size.  x and packed must be
+ * 16-byte aligned (also for tq_q8_0_store_v). */
 int64_t tq_q8_0_bytes(int64_t n_seqs, int64_t tokens);
 int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream);
 /* q [n_seqs, tokens, 128] int8 and scales [n_seqs, tokens, 4] fp32 of such a buffer. */

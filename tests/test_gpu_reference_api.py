@@ -312,3 +312,109 @@ def test_pack_helpers(golden):
     for b in (1, 2, 3, 4):
         assert np.array_equal(utils.pack_indices(golden[f"pack_idx_in_b{b}"], b), golden[f"pack_idx_out_b{b}"])
     assert utils.pack_indices(np.array([3, 0, 1, 2]), 2).tolist() == [0b11000110]
+
+
+# ---- wide vectors (PLAN.md:104-108,146: d = 1536 and 3072) -----------------------------------------
+
+@pytest.mark.parametrize("d", [1536, 3072])
+def test_wide_dims_match_the_oracle(d):
+    """PolarQuant, QJL and TurboQuant at the embedding widths the reference plans to test (1536, 3072): indices
+    and sign bits against the oracle built from the same seeds, float64 outputs to 1e-10 (d-term sums in another
+    order than BLAS), with the dense Haar rotation and in WHT mode (1536 and 3072 are padded to 2048 and 4096)."""
+    rng = np.random.default_rng(d)
+    x = rng.standard_normal((5, d))
+    x[3] = 0.0
+    for rot in ("dense", "wht"):
+        g, o = tqa.PolarQuant(d, 3, seed=11, rotation=rot), O.PolarRef(d, 3, seed=11, rotation=rot)
+        if rot == "dense":
+            assert np.array_equal(g.rotation, o.rotation)
+        ig, ng = g.quantize(x)
+        io, no = o.quantize(x)
+        y, _ = o.rotated(x)
+        n_bad, n_inadm = O.boundary_band_mismatches(y, ig, o.centroids, rel=1e-11)
+        assert n_inadm == 0 and n_bad <= 2, (rot, n_bad, n_inadm)
+        np.testing.assert_allclose(ng, no, rtol=1e-13)
+        np.testing.assert_allclose(g.dequantize(io, no), o.dequantize(io, no), rtol=1e-9, atol=1e-12)
+        assert np.all(g.dequantize(ig, ng)[3] == 0)
+    qg, qo = tqa.QJL(d, seed=5), O.QJLRef(d, seed=5)
+    r = rng.standard_normal((4, d))
+    sg, ng = qg.quantize(r)
+    so, no = qo.quantize(r)
+    proj = qo.project(r)
+    differ = sg != so
+    assert np.all(np.abs(proj[differ]) <= 1e-11 * np.linalg.norm(r, axis=1).max())      # sign flips only at |S r| ~ 0
+    assert differ.sum() <= 2
+    np.testing.assert_allclose(qg.dequantize(so, no), qo.dequantize(so, no), rtol=1e-9, atol=1e-12)
+    if d == 1536:
+        tg, to = tqa.TurboQuant(d, 3, seed=42), O.TurboRef(d, 3, seed=42)
+        xg, xo = tg.dequantize(tg.quantize(x)), to.dequantize(to.quantize(x))
+        np.testing.assert_allclose(xg, xo, rtol=1e-8, atol=1e-10)
+        assert tg.compressed_size_bits(7) == 7 * (d * 3 + 32)
+
+
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_fwht_wide(n):
+    x = np.random.default_rng(n).standard_normal((3, n))
+    got = rotation.fast_walsh_hadamard_transform(x[0])
+    assert np.array_equal(got, O.fwht(x[0]))
+    np.testing.assert_allclose(got, scipy.linalg.hadamard(n) @ x[0] / np.sqrt(n), atol=1e-11)
+
+
+def test_dims_beyond_the_limit_are_refused():
+    with pytest.raises(NotImplementedError, match="1..4096"):
+        tqa.PolarQuant(4097, 2, seed=1, rotation="wht").quantize(np.zeros(4097))
+
+
+# ---- inner-product distortion (tests/test_distortion.py:78-108,138-157) -----------------------------------
+
+@pytest.mark.parametrize("b", [2, 3, 4])
+def test_inner_product_distortion_single_side(b):
+    """Paper Theorem 2: E|<y,x> - <y, Q^-1(Q(x))>|^2 <= sqrt(3 pi^2) |y|^2 / d / 4^b with only x quantised;
+    1000 unit pairs at d = 256, five times the bound allowed for finite d, as the reference's test does."""
+    d = 256
+    rng = np.random.default_rng(456)
+    x, y = rng.standard_normal((1000, d)), rng.standard_normal((1000, d))
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    y /= np.linalg.norm(y, axis=1, keepdims=True)
+    tq = tqa.TurboQuant(d, b, seed=42)
+    x_hat = tq.dequantize(tq.quantize(x))
+    sq = (np.sum(y * x, axis=1) - np.sum(y * x_hat, axis=1)) ** 2
+    bound = np.sqrt(3 * np.pi ** 2) / d / 4 ** b
+    assert sq.mean() < 5.0 * bound, (sq.mean(), bound)
+    # the estimate is unbiased over pairs: the mean error is within four standard errors of zero
+    err = np.sum(y * x_hat, axis=1) - np.sum(y * x, axis=1)
+    assert abs(err.mean()) < 4 * err.std() / np.sqrt(err.size)
+
+
+def test_inner_product_error_decreases_with_bits():
+    d = 256
+    rng = np.random.default_rng(456)
+    x, y = rng.standard_normal((200, d)), rng.standard_normal((200, d))
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    y /= np.linalg.norm(y, axis=1, keepdims=True)
+    errs = {}
+    for b in (2, 3, 4):
+        tq = tqa.TurboQuant(d, b, seed=42)
+        errs[b] = np.abs(np.sum(y * x, axis=1) - np.sum(y * tq.dequantize(tq.quantize(x)), axis=1)).mean()
+    assert errs[2] > errs[3] > errs[4], errs
+
+
+def test_mse_decreases_with_bits_and_both_sides_quantised():
+    """tests/test_distortion.py:163-178 (monotone MSE at d = 256) and :181-207 (both vectors quantised: TurboQuant's
+    inner products stay finite and of the size of PolarQuant's; the reference only prints the two numbers)."""
+    d = 256
+    rng = np.random.default_rng(789)
+    X = rng.standard_normal((200, d))
+    X /= np.linalg.norm(X, axis=1, keepdims=True)
+    mses = {}
+    for b in (1, 2, 3):
+        pq = tqa.PolarQuant(d, b, seed=42)
+        mses[b] = np.mean((pq.dequantize(*pq.quantize(X)) - X) ** 2)
+    assert mses[1] > mses[2] > mses[3]
+    Y = rng.standard_normal((200, d))
+    Y /= np.linalg.norm(Y, axis=1, keepdims=True)
+    pq, tq = tqa.PolarQuant(d, 2, seed=42), tqa.TurboQuant(d, 2, seed=42)
+    ip = np.sum(X * Y, axis=1)
+    e_pq = np.abs(ip - np.sum(pq.dequantize(*pq.quantize(X)) * pq.dequantize(*pq.quantize(Y)), axis=1)).mean()
+    e_tq = np.abs(ip - np.sum(tq.dequantize(tq.quantize(X)) * tq.dequantize(tq.quantize(Y)), axis=1)).mean()
+    assert np.isfinite(e_tq) and e_tq < 10 * e_pq

@@ -66,7 +66,7 @@ def test_argument_errors_map_to_reference_exceptions():
     h = C.c_void_p()
     assert lib.tq_create(C.byref(h), None) == L.ERR_ARG
     cent = np.array([-1.0, 1.0])
-    cfg = L.TQConfig(d=4096, bits=1, rotation=L.ROT_WHT, norm_correction=1, centroids=L.dbl_ptr(cent))
+    cfg = L.TQConfig(d=8192, bits=1, rotation=L.ROT_WHT, norm_correction=1, centroids=L.dbl_ptr(cent))
     assert lib.tq_create(C.byref(h), C.byref(cfg)) == L.ERR_UNSUPPORTED
 
 

@@ -1,8 +1,8 @@
-// Reference-API kernels: float64 arithmetic, any dimension up to 1024.
+// Reference-API kernels: float64 arithmetic, any dimension up to 4096.
 //
 // These back the Python classes that keep the reference's signatures
 // (PolarQuant, QJL, the rotation and codebook free functions, pack helpers).
-// One workgroup of 128 threads handles VB = 8 vectors staged in LDS; the
+// One workgroup of 128 threads handles VB = 8 vectors (4 or 2 for dimensions above 1024 / 2048) staged in LDS; the
 // rotation is either a dense d x d product read from L2 (matrix stored so
 // that consecutive threads read consecutive addresses) or the sign-diagonal
 // Walsh-Hadamard butterfly done in LDS with the reference's stage order, which
@@ -14,34 +14,34 @@ namespace {
 
 using namespace tq64;
 
-template <typename TI, typename TO>
+template <int VB, typename TI, typename TO>
 __global__ __launch_bounds__(NT) void k_rotate64(const TI *x, TO *y, int64_t n, RotArgs r) {
     extern __shared__ double sm[];
     double *xs = sm, *ys = sm + VB * r.pd;
     const int64_t v0 = (int64_t)blockIdx.x * VB;
-    load_block(x, n, v0, r.d, r.pd, xs);
-    rotate_block(r, xs, ys);
+    load_block<VB>(x, n, v0, r.d, r.pd, xs);
+    rotate_block<VB>(r, xs, ys);
     for (int i = threadIdx.x; i < VB * r.d; i += NT) {
         const int v = i / r.d, j = i % r.d;
         if (v0 + v < n) std_(y, (v0 + v) * r.d + j, ys[v * r.pd + j]);
     }
 }
 
-template <typename T>
+template <int VB, typename T>
 __global__ __launch_bounds__(NT) void k_quantize64(const T *x, int64_t n, RotArgs r, const double *bounds, int nb,
                                                   uint8_t *idx, double *norms, double *rotated) {
     extern __shared__ double sm[];
     __shared__ double nrm[VB];
     double *xs = sm, *ys = sm + VB * r.pd;
     const int64_t v0 = (int64_t)blockIdx.x * VB;
-    load_block(x, n, v0, r.d, r.pd, xs);
-    norms_block(xs, r.d, r.pd, nrm);
+    load_block<VB>(x, n, v0, r.d, r.pd, xs);
+    norms_block<VB>(xs, r.d, r.pd, nrm);
     for (int i = threadIdx.x; i < VB * r.pd; i += NT) {
         const double nv = nrm[i / r.pd];
         xs[i] = xs[i] / (nv > 0.0 ? nv : 1.0);
     }
     __syncthreads();
-    rotate_block(r, xs, ys);
+    rotate_block<VB>(r, xs, ys);
     for (int i = threadIdx.x; i < VB * r.d; i += NT) {
         const int v = i / r.d, j = i % r.d;
         if (v0 + v >= n) continue;
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(NT) void k_quantize64(const T *x, int64_t n, RotArg
     if (threadIdx.x < VB && v0 + threadIdx.x < n) norms[v0 + threadIdx.x] = nrm[threadIdx.x];
 }
 
-template <typename T>
+template <int VB, typename T>
 __global__ __launch_bounds__(NT) void k_dequantize64(const uint8_t *idx, const double *norms, int64_t n, RotArgs r,
                                                     const double *centroids, int norm_correction, double *out,
                                                     const T *x, double *residual) {
@@ -68,14 +68,14 @@ __global__ __launch_bounds__(NT) void k_dequantize64(const uint8_t *idx, const d
     }
     __syncthreads();
     if (norm_correction) {
-        norms_block(xs, r.d, r.pd, nrm);
+        norms_block<VB>(xs, r.d, r.pd, nrm);
         for (int i = threadIdx.x; i < VB * r.pd; i += NT) {
             const double nv = nrm[i / r.pd];
             xs[i] = xs[i] / (nv > 1e-10 ? nv : 1.0);
         }
         __syncthreads();
     }
-    rotate_block(r, xs, ys);
+    rotate_block<VB>(r, xs, ys);
     for (int i = threadIdx.x; i < VB * r.d; i += NT) {
         const int v = i / r.d, j = i % r.d;
         if (v0 + v >= n) continue;
@@ -85,15 +85,15 @@ __global__ __launch_bounds__(NT) void k_dequantize64(const uint8_t *idx, const d
     }
 }
 
-template <typename T>
+template <int VB, typename T>
 __global__ __launch_bounds__(NT) void k_qjl_quantize64(const T *x, int64_t n, RotArgs r, int8_t *signs, double *norms) {
     extern __shared__ double sm[];
     __shared__ double nrm[VB];
     double *xs = sm, *ys = sm + VB * r.pd;
     const int64_t v0 = (int64_t)blockIdx.x * VB;
-    load_block(x, n, v0, r.d, r.pd, xs);
-    norms_block(xs, r.d, r.pd, nrm);
-    rotate_block(r, xs, ys);
+    load_block<VB>(x, n, v0, r.d, r.pd, xs);
+    norms_block<VB>(xs, r.d, r.pd, nrm);
+    rotate_block<VB>(r, xs, ys);
     for (int i = threadIdx.x; i < VB * r.d; i += NT) {
         const int v = i / r.d, j = i % r.d;
         if (v0 + v < n) signs[(v0 + v) * r.d + j] = ys[v * r.pd + j] < 0.0 ? (int8_t)-1 : (int8_t)1;
@@ -101,13 +101,14 @@ __global__ __launch_bounds__(NT) void k_qjl_quantize64(const T *x, int64_t n, Ro
     if (threadIdx.x < VB && v0 + threadIdx.x < n) norms[v0 + threadIdx.x] = nrm[threadIdx.x];
 }
 
+template <int VB>
 __global__ __launch_bounds__(NT) void k_qjl_dequantize64(const int8_t *signs, const double *norms, int64_t n, RotArgs r,
                                                         double proj_scale, double shrinkage, double *out) {
     extern __shared__ double sm[];
     double *xs = sm, *ys = sm + VB * r.pd;
     const int64_t v0 = (int64_t)blockIdx.x * VB;
-    load_block(signs, n, v0, r.d, r.pd, xs);
-    rotate_block(r, xs, ys);
+    load_block<VB>(signs, n, v0, r.d, r.pd, xs);
+    rotate_block<VB>(r, xs, ys);
     for (int i = threadIdx.x; i < VB * r.d; i += NT) {
         const int v = i / r.d, j = i % r.d;
         if (v0 + v >= n) continue;
@@ -168,14 +169,23 @@ __global__ void k_pack_indices(const uint8_t *idx, int64_t count, int bits, uint
     packed[i] = (uint8_t)v;
 }
 
-inline size_t lds_bytes(int pd) { return (size_t)2 * VB * pd * sizeof(double); }
+inline size_t lds_bytes(int pd) { return (size_t)2 * vectors_per_workgroup(pd) * pd * sizeof(double); }
 
 // Workgroups that stage more than 48 KB need the limit raised per kernel.
 template <typename K> inline void allow_lds(K kernel, size_t bytes) {
     if (bytes > 48 * 1024)
         (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
-inline unsigned nblocks(int64_t n) { return (unsigned)((n + VB - 1) / VB); }
+inline unsigned nblocks(int64_t n, int pd) {
+    const int vb = vectors_per_workgroup(pd);
+    return (unsigned)((n + vb - 1) / vb);
+}
+// F uses VB as a compile-time constant
+#define DISPATCH_VB(pd, F)                                         \
+    switch (vectors_per_workgroup(pd)) {                           \
+    case 8: { constexpr int VB = 8; F; } break;                    \
+    case 4: { constexpr int VB = 4; F; } break;                    \
+    default: { constexpr int VB = 2; F; } break; }
 
 RotArgs rot_args(const tq_handle *h, int transpose) {
     RotArgs r;
@@ -196,25 +206,22 @@ RotArgs rot_args(const tq_handle *h, int transpose) {
     case TQ_F64: { using TI = double; F; } break; \
     default: tq_set_error("bad dtype %d", dt); return TQ_ERR_ARG; }
 
+template <typename TI, typename TO>
+int launch_rotate_to(const void *x, void *y, int64_t n, const RotArgs &r, hipStream_t s) {
+    const size_t lds = lds_bytes(r.pd);
+    DISPATCH_VB(r.pd, (allow_lds(k_rotate64<VB, TI, TO>, lds),
+                       k_rotate64<VB, TI, TO><<<nblocks(n, r.pd), NT, lds, s>>>((const TI *)x, (TO *)y, n, r)));
+    return tq_check_launch("rotate64");
+}
+
 template <typename TI>
 int launch_rotate(const void *x, void *y, int64_t n, int out_dtype, const RotArgs &r, hipStream_t s) {
-    const size_t lds = lds_bytes(r.pd);
     switch (out_dtype) {
-    case TQ_F16:
-        allow_lds(k_rotate64<TI, __half>, lds);
-        k_rotate64<TI, __half><<<nblocks(n), NT, lds, s>>>((const TI *)x, (__half *)y, n, r);
-        break;
-    case TQ_F32:
-        allow_lds(k_rotate64<TI, float>, lds);
-        k_rotate64<TI, float><<<nblocks(n), NT, lds, s>>>((const TI *)x, (float *)y, n, r);
-        break;
-    case TQ_F64:
-        allow_lds(k_rotate64<TI, double>, lds);
-        k_rotate64<TI, double><<<nblocks(n), NT, lds, s>>>((const TI *)x, (double *)y, n, r);
-        break;
+    case TQ_F16: return launch_rotate_to<TI, __half>(x, y, n, r, s);
+    case TQ_F32: return launch_rotate_to<TI, float>(x, y, n, r, s);
+    case TQ_F64: return launch_rotate_to<TI, double>(x, y, n, r, s);
     default: tq_set_error("bad dtype %d", out_dtype); return TQ_ERR_ARG;
     }
-    return tq_check_launch("rotate64");
 }
 
 }  // namespace
@@ -244,8 +251,9 @@ int tqk_nearest(const double *values, int64_t n, const double *bounds_host, int 
 int tqk_quantize_indices(const tq_handle *h, const void *x, int64_t n, int in_dtype, uint8_t *idx, double *norms,
                          double *rotated, hipStream_t s) {
     const RotArgs r = rot_args(h, 0);
-    DISPATCH_IN(in_dtype, (allow_lds(k_quantize64<TI>, lds_bytes(r.pd)), k_quantize64<TI><<<nblocks(n), NT, lds_bytes(r.pd), s>>>(
-                              (const TI *)x, n, r, h->bounds64, h->n_centroids - 1, idx, norms, rotated)));
+    DISPATCH_IN(in_dtype, DISPATCH_VB(r.pd, (allow_lds(k_quantize64<VB, TI>, lds_bytes(r.pd)),
+                                             k_quantize64<VB, TI><<<nblocks(n, r.pd), NT, lds_bytes(r.pd), s>>>(
+                                                 (const TI *)x, n, r, h->bounds64, h->n_centroids - 1, idx, norms, rotated))));
     return tq_check_launch("quantize64");
 }
 
@@ -253,8 +261,9 @@ int tqk_dequantize_indices(const tq_handle *h, const uint8_t *idx, const double 
                            const void *x, int x_dtype, double *residual, hipStream_t s) {
     const RotArgs r = rot_args(h, 1);
     if (!residual) x_dtype = TQ_F64;
-    DISPATCH_IN(x_dtype, (allow_lds(k_dequantize64<TI>, lds_bytes(r.pd)), k_dequantize64<TI><<<nblocks(n), NT, lds_bytes(r.pd), s>>>(
-                             idx, norms, n, r, h->centroids64, h->norm_correction, out, (const TI *)x, residual)));
+    DISPATCH_IN(x_dtype, DISPATCH_VB(r.pd, (allow_lds(k_dequantize64<VB, TI>, lds_bytes(r.pd)),
+                                            k_dequantize64<VB, TI><<<nblocks(n, r.pd), NT, lds_bytes(r.pd), s>>>(
+                                                idx, norms, n, r, h->centroids64, h->norm_correction, out, (const TI *)x, residual))));
     return tq_check_launch("dequantize64");
 }
 
@@ -265,9 +274,9 @@ int tqk_qjl_quantize(const tq_handle *h, const void *rr, int64_t n, int in_dtype
     r.mode = TQ_ROT_DENSE;
     r.mat = h->proj64_t;  // out[j] = sum_k S[j][k] in[k]
     r.sa = r.sb = nullptr;
-    DISPATCH_IN(in_dtype,
-                (allow_lds(k_qjl_quantize64<TI>, lds_bytes(r.pd)),
-                 k_qjl_quantize64<TI><<<nblocks(n), NT, lds_bytes(r.pd), s>>>((const TI *)rr, n, r, signs, norms)));
+    DISPATCH_IN(in_dtype, DISPATCH_VB(r.pd, (allow_lds(k_qjl_quantize64<VB, TI>, lds_bytes(r.pd)),
+                                             k_qjl_quantize64<VB, TI><<<nblocks(n, r.pd), NT, lds_bytes(r.pd), s>>>(
+                                                 (const TI *)rr, n, r, signs, norms))));
     return tq_check_launch("qjl_quantize64");
 }
 
@@ -278,8 +287,9 @@ int tqk_qjl_dequantize(const tq_handle *h, const int8_t *signs, const double *no
     r.mode = TQ_ROT_DENSE;
     r.mat = h->proj64;  // out[j] = sum_k S[k][j] z[k]
     r.sa = r.sb = nullptr;
-    allow_lds(k_qjl_dequantize64, lds_bytes(r.pd));
-    k_qjl_dequantize64<<<nblocks(n), NT, lds_bytes(r.pd), s>>>(signs, norms, n, r, h->proj_scale, shrinkage, out);
+    DISPATCH_VB(r.pd, (allow_lds(k_qjl_dequantize64<VB>, lds_bytes(r.pd)),
+                       k_qjl_dequantize64<VB><<<nblocks(n, r.pd), NT, lds_bytes(r.pd), s>>>(signs, norms, n, r, h->proj_scale,
+                                                                                          shrinkage, out)));
     return tq_check_launch("qjl_dequantize64");
 }
 

@@ -558,7 +558,7 @@ int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int6
 
 int tq_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream) {
     REQUIRE(x && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_store: bad argument");
-    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_store: packed must be 16-byte aligned");
+    REQUIRE(aligned16(packed) && aligned16(x), TQ_ERR_ALIGN, "tq_q8_0_store: x and packed must be 16-byte aligned");
     return tqk_q8_0_store(x, n_seqs, tokens, in_dtype, packed, (hipStream_t)stream);
 }
 
@@ -569,7 +569,7 @@ int tq_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q
 
 int tq_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, void *stream) {
     REQUIRE(x && packed && n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "tq_q8_0_store_v: bad argument");
-    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_store_v: packed must be 16-byte aligned");
+    REQUIRE(aligned16(packed) && aligned16(x), TQ_ERR_ALIGN, "tq_q8_0_store_v: x and packed must be 16-byte aligned");
     return tqk_q8_0_store_v(x, n_seqs, tokens, in_dtype, packed, (hipStream_t)stream);
 }
 

@@ -2,6 +2,7 @@
 // butterflies, and the packed "pair container" row format.
 #pragma once
 #include "tq_internal.h"
+#include "tq_layout.h"
 
 namespace tqd {
 
@@ -110,35 +111,7 @@ __device__ inline void wht128_wave(float &a, float &b, int lane) {
 #undef TQ_STAGE
 }
 
-// ---- packed rows ----------------------------------------------------------------
-// A row holds 64 pair codes (128 values) in 4*BITS dwords; pair = lo | hi << BITS.
-// The row is four groups of 16 pairs; a group owns BITS dwords and dword j of group g
-// is row dword 4j + g, so 16-byte chunk j of the row holds dword j of the four groups.
-// Inside a group, pair k sits in
-//   BITS 4: byte k%4 of dword k/4
-//   BITS 2: nibble k%8 of dword k/8
-//   BITS 3: bits 6*(k%4).. of dword k/4 for k < 12; pairs 12..15 form a 24-bit tail
-//           (pair k at tail bit 6*(k-12)) whose byte j is the top byte of dword j
-// Pairs 2q, 2q+1 ("quad" q, four values) are contiguous bits in every width, so a
-// reader can index a table by a whole quad with one field extract.
-// A block is 128 rows stored chunk-major [BITS][128][16 B] followed by 128 fp16
-// norms.  K rows: row = token, pair p = dims (2p, 2p+1).  V rows are dim-major
-// inside each 64-token tile: row (token & 64) | (dim & 63) holds dims r and 64+r
-// of the tile's tokens; with tp = (token & 63) / 2 and hf = dim >> 6, tokens 2tp,
-// 2tp+1 are pair 4*(tp/2) + 2*hf + tp%2, so a quad is four consecutive tokens of
-// one dim.
-__host__ __device__ constexpr int row_dwords(int bits) { return 4 * bits; }
-__host__ __device__ constexpr int block_bytes(int bits) { return TQ_ROWS_PER_BLOCK * (16 * bits + 2); }
-__host__ __device__ constexpr int block_code_bytes(int bits) { return TQ_ROWS_PER_BLOCK * 16 * bits; }
-
-// pairs per dword (BITS 3: of the 12 pairs outside the tail)
-__host__ __device__ constexpr int pairs_per_dword(int bits) { return bits == 2 ? 8 : 4; }
-// true for the four pairs of a 3-bit group that live in the split tail
-__host__ __device__ constexpr bool pair_in_tail(int bits, int p) { return bits == 3 && (p & 15) >= 12; }
-// row dword and bit position of pair p (not for tail pairs)
-__host__ __device__ constexpr int pair_dword(int bits, int p) { return 4 * ((p & 15) / pairs_per_dword(bits)) + (p >> 4); }
-__host__ __device__ constexpr int pair_shift(int bits, int p) { return 2 * bits * ((p & 15) % pairs_per_dword(bits)); }
-
+// ---- packed rows: the index arithmetic lives in tq_layout.h (shared with the host checks) -------------
 // 24-bit tail (pairs 12..15) of group g of a 3-bit row
 __device__ __forceinline__ uint32_t tail24(const uint32_t *w, int g) {
     return (w[g] >> 24) | ((w[4 + g] >> 24) << 8) | ((w[8 + g] >> 24) << 16);
@@ -167,19 +140,6 @@ template <int BITS> __device__ __forceinline__ uint32_t quad_lut_offset(const ui
 __device__ inline uint32_t pair_code(const uint32_t *w, int bits, int p) {
     if (pair_in_tail(bits, p)) return (tail24(w, p >> 4) >> (6 * ((p & 15) - 12))) & 63u;
     return (w[pair_dword(bits, p)] >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
-}
-
-// (row, pair, half) of the code of (token, dim) inside its 128-token block
-__device__ inline void locate(int kind, int token, int dim, int &row, int &pair, int &half) {
-    if (kind == TQ_KIND_K) {
-        row = token;
-        pair = dim >> 1;
-        half = dim & 1;
-    } else {
-        row = (token & 64) | (dim & 63);
-        pair = ((token & 60) | ((dim >> 6) << 1)) | ((token >> 1) & 1);
-        half = token & 1;
-    }
 }
 
 }  // namespace tqd

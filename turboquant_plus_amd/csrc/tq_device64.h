@@ -6,8 +6,10 @@
 
 namespace tq64 {
 
-constexpr int VB = 8;    // vectors per workgroup
 constexpr int NT = 128;  // threads per workgroup
+// vectors per workgroup (template parameter VB): two staging arrays of VB * pd doubles must fit in LDS,
+// so wide vectors get fewer per workgroup
+constexpr int vectors_per_workgroup(int pd) { return pd <= 1024 ? 8 : pd <= 2048 ? 4 : 2; }
 
 template <typename T> __device__ inline double ldd(const T *p, int64_t i) { return (double)p[i]; }
 template <> __device__ inline double ldd<__half>(const __half *p, int64_t i) { return (double)__half2float(p[i]); }
@@ -21,6 +23,7 @@ struct RotArgs {
 };
 
 // in: xs[VB][pd] (entries >= d zero in WHT mode); out: ys[VB][pd].  All threads call.
+template <int VB>
 __device__ void rotate_block(const RotArgs &r, double *xs, double *ys) {
     const int tid = threadIdx.x;
     const int d = r.d, pd = r.pd;
@@ -64,7 +67,7 @@ __device__ void rotate_block(const RotArgs &r, double *xs, double *ys) {
     __syncthreads();
 }
 
-template <typename T>
+template <int VB, typename T>
 __device__ void load_block(const T *x, int64_t n, int64_t v0, int d, int pd, double *xs) {
     for (int i = threadIdx.x; i < VB * pd; i += NT) {
         const int v = i / pd, j = i % pd;
@@ -74,6 +77,7 @@ __device__ void load_block(const T *x, int64_t n, int64_t v0, int d, int pd, dou
 }
 
 // L2 norms of the VB staged vectors -> nrm[VB] (shared).
+template <int VB>
 __device__ void norms_block(const double *xs, int d, int pd, double *nrm) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int v = wave; v < VB; v += NT / 64) {

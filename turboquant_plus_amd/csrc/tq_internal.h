@@ -5,7 +5,7 @@
 #include <stdint.h>
 #include "tq.h"
 
-#define TQ_MAX_D 1024
+#define TQ_MAX_D 4096
 #define TQ_ROWS_PER_BLOCK 128
 
 // Device-resident constant tables of a quantiser.  Everything the kernels read

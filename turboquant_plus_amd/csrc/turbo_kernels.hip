@@ -1167,7 +1167,6 @@ struct AppendArgs {
     int64_t pos, n_new, blocks_per_seq, first_block, n_touched;
 };
 
-__device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, int token, int dim);
 __device__ inline float block_norm(const uint8_t *block, int bits, int token);
 
 // one workgroup rebuilds block `wg` (sequence wg / n_touched, touched block wg % n_touched)
@@ -1471,25 +1470,6 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
 }
 
 // ---- K3: packed block -> values ----------------------------------------------------
-__device__ inline uint32_t row_dword(const uint8_t *block, int row, int q) {
-    return *reinterpret_cast<const uint32_t *>(block + (q >> 2) * 2048 + row * 16 + (q & 3) * 4);
-}
-
-__device__ inline uint32_t fetch_code(const uint8_t *block, int bits, int kind, int token, int dim) {
-    int row, p, half;
-    locate(kind, token, dim, row, p, half);
-    uint32_t pc;
-    if (pair_in_tail(bits, p)) {
-        const int g = p >> 4;
-        const uint32_t tail = (row_dword(block, row, g) >> 24) | ((row_dword(block, row, 4 + g) >> 24) << 8) |
-                              ((row_dword(block, row, 8 + g) >> 24) << 16);
-        pc = (tail >> (6 * ((p & 15) - 12))) & 63u;
-    } else {
-        pc = (row_dword(block, row, pair_dword(bits, p)) >> pair_shift(bits, p)) & ((1u << (2 * bits)) - 1u);
-    }
-    return (pc >> (half * bits)) & ((1u << bits) - 1u);
-}
-
 __device__ inline float block_norm(const uint8_t *block, int bits, int token) {
     const __half *nm = reinterpret_cast<const __half *>(block + block_code_bytes(bits));
     return __half2float(nm[token]);
