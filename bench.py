@@ -20,7 +20,10 @@ when a busy stretch starts after idle time the GPU's power management first
 drops the core clock from about 1.93 GHz to about 1.3 GHz and brings it back
 over the next 25-30 ms (read in-kernel from the cycle and wall-clock counters),
 and a 20-step warm-up times that transient (+15-20 % per step) instead of the
-sustained rate a serving loop sees.
+sustained rate a serving loop sees.  When the requested `steps` steps of a leg
+take less than 60 ms (e.g. --steps 20), the leg is therefore timed as several
+consecutive blocks of exactly `steps` steps and the median block is reported
+(`timed_blocks` in the JSON line says how many).
 
 Prints ONE JSON line.  `roofline` prices the store kernel against 8 TB/s with
 the algorithmic bytes per launch (322 B per vector for turbo4: 256 B fp16 in,
@@ -41,9 +44,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 D = 128
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the reading of a
-# 1 GiB device copy (x2.000 and x1.000); figures and commands in profiles/bench_kernels_c2_c3.txt.
+# HBM bytes per launch as recorded in profiles/bench_kernels_c2_c3.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
+# this file's default run, each scaled by the reading of a 1 GiB device copy): recorded constants, not measured in
+# this run; the JSON line names the profile row next to each figure.
 TRAFFIC_BYTES = {"store4": 171.5e6, "store3": 161.8e6, "decode3": 423.5e6}
+TRAFFIC_SOURCE = {"store4": "profiles/bench_kernels_c2_c3.txt, rows k_store_kv<4,4> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)",
+                  "store3": "profiles/bench_kernels_c2_c3.txt, rows k_store_kv<3,3> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)",
+                  "decode3": "profiles/bench_kernels_c2_c3.txt, rows k_decode_attn<turbo3,turbo3> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)"}
 METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
 
 
@@ -58,20 +65,43 @@ def synth_kv(torch, heads, tokens, seed, outliers):
     return x.to(torch.float16)
 
 
-def time_steps(torch, step, steps, warmup):
-    """(wall ms per step with sync brackets, event ms per step on the launch stream)."""
+MIN_TIMED_MS = 60.0   # a leg whose `steps` steps take less than this is timed as several blocks of `steps` steps
+
+
+def time_steps(torch, step, steps, warmup, info=None):
+    """(wall ms per step with sync brackets, event ms per step on the launch stream).
+
+    Exactly `steps` steps are timed between two events / two synchronisations.  When that stretch is shorter
+    than MIN_TIMED_MS it sits inside the clock transient that follows idle time (see the module text), so the
+    measurement is repeated as consecutive blocks of `steps` steps, MIN_TIMED_MS of timed work in all (at
+    least 5 blocks), and the block with the median event time is reported; the wall figure is the mean over the
+    whole stretch.  info["timed_blocks"] says how many blocks were timed."""
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        step(warmup + i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
-    return wall, e0.elapsed_time(e1) / steps
+
+    def run_blocks(n_blocks, first):
+        """n_blocks consecutive blocks of `steps` steps with an event between blocks and no host wait in between
+        (a synchronisation per block would let the clock fall back during the gap)."""
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_blocks + 1)]
+        t0 = time.perf_counter()
+        ev[0].record()
+        for b in range(n_blocks):
+            for i in range(steps):
+                step(first + b * steps + i)
+            ev[b + 1].record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        return [ev[b].elapsed_time(ev[b + 1]) for b in range(n_blocks)], wall
+
+    times, wall = run_blocks(1, warmup)
+    n_blocks = 1
+    if times[0] < MIN_TIMED_MS:
+        n_blocks = int(min(400, max(5, math.ceil(MIN_TIMED_MS / max(times[0], 1e-3)))))
+        times, wall = run_blocks(n_blocks, warmup + steps)
+    if info is not None:
+        info["timed_blocks"] = n_blocks
+    return wall / (n_blocks * steps), sorted(times)[n_blocks // 2] / steps
 
 
 def measured_peaks_leg(torch, tqa, steps, warmup):
@@ -121,7 +151,8 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
         k, v, kp, vp = sets[i % n_sets]
         codec_k.store_kv(codec_v, k, v, out_k=kp, out_v=vp)      # one launch for the layer's K and V
 
-    wall_ms, ev_ms = time_steps(torch, step, steps, warmup)
+    info = {}
+    wall_ms, ev_ms = time_steps(torch, step, steps, warmup, info)
     n_vec = 2 * heads * tokens
     bytes_per_vec = 256 + 16 * bits + 2
     algo = n_vec * bytes_per_vec
@@ -145,7 +176,7 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
         "workload": f"turbo{bits} store, K+V fp16 [8,32768,128], 4 K outlier channels x15, block 128",
         "ms_per_step": wall_ms, "event_ms_per_step": ev_ms, "kernel_us": launch_us,
         "algorithmic_bytes_per_launch": algo, "gbs": gbs, "frac": gbs / HBM_PEAK_GBS,
-        "roundtrip_rel_mse_k": rel, "buffer_sets": n_sets,
+        "roundtrip_rel_mse_k": rel, "buffer_sets": n_sets, "timed_blocks": info["timed_blocks"],
         "decompress": {"us_per_step": lev_ms * 1e3, "launches_per_step": 1, "io": "codes + fp16 norm in, fp16 out",
                        "gbs": load_algo / (lev_ms * 1e-3) / 1e9, "frac": load_algo / (lev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
@@ -173,7 +204,8 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         q, kp, vp = sets[i % n_sets]
         attn(q, kp, vp)
 
-    wall_ms, ev_ms = time_steps(torch, step, steps, warmup)
+    info = {}
+    wall_ms, ev_ms = time_steps(torch, step, steps, warmup, info)
     algo = 2 * B * Hkv * N * 50
     us = ev_ms * 1e3
     gbs = algo / (us * 1e-6) / 1e9
@@ -203,8 +235,10 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
     return {
         "workload": "fused decode attention, turbo3 K/V, B16 Hq32 Hkv8 d128 ctx 32768, queries rotated in-step",
         "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
+        "timed_blocks": info["timed_blocks"],
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES["decode3"], "algorithmic_bytes_per_step": algo,
+                     "traffic": TRAFFIC_BYTES["decode3"], "traffic_source": TRAFFIC_SOURCE["decode3"],
+                     "algorithmic_bytes_per_step": algo,
                      "kernel": "k_decode_attn<turbo3,turbo3> (+ k_attn_combine in the step time)"},
         "buffer_sets": n_sets,
         "serving_step": {"workload": "tq_append_kv of one token per sequence + decode attention",
@@ -231,34 +265,47 @@ def asym_decode_leg(torch, tqa, steps, warmup):
     pos = torch.stack([torch.randperm(N, generator=g, device="cuda")[:64] for _ in range(B * Hq)]).view(B, Hq, 64)
     bias.scatter_(2, pos, 6.0)
     # fraction of (batch, q-head, position) whose final softmax weight is below tau (the definition of the
-    # reference's scripts/measure_skip_rate.py:69-74), from the stored K in fp32
-    below, scale = 0, 1.0 / math.sqrt(D)
-    for s in range(B * Hkv):
-        qi, sc = tqa.q8_0_unpack(kq[s * perk:(s + 1) * perk], 1, N)
-        kd = (qi.view(N, 4, 32).float() * sc.view(N, 4, 1)).view(N, D)
-        b, h = divmod(s, Hkv)
-        logit = q[b, 4 * h:4 * h + 4].float() @ kd.t() * scale + bias[b, 4 * h:4 * h + 4]
-        below += int((torch.softmax(logit, dim=-1) < 1e-6).sum())
-        del qi, sc, kd, logit
-    final_weight_skip = below / float(B * Hq * N)
+    # reference's scripts/measure_skip_rate.py:69-74), from the stored K in fp32; and, with the kernel's own
+    # predicate restated in torch, the fraction of 64-token V rows the kernel does not fetch: it drops a tile's
+    # PV work when all 4 heads x 64 weights are below tau against the running maximum of the split, requests the
+    # next tile's V row ahead only after a tile that was not dropped, and fetches on demand otherwise - so a row
+    # stays unfetched when its tile and the tile before it are both dropped (never the first tile of a split).
+    def cache_stats(qq, n_splits):
+        below, rows_saved, scale = 0, 0, 1.0 / math.sqrt(D)
+        tiles_per_split = -(-(N // 64) // n_splits)
+        for s in range(B * Hkv):
+            qi, sc = tqa.q8_0_unpack(kq[s * perk:(s + 1) * perk], 1, N)
+            kd = (qi.view(N, 4, 32).float() * sc.view(N, 4, 1)).view(N, D)
+            b, h = divmod(s, Hkv)
+            logit = qq[b, 4 * h:4 * h + 4].float() @ kd.t() * scale + bias[b, 4 * h:4 * h + 4]
+            below += int((torch.softmax(logit, dim=-1) < 1e-6).sum())
+            lt = logit.view(4, N // 64 // tiles_per_split, tiles_per_split, 64)      # [head, split, tile, token]
+            run_max = torch.cummax(lt.amax(dim=-1), dim=-1).values                   # running maximum incl. the tile
+            dropped = ((lt - run_max[..., None]).exp() < 1e-6).all(dim=-1).all(dim=0)  # [split, tile]
+            rows_saved += int((dropped[:, 1:] & dropped[:, :-1]).sum())
+            del qi, sc, kd, logit, lt
+        return below / float(B * Hq * N), rows_saved / float(B * Hkv * (N // 64))
     out = {}
     q_peaked = (q.float() * 16.0).to(torch.float16)  # a second input for Sparse V: logits 16 x as spread, few tiles matter
     for name, tau, qq in (("dense", 0.0, q), ("sparse_v", 1e-6, q), ("sparse_v_peaked_queries", 1e-6, q_peaked)):
         attn = tqa.DecodeAttention(None, vc, B, Hq, Hkv, N, sparse_v_tau=tau)
         wall_ms, ev_ms = time_steps(torch, lambda i: attn(qq, kq, vp, bias=bias), steps, warmup)
         skip = attn.skip_rate() if tau else 0.0
-        algo = B * Hkv * N * (136 + (1.0 - 0.0) * 34)  # dense bytes; Sparse V skips whole 64-token V tiles only
+        algo = B * Hkv * N * (136 + 34)               # dense bytes: the roofline figure of every variant
         us = ev_ms * 1e3
         out[name] = {"us_per_step": us, "skip_rate": skip, "n_splits": attn.params.n_splits,
                      "achieved_gbs": algo / (us * 1e-6) / 1e9, "frac": algo / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
-        if tau and qq is q:
+        if tau:
+            final_weight_skip, rows_saved = cache_stats(qq, attn.params.n_splits)
             # the kernel tests exp(logit - running maximum of its split), without the softmax denominator
             out[name]["skip_rate_final_weight"] = final_weight_skip
-        if tau:
-            out[name]["bytes_required"] = B * Hkv * N * (136 + (1.0 - skip) * 34)
+            out[name]["v_rows_not_fetched"] = rows_saved
+            out[name]["bytes_required"] = B * Hkv * N * (136 + (1.0 - rows_saved) * 34)
     out["workload"] = ("decode attention, K q8_0-style + V turbo2, B4 Hq32 Hkv8 ctx 131072, +6 bias on 64 key "
                        "positions per head as an fp32 bias input (67 MB, not counted), Sparse V tau 1e-6; "
-                       "sparse_v_peaked_queries: the same cache with the queries scaled x16")
+                       "sparse_v_peaked_queries: the same cache with the queries scaled x16; skip_rate = (query, position) "
+                       "pairs whose weight the kernel dropped, v_rows_not_fetched = fraction of 64-token V rows it never "
+                       "requested (whole tiles only), bytes_required = K + the V rows it did request")
     out["algorithmic_bytes_per_step"] = B * Hkv * N * 170
     return out
 
@@ -316,14 +363,17 @@ def cpu_baseline(bits):
     v = rng.standard_normal((n, D)).astype(np.float16)
     s1, s2, _ = O.sign_diagonals(D, np.random.default_rng(42))
     cent = O.centroids_for(bits, D)
-    reps = 32                                         # 8 x (one head of K + one head of V) = all of config 2; four times over
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        for x, kind in ((k, "k"), (v, "v")):
-            idx, g, _ = O.turbo_encode(x, s1, s2, cent)
-            O.layout_pack(idx, g, bits, kind)
-    dt = time.perf_counter() - t0
-    algo = reps * 2 * n * (256 + 16 * bits + 2)
+    passes, n_samples = 6, 5                          # a sample = 6 passes over one head of K and one of V (about 2 s)
+    times = []
+    for _ in range(n_samples):
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            for x, kind in ((k, "k"), (v, "v")):
+                idx, g, _ = O.turbo_encode(x, s1, s2, cent)
+                O.layout_pack(idx, g, bits, kind)
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[n_samples // 2]
+    algo = passes * 2 * n * (256 + 16 * bits + 2)
     # attention leg: one (batch, kv head) group of config 3, decompress -> softmax -> PV
     q = rng.standard_normal((4, D))
     idx, g, _ = O.turbo_encode(k, s1, s2, cent)
@@ -334,8 +384,9 @@ def cpu_baseline(bits):
     O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
     dta = time.perf_counter() - t0
     return ({"value": algo / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"NumPy oracle turbo{bits} encode+pack of all 2 x 262144 fp16 vectors of config 2, four times over "
-                       f"(32 passes over one head of K and one of V), {dt:.2f} s, single-threaded NumPy (no BLAS on this path)",
+             "sample": f"NumPy oracle turbo{bits} encode+pack of {passes} x 2 x 32768 fp16 vectors (one head of K and one of V "
+                       f"of config 2, {passes} passes = 3/4 of the layer), median of {n_samples} such samples "
+                       f"({dt:.2f} s; min {min(times):.2f}, max {max(times):.2f}), single-threaded NumPy (no BLAS on this path)",
              "host_cpus": os.cpu_count()},
             {"value": dta * 128 * 1e6, "unit": "µs/step", "cores": blas_threads or 1, "kind": "port",
              "sample": f"NumPy oracle decompress->softmax->PV for 1 of 128 (batch, kv-head) groups at ctx 32768 "
@@ -423,7 +474,8 @@ def main():
         "config": {"workload": s4["workload"], "global_batch": 2 * 8 * 32768, "io": "fp16 in, 4-bit codes + fp16 norm out",
                    "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": s4["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s4["frac"],
-                     "traffic": TRAFFIC_BYTES["store4"], "kernel": "k_store_kv<4,4> (K and V of the layer, one launch per step)",
+                     "traffic": TRAFFIC_BYTES["store4"], "traffic_source": TRAFFIC_SOURCE["store4"],
+                     "kernel": "k_store_kv<4,4> (K and V of the layer, one launch per step)", "timed_blocks": s4["timed_blocks"],
                      "kernel_us": s4["kernel_us"],
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
