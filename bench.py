@@ -429,6 +429,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--legs", default="all",
+                    help="comma-separated subset of store4,store3,decode,asym,tile,boundary,peaks (profiling runs); "
+                         "the JSON line then holds only those legs and is not the benchmark's line")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (5x) so that FETCH_SIZE / WRITE_SIZE counters can be calibrated")
     args = ap.parse_args()
@@ -450,6 +453,25 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.legs != "all":
+        legs = set(args.legs.split(","))
+        part = {"partial_run": sorted(legs), "steps": args.steps, "warmup": args.warmup}
+        if "store4" in legs:
+            part["turbo4_store"] = store_leg(torch, tqa, 4, args.steps, args.warmup)
+        if "store3" in legs:
+            part["turbo3_store"] = store_leg(torch, tqa, 3, args.steps, args.warmup)
+        if "decode" in legs:
+            part["decode_attn"] = decode_leg(torch, tqa, args.steps, args.warmup)
+        if "asym" in legs:
+            part["asym_decode_q8k_turbo2v"] = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+        if "tile" in legs:
+            part["score_tile"] = score_tile_leg(torch, tqa, args.steps, args.warmup)
+        if "boundary" in legs:
+            part["boundary_layer_q8k_q8v"] = boundary_layer_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+        if "peaks" in legs:
+            part["measured_peaks"] = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
+        print(json.dumps(part, ensure_ascii=False))
+        return
     s4 = store_leg(torch, tqa, 4, args.steps, args.warmup)
     s3 = store_leg(torch, tqa, 3, args.steps, args.warmup)
     dec = decode_leg(torch, tqa, args.steps, args.warmup)

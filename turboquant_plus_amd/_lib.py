@@ -11,7 +11,9 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtq_hip.so")
+# TQ_HIP_LIBRARY names another build of the same library (the measurement variants that
+# `make KNOCKOUT=.. OUT=..` produces); unset, the product library next to this file is loaded.
+LIB_PATH = os.environ.get("TQ_HIP_LIBRARY") or os.path.join(_HERE, "libtq_hip.so")
 
 TQ_F16, TQ_F32, TQ_F64 = 0, 1, 2
 ROT_DENSE, ROT_WHT = 0, 1

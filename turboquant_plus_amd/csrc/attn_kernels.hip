@@ -100,7 +100,7 @@ __device__ __forceinline__ uint32_t lead_progress(uint32_t *mark, uint32_t mine,
 template <int BITS> __device__ __forceinline__ void load_row(const uint8_t *block, int row, uint32_t (&w)[4 * BITS]) {
 #pragma unroll
     for (int c = 0; c < BITS; ++c) {
-        const uint4 u = *reinterpret_cast<const uint4 *>(block + c * 2048 + row * 16);
+        const uint4 u = stream_load<STREAM_ATTN_ROWS>(reinterpret_cast<const uint4 *>(block + c * 2048 + row * 16));
         w[4 * c] = u.x; w[4 * c + 1] = u.y; w[4 * c + 2] = u.z; w[4 * c + 3] = u.w;
     }
 }
@@ -1173,7 +1173,7 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) (ubase + (int64_t)(8 * j + i) * nk)[lane_off] = (TO)acc[mb][4 * j + i];
+                            for (int i = 0; i < 4; ++i) stream_store<STREAM_LOGITS>((ubase + (int64_t)(8 * j + i) * nk) + lane_off, (TO)acc[mb][4 * j + i]);
                     } else {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
@@ -1202,7 +1202,7 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
                             if (pair_ok && (full || (qi < (int)nq && k0 + 1 < nk))) {
                                 const uint32_t u = (uint32_t)__half_as_ushort(__float2half_rn(v0)) |
                                                    ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
-                                *reinterpret_cast<uint32_t *>(p) = u;
+                                stream_store<STREAM_LOGITS>(reinterpret_cast<uint32_t *>(p), u);
                             } else if (qi < (int)nq) {
                                 if (k0 < nk) p[0] = __float2half_rn(v0);
                                 if (k0 + 1 < nk) p[1] = __float2half_rn(v1);

@@ -9,6 +9,51 @@ namespace tqd {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
+// ---- streaming stores -----------------------------------------------------------
+// Output that a launch writes once and never reads back goes out with the non-temporal hint: the lines do not
+// wait in the L2 for the end-of-kernel write-back, so the writes overlap the rest of the launch.
+// TQ_STREAM_SITES (bit mask, measurement builds) switches the hint off per family of kernels.
+#ifndef TQ_STREAM_SITES
+#define TQ_STREAM_SITES 0xFFFF
+#endif
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <int SITE> __device__ __forceinline__ void stream_store(uint32_t *p, uint32_t v) {
+    if constexpr ((TQ_STREAM_SITES & SITE) != 0) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+template <int SITE> __device__ __forceinline__ void stream_store(float *p, float v) {
+    if constexpr ((TQ_STREAM_SITES & SITE) != 0) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+template <int SITE> __device__ __forceinline__ void stream_store(uint4 *p, uint4 v) {
+    if constexpr ((TQ_STREAM_SITES & SITE) != 0) {
+        const u32x4_t u = {v.x, v.y, v.z, v.w};
+        __builtin_nontemporal_store(u, reinterpret_cast<u32x4_t *>(p));
+    } else {
+        *p = v;
+    }
+}
+constexpr int STREAM_STORE_CODES = 1, STREAM_LOAD_OUT = 2, STREAM_LOGITS = 4, STREAM_Q8 = 8, STREAM_ATTN_ROWS = 16,
+              STREAM_STORE_V_IN = 32;
+// 16 bytes of input that a launch reads exactly once, every 128-byte line whole within one instruction
+template <int SITE> __device__ __forceinline__ float4 stream_load(const float4 *p) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    if constexpr ((TQ_STREAM_SITES & SITE) != 0) {
+        const f32x4_t u = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(p));
+        return make_float4(u[0], u[1], u[2], u[3]);
+    } else {
+        return *p;
+    }
+}
+template <int SITE> __device__ __forceinline__ uint4 stream_load(const uint4 *p) {
+    if constexpr ((TQ_STREAM_SITES & SITE) != 0) {
+        const u32x4_t u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+        return make_uint4(u[0], u[1], u[2], u[3]);
+    } else {
+        return *p;
+    }
+}
+
 // ---- cross-lane exchange ------------------------------------------------------
 // DPP control words (GCN3+/CDNA): quad_perm = 4 x 2-bit selectors, 0x12n =
 // row_ror:n, 0x141 = row_half_mirror.  Every pattern used here reads a valid

@@ -143,6 +143,21 @@ struct StoreArgs {
     int64_t blocks_per_seq;
 };
 
+// Measurement builds only (make KNOCKOUT=<bits>, default 0 = the product): TQ_KNOCKOUT removes one phase of the
+// fp16 store kernels so that its share of the launch time and of the vector instructions can be read off
+// (results are then meaningless).  1: quantiser compares (a value's code bits come from one xor of its raw
+// bits); 2: four-point butterfly over the input slices; 4: level counts and sum c^2; 8: the sum-of-squares
+// MFMAs (norm = 1); 16: the code stores; 32: the HBM reads (every wavefront reads the same 256 KB).
+#ifndef TQ_KNOCKOUT
+#define TQ_KNOCKOUT 0
+#endif
+// 16 bytes of input (read with the default cache policy: the four loads of a K unit touch every 128-byte line of
+// the unit four times, and with the non-temporal hint each touch went to memory: 20.7 -> 29.8 us for 262 144 K rows)
+__device__ __forceinline__ uint4 load_input16(const uint4 *p) { return *p; }
+__device__ __forceinline__ uint32_t ko_append4(uint32_t w, float y0, float y1, float y2, float y3) {
+    return ((w << 4) ^ __float_as_uint(y0)) + ((__float_as_uint(y1) ^ __float_as_uint(y2)) + __float_as_uint(y3));
+}
+
 // ---- K2, fp16 input: rotation on the matrix cores ------------------------------------
 // R' = D2 H D1 has entries +-1, so with fp16 inputs every product of X R'^T is exact and
 // only the fp32 accumulation rounds (same error class as the butterfly).  Quantisation uses
@@ -412,6 +427,7 @@ __device__ __forceinline__ uint32_t take_ticket(uint32_t *counter, int lane) {
 }
 
 constexpr uint32_t DRAW_TICKET = 0xFFFFFFFFu;
+constexpr int K_UNITS_AHEAD = 1;
 // first_ticket: the wavefront's first two tickets are first_ticket and first_ticket + 1 (the counter starts past
 // them), or DRAW_TICKET to draw them.  `stage` makes the workgroup's LDS copy of the constant operands (frag,
 // flips) readable; it runs after the first inputs have been requested.
@@ -435,6 +451,9 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     // are clamped, and `valid` says whether the data is to be used.
     auto fetch = [&](uint32_t unit, uint4 (&xb)[4], bool &valid) {
         unit = unit < last_unit ? unit : last_unit;
+#if TQ_KNOCKOUT & 32
+        unit &= 63u;  // every wavefront reads the same 256 KB: no HBM reads
+#endif
         const uint4 *p;
         if constexpr (RAGGED) {
             const uint32_t blk = unit >> 3, seq = blk / bps, bis = blk - seq * bps;
@@ -447,7 +466,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             p = reinterpret_cast<const uint4 *>(x + ((int64_t)unit * 16 + n16) * 128 + 32 * kc);
         }
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = p[ks];
+        for (int ks = 0; ks < 4; ++ks) xb[ks] = load_input16(p + ks);
     };
 
     // an exact zero counts as positive only if the middle boundary is below zero
@@ -455,7 +474,9 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     const int diag_sel = n16 & 3;
     const bool diag_here = kc == (n16 >> 2);
 
-    constexpr int DEPTH = 2;  // units of input in flight per wavefront
+    // units of input in flight per wavefront: one ahead measures faster than two (262 144 rows of 3-bit K alone
+    // 16.9 against 18.2 us, the fused K+V launch 34.4 against 36.0 us)
+    constexpr int DEPTH = K_UNITS_AHEAD;
     uint4 xq[DEPTH][4];
     bool xvalid[DEPTH];
     uint32_t cur[DEPTH];
@@ -500,10 +521,14 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             // ||x||^2 on the matrix cores as well: the diagonal of X X^T (the same registers serve as
             // both operands); token n16's entry is element n16 % 4 of lane quarter n16 / 4
             float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+#if TQ_KNOCKOUT & 8
+            gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
+#else
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
                 gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
                                                               gram, 0, 0, 0);
+#endif
             float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
             ss = diag_here ? ss : 0.0f;
             cur[r] = next;
@@ -522,12 +547,16 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             float4_t y[8];
 #pragma unroll
             for (int f0 = 0; f0 < 2; ++f0) {
+#if TQ_KNOCKOUT & 2
+                y[0 + f0] = q[f0][0]; y[2 + f0] = q[f0][1]; y[4 + f0] = q[f0][2]; y[6 + f0] = q[f0][3];
+#else
                 const float4_t s01 = q[f0][0] + q[f0][1], d01 = q[f0][0] - q[f0][1];
                 const float4_t s23 = q[f0][2] + q[f0][3], d23 = q[f0][2] - q[f0][3];
                 y[0 + f0] = s01 + s23;
                 y[2 + f0] = d01 + d23;
                 y[4 + f0] = s01 - s23;
                 y[6 + f0] = d01 - d23;
+#endif
             }
             // value v = 0..31 of this lane (dim 32*kc + v) up to the sign s2
             auto val = [&](int v) -> float { return y[v >> 2][v & 3]; };
@@ -542,9 +571,16 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #pragma unroll
                 for (int j = 3; j >= 0; --j) {
                     const int v = 8 * j;
+#if TQ_KNOCKOUT & 1
+                    uint32_t w = ko_append4(thr[1] > 0.f ? 0u : 1u, val(v + 7), val(v + 6), val(v + 5), val(v + 4));
+                    w = ko_append4(w, val(v + 3), val(v + 2), val(v + 1), val(v));
+#else
                     uint32_t w = append4_b3(0u, val(v + 7), val(v + 6), val(v + 5), val(v + 4), thr);
                     w = append4_b3(w, val(v + 3), val(v + 2), val(v + 1), val(v), thr);
+#endif
+#if !(TQ_KNOCKOUT & 4)
                     count_levels<3>(w, n);
+#endif
                     w4[j] = fold_codes<3>(nonzero ? w ^ flip[j] : (zero_word & 0x00924924u));
                 }
                 g[0] = __builtin_amdgcn_perm(w4[3], w4[0], 0x04020100u);
@@ -560,11 +596,21 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
                         yn[m] = val(v + m) * inv;
+#if TQ_KNOCKOUT & 1
+                        if (m == 0)
+#endif
                         e[m] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(qlut) + quant_lut_offset(yn[m]));
                     }
+#if TQ_KNOCKOUT & 1
+                    uint32_t w = ko_append4(e[0].x & 1u, yn[7], yn[6], yn[5], yn[4]);
+                    w = ko_append4(w, yn[3], yn[2], yn[1], yn[0]);
+#else
                     uint32_t w = append4_lut(0u, yn[7], yn[6], yn[5], yn[4], e[7], e[6], e[5], e[4]);
                     w = append4_lut(w, yn[3], yn[2], yn[1], yn[0], e[3], e[2], e[1], e[0]);
+#endif
+#if !(TQ_KNOCKOUT & 4)
                     count_levels<4>(w, n);
+#endif
                     g[j] = fold_codes<4>(nonzero ? w ^ flip[j] : (zero_word & 0x88888888u));
                 }
             } else {
@@ -580,8 +626,11 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             const uint32_t blk = unit >> 3;
             const int row = (int)(unit & 7) * 16 + n16;
             uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
+#if TQ_KNOCKOUT & 16
+            if (g[0] == 0x12345678u && g[BITS - 1] == 0x9abcdef0u)   // keeps the codes alive; not taken for real data
+#endif
 #pragma unroll
-            for (int j = 0; j < BITS; ++j) *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kc * 4) = g[j];
+            for (int j = 0; j < BITS; ++j) stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kc * 4), g[j]);
 
             float gn = norm;
             if (a.norm_correction) {
@@ -748,7 +797,9 @@ struct StoreVArgs {
 // ticket is the caller's (the counter starts past the tickets given out this way), so the first tile's
 // input is requested before anything is waited for; `stage` then makes the workgroup's copy of the
 // constant operands (frag, s2: LDS) readable.
-template <int BITS, bool RAGGED, typename Stage>
+// STREAM_IN: the input is read with the non-temporal hint (every 128-byte line is touched by two instructions of one
+// wavefront, back to back).  It gains 2 us in the fused K+V launch and loses 1 us in the V-only kernel (measured).
+template <int BITS, bool RAGGED, bool STREAM_IN, typename Stage>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const float *s2, uint32_t first_ticket, Stage &&stage) {
@@ -771,6 +822,9 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // whether the row exists.
     auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
         unit = unit < last_unit ? unit : last_unit;
+#if TQ_KNOCKOUT & 32
+        unit &= 15u;  // every wavefront reads the same 256 KB: no HBM reads
+#endif
         const uint32_t blk = unit >> 1;
         const int tb = (int)(unit & 1) * 64 + 16 * (n16 >> 2) + 4 * u + (n16 & 3);
         const uint4 *p;
@@ -785,7 +839,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             p = reinterpret_cast<const uint4 *>(x + ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq);
         }
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = p[4 * ks];
+        for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
     };
 
     uint4 xq[2][4];
@@ -844,10 +898,14 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                                                                         float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
             // ||x||^2: diagonal of X X^T; element i of this lane is row 4kq + i, column n16
             float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+#if TQ_KNOCKOUT & 8
+            gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
+#else
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
                 gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
                                                               gram, 0, 0, 0);
+#endif
             if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
             else fetch(next, 5 - q, xb, xvalid[q & 1]);
 
@@ -865,12 +923,16 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             float4_t y[4][2];
 #pragma unroll
             for (int d0 = 0; d0 < 2; ++d0) {
+#if TQ_KNOCKOUT & 2
+                y[0][d0] = qq[d0][0] * inv; y[1][d0] = qq[d0][1] * inv; y[2][d0] = qq[d0][2] * inv; y[3][d0] = qq[d0][3] * inv;
+#else
                 const float4_t s01 = qq[d0][0] + qq[d0][1], d01 = qq[d0][0] - qq[d0][1];
                 const float4_t s23 = qq[d0][2] + qq[d0][3], d23 = qq[d0][2] - qq[d0][3];
                 y[0][d0] = (s01 + s23) * inv;
                 y[1][d0] = (d01 + d23) * inv;
                 y[2][d0] = (s01 - s23) * inv;
                 y[3][d0] = (d01 - d23) * inv;
+#endif
             }
             uint32_t n1[4] = {0, 0, 0, 0};  // 2-bit: per-token count of the level bit
             // groups in descending pair order: pair 4u + 2hf + i/2, high code (odd i) first
@@ -880,6 +942,11 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 const int j = grp_word(BITS, 4 * u);
                 const float y0 = y[0 | (hf << 1)][0][i], y1 = y[0 | (hf << 1)][1][i];
                 const float y2 = y[1 | (hf << 1)][0][i], y3 = y[1 | (hf << 1)][1][i];
+#if TQ_KNOCKOUT & 1
+                w[0][j] = (w[0][j] << 1) ^ __float_as_uint(y0); w[1][j] = (w[1][j] << 1) ^ __float_as_uint(y1);
+                w[2][j] = (w[2][j] << 1) ^ __float_as_uint(y2); w[3][j] = (w[3][j] << 1) ^ __float_as_uint(y3);
+                if constexpr (BITS == 99)
+#endif
                 if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
                 else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr0);
                 else {
@@ -893,6 +960,11 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             }
             // level counts of the four tokens, one byte per token, summed over the 16 columns
             uint32_t cnt[NT];
+#if TQ_KNOCKOUT & 4
+#pragma unroll
+            for (int p = 0; p < NT; ++p) cnt[p] = 0x01010101u;
+            if constexpr (BITS == 99)
+#endif
             if constexpr (BITS == 4) {
                 // dword u of every row is complete: vertical sums of the level-bit products over the rows
                 constexpr uint32_t K0 = 0x11111111u;
@@ -933,8 +1005,12 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             }
             float cs = 128.0f * coef[0];
             const int sh = BITS == 4 ? 8 * (((n16 & 1) << 1) | ((n16 >> 1) & 1)) : 8 * (n16 & 3);
+#if TQ_KNOCKOUT & 4
+            cs += (float)(cnt[NT - 1] >> sh);
+#else
 #pragma unroll
             for (int p = 1; p < NT; ++p) cs = fmaf(coef[p], (float)((row16_sum(cnt[p]) >> sh) & 0xFFu), cs);
+#endif
             const int isel = n16 & 3;
             const float nsel = isel == 0 ? nrm[0] : isel == 1 ? nrm[1] : isel == 2 ? nrm[2] : nrm[3];
             const float gn = a.norm_correction ? nsel * __builtin_amdgcn_rsqf(cs) : nsel;
@@ -967,7 +1043,10 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             for (int j = 0; j < BITS; ++j) {
                 uint32_t g = w[dd][j];
                 if constexpr (BITS == 3) g = __builtin_amdgcn_perm(w[dd][3], g, 0x04020100u + ((uint32_t)j << 24));
-                *reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kq * 4) = g;
+#if TQ_KNOCKOUT & 16
+                if (g == 0x12345678u)   // keeps the codes alive; practically never taken
+#endif
+                stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kq * 4), g);
             }
         }
         unit = next;
@@ -990,7 +1069,7 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
     __shared__ __attribute__((aligned(16))) uint4 frag_s[STAGED ? 512 : 1];
     __shared__ uint32_t flip_s[16];
     const int t = threadIdx.x, wave = t >> 6;
-    if ((t & 63) == 0) counter[wave] = 2;  // tickets 0 and 1 are taken without asking
+    if ((t & 63) == 0) counter[wave] = K_UNITS_AHEAD;  // the first tickets are taken without asking
     if constexpr (STAGED) {
         const uint4 c0 = a.afrag[t], c1 = a.afrag[256 + t];
         const uint32_t c3 = a.s2flip[t & 15];
@@ -1026,7 +1105,7 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
         if (t < 128) s2_s[t] = c2;
         __syncthreads();
     };
-    store_v_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
+    store_v_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
                                 stage);
 }
 
@@ -1058,7 +1137,7 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
         if (t < 16) flip_s[t] = c3;
         __syncthreads();
     };
-    store_v_units<VB, RAGGED>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
+    store_v_units<VB, RAGGED, true>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
                               wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v, frag_s, s2_s,
                               (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
     store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
@@ -1684,7 +1763,7 @@ __device__ __forceinline__ void load_k16_body(const uint8_t *packed, __half *out
             const int tr = 4 * c + (lane >> 4);  // token of the unit this lane stores a piece of
             const uint4 piece = *reinterpret_cast<const uint4 *>(mine + tr * XROW + (lane & 15) * 16);
             if (tok_base + tr < a.tokens)
-                *reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok_base + tr) * 128 + 8 * (lane & 15))) = piece;
+                stream_store<STREAM_LOAD_OUT>(reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok_base + tr) * 128 + 8 * (lane & 15))), piece);
         }
     }
 }
@@ -1797,7 +1876,7 @@ __device__ __forceinline__ void load_v16_body(const uint8_t *packed, __half *out
             const int64_t tok = tok_base + 16 * c + 4 * wave + (lane >> 4);
             const uint4 piece = *reinterpret_cast<const uint4 *>(mine + tr * XROW + (lane & 15) * 16);
             if (tok < a.tokens)
-                *reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok) * 128 + 8 * (lane & 15))) = piece;
+                stream_store<STREAM_LOAD_OUT>(reinterpret_cast<uint4 *>(out + (((int64_t)seq * a.tokens + tok) * 128 + 8 * (lane & 15))), piece);
         }
     }
 }
@@ -1931,7 +2010,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store_f16(const __half *x, uint8_t
     uint4 *dst = reinterpret_cast<uint4 *>(packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136));
     for (int i = tid; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) {
         const int c = i >> 7;  // chunks 0..7 of 128 pieces each, then the scales
-        dst[i] = *reinterpret_cast<const uint4 *>(c < 8 ? img + c * Q8_LDS_CHUNK + (i & 127) * 16 : img + 8 * Q8_LDS_CHUNK + (i - 1024) * 16);
+        stream_store<STREAM_Q8>(dst + i, *reinterpret_cast<const uint4 *>(c < 8 ? img + c * Q8_LDS_CHUNK + (i & 127) * 16 : img + 8 * Q8_LDS_CHUNK + (i - 1024) * 16));
     }
 }
 
@@ -1974,7 +2053,7 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v(const TI *x, uint8_t *pack
     }
     __syncthreads();
     uint4 *dst = reinterpret_cast<uint4 *>(packed + blk * (int64_t)(TQ_ROWS_PER_BLOCK * 136));
-    for (int i = threadIdx.x; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) dst[i] = reinterpret_cast<const uint4 *>(img)[i];
+    for (int i = threadIdx.x; i < TQ_ROWS_PER_BLOCK * 136 / 16; i += 256) stream_store<STREAM_Q8>(dst + i, reinterpret_cast<const uint4 *>(img)[i]);
 }
 
 // fp16 input, 16-byte aligned: the block's 32 KB come in as 16-byte pieces that are contiguous across the lanes and
