@@ -259,6 +259,12 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                 ql[idx] = make_uint2((s << (b - 1)) | below, tbits);
             }
             rc = rc ? rc : upload(&h->quant_lut, ql);
+            // two handles whose tables hash alike (FNV-1a over the bytes; the tables are a function of `bits` and the
+            // fp32 boundaries) can share one LDS copy in the fused K+V store
+            uint64_t hash = 1469598103934665603ull;
+            const unsigned char *bytes = reinterpret_cast<const unsigned char *>(ql.data());
+            for (size_t i = 0; i < ql.size() * sizeof(uint2); ++i) hash = (hash ^ bytes[i]) * 1099511628211ull;
+            h->quant_lut_hash = hash;
         }
         // squared centroid of magnitude level m as a multilinear form in the bits of m
         // (Moebius transform over subsets), for counting-based sums of c^2

@@ -43,6 +43,7 @@ struct tq_handle {
                            // rotated value: .x = sign << (bits-1) | number of positive boundaries below the bin,
                            // .y = fp32 bits of the one boundary inside the bin (+inf when there is none)
     int quant_lut_ok;      // every bin holds at most one boundary (else the table cannot decide a level)
+    uint64_t quant_lut_hash;  // hash of the table's contents
     int zero_code;         // codebook index of the value 0.0 (#boundaries below 0)
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };

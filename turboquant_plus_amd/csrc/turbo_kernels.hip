@@ -147,7 +147,7 @@ struct StoreArgs {
 // fp16 store kernels so that its share of the launch time and of the vector instructions can be read off
 // (results are then meaningless).  1: quantiser compares (a value's code bits come from one xor of its raw
 // bits); 2: four-point butterfly over the input slices; 4: level counts and sum c^2; 8: the sum-of-squares
-// MFMAs (norm = 1); 16: the code stores; 32: the HBM reads (every wavefront reads the same 256 KB).
+// MFMAs (norm = 1); 16: the code stores; 32: the HBM reads (a wavefront re-reads the first units of its share).
 #ifndef TQ_KNOCKOUT
 #define TQ_KNOCKOUT 0
 #endif
@@ -452,7 +452,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     auto fetch = [&](uint32_t unit, uint4 (&xb)[4], bool &valid) {
         unit = unit < last_unit ? unit : last_unit;
 #if TQ_KNOCKOUT & 32
-        unit &= 63u;  // every wavefront reads the same 256 KB: no HBM reads
+        unit = lo + (((unit - lo) / step) & 7u) * step;  // the first eight units of the share over and over: no HBM reads
 #endif
         const uint4 *p;
         if constexpr (RAGGED) {
@@ -652,7 +652,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 // 16q + 4u + i (i = 0..3) of dim 16*dd + 64*hf + n for the four rows dd and both dim halves.
 // A group of appends takes one token (u, i) and one dim half and adds its code to the current
 // dword of each of the four rows; sub-tiles run u = 3..0 so that pairs arrive in descending
-// order.  Values are normalised by the token's norm first (thresholds are shared).
+// order.  2- and 3-bit codes compare against the token's scaled boundaries; 4-bit codes normalise the values
+// by the token's norm first (the table is indexed by the normalised value).
 //   m = 64hf + 32d1 + 16d0 + n,  k = 32ks + 8kb + e,  dd = 2 d1 + d0
 //   y'[m] = s2[m] * sum_ks (-1)^popcount((d1 + 2hf) & ks) * Q[d0][ks],  Q[d0][ks] = X[ks] B[d0][ks],
 //   B[d0][ks][8kb + e][n] = s1[k] * H[16 d0 + n][k]
@@ -789,6 +790,7 @@ struct StoreVArgs {
     const float *sqcoef;  // multilinear coefficients of c^2 over the level bits
     const uint2 *quant_lut;  // tq_handle::quant_lut (4-bit codes)
     int norm_correction;
+    int share_k_lut;      // fused K+V store: V's 4-bit table equals K's, which is already in LDS
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
 };
@@ -823,7 +825,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
         unit = unit < last_unit ? unit : last_unit;
 #if TQ_KNOCKOUT & 32
-        unit &= 15u;  // every wavefront reads the same 256 KB: no HBM reads
+        unit = lo + (((unit - lo) / step) & 1u) * step;  // the first two tiles of the share over and over: no HBM reads
 #endif
         const uint32_t blk = unit >> 1;
         const int tb = (int)(unit & 1) * 64 + 16 * (n16 >> 2) + 4 * u + (n16 & 3);
@@ -911,12 +913,20 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 
             float nrm[4];
             float4_t inv;
+            float thr_tok[4][NT];  // 2- and 3-bit codes: this token's boundaries scaled by sqrt(128) ||x|| (as the K rows do)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float ss = row16_sum(n16 == 4 * kq + i ? gram[i] : 0.0f);
                 nrm[i] = __builtin_amdgcn_sqrtf(ss);
                 const bool nz = ss > 0.0f;
-                inv[i] = nz ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;  // 1 / (||x|| sqrt(128))
+                if constexpr (BITS == 4) {
+                    inv[i] = nz ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;  // 1 / (||x|| sqrt(128))
+                } else {
+                    inv[i] = 1.0f;
+                    const float scale = nz ? nrm[i] * 11.313708498984761f : 1.0f;
+#pragma unroll
+                    for (int k = 0; k < NT; ++k) thr_tok[i][k] = thr0[k] * scale;
+                }
                 zbits |= nz ? 0u : 1u << (4 * u + i);
             }
             // butterfly over the input slices, then normalise: y[fh][d0] is row dd = 2(fh % 2) + d0, dim half fh / 2
@@ -928,10 +938,17 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #else
                 const float4_t s01 = qq[d0][0] + qq[d0][1], d01 = qq[d0][0] - qq[d0][1];
                 const float4_t s23 = qq[d0][2] + qq[d0][3], d23 = qq[d0][2] - qq[d0][3];
-                y[0][d0] = (s01 + s23) * inv;
-                y[1][d0] = (d01 + d23) * inv;
-                y[2][d0] = (s01 - s23) * inv;
-                y[3][d0] = (d01 - d23) * inv;
+                if constexpr (BITS == 4) {  // the table is indexed by the normalised value
+                    y[0][d0] = (s01 + s23) * inv;
+                    y[1][d0] = (d01 + d23) * inv;
+                    y[2][d0] = (s01 - s23) * inv;
+                    y[3][d0] = (d01 - d23) * inv;
+                } else {
+                    y[0][d0] = s01 + s23;
+                    y[1][d0] = d01 + d23;
+                    y[2][d0] = s01 - s23;
+                    y[3][d0] = d01 - d23;
+                }
 #endif
             }
             uint32_t n1[4] = {0, 0, 0, 0};  // 2-bit: per-token count of the level bit
@@ -947,8 +964,8 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 w[2][j] = (w[2][j] << 1) ^ __float_as_uint(y2); w[3][j] = (w[3][j] << 1) ^ __float_as_uint(y3);
                 if constexpr (BITS == 99)
 #endif
-                if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr0);
-                else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr0);
+                if constexpr (BITS == 3) append_rows_b3(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3, thr_tok[i]);
+                else if constexpr (BITS == 2) append_rows_b2(w[0][j], w[1][j], w[2][j], w[3][j], n1[i], y0, y1, y2, y3, thr_tok[i]);
                 else {
                     const char *ql = reinterpret_cast<const char *>(qlut);
                     append_rows_lut(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3,
@@ -1128,8 +1145,11 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
     const float c2 = va.s2[t & 127];
     const uint32_t c3 = ka.s2flip[t & 15];
     if (t < 2) counter[t] = t == 0 ? 12u : 0u;  // V: the wavefronts' first tickets are their own numbers
+    const bool share_lut = KB == 4 && VB == 4 && va.share_k_lut;  // equal tables: one 32 KB copy serves both tensors
     if constexpr (KB == 4) load_quant_lut<768>(qlut_k, ka.quant_lut);
-    if constexpr (VB == 4) load_quant_lut<768>(qlut_v, va.quant_lut);
+    if constexpr (VB == 4) {
+        if (!share_lut) load_quant_lut<768>(qlut_v, va.quant_lut);
+    }
     auto stage = [&] {
         frag_s[t] = c0;
         if (t < 256) frag_s[768 + t] = c1;
@@ -1138,7 +1158,7 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
         __syncthreads();
     };
     store_v_units<VB, RAGGED, true>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], qlut_v, frag_s, s2_s,
+                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], share_lut ? qlut_k : qlut_v, frag_s, s2_s,
                               (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
     store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
                               wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s,
@@ -2227,7 +2247,7 @@ static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     StoreVArgs va;
     va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
     va.quant_lut = h->quant_lut;
-    va.norm_correction = h->norm_correction; va.tokens = tokens;
+    va.norm_correction = h->norm_correction; va.tokens = tokens; va.share_k_lut = 0;
     va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
     return va;
 }
@@ -2577,7 +2597,8 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
         return rc ? rc : tqk_store(hv, v, n_seqs, tokens, in_dtype, TQ_KIND_V, packed_v, nullptr, nullptr, s);
     }
     const StoreKArgs ka = make_k_args(hk, tokens, bps, n_blocks);
-    const StoreVArgs va = make_v_args(hv, tokens, bps, n_blocks);
+    StoreVArgs va = make_v_args(hv, tokens, bps, n_blocks);
+    va.share_k_lut = hk->bits == 4 && hv->bits == 4 && hk->quant_lut_hash == hv->quant_lut_hash;
     const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
     // one workgroup of 12 wavefronts per CU
     const unsigned wg = 768;
