@@ -28,11 +28,12 @@
 //   half's scales.
 //   Online softmax in base 2 (log2(e) folded into the query scale).  The wavefronts
 //   of a workgroup (up to 16 splits) merge their results in LDS and write one partial.
-// k_attn_combine / k_attn_combine_few: log-sum-exp merge of the workgroups' partials,
-//   then the transpose of the V rotation.  Queries are rotated and scaled inside
-//   k_decode_attn, so a dense step is two launches.
+//   The last workgroup of a group to finish merges the group's partials (log-sum-exp), applies the transpose
+//   of the V rotation and writes the output rows (merge_group): a step is one launch.  Queries are rotated and
+//   scaled inside the kernel.
 // k_score_tile: TurboQuant inner-product estimate, 32x32x16 fp16 MFMA over a
 //   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+#include <atomic>
 #include <mutex>
 #include <cstring>
 #include <type_traits>
@@ -181,7 +182,17 @@ struct AttnArgs {
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
     float *part_o;                // [groups][workgroups per group][4][128]
     float *part_ml;               // [groups][workgroups per group][4][2]  (m in log2 units, l)
-    unsigned long long *skip_slots;  // Sparse V: [workgroup] (query, position) pairs it skipped
+    unsigned long long *skip_slots;  // Sparse V: [workgroup] nonce tag | (query, position) pairs it skipped; 0 after the count
+    // merge of the workgroups' partials by the last workgroup of a group to finish (see merge_group)
+    float *out;                      // [groups * q_group][128]
+    const float *vs1, *vs2;          // V rotation signs (NULL: V rows are stored unrotated)
+    unsigned long long *flags;       // [workgroup] nonce once the workgroup's partial is in memory, 0 after the merge
+    unsigned long long nonce;        // differs from call to call (and from whatever the workspace held before)
+    int poll_slots;                       // Sparse V: the merging workgroups add the slots up themselves
+    unsigned long long *pass_totals;      // Sparse V: [pass] skipped pairs of each four-head pass of this step
+    unsigned long long *skip_count;       // caller's {skipped, total} or NULL
+    unsigned long long total_pairs;
+    int pass;                             // head_off / 4
     int64_t tokens, blocks_per_seq;
     int n_groups, n_splits, tiles_per_split, n_tiles;
     int q_group, head_off;  // query heads per KV head; first of the (up to) four heads this launch works on
@@ -189,6 +200,7 @@ struct AttnArgs {
 };
 
 constexpr int KFMT_TURBO = 0, KFMT_Q8 = 1;
+constexpr unsigned long long SKIP_COUNT_MASK = (1ull << 40) - 1ull;  // count bits of a Sparse-V slot; the rest is a nonce tag
 constexpr int MERGE_FLOATS = 520;  // LDS floats per wavefront for the end-of-kernel merge: out[4][128], m[4], l[4]
 
 // QK over the 32 dim groups: B = this lane's K row (4 dims per group), A = q from block G % 16
@@ -233,6 +245,119 @@ __device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, cons
 template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 1]; };
 
 constexpr float Q8V_PRESCALE = 64.0f;  // keeps weight * scale products out of fp16's subnormals; 65504 / 64 > any scale
+
+// ---- merging the workgroups' partials inside the launch -------------------------------------
+// A group's partials are written by up to n_splits / wavefronts-per-workgroup workgroups that may run on
+// different dies, whose L2 caches are not coherent with each other for ordinary accesses.  Everything the
+// workgroups exchange therefore moves with device-scope atomic loads and stores (they go through to memory),
+// ordered by waiting for the stores to complete: a workgroup stores its partial, waits, raises its flag, waits,
+// and then reads the group's flags; the workgroup that finds every flag raised merges the group (two may, if
+// they finish together: both write the same values).  A flag holds the call's nonce, so what a fresh workspace
+// happens to contain is not mistaken for a raised flag, and the merging workgroup puts the flags back to zero,
+// so a replay of a captured launch (same nonce) starts clean.  No cache-wide write-back or invalidate is
+// involved, which is what made a merge behind device-scope fences cost more than the second launch it saved.
+__device__ __forceinline__ void st_dev(float *p, float v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_dev(unsigned long long *p, unsigned long long v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_dev(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 ld_dev2(const float *p) {  // 8-byte aligned pair
+    const unsigned long long u = ld_dev(reinterpret_cast<const unsigned long long *>(p));
+    return make_float2(__uint_as_float((uint32_t)u), __uint_as_float((uint32_t)(u >> 32)));
+}
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Log-sum-exp merge of a group's n_parts partials, transpose of the V rotation, output rows; one wavefront per
+// query head (the partials come straight from memory: every load of a head is issued before the first is used
+// when there are at most four).
+__device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_parts, int tid, int n_waves) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const float *ml0 = a.part_ml + (int64_t)group * n_parts * 8;
+    const float *po0 = a.part_o + (int64_t)group * n_parts * 512;
+    for (int head = wave; head < 4; head += n_waves) {
+        if (a.head_off + head >= a.q_group) continue;  // a repeated head of a group with fewer than four left
+        const int64_t r_out = (int64_t)group * a.q_group + a.head_off + head;
+        float M = -INFINITY, L = 0.0f, o0 = 0.0f, o1 = 0.0f;
+        if (n_parts <= 4) {
+            float2 ml[4], v[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int pc = p < n_parts ? p : 0;
+                ml[p] = ld_dev2(ml0 + pc * 8 + head * 2);
+                v[p] = ld_dev2(po0 + (int64_t)pc * 512 + head * 128 + 2 * lane);
+                if (p >= n_parts) ml[p].y = 0.0f;
+            }
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                if (ml[p].y > 0.0f) M = fmaxf(M, ml[p].x);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const float w = ml[p].y > 0.0f ? exp2f(ml[p].x - M) : 0.0f;
+                L = fmaf(ml[p].y, w, L);
+                o0 = fmaf(v[p].x, w, o0);
+                o1 = fmaf(v[p].y, w, o1);
+            }
+        } else {
+            for (int p0 = 0; p0 < n_parts; p0 += 64) {  // lane <-> partial: maximum, then weights
+                const int p = p0 + lane;
+                float m = -INFINITY;
+                if (p < n_parts) {
+                    const float2 e = ld_dev2(ml0 + p * 8 + head * 2);
+                    if (e.y > 0.0f) m = e.x;
+                }
+                for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+                M = fmaxf(M, m);
+            }
+            for (int p0 = 0; p0 < n_parts; p0 += 64) {
+                const int p = p0 + lane;
+                float w = 0.0f, l = 0.0f;
+                if (p < n_parts) {
+                    const float2 e = ld_dev2(ml0 + p * 8 + head * 2);
+                    l = e.y;
+                    w = l > 0.0f ? exp2f(e.x - M) : 0.0f;
+                }
+                float lw = l * w;
+                for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
+                L += lw;
+                const int cnt = min(64, n_parts - p0);
+#pragma unroll 4
+                for (int t = 0; t < cnt; ++t) {
+                    const float wt = __shfl(w, t);
+                    const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * 512 + head * 128 + 2 * lane);
+                    o0 = fmaf(v.x, wt, o0);
+                    o1 = fmaf(v.y, wt, o1);
+                }
+            }
+        }
+        const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+        float2 res;
+        if (!a.vs1) {  // V rows were stored unrotated
+            res = make_float2(o0 * invL, o1 * invL);
+        } else {
+            const float2 s1v = *reinterpret_cast<const float2 *>(a.vs1 + 2 * lane);
+            const float2 s2v = *reinterpret_cast<const float2 *>(a.vs2 + 2 * lane);
+            o0 *= invL * s2v.x;
+            o1 *= invL * s2v.y;
+            wht128_wave(o0, o1, lane);
+            res = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
+        }
+        *reinterpret_cast<float2 *>(a.out + r_out * 128 + 2 * lane) = res;
+    }
+}
+
+// sum over the workgroup of one 64-bit value per thread (every thread gets the total); red: one shared word
+__device__ __forceinline__ unsigned long long block_sum(unsigned long long t, unsigned long long *red, int tid) {
+    if (tid == 0) *red = 0ull;
+    __syncthreads();
+    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
+    if ((tid & 63) == 0 && t) atomicAdd(red, t);
+    __syncthreads();
+    return *red;
+}
 
 // SHARE: K and V decode through one table (same width, same centroids); table positions are
 // compile-time constants so that they fold into the LDS instructions' offset fields.
@@ -589,10 +714,10 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) po[i * 128 + 64 * hf + lane] = acc_o[hf][0][i] + acc_o[hf][1][i];
+            for (int i = 0; i < 4; ++i) st_dev(po + i * 128 + 64 * hf + lane, acc_o[hf][0][i] + acc_o[hf][1][i]);
         if (lane < 4) {
-            pml[2 * j] = m_run;
-            pml[2 * j + 1] = l_tot;
+            st_dev(pml + 2 * j, m_run);
+            st_dev(pml + 2 * j + 1, l_tot);
         }
     } else {
         // per wavefront: out[4][128], then m[4], l[4]
@@ -618,7 +743,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
         for (int e = tid; e < 512; e += 64 * n_waves) {
             float sum = 0.0f;
             for (int w = 0; w < n_waves; ++w) sum += merge_s[w * MS + e];
-            po[e] = sum;
+            st_dev(po + e, sum);
         }
         if (tid < 4) {  // lanes 0..3 of wavefront 0 hold heads 0..3
             float L = 0.0f;
@@ -626,8 +751,8 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
                 const float lw = merge_s[w * MS + 516 + j];
                 if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(merge_s[w * MS + 512 + j] - M), L);
             }
-            pml[2 * j] = M;
-            pml[2 * j + 1] = L;
+            st_dev(pml + 2 * j, M);
+            st_dev(pml + 2 * j + 1, L);
         }
     }
     if constexpr (SPARSE) {
@@ -637,168 +762,106 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
         for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
         if (lane == 0 && tot) atomicAdd(&skipped, tot);
         __syncthreads();
-        if (tid == 0) a.skip_slots[blockIdx.x] = skipped;
+        if (tid == 0) st_dev(a.skip_slots + blockIdx.x, (a.nonce & ~SKIP_COUNT_MASK) | (unsigned long long)skipped);
+    }
+
+    // ---- the group's last workgroup merges the partials and writes the output rows -----------------
+    const int n_parts = wgs_per_group;
+    wait_stores();  // this lane's part of the partial (and the skip slot) is in memory
+    __syncthreads();
+    if (n_parts > 1) {
+        if (tid == 0) {
+            st_dev(a.flags + blockIdx.x, a.nonce);
+            wait_stores();
+        }
+        __syncthreads();  // the flag is up before anybody reads the group's flags
+        int all_up = 1;
+        for (int p = tid; p < n_parts; p += (int)blockDim.x) all_up &= ld_dev(a.flags + (int64_t)group * n_parts + p) == a.nonce;
+        if (!__syncthreads_and(all_up)) return;
+    }
+    // Sparse V: every workgroup's slot carries its count (40 bits: at most 4 heads x 2^31 positions) under 24 bits
+    // of the nonce.  A merging workgroup reads all slots of the launch now, so that the trip to memory overlaps
+    // the merge; the one that finds them all tagged (the merging workgroup of the group that finishes last does)
+    // writes the step's total.  Launches with more workgroups than one can poll are added up by a launch of their
+    // own (poll_slots == 0).
+    int all_in = 1;
+    unsigned long long counted = 0ull;
+    if constexpr (SPARSE) {
+        if (a.poll_slots) {
+            const unsigned long long tag = a.nonce & ~SKIP_COUNT_MASK;
+            for (int g = tid; g < (int)gridDim.x; g += (int)blockDim.x) {
+                const unsigned long long word = ld_dev(a.skip_slots + g);
+                all_in &= (word & ~SKIP_COUNT_MASK) == tag;
+                counted += word & SKIP_COUNT_MASK;
+            }
+        }
+    }
+    merge_group(a, group, n_parts, tid, n_waves);
+    if (n_parts > 1) {
+        for (int p = tid; p < n_parts; p += (int)blockDim.x) st_dev(a.flags + (int64_t)group * n_parts + p, 0ull);
+    }
+    if constexpr (SPARSE) {
+        if (a.poll_slots) {
+            if (!__syncthreads_and(all_in)) return;
+            __shared__ unsigned long long red;
+            const unsigned long long pass_total = block_sum(counted, &red, tid);
+            for (int g = tid; g < (int)gridDim.x; g += (int)blockDim.x) st_dev(a.skip_slots + g, 0ull);
+            if (tid == 0) {
+                // this pass's total is kept apart so that writing the step's total twice (two groups finishing
+                // together) gives the same value both times
+                st_dev(a.pass_totals + a.pass, pass_total);
+                unsigned long long sum = pass_total;
+                for (int k = 0; k < a.pass; ++k) sum += ld_dev(a.pass_totals + k);
+                a.skip_count[0] = sum;
+                a.skip_count[1] = a.total_pairs;
+            }
+        }
     }
 }
 
-// Sparse-V bookkeeping, done by the first workgroup of the merge kernel: skip[0] = the sum of the decode
-// workgroups' slots (none for a dense step), skip[1] = all (query, position) pairs.
-struct SkipArgs {
-    const unsigned long long *slots;
-    int n_slots;
-    unsigned long long *skip;  // NULL: no bookkeeping asked for
-    unsigned long long total_pairs;
-    int accumulate;            // a later launch of the same step: add to skip[0] instead of setting it
-};
-__device__ __forceinline__ void sum_skip_slots(const SkipArgs &k) {
-    if (!k.skip || blockIdx.x != 0) return;
-    __shared__ unsigned long long acc;
-    if (threadIdx.x == 0) acc = 0ull;
-    __syncthreads();
+// Sparse-V bookkeeping for launches with more groups than one workgroup polls (and for a caller that asks for the
+// counts of a dense step): skip[0] = the sum of the decode workgroups' slots (plus the earlier passes'), skip[1] =
+// all (query, position) pairs.  One workgroup.
+__global__ __launch_bounds__(1024) void k_skip_sum(const unsigned long long *slots, int n_slots, unsigned long long *skip,
+                                                   unsigned long long total_pairs, int accumulate) {
+    __shared__ unsigned long long red;
     unsigned long long t = 0ull;
-    for (int i = (int)threadIdx.x; i < k.n_slots; i += (int)blockDim.x) t += k.slots[i];
-    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
-    if ((threadIdx.x & 63) == 0 && t) atomicAdd(&acc, t);
-    __syncthreads();
+    for (int i = (int)threadIdx.x; i < n_slots; i += (int)blockDim.x) t += slots[i] & SKIP_COUNT_MASK;
+    const unsigned long long sum = block_sum(t, &red, (int)threadIdx.x);
     if (threadIdx.x == 0) {
-        k.skip[0] = (k.accumulate ? k.skip[0] : 0ull) + acc;
-        k.skip[1] = k.total_pairs;
+        skip[0] = (accumulate ? skip[0] : 0ull) + sum;
+        skip[1] = total_pairs;
     }
 }
 
-// merge split partials, un-rotate with the V rotation's transpose; one workgroup of NW (4 or 16)
-// wavefronts per query head.  Every wavefront fetches (m, l) of all splits (lane s <-> split s,
-// 64 per pass) so the weights are known after one round trip, streams the partial outputs of
-// its share of the splits with independent loads, and wavefront 0 adds the shares.
-template <int NW>
-__global__ __launch_bounds__(64 * NW) void k_attn_combine(const float *part_o, const float *part_ml, float *out,
-                                                          int64_t n_rows, int n_splits, const float *s1, const float *s2,
-                                                          SkipArgs sk, int q_group, int head_off) {
-    sum_skip_slots(sk);
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int64_t r = blockIdx.x;  // row = group*4 + head
-    const int64_t group = r >> 2;
-    const int head = (int)(r & 3);
-    if (head_off + head >= q_group) return;  // a repeated head of a group with fewer than four left
-    const int64_t r_out = group * q_group + head_off + head;
-    const float *ml = part_ml + (group * n_splits * 4 + head) * 2;   // + s*8
-    const float *po = part_o + (group * n_splits * 4 + head) * 128;  // + s*512
-    float M = -INFINITY;
-    for (int s0 = 0; s0 < n_splits; s0 += 64) {
-        const int s = s0 + lane;
-        float m = -INFINITY;
-        if (s < n_splits && ml[s * 8 + 1] > 0.0f) m = ml[s * 8];
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-        M = fmaxf(M, m);
-    }
-    float L = 0.0f, o0 = 0.0f, o1 = 0.0f;
-    for (int s0 = 0; s0 < n_splits; s0 += 64) {
-        const int s = s0 + lane;
-        float w = 0.0f, l = 0.0f;
-        if (s < n_splits) {
-            l = ml[s * 8 + 1];
-            w = l > 0.0f ? exp2f(ml[s * 8] - M) : 0.0f;
-        }
-        float lw = l * w;
-        for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
-        L += lw;
-        const int cnt = min(64, n_splits - s0);
-#pragma unroll 8
-        for (int t = wv; t < cnt; t += NW) {
-            const float wt = __shfl(w, t);
-            const float2 v = *reinterpret_cast<const float2 *>(po + (int64_t)(s0 + t) * 512 + 2 * lane);
-            o0 = fmaf(v.x, wt, o0);
-            o1 = fmaf(v.y, wt, o1);
-        }
-    }
-    __shared__ float red[NW][130];
-    red[wv][2 * lane] = o0;
-    red[wv][2 * lane + 1] = o1;
-    __syncthreads();
-    if (wv != 0) return;
-    o0 = 0.0f;
-    o1 = 0.0f;
-#pragma unroll
-    for (int q = 0; q < NW; q += 4) {
-        o0 += (red[q][2 * lane] + red[q + 1][2 * lane]) + (red[q + 2][2 * lane] + red[q + 3][2 * lane]);
-        o1 += (red[q][2 * lane + 1] + red[q + 1][2 * lane + 1]) + (red[q + 2][2 * lane + 1] + red[q + 3][2 * lane + 1]);
-    }
-    const float invL = L > 0.0f ? 1.0f / L : 0.0f;
-    if (!s1) {  // V rows were stored unrotated
-        out[r_out * 128 + 2 * lane] = o0 * invL;
-        out[r_out * 128 + 2 * lane + 1] = o1 * invL;
-        return;
-    }
-    o0 *= invL * s2[2 * lane];
-    o1 *= invL * s2[2 * lane + 1];
-    wht128_wave(o0, o1, lane);
-    out[r_out * 128 + 2 * lane] = o0 * (s1[2 * lane] * RSQRT128);
-    out[r_out * 128 + 2 * lane + 1] = o1 * (s1[2 * lane + 1] * RSQRT128);
-}
-
-// the same merge for at most four partials per row: one wavefront per row, every load issued before
-// anything is waited for (one trip to memory instead of three)
-__global__ __launch_bounds__(256) void k_attn_combine_few(const float *part_o, const float *part_ml, float *out, int64_t n_rows,
-                                                          int n_parts, const float *s1, const float *s2, SkipArgs sk, int q_group,
-                                                          int head_off) {
-    sum_skip_slots(sk);
-    const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row = group*4 + head
-    if (r >= n_rows) return;
-    const int64_t group = r >> 2;
-    const int head = (int)(r & 3);
-    if (head_off + head >= q_group) return;
-    const int64_t r_out = group * q_group + head_off + head;
-    const float *ml = part_ml + (group * n_parts * 4 + head) * 2;   // + p*8
-    const float *po = part_o + (group * n_parts * 4 + head) * 128;  // + p*512
-    float m[4], l[4];
-    float2 v[4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int pc = p < n_parts ? p : 0;
-        m[p] = ml[pc * 8];
-        l[p] = p < n_parts ? ml[pc * 8 + 1] : 0.0f;
-        v[p] = *reinterpret_cast<const float2 *>(po + (int64_t)pc * 512 + 2 * lane);
-    }
-    const float2 s1v = s1 ? *reinterpret_cast<const float2 *>(s1 + 2 * lane) : make_float2(1.0f, 1.0f);
-    const float2 s2v = s1 ? *reinterpret_cast<const float2 *>(s2 + 2 * lane) : make_float2(1.0f, 1.0f);
-    float M = -INFINITY;
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-        if (l[p] > 0.0f) M = fmaxf(M, m[p]);
-    float L = 0.0f, o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const float w = l[p] > 0.0f ? exp2f(m[p] - M) : 0.0f;
-        L = fmaf(l[p], w, L);
-        o0 = fmaf(v[p].x, w, o0);
-        o1 = fmaf(v[p].y, w, o1);
-    }
-    const float invL = L > 0.0f ? 1.0f / L : 0.0f;
-    if (!s1) {  // V rows were stored unrotated
-        *reinterpret_cast<float2 *>(out + r_out * 128 + 2 * lane) = make_float2(o0 * invL, o1 * invL);
-        return;
-    }
-    o0 *= invL * s2v.x;
-    o1 *= invL * s2v.y;
-    wht128_wave(o0, o1, lane);
-    *reinterpret_cast<float2 *>(out + r_out * 128 + 2 * lane) = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
-}
+constexpr int MAX_POLLED_SLOTS = 4096;  // workgroups of a launch whose Sparse-V slots the merging workgroups add up themselves
+constexpr int MAX_PASSES = 64;           // four-head passes of one step (query heads per KV head <= 256)
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
+// a value that no earlier call of this process used and that leftovers in a fresh workspace are unlikely to
+// equal (splitmix64 of a process-wide counter; never 0, which is what a lowered flag holds)
+std::atomic<unsigned long long> g_attn_seq{0};
+unsigned long long next_nonce() {
+    unsigned long long z = (g_attn_seq.fetch_add(1, std::memory_order_relaxed) + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (z >> 40) ? z : z | (1ull << 63);  // the upper 24 bits tag the Sparse-V words and must not be zero
+}
+
 struct WsLayout {
-    int64_t qrot, part_o, part_ml, skip_slots, total;
+    int64_t part_o, part_ml, skip_slots, flags, pass_totals, total;
 };
 WsLayout ws_layout(const tq_attn_params *p) {
-    const int64_t rows = (int64_t)p->batch * p->n_q_heads;
     const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
     WsLayout w;
-    w.qrot = 0;
-    w.part_o = align256(rows * 128 * 2);
+    w.part_o = 0;
     w.part_ml = w.part_o + align256(groups * p->n_splits * 4 * 128 * 4);
     w.skip_slots = w.part_ml + align256(groups * p->n_splits * 4 * 2 * 4);
-    w.total = w.skip_slots + align256(groups * p->n_splits * 8);
+    w.flags = w.skip_slots + align256(groups * p->n_splits * 8);
+    w.pass_totals = w.flags + align256(groups * p->n_splits * 8);
+    w.total = w.pass_totals + align256(MAX_PASSES * 8);
     return w;
 }
 
@@ -875,8 +938,22 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     // ceil(G / 4) passes over the same K/V, each with its own merge launch; a last pass with fewer than four
     // heads repeats the group's last head and does not write the repeats.
     a.q_group = p->n_q_heads / p->n_kv_heads;
-    const int64_t rows4 = (int64_t)groups * 4;
+    if ((a.q_group + 3) / 4 > MAX_PASSES) {
+        tq_set_error("tq_decode_attention: %d query heads per KV head (at most %d)", a.q_group, 4 * MAX_PASSES);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    a.out = out;
+    a.vs1 = vs1;
+    a.vs2 = vs2;
+    a.flags = reinterpret_cast<unsigned long long *>((char *)ws + w.flags);
+    a.poll_slots = sparse && grid <= (unsigned)MAX_POLLED_SLOTS;
+    a.pass_totals = reinterpret_cast<unsigned long long *>((char *)ws + w.pass_totals);
+    a.skip_count = skip_count;
+    a.total_pairs = total_pairs;
+    (void)n_parts;
     for (a.head_off = 0; a.head_off < a.q_group; a.head_off += 4) {
+        a.pass = a.head_off / 4;
+        a.nonce = next_nonce();
 #define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, merge_bytes, s>>>(a)
 #define TQ_ATTN(KF, KB, VB)                         \
     if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
@@ -912,22 +989,12 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 #undef TQ_ATTN_ONE
     rc = tq_check_launch("decode_attn");
     if (rc) return rc;
-    // many partials: sixteen wavefronts share a row's
-    SkipArgs sk;
-    sk.slots = a.skip_slots;
-    sk.n_slots = sparse ? (int)grid : 0;
-    sk.skip = skip_count;
-    sk.total_pairs = total_pairs;
-    sk.accumulate = a.head_off > 0;
-    if (n_parts >= 64)
-        k_attn_combine<16><<<(unsigned)rows4, 1024, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group, a.head_off);
-    else if (n_parts > 4)
-        k_attn_combine<4><<<(unsigned)rows4, 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group, a.head_off);
-    else
-        k_attn_combine_few<<<(unsigned)((rows4 + 3) / 4), 256, 0, s>>>(part_o, part_ml, out, rows4, n_parts, vs1, vs2, sk, a.q_group,
-                                                                      a.head_off);
-    rc = tq_check_launch("attn_combine");
-    if (rc) return rc;
+    if (skip_count && !a.poll_slots) {
+        // more groups than the finishing workgroups poll (or a dense step whose caller wants the counts)
+        k_skip_sum<<<1, 1024, 0, s>>>(a.skip_slots, sparse ? (int)grid : 0, skip_count, total_pairs, a.head_off > 0);
+        rc = tq_check_launch("skip_sum");
+        if (rc) return rc;
+    }
     }
     return TQ_OK;
 }
