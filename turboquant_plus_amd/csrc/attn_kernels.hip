@@ -55,14 +55,26 @@ template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t 
     return pair_lut_offset<BITS>(w, p);
 }
 
+// Measurement builds only (make EXTRA=-DTQ_PAIRTAB3=1): 3-bit codes decode through a pair table with one copy
+// per LDS bank (entry e of lane l at dword 64 e + l: no bank conflicts, two 4-byte reads per four values)
+// instead of the 4096-entry quad table (one 8-byte read per four values, about 1.6 conflicts per read).
+#ifndef TQ_PAIRTAB3
+#define TQ_PAIRTAB3 0
+#endif
 // bytes of the decode table of a codebook: quad entries for BITS <= 3, pair entries for 4
 __host__ __device__ constexpr int lut_bytes(int bits) {
+    if (TQ_PAIRTAB3 && bits == 3) return 64 * 64 * 4;
     return bits == 8 ? 0 : bits <= 3 ? 8 << (4 * bits) : 4 << (2 * bits);  // 8: int8 rows, no table
 }
 
 // the four values of quad Q (pairs 2Q, 2Q+1) of a row as an MFMA operand
 template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_t (&w)[4 * BITS], const char *lut, int Q) {
-    if constexpr (BITS <= 3) {
+    if constexpr (TQ_PAIRTAB3 && BITS == 3) {
+        // lut already points at this lane's bank (+ 4 * lane); a pair code selects the 256-byte row
+        const uint32_t o0 = pair_lut_offset<BITS>(w, 2 * Q) << 6, o1 = pair_lut_offset<BITS>(w, 2 * Q + 1) << 6;
+        const uint2 u = make_uint2(*reinterpret_cast<const uint32_t *>(lut + o0), *reinterpret_cast<const uint32_t *>(lut + o1));
+        return __builtin_bit_cast(half4_t, u);
+    } else if constexpr (BITS <= 3) {
         return __builtin_bit_cast(half4_t, *reinterpret_cast<const uint2 *>(lut + quad_lut_offset<BITS>(w, Q)));
     } else {
         const uint2 u = make_uint2(*reinterpret_cast<const uint32_t *>(lut + pair_lut_offset<BITS>(w, 2 * Q)),
@@ -76,7 +88,11 @@ template <int BITS> __device__ __forceinline__ half4_t quad_values(const uint32_
 template <int BITS>
 __device__ __forceinline__ void build_lut(char *dst, const uint32_t *pair_lut, uint32_t mine, int tid, int n_waves) {
     constexpr int NP = 1 << (2 * BITS);
-    if constexpr (BITS == 3) {
+    if constexpr (TQ_PAIRTAB3 && BITS == 3) {
+        uint32_t *t = reinterpret_cast<uint32_t *>(dst);
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        for (int e = wave; e < 64; e += n_waves) t[e * 64 + lane] = (uint32_t)__builtin_amdgcn_readlane((int)mine, e);
+    } else if constexpr (BITS == 3) {
         // lane l holds pair entry l; wavefront w writes the rows hi = w, w + n_waves, ..
         uint2 *t = reinterpret_cast<uint2 *>(dst);
         const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -403,8 +419,8 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
 
     const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
     const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
-    const char *klut_b = klut_s;
-    const char *vlut_b = vlut_s;
+    const char *klut_b = klut_s + (TQ_PAIRTAB3 && KFMT == KFMT_TURBO && KBITS == 3 ? 4 * lane : 0);
+    const char *vlut_b = vlut_s + (TQ_PAIRTAB3 && VBITS == 3 ? 4 * lane : 0);
 
     // The first tile's rows are requested before anything else, so that the query rotation and
     // the table build overlap the first trip to memory.  Afterwards rows are fetched one tile
