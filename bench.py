@@ -114,14 +114,14 @@ def measured_peaks_leg(torch, tqa, steps, warmup):
         b.zero_()
     out = {"bytes_per_launch": n}
     reps, warm = max(20, steps // 10), max(10, warmup // 10)
-    for mode in ("read", "write", "copy"):
+    for mode in ("read", "write", "copy", "read_nt", "write_nt", "copy_nt"):   # _nt: non-temporal hint on every access
         best = 0.0
         for chunked in (False, True):   # lanes striding over the whole buffer, or one contiguous slice per workgroup
             def step(i):
                 src, dst = bufs[2 * (i % 2)], bufs[2 * (i % 2) + 1]
-                probes.probe_stream(mode, None if mode == "write" else src, None if mode == "read" else dst, chunked)
+                probes.probe_stream(mode, None if mode.startswith("write") else src, None if mode.startswith("read") else dst, chunked)
             _, ev_ms = time_steps(torch, step, reps, warm)
-            moved = n * (2 if mode == "copy" else 1)
+            moved = n * (2 if mode.startswith("copy") else 1)
             best = max(best, moved / (ev_ms * 1e-3) / 1e9)
         out[f"hbm_{mode}_gbs"] = best   # the better of the two access orders
     del bufs

@@ -10,8 +10,9 @@ namespace {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-// mode 0: read, 1: write, 2: copy; 16 bytes per lane and step.  CHUNKED: every workgroup a contiguous slice,
+// mode 0: read, 1: write, 2: copy, 3 / 4 / 5: write / read / copy with the non-temporal hint; 16 bytes per lane and step.  CHUNKED: every workgroup a contiguous slice,
 // else all lanes of the grid stride over the buffer.
 template <int MODE, bool CHUNKED>
 __global__ __launch_bounds__(512) void k_probe_stream(const uint4 *src, uint4 *dst, int64_t n16) {
@@ -27,12 +28,20 @@ __global__ __launch_bounds__(512) void k_probe_stream(const uint4 *src, uint4 *d
             acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
         } else if constexpr (MODE == 1) {
             dst[i] = fill;
-        } else {
+        } else if constexpr (MODE == 2) {
             dst[i] = src[i];
+        } else if constexpr (MODE == 3) {
+            __builtin_nontemporal_store(u32x4_t{fill.x, fill.y, fill.z, fill.w}, reinterpret_cast<u32x4_t *>(dst + i));
+        } else if constexpr (MODE == 4) {
+            const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(src + i));
+            acc.x ^= v[0]; acc.y ^= v[1]; acc.z ^= v[2]; acc.w ^= v[3];
+        } else {
+            const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(src + i));
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t *>(dst + i));
         }
     }
     // keeps the reads alive; the condition does not hold for any data a caller would pass
-    if constexpr (MODE == 0) {
+    if constexpr (MODE == 0 || MODE == 4) {
         if ((acc.x & acc.y & acc.z & acc.w) == 0xFFFFFFFFu && dst) dst[0] = acc;
     }
 }
@@ -69,21 +78,23 @@ constexpr int PROBE_MFMA_WGS = 2048;  // 8 workgroups of 4 wavefronts per CU
 
 extern "C" int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream) {
     hipStream_t s = (hipStream_t)stream;
-    if (mode < 0 || mode > 2 || bytes < 16 || (bytes & 15) || (mode != 1 && !src) || (mode != 0 && !dst)) return TQ_PROBE_ERR_ARG;
+    const bool reads = mode == 0 || mode == 2 || mode == 4 || mode == 5, writes = mode == 1 || mode == 2 || mode == 3 || mode == 5;
+    if (mode < 0 || mode > 5 || bytes < 16 || (bytes & 15) || (reads && !src) || (writes && !dst)) return TQ_PROBE_ERR_ARG;
     if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) return TQ_PROBE_ERR_ARG;
     const int64_t n16 = bytes / 16;
     const unsigned grid = 256 * 4;
-    const uint4 *s4 = (const uint4 *)src;
-    uint4 *d4 = (uint4 *)dst;
-    if (chunked) {
-        if (mode == 0) k_probe_stream<0, true><<<grid, 512, 0, s>>>(s4, d4, n16);
-        else if (mode == 1) k_probe_stream<1, true><<<grid, 512, 0, s>>>(nullptr, d4, n16);
-        else k_probe_stream<2, true><<<grid, 512, 0, s>>>(s4, d4, n16);
-    } else {
-        if (mode == 0) k_probe_stream<0, false><<<grid, 512, 0, s>>>(s4, d4, n16);
-        else if (mode == 1) k_probe_stream<1, false><<<grid, 512, 0, s>>>(nullptr, d4, n16);
-        else k_probe_stream<2, false><<<grid, 512, 0, s>>>(s4, d4, n16);
+    const uint4 *s4 = reads ? (const uint4 *)src : nullptr;
+    uint4 *d4 = writes ? (uint4 *)dst : nullptr;
+#define TQ_PROBE_MODE(M)                                                              \
+    case M:                                                                           \
+        if (chunked) k_probe_stream<M, true><<<grid, 512, 0, s>>>(s4, d4, n16);       \
+        else k_probe_stream<M, false><<<grid, 512, 0, s>>>(s4, d4, n16);              \
+        break
+    switch (mode) {
+        TQ_PROBE_MODE(0); TQ_PROBE_MODE(1); TQ_PROBE_MODE(2); TQ_PROBE_MODE(3); TQ_PROBE_MODE(4);
+        default: TQ_PROBE_MODE(5);
     }
+#undef TQ_PROBE_MODE
     return hipGetLastError() == hipSuccess ? 0 : TQ_PROBE_ERR_HIP;
 }
 

@@ -16,7 +16,8 @@ extern "C" {
 #define TQ_PROBE_MAX_ITERS 1000000
 
 /* One launch that reads `bytes` from src (mode 0; dst may be NULL), writes `bytes` to dst (mode 1; src
- * ignored) or copies src to dst (mode 2).  chunked = 0: the lanes of the whole grid stride over the buffer;
+ * ignored) or copies src to dst (mode 2); modes 3, 4, 5 are write, read and copy with the non-temporal hint on
+ * every access.  chunked = 0: the lanes of the whole grid stride over the buffer;
  * 1: every workgroup takes one contiguous slice (reads and writes favour different orders on this part).
  * bytes: a multiple of 16; pointers 16-byte aligned.  stream: hipStream_t.  Returns 0 or a negative code. */
 int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream);

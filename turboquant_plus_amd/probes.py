@@ -27,10 +27,11 @@ def lib():
 
 
 def probe_stream(mode: str, src, dst, chunked: bool = False):
-    """One launch of the streaming probe: "read" src, "write" dst or "copy" src to dst (uint8 device
+    """One launch of the streaming probe: "read" src, "write" dst or "copy" src to dst, or the same with the
+    non-temporal hint ("read_nt", "write_nt", "copy_nt") (uint8 device
     tensors of equal size, a multiple of 16 bytes); chunked gives every workgroup one contiguous slice
     instead of striding all lanes over the buffer.  The caller times it."""
-    code = {"read": 0, "write": 1, "copy": 2}[mode]
+    code = {"read": 0, "write": 1, "copy": 2, "write_nt": 3, "read_nt": 4, "copy_nt": 5}[mode]
     ref = dst if src is None else src
     nbytes = 0 if ref is None else ref.numel()
     rc = lib().tq_probe_stream(code, int(chunked), None if src is None else L.ptr(src),
