@@ -210,6 +210,12 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
     us = ev_ms * 1e3
     gbs = algo / (us * 1e-6) / 1e9
 
+    # the same cache under eight query heads per KV head (64 query heads): one pass of eight heads over the K/V
+    g8 = torch.Generator(device="cuda").manual_seed(301)
+    q64 = torch.randn((B, 2 * Hq, D), generator=g8, device="cuda").to(torch.float16)
+    attn8 = tqa.DecodeAttention(kc, vc, B, 2 * Hq, Hkv, N)
+    _, ev8_ms = time_steps(torch, lambda i: attn8(q64, sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
+
     # a whole serving step: append this step's K and V token of every sequence (the last position of the
     # cache is rewritten each time), then attention; launched one by one and replayed from one HIP graph
     g = torch.Generator(device="cuda").manual_seed(77)
@@ -241,6 +247,9 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
                      "algorithmic_bytes_per_step": algo,
                      "kernel": "k_decode_attn<turbo3,turbo3> (+ k_attn_combine in the step time)"},
         "buffer_sets": n_sets,
+        "gqa8": {"workload": "the same cache, 64 query heads on 8 KV heads (eight heads per pass over K/V)",
+                 "us_per_step": ev8_ms * 1e3, "n_splits": attn8.params.n_splits,
+                 "frac": algo / (ev8_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "serving_step": {"workload": "tq_append_kv of one token per sequence + decode attention",
                          "us_per_step": serve_ms * 1e3, "us_per_step_hip_graph": graph_ms * 1e3 / n_sets},
     }

@@ -228,7 +228,8 @@ int tq_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, in
 
 typedef struct tq_attn_params {
     int32_t batch, n_q_heads, n_kv_heads;  /* GQA group = n_q_heads / n_kv_heads; the kernels take */
-                                           /* four heads of a group per pass over K/V (4 is free) */
+                                           /* four heads of a group per pass over K/V, eight when  */
+                                           /* the group has more than four                          */
     int64_t tokens;                        /* context length per sequence                    */
     int64_t capacity;                      /* tokens per sequence the K/V buffers are laid   */
                                            /* out for (tq_append caches); 0 = tokens         */
@@ -240,7 +241,9 @@ typedef struct tq_attn_params {
     float sparse_v_tau;                    /* 0 = dense; skip V rows with weight < tau       */
 } tq_attn_params;
 
-/* Bytes of workspace tq_decode_attention needs (split partials). */
+/* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four
+ * query heads) per workgroup, plus flags and Sparse-V slots.  The workspace may hold anything on entry; calls
+ * that share one workspace must not overlap in time. */
 int64_t tq_attn_workspace_bytes(const tq_attn_params *p);
 
 /* softmax(scale * q k^T) v over packed K/V (tests/test_kv_cache.py:73-89,128-131
@@ -263,8 +266,8 @@ int tq_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn_
  * Same arguments, kernels and results as tq_decode_attention; the split partials go to a workspace of
  * TQ_STATIC_WORKSPACE_BYTES that is built into the library's device code (every GPU the library runs on
  * holds one copy until the process ends), so the call allocates nothing.  Parameter sets whose
- * tq_attn_workspace_bytes() exceeds that size (about batch * n_kv_heads * n_splits > 7900) are rejected with
- * TQ_ERR_UNSUPPORTED.  All calls on one GPU share the one workspace: calls that overlap in time on the same
+ * tq_attn_workspace_bytes() exceeds that size (about 8000 workgroups: batch * n_kv_heads * n_splits / 16 of them
+ * when n_splits is a multiple of 16) are rejected with TQ_ERR_UNSUPPORTED.  All calls on one GPU share the one workspace: calls that overlap in time on the same
  * GPU (different streams or threads) race; order them.  The workspace's address is looked up once per
  * device, in tq_create or in the first call on that device. */
 #define TQ_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)

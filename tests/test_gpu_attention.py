@@ -320,10 +320,11 @@ def test_decode_attention_rejects_ragged_group():
         tqa.DecodeAttention(kc, vc, 1, 7, 2, 128)
 
 
-@pytest.mark.parametrize("G,n_splits", [(1, 3), (2, 16), (3, 1), (5, 3), (7, 16), (8, 4), (12, 64)])
+@pytest.mark.parametrize("G,n_splits", [(1, 3), (2, 16), (3, 1), (5, 3), (7, 16), (8, 4), (8, 32), (12, 64), (16, 8), (17, 2)])
 def test_decode_attention_other_group_sizes(G, n_splits):
-    """Query-head groups other than four: passes of four heads over the same K/V, short last pass included,
-    with a logit bias per (head, position) and the Sparse V count summed over the passes."""
+    """Query-head groups other than four: up to four heads take one pass of four over the K/V, more take passes of
+    eight (two sets of four against the same dequantised rows), short last pass included, with a logit bias per
+    (head, position) and the Sparse V count summed over the passes."""
     B, Hkv, N = 2, 3, 1500
     Hq = G * Hkv
     k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=900 + G)
@@ -335,13 +336,19 @@ def test_decode_attention_other_group_sizes(G, n_splits):
     out = np_(attn(q, kp, vp, bias=bias_d)).copy()
     ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), bias=bias)
     assert_close(out, ref)
-    # every head of a group against the same head served alone (G = 1 layout, same K/V): bitwise when the split
-    # count is the same, since a head's arithmetic does not depend on which row of the four it sits in
+    # every head of a group against the same head served alone (G = 1 layout, same K/V): a head's arithmetic does
+    # not depend on which row of the MFMA block it sits in, so the results are bitwise equal when the splits are
+    # merged in the same order (groups of up to four heads: workgroups of up to 16 wavefronts, as for one head);
+    # groups of more than four heads run eight heads per pass in workgroups of up to 8 wavefronts, which merges
+    # 16 or more splits in another order
     for h in (0, G - 1):
         sel = [kv * G + h for kv in range(Hkv)]
         one = tqa.DecodeAttention(kc, vc, B, Hkv, Hkv, N, n_splits=n_splits)
         got = np_(one(np.ascontiguousarray(q[:, sel]), kp, vp, bias=L.torch().from_numpy(np.ascontiguousarray(bias[:, sel])).cuda()))
-        assert np.array_equal(got, out[:, sel])
+        if G <= 4 or n_splits < 16:
+            assert np.array_equal(got, out[:, sel])
+        else:
+            np.testing.assert_allclose(got, out[:, sel], rtol=0, atol=2e-6 * np.abs(got).max())
     tau = 1e-3
     sparse = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
     out_s = np_(sparse(q, kp, vp, bias=bias_d)).copy()
@@ -408,3 +415,31 @@ def test_decode_attention_every_format_pair(kfmt, vfmt):
         assert_close(out, ref)
         if tau:
             assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
+
+
+@pytest.mark.parametrize("kfmt,vfmt", [("turbo3", "turbo3"), ("turbo4", "turbo2"), ("q8_0", "turbo2"), ("q8_0", "q8_0"), ("turbo3", "q8_0"),
+                                       ("turbo2", "turbo4")])
+def test_decode_attention_eight_heads_per_kv_head(kfmt, vfmt):
+    """GQA groups of eight (one pass of two sets of four heads over the same K/V rows) for the table and the int8
+    variants, dense and Sparse V with a bias, ragged context, splits that do and do not fill a workgroup."""
+    B, Hkv, G, N = 2, 2, 8, 2048 + 100
+    Hq = G * Hkv
+    rng = np.random.default_rng(FORMATS.index(kfmt) * 7 + FORMATS.index(vfmt))
+    k = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, D)).astype(np.float16)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = (0.7 * rng.standard_normal((B, Hq, N))).astype(np.float32)
+    bias_d = L.torch().from_numpy(bias).cuda()
+    kc = tqa.TurboCodec(int(kfmt[-1]), seed=42) if kfmt != "q8_0" else None
+    vc = tqa.TurboCodec(int(vfmt[-1]), seed=542) if vfmt != "q8_0" else None
+    kp = kc.store(k, kind="k") if kc else tqa.q8_0_store(k)[0]
+    vp = vc.store(v, kind="v") if vc else tqa.q8_0_store(v, kind="v")[0]
+    for n_splits, tau in ((8, 0.0), (24, 1e-3), (3, 1e-3)):
+        attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+        out = np_(attn(q, kp, vp, bias=bias_d))
+        ref, skip_o, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau,
+                                             bias=bias, k_q8=None if kc else kp, v_q8=None if vc else vp)
+        assert_close(out, ref)
+        if tau:
+            assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
+            assert int(attn.skip.cpu()[1]) == B * Hq * N

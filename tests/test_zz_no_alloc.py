@@ -70,7 +70,8 @@ def test_static_workspace_rejects_what_does_not_fit():
     kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
     tt = L.torch()
     B, Hq, Hkv, N = 64, 32, 8, 64 * 64
-    params = L.TQAttnParams(batch=B, n_q_heads=Hq, n_kv_heads=Hkv, tokens=N, capacity=0, n_splits=64,
+    # an odd split count: one wavefront per workgroup, so every split is a partial of its own (512 groups x 63 x 2 KB)
+    params = L.TQAttnParams(batch=B, n_q_heads=Hq, n_kv_heads=Hkv, tokens=N, capacity=0, n_splits=63,
                             k_format=L.KFMT_TURBO, v_format=L.KFMT_TURBO, scale=0.1, sparse_v_tau=0.0)
     assert L.lib().tq_attn_workspace_bytes(C.byref(params)) > 16 * 1024 * 1024
     dummy = tt.zeros(4096, dtype=tt.uint8, device="cuda")      # never read: the size check comes first

@@ -220,38 +220,62 @@ constexpr unsigned long long SKIP_COUNT_MASK = (1ull << 40) - 1ull;  // count bi
 constexpr int MERGE_FLOATS = 520;  // LDS floats per wavefront for the end-of-kernel merge: out[4][128], m[4], l[4]
 
 // QK over the 32 dim groups: B = this lane's K row (4 dims per group), A = q from block G % 16
-template <int BITS, int... G>
+// (HG sets of four query heads share every dequantised operand: one table look-up, HG products)
+template <int BITS, int HG, int... G>
 __device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const uint32_t (&kw)[4 * BITS],
-                                         const char *lut, const half4_t (&qa)[2], float4_t (&acc)[4]) {
-    ((acc[G & 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], quad_values<BITS>(kw, lut, G), acc[G & 3])), ...);
+                                         const char *lut, const half4_t (&qa)[HG][2], float4_t (&acc)[HG][4]) {
+    (([&] {
+         const half4_t kv = quad_values<BITS>(kw, lut, G);
+#pragma unroll
+         for (int hg = 0; hg < HG; ++hg) acc[hg][G & 3] = mfma4_bcast<(G & 15)>(qa[hg][G >> 4], kv, acc[hg][G & 3]);
+     }()),
+     ...);
 }
 
 // q8_0-style K: one accumulator per 32-value block (dim groups 8*blk .. 8*blk+7), scaled afterwards
-template <int... G>
+template <int HG, int... G>
 __device__ __forceinline__ void qk_q8(std::integer_sequence<int, G...>, const uint32_t (&kw)[32],
-                                      const half4_t (&qa)[2], float4_t (&acc)[4]) {
+                                      const half4_t (&qa)[HG][2], float4_t (&acc)[HG][4]) {
     // the values of a dim group come out in the order 0, 2, 1, 3; the kernel parks its queries in the same order
-    ((acc[G >> 3] = mfma4_bcast<(G & 15)>(qa[G >> 4], int8x4_to_half_0213(kw[G]), acc[G >> 3])), ...);
+    (([&] {
+         const half4_t kv = int8x4_to_half_0213(kw[G]);
+#pragma unroll
+         for (int hg = 0; hg < HG; ++hg) acc[hg][G >> 3] = mfma4_bcast<(G & 15)>(qa[hg][G >> 4], kv, acc[hg][G >> 3]);
+     }()),
+     ...);
 }
 
 // PV over the 16 token groups x 2 dim halves: A = weights of block T (broadcast), B = this lane's V row
-template <int BITS, int... T>
+template <int BITS, int HG, int... T>
 __device__ __forceinline__ void pv_all(std::integer_sequence<int, T...>, const uint32_t (&vw)[4 * BITS],
-                                       const char *lut, half4_t pv, float4_t (&acc_o)[2][2]) {
+                                       const char *lut, const half4_t (&pv)[HG], float4_t (&acc_o)[HG][2][2]) {
     // tokens 4T..4T+3 of dim half hf are quad 2T + hf of the row
-    ((acc_o[0][T & 1] = mfma4_bcast<T>(pv, quad_values<BITS>(vw, lut, 2 * T), acc_o[0][T & 1]),
-      acc_o[1][T & 1] = mfma4_bcast<T>(pv, quad_values<BITS>(vw, lut, 2 * T + 1), acc_o[1][T & 1])),
+    (([&] {
+         const half4_t v0 = quad_values<BITS>(vw, lut, 2 * T), v1 = quad_values<BITS>(vw, lut, 2 * T + 1);
+#pragma unroll
+         for (int hg = 0; hg < HG; ++hg) {
+             acc_o[hg][0][T & 1] = mfma4_bcast<T>(pv[hg], v0, acc_o[hg][0][T & 1]);
+             acc_o[hg][1][T & 1] = mfma4_bcast<T>(pv[hg], v1, acc_o[hg][1][T & 1]);
+         }
+     }()),
      ...);
 }
 
 // q8_0-style V rows: dword 16*hf + T of the row = tokens 4T..4T+3 of dim half hf as int8.  a_lo / a_hi: the weights
 // (times the scales of this half-wavefront's 32-dim block of dim half hf) that token groups T < 8 / T >= 8 take
 // from block T % 8 of each half-wavefront.
-template <int... T>
+template <int HG, int... T>
 __device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, const uint32_t (&vw)[32],
-                                          const half4_t (&a_lo)[2], const half4_t (&a_hi)[2], float4_t (&acc_o)[2][2]) {
-    ((acc_o[0][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[0] : a_hi[0], int8x4_to_half_0213(vw[T]), acc_o[0][T & 1]),
-      acc_o[1][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[1] : a_hi[1], int8x4_to_half_0213(vw[16 + T]), acc_o[1][T & 1])),
+                                          const half4_t (&a_lo)[HG][2], const half4_t (&a_hi)[HG][2],
+                                          float4_t (&acc_o)[HG][2][2]) {
+    (([&] {
+         const half4_t v0 = int8x4_to_half_0213(vw[T]), v1 = int8x4_to_half_0213(vw[16 + T]);
+#pragma unroll
+         for (int hg = 0; hg < HG; ++hg) {
+             acc_o[hg][0][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[hg][0] : a_hi[hg][0], v0, acc_o[hg][0][T & 1]);
+             acc_o[hg][1][T & 1] = mfma4_bcast8<(T & 7)>(T < 8 ? a_lo[hg][1] : a_hi[hg][1], v1, acc_o[hg][1][T & 1]);
+         }
+     }()),
      ...);
 }
 
@@ -290,11 +314,13 @@ __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)
 // Log-sum-exp merge of a group's n_parts partials, transpose of the V rotation, output rows; one wavefront per
 // query head (the partials come straight from memory: every load of a head is issued before the first is used
 // when there are at most four).
+template <int HG>
 __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_parts, int tid, int n_waves) {
+    constexpr int NH = 4 * HG, ML = 2 * NH, PO = 128 * NH;  // heads, (m, l) floats and output floats of one partial
     const int lane = tid & 63, wave = tid >> 6;
-    const float *ml0 = a.part_ml + (int64_t)group * n_parts * 8;
-    const float *po0 = a.part_o + (int64_t)group * n_parts * 512;
-    for (int head = wave; head < 4; head += n_waves) {
+    const float *ml0 = a.part_ml + (int64_t)group * n_parts * ML;
+    const float *po0 = a.part_o + (int64_t)group * n_parts * PO;
+    for (int head = wave; head < NH; head += n_waves) {
         if (a.head_off + head >= a.q_group) continue;  // a repeated head of a group with fewer than four left
         const int64_t r_out = (int64_t)group * a.q_group + a.head_off + head;
         float M = -INFINITY, L = 0.0f, o0 = 0.0f, o1 = 0.0f;
@@ -303,8 +329,8 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const int pc = p < n_parts ? p : 0;
-                ml[p] = ld_dev2(ml0 + pc * 8 + head * 2);
-                v[p] = ld_dev2(po0 + (int64_t)pc * 512 + head * 128 + 2 * lane);
+                ml[p] = ld_dev2(ml0 + pc * ML + head * 2);
+                v[p] = ld_dev2(po0 + (int64_t)pc * PO + head * 128 + 2 * lane);
                 if (p >= n_parts) ml[p].y = 0.0f;
             }
 #pragma unroll
@@ -322,7 +348,7 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
                 const int p = p0 + lane;
                 float m = -INFINITY;
                 if (p < n_parts) {
-                    const float2 e = ld_dev2(ml0 + p * 8 + head * 2);
+                    const float2 e = ld_dev2(ml0 + p * ML + head * 2);
                     if (e.y > 0.0f) m = e.x;
                 }
                 for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
@@ -332,7 +358,7 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
                 const int p = p0 + lane;
                 float w = 0.0f, l = 0.0f;
                 if (p < n_parts) {
-                    const float2 e = ld_dev2(ml0 + p * 8 + head * 2);
+                    const float2 e = ld_dev2(ml0 + p * ML + head * 2);
                     l = e.y;
                     w = l > 0.0f ? exp2f(e.x - M) : 0.0f;
                 }
@@ -343,7 +369,7 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
 #pragma unroll 4
                 for (int t = 0; t < cnt; ++t) {
                     const float wt = __shfl(w, t);
-                    const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * 512 + head * 128 + 2 * lane);
+                    const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * PO + head * 128 + 2 * lane);
                     o0 = fmaf(v.x, wt, o0);
                     o1 = fmaf(v.y, wt, o1);
                 }
@@ -387,10 +413,12 @@ __device__ __forceinline__ unsigned long long block_sum(unsigned long long t, un
 // they finish within a tile or two of each other.
 // int8 V rows take 32 registers instead of 8 to 16: those variants run with at most 8 wavefronts per workgroup,
 // which leaves each more than the 128 registers of a 16-wavefront workgroup.
-__host__ __device__ constexpr int max_waves_per_workgroup(int vbits) { return vbits == 8 ? 8 : 16; }
+// Two sets of four query heads per pass (HG = 2: GQA groups of more than four heads read K/V once per eight heads)
+// double the accumulators and the softmax state and run with at most 8 wavefronts too.
+__host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { return vbits == 8 || hg == 2 ? 8 : 16; }
 
-template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE>
-__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_attn(AttnArgs a) {
+template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG>
+__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
     constexpr int VBLOCK = VBITS == 8 ? TQ_ROWS_PER_BLOCK * 136 : TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
@@ -400,7 +428,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
     // instructions): [K table][V table unless shared with K].  Before the tables are built the
     // first 1 KB stages the group's four rotated queries.
     constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
-    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 1024 ? LUT_TOTAL : 1024];
+    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 1024 * HG ? LUT_TOTAL : 1024 * HG];
     __shared__ uint32_t lead;  // tiles finished by the wavefront that is furthest ahead
     __shared__ uint32_t skipped;  // Sparse V: (query, position) pairs skipped by this workgroup
     char *klut_s = smem;
@@ -477,15 +505,15 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
     if constexpr (KFMT == KFMT_TURBO && KBITS == 3) kpair = a.klut[lane];
     if constexpr (!SHARE && VBITS == 3) vpair = a.vlut[lane];
 
-    // one partial per workgroup: index (group, part)
-    float *po = a.part_o + ((int64_t)group * wgs_per_group + part) * 4 * 128;
-    float *pml = a.part_ml + ((int64_t)group * wgs_per_group + part) * 4 * 2;
+    // one partial per workgroup: index (group, part), 4 HG heads each
+    float *po = a.part_o + ((int64_t)group * wgs_per_group + part) * 4 * HG * 128;
+    float *pml = a.part_ml + ((int64_t)group * wgs_per_group + part) * 4 * HG * 2;
 
     // A operand of QK, broadcast from one block per MFMA: lane (b, i) keeps q[head i] for the
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
     // The group's four queries are rotated by the first wavefronts (one 128-point butterfly per
     // head, two values per lane), scaled and parked as fp16 in 1 KB of LDS for everybody.
-    for (int h = wave; h < 4; h += n_waves) {
+    for (int h = wave; h < 4 * HG; h += n_waves) {
         _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + h * 128;
         // heads past the group's last one repeat it (their results are not written)
         const int64_t e = ((int64_t)group * a.q_group + min(a.head_off + h, a.q_group - 1)) * 128 + 2 * lane;
@@ -523,30 +551,36 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
         qw[p1] = (_Float16)(x1 * qscale);
     }
     __syncthreads();
-    half4_t qa[2];
-    {
-        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + j * 128);
-        qa[0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
-        qa[1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
+    half4_t qa[HG][2];
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) {
+        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + (4 * hg + j) * 128);
+        qa[hg][0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
+        qa[hg][1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
     __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
     if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
     if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
     __syncthreads();
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
-    float4_t acc_o[2][2];
+    float4_t acc_o[HG][2][2];
+    float m_run[HG], l_run[HG];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.0f;
+    for (int hg = 0; hg < HG; ++hg) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc_o[hg][c >> 1][c & 1] = float4_t{0.f, 0.f, 0.f, 0.f};
+        m_run[hg] = -INFINITY;
+        l_run[hg] = 0.0f;
+    }
     // additive logit bias of this lane's head and four tokens (natural-log units), one 16-byte load when the row
     // allows it; positions past the context read as 0 (they are masked anyway)
     const bool bias_vec = a.bias && (a.tokens & 3) == 0 && (reinterpret_cast<uintptr_t>(a.bias) & 15u) == 0;
-    auto load_bias = [&](int t, float (&bv)[4]) {
+    auto load_bias = [&](int t, int hg, float (&bv)[4]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) bv[i] = 0.0f;
         if (!a.bias) return;
         const int tk = t * 64 + b4;  // the launcher checks tokens < 2^31
-        const float *row = a.bias + ((int64_t)group * a.q_group + min(a.head_off + j, a.q_group - 1)) * a.tokens;
+        const float *row = a.bias + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.tokens;
         if (bias_vec && tk + 3 < (int)a.tokens) {
             const float4 v = *reinterpret_cast<const float4 *>(row + tk);
             bv[0] = v.x; bv[1] = v.y; bv[2] = v.z; bv[3] = v.w;
@@ -556,8 +590,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
                 if (tk + i < (int)a.tokens) bv[i] = row[tk + i];
         }
     };
-    float bias_next[4];
-    load_bias(min(t_begin, max(t_end - 1, 0)), bias_next);
+    float bias_next[HG][4];
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
     unsigned nskip = 0;
     bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
@@ -582,34 +617,40 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
         const VSide<VBITS> gvu_next = load_vnorm(tile_n);
         const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
-        float bias4[4];
+        float bias4[HG][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bias4[i] = bias_next[i] * LOG2E;
-        load_bias(tile_n, bias_next);
+        for (int hg = 0; hg < HG; ++hg) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bias4[hg][i] = bias_next[hg][i] * LOG2E;
+            load_bias(tile_n, hg, bias_next[hg]);
+        }
 
         // ---- QK ------------------------------------------------------------------
         // D_b[head][token 4b + lane%4]: every lane gets the 4 heads' dot products of its own token
-        float sc[4];
-        if constexpr (KFMT == KFMT_TURBO) {
-            float4_t acc[4];
+        float sc[HG][4];
+        float4_t acc[HG][4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
-            qk_turbo<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa, acc);
+        for (int hg = 0; hg < HG; ++hg)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[hg][c] = float4_t{0.f, 0.f, 0.f, 0.f};
+        if constexpr (KFMT == KFMT_TURBO) {
+            qk_turbo<KBITS, HG>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa, acc);
             const float gk_own = __half2float(__ushort_as_half((unsigned short)kn.x));
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sc[i] = ((acc[0][i] + acc[1][i]) + (acc[2][i] + acc[3][i])) * gk_own;
-        } else {
-            float4_t acc[4];
+            for (int hg = 0; hg < HG; ++hg)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
-            qk_q8(std::make_integer_sequence<int, 32>{}, kw, qa, acc);
+                for (int i = 0; i < 4; ++i) sc[hg][i] = ((acc[hg][0][i] + acc[hg][1][i]) + (acc[hg][2][i] + acc[hg][3][i])) * gk_own;
+        } else {
+            qk_q8<HG>(std::make_integer_sequence<int, 32>{}, kw, qa, acc);
             const uint2 su = kn;
             const float d0 = __half2float(__ushort_as_half((unsigned short)(su.x & 0xffff))) * a.scale_log2e;
             const float d1 = __half2float(__ushort_as_half((unsigned short)(su.x >> 16))) * a.scale_log2e;
             const float d2 = __half2float(__ushort_as_half((unsigned short)(su.y & 0xffff))) * a.scale_log2e;
             const float d3 = __half2float(__ushort_as_half((unsigned short)(su.y >> 16))) * a.scale_log2e;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sc[i] = (acc[0][i] * d0 + acc[1][i] * d1) + (acc[2][i] * d2 + acc[3][i] * d3);
+            for (int hg = 0; hg < HG; ++hg)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[hg][i] = (acc[hg][0][i] * d0 + acc[hg][1][i] * d1) + (acc[hg][2][i] * d2 + acc[hg][3][i] * d3);
         }
         {   // kw is dead now: fetch the next tile's K row into it
             const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
@@ -617,48 +658,49 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
             else load_row<8>(kbn, row_n, kw);
             kn = load_knorm(tile_n);
         }
-        // -> lane (b, j): head j, tokens 4b..4b+3
-        quad_transpose(sc, lane);
-        float s[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s[i] = sc[i] + bias4[i];
-        if (n_valid < 64) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (b4 + i >= n_valid) s[i] = -INFINITY;
-        }
-
-        // ---- online softmax (base 2) ------------------------------------------------
-        const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-        const float m_new = fmaxf(m_run, mx);
-        {
-            // 0 on the first tile, 1 when the maximum stays (also while every position so far is masked with -inf)
-            const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-            l_run *= corr;
-            // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
-            const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                acc_o[c >> 1][c & 1][0] *= c0;
-                acc_o[c >> 1][c & 1][1] *= c1;
-                acc_o[c >> 1][c & 1][2] *= c2;
-                acc_o[c >> 1][c & 1][3] *= c3;
-            }
-            m_run = m_new;
-        }
-        float p[4];
-        const float m_ref = m_run == -INFINITY ? 0.0f : m_run;  // all masked so far: weights are exp2(-inf) = 0, not NaN
+        // -> lane (b, j): head j (of each set), tokens 4b..4b+3; then the online softmax in base 2
+        float p[HG][4];
         bool any_keep = false;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            p[i] = __builtin_amdgcn_exp2f(s[i] - m_ref);  // results below 2^-126 flush to zero
-            l_run += p[i];
-            if constexpr (SPARSE) {
-                const bool in_range = b4 + i < n_valid && a.head_off + j < a.q_group;
-                const bool keep = p[i] >= a.tau;
-                if (in_range && !keep) ++nskip;
-                if (!keep) p[i] = 0.0f;
-                any_keep |= keep && in_range;
+        for (int hg = 0; hg < HG; ++hg) {
+            quad_transpose(sc[hg], lane);
+            float s[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] = sc[hg][i] + bias4[hg][i];
+            if (n_valid < 64) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (b4 + i >= n_valid) s[i] = -INFINITY;
+            }
+            const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+            const float m_new = fmaxf(m_run[hg], mx);
+            {
+                // 0 on the first tile, 1 when the maximum stays (also while every position so far is masked with -inf)
+                const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run[hg] - m_new);
+                l_run[hg] *= corr;
+                // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
+                const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    acc_o[hg][c >> 1][c & 1][0] *= c0;
+                    acc_o[hg][c >> 1][c & 1][1] *= c1;
+                    acc_o[hg][c >> 1][c & 1][2] *= c2;
+                    acc_o[hg][c >> 1][c & 1][3] *= c3;
+                }
+                m_run[hg] = m_new;
+            }
+            const float m_ref = m_run[hg] == -INFINITY ? 0.0f : m_run[hg];  // all masked so far: weights are exp2(-inf) = 0, not NaN
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[hg][i] = __builtin_amdgcn_exp2f(s[i] - m_ref);  // results below 2^-126 flush to zero
+                l_run[hg] += p[hg][i];
+                if constexpr (SPARSE) {
+                    const bool in_range = b4 + i < n_valid && a.head_off + 4 * hg + j < a.q_group;
+                    const bool keep = p[hg][i] >= a.tau;
+                    if (in_range && !keep) ++nskip;
+                    if (!keep) p[hg][i] = 0.0f;
+                    any_keep |= keep && in_range;
+                }
             }
         }
         if constexpr (SPARSE) {
@@ -679,9 +721,6 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
             // The dims of block b lie in 32-dim block b / 8 (+ 2 for the upper dim half), so the weights carry that
             // block's scale and are broadcast inside each half of the wavefront: token group T is served by block
             // T % 8 of both halves, which therefore also needs the weights of the lane 32 away.
-            float ps[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ps[i] = __shfl_xor(p[i], 32);
             auto weights = [&](const float (&w)[4], uint2 sc) {
                 const float s0 = __half2float(__ushort_as_half((unsigned short)(sc.x & 0xffff))) * Q8V_PRESCALE;
                 const float s1 = __half2float(__ushort_as_half((unsigned short)(sc.x >> 16))) * Q8V_PRESCALE;
@@ -695,24 +734,37 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
                 return r;
             };
             const bool upper = lane >= 32;
-            half4_t a_lo[2], a_hi[2];
+            half4_t a_lo[HG][2], a_hi[HG][2];
 #pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
-                const half4_t own = weights(p, gvu.v[2 * hf]), swp = weights(ps, gvu.v[2 * hf + 1]);
-                a_lo[hf] = upper ? swp : own;
-                a_hi[hf] = upper ? own : swp;
+            for (int hg = 0; hg < HG; ++hg) {
+                float ps[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ps[i] = __shfl_xor(p[hg][i], 32);
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const half4_t own = weights(p[hg], gvu.v[2 * hf]), swp = weights(ps, gvu.v[2 * hf + 1]);
+                    a_lo[hg][hf] = upper ? swp : own;
+                    a_hi[hg][hf] = upper ? own : swp;
+                }
             }
-            pv_all_q8(std::make_integer_sequence<int, 16>{}, vw, a_lo, a_hi, acc_o);
+            pv_all_q8<HG>(std::make_integer_sequence<int, 16>{}, vw, a_lo, a_hi, acc_o);
         } else {
-            half4_t pv;
-            pv[0] = (_Float16)(p[0] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x & 0xffff))));
-            pv[1] = (_Float16)(p[1] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x >> 16))));
-            pv[2] = (_Float16)(p[2] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y & 0xffff))));
-            pv[3] = (_Float16)(p[3] * __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y >> 16))));
+            const float g0 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x & 0xffff)));
+            const float g1 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x >> 16)));
+            const float g2 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y & 0xffff)));
+            const float g3 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].y >> 16)));
+            half4_t pv[HG];
+#pragma unroll
+            for (int hg = 0; hg < HG; ++hg) {
+                pv[hg][0] = (_Float16)(p[hg][0] * g0);
+                pv[hg][1] = (_Float16)(p[hg][1] * g1);
+                pv[hg][2] = (_Float16)(p[hg][2] * g2);
+                pv[hg][3] = (_Float16)(p[hg][3] * g3);
+            }
             // V row of this lane: dims lane and 64+lane for the tile's 64 tokens; quad 2T + hf =
             // tokens 4T..4T+3 of dim half hf.  Block b = lane/4 of the MFMA covers dims 4b..4b+3 (+64*hf); the
             // weights of token group T sit in block T and are broadcast to every block.
-            pv_all<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
+            pv_all<VBITS, HG>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
         }
         load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
         v_ahead = true;
@@ -723,52 +775,71 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
     // ---- end of split: the workgroup's wavefronts merge their partials in LDS and write one ------
     if constexpr (VBITS == 8) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc_o[c >> 1][c & 1] *= 1.0f / Q8V_PRESCALE;
+        for (int hg = 0; hg < HG; ++hg)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc_o[hg][c >> 1][c & 1] *= 1.0f / Q8V_PRESCALE;
     }
-    const float l_tot = sum_over_blocks(l_run);
+    float l_tot[HG];
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) l_tot[hg] = sum_over_blocks(l_run[hg]);
     if (n_waves == 1) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
+        for (int hg = 0; hg < HG; ++hg) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) st_dev(po + i * 128 + 64 * hf + lane, acc_o[hf][0][i] + acc_o[hf][1][i]);
-        if (lane < 4) {
-            st_dev(pml + 2 * j, m_run);
-            st_dev(pml + 2 * j + 1, l_tot);
+            for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    st_dev(po + (4 * hg + i) * 128 + 64 * hf + lane, acc_o[hg][hf][0][i] + acc_o[hg][hf][1][i]);
+            if (lane < 4) {
+                st_dev(pml + 2 * (4 * hg + j), m_run[hg]);
+                st_dev(pml + 2 * (4 * hg + j) + 1, l_tot[hg]);
+            }
         }
     } else {
-        // per wavefront: out[4][128], then m[4], l[4]
+        // per wavefront and set of four heads: out[4][128], then m[4], l[4]
         extern __shared__ float merge_s[];
-        constexpr int MS = MERGE_FLOATS;
+        constexpr int MS = MERGE_FLOATS * HG;
         float *mine = merge_s + wave * MS;
-        if (lane < 4) {
-            mine[512 + j] = m_run;
-            mine[516 + j] = l_tot;
+#pragma unroll
+        for (int hg = 0; hg < HG; ++hg)
+            if (lane < 4) {
+                mine[hg * MERGE_FLOATS + 512 + j] = m_run[hg];
+                mine[hg * MERGE_FLOATS + 516 + j] = l_tot[hg];
+            }
+        __syncthreads();
+        float M[HG];
+#pragma unroll
+        for (int hg = 0; hg < HG; ++hg) {
+            // head j's maximum over the wavefronts that saw an unmasked position
+            M[hg] = -INFINITY;
+            for (int w = 0; w < n_waves; ++w)
+                if (merge_s[w * MS + hg * MERGE_FLOATS + 516 + j] > 0.0f) M[hg] = fmaxf(M[hg], merge_s[w * MS + hg * MERGE_FLOATS + 512 + j]);
+            const float f = l_tot[hg] > 0.0f ? __builtin_amdgcn_exp2f(m_run[hg] - M[hg]) : 0.0f;
+            const float f4[4] = {dpp<0x00>(f), dpp<0x55>(f), dpp<0xAA>(f), dpp<0xFF>(f)};
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    mine[hg * MERGE_FLOATS + i * 128 + 64 * hf + lane] = (acc_o[hg][hf][0][i] + acc_o[hg][hf][1][i]) * f4[i];
         }
         __syncthreads();
-        // head j's maximum over the wavefronts that saw an unmasked position
-        float M = -INFINITY;
-        for (int w = 0; w < n_waves; ++w)
-            if (merge_s[w * MS + 516 + j] > 0.0f) M = fmaxf(M, merge_s[w * MS + 512 + j]);
-        const float f = l_tot > 0.0f ? __builtin_amdgcn_exp2f(m_run - M) : 0.0f;
-        const float f4[4] = {dpp<0x00>(f), dpp<0x55>(f), dpp<0xAA>(f), dpp<0xFF>(f)};
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) mine[i * 128 + 64 * hf + lane] = (acc_o[hf][0][i] + acc_o[hf][1][i]) * f4[i];
-        __syncthreads();
-        for (int e = tid; e < 512; e += 64 * n_waves) {
+        for (int e = tid; e < 512 * HG; e += 64 * n_waves) {
+            const int src = (e >> 9) * MERGE_FLOATS + (e & 511);  // partial element e = head e / 128, dim e % 128
             float sum = 0.0f;
-            for (int w = 0; w < n_waves; ++w) sum += merge_s[w * MS + e];
+            for (int w = 0; w < n_waves; ++w) sum += merge_s[w * MS + src];
             st_dev(po + e, sum);
         }
-        if (tid < 4) {  // lanes 0..3 of wavefront 0 hold heads 0..3
-            float L = 0.0f;
-            for (int w = 0; w < n_waves; ++w) {
-                const float lw = merge_s[w * MS + 516 + j];
-                if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(merge_s[w * MS + 512 + j] - M), L);
+        if (tid < 4) {  // lanes 0..3 of wavefront 0 hold heads 0..3 of each set
+#pragma unroll
+            for (int hg = 0; hg < HG; ++hg) {
+                float L = 0.0f;
+                for (int w = 0; w < n_waves; ++w) {
+                    const float lw = merge_s[w * MS + hg * MERGE_FLOATS + 516 + j];
+                    if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(merge_s[w * MS + hg * MERGE_FLOATS + 512 + j] - M[hg]), L);
+                }
+                st_dev(pml + 2 * (4 * hg + j), M[hg]);
+                st_dev(pml + 2 * (4 * hg + j) + 1, L);
             }
-            st_dev(pml + 2 * j, M);
-            st_dev(pml + 2 * j + 1, L);
         }
     }
     if constexpr (SPARSE) {
@@ -812,7 +883,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS)) void k_decode_
             }
         }
     }
-    merge_group(a, group, n_parts, tid, n_waves);
+    merge_group<HG>(a, group, n_parts, tid, n_waves);
     if (n_parts > 1) {
         for (int p = tid; p < n_parts; p += (int)blockDim.x) st_dev(a.flags + (int64_t)group * n_parts + p, 0ull);
     }
@@ -869,14 +940,30 @@ unsigned long long next_nonce() {
 struct WsLayout {
     int64_t part_o, part_ml, skip_slots, flags, pass_totals, total;
 };
+// How a parameter set is run: sets of four query heads per pass (2 when a KV head serves more than four query
+// heads), wavefronts per workgroup (the largest power of two up to the variant's limit that divides the split
+// count) and workgroups = partials per group.
+struct AttnPlan {
+    int hg, wpw, n_parts;
+};
+AttnPlan attn_plan(const tq_attn_params *p) {
+    AttnPlan pl;
+    pl.hg = p->n_q_heads / p->n_kv_heads > 4 ? 2 : 1;
+    pl.wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
+    while (p->n_splits % pl.wpw) pl.wpw >>= 1;
+    pl.n_parts = p->n_splits / pl.wpw;
+    return pl;
+}
 WsLayout ws_layout(const tq_attn_params *p) {
     const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
+    const AttnPlan pl = attn_plan(p);
+    const int64_t parts = groups * pl.n_parts;
     WsLayout w;
     w.part_o = 0;
-    w.part_ml = w.part_o + align256(groups * p->n_splits * 4 * 128 * 4);
-    w.skip_slots = w.part_ml + align256(groups * p->n_splits * 4 * 2 * 4);
-    w.flags = w.skip_slots + align256(groups * p->n_splits * 8);
-    w.pass_totals = w.flags + align256(groups * p->n_splits * 8);
+    w.part_ml = w.part_o + align256(parts * 4 * pl.hg * 128 * 4);
+    w.skip_slots = w.part_ml + align256(parts * 4 * pl.hg * 2 * 4);
+    w.flags = w.skip_slots + align256(parts * 8);
+    w.pass_totals = w.flags + align256(parts * 8);
     w.total = w.pass_totals + align256(MAX_PASSES * 8);
     return w;
 }
@@ -941,20 +1028,22 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: sparse_v_tau > 0 needs skip_count");
         return TQ_ERR_ARG;
     }
-    // wavefronts per workgroup: the largest power of two up to 16 (8 for int8 V rows) that divides the split count
-    int wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? hv->bits : 8);
-    while (p->n_splits % wpw) wpw >>= 1;
-    const unsigned grid = (unsigned)((int64_t)groups * (p->n_splits / wpw));
+    // wavefronts per workgroup: the largest power of two up to 16 (8 for int8 V rows and for eight heads per pass)
+    // that divides the split count
+    const AttnPlan pl = attn_plan(p);
+    const int wpw = pl.wpw, hg = pl.hg;
+    const unsigned grid = (unsigned)((int64_t)groups * pl.n_parts);
     const unsigned wg = 64u * (unsigned)wpw;
-    const int n_parts = p->n_splits / wpw;  // partials per group: the wavefronts of a workgroup merge theirs in LDS
-    const size_t merge_bytes = wpw > 1 ? (size_t)wpw * MERGE_FLOATS * sizeof(float) : 0;
+    const int n_parts = pl.n_parts;  // partials per group: the wavefronts of a workgroup merge theirs in LDS
+    const size_t merge_bytes = wpw > 1 ? (size_t)wpw * hg * MERGE_FLOATS * sizeof(float) : 0;
     const int vb = turbo_v ? hv->bits : 8;
     const int kb = turbo_k ? hk->bits : 8;
-    // The kernels work on four query heads of a KV head at a time (the 4-row MFMA block): a group of G heads takes
-    // ceil(G / 4) passes over the same K/V, each with its own merge launch; a last pass with fewer than four
-    // heads repeats the group's last head and does not write the repeats.
+    // The kernels work on four query heads of a KV head at a time (the 4-row MFMA block), or on eight (two sets
+    // against the same dequantised rows) when a KV head serves more than four: a group of G heads takes
+    // ceil(G / 8) passes over the same K/V; a last pass with fewer heads than it has rows repeats the group's
+    // last head and does not write the repeats.
     a.q_group = p->n_q_heads / p->n_kv_heads;
-    if ((a.q_group + 3) / 4 > MAX_PASSES) {
+    if ((a.q_group + 4 * hg - 1) / (4 * hg) > MAX_PASSES) {
         tq_set_error("tq_decode_attention: %d query heads per KV head (at most %d)", a.q_group, 4 * MAX_PASSES);
         return TQ_ERR_UNSUPPORTED;
     }
@@ -967,18 +1056,23 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.skip_count = skip_count;
     a.total_pairs = total_pairs;
     (void)n_parts;
-    for (a.head_off = 0; a.head_off < a.q_group; a.head_off += 4) {
-        a.pass = a.head_off / 4;
+    (void)kb;
+    for (a.head_off = 0; a.head_off < a.q_group; a.head_off += 4 * hg) {
+        a.pass = a.head_off / (4 * hg);
         a.nonce = next_nonce();
-#define TQ_ATTN_ONE(KF, KB, VB, SP, SH) k_decode_attn<KF, KB, VB, SP, SH><<<grid, wg, merge_bytes, s>>>(a)
+#define TQ_ATTN_ONE(KF, KB, VB, SP, SH)                                            \
+    {                                                                             \
+        if (hg == 2) k_decode_attn<KF, KB, VB, SP, SH, 2><<<grid, wg, merge_bytes, s>>>(a); \
+        else k_decode_attn<KF, KB, VB, SP, SH, 1><<<grid, wg, merge_bytes, s>>>(a);         \
+    }
 #define TQ_ATTN(KF, KB, VB)                         \
-    if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false); \
+    if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false)  \
     else TQ_ATTN_ONE(KF, KB, VB, false, false)
     // same width and same centroids: one table
 #define TQ_ATTN_SAME(B)                                         \
-    if (share && sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, true);   \
-    else if (share) TQ_ATTN_ONE(KFMT_TURBO, B, B, false, true);       \
-    else if (sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, false);      \
+    if (share && sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, true)    \
+    else if (share) TQ_ATTN_ONE(KFMT_TURBO, B, B, false, true)        \
+    else if (sparse) TQ_ATTN_ONE(KFMT_TURBO, B, B, true, false)       \
     else TQ_ATTN_ONE(KFMT_TURBO, B, B, false, false)
     if (turbo_k && kb == 3 && vb == 3) { TQ_ATTN_SAME(3); }
     else if (turbo_k && kb == 4 && vb == 4) { TQ_ATTN_SAME(4); }

@@ -327,8 +327,9 @@ def q8_0_unpack(packed, n_seqs: int, tokens: int, kind: str = "k"):
 class DecodeAttention:
     """softmax(scale * q k^T) v over packed K/V; n_q_heads a multiple of n_kv_heads.
 
-    The kernels take four query heads of a KV head per pass over its K/V, so a
-    group of 4 reads the cache once and a group of G reads it ceil(G / 4) times.
+    The kernels take four query heads of a KV head per pass over its K/V, or
+    eight when the group has more than four, so groups of up to 8 read the cache
+    once and a group of G > 8 reads it ceil(G / 8) times.
 
     Holds the parameter block and the split workspace so that repeated steps
     allocate nothing.  K is a turbo buffer (k_codec given) or a q8_0-style
