@@ -1234,7 +1234,9 @@ __global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, i
 // step by step, with the next tile's while the last sub-block is being multiplied, so every query
 // operand crosses the vector memory path once per workgroup and a whole tile ahead of its use.
 constexpr int SCORE_KEYS = 256;  // keys per workgroup (two 128-row blocks)
-template <int BITS, typename TO>
+// PAIRS (fp16 logits only): the key count is even and the logits are 4-byte aligned, so a lane stores two at once.
+// DRAIN false is the measurement mode: everything but the stores (logits is NULL).
+template <int BITS, typename TO, bool PAIRS, bool DRAIN>
 __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
                                                       const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
                                                       const float *cent, float proj_scale) {
@@ -1282,9 +1284,8 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
     // two MFMA tiles of 32 x 32 per (64 queries, 32 keys): lane l of a result tile holds key column
     // l % 32 for the query rows 8j + 4(l/32) + i, so a store instruction writes two runs of 32 consecutive
     // logits (a whole 128-byte line for fp32).
-    const int qh = __builtin_amdgcn_readfirstlane(w);  // wave-uniform: row addresses of the stores stay scalar
+    const int qh = __builtin_amdgcn_readfirstlane(w);  // wave-uniform: the bases of the stores stay scalar
     const int c32 = lane & 31, kb = lane >> 5;
-    const uint32_t lane_off = (uint32_t)(4 * kb) * (uint32_t)nk + (uint32_t)c32;  // this lane's place relative to a row block
     constexpr int QT = 512;
     const int n_qt = (int)((nq + QT - 1) / QT);
     const int nq_last = (int)nq - 1;  // the launcher checks the query count
@@ -1306,91 +1307,144 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
 #pragma unroll
     for (int t = 0; t < 16; ++t) load_queries(t);
     const _Float16 *krow0 = kt + c32 * KT_STRIDE + 8 * kb;
-#pragma unroll 1
-    for (int qt = 0; qt < n_qt; ++qt) {
-        const int qbase = qt * QT + qh * 64;
-        point_queries(min(qt + 1, n_qt - 1));  // the last tile re-reads itself
-        // one 32-key sub-block against the resident query tile; the last one of a tile also fetches the next tile
-        auto sub_block = [&](const int ks, auto prefetch) {
-            float16_t acc[2];
+
+    // A finished (64 queries, 32 keys) block is written while the next one is being multiplied: its store
+    // instructions go out one after each matrix instruction of the next block, from a second set of accumulators,
+    // so a wavefront never sits in a store-only phase.  The stores are buffer stores whose resource starts at the
+    // row a store writes (scalar arithmetic) and ends after the block's last existing row, and whose only vector
+    // operand is the lane's place relative to that row (one register for the whole kernel): rows past the last
+    // query fall outside the resource and the hardware drops them, lanes whose key does not exist get an offset
+    // outside every resource, and no store needs an address register or a branch.
+    constexpr bool PAIRED = sizeof(TO) == 2 && PAIRS;  // fp16: two logits per store
+    constexpr int N_GROUPS = PAIRED ? 16 : 32;         // store instructions per block
+    constexpr int NT_AUX = (TQ_STREAM_SITES & STREAM_LOGITS) ? 2 : 0;  // the non-temporal bit of a buffer instruction
+    constexpr uint32_t DROPPED = 0x80000000u;          // beyond any resource (the launcher keeps 64 rows below 2 GiB)
+    const uint32_t row_bytes = (uint32_t)nk * (uint32_t)sizeof(TO);
+    const bool odd = lane & 1;
+    // paired: even lanes store rows 8j + 4kb + h, odd lanes rows 8j + 4kb + 2 + h, keys (c32 & ~1, c32 | 1)
+    const uint32_t lane_bytes = (uint32_t)(4 * kb) * row_bytes +
+                                (PAIRED ? (odd ? 2u * row_bytes + (uint32_t)(c32 - 1) * 2u : (uint32_t)c32 * 2u)
+                                        : (uint32_t)c32 * (uint32_t)sizeof(TO));
+    struct Pending {
+        TO *base[2];        // first logit of the two 32-row blocks
+        int rows[2];        // rows of each that exist (0: nothing is pending)
+        uint32_t voff;      // lane_bytes, or DROPPED where the lane's key does not exist
+    };
+    auto pend = [&](int qbase, int ks) __attribute__((always_inline)) {
+        Pending pb;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+#ifdef TQ_SCORE_L2  // measurement build: every query tile lands on the first 64 rows, so the logits stay in L2
+            pb.base[mb] = logits + (int64_t)((qbase & 63) + mb * 32) * nk + (key0 + ks * 32);
+#else
+            pb.base[mb] = logits + (int64_t)(qbase + mb * 32) * nk + (key0 + ks * 32);
+#endif
+            pb.rows[mb] = max(0, min(32, (int)nq - (qbase + mb * 32)));
+            // wave-uniform by construction; said explicitly so that the resources are built by scalar instructions
+            pb.rows[mb] = __builtin_amdgcn_readfirstlane(pb.rows[mb]);
+            const uint64_t b = reinterpret_cast<uint64_t>(pb.base[mb]);
+            pb.base[mb] = reinterpret_cast<TO *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                                                 (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
+        }
+        const int64_t first_key = key0 + ks * 32 + (PAIRED ? (c32 & ~1) : c32);  // paired: the key count is even
+        pb.voff = first_key < nk ? lane_bytes : DROPPED;
+        return pb;
+    };
+    // store group n of a pending block: unpaired, accumulator element n % 16 of row block n / 16 (rows 8j + 4kb + i,
+    // e = 4j + i); paired, rows 8j + 4kb + {h, 2 + h} of row block n / 8, j = (n % 8) / 2, h = n % 2
+    auto store_group = [&](const Pending &pb, const float16_t (&acc)[2], const int n) __attribute__((always_inline)) {
+        const int mb = PAIRED ? n >> 3 : n >> 4;
+        const int row = PAIRED ? 8 * ((n >> 1) & 3) + (n & 1) : 8 * ((n & 15) >> 2) + (n & 3);  // of lane half kb = 0
+        const int left = max(pb.rows[mb] - row, 0);
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc(pb.base[mb] + (int64_t)row * nk, 0, (int)((uint32_t)left * row_bytes), 0x00020000);
+        if constexpr (PAIRED) {
+            // neighbouring lanes (keys c32, c32 ^ 1) trade two of their four rows
+            const int j = (n >> 1) & 3, h = n & 1;
+            const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
+            const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
+            const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;
+            const uint32_t u = (uint32_t)__half_as_ushort(__float2half_rn(v0)) | ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
+            __builtin_amdgcn_raw_buffer_store_b32(u, rs, (int)pb.voff, 0, NT_AUX);
+        } else if constexpr (sizeof(TO) == 4) {
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mb][n & 15]), rs, (int)pb.voff, 0, NT_AUX);
+        } else {
+            __builtin_amdgcn_raw_buffer_store_b16(__half_as_ushort(__float2half_rn(acc[mb][n & 15])), rs, (int)pb.voff, 0, NT_AUX);
+        }
+    };
+
+    float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
+    // one 32-key sub-block against the resident query tile into acc, while the pending block leaves from pacc
+    auto sub_block = [&](const int ks, auto prefetch, auto drain, float16_t (&acc)[2], const float16_t (&pacc)[2],
+                         const Pending &pb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mb][e] = 0.0f;
+        // (the sub-block number is made opaque: with a constant the compiler keeps one address register per step
+        // instead of one base and sixteen immediate offsets)
+        int ks_opaque = ks;
+        asm volatile("" : "+s"(ks_opaque));
+        const _Float16 *krow = krow0 + ks_opaque * 32 * KT_STRIDE;
+        // key operands come from LDS AHEAD steps ahead; the scheduling fence after every step keeps the
+        // compiler from hoisting all sixteen steps' reads to the top
+        constexpr int AHEAD = 3;
+        half8_t kf[AHEAD + 1];
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t) kf[t] = *reinterpret_cast<const half8_t *>(krow + t * 16);
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            if (t + AHEAD < 16) kf[(t + AHEAD) & AHEAD] = *reinterpret_cast<const half8_t *>(krow + (t + AHEAD) * 16);
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[t][mb], kf[t & AHEAD], acc[mb], 0, 0, 0);
+                if constexpr (decltype(drain)::value) {
+                    const int n = 2 * t + mb;
+                    if (N_GROUPS == 32 || (n & 1)) store_group(pb, pacc, N_GROUPS == 32 ? n : n >> 1);
+                }
+            }
+            if constexpr (decltype(prefetch)::value) load_queries(t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (!decltype(drain)::value) {
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) acc[mb][e] = 0.0f;
-            const _Float16 *krow = krow0 + ks * 32 * KT_STRIDE;
-            // key operands come from LDS one step ahead; the scheduling fence after every step keeps the
-            // compiler from hoisting all sixteen steps' reads to the top
-            half8_t kf[2];
-            kf[0] = *reinterpret_cast<const half8_t *>(krow);
+                for (int e = 0; e < 16; ++e) keep += acc[mb][e];
+        }
+    };
+    auto sweep = [&](auto drain) __attribute__((always_inline)) {
+        float16_t acc_a[2], acc_b[2];
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                if (t + 1 < 16) kf[(t + 1) & 1] = *reinterpret_cast<const half8_t *>(krow + (t + 1) * 16);
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int mb = 0; mb < 2; ++mb)
-                    acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[t][mb], kf[t & 1], acc[mb], 0, 0, 0);
-                if constexpr (decltype(prefetch)::value) load_queries(t);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (!logits) {  // measurement mode: nothing is stored; the products stay live through a store that never happens
-                float keep = 0.0f;
-#pragma unroll
-                for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) keep += acc[mb][e];
-                if (keep == 1.25e38f) reinterpret_cast<float *>(const_cast<__half *>(qa))[0] = keep;
-                return;
-            }
-            const bool full = key0 + ks * 32 + 32 <= nk && qbase + 64 <= (int)nq;
-            const int64_t key = key0 + ks * 32 + c32;
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
-                TO *ubase = logits + (int64_t)(qbase + mb * 32) * nk + (key0 + ks * 32);  // uniform: row 0 of the block
-                if constexpr (sizeof(TO) == 4) {
-                    if (full) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) stream_store<STREAM_LOGITS>((ubase + (int64_t)(8 * j + i) * nk) + lane_off, (TO)acc[mb][4 * j + i]);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) {
-                                const int qi = qbase + mb * 32 + 8 * j + 4 * kb + i;
-                                if (qi < (int)nq && key < nk) (ubase + (int64_t)(8 * j + i) * nk)[lane_off] = (TO)acc[mb][4 * j + i];
-                            }
-                    }
-                } else {
-                    // fp16: neighbouring lanes (keys c32, c32 ^ 1) trade two of their four rows so that every
-                    // lane stores two logits at once: even lanes rows i = 0, 1, odd lanes rows i = 2, 3
-                    const bool odd = lane & 1;
-                    const bool pair_ok = (nk & 1) == 0 && (reinterpret_cast<uintptr_t>(logits) & 3u) == 0;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-#pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
-                            const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
-                            const int i = odd ? 2 + h : h;
-                            const int qi = qbase + mb * 32 + 8 * j + 4 * kb + i;
-                            const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;  // keys (c32 & ~1), (c32 | 1)
-                            __half *p = reinterpret_cast<__half *>(ubase + (int64_t)(8 * j + h) * nk) + (lane_off + (odd ? 2u * (uint32_t)nk - 1u : 0u));
-                            const int64_t k0 = key - (odd ? 1 : 0);
-                            if (pair_ok && (full || (qi < (int)nq && k0 + 1 < nk))) {
-                                const uint32_t u = (uint32_t)__half_as_ushort(__float2half_rn(v0)) |
-                                                   ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
-                                stream_store<STREAM_LOGITS>(reinterpret_cast<uint32_t *>(p), u);
-                            } else if (qi < (int)nq) {
-                                if (k0 < nk) p[0] = __float2half_rn(v0);
-                                if (k0 + 1 < nk) p[1] = __float2half_rn(v1);
-                            }
-                        }
-                }
-            }
-        };
+            for (int e = 0; e < 16; ++e) acc_b[mb][e] = 0.0f;
+        Pending pb = pend(0, 0);
+        pb.rows[0] = pb.rows[1] = 0;  // nothing is pending before the first block
 #pragma unroll 1
-        for (int ks = 0; ks < SCORE_KEYS / 32 - 1; ++ks) sub_block(ks, std::false_type{});
-        sub_block(SCORE_KEYS / 32 - 1, std::true_type{});
+        for (int qt = 0; qt < n_qt; ++qt) {
+            const int qbase = qt * QT + qh * 64;
+            point_queries(min(qt + 1, n_qt - 1));  // the last tile re-reads itself
+#pragma unroll 1
+            for (int kp = 0; kp < SCORE_KEYS / 64 - 1; ++kp) {
+                sub_block(2 * kp, std::false_type{}, drain, acc_a, acc_b, pb);
+                pb = pend(qbase, 2 * kp);
+                sub_block(2 * kp + 1, std::false_type{}, drain, acc_b, acc_a, pb);
+                pb = pend(qbase, 2 * kp + 1);
+            }
+            sub_block(SCORE_KEYS / 32 - 2, std::false_type{}, drain, acc_a, acc_b, pb);
+            pb = pend(qbase, SCORE_KEYS / 32 - 2);
+            sub_block(SCORE_KEYS / 32 - 1, std::true_type{}, drain, acc_b, acc_a, pb);  // also fetches the next tile's queries
+            pb = pend(qbase, SCORE_KEYS / 32 - 1);
+        }
+        if constexpr (decltype(drain)::value) {  // the last block (in acc_b)
+#pragma unroll
+            for (int n = 0; n < N_GROUPS; ++n) store_group(pb, acc_b, n);
+        }
+    };
+    sweep(std::integral_constant<bool, DRAIN>{});
+    if constexpr (!DRAIN) {
+        if (keep == 1.25e38f) reinterpret_cast<float *>(const_cast<__half *>(qa))[0] = keep;
     }
 }
 
@@ -1402,6 +1456,12 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
     (void)ws_bytes;
     if (nq >= ((int64_t)1 << 31) / 128) {
         tq_set_error("tq_score_tile: %lld queries beyond 2^24 - 1", (long long)nq);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    // the kernel addresses a block of 64 logit rows with 32-bit byte offsets
+    if ((uint64_t)nk * (out_dtype == TQ_F32 ? 4 : 2) * 64 >= 0x7FFFFFFFull) {
+        tq_set_error("tq_score_tile: %lld keys per call beyond %lld (64 rows of logits must stay below 2 GiB): score the keys in slices",
+                     (long long)nk, (long long)(0x7FFFFFFFll / 64 / (out_dtype == TQ_F32 ? 4 : 2)));
         return TQ_ERR_UNSUPPORTED;
     }
     __half *qa = reinterpret_cast<__half *>(ws);
@@ -1416,18 +1476,25 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
     if (rc) return rc;
     const unsigned grid = (unsigned)((nk + SCORE_KEYS - 1) / SCORE_KEYS);
     const size_t lds = (size_t)SCORE_KEYS * KT_STRIDE * sizeof(_Float16);
-#define TQ_SCORE(B, T)                                                                                          \
-    {                                                                                                           \
-        (void)hipFuncSetAttribute((const void *)k_score_tile<B, T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                  (int)lds);                                                                    \
-        k_score_tile<B, T><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
-                                                  nq, nk, (T *)logits, h->centroids32, (float)h->proj_scale);   \
+#define TQ_SCORE(B, T, P, DR)                                                                                          \
+    {                                                                                                                  \
+        (void)hipFuncSetAttribute((const void *)k_score_tile<B, T, P, DR>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                  (int)lds);                                                                           \
+        k_score_tile<B, T, P, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
+                                                         nq, nk, (T *)logits, h->centroids32, (float)h->proj_scale);   \
     }
-    if (out_dtype == TQ_F32) {
-        if (h->bits == 2) TQ_SCORE(2, float) else if (h->bits == 3) TQ_SCORE(3, float) else TQ_SCORE(4, float)
+#define TQ_SCORE_BITS(T, P, DR)                                                                              \
+    if (h->bits == 2) TQ_SCORE(2, T, P, DR) else if (h->bits == 3) TQ_SCORE(3, T, P, DR) else TQ_SCORE(4, T, P, DR)
+    if (!logits) {
+        TQ_SCORE_BITS(float, false, false)
+    } else if (out_dtype == TQ_F32) {
+        TQ_SCORE_BITS(float, false, true)
+    } else if ((nk & 1) == 0 && (reinterpret_cast<uintptr_t>(logits) & 3u) == 0) {
+        TQ_SCORE_BITS(__half, true, true)
     } else {
-        if (h->bits == 2) TQ_SCORE(2, __half) else if (h->bits == 3) TQ_SCORE(3, __half) else TQ_SCORE(4, __half)
+        TQ_SCORE_BITS(__half, false, true)
     }
+#undef TQ_SCORE_BITS
 #undef TQ_SCORE
     return tq_check_launch("score_tile");
 }
