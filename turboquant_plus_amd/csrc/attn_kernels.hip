@@ -1169,62 +1169,72 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int KT_STRIDE = 264;  // halves per staged key row (256 + 8: 16-byte reads of 16 rows hit 64 distinct banks)
 
-// [R q | S q] as fp16; a wavefront takes PREP_Q queries so that every row of the projection it fetches serves
-// all of them (one query per wavefront made the launch wait for 2048 x 64 KB of L2 reads)
-constexpr int PREP_Q = 4;
+// [R q | S q] as fp16 on the matrix cores: a workgroup of four wavefronts takes 32 queries, wavefront w the output
+// rows 32w .. 32w+31 of the rotation and of the projection, as (W Q^T) with W's fragments prepared with the handle
+// (rotation: +-1 entries, exact; projection: two fp16 terms) and the queries as the column side.  Queries that are
+// not fp16 are split into two fp16 terms as well, so that every product is exact and the sums carry fp32 rounding
+// only (as the scalar loop did).  Lane l ends up with query l % 32 and four consecutive outputs per register
+// group: an 8-byte store, 512 contiguous bytes per wavefront.
 template <typename TI>
-__global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, int64_t nq, const float *s1,
-                                                      const float *s2, const float *projT) {
-    __shared__ float qs[4][PREP_Q][128];
+__global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, int64_t nq, const uint4 *wfrag) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int64_t v0 = ((int64_t)blockIdx.x * 4 + w) * PREP_Q;
-    float x0[PREP_Q], x1[PREP_Q];
+    const int r = lane & 31, kb = lane >> 5;
+    const int64_t blk = blockIdx.x;
+    const int64_t v = min(blk * 32 + r, nq - 1);  // rows past the last query repeat it (their block is allocated)
+    constexpr bool SPLIT = !std::is_same<TI, __half>::value;
+    half8_t xh[8], xl[8];
 #pragma unroll
-    for (int i = 0; i < PREP_Q; ++i) {
-        const bool have = v0 + i < nq;
-        x0[i] = have ? ldf(q + (v0 + i) * 128 + 2 * lane) : 0.f;
-        x1[i] = have ? ldf(q + (v0 + i) * 128 + 2 * lane + 1) : 0.f;
-        qs[w][i][2 * lane] = x0[i];
-        qs[w][i][2 * lane + 1] = x1[i];
-    }
-    __syncthreads();
-    if (v0 >= nq) return;
-    float p0[PREP_Q], p1[PREP_Q];  // (S q)[2*lane], (S q)[2*lane+1]
+    for (int t = 0; t < 8; ++t) {
+        const TI *src = q + v * 128 + 16 * t + 8 * kb;
+        if constexpr (!SPLIT) {
+            xh[t] = *reinterpret_cast<const half8_t *>(src);
+        } else {
 #pragma unroll
-    for (int i = 0; i < PREP_Q; ++i) p0[i] = p1[i] = 0.f;
-#pragma unroll 8
-    for (int k = 0; k < 128; ++k) {
-        const float2 pt = *reinterpret_cast<const float2 *>(projT + k * 128 + 2 * lane);
-#pragma unroll
-        for (int i = 0; i < PREP_Q; ++i) {
-            const float qk = qs[w][i][k];
-            p0[i] = fmaf(pt.x, qk, p0[i]);
-            p1[i] = fmaf(pt.y, qk, p1[i]);
+            for (int e = 0; e < 8; ++e) {
+                const float x = ldf(src + e);
+                const _Float16 hi = (_Float16)x;
+                xh[t][e] = hi;
+                xl[t][e] = (_Float16)(x - (float)hi);
+            }
         }
     }
-    const float a0 = s1[2 * lane], a1 = s1[2 * lane + 1];
-    const float b0 = s2[2 * lane] * RSQRT128, b1 = s2[2 * lane + 1] * RSQRT128;
-    __half2 *qa2 = reinterpret_cast<__half2 *>(qa);
+    constexpr int SET = 4 * 8 * 64;  // fragments (16 bytes) per set
+    const uint4 *fr = wfrag + (w * 8) * 64 + lane;
+    float16_t rot, prj;
 #pragma unroll
-    for (int i = 0; i < PREP_Q; ++i) {
-        const int64_t v = v0 + i;
-        if (v >= nq) break;
-        float y0 = x0[i] * a0, y1 = x1[i] * a1;
-        wht128_wave(y0, y1, lane);
-        y0 *= b0;
-        y1 *= b1;
-        // operand-major layout: the 16-byte chunk (row r of query block v / 32, K values 16t + 8kb .. + 7) that
-        // lane r + 32kb of the score tile's MFMA reads in K step t sits at chunk index (block * 16 + t) * 64 + r + 32kb,
-        // so one wave-wide operand load is 1 KB of contiguous memory
-        const int64_t blk = v >> 5;
-        const int r = (int)(v & 31);
-        auto chunk_pair = [&](int k) {  // index of the half2 holding K values k, k + 1 (k even)
-            const int t = k >> 4, kb = (k >> 3) & 1, e = k & 7;
-            return (((blk * 16 + t) * 64 + r + 32 * kb) * 8 + e) >> 1;
-        };
-        qa2[chunk_pair(2 * lane)] = __halves2half2(__float2half_rn(y0), __float2half_rn(y1));
-        qa2[chunk_pair(128 + 2 * lane)] = __halves2half2(__float2half_rn(p0[i]), __float2half_rn(p1[i]));
+    for (int e = 0; e < 16; ++e) rot[e] = prj[e] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const half8_t wr = __builtin_bit_cast(half8_t, fr[t * 64]);
+        const half8_t wh = __builtin_bit_cast(half8_t, fr[SET + t * 64]);
+        const half8_t wl = __builtin_bit_cast(half8_t, fr[2 * SET + t * 64]);
+        rot = __builtin_amdgcn_mfma_f32_32x32x16_f16(wr, xh[t], rot, 0, 0, 0);
+        prj = __builtin_amdgcn_mfma_f32_32x32x16_f16(wl, xh[t], prj, 0, 0, 0);
+        if constexpr (SPLIT) {
+            rot = __builtin_amdgcn_mfma_f32_32x32x16_f16(wr, xl[t], rot, 0, 0, 0);
+            prj = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh, xl[t], prj, 0, 0, 0);
+        }
+        prj = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh, xh[t], prj, 0, 0, 0);
     }
+    // operand-major layout: the 16-byte chunk (row r of query block v / 32, K values 16t + 8kb .. + 7) that
+    // lane r + 32kb of the score tile's MFMA reads in K step t sits at chunk index (block * 16 + t) * 64 + r + 32kb,
+    // so one wave-wide operand load is 1 KB of contiguous memory.  Register group j of this lane holds outputs
+    // 32w + 8j + 4kb + i, i = 0..3: elements 4kb .. 4kb+3 of the chunk of step (32w + 8j) / 16, half (j & 1).
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int o = 128 * part + 32 * w + 8 * j;  // first K value of the chunk
+            const int t = o >> 4, half_sel = (o >> 3) & 1;
+            const float sc = part == 0 ? RSQRT128 : 1.0f;
+            const float16_t &a = part == 0 ? rot : prj;
+            const __half2 lo2 = __halves2half2(__float2half_rn(a[4 * j] * sc), __float2half_rn(a[4 * j + 1] * sc));
+            const __half2 hi2 = __halves2half2(__float2half_rn(a[4 * j + 2] * sc), __float2half_rn(a[4 * j + 3] * sc));
+            uint2 u;
+            u.x = *reinterpret_cast<const uint32_t *>(&lo2);
+            u.y = *reinterpret_cast<const uint32_t *>(&hi2);
+            *reinterpret_cast<uint2 *>(qa + (((blk * 16 + t) * 64 + r + 32 * half_sel) * 8 + 4 * kb)) = u;
+        }
 }
 
 // One workgroup of eight wavefronts per 256 keys: dequantise them once into LDS as fp16
@@ -1239,32 +1249,42 @@ constexpr int SCORE_KEYS = 256;  // keys per workgroup (two 128-row blocks)
 template <int BITS, typename TO, bool PAIRS, bool DRAIN>
 __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
                                                       const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
-                                                      const float *cent, float proj_scale) {
-    extern __shared__ _Float16 kt[];  // [SCORE_KEYS][KT_STRIDE]
-    __shared__ float cent_s[16];
+                                                      const uint32_t *pair_lut, float proj_scale) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 kt[];  // [SCORE_KEYS][KT_STRIDE]
+    __shared__ uint32_t ptab[1 << (2 * BITS)];  // pair code -> (c[lo], c[hi]) as two halves
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int64_t key0 = (int64_t)blockIdx.x * SCORE_KEYS;
-    if (tid < (1 << BITS)) cent_s[tid] = cent[tid];
+    if (tid < (1 << (2 * BITS))) ptab[tid] = pair_lut[tid];
     __syncthreads();
     {
+        // threads 0..255 dequantise the codes of one key each, threads 256..511 its sign bits; eight halves
+        // (16 bytes) per LDS write
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
         const int key = tid & (SCORE_KEYS - 1), part = tid >> 8;
-        _Float16 *row = kt + key * KT_STRIDE;
+        uint4 *row = reinterpret_cast<uint4 *>(kt + key * KT_STRIDE) + part * 16;
         const bool valid = key0 + key < nk;
         if (part == 0) {
             if (valid) {
                 const uint8_t *block = packed + (key0 + key) / TQ_ROWS_PER_BLOCK * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
                 uint32_t wv[4 * BITS];
                 load_row<BITS>(block, key & (TQ_ROWS_PER_BLOCK - 1), wv);
-                const float g = __half2float(reinterpret_cast<const __half *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key & (TQ_ROWS_PER_BLOCK - 1)]);
+                const _Float16 g = __builtin_bit_cast(
+                    _Float16, reinterpret_cast<const unsigned short *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key & (TQ_ROWS_PER_BLOCK - 1)]);
+                const half2_t g2 = {g, g};
 #pragma unroll
-                for (int p = 0; p < 64; ++p) {
-                    const uint32_t pc = pair_off<BITS>(wv, p) >> 2;
-                    row[2 * p] = (_Float16)(cent_s[pc & ((1u << BITS) - 1u)] * g);
-                    row[2 * p + 1] = (_Float16)(cent_s[pc >> BITS] * g);
+                for (int c = 0; c < 16; ++c) {
+                    uint32_t u[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t e = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(ptab) +
+                                                                               pair_off<BITS>(wv, 4 * c + i));
+                        u[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, e) * g2);
+                    }
+                    row[c] = make_uint4(u[0], u[1], u[2], u[3]);
                 }
             } else {
 #pragma unroll
-                for (int p = 0; p < 128; ++p) row[p] = (_Float16)0.0f;
+                for (int c = 0; c < 16; ++c) row[c] = make_uint4(0, 0, 0, 0);
             }
         } else {
             float rs = 0.f;
@@ -1274,9 +1294,19 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
                 sb = *reinterpret_cast<const uint4 *>(sign_bits + (key0 + key) * 16);
             }
             const uint32_t sw[4] = {sb.x, sb.y, sb.z, sb.w};
-            const _Float16 pos = (_Float16)rs, neg = (_Float16)(-rs);
+            // +rs where the bit is set, -rs where it is clear: two halves per word, the sign bits from the inverted bits
+            const uint32_t mag = (uint32_t)__half_as_ushort(__float2half_rn(rs)) * 0x00010001u;
 #pragma unroll
-            for (int jj = 0; jj < 128; ++jj) row[128 + jj] = ((sw[jj >> 5] >> (jj & 31)) & 1u) ? pos : neg;
+            for (int c = 0; c < 16; ++c) {
+                uint32_t u[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int jj = 8 * c + 2 * i;  // sign bits jj, jj + 1
+                    const uint32_t nb = ~sw[jj >> 5] >> (jj & 31);
+                    u[i] = mag ^ (((nb & 1u) << 15) | ((nb & 2u) << 30));
+                }
+                row[c] = make_uint4(u[0], u[1], u[2], u[3]);
+            }
         }
     }
     __syncthreads();
@@ -1465,11 +1495,12 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
         return TQ_ERR_UNSUPPORTED;
     }
     __half *qa = reinterpret_cast<__half *>(ws);
-    const unsigned qgrid = (unsigned)((nq + 4 * PREP_Q - 1) / (4 * PREP_Q));
+    const unsigned qgrid = (unsigned)((nq + 31) / 32);
+    const uint4 *wfrag = reinterpret_cast<const uint4 *>(h->score_wfrag);
     switch (q_dtype) {
-    case TQ_F16: k_prep_score_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
-    case TQ_F32: k_prep_score_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
-    case TQ_F64: k_prep_score_q<double><<<qgrid, 256, 0, s>>>((const double *)q, qa, nq, h->s1_32, h->s2_32, h->projT32); break;
+    case TQ_F16: k_prep_score_q<__half><<<qgrid, 256, 0, s>>>((const __half *)q, qa, nq, wfrag); break;
+    case TQ_F32: k_prep_score_q<float><<<qgrid, 256, 0, s>>>((const float *)q, qa, nq, wfrag); break;
+    case TQ_F64: k_prep_score_q<double><<<qgrid, 256, 0, s>>>((const double *)q, qa, nq, wfrag); break;
     default: tq_set_error("bad q dtype %d", q_dtype); return TQ_ERR_ARG;
     }
     int rc = tq_check_launch("prep_score_q");
@@ -1481,7 +1512,7 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
         (void)hipFuncSetAttribute((const void *)k_score_tile<B, T, P, DR>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                   (int)lds);                                                                           \
         k_score_tile<B, T, P, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
-                                                         nq, nk, (T *)logits, h->centroids32, (float)h->proj_scale);   \
+                                                         nq, nk, (T *)logits, (const uint32_t *)h->pair_lut, (float)h->proj_scale);   \
     }
 #define TQ_SCORE_BITS(T, P, DR)                                                                              \
     if (h->bits == 2) TQ_SCORE(2, T, P, DR) else if (h->bits == 3) TQ_SCORE(3, T, P, DR) else TQ_SCORE(4, T, P, DR)

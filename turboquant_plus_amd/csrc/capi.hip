@@ -32,6 +32,14 @@ uint16_t f64_to_f16_bits(double v) {
     return sign | (uint16_t)bits;
 }
 
+double f16_bits_to_f64(uint16_t b) {
+    const double sign = (b & 0x8000) ? -1.0 : 1.0;
+    const int e = (b >> 10) & 31, m = b & 1023;
+    if (e == 0) return sign * std::ldexp((double)m, -24);
+    if (e == 31) return m ? NAN : sign * INFINITY;
+    return sign * std::ldexp(1.0 + m / 1024.0, e - 15);
+}
+
 template <typename T> int upload(T **dst, const std::vector<T> &src) {
     *dst = nullptr;
     if (src.empty()) return TQ_OK;
@@ -281,7 +289,6 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         if (cfg->projection) {
             // M = S R^T with R[k][m] = s2[k] H[k][m] s1[m] / sqrt(128); stored as [k*128+j] = M[j][k]
             std::vector<double> mt((size_t)128 * 128);
-            std::vector<float> pT((size_t)128 * 128);
             const double rs = 1.0 / std::sqrt(128.0);
             for (int j = 0; j < 128; ++j)
                 for (int k = 0; k < 128; ++k) {
@@ -291,10 +298,27 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                         acc += S[(size_t)j * 128 + m] * (s2[k] * hkm * s1[m]);
                     }
                     mt[(size_t)k * 128 + j] = acc * rs;
-                    pT[(size_t)k * 128 + j] = (float)S[(size_t)j * 128 + k];
                 }
             rc = rc ? rc : upload(&h->projrot64_t, mt);
-            rc = rc ? rc : upload(&h->projT32, pT);
+            // Operand fragments of the query preparation (score tile): W = [D2 H D1 ; S] as the row side of
+            // 32 x 32 x 16 matrix instructions.  Set 0: the rotation's +-1 entries (its 1/sqrt(128) is applied to the
+            // sums), sets 1 and 2: S split into two fp16 terms (S = hi + lo to 2^-22).  Fragment (row block cb, step
+            // t), lane l, element e = W[32 cb + l % 32][16 t + 8 (l / 32) + e].
+            std::vector<uint16_t> wf((size_t)3 * 4 * 8 * 64 * 8);
+            for (int cb = 0; cb < 4; ++cb)
+                for (int t = 0; t < 8; ++t)
+                    for (int l = 0; l < 64; ++l)
+                        for (int e = 0; e < 8; ++e) {
+                            const int j = 32 * cb + (l & 31), k = 16 * t + 8 * (l >> 5) + e;
+                            const size_t at = ((((size_t)cb * 8 + t) * 64) + l) * 8 + e, set = (size_t)4 * 8 * 64 * 8;
+                            const double r = s2[j] * ((__builtin_popcount(j & k) & 1) ? -1.0 : 1.0) * s1[k];
+                            wf[at] = r < 0 ? 0xBC00 : 0x3C00;
+                            const double sv = S[(size_t)j * 128 + k];
+                            const uint16_t hi = f64_to_f16_bits(sv);
+                            wf[set + at] = hi;
+                            wf[2 * set + at] = f64_to_f16_bits(sv - f16_bits_to_f64(hi));
+                        }
+            rc = rc ? rc : upload(&h->score_wfrag, wf);
         }
     }
     if (rc) {
@@ -308,7 +332,7 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
 void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
-                    h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->projT32,
+                    h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->score_wfrag,
                     h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v, h->quant_lut,
                     h->rfrag16k_inv};
     for (void *p : ptrs)
