@@ -1419,26 +1419,50 @@ struct StoreQjlArgs {
     int64_t tokens, blocks_per_seq;
 };
 
-// One workgroup of eight wavefronts per CU, looping over 128-token blocks, with the projection (S R^T, 128 KB
-// of doubles) resident in LDS; a wavefront takes 16 tokens of the block, lane (token n16, quarter kq) holding
-// the 32 dims d = 4 s + kq: norms and the first two butterfly stages (in the reference's stage order) exchange
-// across the lane quarters, the other five stages are in-lane, and the residual in the rotated domain, taken
-// against the reconstruction the decoder will see (stored fp16 norm), is at once the A operand of
-// v_mfma_f64_16x16x4_f64: 256 of them per 16 tokens against the matrix in LDS.  The sign bits of a token's 16
-// projections of one column block are one quarter of a ballot.
+// One workgroup of eight wavefronts per CU with the projection (S R^T, 128 KB of doubles) resident in LDS.  The
+// wavefronts are independent after the matrix is in place: each takes units of 16 tokens (a strided share), lane
+// (token n16, quarter kq) holding the 32 dims d = 4 s + kq.  Norms and the first two butterfly stages (in the
+// reference's stage order) exchange across the lane quarters, the other five stages are in-lane, and the residual
+// in the rotated domain, taken against the reconstruction the decoder will see (stored fp16 norm), is at once the
+// A operand of v_mfma_f64_16x16x4_f64: 256 of them per unit against the matrix in LDS.  No barrier ties the
+// wavefronts together, and the next unit's input is requested before the matrix phase starts.  The sign bits of a
+// token's 16 projections of one column block are one quarter of a ballot.  A wavefront packs its own 16 rows (rows
+// of a K block are independent).
+// Matrix rows k and k + 1 hold their 16-column groups in swapped order (column j of row k at j ^ 16 (k & 1)): the
+// two lane quarters that share a pass of an 8-byte LDS read then hit different halves of the banks.
+// (Float64 matrix instructions and float64 vector instructions do not overlap on this chip: staggering the two
+// wavefronts of a SIMD so that one's vector phase falls into the other's matrix phase gains nothing, measured.)
 typedef double double4_t __attribute__((ext_vector_type(4)));
 template <int BITS, typename TI>
 __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *packed, uint8_t *sign_bits, __half *rnorms,
                                                        StoreQjlArgs a, int64_t n_blocks) {
     using namespace tq64;
     constexpr int NB = (1 << BITS) - 1;
-    extern __shared__ double mat_s[];  // [k][j] = (S R^T)[j][k]
-    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
-    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
-    __shared__ double cent_s[1 << BITS], bnd_s[1 << BITS];
+    extern __shared__ double mat_s[];  // [k][j ^ 16 (k & 1)] = (S R^T)[j][k]
+    __shared__ __attribute__((aligned(16))) uint8_t codes_s[8][16 * CODE_STRIDE];
+    __shared__ double cent_s[1 << BITS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kq = lane >> 4;
+    uint8_t *codes = codes_s[wave];
+
+    const int64_t n_units = n_blocks * 8;
+    const int64_t unit_step = (int64_t)gridDim.x * 8;
+    int64_t unit = (int64_t)blockIdx.x * 8 + wave;
+    // this lane's 32 inputs of a unit, as stored (converted when the unit is processed)
+    TI xin[32];
+    bool xvalid = false;
+    auto fetch = [&](int64_t un) {
+        const int64_t blk = un >> 3;
+        const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
+        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + (un & 7) * 16 + n16;
+        xvalid = un < n_units && tok < a.tokens;
+        const TI *src = x + (seq * a.tokens + (xvalid ? tok : 0)) * 128 + kq;
+        if (un >= n_units) src = x + kq;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) xin[s] = src[4 * s];
+    };
+    fetch(unit);
 
     // the matrix is fetched once per workgroup, sixteen 16-byte pieces per thread, eight in flight at a time
 #pragma unroll
@@ -1447,10 +1471,17 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
 #pragma unroll
         for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const double2 *>(a.projrot_t)[tid + 512 * (8 * b + i)];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) reinterpret_cast<double2 *>(mat_s)[tid + 512 * (8 * b + i)] = piece[i];
+        for (int i = 0; i < 8; ++i) {
+            const int pi = tid + 512 * (8 * b + i);  // row pi / 64, columns 2 (pi % 64), + 1
+            reinterpret_cast<double2 *>(mat_s)[pi ^ (((pi >> 6) & 1) << 3)] = piece[i];
+        }
     }
     if (tid < (1 << BITS)) cent_s[tid] = a.cent[tid];
-    if (tid < NB) bnd_s[tid] = a.bounds[tid];
+    // the boundaries stay in registers (the byte stores of the code stage may alias anything as far as the compiler
+    // knows, so boundaries kept in LDS were read again for every value)
+    double bnd[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) bnd[k] = a.bounds[k];
     uint32_t neg1 = 0, neg2 = 0;  // bit s: s1 / s2 of dim 4 s + kq is -1
 #pragma unroll
     for (int s = 0; s < 32; ++s) {
@@ -1461,24 +1492,24 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
     // one reciprocal instead of 32 divisions per token, and 1 / sqrt(128) as a factor: at most one unit in the
     // last place away from the quotients, far inside the 1e-6 band the codes and signs are held to
     const double inv_rn = 1.0 / sqrt(128.0);
+    auto quarter_sum = [&](double v) {
+        v += xor_lane<16>(v);
+        v += xor_lane<32>(v);
+        return v;
+    };
 
 #pragma unroll 1
-    for (int64_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
-    const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
-    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
-    const int64_t row0 = seq * a.tokens;
-    {
-        const int u = wave;  // eight wavefronts, 16 tokens each
+    for (; unit < n_units; unit += unit_step) {
+        const int64_t blk = unit >> 3;
+        const int u = (int)(unit & 7);
+        const int64_t seq = blk / a.blocks_per_seq, bis = blk % a.blocks_per_seq;
+        const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+        const int64_t row0 = seq * a.tokens;
         const int t = u * 16 + n16;
-        const bool valid = tok0 + t < a.tokens;
+        const bool valid = xvalid;
         double e[32];
 #pragma unroll
-        for (int s = 0; s < 32; ++s) e[s] = valid ? ldd(x, (row0 + tok0 + t) * 128 + 4 * s + kq) : 0.0;
-        auto quarter_sum = [&](double v) {
-            v += xor_lane<16>(v);
-            v += xor_lane<32>(v);
-            return v;
-        };
+        for (int s = 0; s < 32; ++s) e[s] = valid ? ldd(xin, s) : 0.0;
         double ss = 0.0;
 #pragma unroll
         for (int s = 0; s < 32; ++s) ss = fma(e[s], e[s], ss);
@@ -1510,35 +1541,64 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
                     e[s + hb] = p - q;
                 }
         uint32_t cw[4] = {0u, 0u, 0u, 0u};  // the 32 codes, 4 bits each
-        double cs = 0.0;
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
             double yv = e[s] * inv_rn;
             if ((neg2 >> s) & 1u) yv = -yv;
             e[s] = yv;
-            int c = 0;
+            uint32_t c = 0;
 #pragma unroll
-            for (int k = 0; k < NB; ++k) c += (bnd_s[k] < yv) ? 1 : 0;
-            codes[t * CODE_STRIDE + 4 * s + kq] = (uint8_t)c;
-            cw[s >> 3] |= (uint32_t)c << (4 * (s & 7));
-            const double cv = cent_s[c];
-            cs = fma(cv, cv, cs);
+            for (int k = 0; k < NB; ++k) c += (bnd[k] < yv) ? 1u : 0u;
+            cw[s >> 3] |= c << (4 * (s & 7));
+        }
+        // the code stage takes the lane's codes as bytes (dim 4 s + kq of token n16)
+#pragma unroll
+        for (int s = 0; s < 32; ++s) codes[n16 * CODE_STRIDE + 4 * s + kq] = (uint8_t)((cw[s >> 3] >> (4 * (s & 7))) & 15u);
+        double cv[32];
+        double cs = 0.0;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            cv[s] = cent_s[(cw[s >> 3] >> (4 * (s & 7))) & 15u];
+            cs = fma(cv[s], cv[s], cs);
         }
         const double cn = sqrt(quarter_sum(cs));
         double g = nrm;
         if (a.norm_correction) g = nrm / (cn > 1e-10 ? cn : 1.0);
         const __half gh = double_to_half_rn(g);
         const double g16 = (double)__half2float(gh);
-        if (kq == 0) norms_s[t] = __half2float(gh);
+        uint8_t *block = packed + blk * block_bytes(BITS);
+        if (kq == 0) reinterpret_cast<__half *>(block + block_code_bytes(BITS))[t] = gh;
         // residual in the rotated domain against the reconstruction the decoder will see
         double rs = 0.0;
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
-            e[s] = nrm * e[s] - g16 * cent_s[(cw[s >> 3] >> (4 * (s & 7))) & 15u];
+            e[s] = nrm * e[s] - g16 * cv[s];
             rs = fma(e[s], e[s], rs);
         }
         const double rnorm = sqrt(quarter_sum(rs));
         if (valid && kq == 0) rnorms[row0 + tok0 + t] = double_to_half_rn(rnorm);
+        // the wavefront's 16 rows of the block: chunk c, row r = lane / 4, dword k = lane % 4 (pack_block's word)
+        __builtin_amdgcn_wave_barrier();
+        {
+            constexpr int PER = pairs_per_dword(BITS);
+            const int r = lane >> 2, k = lane & 3;
+#pragma unroll
+            for (int c = 0; c < BITS; ++c) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int i = 0; i < PER; ++i) word |= pair_from_stage<BITS>(codes, TQ_KIND_K, r, 16 * k + PER * c + i) << (2 * BITS * i);
+                if constexpr (BITS == 3) {
+                    uint32_t tail = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) tail |= pair_from_stage<3>(codes, TQ_KIND_K, r, 16 * k + 12 + i) << (6 * i);
+                    word |= ((tail >> (8 * c)) & 0xFFu) << 24;
+                }
+                reinterpret_cast<uint32_t *>(block)[c * 512 + (u * 16 + r) * 4 + k] = word;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        // the next unit's input is under way while the matrix phase runs
+        fetch(unit + unit_step);
         // (S R^T) e for the 16 tokens: D[token][j] += E[token][k] M[k][j], 8 column blocks x 32 steps of 4
         double4_t acc[8];
 #pragma unroll
@@ -1547,7 +1607,8 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
         for (int s = 0; s < 32; ++s) {
             const double *mrow = mat_s + (4 * s + kq) * 128 + n16;
 #pragma unroll
-            for (int jb = 0; jb < 8; ++jb) acc[jb] = __builtin_amdgcn_mfma_f64_16x16x4f64(e[s], mrow[16 * jb], acc[jb], 0, 0, 0);
+            for (int jb = 0; jb < 8; ++jb)
+                acc[jb] = __builtin_amdgcn_mfma_f64_16x16x4f64(e[s], mrow[16 * (jb ^ (kq & 1))], acc[jb], 0, 0, 0);
         }
         // lane (n16, kq) now holds the projections j = 16 jb + n16 of tokens 4 i + kq (register i of the result)
 #pragma unroll
@@ -1561,10 +1622,6 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
             const int64_t tk = tok0 + u * 16 + 4 * i + kq;
             if (n16 < 8 && tk < a.tokens) reinterpret_cast<uint16_t *>(sign_bits)[(row0 + tk) * 8 + n16] = (uint16_t)piece;
         }
-    }
-    __syncthreads();
-    pack_block<BITS, 512>(codes, norms_s, packed + blk * block_bytes(BITS), TQ_KIND_K);
-    __syncthreads();  // the code stage is free for the next block
     }
 }
 
