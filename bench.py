@@ -245,7 +245,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                      "traffic": TRAFFIC_BYTES["decode3"], "traffic_source": TRAFFIC_SOURCE["decode3"],
                      "algorithmic_bytes_per_step": algo,
-                     "kernel": "k_decode_attn<turbo3,turbo3> (+ k_attn_combine in the step time)"},
+                     "kernel": "k_decode_attn<turbo3,turbo3> (one launch: the last workgroup of a group merges the partials)"},
         "buffer_sets": n_sets,
         "gqa8": {"workload": "the same cache, 64 query heads on 8 KV heads (eight heads per pass over K/V)",
                  "us_per_step": ev8_ms * 1e3, "n_splits": attn8.params.n_splits,
