@@ -44,13 +44,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 D = 128
-# HBM bytes per launch as recorded in profiles/bench_kernels_c2_c3.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
-# this file's default run, each scaled by the reading of a 1 GiB device copy): recorded constants, not measured in
-# this run; the JSON line names the profile row next to each figure.
-TRAFFIC_BYTES = {"store4": 171.5e6, "store3": 161.8e6, "decode3": 423.5e6}
-TRAFFIC_SOURCE = {"store4": "profiles/bench_kernels_c2_c3.txt, rows k_store_kv<4,4> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)",
-                  "store3": "profiles/bench_kernels_c2_c3.txt, rows k_store_kv<3,3> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)",
-                  "decode3": "profiles/bench_kernels_c2_c3.txt, rows k_decode_attn<turbo3,turbo3> FETCH_SIZE + WRITE_SIZE (recorded, not measured in this run)"}
+# HBM bytes per launch as recorded in profiles/bench_all_legs_trace_hbm_sq.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
+# this file's run, each scaled by the reading of a 1 GiB device copy): recorded constants, not measured in this run;
+# the JSON line names the profile row next to each figure.
+TRAFFIC_BYTES = {"store4": 179.0e6, "store3": 170.8e6, "decode3": 443.9e6}
+_TRAFFIC_FILE = "profiles/bench_all_legs_trace_hbm_sq.txt"
+TRAFFIC_SOURCE = {"store4": _TRAFFIC_FILE + ", row k_store_kv<4, 4, false> of the HBM traffic table (recorded, not measured in this run)",
+                  "store3": _TRAFFIC_FILE + ", row k_store_kv<3, 3, false> of the HBM traffic table (recorded, not measured in this run)",
+                  "decode3": _TRAFFIC_FILE + ", row k_decode_attn<0, 3, 3, false, true, 1> of the HBM traffic table (recorded, not measured in this run)"}
 METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
 
 
