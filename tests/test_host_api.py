@@ -44,9 +44,14 @@ def test_size_entry_points_need_no_gpu():
     assert lib.tq_q8_0_bytes(1, 128) == 128 * 136
     p = L.TQAttnParams(batch=16, n_q_heads=32, n_kv_heads=8, tokens=32768, n_splits=16,
                        k_format=L.KFMT_TURBO, scale=0.088, sparse_v_tau=0.0)
-    assert lib.tq_attn_workspace_bytes(C.byref(p)) > 16 * 8 * 16 * 4 * 128 * 4
+    # one partial (four heads x (128 outputs + maximum + sum)) per workgroup, and the 16 splits of a group are one workgroup
+    one_per_group = 16 * 8 * 4 * 130 * 4
+    assert one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 2 * one_per_group
     p.n_q_heads = 16                                       # groups of 2: two of the four head rows per pass idle
-    assert lib.tq_attn_workspace_bytes(C.byref(p)) > 16 * 8 * 16 * 4 * 128 * 4
+    assert one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 2 * one_per_group
+    p.n_q_heads, p.n_splits = 64, 32                       # groups of 8: eight heads per pass, eight wavefronts per workgroup
+    assert 4 * 2 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 4 * 2 * one_per_group + 65536
+    p.n_splits = 16
     p.n_q_heads = 20                                       # not a multiple of the KV head count
     assert lib.tq_attn_workspace_bytes(C.byref(p)) == -1
     assert "multiple of the KV head count" in L.last_error()
