@@ -532,7 +532,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
             ss = diag_here ? ss : 0.0f;
             cur[r] = next;
-            fetch(next, xb, xvalid[r]);
+            if (next < end) fetch(next, xb, xvalid[r]);  // nothing is requested past the share
             ss += xor_lane<16>(ss);
             ss += xor_lane<32>(ss);
             const float norm = __builtin_amdgcn_sqrtf(ss);  // 1 ulp: scales boundaries (1e-7 relative) and the stored fp16 norm
@@ -909,7 +909,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                                                               gram, 0, 0, 0);
 #endif
             if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-            else fetch(next, 5 - q, xb, xvalid[q & 1]);
+            else if (next < end) fetch(next, 5 - q, xb, xvalid[q & 1]);  // nothing is requested past the share
 
             float nrm[4];
             float4_t inv;
