@@ -594,9 +594,12 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     float bias_next[HG][4];
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
-    unsigned nskip = 0;
+    unsigned nskip = 0;  // Sparse V: skipped (query, position) pairs of this wavefront (wave-uniform: counted from lane masks)
     bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
+    unsigned long long head_ok[HG];  // lanes whose head (lane % 4 of each set) exists in this pass
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) head_ok[hg] = __builtin_amdgcn_ballot_w64(a.head_off + 4 * hg + j < a.q_group);
 #pragma unroll 1
     while (tile < t_end) {
         const int64_t blk = tile >> 1;
@@ -661,7 +664,15 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         }
         // -> lane (b, j): head j (of each set), tokens 4b..4b+3; then the online softmax in base 2
         float p[HG][4];
-        bool any_keep = false;
+        // Sparse V bookkeeping on the scalar unit: a compare leaves a lane mask, and counting, the in-range test and
+        // "does any lane keep anything" are mask arithmetic (the vector ALU only compares and zeroes the weight)
+        unsigned long long any_keep = 0, token_ok[4] = {~0ull, ~0ull, ~0ull, ~0ull};
+        if constexpr (SPARSE) {
+            if (n_valid < 64) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) token_ok[i] = __builtin_amdgcn_ballot_w64(b4 + i < n_valid);
+            }
+        }
 #pragma unroll
         for (int hg = 0; hg < HG; ++hg) {
             quad_transpose(sc[hg], lane);
@@ -696,18 +707,19 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
                 p[hg][i] = __builtin_amdgcn_exp2f(s[i] - m_ref);  // results below 2^-126 flush to zero
                 l_run[hg] += p[hg][i];
                 if constexpr (SPARSE) {
-                    const bool in_range = b4 + i < n_valid && a.head_off + 4 * hg + j < a.q_group;
                     const bool keep = p[hg][i] >= a.tau;
-                    if (in_range && !keep) ++nskip;
+                    const unsigned long long keep_m = __builtin_amdgcn_ballot_w64(keep);
+                    const unsigned long long in_range = token_ok[i] & head_ok[hg];
+                    nskip += (unsigned)__builtin_popcountll(in_range & ~keep_m);
                     if (!keep) p[hg][i] = 0.0f;
-                    any_keep |= keep && in_range;
+                    any_keep |= keep_m & in_range;
                 }
             }
         }
         if constexpr (SPARSE) {
             // Every V row of the tile skipped: no dequant, and the next tile's V row is not requested in
             // advance (negligible weights come in runs); a tile that then does need its row fetches it here.
-            if (__builtin_amdgcn_ballot_w64(any_keep) == 0) {
+            if (any_keep == 0) {
                 gvu = gvu_next;
                 tile = tile_next;
                 v_ahead = false;
@@ -846,9 +858,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     if constexpr (SPARSE) {
         // one slot per workgroup, added up by the merge kernel: thousands of wavefronts finishing together
         // on one atomic would queue for longer than the kernel's own tail, and nothing needs clearing
-        unsigned tot = nskip;
-        for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
-        if (lane == 0 && tot) atomicAdd(&skipped, tot);
+        if (lane == 0 && nskip) atomicAdd(&skipped, nskip);
         __syncthreads();
         if (tid == 0) st_dev(a.skip_slots + blockIdx.x, (a.nonce & ~SKIP_COUNT_MASK) | (unsigned long long)skipped);
     }
