@@ -1356,16 +1356,20 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
     // operand is the lane's place relative to that row (one register for the whole kernel): rows past the last
     // query fall outside the resource and the hardware drops them, lanes whose key does not exist get an offset
     // outside every resource, and no store needs an address register or a branch.
-    constexpr bool PAIRED = sizeof(TO) == 2 && PAIRS;  // fp16: two logits per store
-    constexpr int N_GROUPS = PAIRED ? 16 : 32;         // store instructions per block
+    constexpr bool PAIRED = sizeof(TO) == 2 && PAIRS;  // fp16: two logits per lane and store, whole 128-byte lines
+    constexpr int N_GROUPS = PAIRED ? 16 : 32;         // store groups per block
     constexpr int NT_AUX = (TQ_STREAM_SITES & STREAM_LOGITS) ? 2 : 0;  // the non-temporal bit of a buffer instruction
     constexpr uint32_t DROPPED = 0x80000000u;          // beyond any resource (the launcher keeps 64 rows below 2 GiB)
     const uint32_t row_bytes = (uint32_t)nk * (uint32_t)sizeof(TO);
     const bool odd = lane & 1;
-    // paired: even lanes store rows 8j + 4kb + h, odd lanes rows 8j + 4kb + 2 + h, keys (c32 & ~1, c32 | 1)
-    const uint32_t lane_bytes = (uint32_t)(4 * kb) * row_bytes +
-                                (PAIRED ? (odd ? 2u * row_bytes + (uint32_t)(c32 - 1) * 2u : (uint32_t)c32 * 2u)
-                                        : (uint32_t)c32 * (uint32_t)sizeof(TO));
+    // Paired fp16: two neighbouring 32-key sub-blocks leave together.  A lane packs two logits (keys c32 & ~1, c32 | 1;
+    // even lanes rows 8j + 4kb + h, odd lanes rows 8j + 4kb + 2 + h, by trading with the neighbouring lane), the packed
+    // words of the first sub-block wait in 16 registers, and when the second is packed one v_permlane32_swap per
+    // register puts the first sub-block's words of the rows kb = 0 into lanes 0..31 and the second's into lanes
+    // 32..63 (and likewise for kb = 1), so that a store instruction writes 64 consecutive logits = one whole
+    // 128-byte line of each of two rows.  The lane's place: (its parity's row, its half's sub-block, its key pair).
+    const uint32_t lane_bytes = PAIRED ? (odd ? 2u * row_bytes : 0u) + (uint32_t)kb * 64u + (uint32_t)(c32 & ~1) * 2u
+                                       : (uint32_t)(4 * kb) * row_bytes + (uint32_t)c32 * (uint32_t)sizeof(TO);
     struct Pending {
         TO *base[2];        // first logit of the two 32-row blocks
         int rows[2];        // rows of each that exist (0: nothing is pending)
@@ -1387,36 +1391,51 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
             pb.base[mb] = reinterpret_cast<TO *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
                                                  (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
         }
-        const int64_t first_key = key0 + ks * 32 + (PAIRED ? (c32 & ~1) : c32);  // paired: the key count is even
+        // paired: ks is the first sub-block of the pair, lanes 32..63 hold the second one's keys; the key count is even
+        const int64_t first_key = key0 + ks * 32 + (PAIRED ? 32 * kb + (c32 & ~1) : c32);
         pb.voff = first_key < nk ? lane_bytes : DROPPED;
         return pb;
     };
-    // store group n of a pending block: unpaired, accumulator element n % 16 of row block n / 16 (rows 8j + 4kb + i,
-    // e = 4j + i); paired, rows 8j + 4kb + {h, 2 + h} of row block n / 8, j = (n % 8) / 2, h = n % 2
+    // store group n of a pending block, unpaired: accumulator element n % 16 of row block n / 16 (rows 8j + 4kb + i,
+    // e = 4j + i)
     auto store_group = [&](const Pending &pb, const float16_t (&acc)[2], const int n) __attribute__((always_inline)) {
-        const int mb = PAIRED ? n >> 3 : n >> 4;
-        const int row = PAIRED ? 8 * ((n >> 1) & 3) + (n & 1) : 8 * ((n & 15) >> 2) + (n & 3);  // of lane half kb = 0
+        const int mb = n >> 4;
+        const int row = 8 * ((n & 15) >> 2) + (n & 3);  // of lane half kb = 0
         const int left = max(pb.rows[mb] - row, 0);
         const __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc(pb.base[mb] + (int64_t)row * nk, 0, (int)((uint32_t)left * row_bytes), 0x00020000);
-        if constexpr (PAIRED) {
-            // neighbouring lanes (keys c32, c32 ^ 1) trade two of their four rows
-            const int j = (n >> 1) & 3, h = n & 1;
-            const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
-            const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
-            const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;
-            const uint32_t u = (uint32_t)__half_as_ushort(__float2half_rn(v0)) | ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
-            __builtin_amdgcn_raw_buffer_store_b32(u, rs, (int)pb.voff, 0, NT_AUX);
-        } else if constexpr (sizeof(TO) == 4) {
+        if constexpr (sizeof(TO) == 4) {
             __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mb][n & 15]), rs, (int)pb.voff, 0, NT_AUX);
         } else {
             __builtin_amdgcn_raw_buffer_store_b16(__half_as_ushort(__float2half_rn(acc[mb][n & 15])), rs, (int)pb.voff, 0, NT_AUX);
         }
     };
+    // paired: group n = rows 8j + 4kb + {h, 2 + h} of row block n / 8, j = (n % 8) / 2, h = n % 2, as two packed halves
+    auto pack_group = [&](const float16_t (&acc)[2], const int n) __attribute__((always_inline)) -> uint32_t {
+        const int mb = n >> 3, j = (n >> 1) & 3, h = n & 1;
+        const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
+        const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
+        const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;  // keys (c32 & ~1), (c32 | 1)
+        return (uint32_t)__half_as_ushort(__float2half_rn(v0)) | ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
+    };
+    // paired: group n of a pair of sub-blocks (first sub-block's packed word, second's) -> two stores of two lines each
+    auto store_pair_group = [&](const Pending &pb, const uint32_t first, const uint32_t second, const int n) __attribute__((always_inline)) {
+        const int mb = n >> 3, row = 8 * ((n >> 1) & 3) + (n & 1);
+        const auto r = __builtin_amdgcn_permlane32_swap(first, second, false, false);  // [0]: rows kb = 0, [1]: rows kb = 1
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            const int left = max(pb.rows[mb] - (row + 4 * hi), 0);
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(pb.base[mb] + (int64_t)(row + 4 * hi) * nk, 0,
+                                                                                 (int)((uint32_t)left * row_bytes), 0x00020000);
+            __builtin_amdgcn_raw_buffer_store_b32(r[hi], rs, (int)pb.voff, 0, NT_AUX);
+        }
+    };
+    uint32_t first_packed[PAIRED ? 16 : 1];  // paired: the first sub-block of the pair, packed, waiting for the second
 
     float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
     // one 32-key sub-block against the resident query tile into acc, while the pending block leaves from pacc
-    auto sub_block = [&](const int ks, auto prefetch, auto drain, float16_t (&acc)[2], const float16_t (&pacc)[2],
+    // prev_second (paired fp16): the previous sub-block was the second of its pair
+    auto sub_block = [&](const int ks, auto prefetch, auto drain, auto prev_second, float16_t (&acc)[2], const float16_t (&pacc)[2],
                          const Pending &pb) __attribute__((always_inline)) {
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
@@ -1441,7 +1460,14 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
                 acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[t][mb], kf[t & AHEAD], acc[mb], 0, 0, 0);
                 if constexpr (decltype(drain)::value) {
                     const int n = 2 * t + mb;
-                    if (N_GROUPS == 32 || (n & 1)) store_group(pb, pacc, N_GROUPS == 32 ? n : n >> 1);
+                    if constexpr (!PAIRED) {
+                        store_group(pb, pacc, n);
+                    } else if (n & 1) {
+                        // the previous sub-block is packed; if it was the second of its pair, the pair leaves
+                        const uint32_t u = pack_group(pacc, n >> 1);
+                        if constexpr (decltype(prev_second)::value) store_pair_group(pb, first_packed[n >> 1], u, n >> 1);
+                        else first_packed[n >> 1] = u;
+                    }
                 }
             }
             if constexpr (decltype(prefetch)::value) load_queries(t);
@@ -1460,27 +1486,39 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc_b[mb][e] = 0.0f;
+        if constexpr (PAIRED) {
+#pragma unroll
+            for (int n = 0; n < 16; ++n) first_packed[n] = 0u;
+        }
         Pending pb = pend(0, 0);
         pb.rows[0] = pb.rows[1] = 0;  // nothing is pending before the first block
+        constexpr std::true_type second{};
+        constexpr std::false_type first{};
+        // unpaired: the pending block is the previous sub-block; paired: the previous pair (set when its second ends)
 #pragma unroll 1
         for (int qt = 0; qt < n_qt; ++qt) {
             const int qbase = qt * QT + qh * 64;
             point_queries(min(qt + 1, n_qt - 1));  // the last tile re-reads itself
 #pragma unroll 1
             for (int kp = 0; kp < SCORE_KEYS / 64 - 1; ++kp) {
-                sub_block(2 * kp, std::false_type{}, drain, acc_a, acc_b, pb);
-                pb = pend(qbase, 2 * kp);
-                sub_block(2 * kp + 1, std::false_type{}, drain, acc_b, acc_a, pb);
-                pb = pend(qbase, 2 * kp + 1);
+                sub_block(2 * kp, std::false_type{}, drain, second, acc_a, acc_b, pb);
+                if constexpr (!PAIRED) pb = pend(qbase, 2 * kp);
+                sub_block(2 * kp + 1, std::false_type{}, drain, first, acc_b, acc_a, pb);
+                pb = pend(qbase, PAIRED ? 2 * kp : 2 * kp + 1);
             }
-            sub_block(SCORE_KEYS / 32 - 2, std::false_type{}, drain, acc_a, acc_b, pb);
-            pb = pend(qbase, SCORE_KEYS / 32 - 2);
-            sub_block(SCORE_KEYS / 32 - 1, std::true_type{}, drain, acc_b, acc_a, pb);  // also fetches the next tile's queries
-            pb = pend(qbase, SCORE_KEYS / 32 - 1);
+            sub_block(SCORE_KEYS / 32 - 2, std::false_type{}, drain, second, acc_a, acc_b, pb);
+            if constexpr (!PAIRED) pb = pend(qbase, SCORE_KEYS / 32 - 2);
+            sub_block(SCORE_KEYS / 32 - 1, std::true_type{}, drain, first, acc_b, acc_a, pb);  // also fetches the next tile's queries
+            pb = pend(qbase, PAIRED ? SCORE_KEYS / 32 - 2 : SCORE_KEYS / 32 - 1);
         }
         if constexpr (decltype(drain)::value) {  // the last block (in acc_b)
+            if constexpr (PAIRED) {
 #pragma unroll
-            for (int n = 0; n < N_GROUPS; ++n) store_group(pb, acc_b, n);
+                for (int n = 0; n < 16; ++n) store_pair_group(pb, first_packed[n], pack_group(acc_b, n), n);
+            } else {
+#pragma unroll
+                for (int n = 0; n < N_GROUPS; ++n) store_group(pb, acc_b, n);
+            }
         }
     };
     sweep(std::integral_constant<bool, DRAIN>{});
