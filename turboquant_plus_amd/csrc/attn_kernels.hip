@@ -454,8 +454,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     // the table build overlap the first trip to memory.  Afterwards rows are fetched one tile
     // ahead into the same registers: the next K row right after QK has consumed the current
     // one, the next V row right after PV (with Sparse V only after a tile that used its V row).  After the split's last
-    // tile nothing is requested (a wave-uniform branch: the rows are read with the non-temporal hint, and a clamped
-    // re-read of the last row went to memory again, one row in sixteen at 1024 tokens per split).  The norms
+    // tile the prefetch has every lane read row 0 of that tile's block (a handful of lines, never used): the rows are
+    // read with the non-temporal hint, and a clamped re-read of the last tile's 64 rows went to memory again, one tile
+    // in sixteen at 1024 tokens per split; a branch around the loads cost the eight-head variant 11 us.  The norms
     // travel with the rows, so no load is waited for in the tile that issued it.
     uint32_t kw[KROW_DW];
     uint32_t vw[4 * VBITS];
@@ -617,7 +618,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         }
         const int tile_next = tile + 1;
         const int tile_n = min(tile_next, t_end - 1);
-        const int row_n = (tile_n & 1) * 64 + lane;
+        const int row_n = tile_next < t_end ? (tile_n & 1) * 64 + lane : 0;  // past the split: every lane the same row
         const VSide<VBITS> gvu_next = load_vnorm(tile_n);
         const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
@@ -656,7 +657,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
 #pragma unroll
                 for (int i = 0; i < 4; ++i) sc[hg][i] = (acc[hg][0][i] * d0 + acc[hg][1][i] * d1) + (acc[hg][2][i] * d2 + acc[hg][3][i] * d3);
         }
-        if (tile_next < t_end) {   // kw is dead now: fetch the next tile's K row into it (wave-uniform branch)
+        {   // kw is dead now: fetch the next tile's K row into it
             const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
             if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, row_n, kw);
             else load_row<8>(kbn, row_n, kw);
@@ -779,7 +780,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             // weights of token group T sit in block T and are broadcast to every block.
             pv_all<VBITS, HG>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv, acc_o);
         }
-        if (tile_next < t_end) load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
+        load_row<VBITS>(vbase + (int64_t)(tile_n >> 1) * VBLOCK, row_n, vw);
         v_ahead = true;
         gvu = gvu_next;
         tile = tile_next;

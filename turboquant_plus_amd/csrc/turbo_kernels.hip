@@ -450,6 +450,10 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     // The address is always valid: units past the end and rows past a sequence's last token
     // are clamped, and `valid` says whether the data is to be used.
     auto fetch = [&](uint32_t unit, uint4 (&xb)[4], bool &valid) {
+        // A prefetch past the share (its data is never used) reads the tensor's first bytes, every lane the same
+        // ones: a clamped re-read of the last unit would go to memory again where rows are read with the
+        // non-temporal hint, and a branch around the loads costs registers.
+        const bool beyond = unit > last_unit;
         unit = unit < last_unit ? unit : last_unit;
 #if TQ_KNOCKOUT & 32
         unit = lo + (((unit - lo) / step) & 7u) * step;  // the first eight units of the share over and over: no HBM reads
@@ -460,10 +464,10 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + (unit & 7) * 16 + n16;
             valid = tok < a.tokens;
             tok = valid ? tok : a.tokens - 1;
-            p = reinterpret_cast<const uint4 *>(x + ((int64_t)seq * a.tokens + tok) * 128 + 32 * kc);
+            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)seq * a.tokens + tok) * 128 + 32 * kc));
         } else {
             valid = true;
-            p = reinterpret_cast<const uint4 *>(x + ((int64_t)unit * 16 + n16) * 128 + 32 * kc);
+            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)unit * 16 + n16) * 128 + 32 * kc));
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) xb[ks] = load_input16(p + ks);
@@ -532,7 +536,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
             ss = diag_here ? ss : 0.0f;
             cur[r] = next;
-            if (next < end) fetch(next, xb, xvalid[r]);  // nothing is requested past the share
+            fetch(next, xb, xvalid[r]);
             ss += xor_lane<16>(ss);
             ss += xor_lane<32>(ss);
             const float norm = __builtin_amdgcn_sqrtf(ss);  // 1 ulp: scales boundaries (1e-7 relative) and the stored fp16 norm
@@ -823,6 +827,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // supplies inputs 32ks + 8kq .. +7.  The address is always valid (clamped); `valid` says
     // whether the row exists.
     auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
+        const bool beyond = unit > last_unit;  // past the share: every lane reads the tensor's first bytes (see the K units)
         unit = unit < last_unit ? unit : last_unit;
 #if TQ_KNOCKOUT & 32
         unit = lo + (((unit - lo) / step) & 1u) * step;  // the first two tiles of the share over and over: no HBM reads
@@ -835,10 +840,10 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + tb;
             valid = tok < a.tokens;
             tok = valid ? tok : a.tokens - 1;
-            p = reinterpret_cast<const uint4 *>(x + ((int64_t)seq * a.tokens + tok) * 128 + 8 * kq);
+            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)seq * a.tokens + tok) * 128 + 8 * kq));
         } else {
             valid = true;
-            p = reinterpret_cast<const uint4 *>(x + ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq);
+            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq));
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
@@ -909,7 +914,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                                                               gram, 0, 0, 0);
 #endif
             if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-            else if (next < end) fetch(next, 5 - q, xb, xvalid[q & 1]);  // nothing is requested past the share
+            else fetch(next, 5 - q, xb, xvalid[q & 1]);
 
             float nrm[4];
             float4_t inv;
