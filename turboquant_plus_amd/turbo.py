@@ -267,16 +267,24 @@ class TurboCodec:
         return out.reshape(xd.shape)
 
     # ---- prefill-shaped inner-product estimator --------------------------------
-    def score_tile(self, q, packed, sign_bits, rnorms, n_keys: int, out_dtype=None, store: bool = True):
+    def score_tile(self, q, packed, sign_bits, rnorms, n_keys: int, out_dtype=None, store: bool = True, out=None):
         """logits [nq, n_keys] = <R q, g c[idx]> + scale * rnorm * <S q, z>.  store=False runs the
-        computation without writing the logits (a measurement aid) and returns None."""
+        computation without writing the logits (a measurement aid) and returns None.  out: a
+        contiguous [nq, n_keys] tensor of the output type to write into instead of a new one."""
         tt = L.torch()
         qd = L.to_device(q).reshape(-1, HEAD_DIM)
         nq = qd.shape[0]
+        if out is not None:
+            out_dtype = out.dtype
         out_dtype = tt.float32 if out_dtype is None else out_dtype
         if out_dtype not in (tt.float32, tt.float16):
             raise TypeError(f"logits must be float32 or float16, not {out_dtype}")
-        logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device) if store else None
+        if out is not None:
+            if tuple(out.shape) != (nq, n_keys) or not out.is_contiguous() or not out.is_cuda:
+                raise ValueError(f"out must be a contiguous device tensor of shape ({nq}, {n_keys})")
+            logits = out
+        else:
+            logits = tt.empty((nq, n_keys), dtype=out_dtype, device=qd.device) if store else None
         ws = tt.empty(max((nq + 31) // 32 * 32 * 512, 16), dtype=tt.uint8, device=qd.device)
         L.check(L.lib().tq_score_tile(self.handle.h, L.ptr(qd), L.dtype_code(qd), nq, L.ptr(packed), L.ptr(sign_bits),
                                       L.ptr(rnorms), n_keys, L.ptr(logits) if store else None,
