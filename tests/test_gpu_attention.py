@@ -409,15 +409,15 @@ def test_score_tile_edges(nk, nq):
     scale = np.linalg.norm(qs.astype(np.float64), axis=1).max() * np.linalg.norm(keys.astype(np.float64), axis=1).max()
     for dt, tol in ((tt.float32, 2e-3 * scale / np.sqrt(D) * 4), (tt.float16, 4e-3 * max(np.abs(ref).max(), 1.0))):
         # the logits sit in the middle of a larger buffer filled with a sentinel
-        pad = 64
-        buf = tt.full((nq * nk + 2 * pad,), 1024.0, dtype=dt, device="cuda")
-        out = buf[pad:pad + nq * nk].view(nq, nk)
-        got = codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt, out=out)
-        assert got.data_ptr() == out.data_ptr()
-        a = np_(out).astype(np.float64)
-        assert np.abs(a - ref).max() <= tol, (nk, nq, str(dt))
-        edge = np_(buf).astype(np.float64)
-        assert (edge[:pad] == 1024.0).all() and (edge[pad + nq * nk:] == 1024.0).all()
+        for pad in (64,):  # the entry point asks for 16-byte aligned logits
+            buf = tt.full((nq * nk + 2 * pad,), 1024.0, dtype=dt, device="cuda")
+            out = buf[pad:pad + nq * nk].view(nq, nk)
+            got = codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt, out=out)
+            assert got.data_ptr() == out.data_ptr()
+            a = np_(out).astype(np.float64)
+            assert np.abs(a - ref).max() <= tol, (nk, nq, str(dt), pad)
+            edge = np_(buf).astype(np.float64)
+            assert (edge[:pad] == 1024.0).all() and (edge[pad + nq * nk:] == 1024.0).all()
 
 
 FORMATS = ["turbo2", "turbo3", "turbo4", "q8_0"]
