@@ -1528,6 +1528,226 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
     }
 }
 
+
+// Row-major variant of the score tile.  The dequantised keys leave LDS for registers (a wavefront keeps the
+// operands of 64 keys, 128 registers) and the queries pass through LDS instead, 128 at a time, double-buffered
+// over the memory the keys were staged in.  Wavefront w works on key group w % 4 (64 keys) and on the query half
+// w / 4 of the tile, 32 queries at a time: per K step one query operand from LDS feeds two matrix instructions
+// (the two 32-key halves of the group).  The four wavefronts of a query half thus finish the same 32 logit rows
+// at about the same time, each its own 256 bytes of them: a row leaves the workgroup as 1 KB of consecutive
+// addresses instead of eight 128-byte pieces spread over the sweep, which the memory side takes faster.
+constexpr int SCORE_QT = 128;  // queries per LDS tile: four operand blocks of 16 KB
+template <int BITS, typename TO, bool DRAIN>
+__global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
+                                                      const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
+                                                      const uint32_t *pair_lut, float proj_scale) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 kt[];  // keys [SCORE_KEYS][KT_STRIDE], then two query tiles
+    __shared__ uint32_t ptab[1 << (2 * BITS)];                     // pair code -> (c[lo], c[hi]) as two halves
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int64_t key0 = (int64_t)blockIdx.x * SCORE_KEYS;
+    const int n_blocks = (int)((nq + 31) / 32);  // operand blocks the preparation wrote
+    const int n_tiles = (int)((nq + SCORE_QT - 1) / SCORE_QT);
+    typedef uint32_t chunk_t __attribute__((ext_vector_type(4)));   // 16 bytes: what a lane feeds to one matrix instruction
+    const chunk_t *qchunks = reinterpret_cast<const chunk_t *>(qa);  // [block][K step][lane]
+    // chunk group g (0..7) of a tile: lanes tid + 512 g of its 4096 chunks, i.e. half g % 2 of operand block g / 2
+    auto tile_chunk = [&](int tile, int g) __attribute__((always_inline)) {
+        const int blk = min(tile * (SCORE_QT / 32) + (g >> 1), n_blocks - 1);  // past the end: the last block again
+        return qchunks + (int64_t)blk * 1024 + (g & 1) * 512 + tid;
+    };
+    // the first tile is requested before anything else and waits in registers until the keys have left LDS
+    chunk_t first_tile[8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g) first_tile[g] = *tile_chunk(0, g);
+    if (tid < (1 << (2 * BITS))) ptab[tid] = pair_lut[tid];
+    __syncthreads();
+    {
+        // threads 0..255 dequantise the codes of one key each, threads 256..511 its sign bits; eight halves
+        // (16 bytes) per LDS write
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        const int key = tid & (SCORE_KEYS - 1), part = tid >> 8;
+        uint4 *row = reinterpret_cast<uint4 *>(kt + key * KT_STRIDE) + part * 16;
+        const bool valid = key0 + key < nk;
+        if (part == 0) {
+            if (valid) {
+                const uint8_t *block = packed + (key0 + key) / TQ_ROWS_PER_BLOCK * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
+                uint32_t wv[4 * BITS];
+                load_row<BITS>(block, key & (TQ_ROWS_PER_BLOCK - 1), wv);
+                const _Float16 g = __builtin_bit_cast(
+                    _Float16, reinterpret_cast<const unsigned short *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key & (TQ_ROWS_PER_BLOCK - 1)]);
+                const half2_t g2 = {g, g};
+#pragma unroll
+                for (int c = 0; c < 16; ++c) {
+                    uint32_t u[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t e = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(ptab) +
+                                                                               pair_off<BITS>(wv, 4 * c + i));
+                        u[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, e) * g2);
+                    }
+                    row[c] = make_uint4(u[0], u[1], u[2], u[3]);
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 16; ++c) row[c] = make_uint4(0, 0, 0, 0);
+            }
+        } else {
+            float rs = 0.f;
+            uint4 sb = make_uint4(0, 0, 0, 0);
+            if (valid) {
+                rs = proj_scale * __half2float(rnorms[key0 + key]);
+                sb = *reinterpret_cast<const uint4 *>(sign_bits + (key0 + key) * 16);
+            }
+            const uint32_t sw[4] = {sb.x, sb.y, sb.z, sb.w};
+            // +rs where the bit is set, -rs where it is clear: two halves per word, the sign bits from the inverted bits
+            const uint32_t mag = (uint32_t)__half_as_ushort(__float2half_rn(rs)) * 0x00010001u;
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                uint32_t u[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int jj = 8 * c + 2 * i;  // sign bits jj, jj + 1
+                    const uint32_t nb = ~sw[jj >> 5] >> (jj & 31);
+                    u[i] = mag ^ (((nb & 1u) << 15) | ((nb & 2u) << 30));
+                }
+                row[c] = make_uint4(u[0], u[1], u[2], u[3]);
+            }
+        }
+    }
+    __syncthreads();
+
+    // lane l of a 32 x 32 result tile holds key column l % 32 for the query rows 8j + 4(l/32) + i
+    const int kg = __builtin_amdgcn_readfirstlane(w & 3), qh = __builtin_amdgcn_readfirstlane(w >> 2);
+    const int c32 = lane & 31, kb = lane >> 5;
+    half8_t kf[2][16];  // [32-key half of the group][K step of 16]
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            kf[kh][t] = *reinterpret_cast<const half8_t *>(kt + (kg * 64 + kh * 32 + c32) * KT_STRIDE + t * 16 + 8 * kb);
+    __syncthreads();  // every wavefront has its keys: the memory now holds query tiles
+    chunk_t *qtile = reinterpret_cast<chunk_t *>(kt);  // [2][4096] chunks
+#pragma unroll
+    for (int g = 0; g < 8; ++g) qtile[g * 512 + tid] = first_tile[g];
+    // (LDS only: a __syncthreads would also wait for the logit stores in flight)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // A finished (32 queries, 64 keys) block is written while the next one is being multiplied: one store
+    // instruction after each matrix instruction, from a second set of accumulators.  One v_permlane32_swap per
+    // accumulator pair puts the row 8j + i of both key halves into one register (lanes 0..31 the first half's 32
+    // keys, lanes 32..63 the second's) and the row 8j + 4 + i into the other, so a store writes 64 consecutive
+    // logits of one row.  The stores are buffer stores whose resource is that row's piece (scalar arithmetic): its
+    // size is 0 for a row past the last query and ends at the last key, so the hardware drops what does not exist
+    // and no store needs an address register or a branch.
+    constexpr int NT_AUX = (TQ_STREAM_SITES & STREAM_LOGITS) ? 2 : 0;  // the non-temporal bit of a buffer instruction
+    const int64_t key0w = key0 + kg * 64;
+    const uint32_t piece_bytes = (uint32_t)max((int64_t)0, min((int64_t)64, nk - key0w)) * (uint32_t)sizeof(TO);
+    const int lane_off = lane * (int)sizeof(TO);
+    struct Pending {
+        TO *base;  // first logit of the block's first row in this wavefront's key group
+        int rows;  // rows of the block that exist (0: nothing is pending)
+    };
+    auto pend = [&](int row0) __attribute__((always_inline)) {
+        Pending pb;
+        pb.rows = __builtin_amdgcn_readfirstlane(max(0, min(32, (int)nq - row0)));
+        const uint64_t b = reinterpret_cast<uint64_t>(logits + (int64_t)row0 * nk + key0w);
+        // wave-uniform by construction; said explicitly so that the resources are built by scalar instructions
+        pb.base = reinterpret_cast<TO *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                                         (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
+        return pb;
+    };
+    auto store_row = [&](const Pending &pb, const uint32_t bits, const int row) __attribute__((always_inline)) {
+        const uint32_t size = row < pb.rows ? piece_bytes : 0u;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(pb.base + (int64_t)row * nk, 0, (int)size, 0x00020000);
+        if constexpr (sizeof(TO) == 4) {
+            __builtin_amdgcn_raw_buffer_store_b32(bits, rs, lane_off, 0, NT_AUX);
+        } else {
+            __builtin_amdgcn_raw_buffer_store_b16(__half_as_ushort(__float2half_rn(__uint_as_float(bits))), rs, lane_off, 0, NT_AUX);
+        }
+    };
+
+    float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
+    chunk_t staged[4];  // half of the next tile's chunks on their way from memory to LDS
+    // one block of 32 queries (operand block `b` of the tile in `cur`) against the 64 resident keys into acc, while
+    // the pending block leaves from pacc and half of the next tile (chunk groups 4 * half .. + 3) is brought in
+    auto block = [&](const chunk_t *cur, chunk_t *next, const int b, auto half, const int tile_next, float16_t (&acc)[2],
+                     const float16_t (&pacc)[2], const Pending &pb) __attribute__((always_inline)) {
+        constexpr int HALF = decltype(half)::value;
+        const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const chunk_t *arow = cur + b * 1024 + lane;
+        // query operands come from LDS AHEAD steps ahead; the scheduling fence after every step keeps the
+        // compiler from hoisting all sixteen steps' reads to the top
+        constexpr int AHEAD = 3;
+        half8_t af[AHEAD + 1];
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t) af[t] = __builtin_bit_cast(half8_t, arow[t * 64]);
+        uint32_t swapped = 0u;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            if (t + AHEAD < 16) af[(t + AHEAD) & AHEAD] = __builtin_bit_cast(half8_t, arow[(t + AHEAD) * 64]);
+            if (t == 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) staged[g] = *tile_chunk(tile_next, 4 * HALF + g);
+            }
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                acc[kh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & AHEAD], kf[kh][t], t == 0 ? zero : acc[kh], 0, 0, 0);
+                if constexpr (DRAIN) {
+                    // accumulator element t = 4j + i: rows 8j + i (kh = 0 here) and 8j + 4 + i (kh = 1)
+                    const int row = 8 * (t >> 2) + (t & 3);
+                    if (kh == 0) {
+                        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(pacc[0][t]), __float_as_uint(pacc[1][t]), false, false);
+                        swapped = r[1];
+                        store_row(pb, r[0], row);
+                    } else {
+                        store_row(pb, swapped, row + 4);
+                    }
+                }
+            }
+            if (t == 15) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) next[(4 * HALF + g) * 512 + tid] = staged[g];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (!DRAIN) {
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) keep += acc[kh][e];
+        }
+    };
+    float16_t acc_a[2], acc_b[2];
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc_b[kh][e] = 0.0f;
+    Pending pb = pend(0);
+    pb.rows = 0;  // nothing is pending before the first block
+#pragma unroll 1
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const chunk_t *cur = qtile + (tile & 1) * 4096;
+        chunk_t *next = qtile + ((tile + 1) & 1) * 4096;
+        const int row0 = tile * SCORE_QT + qh * 64;
+        const int tile_next = min(tile + 1, n_tiles - 1);  // the last tile re-reads itself
+        block(cur, next, 2 * qh, std::integral_constant<int, 0>{}, tile_next, acc_a, acc_b, pb);
+        pb = pend(row0);
+        block(cur, next, 2 * qh + 1, std::integral_constant<int, 1>{}, tile_next, acc_b, acc_a, pb);
+        pb = pend(row0 + 32);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    if constexpr (DRAIN) {  // the last block (in acc_b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc_b[0][e]), __float_as_uint(acc_b[1][e]), false, false);
+            const int row = 8 * (e >> 2) + (e & 3);
+            store_row(pb, r[0], row);
+            store_row(pb, r[1], row + 4);
+        }
+    } else {
+        if (keep == 1.25e38f) reinterpret_cast<float *>(const_cast<__half *>(qa))[0] = keep;
+    }
+}
+
 }  // namespace
 
 int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
@@ -1566,6 +1786,25 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
     }
 #define TQ_SCORE_BITS(T, P, DR)                                                                              \
     if (h->bits == 2) TQ_SCORE(2, T, P, DR) else if (h->bits == 3) TQ_SCORE(3, T, P, DR) else TQ_SCORE(4, T, P, DR)
+#ifndef TQ_SCORE_COLUMNS
+#define TQ_ROWS(B, T, DR)                                                                                              \
+    {                                                                                                                  \
+        (void)hipFuncSetAttribute((const void *)k_score_rows<B, T, DR>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                  (int)lds);                                                                           \
+        k_score_rows<B, T, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
+                                                      nq, nk, (T *)logits, (const uint32_t *)h->pair_lut, (float)h->proj_scale); \
+    }
+#define TQ_ROWS_BITS(T, DR)                                                                              \
+    if (h->bits == 2) TQ_ROWS(2, T, DR) else if (h->bits == 3) TQ_ROWS(3, T, DR) else TQ_ROWS(4, T, DR)
+    if (!logits) {
+        TQ_ROWS_BITS(float, false)
+    } else if (out_dtype == TQ_F32) {
+        TQ_ROWS_BITS(float, true)
+    } else {
+        TQ_ROWS_BITS(__half, true)
+    }
+    return tq_check_launch("score_tile");
+#endif
     if (!logits) {
         TQ_SCORE_BITS(float, false, false)
     } else if (out_dtype == TQ_F32) {
