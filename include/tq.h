@@ -281,10 +281,9 @@ int tq_decode_attention_static(const tq_handle *hk, const tq_handle *hv, const t
  * rnorms from tq_store_qjl with n_seqs = 1, logits [nq, nk] fp32 (or fp16 when
  * out_dtype == TQ_F16).  workspace: 512 bytes per query, query count rounded up to a
  * multiple of 32.  logits == NULL runs the whole computation and stores nothing (for
- * measuring the contraction without the logit stores).  Limits: nq < 2^24, and 64 rows of
- * logits below 2 GiB (nk < 8 388 608 for fp32, twice that for fp16; TQ_ERR_UNSUPPORTED beyond:
- * score the keys in slices).  fp16 logits are stored two at a time when nk is even and
- * logits is 4-byte aligned, singly otherwise. */
+ * measuring the contraction without the logit stores).  Limit: nq < 2^24 (TQ_ERR_UNSUPPORTED
+ * beyond: score the queries in slices); any nk.  logits needs only the alignment of its
+ * element type. */
 int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, const void *packed,
                   const uint8_t *sign_bits, const void *rnorms_f16, int64_t nk, void *logits, int out_dtype,
                   void *workspace, int64_t workspace_bytes, void *stream);

@@ -390,11 +390,13 @@ def test_score_tile(projection, nk, nq):
     assert np.abs(h - ref).max() <= 4e-3 * np.abs(ref).max()
 
 
-@pytest.mark.parametrize("nk,nq", [(1, 1), (31, 33), (32, 64), (33, 31), (255, 65), (257, 1), (510, 130), (769, 513)])
+@pytest.mark.parametrize("nk,nq", [(1, 1), (31, 33), (32, 64), (33, 31), (63, 127), (65, 129), (127, 95), (129, 97),
+                                   (191, 160), (193, 255), (255, 65), (257, 1), (510, 130), (769, 513)])
 def test_score_tile_edges(nk, nq):
-    """Row and key edges of the estimator tile: key counts around the 32-key sub-block and the 256-key workgroup,
-    odd ones (fp16 logits then leave singly), query counts around the 32- and 64-row blocks and the 512-query tile.
-    Everything outside [nq, nk] must stay untouched (the stores rely on the hardware's range check)."""
+    """Row and key edges of the estimator tile: key counts around the 32-key half, the 64-key group of a wavefront
+    and the 256-key workgroup, odd ones among them; query counts around the 32-row block, the 64-row half and the
+    128-query tile.  Everything outside [nq, nk] must stay untouched (the stores rely on the hardware's range
+    check)."""
     tt = L.torch()
     rng = np.random.default_rng(1000 * nk + nq)
     keys = rng.standard_normal((nk, D)).astype(np.float32)
@@ -418,6 +420,28 @@ def test_score_tile_edges(nk, nq):
             assert np.abs(a - ref).max() <= tol, (nk, nq, str(dt), pad)
             edge = np_(buf).astype(np.float64)
             assert (edge[:pad] == 1024.0).all() and (edge[pad + nq * nk:] == 1024.0).all()
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_score_tile_other_widths(bits):
+    """The estimator tile at the other code widths (their own dequantisation path), fp32 and fp16 logits."""
+    tt = L.torch()
+    nk, nq = 700, 150
+    rng = np.random.default_rng(40 + bits)
+    keys = rng.standard_normal((nk, D)).astype(np.float32)
+    qs = rng.standard_normal((nq, D)).astype(np.float32)
+    codec = tqa.TurboCodec(bits, seed=42, projection="gaussian", projection_seed=5)
+    packed, sbits, rn = codec.store_qjl(keys)
+    idx, g = codec.unpack_codes(packed, 1, nk)
+    z = np.unpackbits(np_(sbits), axis=1, bitorder="little")[:, :D].astype(np.float64) * 2 - 1
+    ref = O.score_tile(qs.astype(np.float64), np_(idx)[0], np_(g)[0].astype(np.float64), codec.centroids,
+                       lambda a: O.rotate_fast(a, codec.signs1, codec.signs2, D), codec.S, z,
+                       np_(rn).astype(np.float64), codec.projection_scale)
+    scale = np.linalg.norm(qs.astype(np.float64), axis=1).max() * np.linalg.norm(keys.astype(np.float64), axis=1).max()
+    logits = np_(codec.score_tile(qs, packed, sbits, rn, nk)).astype(np.float64)
+    assert np.abs(logits - ref).max() <= 2e-3 * scale / np.sqrt(D) * 4
+    h = np_(codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=tt.float16)).astype(np.float64)
+    assert np.abs(h - ref).max() <= 4e-3 * np.abs(ref).max()
 
 
 FORMATS = ["turbo2", "turbo3", "turbo4", "q8_0"]

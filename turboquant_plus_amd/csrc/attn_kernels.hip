@@ -32,7 +32,8 @@
 //   of the V rotation and writes the output rows (merge_group): a step is one launch.  Queries are rotated and
 //   scaled inside the kernel.
 // k_score_tile: TurboQuant inner-product estimate, 32x32x16 fp16 MFMA over a
-//   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]).
+//   K = 256 contraction ([R q | S q] against [g c[idx] | scale*rnorm*z]); key operands in registers, queries
+//   through LDS, logit rows written 64 consecutive logits per store.
 #include <atomic>
 #include <mutex>
 #include <cstring>
@@ -1249,296 +1250,19 @@ __global__ __launch_bounds__(256) void k_prep_score_q(const TI *q, __half *qa, i
         }
 }
 
-// One workgroup of eight wavefronts per 256 keys: dequantise them once into LDS as fp16
-// [g*c[idx] | scale*rnorm*z], then sweep all queries with 32x32x16 MFMA tiles (queries on the M side,
-// keys on the N side).  A wavefront owns 64 queries of each 512-query tile: their operands (64 x 256
-// halves) live in registers, are used against the eight 32-key sub-blocks in turn, and are replaced,
-// step by step, with the next tile's while the last sub-block is being multiplied, so every query
-// operand crosses the vector memory path once per workgroup and a whole tile ahead of its use.
+// One workgroup of eight wavefronts per 256 keys.  The keys are dequantised once into LDS as fp16
+// [g*c[idx] | scale*rnorm*z]; every wavefront then takes the operands of its 64 keys into registers (128 of
+// them) and the same LDS carries the queries instead, 128 at a time, double-buffered, brought in by loads that
+// write LDS directly.  Matrix tiles are 32 x 32 x 16 with the queries on the M side and the keys on the N side.
+// Wavefront w works on key group w % 4 (64 keys) and on the query half w / 4 of a tile, 32 queries at a time:
+// per K step one query operand from LDS feeds two matrix instructions (the two 32-key halves of the group).
+// The four wavefronts of a query half finish the same 32 logit rows at about the same time, each its own 64
+// logits of them, so a row leaves the workgroup as 256 consecutive logits (1 KB in fp32) within a short time,
+// not as 128-byte pieces spread over a sweep: the memory side takes that order markedly faster.
 constexpr int SCORE_KEYS = 256;  // keys per workgroup (two 128-row blocks)
-// PAIRS (fp16 logits only): the key count is even and the logits are 4-byte aligned, so a lane stores two at once.
-// DRAIN false is the measurement mode: everything but the stores (logits is NULL).
-template <int BITS, typename TO, bool PAIRS, bool DRAIN>
-__global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
-                                                      const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
-                                                      const uint32_t *pair_lut, float proj_scale) {
-    extern __shared__ __attribute__((aligned(16))) _Float16 kt[];  // [SCORE_KEYS][KT_STRIDE]
-    __shared__ uint32_t ptab[1 << (2 * BITS)];  // pair code -> (c[lo], c[hi]) as two halves
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int64_t key0 = (int64_t)blockIdx.x * SCORE_KEYS;
-    if (tid < (1 << (2 * BITS))) ptab[tid] = pair_lut[tid];
-    __syncthreads();
-    {
-        // threads 0..255 dequantise the codes of one key each, threads 256..511 its sign bits; eight halves
-        // (16 bytes) per LDS write
-        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-        const int key = tid & (SCORE_KEYS - 1), part = tid >> 8;
-        uint4 *row = reinterpret_cast<uint4 *>(kt + key * KT_STRIDE) + part * 16;
-        const bool valid = key0 + key < nk;
-        if (part == 0) {
-            if (valid) {
-                const uint8_t *block = packed + (key0 + key) / TQ_ROWS_PER_BLOCK * (TQ_ROWS_PER_BLOCK * (16 * BITS + 2));
-                uint32_t wv[4 * BITS];
-                load_row<BITS>(block, key & (TQ_ROWS_PER_BLOCK - 1), wv);
-                const _Float16 g = __builtin_bit_cast(
-                    _Float16, reinterpret_cast<const unsigned short *>(block + TQ_ROWS_PER_BLOCK * 16 * BITS)[key & (TQ_ROWS_PER_BLOCK - 1)]);
-                const half2_t g2 = {g, g};
-#pragma unroll
-                for (int c = 0; c < 16; ++c) {
-                    uint32_t u[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t e = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(ptab) +
-                                                                               pair_off<BITS>(wv, 4 * c + i));
-                        u[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, e) * g2);
-                    }
-                    row[c] = make_uint4(u[0], u[1], u[2], u[3]);
-                }
-            } else {
-#pragma unroll
-                for (int c = 0; c < 16; ++c) row[c] = make_uint4(0, 0, 0, 0);
-            }
-        } else {
-            float rs = 0.f;
-            uint4 sb = make_uint4(0, 0, 0, 0);
-            if (valid) {
-                rs = proj_scale * __half2float(rnorms[key0 + key]);
-                sb = *reinterpret_cast<const uint4 *>(sign_bits + (key0 + key) * 16);
-            }
-            const uint32_t sw[4] = {sb.x, sb.y, sb.z, sb.w};
-            // +rs where the bit is set, -rs where it is clear: two halves per word, the sign bits from the inverted bits
-            const uint32_t mag = (uint32_t)__half_as_ushort(__float2half_rn(rs)) * 0x00010001u;
-#pragma unroll
-            for (int c = 0; c < 16; ++c) {
-                uint32_t u[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int jj = 8 * c + 2 * i;  // sign bits jj, jj + 1
-                    const uint32_t nb = ~sw[jj >> 5] >> (jj & 31);
-                    u[i] = mag ^ (((nb & 1u) << 15) | ((nb & 2u) << 30));
-                }
-                row[c] = make_uint4(u[0], u[1], u[2], u[3]);
-            }
-        }
-    }
-    __syncthreads();
-
-    // two MFMA tiles of 32 x 32 per (64 queries, 32 keys): lane l of a result tile holds key column
-    // l % 32 for the query rows 8j + 4(l/32) + i, so a store instruction writes two runs of 32 consecutive
-    // logits (a whole 128-byte line for fp32).
-    const int qh = __builtin_amdgcn_readfirstlane(w);  // wave-uniform: the bases of the stores stay scalar
-    const int c32 = lane & 31, kb = lane >> 5;
-    constexpr int QT = 512;
-    const int n_qt = (int)((nq + QT - 1) / QT);
-    const int nq_last = (int)nq - 1;  // the launcher checks the query count
-    half8_t qf[16][2];  // [K step of 16][32-query row block] of the current query tile
-    // rows past the last query are clamped (loaded, multiplied, never stored): no branch in the loop
-    const char *qrow[2];
-    auto point_queries = [&](int qt) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            const int qi = min(qt * QT + qh * 64 + mb * 32 + c32, nq_last);
-            qrow[mb] = reinterpret_cast<const char *>(qa) + ((int64_t)(qi >> 5) * 16 * 64 + (qi & 31) + 32 * kb) * 16;
-        }
-    };
-    auto load_queries = [&](int t) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) qf[t][mb] = *reinterpret_cast<const half8_t *>(qrow[mb] + t * 1024);
-    };
-    point_queries(0);
-#pragma unroll
-    for (int t = 0; t < 16; ++t) load_queries(t);
-    const _Float16 *krow0 = kt + c32 * KT_STRIDE + 8 * kb;
-
-    // A finished (64 queries, 32 keys) block is written while the next one is being multiplied: its store
-    // instructions go out one after each matrix instruction of the next block, from a second set of accumulators,
-    // so a wavefront never sits in a store-only phase.  The stores are buffer stores whose resource starts at the
-    // row a store writes (scalar arithmetic) and ends after the block's last existing row, and whose only vector
-    // operand is the lane's place relative to that row (one register for the whole kernel): rows past the last
-    // query fall outside the resource and the hardware drops them, lanes whose key does not exist get an offset
-    // outside every resource, and no store needs an address register or a branch.
-    constexpr bool PAIRED = sizeof(TO) == 2 && PAIRS;  // fp16: two logits per lane and store, whole 128-byte lines
-    constexpr int N_GROUPS = PAIRED ? 16 : 32;         // store groups per block
-    constexpr int NT_AUX = (TQ_STREAM_SITES & STREAM_LOGITS) ? 2 : 0;  // the non-temporal bit of a buffer instruction
-    constexpr uint32_t DROPPED = 0x80000000u;          // beyond any resource (the launcher keeps 64 rows below 2 GiB)
-    const uint32_t row_bytes = (uint32_t)nk * (uint32_t)sizeof(TO);
-    const bool odd = lane & 1;
-    // Paired fp16: two neighbouring 32-key sub-blocks leave together.  A lane packs two logits (keys c32 & ~1, c32 | 1;
-    // even lanes rows 8j + 4kb + h, odd lanes rows 8j + 4kb + 2 + h, by trading with the neighbouring lane), the packed
-    // words of the first sub-block wait in 16 registers, and when the second is packed one v_permlane32_swap per
-    // register puts the first sub-block's words of the rows kb = 0 into lanes 0..31 and the second's into lanes
-    // 32..63 (and likewise for kb = 1), so that a store instruction writes 64 consecutive logits = one whole
-    // 128-byte line of each of two rows.  The lane's place: (its parity's row, its half's sub-block, its key pair).
-    const uint32_t lane_bytes = PAIRED ? (odd ? 2u * row_bytes : 0u) + (uint32_t)kb * 64u + (uint32_t)(c32 & ~1) * 2u
-                                       : (uint32_t)(4 * kb) * row_bytes + (uint32_t)c32 * (uint32_t)sizeof(TO);
-    struct Pending {
-        TO *base[2];        // first logit of the two 32-row blocks
-        int rows[2];        // rows of each that exist (0: nothing is pending)
-        uint32_t voff;      // lane_bytes, or DROPPED where the lane's key does not exist
-    };
-    auto pend = [&](int qbase, int ks) __attribute__((always_inline)) {
-        Pending pb;
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-#ifdef TQ_SCORE_L2  // measurement build: every query tile lands on the first 64 rows, so the logits stay in L2
-            pb.base[mb] = logits + (int64_t)((qbase & 63) + mb * 32) * nk + (key0 + ks * 32);
-#else
-            pb.base[mb] = logits + (int64_t)(qbase + mb * 32) * nk + (key0 + ks * 32);
-#endif
-            pb.rows[mb] = max(0, min(32, (int)nq - (qbase + mb * 32)));
-            // wave-uniform by construction; said explicitly so that the resources are built by scalar instructions
-            pb.rows[mb] = __builtin_amdgcn_readfirstlane(pb.rows[mb]);
-            const uint64_t b = reinterpret_cast<uint64_t>(pb.base[mb]);
-            pb.base[mb] = reinterpret_cast<TO *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
-                                                 (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
-        }
-        // paired: ks is the first sub-block of the pair, lanes 32..63 hold the second one's keys; the key count is even
-        const int64_t first_key = key0 + ks * 32 + (PAIRED ? 32 * kb + (c32 & ~1) : c32);
-        pb.voff = first_key < nk ? lane_bytes : DROPPED;
-        return pb;
-    };
-    // store group n of a pending block, unpaired: accumulator element n % 16 of row block n / 16 (rows 8j + 4kb + i,
-    // e = 4j + i)
-    auto store_group = [&](const Pending &pb, const float16_t (&acc)[2], const int n) __attribute__((always_inline)) {
-        const int mb = n >> 4;
-        const int row = 8 * ((n & 15) >> 2) + (n & 3);  // of lane half kb = 0
-        const int left = max(pb.rows[mb] - row, 0);
-        const __amdgpu_buffer_rsrc_t rs =
-            __builtin_amdgcn_make_buffer_rsrc(pb.base[mb] + (int64_t)row * nk, 0, (int)((uint32_t)left * row_bytes), 0x00020000);
-        if constexpr (sizeof(TO) == 4) {
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mb][n & 15]), rs, (int)pb.voff, 0, NT_AUX);
-        } else {
-            __builtin_amdgcn_raw_buffer_store_b16(__half_as_ushort(__float2half_rn(acc[mb][n & 15])), rs, (int)pb.voff, 0, NT_AUX);
-        }
-    };
-    // paired: group n = rows 8j + 4kb + {h, 2 + h} of row block n / 8, j = (n % 8) / 2, h = n % 2, as two packed halves
-    auto pack_group = [&](const float16_t (&acc)[2], const int n) __attribute__((always_inline)) -> uint32_t {
-        const int mb = n >> 3, j = (n >> 1) & 3, h = n & 1;
-        const float mine_lo = acc[mb][4 * j + h], mine_hi = acc[mb][4 * j + 2 + h];
-        const float got = xor_lane<1>(odd ? mine_lo : mine_hi);
-        const float v0 = odd ? got : mine_lo, v1 = odd ? mine_hi : got;  // keys (c32 & ~1), (c32 | 1)
-        return (uint32_t)__half_as_ushort(__float2half_rn(v0)) | ((uint32_t)__half_as_ushort(__float2half_rn(v1)) << 16);
-    };
-    // paired: group n of a pair of sub-blocks (first sub-block's packed word, second's) -> two stores of two lines each
-    auto store_pair_group = [&](const Pending &pb, const uint32_t first, const uint32_t second, const int n) __attribute__((always_inline)) {
-        const int mb = n >> 3, row = 8 * ((n >> 1) & 3) + (n & 1);
-        const auto r = __builtin_amdgcn_permlane32_swap(first, second, false, false);  // [0]: rows kb = 0, [1]: rows kb = 1
-#pragma unroll
-        for (int hi = 0; hi < 2; ++hi) {
-            const int left = max(pb.rows[mb] - (row + 4 * hi), 0);
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(pb.base[mb] + (int64_t)(row + 4 * hi) * nk, 0,
-                                                                                 (int)((uint32_t)left * row_bytes), 0x00020000);
-            __builtin_amdgcn_raw_buffer_store_b32(r[hi], rs, (int)pb.voff, 0, NT_AUX);
-        }
-    };
-    uint32_t first_packed[PAIRED ? 16 : 1];  // paired: the first sub-block of the pair, packed, waiting for the second
-
-    float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
-    // one 32-key sub-block against the resident query tile into acc, while the pending block leaves from pacc
-    // prev_second (paired fp16): the previous sub-block was the second of its pair
-    auto sub_block = [&](const int ks, auto prefetch, auto drain, auto prev_second, float16_t (&acc)[2], const float16_t (&pacc)[2],
-                         const Pending &pb) __attribute__((always_inline)) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[mb][e] = 0.0f;
-        // (the sub-block number is made opaque: with a constant the compiler keeps one address register per step
-        // instead of one base and sixteen immediate offsets)
-        int ks_opaque = ks;
-        asm volatile("" : "+s"(ks_opaque));
-        const _Float16 *krow = krow0 + ks_opaque * 32 * KT_STRIDE;
-        // key operands come from LDS AHEAD steps ahead; the scheduling fence after every step keeps the
-        // compiler from hoisting all sixteen steps' reads to the top
-        constexpr int AHEAD = 3;
-        half8_t kf[AHEAD + 1];
-#pragma unroll
-        for (int t = 0; t < AHEAD; ++t) kf[t] = *reinterpret_cast<const half8_t *>(krow + t * 16);
-#pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            if (t + AHEAD < 16) kf[(t + AHEAD) & AHEAD] = *reinterpret_cast<const half8_t *>(krow + (t + AHEAD) * 16);
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
-                acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[t][mb], kf[t & AHEAD], acc[mb], 0, 0, 0);
-                if constexpr (decltype(drain)::value) {
-                    const int n = 2 * t + mb;
-                    if constexpr (!PAIRED) {
-                        store_group(pb, pacc, n);
-                    } else if (n & 1) {
-                        // the previous sub-block is packed; if it was the second of its pair, the pair leaves
-                        const uint32_t u = pack_group(pacc, n >> 1);
-                        if constexpr (decltype(prev_second)::value) store_pair_group(pb, first_packed[n >> 1], u, n >> 1);
-                        else first_packed[n >> 1] = u;
-                    }
-                }
-            }
-            if constexpr (decltype(prefetch)::value) load_queries(t);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if constexpr (!decltype(drain)::value) {
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) keep += acc[mb][e];
-        }
-    };
-    auto sweep = [&](auto drain) __attribute__((always_inline)) {
-        float16_t acc_a[2], acc_b[2];
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc_b[mb][e] = 0.0f;
-        if constexpr (PAIRED) {
-#pragma unroll
-            for (int n = 0; n < 16; ++n) first_packed[n] = 0u;
-        }
-        Pending pb = pend(0, 0);
-        pb.rows[0] = pb.rows[1] = 0;  // nothing is pending before the first block
-        constexpr std::true_type second{};
-        constexpr std::false_type first{};
-        // unpaired: the pending block is the previous sub-block; paired: the previous pair (set when its second ends)
-#pragma unroll 1
-        for (int qt = 0; qt < n_qt; ++qt) {
-            const int qbase = qt * QT + qh * 64;
-            point_queries(min(qt + 1, n_qt - 1));  // the last tile re-reads itself
-#pragma unroll 1
-            for (int kp = 0; kp < SCORE_KEYS / 64 - 1; ++kp) {
-                sub_block(2 * kp, std::false_type{}, drain, second, acc_a, acc_b, pb);
-                if constexpr (!PAIRED) pb = pend(qbase, 2 * kp);
-                sub_block(2 * kp + 1, std::false_type{}, drain, first, acc_b, acc_a, pb);
-                pb = pend(qbase, PAIRED ? 2 * kp : 2 * kp + 1);
-            }
-            sub_block(SCORE_KEYS / 32 - 2, std::false_type{}, drain, second, acc_a, acc_b, pb);
-            if constexpr (!PAIRED) pb = pend(qbase, SCORE_KEYS / 32 - 2);
-            sub_block(SCORE_KEYS / 32 - 1, std::true_type{}, drain, first, acc_b, acc_a, pb);  // also fetches the next tile's queries
-            pb = pend(qbase, PAIRED ? SCORE_KEYS / 32 - 2 : SCORE_KEYS / 32 - 1);
-        }
-        if constexpr (decltype(drain)::value) {  // the last block (in acc_b)
-            if constexpr (PAIRED) {
-#pragma unroll
-                for (int n = 0; n < 16; ++n) store_pair_group(pb, first_packed[n], pack_group(acc_b, n), n);
-            } else {
-#pragma unroll
-                for (int n = 0; n < N_GROUPS; ++n) store_group(pb, acc_b, n);
-            }
-        }
-    };
-    sweep(std::integral_constant<bool, DRAIN>{});
-    if constexpr (!DRAIN) {
-        if (keep == 1.25e38f) reinterpret_cast<float *>(const_cast<__half *>(qa))[0] = keep;
-    }
-}
-
-
-// Row-major variant of the score tile.  The dequantised keys leave LDS for registers (a wavefront keeps the
-// operands of 64 keys, 128 registers) and the queries pass through LDS instead, 128 at a time, double-buffered
-// over the memory the keys were staged in.  Wavefront w works on key group w % 4 (64 keys) and on the query half
-// w / 4 of the tile, 32 queries at a time: per K step one query operand from LDS feeds two matrix instructions
-// (the two 32-key halves of the group).  The four wavefronts of a query half thus finish the same 32 logit rows
-// at about the same time, each its own 256 bytes of them: a row leaves the workgroup as 1 KB of consecutive
-// addresses instead of eight 128-byte pieces spread over the sweep, which the memory side takes faster.
 constexpr int SCORE_QT = 128;  // queries per LDS tile: four operand blocks of 16 KB
 template <int BITS, typename TO, bool DRAIN>
-__global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
+__global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const uint8_t *packed, const uint8_t *sign_bits,
                                                       const __half *rnorms, int64_t nq, int64_t nk, TO *logits,
                                                       const uint32_t *pair_lut, float proj_scale) {
     extern __shared__ __attribute__((aligned(16))) _Float16 kt[];  // keys [SCORE_KEYS][KT_STRIDE], then two query tiles
@@ -1666,9 +1390,9 @@ __global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const u
     };
 
     float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
-    chunk_t staged[4];  // half of the next tile's chunks on their way from memory to LDS
     // one block of 32 queries (operand block `b` of the tile in `cur`) against the 64 resident keys into acc, while
-    // the pending block leaves from pacc and half of the next tile (chunk groups 4 * half .. + 3) is brought in
+    // the pending block leaves from pacc; the first block of a tile also asks for the next tile (eight loads that
+    // write LDS directly, one per step: no registers, no LDS write instructions, and a lead of at least 24 steps)
     auto block = [&](const chunk_t *cur, chunk_t *next, const int b, auto half, const int tile_next, float16_t (&acc)[2],
                      const float16_t (&pacc)[2], const Pending &pb) __attribute__((always_inline)) {
         constexpr int HALF = decltype(half)::value;
@@ -1684,9 +1408,11 @@ __global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const u
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             if (t + AHEAD < 16) af[(t + AHEAD) & AHEAD] = __builtin_bit_cast(half8_t, arow[(t + AHEAD) * 64]);
-            if (t == 0) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) staged[g] = *tile_chunk(tile_next, 4 * HALF + g);
+            if (HALF == 0 && t < 8) {
+                // lane l of the wavefront brings chunk l of the wavefront's 1 KB piece of chunk group g
+                const int g = t;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(tile_chunk(tile_next, g)),
+                                                 (__attribute__((address_space(3))) void *)(next + g * 512 + w * 64), 16, 0, 0);
             }
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh) {
@@ -1702,10 +1428,6 @@ __global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const u
                         store_row(pb, swapped, row + 4);
                     }
                 }
-            }
-            if (t == 15) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) next[(4 * HALF + g) * 512 + tid] = staged[g];
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -1733,7 +1455,11 @@ __global__ __launch_bounds__(512, 1) void k_score_rows(const __half *qa, const u
         pb = pend(row0);
         block(cur, next, 2 * qh + 1, std::integral_constant<int, 1>{}, tile_next, acc_b, acc_a, pb);
         pb = pend(row0 + 32);
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // The next tile must have arrived.  Vector memory operations complete in the order they were issued and 25
+        // steps of two stores each follow the tile's last load, so "at most 32 outstanding" covers the loads with a
+        // margin and leaves the youngest stores in flight (a __syncthreads would wait for all of them).
+        if constexpr (DRAIN) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
     if constexpr (DRAIN) {  // the last block (in acc_b)
 #pragma unroll
@@ -1758,12 +1484,6 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
         tq_set_error("tq_score_tile: %lld queries beyond 2^24 - 1", (long long)nq);
         return TQ_ERR_UNSUPPORTED;
     }
-    // the kernel addresses a block of 64 logit rows with 32-bit byte offsets
-    if ((uint64_t)nk * (out_dtype == TQ_F32 ? 4 : 2) * 64 >= 0x7FFFFFFFull) {
-        tq_set_error("tq_score_tile: %lld keys per call beyond %lld (64 rows of logits must stay below 2 GiB): score the keys in slices",
-                     (long long)nk, (long long)(0x7FFFFFFFll / 64 / (out_dtype == TQ_F32 ? 4 : 2)));
-        return TQ_ERR_UNSUPPORTED;
-    }
     __half *qa = reinterpret_cast<__half *>(ws);
     const unsigned qgrid = (unsigned)((nq + 31) / 32);
     const uint4 *wfrag = reinterpret_cast<const uint4 *>(h->score_wfrag);
@@ -1777,42 +1497,21 @@ int tqk_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, c
     if (rc) return rc;
     const unsigned grid = (unsigned)((nk + SCORE_KEYS - 1) / SCORE_KEYS);
     const size_t lds = (size_t)SCORE_KEYS * KT_STRIDE * sizeof(_Float16);
-#define TQ_SCORE(B, T, P, DR)                                                                                          \
+#define TQ_SCORE(B, T, DR)                                                                                             \
     {                                                                                                                  \
-        (void)hipFuncSetAttribute((const void *)k_score_tile<B, T, P, DR>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+        (void)hipFuncSetAttribute((const void *)k_score_tile<B, T, DR>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
                                   (int)lds);                                                                           \
-        k_score_tile<B, T, P, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
-                                                         nq, nk, (T *)logits, (const uint32_t *)h->pair_lut, (float)h->proj_scale);   \
-    }
-#define TQ_SCORE_BITS(T, P, DR)                                                                              \
-    if (h->bits == 2) TQ_SCORE(2, T, P, DR) else if (h->bits == 3) TQ_SCORE(3, T, P, DR) else TQ_SCORE(4, T, P, DR)
-#ifndef TQ_SCORE_COLUMNS
-#define TQ_ROWS(B, T, DR)                                                                                              \
-    {                                                                                                                  \
-        (void)hipFuncSetAttribute((const void *)k_score_rows<B, T, DR>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
-                                  (int)lds);                                                                           \
-        k_score_rows<B, T, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
+        k_score_tile<B, T, DR><<<grid, 512, lds, s>>>(qa, (const uint8_t *)packed, sign_bits, (const __half *)rnorms, \
                                                       nq, nk, (T *)logits, (const uint32_t *)h->pair_lut, (float)h->proj_scale); \
     }
-#define TQ_ROWS_BITS(T, DR)                                                                              \
-    if (h->bits == 2) TQ_ROWS(2, T, DR) else if (h->bits == 3) TQ_ROWS(3, T, DR) else TQ_ROWS(4, T, DR)
+#define TQ_SCORE_BITS(T, DR)                                                                              \
+    if (h->bits == 2) TQ_SCORE(2, T, DR) else if (h->bits == 3) TQ_SCORE(3, T, DR) else TQ_SCORE(4, T, DR)
     if (!logits) {
-        TQ_ROWS_BITS(float, false)
+        TQ_SCORE_BITS(float, false)  // measurement mode: everything but the stores
     } else if (out_dtype == TQ_F32) {
-        TQ_ROWS_BITS(float, true)
+        TQ_SCORE_BITS(float, true)
     } else {
-        TQ_ROWS_BITS(__half, true)
-    }
-    return tq_check_launch("score_tile");
-#endif
-    if (!logits) {
-        TQ_SCORE_BITS(float, false, false)
-    } else if (out_dtype == TQ_F32) {
-        TQ_SCORE_BITS(float, false, true)
-    } else if ((nk & 1) == 0 && (reinterpret_cast<uintptr_t>(logits) & 3u) == 0) {
-        TQ_SCORE_BITS(__half, true, true)
-    } else {
-        TQ_SCORE_BITS(__half, false, true)
+        TQ_SCORE_BITS(__half, true)
     }
 #undef TQ_SCORE_BITS
 #undef TQ_SCORE
