@@ -125,6 +125,23 @@ def measured_peaks_leg(torch, tqa, steps, warmup):
             moved = n * (2 if mode.startswith("copy") else 1)
             best = max(best, moved / (ev_ms * 1e-3) / 1e9)
         out[f"hbm_{mode}_gbs"] = best   # the better of the two access orders
+    # short-lived workgroups in dispatch order (one compact window moving through memory): the read/write mixes of the
+    # fused K+V store at config 2 (128 MiB of fp16 rows in, 13/64 or 17/64 of that out) and the fp32 logits of config 5
+    # (512 MiB written) as bare traffic, the floor a kernel with that traffic and nothing else would reach on this box
+    flat = {}
+    units = (128 << 20) // 16384
+    for name, w64 in (("store_mix_turbo3", 13), ("store_mix_turbo4", 17), ("read_128MiB", 0)):
+        def step(i, w64=w64):
+            probes.probe_flat(bufs[i % 4], bufs[(i + 1) % 4][(512 << 20):], units, w64)
+        _, ev_ms = time_steps(torch, step, steps, warmup)   # short launches: as many as the store legs, past the clock transient
+        moved = units * (16384 + 256 * w64)
+        flat[name] = {"us": ev_ms * 1e3, "gbs": moved / (ev_ms * 1e-3) / 1e9}
+
+    def wstep(i):
+        probes.probe_flat(None, bufs[i % 4], (512 << 20) // 16384, 64)
+    _, ev_ms = time_steps(torch, wstep, max(reps, steps // 4), max(warm, warmup // 4))
+    flat["write_512MiB"] = {"us": ev_ms * 1e3, "gbs": (512 << 20) / (ev_ms * 1e-3) / 1e9}
+    out["flat"] = flat
     del bufs
     sink = torch.zeros(4, dtype=torch.float32, device="cuda")
     flops = [0]

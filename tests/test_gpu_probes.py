@@ -1,4 +1,4 @@
-"""GPU tests of the benchmark's measurement probes (libtq_probe.so: tq_probe_stream, tq_probe_mfma_f16) and of
+"""GPU tests of the benchmark's measurement probes (libtq_probe.so: tq_probe_stream, tq_probe_flat, tq_probe_mfma_f16) and of
 the score tile's store-less mode.  They have no counterpart in the reference: the checks are that the streaming probe
 moves exactly the bytes it is asked to, in both access orders, and that the other two run and report."""
 import numpy as np
@@ -39,6 +39,37 @@ def test_stream_probe_rejects_bad_sizes():
         probes.probe_stream("copy", buf[:24], buf[32:56])
     with pytest.raises(ValueError):
         probes.probe_stream("write", None, None)
+
+
+@pytest.mark.parametrize("w64", [0, 13, 17, 64])
+def test_flat_probe_touches_exactly_its_share(w64):
+    """Every workgroup writes its own write_64ths/64 of 16 KB, back to back with its neighbours', and nothing else;
+    what it writes is the xor of the four chunks a lane read with the lane's fill word."""
+    tt = L.torch()
+    units = 5
+    src = tt.randint(0, 256, (units * 16384,), dtype=tt.uint8, device="cuda")
+    out_bytes = units * 256 * w64
+    dst = tt.full((out_bytes + 64,), 7, dtype=tt.uint8, device="cuda")
+    before = np_(src).copy()
+    probes.probe_flat(src, dst, units, w64)
+    got = np_(dst)
+    assert np.array_equal(np_(src), before)
+    assert (got[out_bytes:] == 7).all(), "wrote past the end"
+    if w64:
+        words = before.view(np.uint32).reshape(units, 4, 256, 4)           # [unit][load][lane][word]
+        acc = words[:, 0] ^ words[:, 1] ^ words[:, 2] ^ words[:, 3]        # [unit][lane][word]
+        acc = acc ^ np.stack([np.arange(256), np.full(256, 1), np.full(256, 2), np.full(256, 3)], axis=1).astype(np.uint32)
+        want = np.stack([acc[u][np.arange(16 * w64) % 256] for u in range(units)])
+        assert np.array_equal(got[:out_bytes].view(np.uint32).reshape(units, 16 * w64, 4), want)
+        # write-only form
+        probes.probe_flat(None, dst, units, w64, nontemporal=False)
+        got = np_(dst)
+        assert (got[out_bytes:] == 7).all()
+        assert (got[:out_bytes].view(np.uint32).reshape(-1, 4)[:, 1:] == [1, 2, 3]).all()
+    with pytest.raises(ValueError):
+        probes.probe_flat(None, None, units, 0)
+    with pytest.raises(ValueError):
+        probes.probe_flat(src, dst, units + 1, w64)
 
 
 def test_mfma_probe_reports_its_work():

@@ -183,4 +183,4 @@ def test_probe_library_is_separate_from_the_codec_abi():
     from turboquant_plus_amd import probes
     assert not any(n.startswith("tq_probe") for n in header_symbols())
     assert not hasattr(L.lib(), "tq_probe_stream")
-    assert hasattr(probes.lib(), "tq_probe_stream") and hasattr(probes.lib(), "tq_probe_mfma_f16")
+    assert all(hasattr(probes.lib(), n) for n in ("tq_probe_stream", "tq_probe_flat", "tq_probe_mfma_f16"))

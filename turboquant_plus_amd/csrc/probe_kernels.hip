@@ -46,6 +46,30 @@ __global__ __launch_bounds__(512) void k_probe_stream(const uint4 *src, uint4 *d
     }
 }
 
+// Short-lived workgroups in dispatch order: workgroup u reads the 16 KB unit u of src (four 16-byte loads per
+// lane, when READS) and writes 16 * W chunks of 16 bytes at dst + u * 16 * W chunks (the first lanes, when W > 0).
+// The memory side sees one compact window that moves through both buffers, which this part serves faster than
+// the strided sweeps of long-lived workgroups above (writes above all).
+template <bool READS, bool NT>
+__global__ __launch_bounds__(256) void k_probe_flat(const u32x4_t *src, u32x4_t *dst, int w64) {
+    const int64_t u = blockIdx.x;
+    u32x4_t acc = {threadIdx.x, 1u, 2u, 3u};
+    if constexpr (READS) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u32x4_t *p = src + u * 1024 + j * 256 + threadIdx.x;
+            acc ^= NT ? __builtin_nontemporal_load(p) : *p;
+        }
+    }
+    for (int c = threadIdx.x; c < 16 * w64; c += 256) {
+        u32x4_t *q = dst + u * 16 * w64 + c;
+        if (NT) __builtin_nontemporal_store(acc, q);
+        else *q = acc;
+    }
+    // keeps the reads alive when nothing is written; the condition does not hold for any data a caller would pass
+    if (READS && w64 == 0 && dst && (acc[0] & acc[1] & acc[2] & acc[3]) == 0xFFFFFFFFu) dst[0] = acc;
+}
+
 // 8 independent accumulator tiles per wavefront, `iters` rounds of one MFMA on each
 __global__ __launch_bounds__(256) void k_probe_mfma(int64_t iters, float *sink) {
     const int lane = threadIdx.x & 63;
@@ -95,6 +119,21 @@ extern "C" int tq_probe_stream(int mode, int chunked, const void *src, void *dst
         default: TQ_PROBE_MODE(5);
     }
 #undef TQ_PROBE_MODE
+    return hipGetLastError() == hipSuccess ? 0 : TQ_PROBE_ERR_HIP;
+}
+
+extern "C" int tq_probe_flat(const void *src, void *dst, int64_t units, int write_64ths, int nontemporal, void *stream) {
+    if (units < 1 || units > 0x7FFFFFFF || write_64ths < 0 || write_64ths > 64 || (!src && write_64ths == 0) || (write_64ths > 0 && !dst))
+        return TQ_PROBE_ERR_ARG;
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) return TQ_PROBE_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const u32x4_t *s4 = (const u32x4_t *)src;
+    u32x4_t *d4 = (u32x4_t *)dst;
+    const unsigned grid = (unsigned)units;
+    if (src && nontemporal) k_probe_flat<true, true><<<grid, 256, 0, s>>>(s4, d4, write_64ths);
+    else if (src) k_probe_flat<true, false><<<grid, 256, 0, s>>>(s4, d4, write_64ths);
+    else if (nontemporal) k_probe_flat<false, true><<<grid, 256, 0, s>>>(s4, d4, write_64ths);
+    else k_probe_flat<false, false><<<grid, 256, 0, s>>>(s4, d4, write_64ths);
     return hipGetLastError() == hipSuccess ? 0 : TQ_PROBE_ERR_HIP;
 }
 

@@ -22,6 +22,13 @@ extern "C" {
  * bytes: a multiple of 16; pointers 16-byte aligned.  stream: hipStream_t.  Returns 0 or a negative code. */
 int tq_probe_stream(int mode, int chunked, const void *src, void *dst, int64_t bytes, void *stream);
 
+/* One launch of `units` short-lived workgroups in dispatch order: workgroup u reads the 16 KB unit u of src
+ * (src == NULL: reads nothing) and writes write_64ths / 64 of 16 KB (0 .. 64; 0: writes nothing) at
+ * dst + u * 256 * write_64ths bytes: a read, a write, or a kernel's mix of the two (13: 3-bit K+V codes from
+ * fp16 rows, 17: 4-bit) as one compact window moving through memory.  nontemporal != 0: the hint on every access.
+ * src: units * 16 KB; dst: units * 256 * write_64ths bytes (16 bytes when write_64ths == 0); 16-byte aligned. */
+int tq_probe_flat(const void *src, void *dst, int64_t units, int write_64ths, int nontemporal, void *stream);
+
 /* One launch of `iters` (1 .. TQ_PROBE_MAX_ITERS) rounds of eight independent v_mfma_f32_32x32x16_f16 per
  * wavefront on every SIMD of the chip.  Returns the floating-point operations launched (> 0) or an error code
  * (< 0).  sink: 4 bytes of device memory (never written for valid inputs). */

@@ -21,6 +21,8 @@ def lib():
         h = C.CDLL(LIB_PATH)
         h.tq_probe_stream.restype, h.tq_probe_stream.argtypes = C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                                                           C.c_int64, C.c_void_p]
+        h.tq_probe_flat.restype, h.tq_probe_flat.argtypes = C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int,
+                                                                      C.c_void_p]
         h.tq_probe_mfma_f16.restype, h.tq_probe_mfma_f16.argtypes = C.c_int64, [C.c_int64, C.c_void_p, C.c_void_p]
         _lib = h
     return _lib
@@ -38,6 +40,20 @@ def probe_stream(mode: str, src, dst, chunked: bool = False):
                                None if dst is None else L.ptr(dst), nbytes, L.stream_ptr())
     if rc:
         raise ValueError(f"tq_probe_stream: bad argument (mode {mode}, {nbytes} bytes)") if rc == -1 else RuntimeError("HIP error")
+
+
+def probe_flat(src, dst, units: int, write_64ths: int, nontemporal: bool = True):
+    """One launch of the flat probe: `units` short-lived workgroups in dispatch order, each reading 16 KB of src
+    (None: no reads) and writing write_64ths/64 of 16 KB of dst (0: no writes).  uint8 device tensors of at least
+    units * 16 KB and units * 256 * write_64ths bytes.  The caller times it."""
+    if src is not None and src.numel() < units * 16384:
+        raise ValueError("probe_flat: src too small")
+    if write_64ths and (dst is None or dst.numel() < units * 256 * write_64ths):
+        raise ValueError("probe_flat: dst too small")
+    rc = lib().tq_probe_flat(None if src is None else L.ptr(src), None if dst is None else L.ptr(dst), units, write_64ths,
+                             int(nontemporal), L.stream_ptr())
+    if rc:
+        raise ValueError("tq_probe_flat: bad argument") if rc == -1 else RuntimeError("HIP error")
 
 
 def probe_mfma_f16(iters: int, sink) -> int:
