@@ -47,7 +47,7 @@ D = 128
 # HBM bytes per launch as recorded in profiles/bench_all_legs_trace_hbm_sq.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
 # this file's run, each scaled by the reading of a 1 GiB device copy): recorded constants, not measured in this run;
 # the JSON line names the profile row next to each figure.
-TRAFFIC_BYTES = {"store4": 169.8e6, "store3": 161.1e6, "decode3": 424.2e6}
+TRAFFIC_BYTES = {"store4": 169.7e6, "store3": 161.1e6, "decode3": 424.2e6}
 _TRAFFIC_FILE = "profiles/bench_all_legs_trace_hbm_sq.txt"
 TRAFFIC_SOURCE = {"store4": _TRAFFIC_FILE + ", row k_store_kv<4, 4, false> of the HBM traffic table (recorded, not measured in this run)",
                   "store3": _TRAFFIC_FILE + ", row k_store_kv<3, 3, false> of the HBM traffic table (recorded, not measured in this run)",
