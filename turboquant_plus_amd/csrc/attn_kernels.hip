@@ -1392,22 +1392,35 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
     float keep = 0.0f;  // measurement mode (no logits): the products stay live through a store that never happens
     // one block of 32 queries (operand block `b` of the tile in `cur`) against the 64 resident keys into acc, while
     // the pending block leaves from pacc; the first block of a tile also asks for the next tile (eight loads that
-    // write LDS directly, one per step: no registers, no LDS write instructions, and a lead of at least 24 steps)
-    auto block = [&](const chunk_t *cur, chunk_t *next, const int b, auto half, const int tile_next, float16_t (&acc)[2],
-                     const float16_t (&pacc)[2], const Pending &pb) __attribute__((always_inline)) {
+    // write LDS directly, one per step: no registers, no LDS write instructions, and a lead of at least 20 steps).
+    // Query operands come from LDS AHEAD steps ahead, across blocks too: `pre` holds the first AHEAD operands of this
+    // block on entry and those of the block that follows (operand block `b_after` of the buffer `after`) on exit.  The
+    // second block of a tile therefore carries the tile's barrier, at the step in which its own last operand read has
+    // been issued: behind it no wavefront reads `cur` any more, so the next tile may start filling it, and `next` is
+    // complete.  Vector memory operations complete in issue order and 21 steps of two stores each lie between a
+    // tile's last load and that step, so "at most 32 outstanding" covers the loads with a margin and leaves the
+    // youngest logit stores in flight (a __syncthreads would wait for all of them).
+    constexpr int AHEAD = 3;
+    auto block = [&](const chunk_t *cur, chunk_t *next, const int b, const chunk_t *after, const int b_after, auto half,
+                     const int tile_next, half8_t (&pre)[AHEAD], float16_t (&acc)[2], const float16_t (&pacc)[2],
+                     const Pending &pb) __attribute__((always_inline)) {
         constexpr int HALF = decltype(half)::value;
         const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         const chunk_t *arow = cur + b * 1024 + lane;
-        // query operands come from LDS AHEAD steps ahead; the scheduling fence after every step keeps the
-        // compiler from hoisting all sixteen steps' reads to the top
-        constexpr int AHEAD = 3;
+        const chunk_t *arow_after = after + b_after * 1024 + lane;
+        // the scheduling fence after every step keeps the compiler from hoisting all sixteen steps' reads to the top
         half8_t af[AHEAD + 1];
 #pragma unroll
-        for (int t = 0; t < AHEAD; ++t) af[t] = __builtin_bit_cast(half8_t, arow[t * 64]);
+        for (int t = 0; t < AHEAD; ++t) af[t] = pre[t];
         uint32_t swapped = 0u;
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             if (t + AHEAD < 16) af[(t + AHEAD) & AHEAD] = __builtin_bit_cast(half8_t, arow[(t + AHEAD) * 64]);
+            if (HALF == 1 && t + AHEAD == 16) {
+                if constexpr (DRAIN) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+            if (t + AHEAD >= 16) pre[t + AHEAD - 16] = __builtin_bit_cast(half8_t, arow_after[(t + AHEAD - 16) * 64]);
             if (HALF == 0 && t < 8) {
                 // lane l of the wavefront brings chunk l of the wavefront's 1 KB piece of chunk group g
                 const int g = t;
@@ -1445,21 +1458,19 @@ __global__ __launch_bounds__(512, 1) void k_score_tile(const __half *qa, const u
         for (int e = 0; e < 16; ++e) acc_b[kh][e] = 0.0f;
     Pending pb = pend(0);
     pb.rows = 0;  // nothing is pending before the first block
+    half8_t pre[AHEAD];
+#pragma unroll
+    for (int t = 0; t < AHEAD; ++t) pre[t] = __builtin_bit_cast(half8_t, qtile[(2 * qh) * 1024 + t * 64 + lane]);
 #pragma unroll 1
     for (int tile = 0; tile < n_tiles; ++tile) {
         const chunk_t *cur = qtile + (tile & 1) * 4096;
         chunk_t *next = qtile + ((tile + 1) & 1) * 4096;
         const int row0 = tile * SCORE_QT + qh * 64;
         const int tile_next = min(tile + 1, n_tiles - 1);  // the last tile re-reads itself
-        block(cur, next, 2 * qh, std::integral_constant<int, 0>{}, tile_next, acc_a, acc_b, pb);
+        block(cur, next, 2 * qh, cur, 2 * qh + 1, std::integral_constant<int, 0>{}, tile_next, pre, acc_a, acc_b, pb);
         pb = pend(row0);
-        block(cur, next, 2 * qh + 1, std::integral_constant<int, 1>{}, tile_next, acc_b, acc_a, pb);
+        block(cur, next, 2 * qh + 1, next, 2 * qh, std::integral_constant<int, 1>{}, tile_next, pre, acc_b, acc_a, pb);
         pb = pend(row0 + 32);
-        // The next tile must have arrived.  Vector memory operations complete in the order they were issued and 25
-        // steps of two stores each follow the tile's last load, so "at most 32 outstanding" covers the loads with a
-        // margin and leaves the youngest stores in flight (a __syncthreads would wait for all of them).
-        if constexpr (DRAIN) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
     if constexpr (DRAIN) {  // the last block (in acc_b)
 #pragma unroll
