@@ -300,6 +300,50 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                     mt[(size_t)k * 128 + j] = acc * rs;
                 }
             rc = rc ? rc : upload(&h->projrot64_t, mt);
+            // The QJL store's projection: 64 M split into three fp16 terms (hi + mid to 2^-22 of the entry, all three to
+            // 2^-31; the factor keeps the middle terms out of fp16's subnormals), laid out as B operands of
+            // v_mfma_f32_16x16x32_f16.  Fragment (step c, column block jb), lane l, element e =
+            // 64 M[j = 16 jb + l % 16][k = 4 (8 c + e) + l / 16]: the contraction runs over the dims in the order in
+            // which a lane of the store kernel holds them.
+            // First pass, matrix cores: the kernel scales a token's residual r by a power of two to x with
+            // 512 <= |x| < 1024, splits x into two fp16 terms and accumulates hi*hi in one fp32 accumulator and
+            // hi*mid + lo*hi in another.  Against the exact sum the result is off by at most
+            //   (128 * 2^-23 [main term: one fp32 rounding per product, taken as truncation, partial sums bounded by
+            //   sum |x_k| |64 M_jk|] + 3 * 2^-22 [both splits and the dropped lo*mid] + 2^-23 [the small terms'
+            //   roundings and the final addition]) * |x| |64 M_j| + 6.8e-4 (|x| + |64 M_j|) [fp16 subnormals of the
+            //   low terms, should the matrix cores flush them]
+            //   <=  (1.61e-5 max_j |64 M_j| + 6.8e-4 (1 + max_j |64 M_j| / 512)) |x|,
+            // so a projection whose fast value is at least qjl_tau |x| (that bound with 2.0e-5 for 1.61e-5) away from
+            // zero has the sign of the exact one.  Second pass, for the few that are closer (about one in 3000): the
+            // float64 residual against hi + mid + lo in float64, off by at most 2^-31 |r| |64 M_j|; qjl_tau2 |r| (twice
+            // that) settles all but one in 10^8 of those, which a third pass takes from the float64 matrix in memory.
+            {
+                std::vector<uint16_t> qf((size_t)3 * 4 * 8 * 64 * 8);
+                const size_t set = (size_t)4 * 8 * 64 * 8;
+                double maxrow = 0.0;
+                for (int j = 0; j < 128; ++j) {
+                    double ss = 0.0;
+                    for (int k = 0; k < 128; ++k) ss += mt[(size_t)k * 128 + j] * mt[(size_t)k * 128 + j];
+                    maxrow = std::max(maxrow, 64.0 * std::sqrt(ss));
+                }
+                for (int c = 0; c < 4; ++c)
+                    for (int jb = 0; jb < 8; ++jb)
+                        for (int l = 0; l < 64; ++l)
+                            for (int e = 0; e < 8; ++e) {
+                                const int j = 16 * jb + (l & 15), k = 4 * (8 * c + e) + (l >> 4);
+                                const double mv = 64.0 * mt[(size_t)k * 128 + j];
+                                const size_t at = ((((size_t)c * 8 + jb) * 64) + l) * 8 + e;
+                                const uint16_t hi = f64_to_f16_bits(mv);
+                                const double r1 = mv - f16_bits_to_f64(hi);
+                                const uint16_t mid = f64_to_f16_bits(r1);
+                                qf[at] = hi;
+                                qf[set + at] = mid;
+                                qf[2 * set + at] = f64_to_f16_bits(r1 - f16_bits_to_f64(mid));
+                            }
+                rc = rc ? rc : upload(&h->qjl_frag, qf);
+                h->qjl_tau = (float)(2.0e-5 * maxrow + 6.8e-4 * (1.0 + maxrow / 512.0));
+                h->qjl_tau2 = 2.0 * std::ldexp(1.0, -31) * maxrow;
+            }
             // Operand fragments of the query preparation (score tile): W = [D2 H D1 ; S] as the row side of
             // 32 x 32 x 16 matrix instructions.  Set 0: the rotation's +-1 entries (its 1/sqrt(128) is applied to the
             // sums), sets 1 and 2: S split into two fp16 terms (S = hi + lo to 2^-22).  Fragment (row block cb, step
@@ -332,7 +376,7 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
 void tq_destroy(tq_handle *h) {
     if (!h) return;
     void *ptrs[] = {h->centroids64, h->bounds64, h->s1_64,  h->s2_64,       h->rot64, h->rot64_t,  h->proj64, h->proj64_t,
-                    h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->score_wfrag,
+                    h->centroids32, h->bounds32, h->s1_32,  h->s2_32,       h->projrot64_t, h->pair_lut, h->score_wfrag, h->qjl_frag,
                     h->symthr32,    h->rfrag16k,    h->sqcoef32, h->s2flip,      h->rfrag16v, h->quant_lut,
                     h->rfrag16k_inv};
     for (void *p : ptrs)

@@ -30,6 +30,9 @@ struct tq_handle {
     double *projrot64_t;   // [128*128] entry [k*128+j] = (S R^T)[j][k]   (d == 128, WHT, projection)
     void *pair_lut;        // [4^bits] half2: (c[lo], c[hi]) for a pair code (bits <= 3), or [256] for 4
     uint32_t pair_lut_host[256];  // host copy of pair_lut (two handles with equal tables can share one LDS copy)
+    uint16_t *qjl_frag;    // [3][4][8][64][8] fp16: 64 (S R^T) split into three fp16 terms, as B operands of 16x16x32 matrix instructions (QJL store)
+    float qjl_tau;         // first pass (fp16 matrix cores): |value| below qjl_tau * |scaled residual| goes to the second pass
+    double qjl_tau2;       // second pass (float64 against the three terms): |value| below qjl_tau2 * |residual| goes to the float64 matrix
     uint16_t *score_wfrag; // [3][4][8][64][8] fp16: operand fragments of [D2 H D1 ; S hi ; S lo] (query preparation, score tile)
     void *rfrag16k;        // [8][64][8] fp16 +-1: fragment f0*4+ks, lane l, element e = s1[k] H[m][k] with
                            // m = 32(l%16/4) + 4 f0 + l%4, k = 32(l/16) + 8 ks + e (factored transform, K rows)

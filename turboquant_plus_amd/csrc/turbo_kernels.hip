@@ -1415,30 +1415,38 @@ __global__ __launch_bounds__(256) void k_append_kv(const TI *xk, uint8_t *pk, Ap
 struct StoreQjlArgs {
     const double *s1, *s2, *bounds, *cent;
     const double *projrot_t;  // [128*128]: entry [k*128+j] = (S R^T)[j][k]
+    const uint4 *frag;        // [3][4][8][64] B operands of the projection: 64 (S R^T) as three fp16 terms
+    float tau;                // first pass: closer to zero than tau * |scaled residual| -> second pass
+    double tau2;              // second pass: closer to zero than tau2 * |residual| -> third pass
     int norm_correction;
     int64_t tokens, blocks_per_seq;
 };
 
-// One workgroup of eight wavefronts per CU with the projection (S R^T, 128 KB of doubles) resident in LDS.  The
-// wavefronts are independent after the matrix is in place: each takes units of 16 tokens (a strided share), lane
-// (token n16, quarter kq) holding the 32 dims d = 4 s + kq.  Norms and the first two butterfly stages (in the
-// reference's stage order) exchange across the lane quarters, the other five stages are in-lane, and the residual
-// in the rotated domain, taken against the reconstruction the decoder will see (stored fp16 norm), is at once the
-// A operand of v_mfma_f64_16x16x4_f64: 256 of them per unit against the matrix in LDS.  No barrier ties the
-// wavefronts together, and the next unit's input is requested before the matrix phase starts.  The sign bits of a
-// token's 16 projections of one column block are one quarter of a ballot.  A wavefront packs its own 16 rows (rows
-// of a K block are independent).
-// Matrix rows k and k + 1 hold their 16-column groups in swapped order (column j of row k at j ^ 16 (k & 1)): the
-// two lane quarters that share a pass of an 8-byte LDS read then hit different halves of the banks.
-// (Float64 matrix instructions and float64 vector instructions do not overlap on this chip: staggering the two
-// wavefronts of a SIMD so that one's vector phase falls into the other's matrix phase gains nothing, measured.)
+// One workgroup of eight wavefronts per CU.  The wavefronts are independent after the constants are in place: each
+// takes units of 16 tokens (a strided share), lane (token n16, quarter kq) holding the 32 dims d = 4 s + kq.  Norms
+// and the first two butterfly stages (in the reference's stage order) exchange across the lane quarters, the other
+// five stages are in-lane, all in float64, and so is the residual in the rotated domain, taken against the
+// reconstruction the decoder will see (stored fp16 norm).
+// Only the signs of the 128 projections (S R^T) r are stored, so the projection runs on the fp16 matrix cores with an
+// error bound instead of on the float64 ones: the residual is scaled by a power of two to 512 <= |x| < 1024 and split
+// into two fp16 terms, the matrix (times 64) was split into three when the handle was made (96 KB in LDS, laid out
+// as B operands; the contraction runs over the dims in the order a lane holds them, so the A operands are the lane's
+// own values), and hi*hi + hi*mid + lo*hi accumulate in fp32 on v_mfma_f32_16x16x32_f16: 96 instructions of 16
+// clocks per unit instead of 256 float64 ones of 64 clocks.  A result at least tau |x| away from zero (the bound on
+// this pass's error, worked out where the handle is made) has the exact projection's sign.  The others, about one
+// per unit, get a second pass: the four lanes that hold the token multiply its float64 residual with hi + mid + lo,
+// read from the same LDS, in float64 (error 2^-31 relative); the one in 10^8 of those that is still too close goes
+// to the float64 matrix in memory.
+// The sign bits of a token's 16 projections of one column block are one quarter of a ballot.  A wavefront packs its
+// own 16 rows (rows of a K block are independent).  No barrier ties the wavefronts together, and the next unit's
+// input is requested before the matrix phase starts.
 typedef double double4_t __attribute__((ext_vector_type(4)));
 template <int BITS, typename TI>
 __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *packed, uint8_t *sign_bits, __half *rnorms,
                                                        StoreQjlArgs a, int64_t n_blocks) {
     using namespace tq64;
     constexpr int NB = (1 << BITS) - 1;
-    extern __shared__ double mat_s[];  // [k][j ^ 16 (k & 1)] = (S R^T)[j][k]
+    extern __shared__ uint4 frag_s[];  // [3 terms][4 steps][8 column blocks][64 lanes]: B operands of the projection
     __shared__ __attribute__((aligned(16))) uint8_t codes_s[8][16 * CODE_STRIDE];
     __shared__ double cent_s[1 << BITS];
 
@@ -1464,17 +1472,13 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
     };
     fetch(unit);
 
-    // the matrix is fetched once per workgroup, sixteen 16-byte pieces per thread, eight in flight at a time
+    // the matrix operands are fetched once per workgroup, twelve 16-byte pieces per thread
+    {
+        uint4 piece[12];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        double2 piece[8];
+        for (int i = 0; i < 12; ++i) piece[i] = a.frag[tid + 512 * i];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const double2 *>(a.projrot_t)[tid + 512 * (8 * b + i)];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int pi = tid + 512 * (8 * b + i);  // row pi / 64, columns 2 (pi % 64), + 1
-            reinterpret_cast<double2 *>(mat_s)[pi ^ (((pi >> 6) & 1) << 3)] = piece[i];
-        }
+        for (int i = 0; i < 12; ++i) frag_s[tid + 512 * i] = piece[i];
     }
     if (tid < (1 << BITS)) cent_s[tid] = a.cent[tid];
     // the boundaries stay in registers (the byte stores of the code stage may alias anything as far as the compiler
@@ -1599,28 +1603,104 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
         __builtin_amdgcn_wave_barrier();
         // the next unit's input is under way while the matrix phase runs
         fetch(unit + unit_step);
-        // (S R^T) e for the 16 tokens: D[token][j] += E[token][k] M[k][j], 8 column blocks x 32 steps of 4
-        double4_t acc[8];
-#pragma unroll
-        for (int jb = 0; jb < 8; ++jb) acc[jb] = double4_t{0.0, 0.0, 0.0, 0.0};
+        // the residual as fp16 pairs: x = e * 2^p with |x| < 1024 (p from the token's residual norm), x = hi + lo
+        int ex;
+        (void)frexp(rnorm, &ex);
+        const double pw = ldexp(1.0, 10 - ex);
+        half8_t xh[4], xl[4];
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
-            const double *mrow = mat_s + (4 * s + kq) * 128 + n16;
-#pragma unroll
-            for (int jb = 0; jb < 8; ++jb)
-                acc[jb] = __builtin_amdgcn_mfma_f64_16x16x4f64(e[s], mrow[16 * (jb ^ (kq & 1))], acc[jb], 0, 0, 0);
+            const float xf = (float)(e[s] * pw);
+            const _Float16 hi = (_Float16)xf;
+            xh[s >> 3][s & 7] = hi;
+            xl[s >> 3][s & 7] = (_Float16)(xf - (float)hi);
         }
-        // lane (n16, kq) now holds the projections j = 16 jb + n16 of tokens 4 i + kq (register i of the result)
+        // first-pass threshold of this lane's token (0 for a token without a residual: nothing to recompute)
+        const float tau_own = a.tau * (float)(rnorm * pw);
+        // (S R^T) x for the 16 tokens: D[token][j] += X[token][k] M[k][j], 8 column blocks x 4 steps of 32 dims
+        // (the two small terms have an accumulator of their own: the rounding of their 256 additions is then
+        // relative to sums 2^-10 of the main term's and drops out of the error bound)
+        float4_t acc[8], acc_s[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t piece = 0;
+        for (int jb = 0; jb < 8; ++jb) acc[jb] = acc_s[jb] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
 #pragma unroll
             for (int jb = 0; jb < 8; ++jb) {
-                const uint64_t m = __builtin_amdgcn_ballot_w64(acc[jb][i] >= 0.0);
-                if (n16 == jb) piece = (uint32_t)(m >> (16 * kq)) & 0xFFFFu;
+                const half8_t mh = __builtin_bit_cast(half8_t, frag_s[(c * 8 + jb) * 64 + lane]);
+                const half8_t ml = __builtin_bit_cast(half8_t, frag_s[2048 + (c * 8 + jb) * 64 + lane]);
+                acc_s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl[c], mh, acc_s[jb], 0, 0, 0);
+                acc_s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh[c], ml, acc_s[jb], 0, 0, 0);
+                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh[c], mh, acc[jb], 0, 0, 0);
             }
-            const int64_t tk = tok0 + u * 16 + 4 * i + kq;
-            if (n16 < 8 && tk < a.tokens) reinterpret_cast<uint16_t *>(sign_bits)[(row0 + tk) * 8 + n16] = (uint16_t)piece;
+        }
+#pragma unroll
+        for (int jb = 0; jb < 8; ++jb) acc[jb] += acc_s[jb];
+        // lane (n16, kq) now holds the projections j = 16 jb + n16 of tokens 4 kq + i (register i of the result).
+        // The sign bits of token 4 kq + i, column block jb, are a quarter of a ballot; lane (jb, kq) collects them for
+        // its four tokens in `signs` (16 bits per i).  `doubt` marks this lane's results that are too close to zero
+        // for the first pass to settle the sign (bit 31 - (8 i + jb)).
+        uint64_t signs = 0;
+        uint32_t doubt = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float tau_i = __shfl(tau_own, 4 * kq + i);  // of token 4 kq + i (held by lane quarter 0)
+#pragma unroll
+            for (int jb = 0; jb < 8; ++jb) {
+                const uint64_t m = __builtin_amdgcn_ballot_w64(acc[jb][i] >= 0.0f);
+                if (n16 == jb) signs |= (uint64_t)((uint32_t)(m >> (16 * kq)) & 0xFFFFu) << (16 * i);
+                doubt = (doubt << 1) | (fabsf(acc[jb][i]) < tau_i ? 1u : 0u);
+            }
+        }
+        // The doubtful ones: one loop for all of them (wave-uniform control flow), the work done by the four lanes
+        // that hold the token's residual.
+        uint64_t who = __builtin_amdgcn_ballot_w64(doubt != 0u);
+#pragma unroll 1
+        while (who) {
+            const int l = __builtin_ctzll(who);
+            who &= who - 1;
+            uint32_t bits = (uint32_t)__builtin_amdgcn_readlane((int)doubt, l);
+#pragma unroll 1
+            while (bits) {
+                const int idx = __builtin_clz(bits);  // 8 i + jb
+                bits &= ~(0x80000000u >> idx);
+                const int i = idx >> 3, jb = idx & 7;
+                const int tokl = 4 * (l >> 4) + i, j = 16 * jb + (l & 15);
+                // second pass: e . (hi + mid + lo) in float64; this lane's 32 dims are its own elements of the fragments
+                double part = 0.0;
+                if (n16 == tokl) {
+                    const uint4 *fr = frag_s + jb * 64 + 16 * kq + (l & 15);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const half8_t m1 = __builtin_bit_cast(half8_t, fr[c * 512]);
+                        const half8_t m2 = __builtin_bit_cast(half8_t, fr[2048 + c * 512]);
+                        const half8_t m3 = __builtin_bit_cast(half8_t, fr[4096 + c * 512]);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
+                            part = fma(e[8 * c + k], (double)((float)m1[k] + (float)m2[k]) + (double)(float)m3[k], part);
+                    }
+                }
+                part = quarter_sum(part);
+                double settled = __shfl(part, tokl);
+                const double rn_tok = __shfl(rnorm, tokl);
+                if (fabs(settled) < a.tau2 * rn_tok) {  // third pass (wave-uniform: every lane holds the same values)
+                    part = 0.0;
+                    if (n16 == tokl) {
+#pragma unroll
+                        for (int s = 0; s < 32; ++s) part = fma(e[s], a.projrot_t[(4 * s + kq) * 128 + j], part);
+                    }
+                    part = quarter_sum(part);
+                    settled = __shfl(part, tokl);
+                }
+                const int holder = 16 * (l >> 4) + jb, bit = 16 * i + (l & 15);  // where the first pass put the sign
+                if (lane == holder && (((signs >> bit) & 1ull) != 0ull) != (settled >= 0.0)) signs ^= 1ull << bit;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t tk = tok0 + u * 16 + 4 * kq + i;
+            if (n16 < 8 && tk < a.tokens)
+                reinterpret_cast<uint16_t *>(sign_bits)[(row0 + tk) * 8 + n16] = (uint16_t)(signs >> (16 * i));
         }
     }
 }
@@ -2326,16 +2406,19 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
     if (sign_bits) {
-        if (!h->has_proj || !h->projrot64_t) {
+        if (!h->has_proj || !h->projrot64_t || !h->qjl_frag) {
             tq_set_error("tq_store_qjl: handle has no projection");
             return TQ_ERR_ARG;
         }
         StoreQjlArgs a;
         a.s1 = h->s1_64; a.s2 = h->s2_64; a.bounds = h->bounds64; a.cent = h->centroids64;
         a.projrot_t = h->projrot64_t;
+        a.frag = reinterpret_cast<const uint4 *>(h->qjl_frag);
+        a.tau = h->qjl_tau;
+        a.tau2 = h->qjl_tau2;
         a.norm_correction = h->norm_correction;
         a.tokens = tokens; a.blocks_per_seq = bps;
-        constexpr int MAT_BYTES = 128 * 128 * (int)sizeof(double);
+        constexpr int MAT_BYTES = 3 * 4 * 8 * 64 * 16;
         const unsigned qgrid = grid < 256u ? grid : 256u;  // one workgroup per CU (the matrix fills its LDS), looping over blocks
 #define TQ_STOREQ_BITS(B)                                                                                          \
     DISPATCH_T(in_dtype, TI,                                                                                       \
