@@ -325,6 +325,59 @@ def test_store_qjl_matches_oracle(projection, bits):
     assert np_(rn)[4] == 0 and g[4] == 0
 
 
+def _qjl_reference(codec, x):
+    idx_o, g_o, _ = O.turbo_encode(x, codec.signs1, codec.signs2, codec.centroids)
+    resid = x.astype(np.float64) - O.turbo_decode(idx_o, g_o, codec.centroids, codec.signs1, codec.signs2)
+    return resid, resid @ codec.S.T
+
+
+def test_store_qjl_signs_at_volume():
+    """A million projections: some hundreds of them fall inside the fp16 matrix-core pass's error bound and are
+    settled by the float64 pass.  Same bar as above: a sign may differ from the oracle's only inside the 1e-6 band."""
+    codec = tqa.TurboCodec(3, seed=42, projection="gaussian", projection_seed=2)
+    x = np.random.default_rng(19).standard_normal((8192, D)).astype(np.float32)
+    x *= np.exp(np.random.default_rng(20).uniform(-6, 6, (8192, 1))).astype(np.float32)  # norms over five decades
+    _, sbits, _ = codec.store_qjl(x)
+    resid, proj = _qjl_reference(codec, x)
+    z = np.unpackbits(np_(sbits), axis=1, bitorder="little")[:, :D].astype(np.int64) * 2 - 1
+    bad = z != np.where(proj >= 0, 1, -1)
+    band = 1e-6 * np.linalg.norm(resid, axis=1, keepdims=True) / np.sqrt(D) * np.ones_like(proj)
+    assert np.all(np.abs(proj)[bad] <= band[bad]), "sign mismatch outside the band"
+    assert bad.sum() <= 4
+    # the first pass alone would not do: there are projections far outside the band that it cannot settle
+    rel = np.abs(proj) / (np.linalg.norm(resid, axis=1, keepdims=True) * np.linalg.norm(codec.S, axis=1)[None, :])
+    assert (rel < 1e-5).sum() > 50 and (rel[rel < 1e-5] > 1e-7).any()
+
+
+def test_store_qjl_sign_passes():
+    """Projection rows built to end in each of the three passes of the sign computation: a zero row (exactly 0 in
+    every pass: 'not negative'), a row and its negative (opposite signs), a row scaled by 1e-4 (inside the first
+    pass's bound, settled by the float64 pass against the split matrix) and one scaled by 1e-9 (inside the second
+    pass's bound too, settled by the float64 matrix).  Scaled rows must give the signs of the unscaled row."""
+    codec = tqa.TurboCodec(3, seed=42, projection="gaussian", projection_seed=2)
+    S = codec.S.copy()
+    S[0] = 0.0
+    S[2] = -S[1]
+    S[3] = 1e-4 * S[5]
+    S[4] = 1e-9 * S[6]
+    codec.S = S
+    x = np.random.default_rng(21).standard_normal((2048, D)).astype(np.float32)
+    x[7] = 0
+    _, sbits, _ = codec.store_qjl(x)
+    resid, proj = _qjl_reference(codec, x)
+    z = np.unpackbits(np_(sbits), axis=1, bitorder="little")[:, :D].astype(np.int64) * 2 - 1
+    assert (z[:, 0] == 1).all()
+    assert (z[7] == 1).all()                       # a zero key: every projection is exactly 0
+    live = np.arange(2048) != 7
+    rn = np.linalg.norm(resid, axis=1)
+    for scaled, plain in ((3, 5), (4, 6), (2, 1)):
+        want = np.where(proj[:, plain] >= 0, 1, -1) * (-1 if scaled == 2 else 1)
+        clear = live & (np.abs(proj[:, plain]) > 1e-9 * rn * np.linalg.norm(S[plain]))
+        assert clear.sum() > 2000
+        assert np.array_equal(z[clear, scaled], want[clear]), scaled
+        assert np.array_equal(z[clear, plain], np.where(proj[clear, plain] >= 0, 1, -1))
+
+
 # ---- q8_0-style K blocks ----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("tokens", [128, 200])
