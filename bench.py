@@ -349,7 +349,8 @@ def score_tile_leg(torch, tqa, steps, warmup):
     out = {"workload": "TurboQuant estimator tile, 65536 keys (3-bit + QJL, gaussian S seed 2) x 2048 fp16 queries"}
     _, q_ms = time_steps(torch, lambda i: codec.store_qjl(keys), max(5, steps // 20), max(2, warmup // 20))
     out["qjl_store"] = {"us_per_call": q_ms * 1e3, "keys_per_s": nk / (q_ms * 1e-3),
-                        "what": "codes + corrected norm + residual norm + 128 sign bits per key, float64 arithmetic"}
+                        "what": "codes + corrected norm + residual norm + 128 sign bits per key; float64 arithmetic, the sign "
+                                "sketch on the fp16 matrix cores with an error bound and a float64 second pass"}
     flops = 2.0 * nq * nk * 256
     for name, dt in (("fp32_logits", torch.float32), ("fp16_logits", torch.float16)):
         logits = None
