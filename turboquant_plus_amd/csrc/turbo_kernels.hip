@@ -1640,7 +1640,7 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
         // The sign bits of token 4 kq + i, column block jb, are a quarter of a ballot; lane (jb, kq) collects them for
         // its four tokens in `signs` (16 bits per i).  `doubt` marks this lane's results that are too close to zero
         // for the first pass to settle the sign (bit 31 - (8 i + jb)).
-        uint64_t signs = 0;
+        uint32_t piece[4] = {0u, 0u, 0u, 0u};
         uint32_t doubt = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -1648,10 +1648,11 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
 #pragma unroll
             for (int jb = 0; jb < 8; ++jb) {
                 const uint64_t m = __builtin_amdgcn_ballot_w64(acc[jb][i] >= 0.0f);
-                if (n16 == jb) signs |= (uint64_t)((uint32_t)(m >> (16 * kq)) & 0xFFFFu) << (16 * i);
+                if (n16 == jb) piece[i] = (uint32_t)(m >> (16 * kq));
                 doubt = (doubt << 1) | (fabsf(acc[jb][i]) < tau_i ? 1u : 0u);
             }
         }
+        uint64_t signs = (uint64_t)((piece[0] & 0xFFFFu) | (piece[1] << 16)) | ((uint64_t)((piece[2] & 0xFFFFu) | (piece[3] << 16)) << 32);
         // The doubtful ones: one loop for all of them (wave-uniform control flow), the work done by the four lanes
         // that hold the token's residual.
         uint64_t who = __builtin_amdgcn_ballot_w64(doubt != 0u);
