@@ -194,6 +194,9 @@ int tq_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int6
  * sign_bits [n,16] uint8: bit j%8 of byte j/8 is set when (S r)_j >= 0 (zero maps
  * to +1 as in qjl.py:89-90); rnorms [n] fp16 = ||residual||.  The handle needs a
  * projection.  n = n_seqs*tokens rows; sign_bits / rnorms are in token order.
+ * Codes, norms and the residual are computed in float64; a sign bit is the sign of
+ * the float64 projection (taken from an fp16 matrix-core pass where that pass's error
+ * bound settles it, recomputed in float64 where it does not).
  * The k argument of TQ_KFMT_Q8_0 attention is a tq_q8_0_store buffer. */
 int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed,
                  uint8_t *sign_bits, void *rnorms_f16, void *stream);
