@@ -166,6 +166,15 @@ __device__ __forceinline__ uint32_t ko_append4(uint32_t w, float y0, float y1, f
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
+// a * s + b per element (the table path of 4-bit codes normalises inside the last butterfly stage: two products and
+// four fused multiply-adds per four outputs instead of four additions and four products)
+__device__ __forceinline__ float4_t fma4(float4_t a, float4_t s, float4_t b) {
+    float4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = __builtin_fmaf(a[i], s[i], b[i]);
+    return r;
+}
+
 // ---- K2, fp16 input, K rows: codes packed in registers ---------------------------------
 // Index bits of H128[m][k] = (-1)^popcount(m & k) pair up, so the transform splits as
 //   m = 32c + 8fh + 4f0 + i  (c = lane quarter, fh/f0 = fragment, i = row in the lane)
@@ -552,14 +561,24 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #pragma unroll
             for (int f0 = 0; f0 < 2; ++f0) {
 #if TQ_KNOCKOUT & 2
-                y[0 + f0] = q[f0][0]; y[2 + f0] = q[f0][1]; y[4 + f0] = q[f0][2]; y[6 + f0] = q[f0][3];
+                const float ko_s = BITS == 4 ? inv : 1.0f;  // the table path expects normalised values
+                y[0 + f0] = q[f0][0] * ko_s; y[2 + f0] = q[f0][1] * ko_s; y[4 + f0] = q[f0][2] * ko_s; y[6 + f0] = q[f0][3] * ko_s;
 #else
                 const float4_t s01 = q[f0][0] + q[f0][1], d01 = q[f0][0] - q[f0][1];
                 const float4_t s23 = q[f0][2] + q[f0][3], d23 = q[f0][2] - q[f0][3];
-                y[0 + f0] = s01 + s23;
-                y[2 + f0] = d01 + d23;
-                y[4 + f0] = s01 - s23;
-                y[6 + f0] = d01 - d23;
+                if constexpr (BITS == 4) {  // the table is indexed by the normalised value
+                    const float4_t iv = {inv, inv, inv, inv};
+                    const float4_t s23i = s23 * iv, d23i = d23 * iv;
+                    y[0 + f0] = fma4(s01, iv, s23i);
+                    y[2 + f0] = fma4(d01, iv, d23i);
+                    y[4 + f0] = fma4(s01, iv, -s23i);
+                    y[6 + f0] = fma4(d01, iv, -d23i);
+                } else {
+                    y[0 + f0] = s01 + s23;
+                    y[2 + f0] = d01 + d23;
+                    y[4 + f0] = s01 - s23;
+                    y[6 + f0] = d01 - d23;
+                }
 #endif
             }
             // value v = 0..31 of this lane (dim 32*kc + v) up to the sign s2
@@ -599,7 +618,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
                     uint2 e[8];
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
-                        yn[m] = val(v + m) * inv;
+                        yn[m] = val(v + m);  // normalised in the butterfly
 #if TQ_KNOCKOUT & 1
                         if (m == 0)
 #endif
@@ -939,10 +958,11 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 const float4_t s01 = qq[d0][0] + qq[d0][1], d01 = qq[d0][0] - qq[d0][1];
                 const float4_t s23 = qq[d0][2] + qq[d0][3], d23 = qq[d0][2] - qq[d0][3];
                 if constexpr (BITS == 4) {  // the table is indexed by the normalised value
-                    y[0][d0] = (s01 + s23) * inv;
-                    y[1][d0] = (d01 + d23) * inv;
-                    y[2][d0] = (s01 - s23) * inv;
-                    y[3][d0] = (d01 - d23) * inv;
+                    const float4_t s23i = s23 * inv, d23i = d23 * inv;
+                    y[0][d0] = fma4(s01, inv, s23i);
+                    y[1][d0] = fma4(d01, inv, d23i);
+                    y[2][d0] = fma4(s01, inv, -s23i);
+                    y[3][d0] = fma4(d01, inv, -d23i);
                 } else {
                     y[0][d0] = s01 + s23;
                     y[1][d0] = d01 + d23;
