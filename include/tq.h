@@ -128,6 +128,18 @@ int tq_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, 
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                 int64_t tokens, int in_dtype, void *packed_k, void *packed_v, void *stream);
 
+/* Prefill of a growing cache: tq_store_kv of the `tokens` tokens of every sequence into buffers laid out
+ * for `capacity` tokens per sequence (tq_packed_bytes(bits, n_seqs, capacity), the layout tq_append_kv and
+ * tq_decode_attention use), written from position 0.  Sequence i's first ceil(tokens/128) blocks hold the
+ * same bytes that tq_store_kv writes for it (positions past `tokens` in the last of them hold the code of
+ * a zero vector, as after tq_append_kv); the other blocks are not touched.  Same kernels and speed as
+ * tq_store_kv for fp16 input; where that call falls back to the butterfly kernels this one runs
+ * tq_append_kv from position 0.  No counterpart in the reference, whose cache (kv_cache.py:41-66) is
+ * rebuilt from whole tensors. */
+int tq_store_kv_cache(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
+                      int64_t tokens, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, void *stream);
+
+
 /* Streaming append: n_new tokens per sequence at token positions pos .. pos+n_new-1 of a
  * packed buffer laid out for `capacity` tokens per sequence (tq_packed_bytes(bits, n_seqs,
  * capacity)); x is [n_seqs, n_new, 128].  The per-token compress step that kv_cache.py:65-66

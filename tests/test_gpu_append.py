@@ -372,3 +372,86 @@ def test_store_into_a_capacity_buffer_is_rejected_for_several_sequences():
         kc.store_kv(vc, x, x, out_k=cache, out_v=cache.clone())
     one = kc.store(x[:1], kind="k", out=cache)           # a single sequence has no stride: allowed
     assert one is cache
+
+
+@pytest.mark.parametrize("kb,vb", [(3, 3), (4, 4), (3, 2)])
+@pytest.mark.parametrize("tokens", [64, 200, 256])
+def test_prefill_into_a_cache_laid_out_for_more_tokens(kb, vb, tokens):
+    """tq_store_kv_cache: fp16 prompts go through the matrix-core store straight into buffers laid out for `capacity`
+    tokens per sequence.  Every sequence's first blocks hold the bytes tq_store_kv writes for it, the other blocks stay
+    untouched, and the cache then grows by appends as one that was filled by appends: the prefix is kept bit for bit and
+    the appended token gets the same codes."""
+    tt = L.torch()
+    n_seqs, capacity = 3, 512
+    kc, vc = tqa.TurboCodec(kb, seed=42), tqa.TurboCodec(vb, seed=542)
+    rng = np.random.default_rng(100 * kb + tokens)
+    k = rng.standard_normal((n_seqs, tokens + 1, D)).astype(np.float16)
+    v = rng.standard_normal((n_seqs, tokens + 1, D)).astype(np.float16)
+    ck = tt.full((tqa.packed_bytes(kb, n_seqs, capacity),), 0xA5, dtype=tt.uint8, device="cuda")
+    cv = tt.full((tqa.packed_bytes(vb, n_seqs, capacity),), 0xA5, dtype=tt.uint8, device="cuda")
+    kc.store_kv(vc, k[:, :tokens], v[:, :tokens], out_k=ck, out_v=cv, capacity=capacity)
+    pk, pv = kc.store_kv(vc, k[:, :tokens], v[:, :tokens])
+    nb = -(-tokens // 128)
+    for bits, cache, plain in ((kb, ck, pk), (vb, cv, pv)):
+        got = np_(cache).reshape(n_seqs, capacity // 128, -1)
+        assert np.array_equal(got[:, :nb], np_(plain).reshape(n_seqs, nb, -1))
+        assert (got[:, nb:] == 0xA5).all(), "touched a block past the prompt"
+    # grow both this cache and one filled by appends (zeroed, as new_cache() hands them out) by one token
+    ak = tt.zeros_like(ck)
+    av = tt.zeros_like(cv)
+    kc.append_kv(vc, k[:, :tokens], v[:, :tokens], ak, av, 0, capacity)
+    for a, b in ((ck, cv), (ak, av)):
+        kc.append_kv(vc, k[:, tokens:], v[:, tokens:], a, b, tokens, capacity)
+    for codec, kind, mine, theirs, plain in ((kc, "k", ck, ak, pk), (vc, "v", cv, av, pv)):
+        idx_m, g_m = (np_(t) for t in codec.unpack_codes(mine, n_seqs, capacity, kind=kind))
+        idx_t, g_t = (np_(t) for t in codec.unpack_codes(theirs, n_seqs, capacity, kind=kind))
+        idx_p, g_p = (np_(t) for t in codec.unpack_codes(plain, n_seqs, tokens, kind=kind))
+        assert np.array_equal(idx_m[:, :tokens], idx_p) and np.array_equal(g_m[:, :tokens], g_p), "the append moved the prefix"
+        assert np.array_equal(idx_m[:, tokens], idx_t[:, tokens]) and np.array_equal(g_m[:, tokens], g_t[:, tokens])
+        # matrix-core store against butterfly append of the same fp16 rows: the same codes but for values at a boundary
+        assert (idx_m[:, :tokens] != idx_t[:, :tokens]).mean() < 1e-4
+
+
+def test_prefill_falls_back_to_the_append_for_fp32_rows_and_checks_its_arguments():
+    tt = L.torch()
+    n_seqs, tokens, capacity = 2, 150, 384
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    rng = np.random.default_rng(8)
+    k = rng.standard_normal((n_seqs, tokens, D)).astype(np.float32)
+    v = rng.standard_normal((n_seqs, tokens, D)).astype(np.float32)
+    ck, cv = (tt.zeros(tqa.packed_bytes(3, n_seqs, capacity), dtype=tt.uint8, device="cuda") for _ in range(2))
+    ak, av = tt.zeros_like(ck), tt.zeros_like(cv)
+    kc.store_kv(vc, k, v, out_k=ck, out_v=cv, capacity=capacity)
+    kc.append_kv(vc, k, v, ak, av, 0, capacity)
+    assert np.array_equal(np_(ck), np_(ak)) and np.array_equal(np_(cv), np_(av))
+    with pytest.raises(ValueError):
+        kc.store_kv(vc, k, v, out_k=ck, out_v=cv, capacity=tokens - 1)
+    with pytest.raises(ValueError):
+        kc.store_kv(vc, k, v, out_k=ck[:-128], out_v=cv, capacity=capacity)
+    with pytest.raises(ValueError):
+        kc.store_kv(vc, k, v, capacity=capacity)
+
+
+@pytest.mark.parametrize("fmt", [("turbo3", "turbo3"), ("q8_0", "turbo2")])
+def test_layer_prefill_then_decode(fmt):
+    """LayerKV.prefill (fp16 prompt) followed by single-token appends: attention over the growing cache against the
+    oracle on the same buffers' codes."""
+    from test_gpu_attention import assert_close, reference_attention
+    B, Hq, Hkv, capacity, prompt = 2, 8, 2, 384, 200
+    layer = tqa.LayerKV(tqa.LayerFormat(*fmt), seed=3)
+    rng = np.random.default_rng(13)
+    k = rng.standard_normal((B * Hkv, prompt + 3, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, prompt + 3, D)).astype(np.float16)
+    kc, vc = layer.new_cache(B * Hkv, capacity)
+    layer.prefill(k[:, :prompt], v[:, :prompt], kc, vc, capacity)
+    attn = layer.attention(B, Hq, Hkv, prompt, n_splits=2, capacity=capacity)
+    pos = prompt
+    for _ in range(3):
+        layer.append(k[:, pos:pos + 1], v[:, pos:pos + 1], kc, vc, pos, capacity)
+        pos += 1
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    attn.set_tokens(pos)
+    out = np_(attn(q, kc, vc)).copy()
+    ref, _, _ = reference_attention(q, layer.k_codec, layer.v_codec, kc, vc, B, Hq, Hkv, pos, 1 / np.sqrt(D), capacity=capacity,
+                                    k_q8=kc if layer.k_codec is None else None, v_q8=vc if layer.v_codec is None else None)
+    assert_close(out, ref)

@@ -22,23 +22,25 @@ def np_(t):
 
 
 def reference_attention(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, n_splits=1, tau=0.0, bias=None,
-                        k_q8=None, v_q8=None):
-    """Oracle attention on the GPU-stored codes -> (out [B,Hq,128], skip rate, final-weight rate)."""
+                        k_q8=None, v_q8=None, capacity=None):
+    """Oracle attention on the GPU-stored codes -> (out [B,Hq,128], skip rate, final-weight rate).
+    capacity: the buffers are caches laid out for that many tokens per sequence, of which the first N count."""
     G = Hq // Hkv
+    L_ = N if capacity is None else capacity   # tokens per sequence the buffers are laid out for
     if k_q8 is None:
-        ki, kg = kc.unpack_codes(k_packed, B * Hkv, N, kind="k")
-        k_rot = O.turbo_decode_rotated(np_(ki), np_(kg).astype(np.float64), kc.centroids)
+        ki, kg = kc.unpack_codes(k_packed, B * Hkv, L_, kind="k")
+        k_rot = O.turbo_decode_rotated(np_(ki)[:, :N], np_(kg)[:, :N].astype(np.float64), kc.centroids)
         q_rot = O.rotate_fast(q.astype(np.float64), kc.signs1, kc.signs2, D)
     else:
-        qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, N)
-        k_rot = O.q8_0_dequantize(np_(qq), np_(ss))
+        qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, L_)
+        k_rot = O.q8_0_dequantize(np_(qq), np_(ss))[:, :N]
         q_rot = q.astype(np.float64)
     if v_q8 is None:
-        vi, vg = vc.unpack_codes(v_packed, B * Hkv, N, kind="v")
-        v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids)
+        vi, vg = vc.unpack_codes(v_packed, B * Hkv, L_, kind="v")
+        v_rot = O.turbo_decode_rotated(np_(vi)[:, :N], np_(vg)[:, :N].astype(np.float64), vc.centroids)
     else:  # q8_0-style V: stored unrotated
-        qq, ss = tqa.q8_0_unpack(v_q8, B * Hkv, N, kind="v")
-        v_rot = O.q8_0_dequantize(np_(qq), np_(ss))
+        qq, ss = tqa.q8_0_unpack(v_q8, B * Hkv, L_, kind="v")
+        v_rot = O.q8_0_dequantize(np_(qq), np_(ss))[:, :N]
     out = np.zeros((B, Hq, D))
     skipped = below = 0.0
     for b in range(B):

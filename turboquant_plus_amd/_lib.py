@@ -58,6 +58,7 @@ PROTOTYPES = {
     "tq_packed_bytes": (_L, [C.c_int32, _L, _L]),
     "tq_store": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
     "tq_store_kv": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P]),
+    "tq_store_kv_cache": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _P, _P, _P]),
     "tq_append": (_I, [_P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_append_kv": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _P, _P]),
     "tq_requantize": (_I, [_P, _P, _P, _L, _L, _I, _P, _P]),

@@ -578,7 +578,22 @@ int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const v
     REQUIRE(k && v && packed_k && packed_v, TQ_ERR_ARG, "tq_store_kv: null pointer");
     REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
             "tq_store_kv: inputs and outputs must be 16-byte aligned");
-    return tqk_store_kv(hk, hv, k, v, n_seqs, tokens, in_dtype, packed_k, packed_v, (hipStream_t)stream);
+    return tqk_store_kv(hk, hv, k, v, n_seqs, tokens, 0, in_dtype, packed_k, packed_v, (hipStream_t)stream);
+}
+
+int tq_store_kv_cache(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
+                      int64_t capacity, int in_dtype, void *packed_k, void *packed_v, void *stream) {
+    int rc = check_fast(hk, "tq_store_kv_cache");
+    rc = rc ? rc : check_fast(hv, "tq_store_kv_cache");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && tokens >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_store_kv_cache: bad argument");
+    REQUIRE(tokens <= capacity, TQ_ERR_ARG, "tq_store_kv_cache: %lld tokens do not fit a capacity of %lld", (long long)tokens,
+            (long long)capacity);
+    if (n_seqs == 0 || tokens == 0) return TQ_OK;
+    REQUIRE(k && v && packed_k && packed_v, TQ_ERR_ARG, "tq_store_kv_cache: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
+            "tq_store_kv_cache: inputs and outputs must be 16-byte aligned");
+    return tqk_store_kv(hk, hv, k, v, n_seqs, tokens, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream);
 }
 
 int tq_store_qjl(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed,

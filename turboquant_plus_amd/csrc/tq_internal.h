@@ -87,7 +87,7 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                     hipStream_t s);
 int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
-                 int in_dtype, void *packed_k, void *packed_v, hipStream_t s);
+                 int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s);
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,
              int out_dtype, int domain, hipStream_t s);
 int tqk_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, const void *packed_v, int64_t n_seqs,

@@ -401,6 +401,7 @@ struct StoreKArgs {
     int norm_correction;
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
+    uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
 };
 
 // copy a handle's quantiser table (4096 x 8 B) into LDS with NT threads; every load is issued before the
@@ -648,7 +649,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             }
             const uint32_t blk = unit >> 3;
             const int row = (int)(unit & 7) * 16 + n16;
-            uint8_t *block = packed + (int64_t)blk * block_bytes(BITS);
+            const uint32_t oblk = RAGGED ? (blk / bps) * a.out_blocks_per_seq + blk % bps : blk;
+            uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
 #if TQ_KNOCKOUT & 16
             if (g[0] == 0x12345678u && g[BITS - 1] == 0x9abcdef0u)   // keeps the codes alive; not taken for real data
 #endif
@@ -816,6 +818,7 @@ struct StoreVArgs {
     int share_k_lut;      // fused K+V store: V's 4-bit table equals K's, which is already in LDS
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
+    uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
 };
 
 // Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.  The first
@@ -890,7 +893,8 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #pragma unroll 1
     for (; unit < end;) {
         const uint32_t next = lo + step * take_ticket(counter, lane);
-        uint8_t *block = packed + (int64_t)(unit >> 1) * block_bytes(BITS);
+        const uint32_t oblk = RAGGED ? ((unit >> 1) / bps) * a.out_blocks_per_seq + (unit >> 1) % bps : unit >> 1;
+        uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
         const int half = (int)(unit & 1);
         __half *norms_out = reinterpret_cast<__half *>(block + block_code_bytes(BITS)) + half * 64 + 16 * kq;
         uint32_t w[4][NW];
@@ -2398,6 +2402,7 @@ static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     ka.quant_lut = h->quant_lut;
     ka.norm_correction = h->norm_correction; ka.tokens = tokens;
     ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
+    ka.out_blocks_per_seq = (uint32_t)bps;
     return ka;
 }
 
@@ -2407,6 +2412,7 @@ static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     va.quant_lut = h->quant_lut;
     va.norm_correction = h->norm_correction; va.tokens = tokens; va.share_k_lut = 0;
     va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
+    va.out_blocks_per_seq = (uint32_t)bps;
     return va;
 }
 
@@ -2749,18 +2755,24 @@ int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, i
     return tq_check_launch("append");
 }
 
+// capacity > 0: the packed buffers are caches laid out for `capacity` tokens per sequence (tq_append's layout) and the
+// `tokens` tokens of every sequence go to its first blocks; 0: sequences follow each other at blocks_for(tokens)
 int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
-                 int in_dtype, void *packed_k, void *packed_v, hipStream_t s) {
+                 int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s) {
     const int64_t bps = blocks_for(tokens), n_blocks = n_seqs * bps;
+    const int64_t out_bps = capacity > 0 ? blocks_for(capacity) : bps;
     if (n_blocks == 0) return TQ_OK;
-    if (!store_fast_ok(hk, in_dtype, n_blocks) || !store_fast_ok(hv, in_dtype, n_blocks)) {
+    if (!store_fast_ok(hk, in_dtype, n_blocks) || !store_fast_ok(hv, in_dtype, n_blocks) || out_bps * n_seqs >= (1ll << 28)) {
+        if (out_bps != bps)  // the block-rebuilding append writes the same codes as the butterfly store
+            return tqk_append_kv(hk, hv, k, v, n_seqs, 0, tokens, capacity, in_dtype, packed_k, packed_v, s);
         const int rc = tqk_store(hk, k, n_seqs, tokens, in_dtype, TQ_KIND_K, packed_k, nullptr, nullptr, s);
         return rc ? rc : tqk_store(hv, v, n_seqs, tokens, in_dtype, TQ_KIND_V, packed_v, nullptr, nullptr, s);
     }
-    const StoreKArgs ka = make_k_args(hk, tokens, bps, n_blocks);
+    StoreKArgs ka = make_k_args(hk, tokens, bps, n_blocks);
     StoreVArgs va = make_v_args(hv, tokens, bps, n_blocks);
+    ka.out_blocks_per_seq = va.out_blocks_per_seq = (uint32_t)out_bps;
     va.share_k_lut = hk->bits == 4 && hv->bits == 4 && hk->quant_lut_hash == hv->quant_lut_hash;
-    const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
+    const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK || out_bps != bps;
     // one workgroup of 12 wavefronts per CU
     const unsigned wg = 768;
     const unsigned grid = (unsigned)((va.n_units + 11) / 12 < 256 ? (va.n_units + 11) / 12 : 256);

@@ -130,5 +130,14 @@ class LayerKV:
             self.v_codec.append(v, v_cache, pos, capacity, kind="v")
         return k_cache, v_cache
 
+    def prefill(self, k, v, k_cache, v_cache, capacity: int):
+        """The prompt's K and V [n_seqs, tokens, 128] into caches laid out for `capacity` tokens, from position 0:
+        turbo K with turbo V through the fused store (TurboCodec.store_kv(capacity=...), the matrix-core kernels for
+        fp16 rows), any other pair through append() at position 0."""
+        if self.k_codec is not None and self.v_codec is not None:
+            self.k_codec.store_kv(self.v_codec, k, v, out_k=k_cache, out_v=v_cache, capacity=capacity)
+            return k_cache, v_cache
+        return self.append(k, v, k_cache, v_cache, 0, capacity)
+
     def attention(self, batch: int, n_q_heads: int, n_kv_heads: int, tokens: int, **kw) -> DecodeAttention:
         return DecodeAttention(self.k_codec, self.v_codec, batch, n_q_heads, n_kv_heads, tokens, **kw)

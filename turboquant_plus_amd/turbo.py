@@ -119,14 +119,30 @@ class TurboCodec:
                                  L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
 
-    def store_kv(self, v_codec: "TurboCodec", k, v, out_k=None, out_v=None):
+    def store_kv(self, v_codec: "TurboCodec", k, v, out_k=None, out_v=None, capacity: int | None = None):
         """K with this codec and V with `v_codec` in one launch -> (packed_k, packed_v);
-        the same bytes as store(k, "k") and v_codec.store(v, "v")."""
+        the same bytes as store(k, "k") and v_codec.store(v, "v").
+
+        capacity: prefill of a growing cache (tq_store_kv_cache): out_k / out_v are buffers of
+        packed_bytes(bits, n_seqs, capacity) bytes, the layout of append_kv() and DecodeAttention(capacity=...),
+        and every sequence's tokens go to its first blocks."""
         tt = L.torch()
         kd, n_seqs, tokens = self._as_seqs(k)
         vd, n_seqs_v, tokens_v = v_codec._as_seqs(v)
         if (n_seqs, tokens) != (n_seqs_v, tokens_v) or kd.dtype != vd.dtype:
             raise ValueError("k and v must have the same shape and dtype")
+        if capacity is not None:
+            if tokens > capacity:
+                raise ValueError(f"{tokens} tokens do not fit a capacity of {capacity}")
+            if out_k is None or out_v is None:
+                raise ValueError("prefill needs the cache buffers (out_k, out_v)")
+            nk, nv = packed_bytes(self.bits, n_seqs, capacity), packed_bytes(v_codec.bits, n_seqs, capacity)
+            if out_k.numel() != nk or out_v.numel() != nv:
+                raise ValueError(f"cache buffers hold {out_k.numel()} and {out_v.numel()} bytes, a capacity of {capacity} "
+                                 f"tokens for {n_seqs} sequences takes {nk} and {nv}")
+            L.check(L.lib().tq_store_kv_cache(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, tokens, capacity,
+                                              L.dtype_code(kd), L.ptr(out_k), L.ptr(out_v), L.stream_ptr()))
+            return out_k, out_v
         nk, nv = packed_bytes(self.bits, n_seqs, tokens), packed_bytes(v_codec.bits, n_seqs, tokens)
         pk = tt.empty(nk, dtype=tt.uint8, device=kd.device) if out_k is None else out_k
         pv = tt.empty(nv, dtype=tt.uint8, device=kd.device) if out_v is None else out_v
@@ -135,7 +151,7 @@ class TurboCodec:
         if n_seqs > 1 and (pk.numel() != nk or pv.numel() != nv):
             raise ValueError(f"output buffers hold {pk.numel()} and {pv.numel()} bytes but {n_seqs} sequences of "
                              f"{tokens} tokens take exactly {nk} and {nv}; fill a cache laid out for a larger "
-                             "capacity with append_kv()")
+                             "capacity with store_kv(capacity=...) or append_kv()")
         L.check(L.lib().tq_store_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, tokens,
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
