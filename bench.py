@@ -197,6 +197,17 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
     run_two(max(steps, 1000))
     torch.cuda.synchronize()
     two_us = (time.perf_counter() - t0) / max(steps, 1000) * 1e6
+    # the same tensors as the prompt of a cache laid out for 40 960 tokens per sequence (tq_store_kv_cache)
+    cap = tokens + 8192
+    caches = [(torch.empty(tqa.packed_bytes(bits, heads, cap), dtype=torch.uint8, device="cuda"),
+               torch.empty(tqa.packed_bytes(bits, heads, cap), dtype=torch.uint8, device="cuda")) for _ in range(2)]
+
+    def pstep(i):
+        k_, v_, _, _ = sets[i % n_sets]
+        ck_, cv_ = caches[i % 2]
+        codec_k.store_kv(codec_v, k_, v_, out_k=ck_, out_v=cv_, capacity=cap)
+    _, pev_ms = time_steps(torch, pstep, steps, warmup)
+    del caches
     # round-trip error of the last set
     k, v, kp, vp = sets[0]
     rec = codec_k.load(kp, heads, tokens, kind="k", domain="original")
@@ -216,6 +227,8 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
         "ms_per_step": wall_ms, "event_ms_per_step": ev_ms, "kernel_us": launch_us,
         "algorithmic_bytes_per_launch": algo, "gbs": gbs, "frac": gbs / HBM_PEAK_GBS,
         "roundtrip_rel_mse_k": rel, "buffer_sets": n_sets, "timed_blocks": info["timed_blocks"],
+        "prefill_into_cache": {"us_per_launch": pev_ms * 1e3, "capacity": cap,
+                               "what": "the same K and V as the prompt of caches laid out for `capacity` tokens per sequence"},
         "several_streams": {"streams": 4, "us_per_launch": two_us, "gbs": algo / (two_us * 1e-6) / 1e9, "frac": algo / (two_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
                         "what": "the same launches issued round-robin on four streams, wall clock per launch; not the roofline figure"},
         "decompress": {"us_per_step": lev_ms * 1e3, "launches_per_step": 1, "io": "codes + fp16 norm in, fp16 out",
