@@ -158,6 +158,16 @@ int tq_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, in
 int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
                  int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, void *stream);
 
+/* tq_append_kv with the position read from device memory when the launch runs (*pos_dev, an int64): a decode
+ * step captured once (HIP graph) can be replayed while the cache grows; the caller advances the counter
+ * between replays (any kernel on the same stream).  A position that is negative or does not leave room for
+ * n_new tokens writes nothing.  Together with tq_attn_params.tokens_dev.  No counterpart in the reference;
+ * for the callers that replay captured launches. */
+int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
+                    const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k,
+                    void *packed_v, void *stream);
+
+
 /* Temporal decay: re-quantise a packed buffer to a narrower width without going back to the
  * original vectors (`requantize_3to2`, benchmarks/temporal_decay_prototype.py:93-125): per row
  * decode with the stored norm, renormalise, nearest centroid of `dst`'s codebook (a value equal
@@ -254,6 +264,12 @@ typedef struct tq_attn_params {
     int32_t v_format;                      /* the same for V: TQ_KFMT_TURBO (0) | TQ_KFMT_Q8_0 */
     float scale;                           /* logit scale, e.g. 1/sqrt(128)                  */
     float sparse_v_tau;                    /* 0 = dense; skip V rows with weight < tau       */
+    const int64_t *tokens_dev;             /* NULL, or device memory the step's context      */
+                                           /* length is read from when the launch runs       */
+                                           /* (clamped to 0 .. tokens; `tokens` then is the  */
+                                           /* maximum, sizes the workspace and is the stride */
+                                           /* of the bias rows): one captured launch replays */
+                                           /* at a growing length.  skip_count must be NULL. */
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four

@@ -455,3 +455,101 @@ def test_layer_prefill_then_decode(fmt):
     ref, _, _ = reference_attention(q, layer.k_codec, layer.v_codec, kc, vc, B, Hq, Hkv, pos, 1 / np.sqrt(D), capacity=capacity,
                                     k_q8=kc if layer.k_codec is None else None, v_q8=vc if layer.v_codec is None else None)
     assert_close(out, ref)
+
+
+def test_attention_with_the_context_length_on_the_device():
+    """tq_attn_params.tokens_dev: the same launch parameters at several context lengths, the length read from device
+    memory, against objects built for each length on the host (the split geometry follows the length in the same way,
+    so the results are equal bit for bit); lengths above the maximum are clamped to it."""
+    tt = L.torch()
+    B, Hq, Hkv, cap = 2, 8, 2, 1280
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    rng = np.random.default_rng(31)
+    k = rng.standard_normal((B * Hkv, cap, D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, cap, D)).astype(np.float16)
+    ck, cv = kc.store_kv(vc, k, v)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = tt.from_numpy(rng.standard_normal((B, Hq, cap)).astype(np.float32)).cuda()
+    n_dev = tt.zeros(1, dtype=tt.int64, device="cuda")
+    moving = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, cap, n_splits=4, capacity=cap, tokens_on_device=n_dev)
+    for n in (1, 63, 64, 65, 200, 1000, 1279, 1280):
+        n_dev.fill_(n)
+        fixed = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, n, n_splits=4, capacity=cap)
+        got = np_(moving(q, ck, cv)).copy()
+        assert np.array_equal(got, np_(fixed(q, ck, cv))), n
+        # with a bias: its rows keep the stride of the maximum length
+        got_b = np_(moving(q, ck, cv, bias=bias)).copy()
+        want_b = np_(fixed(q, ck, cv, bias=bias[:, :, :n].contiguous()))
+        assert np.array_equal(got_b, want_b), n
+    n_dev.fill_(5000)
+    assert np.array_equal(np_(moving(q, ck, cv)), got)
+    with pytest.raises(ValueError):
+        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, cap, capacity=cap, tokens_on_device=n_dev, sparse_v_tau=1e-3)
+
+
+@pytest.mark.parametrize("n_new", [1, 3])
+def test_decode_loop_replayed_from_one_hip_graph(n_new):
+    """A whole decode step - append at a position held in device memory, advance it, attention over the new length -
+    captured once and replayed while the cache grows across a block boundary; every replay against the eager step
+    with host positions (bit for bit, cache bytes included), with eager work between the replays."""
+    tt = L.torch()
+    B, Hq, Hkv, cap, start = 2, 8, 2, 512, 250
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    rng = np.random.default_rng(6)
+    k0 = rng.standard_normal((B * Hkv, start, D)).astype(np.float16)
+    v0 = rng.standard_normal((B * Hkv, start, D)).astype(np.float16)
+    ck = tt.zeros(tqa.packed_bytes(3, B * Hkv, cap), dtype=tt.uint8, device="cuda")
+    cv = tt.zeros_like(ck)
+    kc.store_kv(vc, k0, v0, out_k=ck, out_v=cv, capacity=cap)
+    ek, ev = ck.clone(), cv.clone()                      # the eager loop's cache
+    pos_d = tt.full((1,), start, dtype=tt.int64, device="cuda")
+    len_d = tt.full((1,), start, dtype=tt.int64, device="cuda")
+    q_s = tt.zeros((B, Hq, D), dtype=tt.float16, device="cuda")
+    kn_s = tt.zeros((B * Hkv, n_new, D), dtype=tt.float16, device="cuda")
+    vn_s = tt.zeros_like(kn_s)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, cap, n_splits=4, capacity=cap, tokens_on_device=len_d)
+
+    def step():
+        kc.append_kv(vc, kn_s, vn_s, ck, cv, pos_d, cap)
+        pos_d.add_(n_new)
+        len_d.add_(n_new)
+        return attn(q_s, ck, cv)
+
+    side = tt.cuda.Stream()
+    side.wait_stream(tt.cuda.current_stream())
+    with tt.cuda.stream(side):
+        step()                                           # warm-up outside the capture, then undone
+    tt.cuda.current_stream().wait_stream(side)
+    ck.copy_(ek)
+    cv.copy_(ev)
+    pos_d.fill_(start)
+    len_d.fill_(start)
+    graph = tt.cuda.CUDAGraph()
+    with tt.cuda.graph(graph):
+        out_g = step()
+    ck.copy_(ek)                                         # the capture does not run the kernels; start clean anyway
+    cv.copy_(ev)
+    pos_d.fill_(start)
+    len_d.fill_(start)
+    pos = start
+    for trial in range(6):                               # 250 -> 256 / 268: crosses the block boundary at 256
+        q = tt.from_numpy(rng.standard_normal((B, Hq, D)).astype(np.float16)).cuda()
+        kn = tt.from_numpy(rng.standard_normal((B * Hkv, n_new, D)).astype(np.float16)).cuda()
+        vn = tt.from_numpy(rng.standard_normal((B * Hkv, n_new, D)).astype(np.float16)).cuda()
+        kc.append_kv(vc, kn, vn, ek, ev, pos, cap)
+        pos += n_new
+        want = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, pos, n_splits=4, capacity=cap)(q, ek, ev).clone()
+        tt.cuda.synchronize()
+        q_s.copy_(q)
+        kn_s.copy_(kn)
+        vn_s.copy_(vn)
+        graph.replay()
+        tt.cuda.synchronize()
+        assert int(pos_d.item()) == pos and int(len_d.item()) == pos
+        assert tt.equal(ck, ek) and tt.equal(cv, ev), f"cache after replay {trial}"
+        assert tt.equal(out_g, want), f"replay {trial}"
+    # a position that leaves no room writes nothing
+    pos_d.fill_(cap)
+    before = ck.clone()
+    kc.append_kv(vc, kn_s, vn_s, ck, cv, pos_d, cap)
+    assert tt.equal(ck, before)

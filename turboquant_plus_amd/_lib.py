@@ -33,7 +33,7 @@ class TQConfig(C.Structure):
 class TQAttnParams(C.Structure):
     _fields_ = [("batch", C.c_int32), ("n_q_heads", C.c_int32), ("n_kv_heads", C.c_int32), ("tokens", C.c_int64),
                 ("capacity", C.c_int64), ("n_splits", C.c_int32), ("k_format", C.c_int32), ("v_format", C.c_int32),
-                ("scale", C.c_float), ("sparse_v_tau", C.c_float)]
+                ("scale", C.c_float), ("sparse_v_tau", C.c_float), ("tokens_dev", C.c_void_p)]
 
 
 _P, _I, _L, _D = C.c_void_p, C.c_int, C.c_int64, C.c_double
@@ -61,6 +61,7 @@ PROTOTYPES = {
     "tq_store_kv_cache": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _P, _P, _P]),
     "tq_append": (_I, [_P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_append_kv": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _P, _P]),
+    "tq_append_kv_at": (_I, [_P, _P, _P, _P, _L, _P, _L, _L, _I, _P, _P, _P]),
     "tq_requantize": (_I, [_P, _P, _P, _L, _L, _I, _P, _P]),
     "tq_fork_block_bytes": (_L, [C.c_int32]),
     "tq_export_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),

@@ -211,6 +211,7 @@ struct AttnArgs {
     unsigned long long total_pairs;
     int pass;                             // head_off / 4
     int64_t tokens, blocks_per_seq;
+    const int64_t *tokens_dev;  // NULL, or where the step's context length is read from (<= tokens, which then is the maximum)
     int n_groups, n_splits, tiles_per_split, n_tiles;
     int q_group, head_off;  // query heads per KV head; first of the (up to) four heads this launch works on
     float tau;
@@ -441,8 +442,17 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     const int wgs_per_group = a.n_splits / n_waves;
     const int group = (int)(blockIdx.x / wgs_per_group), part = (int)(blockIdx.x % wgs_per_group);
     const int split = part * n_waves + wave;  // index of this wavefront's partial
-    const int t_begin = split * a.tiles_per_split;
-    const int t_end = min(t_begin + a.tiles_per_split, a.n_tiles);
+    // The context length: a kernel argument, or read from memory when the caller replays one captured launch at
+    // changing lengths (the split geometry then follows the length; a.tokens stays the bias rows' stride).
+    int tokens_now = (int)a.tokens, n_tiles = a.n_tiles, tiles_per_split = a.tiles_per_split;
+    if (a.tokens_dev) {
+        const int64_t t = *a.tokens_dev;
+        tokens_now = __builtin_amdgcn_readfirstlane((int)(t < 0 ? 0 : (t < a.tokens ? t : a.tokens)));
+        n_tiles = (tokens_now + 63) >> 6;
+        tiles_per_split = (n_tiles + a.n_splits - 1) / a.n_splits;
+    }
+    const int t_begin = split * tiles_per_split;
+    const int t_end = min(t_begin + tiles_per_split, n_tiles);
     const int b4 = lane & ~3;  // 4 * block index
     const int j = lane & 3;    // query head of the logits this lane holds; sub-row for V
 
@@ -584,13 +594,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         if (!a.bias) return;
         const int tk = t * 64 + b4;  // the launcher checks tokens < 2^31
         const float *row = a.bias + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.tokens;
-        if (bias_vec && tk + 3 < (int)a.tokens) {
+        if (bias_vec && tk + 3 < tokens_now) {
             const float4 v = *reinterpret_cast<const float4 *>(row + tk);
             bv[0] = v.x; bv[1] = v.y; bv[2] = v.z; bv[3] = v.w;
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (tk + i < (int)a.tokens) bv[i] = row[tk + i];
+                if (tk + i < tokens_now) bv[i] = row[tk + i];
         }
     };
     float bias_next[HG][4];
@@ -621,7 +631,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         const int tile_n = min(tile_next, t_end - 1);
         const int row_n = tile_next < t_end ? (tile_n & 1) * 64 + lane : 0;  // past the split: every lane the same row
         const VSide<VBITS> gvu_next = load_vnorm(tile_n);
-        const int n_valid = (int)a.tokens - tile * 64;   // >= 64 except in the sequence's last tile
+        const int n_valid = tokens_now - tile * 64;   // >= 64 except in the sequence's last tile
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
         float bias4[HG][4];
 #pragma unroll
@@ -1030,6 +1040,11 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         return TQ_ERR_UNSUPPORTED;
     }
     a.tokens = p->tokens;
+    a.tokens_dev = p->tokens_dev;
+    if (p->tokens_dev && skip_count) {
+        tq_set_error("tq_decode_attention: the Sparse-V count is not kept for a context length read from memory (tokens_dev)");
+        return TQ_ERR_UNSUPPORTED;
+    }
     a.blocks_per_seq = ((p->capacity > 0 ? p->capacity : p->tokens) + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
     a.n_groups = groups;
     a.n_splits = p->n_splits;

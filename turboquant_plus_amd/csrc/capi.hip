@@ -529,6 +529,23 @@ int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
     return tqk_append_kv(hk, hv, k, v, n_seqs, pos, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream);
 }
 
+int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
+                    const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v,
+                    void *stream) {
+    int rc = check_fast(hk, "tq_append_kv_at");
+    rc = rc ? rc : check_fast(hv, "tq_append_kv_at");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_append_kv_at: bad argument");
+    REQUIRE(n_new <= capacity, TQ_ERR_ARG, "tq_append_kv_at: %lld tokens do not fit a capacity of %lld", (long long)n_new,
+            (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(k && v && packed_k && packed_v && pos_dev, TQ_ERR_ARG, "tq_append_kv_at: null pointer");
+    REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
+            "tq_append_kv_at: inputs and packed buffers must be 16-byte aligned");
+    REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_append_kv_at: pos_dev must be 8-byte aligned");
+    return tqk_append_kv(hk, hv, k, v, n_seqs, 0, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream, pos_dev);
+}
+
 int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs, int64_t tokens,
                   int kind, void *packed_dst, void *stream) {
     int rc = check_fast(src_h, "tq_requantize");

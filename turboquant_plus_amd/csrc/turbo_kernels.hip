@@ -1288,7 +1288,21 @@ struct AppendArgs {
     const float *s1, *s2, *bounds, *cent;
     int kind, norm_correction, zero_code;
     int64_t pos, n_new, blocks_per_seq, first_block, n_touched;
+    const int64_t *pos_dev;  // NULL, or where the position is read from when the launch runs (n_touched is then the
+    int64_t capacity;        // largest number of blocks n_new tokens can touch, and some workgroups find nothing to do)
 };
+
+// Position from device memory (a captured launch replayed while the cache grows): fills in pos and first_block and
+// says whether workgroup `wg` has a block to rebuild.  Positions that do not fit the capacity write nothing.
+__device__ __forceinline__ bool resolve_append(AppendArgs &a, int64_t wg) {
+    if (!a.pos_dev) return true;
+    const int64_t pos = *a.pos_dev;
+    if (pos < 0 || pos + a.n_new > a.capacity) return false;
+    a.pos = pos;
+    a.first_block = pos / TQ_ROWS_PER_BLOCK;
+    const int64_t touched = (pos + a.n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
+    return wg % a.n_touched < touched;
+}
 
 __device__ inline float block_norm(const uint8_t *block, int bits, int token);
 
@@ -1424,6 +1438,7 @@ __device__ __forceinline__ void append_block(const TI *x, uint8_t *packed, const
 
 template <int BITS, typename TI>
 __global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, AppendArgs a) {
+    if (!resolve_append(a, blockIdx.x)) return;
     append_block<BITS, TI>(x, packed, a, blockIdx.x);
 }
 
@@ -1431,8 +1446,11 @@ __global__ __launch_bounds__(256) void k_append(const TI *x, uint8_t *packed, Ap
 template <int KB, int VB, typename TI>
 __global__ __launch_bounds__(256) void k_append_kv(const TI *xk, uint8_t *pk, AppendArgs ka, const TI *xv, uint8_t *pv, AppendArgs va) {
     const unsigned half = gridDim.x >> 1;
-    if (blockIdx.x < half) append_block<KB, TI>(xk, pk, ka, blockIdx.x);
-    else append_block<VB, TI>(xv, pv, va, blockIdx.x - half);
+    if (blockIdx.x < half) {
+        if (resolve_append(ka, blockIdx.x)) append_block<KB, TI>(xk, pk, ka, blockIdx.x);
+    } else {
+        if (resolve_append(va, blockIdx.x - half)) append_block<VB, TI>(xv, pv, va, blockIdx.x - half);
+    }
 }
 
 // ---- K2 + K4 in float64: codes, corrected norm, residual sign sketch ---------------
@@ -2704,21 +2722,25 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
     return tq_check_launch("fork_blocks");
 }
 
-static AppendArgs make_append_args(const tq_handle *h, int64_t pos, int64_t n_new, int64_t capacity, int kind) {
+static AppendArgs make_append_args(const tq_handle *h, int64_t pos, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
+                                   int kind) {
     AppendArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
     a.kind = kind; a.norm_correction = h->norm_correction; a.zero_code = h->zero_code;
     a.pos = pos; a.n_new = n_new; a.blocks_per_seq = blocks_for(capacity);
+    a.pos_dev = pos_dev; a.capacity = capacity;
     a.first_block = pos / TQ_ROWS_PER_BLOCK;
-    a.n_touched = (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
+    a.n_touched = pos_dev ? (n_new + TQ_ROWS_PER_BLOCK - 2) / TQ_ROWS_PER_BLOCK + 1  // at the worst alignment
+                          : (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
     return a;
 }
 
 int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
-                  int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s) {
+                  int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s,
+                  const int64_t *pos_dev) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
-    const AppendArgs ka = make_append_args(hk, pos, n_new, capacity, TQ_KIND_K);
-    const AppendArgs va = make_append_args(hv, pos, n_new, capacity, TQ_KIND_V);
+    const AppendArgs ka = make_append_args(hk, pos, pos_dev, n_new, capacity, TQ_KIND_K);
+    const AppendArgs va = make_append_args(hv, pos, pos_dev, n_new, capacity, TQ_KIND_V);
     const unsigned grid = 2u * (unsigned)(n_seqs * ka.n_touched);
     const int kb = hk->bits, vb = hv->bits;
 #define TQ_APPEND_KV(KB, VB)                                                                                                   \
@@ -2731,17 +2753,17 @@ int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const
     else if (kb == 3 && vb == 2) { TQ_APPEND_KV(3, 2); }
     else if (kb == 4 && vb == 3) { TQ_APPEND_KV(4, 3); }
     else {  // other pairs: two launches
-        const int rc = tqk_append(hk, k, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_K, packed_k, s);
-        return rc ? rc : tqk_append(hv, v, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_V, packed_v, s);
+        const int rc = tqk_append(hk, k, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_K, packed_k, s, pos_dev);
+        return rc ? rc : tqk_append(hv, v, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_V, packed_v, s, pos_dev);
     }
 #undef TQ_APPEND_KV
     return tq_check_launch("append_kv");
 }
 
 int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
-               int kind, void *packed, hipStream_t s) {
+               int kind, void *packed, hipStream_t s, const int64_t *pos_dev) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
-    const AppendArgs a = make_append_args(h, pos, n_new, capacity, kind);
+    const AppendArgs a = make_append_args(h, pos, pos_dev, n_new, capacity, kind);
     const unsigned grid = (unsigned)(n_seqs * a.n_touched);
 #define TQ_APPEND_BITS(B) \
     DISPATCH_T(in_dtype, TI, (k_append<B, TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, a)))

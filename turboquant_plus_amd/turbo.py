@@ -167,9 +167,10 @@ class TurboCodec:
                                   L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
         return packed
 
-    def append_kv(self, v_codec: "TurboCodec", k, v, packed_k, packed_v, pos: int, capacity: int):
+    def append_kv(self, v_codec: "TurboCodec", k, v, packed_k, packed_v, pos, capacity: int):
         """append() of the K tokens (this codec) and the V tokens (`v_codec`) of one decode step
-        in one launch (tq_append_kv)."""
+        in one launch (tq_append_kv).  pos: an int, or an int64 device tensor with one element that holds the
+        position when the launch runs (tq_append_kv_at: a captured step replayed while the cache grows)."""
         kd, n_seqs, n_new = self._as_seqs(k)
         vd, vs, vn = self._as_seqs(v)
         if (vs, vn) != (n_seqs, n_new) or vd.dtype != kd.dtype:
@@ -178,6 +179,13 @@ class TurboCodec:
             need = packed_bytes(codec.bits, n_seqs, capacity)
             if buf.numel() < need:
                 raise ValueError(f"packed holds {buf.numel()} bytes, need {need}")
+        if not isinstance(pos, (int, np.integer)):
+            tt = L.torch()
+            if pos.dtype != tt.int64 or not pos.is_cuda or pos.numel() != 1:
+                raise ValueError("a position on the device must be an int64 device tensor with one element")
+            L.check(L.lib().tq_append_kv_at(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, L.ptr(pos), n_new,
+                                            capacity, L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
+            return packed_k, packed_v
         L.check(L.lib().tq_append_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, pos, n_new, capacity,
                                      L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
         return packed_k, packed_v
@@ -363,7 +371,10 @@ class DecodeAttention:
 
     def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec | None, batch: int, n_q_heads: int, n_kv_heads: int,
                  tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0,
-                 capacity: int = 0):
+                 capacity: int = 0, tokens_on_device=None):
+        """tokens_on_device: an int64 device tensor (one element) that holds the context length when a call runs;
+        `tokens` is then the largest length it may take.  One captured launch (HIP graph) can so be replayed while
+        the cache grows; Sparse V is not available in this mode."""
         tt = L.torch()
         dev = L.require_gpu()
         self.k_codec, self.v_codec = k_codec, v_codec
@@ -374,6 +385,13 @@ class DecodeAttention:
                                      v_format=L.KFMT_TURBO if v_codec is not None else L.KFMT_Q8_0,
                                      scale=(1.0 / math.sqrt(HEAD_DIM)) if scale is None else scale,
                                      sparse_v_tau=sparse_v_tau)
+        self.tokens_on_device = tokens_on_device   # kept alive with the object
+        if tokens_on_device is not None:
+            if tokens_on_device.dtype != tt.int64 or not tokens_on_device.is_cuda or tokens_on_device.numel() != 1:
+                raise ValueError("tokens_on_device must be an int64 device tensor with one element")
+            if sparse_v_tau > 0:
+                raise ValueError("Sparse V keeps no count for a context length read from device memory")
+            self.params.tokens_dev = tokens_on_device.data_ptr()
         nbytes = L.lib().tq_attn_workspace_bytes(C.byref(self.params))
         if nbytes < 0:
             L.check(L.ERR_ARG)
