@@ -154,7 +154,7 @@ def measured_peaks_leg(torch, tqa, steps, warmup):
     return out
 
 
-def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
+def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
     heads, tokens = 8, 32768
     codec_k, codec_v = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
     sets = []
@@ -176,27 +176,30 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
     algo = n_vec * bytes_per_vec
     launch_us = ev_ms * 1e3                          # one launch (K and V) per step
     gbs = algo / (launch_us * 1e-6) / 1e9
-    # consecutive layers issued on several streams (what a serving loop that stores a layer's K and V per step can do:
-    # layers are independent, so one launch's tail overlaps the next one's start); wall clock over the whole loop
-    # (the C entry point is called with prepared arguments, so that the host's share of a call stays well below a launch)
-    import ctypes
-    from turboquant_plus_amd import _lib as L
-    streams = [torch.cuda.Stream() for _ in range(4)]   # four: one per hardware queue of the process
-    sp = [ctypes.c_void_p(st.cuda_stream) for st in streams]
-    fn, hk, hv, code = L.lib().tq_store_kv, codec_k.handle.h, codec_v.handle.h, L.dtype_code(sets[0][0])
-    prepared = [tuple(L.ptr(t) for t in st) for st in sets]
+    # consecutive layers issued on several streams (--several-streams; what a serving loop that stores a layer's K and V
+    # per step can do: layers are independent, so one launch's tail overlaps the next one's start); wall clock over the
+    # whole loop.  Off by default: its launches overlap, which would blur the kernel's row in a trace of the default run.
+    two_us = None
+    if several_streams:
+        # (the C entry point is called with prepared arguments, so that the host's share of a call stays well below a launch)
+        import ctypes
+        from turboquant_plus_amd import _lib as L
+        streams = [torch.cuda.Stream() for _ in range(4)]   # four: one per hardware queue of the process
+        sp = [ctypes.c_void_p(st.cuda_stream) for st in streams]
+        fn, hk, hv, code = L.lib().tq_store_kv, codec_k.handle.h, codec_v.handle.h, L.dtype_code(sets[0][0])
+        prepared = [tuple(L.ptr(t) for t in st) for st in sets]
 
-    def run_two(n):
-        for i in range(n):
-            pk_, pv_, pkp, pvp = prepared[i % n_sets]
-            if fn(hk, hv, pk_, pv_, heads, tokens, code, pkp, pvp, sp[i % 4]):
-                raise RuntimeError(L.last_error())
-    run_two(warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_two(max(steps, 1000))
-    torch.cuda.synchronize()
-    two_us = (time.perf_counter() - t0) / max(steps, 1000) * 1e6
+        def run_two(n):
+            for i in range(n):
+                pk_, pv_, pkp, pvp = prepared[i % n_sets]
+                if fn(hk, hv, pk_, pv_, heads, tokens, code, pkp, pvp, sp[i % 4]):
+                    raise RuntimeError(L.last_error())
+        run_two(warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_two(max(steps, 1000))
+        torch.cuda.synchronize()
+        two_us = (time.perf_counter() - t0) / max(steps, 1000) * 1e6
     # the same tensors as the prompt of a cache laid out for 40 960 tokens per sequence (tq_store_kv_cache)
     cap = tokens + 8192
     caches = [(torch.empty(tqa.packed_bytes(bits, heads, cap), dtype=torch.uint8, device="cuda"),
@@ -229,8 +232,9 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4):
         "roundtrip_rel_mse_k": rel, "buffer_sets": n_sets, "timed_blocks": info["timed_blocks"],
         "prefill_into_cache": {"us_per_launch": pev_ms * 1e3, "capacity": cap,
                                "what": "the same K and V as the prompt of caches laid out for `capacity` tokens per sequence"},
-        "several_streams": {"streams": 4, "us_per_launch": two_us, "gbs": algo / (two_us * 1e-6) / 1e9, "frac": algo / (two_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                        "what": "the same launches issued round-robin on four streams, wall clock per launch; not the roofline figure"},
+        "several_streams": None if two_us is None else {
+            "streams": 4, "us_per_launch": two_us, "gbs": algo / (two_us * 1e-6) / 1e9, "frac": algo / (two_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "what": "the same launches issued round-robin on four streams, wall clock per launch; not the roofline figure"},
         "decompress": {"us_per_step": lev_ms * 1e3, "launches_per_step": 1, "io": "codes + fp16 norm in, fp16 out",
                        "gbs": load_algo / (lev_ms * 1e-3) / 1e9, "frac": load_algo / (lev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
@@ -496,6 +500,8 @@ def main():
     ap.add_argument("--legs", default="all",
                     help="comma-separated subset of store4,store3,decode,asym,tile,boundary,peaks (profiling runs); "
                          "the JSON line then holds only those legs and is not the benchmark's line")
+    ap.add_argument("--several-streams", action="store_true",
+                    help="store legs: also time the launches issued round-robin on four streams (overlapping launches)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (5x) so that FETCH_SIZE / WRITE_SIZE counters can be calibrated")
     args = ap.parse_args()
@@ -521,9 +527,9 @@ def main():
         legs = set(args.legs.split(","))
         part = {"partial_run": sorted(legs), "steps": args.steps, "warmup": args.warmup}
         if "store4" in legs:
-            part["turbo4_store"] = store_leg(torch, tqa, 4, args.steps, args.warmup)
+            part["turbo4_store"] = store_leg(torch, tqa, 4, args.steps, args.warmup, several_streams=args.several_streams)
         if "store3" in legs:
-            part["turbo3_store"] = store_leg(torch, tqa, 3, args.steps, args.warmup)
+            part["turbo3_store"] = store_leg(torch, tqa, 3, args.steps, args.warmup, several_streams=args.several_streams)
         if "decode" in legs:
             part["decode_attn"] = decode_leg(torch, tqa, args.steps, args.warmup)
         if "asym" in legs:
@@ -536,8 +542,8 @@ def main():
             part["measured_peaks"] = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
         print(json.dumps(part, ensure_ascii=False))
         return
-    s4 = store_leg(torch, tqa, 4, args.steps, args.warmup)
-    s3 = store_leg(torch, tqa, 3, args.steps, args.warmup)
+    s4 = store_leg(torch, tqa, 4, args.steps, args.warmup, several_streams=args.several_streams)
+    s3 = store_leg(torch, tqa, 3, args.steps, args.warmup, several_streams=args.several_streams)
     dec = decode_leg(torch, tqa, args.steps, args.warmup)
     torch.cuda.empty_cache()
     asym = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
