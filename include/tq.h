@@ -166,6 +166,11 @@ int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
 int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                     const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k,
                     void *packed_v, void *stream);
+/* The same for one tensor (tq_append) and for q8_0-style buffers (tq_q8_0_append). */
+int tq_append_at(const tq_handle *h, const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new,
+                 int64_t capacity, int in_dtype, int kind, void *packed, void *stream);
+int tq_q8_0_append_at(const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
+                      int in_dtype, int kind, void *packed, void *stream);
 
 
 /* Temporal decay: re-quantise a packed buffer to a narrower width without going back to the

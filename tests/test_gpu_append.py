@@ -553,3 +553,30 @@ def test_decode_loop_replayed_from_one_hip_graph(n_new):
     before = ck.clone()
     kc.append_kv(vc, kn_s, vn_s, ck, cv, pos_d, cap)
     assert tt.equal(ck, before)
+
+
+@pytest.mark.parametrize("fmt", [("q8_0", "turbo2"), ("turbo3", "q8_0"), ("q8_0", "q8_0"), ("turbo4", "turbo3")])
+def test_layer_appends_at_a_position_on_the_device(fmt):
+    """LayerKV.append with the position in device memory (tq_append_kv_at, tq_append_at, tq_q8_0_append_at) against the
+    same appends at host positions: equal caches, at several alignments, and nothing written where there is no room."""
+    tt = L.torch()
+    n_seqs, cap = 3, 384
+    layer = tqa.LayerKV(tqa.LayerFormat(*fmt), seed=5)
+    rng = np.random.default_rng(17)
+    k = rng.standard_normal((n_seqs, 300, D)).astype(np.float32)
+    v = rng.standard_normal((n_seqs, 300, D)).astype(np.float32)
+    ak, av = layer.new_cache(n_seqs, cap)
+    bk, bv = layer.new_cache(n_seqs, cap)
+    pos_d = tt.zeros(1, dtype=tt.int64, device="cuda")
+    pos = 0
+    for n_new in (100, 27, 1, 1, 130, 1):          # 0 -> 100 -> 127 -> 128 -> 129 -> 259 -> 260
+        layer.append(k[:, pos:pos + n_new], v[:, pos:pos + n_new], ak, av, pos, cap)
+        pos_d.fill_(pos)
+        layer.append(k[:, pos:pos + n_new], v[:, pos:pos + n_new], bk, bv, pos_d, cap)
+        pos += n_new
+        assert tt.equal(ak, bk) and tt.equal(av, bv), f"after {pos} tokens"
+    pos_d.fill_(cap - 1)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap)
+    assert tt.equal(ak, bk) and tt.equal(av, bv)
+    with pytest.raises(ValueError):
+        layer.append(k[:, :2], v[:, :2], bk, bv, tt.zeros(1, dtype=tt.int32, device="cuda"), cap)

@@ -529,6 +529,34 @@ int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
     return tqk_append_kv(hk, hv, k, v, n_seqs, pos, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream);
 }
 
+int tq_append_at(const tq_handle *h, const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
+                 int in_dtype, int kind, void *packed, void *stream) {
+    int rc = check_fast(h, "tq_append_at");
+    if (rc) return rc;
+    REQUIRE(n_seqs >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_append_at: bad argument");
+    REQUIRE(n_new <= capacity, TQ_ERR_ARG, "tq_append_at: %lld tokens do not fit a capacity of %lld", (long long)n_new,
+            (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(x && packed && pos_dev, TQ_ERR_ARG, "tq_append_at: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_append_at: bad kind %d", kind);
+    REQUIRE(aligned16(x) && aligned16(packed), TQ_ERR_ALIGN, "tq_append_at: x and packed must be 16-byte aligned");
+    REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_append_at: pos_dev must be 8-byte aligned");
+    return tqk_append(h, x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev);
+}
+
+int tq_q8_0_append_at(const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype,
+                      int kind, void *packed, void *stream) {
+    REQUIRE(n_seqs >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_q8_0_append_at: bad argument");
+    REQUIRE(n_new <= capacity, TQ_ERR_ARG, "tq_q8_0_append_at: %lld tokens do not fit a capacity of %lld", (long long)n_new,
+            (long long)capacity);
+    if (n_seqs == 0 || n_new == 0) return TQ_OK;
+    REQUIRE(x && packed && pos_dev, TQ_ERR_ARG, "tq_q8_0_append_at: null pointer");
+    REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_q8_0_append_at: bad kind %d", kind);
+    REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_append_at: packed must be 16-byte aligned");
+    REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_q8_0_append_at: pos_dev must be 8-byte aligned");
+    return tqk_q8_0_append(x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev);
+}
+
 int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                     const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v,
                     void *stream) {

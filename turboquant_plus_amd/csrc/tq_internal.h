@@ -97,7 +97,7 @@ int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int
                      float *norms, hipStream_t s);
 int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
 int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
-                    void *packed, hipStream_t s);
+                    void *packed, hipStream_t s, const int64_t *pos_dev = nullptr);
 int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
 int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, int kind, hipStream_t s);
 

@@ -2322,7 +2322,14 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v_f16(const __half *x, uint8
 // the V layout; byte stores keep them apart.
 template <typename TI, int KIND>
 __global__ __launch_bounds__(256) void k_q8_0_append(const TI *x, uint8_t *packed, int64_t pos, int64_t n_new,
-                                                     int64_t blocks_per_seq, int64_t first_block, int64_t n_touched) {
+                                                     int64_t blocks_per_seq, int64_t first_block, int64_t n_touched,
+                                                     const int64_t *pos_dev, int64_t capacity) {
+    if (pos_dev) {  // the position is read when the launch runs (see resolve_append)
+        pos = *pos_dev;
+        if (pos < 0 || pos + n_new > capacity) return;
+        first_block = pos / TQ_ROWS_PER_BLOCK;
+        if ((int64_t)(blockIdx.x % n_touched) >= (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - first_block + 1) return;
+    }
     const int64_t seq = blockIdx.x / n_touched, bis = first_block + blockIdx.x % n_touched;
     const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
     uint8_t *block = packed + (seq * blocks_per_seq + bis) * (int64_t)(TQ_ROWS_PER_BLOCK * 136);
@@ -2946,17 +2953,19 @@ int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype
 }
 
 int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
-                    void *packed, hipStream_t s) {
+                    void *packed, hipStream_t s, const int64_t *pos_dev) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
     const int64_t bps = blocks_for(capacity);
-    const int64_t first = pos / TQ_ROWS_PER_BLOCK, n_touched = (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - first + 1;
+    const int64_t first = pos / TQ_ROWS_PER_BLOCK;
+    const int64_t n_touched = pos_dev ? (n_new + TQ_ROWS_PER_BLOCK - 2) / TQ_ROWS_PER_BLOCK + 1  // at the worst alignment
+                                      : (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - first + 1;
     const unsigned grid = (unsigned)(n_seqs * n_touched);
     if (kind == TQ_KIND_V) {
         DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_V><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
-                                                                                   bps, first, n_touched)));
+                                                                                   bps, first, n_touched, pos_dev, capacity)));
     } else {
         DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_K><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
-                                                                                   bps, first, n_touched)));
+                                                                                   bps, first, n_touched, pos_dev, capacity)));
     }
     return tq_check_launch("q8_0_append");
 }

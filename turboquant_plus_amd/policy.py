@@ -115,8 +115,9 @@ class LayerKV:
         return (tt.zeros(nbytes(self.k_codec), dtype=tt.uint8, device=dev),
                 tt.zeros(nbytes(self.v_codec), dtype=tt.uint8, device=dev))
 
-    def append(self, k, v, k_cache, v_cache, pos: int, capacity: int):
-        """The K and V tokens [n_seqs, n_new, 128] of a decode step at positions pos .. pos+n_new-1."""
+    def append(self, k, v, k_cache, v_cache, pos, capacity: int):
+        """The K and V tokens [n_seqs, n_new, 128] of a decode step at positions pos .. pos+n_new-1 (pos: an int, or an
+        int64 device tensor with one element read when the launches run)."""
         if self.k_codec is not None and self.v_codec is not None:
             self.k_codec.append_kv(self.v_codec, k, v, k_cache, v_cache, pos, capacity)
             return k_cache, v_cache

@@ -156,13 +156,18 @@ class TurboCodec:
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
 
-    def append(self, x, packed, pos: int, capacity: int, kind: str = "k"):
+    def append(self, x, packed, pos, capacity: int, kind: str = "k"):
         """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of
-        `packed`, a buffer of packed_bytes(bits, n_seqs, capacity) bytes (tq_append)."""
+        `packed`, a buffer of packed_bytes(bits, n_seqs, capacity) bytes (tq_append).  pos: an int, or an int64
+        device tensor with one element that holds the position when the launch runs (tq_append_at)."""
         xd, n_seqs, n_new = self._as_seqs(x)
         need = packed_bytes(self.bits, n_seqs, capacity)
         if packed.numel() < need:
             raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
+        if _position_on_device(pos):
+            L.check(L.lib().tq_append_at(self.handle.h, L.ptr(xd), n_seqs, L.ptr(pos), n_new, capacity, L.dtype_code(xd),
+                                         L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+            return packed
         L.check(L.lib().tq_append(self.handle.h, L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
                                   L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
         return packed
@@ -179,10 +184,7 @@ class TurboCodec:
             need = packed_bytes(codec.bits, n_seqs, capacity)
             if buf.numel() < need:
                 raise ValueError(f"packed holds {buf.numel()} bytes, need {need}")
-        if not isinstance(pos, (int, np.integer)):
-            tt = L.torch()
-            if pos.dtype != tt.int64 or not pos.is_cuda or pos.numel() != 1:
-                raise ValueError("a position on the device must be an int64 device tensor with one element")
+        if _position_on_device(pos):
             L.check(L.lib().tq_append_kv_at(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, L.ptr(pos), n_new,
                                             capacity, L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
             return packed_k, packed_v
@@ -334,13 +336,28 @@ def q8_0_store(x, kind: str = "k"):
     return out, n_seqs, tokens
 
 
-def q8_0_append(x, packed, pos: int, capacity: int, kind: str = "k"):
+def _position_on_device(pos) -> bool:
+    """False for a host integer; True for an int64 device tensor with one element (anything else raises)."""
+    if isinstance(pos, (int, np.integer)):
+        return False
+    tt = L.torch()
+    if not isinstance(pos, tt.Tensor) or pos.dtype != tt.int64 or not pos.is_cuda or pos.numel() != 1:
+        raise ValueError("a position on the device must be an int64 device tensor with one element")
+    return True
+
+
+def q8_0_append(x, packed, pos, capacity: int, kind: str = "k"):
     """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of a q8_0-style buffer laid
-    out for `capacity` tokens per sequence (zero-initialised; tq_q8_0_append)."""
+    out for `capacity` tokens per sequence (zero-initialised; tq_q8_0_append).  pos: an int, or an int64 device
+    tensor with one element read when the launch runs (tq_q8_0_append_at)."""
     xd, n_seqs, n_new = TurboCodec._as_seqs(x)
     need = int(L.lib().tq_q8_0_bytes(n_seqs, capacity))
     if packed.numel() < need:
         raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
+    if _position_on_device(pos):
+        L.check(L.lib().tq_q8_0_append_at(L.ptr(xd), n_seqs, L.ptr(pos), n_new, capacity, L.dtype_code(xd),
+                                          L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+        return packed
     L.check(L.lib().tq_q8_0_append(L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
                                    L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
     return packed
