@@ -1503,8 +1503,9 @@ struct StoreQjlArgs {
 // own values), and hi*hi + hi*mid + lo*hi accumulate in fp32 on v_mfma_f32_16x16x32_f16: 96 instructions of 16
 // clocks per unit instead of 256 float64 ones of 64 clocks.  A result at least tau |x| away from zero (the bound on
 // this pass's error, worked out where the handle is made) has the exact projection's sign.  The others, about one
-// per unit, get a second pass: the four lanes that hold the token multiply its float64 residual with hi + mid + lo,
-// read from the same LDS, in float64 (error 2^-31 relative); the one in 10^8 of those that is still too close goes
+// per unit, get a second pass: the token's float64 residual goes through 1 KB of LDS, every lane multiplies two dims
+// of it with hi + mid + lo read from the same operand table, and the wavefront adds the 64 partial products in float64
+// (error 2^-31 relative; left to the four lanes that hold the token it took 0.7 us per value); the one in 10^8 of those that is still too close goes
 // to the float64 matrix in memory.
 // The sign bits of a token's 16 projections of one column block are one quarter of a ballot.  A wavefront packs its
 // own 16 rows (rows of a K block are independent).  No barrier ties the wavefronts together, and the next unit's
@@ -1522,6 +1523,7 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kq = lane >> 4;
     uint8_t *codes = codes_s[wave];
+    double *stage = reinterpret_cast<double *>(frag_s + 3 * 4 * 8 * 64) + 128 * wave;  // second pass: one token's residual
 
     const int64_t n_units = n_blocks * 8;
     const int64_t unit_step = (int64_t)gridDim.x * 8;
@@ -1722,8 +1724,7 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
             }
         }
         uint64_t signs = (uint64_t)((piece[0] & 0xFFFFu) | (piece[1] << 16)) | ((uint64_t)((piece[2] & 0xFFFFu) | (piece[3] << 16)) << 32);
-        // The doubtful ones: one loop for all of them (wave-uniform control flow), the work done by the four lanes
-        // that hold the token's residual.
+        // The doubtful ones: one loop for all of them (wave-uniform control flow), each shared by the whole wavefront.
         uint64_t who = __builtin_amdgcn_ballot_w64(doubt != 0u);
 #pragma unroll 1
         while (who) {
@@ -1736,22 +1737,25 @@ __global__ __launch_bounds__(512) void k_store_qjl_mfma(const TI *x, uint8_t *pa
                 bits &= ~(0x80000000u >> idx);
                 const int i = idx >> 3, jb = idx & 7;
                 const int tokl = 4 * (l >> 4) + i, j = 16 * jb + (l & 15);
-                // second pass: e . (hi + mid + lo) in float64; this lane's 32 dims are its own elements of the fragments
-                double part = 0.0;
+                // second pass: e . (hi + mid + lo) in float64.  The token's residual goes through LDS (stage[32 kq + s] =
+                // dim 4 s + kq) so that the whole wavefront shares the product: lane (sp, kq') = (lane / 4, lane % 4)
+                // takes dims 4 (2 sp) + kq' and 4 (2 sp + 1) + kq', two neighbouring halves of one fragment dword.
                 if (n16 == tokl) {
-                    const uint4 *fr = frag_s + jb * 64 + 16 * kq + (l & 15);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const half8_t m1 = __builtin_bit_cast(half8_t, fr[c * 512]);
-                        const half8_t m2 = __builtin_bit_cast(half8_t, fr[2048 + c * 512]);
-                        const half8_t m3 = __builtin_bit_cast(half8_t, fr[4096 + c * 512]);
-#pragma unroll
-                        for (int k = 0; k < 8; ++k)
-                            part = fma(e[8 * c + k], (double)((float)m1[k] + (float)m2[k]) + (double)(float)m3[k], part);
-                    }
+                    for (int s2 = 0; s2 < 32; s2 += 2) *reinterpret_cast<double2 *>(stage + 32 * kq + s2) = make_double2(e[s2], e[s2 + 1]);
                 }
-                part = quarter_sum(part);
-                double settled = __shfl(part, tokl);
+                __builtin_amdgcn_wave_barrier();
+                const int kqp = lane & 3, sp = lane >> 2;
+                const double2 ev = *reinterpret_cast<const double2 *>(stage + 32 * kqp + 2 * sp);
+                const uint32_t *fw = reinterpret_cast<const uint32_t *>(frag_s) + (((sp >> 2) * 8 + jb) * 64 + 16 * kqp + (l & 15)) * 4 + (sp & 3);
+                const half2_t m1 = __builtin_bit_cast(half2_t, fw[0]);
+                const half2_t m2 = __builtin_bit_cast(half2_t, fw[2048 * 4]);
+                const half2_t m3 = __builtin_bit_cast(half2_t, fw[4096 * 4]);
+                double part = ev.x * ((double)((float)m1[0] + (float)m2[0]) + (double)(float)m3[0]);
+                part = fma(ev.y, (double)((float)m1[1] + (float)m2[1]) + (double)(float)m3[1], part);
+                __builtin_amdgcn_wave_barrier();
+                part = quarter_sum(row16_sum(part));
+                double settled = part;  // every lane holds the sum
                 const double rn_tok = __shfl(rnorm, tokl);
                 if (fabs(settled) < a.tau2 * rn_tok) {  // third pass (wave-uniform: every lane holds the same values)
                     part = 0.0;
@@ -2497,7 +2501,7 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
         a.tau2 = h->qjl_tau2;
         a.norm_correction = h->norm_correction;
         a.tokens = tokens; a.blocks_per_seq = bps;
-        constexpr int MAT_BYTES = 3 * 4 * 8 * 64 * 16;
+        constexpr int MAT_BYTES = 3 * 4 * 8 * 64 * 16 + 8 * 128 * 8;  // the operands and, per wavefront, one token's residual
         const unsigned qgrid = grid < 256u ? grid : 256u;  // one workgroup per CU (the matrix fills its LDS), looping over blocks
 #define TQ_STOREQ_BITS(B)                                                                                          \
     DISPATCH_T(in_dtype, TI,                                                                                       \
