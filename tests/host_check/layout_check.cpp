@@ -15,7 +15,42 @@
 
 #include "tq_layout.h"
 
+// `layout_check fastdiv`: tqd::FastDiv against the division it replaces, for small divisors exhaustively over a
+// range of numerators and for the extreme numerators and divisors.
+static int check_fast_div() {
+    const uint32_t edge[] = {0u, 1u, 2u, 3u, 127u, 128u, 255u, 65535u, 65536u, 0x7FFFFFFFu, 0x80000000u, 0xFFFFFFFEu, 0xFFFFFFFFu};
+    auto one = [](uint32_t n, uint32_t d, const tqd::FastDiv &f) {
+        if (f.div(n) != n / d) {
+            printf("fastdiv: %u / %u gave %u\n", n, d, f.div(n));
+            return 1;
+        }
+        return 0;
+    };
+    for (uint32_t d = 1; d <= 4100; ++d) {
+        const tqd::FastDiv f = tqd::make_fast_div(d);
+        for (uint32_t n = 0; n < 70000; ++n)
+            if (one(n, d, f)) return 1;
+        for (uint32_t e : edge) {
+            if (one(e, d, f)) return 1;
+            // numerators next to multiples of d near the top of the range
+            const uint32_t q = 0xFFFFFFFFu / d;
+            if (one(q * d, d, f) || one(q * d - 1u, d, f) || (q * d + (d - 1u) >= q * d && one(q * d + (d - 1u), d, f))) return 1;
+        }
+    }
+    const uint32_t big[] = {4097u, 65535u, 65536u, 65537u, 1000003u, 0x40000000u, 0x7FFFFFFFu, 0x80000000u};
+    for (uint32_t d : big) {
+        const tqd::FastDiv f = tqd::make_fast_div(d);
+        for (uint32_t e : edge)
+            if (one(e, d, f)) return 1;
+        for (uint32_t k = 0; k < 100000; ++k)
+            if (one(k * 42949u + 7u, d, f)) return 1;
+    }
+    printf("fastdiv ok\n");
+    return 0;
+}
+
 int main(int argc, char **argv) {
+    if (argc == 2 && strcmp(argv[1], "fastdiv") == 0) return check_fast_div();
     if (argc != 2) return 2;
     FILE *f = fopen(argv[1], "rb");
     if (!f) return 2;

@@ -49,6 +49,13 @@ def test_layout_arithmetic_under_sanitizers(layout_check, tmp_path, bits, kind, 
     assert "layout ok" in r.stdout
 
 
+def test_launch_constant_divider(layout_check):
+    """tqd::FastDiv (the kernels' division by the blocks per sequence) equals the plain division."""
+    r = subprocess.run([layout_check, "fastdiv"], capture_output=True, text=True, env=ENV)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "fastdiv ok" in r.stdout
+
+
 def test_abi_argument_paths_under_sanitizers(tmp_path):
     hipcc = shutil.which("hipcc")
     if hipcc is None:

@@ -110,4 +110,27 @@ TQ_HD inline void put_code(uint8_t *block, int bits, int kind, int token, int di
 // byte offset of token's fp16 norm inside the block
 TQ_HD constexpr int norm_offset(int bits, int token) { return block_code_bytes(bits) + 2 * token; }
 
+// Division of a 32-bit unit or block number by a divisor fixed at launch (blocks per sequence): a multiply-high,
+// a subtraction, two shifts and an addition instead of the instruction sequence of a 32-bit division.  Exact for every
+// n < 2^32 and 1 <= d <= 2^31 (round-up method: s = ceil(log2 d), m = floor(2^32 (2^s - d) / d) + 1,
+// q = (t + ((n - t) >> min(s, 1))) >> (s - min(s, 1)) with t = high word of n m).
+struct FastDiv {
+    uint32_t d, m, s1, s2;
+    TQ_HD uint32_t div(uint32_t n) const {
+        const uint32_t t = (uint32_t)(((uint64_t)n * m) >> 32);
+        return (t + ((n - t) >> s1)) >> s2;
+    }
+};
+inline FastDiv make_fast_div(uint32_t d) {
+    FastDiv f;
+    d = d ? d : 1u;  // an empty launch divides nothing
+    f.d = d;
+    uint32_t s = 0;
+    while ((1ull << s) < d) ++s;
+    f.m = (uint32_t)((((1ull << s) - d) << 32) / d + 1);
+    f.s1 = s < 1u ? s : 1u;
+    f.s2 = s - f.s1;
+    return f;
+}
+
 }  // namespace tqd

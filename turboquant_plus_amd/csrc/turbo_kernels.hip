@@ -426,6 +426,7 @@ struct StoreKArgs {
     int norm_correction;
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
+    FastDiv bps_div;                   // division by blocks_per_seq
     uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
 };
 
@@ -495,7 +496,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #endif
         const uint4 *p;
         if constexpr (RAGGED) {
-            const uint32_t blk = unit >> 3, seq = blk / bps, bis = blk - seq * bps;
+            const uint32_t blk = unit >> 3, seq = a.bps_div.div(blk), bis = blk - seq * bps;
             int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + (unit & 7) * 16 + n16;
             valid = tok < a.tokens;
             tok = valid ? tok : a.tokens - 1;
@@ -676,7 +677,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             }
             const uint32_t blk = unit >> 3;
             const int row = (int)(unit & 7) * 16 + n16;
-            const uint32_t oblk = RAGGED ? (blk / bps) * a.out_blocks_per_seq + blk % bps : blk;
+            const uint32_t oseq = RAGGED ? a.bps_div.div(blk) : 0u;
+            const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + (blk - oseq * bps) : blk;
             uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
 #if TQ_KNOCKOUT & 16
             if (g[0] == 0x12345678u && g[BITS - 1] == 0x9abcdef0u)   // keeps the codes alive; not taken for real data
@@ -845,6 +847,7 @@ struct StoreVArgs {
     int share_k_lut;      // fused K+V store: V's 4-bit table equals K's, which is already in LDS
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
+    FastDiv bps_div;                   // division by blocks_per_seq
     uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
 };
 
@@ -885,7 +888,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
         const int tb = (int)(unit & 1) * 64 + 16 * (n16 >> 2) + 4 * u + (n16 & 3);
         const uint4 *p;
         if constexpr (RAGGED) {
-            const uint32_t seq = blk / bps, bis = blk - seq * bps;
+            const uint32_t seq = a.bps_div.div(blk), bis = blk - seq * bps;
             int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + tb;
             valid = tok < a.tokens;
             tok = valid ? tok : a.tokens - 1;
@@ -920,7 +923,8 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #pragma unroll 1
     for (; unit < end;) {
         const uint32_t next = lo + step * take_ticket(counter, lane);
-        const uint32_t oblk = RAGGED ? ((unit >> 1) / bps) * a.out_blocks_per_seq + (unit >> 1) % bps : unit >> 1;
+        const uint32_t oseq = RAGGED ? a.bps_div.div(unit >> 1) : 0u;
+        const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + ((unit >> 1) - oseq * bps) : unit >> 1;
         uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
         const int half = (int)(unit & 1);
         __half *norms_out = reinterpret_cast<__half *>(block + block_code_bytes(BITS)) + half * 64 + 16 * kq;
@@ -1884,6 +1888,7 @@ struct LoadK16Args {
     const uint32_t *pair_lut;  // half2 per pair code
     int64_t tokens;
     uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
+    FastDiv bps_div;                   // division by blocks_per_seq
 };
 
 // byte offset (pair code * 4) of pair k = 0..15 of a group, from the group's dwords (3-bit: and its 24-bit tail)
@@ -1964,7 +1969,7 @@ __device__ __forceinline__ void load_k16_body(const uint8_t *packed, __half *out
     fetch(bid * 4 + wave, cw_next, g_next);
 #pragma unroll 1
     for (uint32_t u = bid * 4 + wave; u < a.n_units; u += nb * 4) {
-        const uint32_t blk = u >> 3, seq = blk / bps, bis = blk - seq * bps;
+        const uint32_t blk = u >> 3, seq = a.bps_div.div(blk), bis = blk - seq * bps;
         uint32_t cw[BITS];
 #pragma unroll
         for (int j = 0; j < BITS; ++j) cw[j] = cw_next[j];
@@ -2058,7 +2063,7 @@ __device__ __forceinline__ void load_v16_body(const uint8_t *packed, __half *out
     fetch_tile(bid);
 #pragma unroll 1
     for (uint32_t tile = bid; tile < a.n_units; tile += nb) {
-        const uint32_t blk = tile >> 1, half = tile & 1, seq = blk / bps, bis = blk - seq * bps;
+        const uint32_t blk = tile >> 1, half = tile & 1, seq = a.bps_div.div(blk), bis = blk - seq * bps;
         __syncthreads();  // the previous tile's codes are no longer needed
         if (tid < PIECES) reinterpret_cast<uint4 *>(tile_s)[tid] = pre0;
         if constexpr (PIECES > 256) {
@@ -2457,7 +2462,7 @@ static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
     ka.quant_lut = h->quant_lut;
     ka.norm_correction = h->norm_correction; ka.tokens = tokens;
-    ka.blocks_per_seq = (uint32_t)bps; ka.n_units = (uint32_t)(n_blocks * 8);
+    ka.blocks_per_seq = (uint32_t)bps; ka.bps_div = make_fast_div((uint32_t)bps); ka.n_units = (uint32_t)(n_blocks * 8);
     ka.out_blocks_per_seq = (uint32_t)bps;
     return ka;
 }
@@ -2467,7 +2472,7 @@ static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     va.bfrag = (const uint4 *)h->rfrag16v; va.s2 = h->s2_32; va.symthr = h->symthr32; va.sqcoef = h->sqcoef32;
     va.quant_lut = h->quant_lut;
     va.norm_correction = h->norm_correction; va.tokens = tokens; va.share_k_lut = 0;
-    va.blocks_per_seq = (uint32_t)bps; va.n_units = (uint32_t)(n_blocks * 2);
+    va.blocks_per_seq = (uint32_t)bps; va.bps_div = make_fast_div((uint32_t)bps); va.n_units = (uint32_t)(n_blocks * 2);
     va.out_blocks_per_seq = (uint32_t)bps;
     return va;
 }
@@ -2869,9 +2874,9 @@ int tqk_load_kv(const tq_handle *hk, const tq_handle *hv, const void *packed_k, 
     }
     LoadK16Args ak, av;
     ak.afrag = (const uint4 *)hk->rfrag16k_inv; ak.s1 = hk->s1_32; ak.pair_lut = (const uint32_t *)hk->pair_lut;
-    ak.tokens = tokens; ak.blocks_per_seq = (uint32_t)bps; ak.n_units = (uint32_t)(n_seqs * bps * 8);
+    ak.tokens = tokens; ak.blocks_per_seq = (uint32_t)bps; ak.bps_div = make_fast_div((uint32_t)bps); ak.n_units = (uint32_t)(n_seqs * bps * 8);
     av.afrag = (const uint4 *)hv->rfrag16k_inv; av.s1 = hv->s1_32; av.pair_lut = (const uint32_t *)hv->pair_lut;
-    av.tokens = tokens; av.blocks_per_seq = (uint32_t)bps; av.n_units = (uint32_t)(n_seqs * bps * 2);
+    av.tokens = tokens; av.blocks_per_seq = (uint32_t)bps; av.bps_div = make_fast_div((uint32_t)bps); av.n_units = (uint32_t)(n_seqs * bps * 2);
     unsigned fit = 0;
 #define TQ_LKV(KB, VB)                                                                                             \
     {                                                                                                              \
@@ -2913,7 +2918,7 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
     if (out_dtype == TQ_F16 && kind == TQ_KIND_V && domain == TQ_DOMAIN_ORIGINAL && h->rfrag16k_inv) {
         LoadK16Args k;
         k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
-        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 2);
+        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.bps_div = make_fast_div((uint32_t)bps); k.n_units = (uint32_t)(n_seqs * bps * 2);
         static const unsigned fit[3] = {resident_workgroups(k_load_v16<2>), resident_workgroups(k_load_v16<3>),
                                         resident_workgroups(k_load_v16<4>)};
         const unsigned g16 = (unsigned)std::min<int64_t>((int64_t)k.n_units, fit[h->bits - 2]);
@@ -2927,7 +2932,7 @@ int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tok
     if (out_dtype == TQ_F16 && kind == TQ_KIND_K && domain == TQ_DOMAIN_ORIGINAL && h->rfrag16k_inv) {
         LoadK16Args k;
         k.afrag = (const uint4 *)h->rfrag16k_inv; k.s1 = h->s1_32; k.pair_lut = (const uint32_t *)h->pair_lut;
-        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.n_units = (uint32_t)(n_seqs * bps * 8);
+        k.tokens = tokens; k.blocks_per_seq = (uint32_t)bps; k.bps_div = make_fast_div((uint32_t)bps); k.n_units = (uint32_t)(n_seqs * bps * 8);
         static const unsigned fit[3] = {resident_workgroups(k_load_k16<2>), resident_workgroups(k_load_k16<3>),
                                         resident_workgroups(k_load_k16<4>)};
         const unsigned g16 = (unsigned)std::min<int64_t>(((int64_t)k.n_units + 3) / 4, fit[h->bits - 2]);
