@@ -375,14 +375,14 @@ def test_store_into_a_capacity_buffer_is_rejected_for_several_sequences():
 
 
 @pytest.mark.parametrize("kb,vb", [(3, 3), (4, 4), (3, 2)])
-@pytest.mark.parametrize("tokens", [64, 200, 256])
+@pytest.mark.parametrize("tokens", [64, 200, 256, 300, 700])
 def test_prefill_into_a_cache_laid_out_for_more_tokens(kb, vb, tokens):
     """tq_store_kv_cache: fp16 prompts go through the matrix-core store straight into buffers laid out for `capacity`
     tokens per sequence.  Every sequence's first blocks hold the bytes tq_store_kv writes for it, the other blocks stay
     untouched, and the cache then grows by appends as one that was filled by appends: the prefix is kept bit for bit and
     the appended token gets the same codes."""
     tt = L.torch()
-    n_seqs, capacity = 3, 512
+    n_seqs, capacity = 3, 512 if tokens < 500 else 1024
     kc, vc = tqa.TurboCodec(kb, seed=42), tqa.TurboCodec(vb, seed=542)
     rng = np.random.default_rng(100 * kb + tokens)
     k = rng.standard_normal((n_seqs, tokens + 1, D)).astype(np.float16)

@@ -123,6 +123,7 @@ def test_store_ragged_token_counts(tokens, bits, dtype):
 
 @pytest.mark.parametrize("kbits,vbits", [(3, 3), (4, 4), (2, 2), (4, 2), (3, 4)])
 @pytest.mark.parametrize("shape,dtype", [((2, 1024, D), np.float16), ((3, 200, D), np.float16), ((5, 40, D), np.float16),
+                                         ((4, 300, D), np.float16), ((3, 700, D), np.float16),   # 3 and 6 blocks per sequence
                                          ((2, 130, D), np.float32)])
 def test_store_kv_equals_separate_stores(kbits, vbits, shape, dtype):
     """One launch for K and V writes the same bytes as the two single-tensor stores
@@ -177,7 +178,7 @@ def test_load_both_domains(bits, kind):
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("kind", ["k", "v"])
-@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (5, 64)])
+@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (5, 64), (4, 300), (3, 700)])
 def test_load_fp16_matches_fp32_load(bits, kind, n_seqs, tokens):
     """fp16 output in the original domain runs the transposed rotation on the matrix cores with fp16
     centroids; the fp32 output keeps the fp32 butterfly.  Both decode the same codes: they agree to the
@@ -199,7 +200,7 @@ def test_load_fp16_matches_fp32_load(bits, kind, n_seqs, tokens):
 
 
 @pytest.mark.parametrize("kbits,vbits", [(2, 2), (3, 3), (4, 4), (4, 2), (3, 4), (2, 3)])
-@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (8, 4096)])
+@pytest.mark.parametrize("n_seqs,tokens", [(1, 16), (3, 129), (2, 1000), (8, 4096), (4, 300), (3, 700)])
 def test_load_kv_equals_two_loads(kbits, vbits, n_seqs, tokens):
     """tq_load_kv (K and V of a layer to fp16 in one launch) returns the bytes of the two tq_load calls it
     replaces, for every width pair, ragged sequence ends and grids smaller than the device, and writes nothing
