@@ -491,6 +491,44 @@ def boundary_layer_leg(torch, tqa, steps, warmup):
                         "note": "includes the allocation of the output buffer by the host wrapper"}}
 
 
+def cache_maintenance_leg(torch, tqa, steps, warmup):
+    """The kernels that rework a packed cache without the original vectors, on config 2's K tensor (262 144 vectors):
+    temporal decay (tq_requantize 3 -> 2 bits), export to and import from the llama.cpp fork's per-vector blocks.
+    Each is timed through the C ABI with the output allocated beforehand; bytes = the packed buffers read and written."""
+    import ctypes
+    from turboquant_plus_amd import _lib as L
+    heads, tokens = 8, 32768
+    c3, c2 = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(2, seed=42)
+    k = synth_kv(torch, heads, tokens, 900, outliers=4)
+    packed3 = c3.store(k, kind="k")
+    n3, n2 = tqa.packed_bytes(3, heads, tokens), tqa.packed_bytes(2, heads, tokens)
+    fb = int(L.lib().tq_fork_block_bytes(3))
+    out2 = torch.empty(n2, dtype=torch.uint8, device="cuda")
+    blocks = torch.empty((heads, tokens, fb), dtype=torch.uint8, device="cuda")
+    back3 = torch.empty(n3, dtype=torch.uint8, device="cuda")
+    lib = L.lib()
+
+    def requant(i):
+        L.check(lib.tq_requantize(c3.handle.h, c2.handle.h, L.ptr(packed3), heads, tokens, L.KIND_K, L.ptr(out2), L.stream_ptr()))
+
+    def export(i):
+        L.check(lib.tq_export_fork_blocks(c3.handle.h, L.ptr(packed3), heads, tokens, L.KIND_K, L.ptr(blocks), L.stream_ptr()))
+
+    def imp(i):
+        L.check(lib.tq_import_fork_blocks(c3.handle.h, L.ptr(blocks), heads, tokens, L.KIND_K, L.ptr(back3), L.stream_ptr()))
+
+    out = {"workload": "config 2's K tensor (8 heads x 32768 tokens, turbo3 codes) reworked in place of the original vectors"}
+    for name, fn, nbytes in (("requantize_3to2", requant, n3 + n2), ("export_fork_blocks", export, n3 + heads * tokens * fb),
+                             ("import_fork_blocks", imp, n3 + heads * tokens * fb)):
+        _, ms = time_steps(torch, fn, steps, warmup)
+        out[name] = {"us_per_call": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+                     "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    torch.cuda.synchronize()
+    if not torch.equal(back3, packed3):
+        raise RuntimeError("export followed by import changed the packed cache")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -538,6 +576,8 @@ def main():
             part["score_tile"] = score_tile_leg(torch, tqa, args.steps, args.warmup)
         if "boundary" in legs:
             part["boundary_layer_q8k_q8v"] = boundary_layer_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+        if "maintenance" in legs:
+            part["cache_maintenance"] = cache_maintenance_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
         if "peaks" in legs:
             part["measured_peaks"] = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
         print(json.dumps(part, ensure_ascii=False))
@@ -551,6 +591,8 @@ def main():
     tile = score_tile_leg(torch, tqa, args.steps, args.warmup)
     torch.cuda.empty_cache()
     boundary = boundary_layer_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
+    torch.cuda.empty_cache()
+    maintenance = cache_maintenance_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
     torch.cuda.empty_cache()
     peaks = measured_peaks_leg(torch, tqa, args.steps, args.warmup)
     if args.skip_cpu:
@@ -572,7 +614,8 @@ def main():
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu_store,
         "turbo4_store": s4, "turbo3_store": s3, "decode_attn": dec, "asym_decode_q8k_turbo2v": asym,
-        "score_tile": tile, "boundary_layer_q8k_q8v": boundary, "measured_peaks": peaks,
+        "score_tile": tile, "boundary_layer_q8k_q8v": boundary, "cache_maintenance": maintenance,
+        "measured_peaks": peaks,
     }
     print(json.dumps(line, ensure_ascii=False))
 

@@ -187,7 +187,8 @@ int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *pa
  * (qs[j/4] >> ((j%4)*2)) & 3, hi1 = (signs[j/8] >> (j%8)) & 1; docs/papers/block-size-experiment.md:33-39,
  * docs/papers/turbo4-resurrection.md:130-134), norm | qs[64] nibbles (turbo4, 66 B; :169), norm | qs[32]
  * (turbo2, 34 B).  The norm is the corrected group norm in both formats, so codes and norms move
- * unchanged; blocks is [n_seqs, tokens, tq_fork_block_bytes(bits)] bytes.  Import fills the rows
+ * unchanged; blocks is [n_seqs, tokens, tq_fork_block_bytes(bits)] bytes, 2-byte aligned (every block size is
+ * even and a block starts with its fp16 norm; TQ_ERR_ALIGN otherwise).  Import fills the rows
  * past `tokens` of the last block like tq_store does.  The layout is known from the fork's
  * documents only (the reference tree holds no code for it). */
 int64_t tq_fork_block_bytes(int32_t bits);

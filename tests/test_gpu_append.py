@@ -300,6 +300,21 @@ def test_fork_blocks_rejects_wrong_width():
         codec.import_fork_blocks(np.zeros((1, 128, 66), dtype=np.uint8))
 
 
+def test_fork_blocks_reject_an_odd_address():
+    """A fork block starts with its fp16 norm and every block size is even: the kernels read and write rows as
+    16-bit pieces, so a blocks buffer at an odd address is refused (TQ_ERR_ALIGN) before anything is launched."""
+    tt = L.torch()
+    codec = tqa.TurboCodec(3, seed=42)
+    packed = codec.store(np.random.default_rng(3).standard_normal((1, 128, D)).astype(np.float16))
+    raw = tt.zeros(128 * 50 + 2, dtype=tt.uint8, device="cuda")
+    lib = L.lib()
+    rc = lib.tq_export_fork_blocks(codec.handle.h, L.ptr(packed), 1, 128, L.KIND_K, L.ptr(raw[1:]), L.stream_ptr())
+    assert rc == L.ERR_ALIGN
+    rc = lib.tq_import_fork_blocks(codec.handle.h, L.ptr(raw[1:]), 1, 128, L.KIND_K, L.ptr(packed), L.stream_ptr())
+    assert rc == L.ERR_ALIGN
+    assert (np_(raw) == 0).all()
+
+
 # ---- q8_0-style buffers (boundary layers of a layer-adaptive policy) ---------------------------------------
 
 @pytest.mark.parametrize("kind", ["k", "v"])

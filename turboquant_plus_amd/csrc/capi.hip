@@ -598,6 +598,7 @@ static int fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t
     REQUIRE(src && dst, TQ_ERR_ARG, "%s: null pointer", who);
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "%s: bad kind %d", who, kind);
     REQUIRE(aligned16(to_fork ? src : dst), TQ_ERR_ALIGN, "%s: the packed buffer must be 16-byte aligned", who);
+    REQUIRE(((uintptr_t)(to_fork ? dst : src) & 1u) == 0, TQ_ERR_ALIGN, "%s: the blocks must be 2-byte aligned (a block starts with an fp16 norm)", who);
     return tqk_fork_blocks(h, to_fork, src, n_seqs, tokens, kind, dst, (hipStream_t)stream);
 }
 

@@ -114,13 +114,31 @@ __device__ inline void pack_block(const uint8_t *codes, const float *norms, uint
         constexpr int PER = pairs_per_dword(BITS);
         const int g = k, j = c;
         uint32_t word = 0;
+        if (kind == TQ_KIND_K) {
+            // a K row's pairs are neighbouring bytes of the stage: the dword's 2 PER codes (and the 3-bit tail's
+            // eight) come in 8-byte reads, code i at bit BITS i
+            const uint8_t *src = codes + r * CODE_STRIDE + 32 * g;
+            auto gather8 = [](uint2 v) {
+                uint32_t w = 0;
 #pragma unroll
-        for (int t = 0; t < PER; ++t) word |= pair_from_stage<BITS>(codes, kind, r, 16 * g + PER * j + t) << (2 * BITS * t);
-        if constexpr (BITS == 3) {
-            uint32_t tail = 0;
+                for (int i = 0; i < 4; ++i) {
+                    w |= ((v.x >> (8 * i)) & 0xFFu) << (BITS * i);
+                    w |= ((v.y >> (8 * i)) & 0xFFu) << (BITS * (4 + i));
+                }
+                return w;
+            };
+            word = gather8(*reinterpret_cast<const uint2 *>(src + 2 * PER * j));
+            if constexpr (BITS == 2) word |= gather8(*reinterpret_cast<const uint2 *>(src + 16 * j + 8)) << 16;
+            if constexpr (BITS == 3) word |= ((gather8(*reinterpret_cast<const uint2 *>(src + 24)) >> (8 * j)) & 0xFFu) << 24;
+        } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) tail |= pair_from_stage<3>(codes, kind, r, 16 * g + 12 + t) << (6 * t);
-            word |= ((tail >> (8 * j)) & 0xFFu) << 24;
+            for (int t = 0; t < PER; ++t) word |= pair_from_stage<BITS>(codes, kind, r, 16 * g + PER * j + t) << (2 * BITS * t);
+            if constexpr (BITS == 3) {
+                uint32_t tail = 0;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) tail |= pair_from_stage<3>(codes, kind, r, 16 * g + 12 + t) << (6 * t);
+                word |= ((tail >> (8 * j)) & 0xFFu) << 24;
+            }
         }
         out[o] = word;
     }
@@ -2590,33 +2608,33 @@ struct RequantArgs {
 template <int SB, int DB>
 __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t *dst, RequantArgs a) {
     constexpr int NB = (1 << DB) - 1;
+    constexpr int SRC_BYTES = block_bytes(SB);
+    __shared__ __attribute__((aligned(16))) uint8_t block_s[SRC_BYTES];  // the source block, copied with 16-byte loads
     __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
     __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
     __shared__ float csrc_s[1 << SB], cdst_s[1 << DB];
     const int tid = threadIdx.x, lane = tid & 63;
     const int li = lane & 15, grp = tid >> 4;
-    const uint8_t *sblock = src + (int64_t)blockIdx.x * block_bytes(SB);
+    {
+        const uint4 *sb = reinterpret_cast<const uint4 *>(src + (int64_t)blockIdx.x * SRC_BYTES);
+        for (int e = tid; e < SRC_BYTES / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = sb[e];
+    }
     if (tid < (1 << SB)) csrc_s[tid] = a.cent_src[tid];
     if (tid < (1 << DB)) cdst_s[tid] = a.cent_dst[tid];
     float bnd[NB];
 #pragma unroll
     for (int k = 0; k < NB; ++k) bnd[k] = a.bounds_dst[k];
-    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
-        const int t = e >> 7, dim = e & 127;
-        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(sblock, SB, a.kind, t, dim);
-    }
     __syncthreads();
 #pragma unroll 1
     for (int it = 0; it < 8; ++it) {
         const int t = it * 16 + grp;
-        const uint2 c8 = *reinterpret_cast<const uint2 *>(&codes[t * CODE_STRIDE + 8 * li]);
-        const float g = block_norm(sblock, SB, t);
+        const uint32_t c8 = load_codes8<SB>(block_s, a.kind, t, li);
+        const float g = block_norm(block_s, SB, t);
         float v[8];
         float ss = 0.0f;
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
-            const uint32_t c = ((m < 4 ? c8.x : c8.y) >> (8 * (m & 3))) & 0xFFu;
-            v[m] = csrc_s[c] * g;
+            v[m] = csrc_s[(c8 >> (m * SB)) & ((1u << SB) - 1u)] * g;
             ss = fmaf(v[m], v[m], ss);
         }
         ss = row16_sum(ss);
@@ -2637,7 +2655,6 @@ __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t 
             else w1 |= c << (8 * (m - 4));
         }
         cs = row16_sum(cs);
-        __builtin_amdgcn_wave_barrier();
         *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(w0, w1);
         if (li == 0) {
             const float cn = sqrtf(cs);
@@ -2671,41 +2688,45 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
 // in qs, the third in signs; 4-bit: nibbles; 2-bit: qs only) - 50 / 66 / 34 bytes.
 __host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 66 : 34; }
 
+// Sixteen lanes per row: lane li owns the codes of dims 8 li .. 8 li + 7, which are whole bytes of the fork's row in
+// every width (4-bit: four nibble bytes; 3-bit: two qs bytes and one signs byte; 2-bit: two qs bytes).
 template <int BITS>
 __global__ __launch_bounds__(256) void k_fork_export(const uint8_t *packed, uint8_t *out, int kind, int64_t tokens,
                                                      int64_t blocks_per_seq) {
     constexpr int FB = fork_block_bytes(BITS);
-    __shared__ uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
-    const int tid = threadIdx.x;
+    constexpr int SRC_BYTES = block_bytes(BITS);
+    __shared__ __attribute__((aligned(16))) uint8_t block_s[SRC_BYTES];  // the block, copied with 16-byte loads
+    const int tid = threadIdx.x, li = tid & 15, grp = tid >> 4;
     const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
-    const uint8_t *block = packed + blk * block_bytes(BITS);
-    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
-        const int t = e >> 7, dim = e & 127;
-        codes[t * CODE_STRIDE + dim] = (uint8_t)fetch_code(block, BITS, kind, t, dim);
+    {
+        const uint4 *sb = reinterpret_cast<const uint4 *>(packed + blk * SRC_BYTES);
+        for (int e = tid; e < SRC_BYTES / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = sb[e];
     }
     __syncthreads();
-    // one output byte per thread and step: byte b of the row of token t
-    for (int e = tid; e < TQ_ROWS_PER_BLOCK * FB; e += 256) {
-        const int t = e / FB, b = e % FB;
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
         const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
         if (tok >= tokens) continue;
-        const uint8_t *c = codes + t * CODE_STRIDE;
-        uint32_t v;
-        if (b < 2) {
-            v = (reinterpret_cast<const uint16_t *>(block + block_code_bytes(BITS))[t] >> (8 * b)) & 0xFFu;
-        } else if (BITS == 4) {
-            const int j = 2 * (b - 2);
-            v = c[j] | (c[j + 1] << 4);
-        } else if (b < 34) {
-            const int j = 4 * (b - 2);
-            v = (c[j] & 3) | ((c[j + 1] & 3) << 2) | ((c[j + 2] & 3) << 4) | ((c[j + 3] & 3) << 6);
+        const uint32_t w = load_codes8<BITS>(block_s, kind, t, li);  // code m at bit m BITS
+        uint8_t *row = out + (seq * tokens + tok) * FB;             // FB is even: the row is 2-byte aligned
+        if (li == 0) *reinterpret_cast<uint16_t *>(row) = reinterpret_cast<const uint16_t *>(block_s + block_code_bytes(BITS))[t];
+        if constexpr (BITS == 4) {
+            reinterpret_cast<uint16_t *>(row + 2)[2 * li] = (uint16_t)w;
+            reinterpret_cast<uint16_t *>(row + 2)[2 * li + 1] = (uint16_t)(w >> 16);
+        } else if constexpr (BITS == 2) {
+            reinterpret_cast<uint16_t *>(row + 2)[li] = (uint16_t)w;
         } else {
-            const int j = 8 * (b - 34);
-            v = 0;
+            uint32_t qs = 0, sg = 0;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v |= ((c[j + k] >> 2) & 1u) << k;
+            for (int m = 0; m < 8; ++m) {
+                const uint32_t c = (w >> (3 * m)) & 7u;
+                qs |= (c & 3u) << (2 * m);
+                sg |= (c >> 2) << m;
+            }
+            reinterpret_cast<uint16_t *>(row + 2)[li] = (uint16_t)qs;
+            row[34 + li] = (uint8_t)sg;
         }
-        out[(seq * tokens + tok) * FB + b] = (uint8_t)v;
     }
 }
 
@@ -2715,30 +2736,34 @@ __global__ __launch_bounds__(256) void k_fork_import(const uint8_t *in, uint8_t 
     constexpr int FB = fork_block_bytes(BITS);
     __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
     __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, li = tid & 15, grp = tid >> 4;
     const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
-    for (int e = tid; e < TQ_ROWS_PER_BLOCK * 128; e += 256) {
-        const int t = e >> 7, j = e & 127;
+#pragma unroll 1
+    for (int it = 0; it < 8; ++it) {
+        const int t = it * 16 + grp;
         const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
-        uint32_t c = zero_code;  // rows past the end: what the store kernels write there
+        uint32_t c[8];
+        float g = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) c[m] = zero_code;  // rows past the end: what the store kernels write there
         if (tok < tokens) {
             const uint8_t *row = in + (seq * tokens + tok) * FB;
-            if (BITS == 4) c = (row[2 + j / 2] >> ((j % 2) * 4)) & 0xFu;
-            else {
-                c = (row[2 + j / 4] >> ((j % 4) * 2)) & 3u;
-                if (BITS == 3) c |= ((row[34 + j / 8] >> (j % 8)) & 1u) << 2;
+            g = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(row)));
+            if constexpr (BITS == 4) {
+                const uint32_t w = reinterpret_cast<const uint16_t *>(row + 2)[2 * li] |
+                                   ((uint32_t) reinterpret_cast<const uint16_t *>(row + 2)[2 * li + 1] << 16);
+#pragma unroll
+                for (int m = 0; m < 8; ++m) c[m] = (w >> (4 * m)) & 15u;
+            } else {
+                const uint32_t qs = reinterpret_cast<const uint16_t *>(row + 2)[li];
+                const uint32_t sg = BITS == 3 ? row[34 + li] : 0u;
+#pragma unroll
+                for (int m = 0; m < 8; ++m) c[m] = ((qs >> (2 * m)) & 3u) | (((sg >> m) & 1u) << 2);
             }
         }
-        codes[t * CODE_STRIDE + j] = (uint8_t)c;
-    }
-    for (int t = tid; t < TQ_ROWS_PER_BLOCK; t += 256) {
-        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
-        float g = 0.0f;
-        if (tok < tokens) {
-            const uint8_t *row = in + (seq * tokens + tok) * FB;
-            g = __half2float(__ushort_as_half((unsigned short)(row[0] | (row[1] << 8))));
-        }
-        norms_s[t] = g;
+        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) =
+            make_uint2(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
+        if (li == 0) norms_s[t] = g;
     }
     __syncthreads();
     pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), kind);
