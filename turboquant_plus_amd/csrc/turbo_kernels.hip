@@ -328,7 +328,19 @@ __device__ __forceinline__ uint32_t append4_b2(uint32_t w, float y0, float y1, f
 // 4-bit codes by table: entry e of a value (tq_handle::quant_lut, indexed by the value's top 12 bits) holds in
 // .x the unfolded field [sign, boundaries below the bin] and in .y the one boundary inside the bin, so
 // field = e.x + (|y| > e.y): one compare and one add-with-carry per value instead of a three-level search.
-__device__ __forceinline__ uint32_t quant_lut_offset(float y) { return (__float_as_uint(y) >> 17) & 0x7ff8u; }
+// DUP: the table holds every entry twice (8192 x 8 B, load_quant_lut_dup), so that the byte offset is a plain mask of the
+// value's upper half - one instruction with sub-dword operand selection instead of a shift and a mask.
+template <bool DUP> __device__ __forceinline__ uint32_t quant_lut_offset(float y) {
+    if constexpr (DUP) {
+        uint32_t off;
+        asm("v_and_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+            : "=v"(off)
+            : "v"(0xfff8u), "v"(y));
+        return off;
+    } else {
+        return (__float_as_uint(y) >> 17) & 0x7ff8u;
+    }
+}
 
 __device__ __forceinline__ uint32_t append4_lut(uint32_t w, float y0, float y1, float y2, float y3, uint2 e0, uint2 e1, uint2 e2,
                                                 uint2 e3) {
@@ -467,6 +479,27 @@ template <int NT> __device__ __forceinline__ void load_quant_lut(uint2 *dst, con
     }
 }
 
+// the same table with every entry twice (entry i at 2i and 2i + 1): 64 KB, indexed by the value's top 13 bits
+template <int NT> __device__ __forceinline__ void load_quant_lut_dup(uint2 *dst, const uint2 *src) {
+    constexpr int N16 = 2048, PER = (N16 + NT - 1) / NT;  // 16-byte pieces of the source = pairs of entries
+    const uint4 *s4 = reinterpret_cast<const uint4 *>(src);
+    uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+    uint4 v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = (int)threadIdx.x + i * NT;
+        v[i] = s4[e < N16 ? e : N16 - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = (int)threadIdx.x + i * NT;
+        if (e < N16) {
+            d4[2 * e] = make_uint4(v[i].x, v[i].y, v[i].x, v[i].y);
+            d4[2 * e + 1] = make_uint4(v[i].z, v[i].w, v[i].z, v[i].w);
+        }
+    }
+}
+
 // RAGGED: sequences whose token count is not a multiple of the block size (rows past the
 // end are quantised as zeros, and the block index needs a division by blocks per sequence).
 // Units lo, lo + step, .. below end are handed out through a ticket counter in LDS (zero on
@@ -485,7 +518,7 @@ constexpr int K_UNITS_AHEAD = 1;
 // first_ticket: the wavefront's first two tickets are first_ticket and first_ticket + 1 (the counter starts past
 // them), or DRAW_TICKET to draw them.  `stage` makes the workgroup's LDS copy of the constant operands (frag,
 // flips) readable; it runs after the first inputs have been requested.
-template <int BITS, bool RAGGED, typename Stage>
+template <int BITS, bool RAGGED, bool DUP_LUT, typename Stage>
 __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const uint32_t *flips, uint32_t first_ticket, Stage &&stage) {
@@ -668,7 +701,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
 #if TQ_KNOCKOUT & 1
                         if (m == 0)
 #endif
-                        e[m] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(qlut) + quant_lut_offset(yn[m]));
+                        e[m] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(qlut) + quant_lut_offset<DUP_LUT>(yn[m]));
                     }
 #if TQ_KNOCKOUT & 1
                     uint32_t w = ko_append4(e[0].x & 1u, yn[7], yn[6], yn[5], yn[4]);
@@ -875,7 +908,7 @@ struct StoreVArgs {
 // constant operands (frag, s2: LDS) readable.
 // STREAM_IN: the input is read with the non-temporal hint (every 128-byte line is touched by two instructions of one
 // wavefront, back to back).  It gains 2 us in the fused K+V launch and loses 1 us in the V-only kernel (measured).
-template <int BITS, bool RAGGED, bool STREAM_IN, typename Stage>
+template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, typename Stage>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const float *s2, uint32_t first_ticket, Stage &&stage) {
@@ -1042,10 +1075,10 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 else {
                     const char *ql = reinterpret_cast<const char *>(qlut);
                     append_rows_lut(w[0][j], w[1][j], w[2][j], w[3][j], y0, y1, y2, y3,
-                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y0)),
-                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y1)),
-                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y2)),
-                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset(y3)));
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset<DUP_LUT>(y0)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset<DUP_LUT>(y1)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset<DUP_LUT>(y2)),
+                                    *reinterpret_cast<const uint2 *>(ql + quant_lut_offset<DUP_LUT>(y3)));
                 }
             }
             // level counts of the four tokens, one byte per token, summed over the 16 columns
@@ -1170,10 +1203,10 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
             if (t < 16) flip_s[t] = c3;
             __syncthreads();
         };
-        store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s,
+        store_k_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s,
                                     flip_s, 0u, stage);
     } else {
-        store_k_units<BITS, RAGGED>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, a.afrag,
+        store_k_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, a.afrag,
                                     a.s2flip, 0u, [] {});
     }
 }
@@ -1195,7 +1228,7 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
         if (t < 128) s2_s[t] = c2;
         __syncthreads();
     };
-    store_v_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
+    store_v_units<BITS, RAGGED, false, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
                                 stage);
 }
 
@@ -1207,8 +1240,8 @@ template <int KB, int VB, bool RAGGED>
 __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk, StoreKArgs ka, const __half *xv, uint8_t *pv,
                                                   StoreVArgs va) {
     __shared__ uint32_t counter[2];
-    __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 4096 : 2];
-    __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 4096 : 2];
+    __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 8192 : 2];  // every entry twice (load_quant_lut_dup)
+    __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 8192 : 2];
     __shared__ __attribute__((aligned(16))) uint4 frag_s[1024];  // V fragments, then K fragments
     __shared__ float s2_s[128];
     __shared__ uint32_t flip_s[16];
@@ -1218,10 +1251,10 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
     const float c2 = va.s2[t & 127];
     const uint32_t c3 = ka.s2flip[t & 15];
     if (t < 2) counter[t] = t == 0 ? 12u : 0u;  // V: the wavefronts' first tickets are their own numbers
-    const bool share_lut = KB == 4 && VB == 4 && va.share_k_lut;  // equal tables: one 32 KB copy serves both tensors
-    if constexpr (KB == 4) load_quant_lut<768>(qlut_k, ka.quant_lut);
+    const bool share_lut = KB == 4 && VB == 4 && va.share_k_lut;  // equal tables: one copy serves both tensors
+    if constexpr (KB == 4) load_quant_lut_dup<768>(qlut_k, ka.quant_lut);
     if constexpr (VB == 4) {
-        if (!share_lut) load_quant_lut<768>(qlut_v, va.quant_lut);
+        if (!share_lut) load_quant_lut_dup<768>(qlut_v, va.quant_lut);
     }
     auto stage = [&] {
         frag_s[t] = c0;
@@ -1230,10 +1263,10 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk,
         if (t < 16) flip_s[t] = c3;
         __syncthreads();
     };
-    store_v_units<VB, RAGGED, true>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
+    store_v_units<VB, RAGGED, true, true>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
                               wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], share_lut ? qlut_k : qlut_v, frag_s, s2_s,
                               (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
-    store_k_units<KB, RAGGED>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
+    store_k_units<KB, RAGGED, true>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
                               wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s,
                               DRAW_TICKET, [] {});
 }
