@@ -10,6 +10,9 @@ A step is one pass of the hot path over one batch of synthetic input:
   * the same leg in turbo3 (the bit width the 70 % target is stated for);
   * decode leg (BASELINE config 3): fused decode attention over turbo3 K/V,
     batch 16, 32 query heads on 8 KV heads, context 32768.
+Further legs, each under its own key of the line: config 4 (q8_0-style K, turbo2 V, Sparse V), the config 5 score
+tile and QJL store, a boundary layer (q8_0-style K and V), the kernels that rework a packed cache (requantise, export
+to and import from the fork's blocks) and the measured peaks of this box (stream probes, fp16 MFMA loop).
 Inputs are resident in HBM before the timed region; every step cycles through
 several distinct buffer sets so that the 256 MB Infinity Cache cannot serve
 the reads.  Kernel durations come from HIP events recorded on the stream the
@@ -536,7 +539,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--legs", default="all",
-                    help="comma-separated subset of store4,store3,decode,asym,tile,boundary,peaks (profiling runs); "
+                    help="comma-separated subset of store4,store3,decode,asym,tile,boundary,maintenance,peaks (profiling runs); "
                          "the JSON line then holds only those legs and is not the benchmark's line")
     ap.add_argument("--several-streams", action="store_true",
                     help="store legs: also time the launches issued round-robin on four streams (overlapping launches)")
