@@ -121,6 +121,21 @@ def test_store_ragged_token_counts(tokens, bits, dtype):
         assert np.all(i_full[:, tokens:] == zero_code) and np.all(g_full.reshape(3, -1)[:, tokens:] == 0)
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("tokens", [16384, 16448])
+def test_large_v_tensor_store_equals_the_kv_launch(bits, tokens):
+    """A V tensor of 512 blocks or more goes through the K+V kernel with an empty K share: the same bytes as the V
+    output of the K+V launch (which the tests above hold against the oracle), whole and ragged last blocks."""
+    tt = L.torch()
+    c = tqa.TurboCodec(bits, seed=542)
+    g = tt.Generator(device="cuda").manual_seed(bits * 7 + tokens)
+    v = tt.randn((4, tokens, D), generator=g, device="cuda").to(tt.float16)
+    v[1, 5] = 0
+    alone = c.store(v, kind="v")
+    _, both = tqa.TurboCodec(bits, seed=42).store_kv(c, v, v)
+    assert tt.equal(alone, both)
+
+
 @pytest.mark.parametrize("kbits,vbits", [(3, 3), (4, 4), (2, 2), (4, 2), (3, 4)])
 @pytest.mark.parametrize("shape,dtype", [((2, 1024, D), np.float16), ((3, 200, D), np.float16), ((5, 40, D), np.float16),
                                          ((4, 300, D), np.float16), ((3, 700, D), np.float16),   # 3 and 6 blocks per sequence
