@@ -254,8 +254,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         for b in range(B):                            # generated as in the store config, per sequence
             k = synth_kv(torch, Hkv, N, 100 + 16 * s + b, outliers=4)
             v = synth_kv(torch, Hkv, N, 200 + 16 * s + b, outliers=0)
-            kc.store(k, kind="k", out=kp[b * per:(b + 1) * per])
-            vc.store(v, kind="v", out=vp[b * per:(b + 1) * per])
+            kc.store_kv(vc, k, v, out_k=kp[b * per:(b + 1) * per], out_v=vp[b * per:(b + 1) * per])   # as a prefill does
         g = torch.Generator(device="cuda").manual_seed(300 + s)
         q = torch.randn((B, Hq, D), generator=g, device="cuda").to(torch.float16)
         sets.append((q, kp, vp))
