@@ -555,6 +555,16 @@ def main():
         print("bench.py: no GPU visible; the codec has no CPU path", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
+    # Bring the device out of idle before the first leg: a quarter of a second of plain device work, untimed and
+    # apart from every leg's own W warm-up steps, so that the first leg does not start on a clock that is still
+    # settling after the process's start-up (the store leg, which carries `value`, runs first).
+    scratch = torch.zeros(1 << 26, dtype=torch.float32, device="cuda")
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.25:
+        for _ in range(20):
+            scratch.add_(1.0)
+        torch.cuda.synchronize()
+    del scratch
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
