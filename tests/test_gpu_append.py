@@ -294,6 +294,35 @@ def test_fork_blocks_export_import(bits, kind):
     assert np.array_equal(np_(i2).reshape(-1, D), ridx) and np.array_equal(np_(g2).reshape(-1).astype(np.float16), rg)
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_fork_blocks_and_requantize_at_config_2_size(bits, kind):
+    """262 144 vectors (8 heads x 32768 tokens, the store configuration): export followed by import gives the packed
+    buffer back byte for byte; sampled rows of the export equal the oracle's packing of the unpacked codes; and a
+    requantised buffer decodes, on sampled rows, to the codes the oracle's requantisation of those rows gives."""
+    tt = L.torch()
+    heads, tokens = 8, 32768
+    codec = tqa.TurboCodec(bits, seed=42)
+    g = tt.Generator(device="cuda").manual_seed(50 + bits)
+    x = tt.randn((heads, tokens, D), generator=g, device="cuda").to(tt.float16)
+    packed = codec.store(x, kind=kind)
+    blocks = codec.export_fork_blocks(packed, heads, tokens, kind=kind)
+    assert tt.equal(codec.import_fork_blocks(blocks, kind=kind), packed)
+    idx, gn = codec.unpack_codes(packed, heads, tokens, kind=kind)
+    rows = np.random.default_rng(bits).integers(0, heads * tokens, size=256)
+    idx_s = np_(idx).reshape(-1, D)[rows]
+    g_s = np_(gn).reshape(-1)[rows].astype(np.float16)
+    assert np.array_equal(np_(blocks).reshape(heads * tokens, -1)[rows], O.fork_blocks_pack(idx_s, g_s, bits))
+    if bits > 2:
+        dst = tqa.TurboCodec(bits - 1, seed=42)
+        narrow = codec.requantize_to(dst, packed, heads, tokens, kind=kind)
+        i2, g2 = dst.unpack_codes(narrow, heads, tokens, kind=kind)
+        want_i, want_g = O.requantize(idx_s, g_s.astype(np.float32), codec.centroids, dst.centroids)
+        got_i = np_(i2).reshape(-1, D)[rows]
+        assert (got_i != want_i).mean() < 1e-4                       # fp32 on the device, float64 in the oracle: boundary cases
+        assert np.allclose(np_(g2).reshape(-1)[rows], want_g, rtol=2e-3)
+
+
 def test_fork_blocks_rejects_wrong_width():
     codec = tqa.TurboCodec(3, seed=42)
     with pytest.raises(ValueError):
