@@ -161,16 +161,21 @@ int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
 /* tq_append_kv with the position read from device memory when the launch runs (*pos_dev, an int64): a decode
  * step captured once (HIP graph) can be replayed while the cache grows; the caller advances the counter
  * between replays (any kernel on the same stream).  A position that is negative or does not leave room for
- * n_new tokens writes nothing.  Together with tq_attn_params.tokens_dev.  No counterpart in the reference;
- * for the callers that replay captured launches. */
+ * n_new tokens writes nothing to the cache; when overrun_dev is not NULL (a 4-byte aligned uint32 in device
+ * memory that the caller zeroes once) such a launch ORs TQ_OVERRUN_NEGATIVE or TQ_OVERRUN_NO_ROOM into it, and the
+ * word keeps the bits until the caller clears it: a serving loop reads it once after its graph replays instead
+ * of trusting TQ_OK, which only says that the launch was issued.  Together with tq_attn_params.tokens_dev.  No
+ * counterpart in the reference; for the callers that replay captured launches. */
+#define TQ_OVERRUN_NEGATIVE 1u /* *pos_dev < 0                      */
+#define TQ_OVERRUN_NO_ROOM 2u  /* *pos_dev + n_new > capacity       */
 int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                     const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k,
-                    void *packed_v, void *stream);
+                    void *packed_v, uint32_t *overrun_dev, void *stream);
 /* The same for one tensor (tq_append) and for q8_0-style buffers (tq_q8_0_append). */
 int tq_append_at(const tq_handle *h, const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new,
-                 int64_t capacity, int in_dtype, int kind, void *packed, void *stream);
+                 int64_t capacity, int in_dtype, int kind, void *packed, uint32_t *overrun_dev, void *stream);
 int tq_q8_0_append_at(const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
-                      int in_dtype, int kind, void *packed, void *stream);
+                      int in_dtype, int kind, void *packed, uint32_t *overrun_dev, void *stream);
 
 
 /* Temporal decay: re-quantise a packed buffer to a narrower width without going back to the
@@ -185,10 +190,13 @@ int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *pa
 /* Interchange with the llama.cpp fork's per-128 block layout, one block per vector in token
  * order: norm fp16 | qs[32] | signs[16] (turbo3, 50 B: idx = low2 | hi1 << 2, low2 =
  * (qs[j/4] >> ((j%4)*2)) & 3, hi1 = (signs[j/8] >> (j%8)) & 1; docs/papers/block-size-experiment.md:33-39,
- * docs/papers/turbo4-resurrection.md:130-134), norm | qs[64] nibbles (turbo4, 66 B; :169), norm | qs[32]
- * (turbo2, 34 B).  The norm is the corrected group norm in both formats, so codes and norms move
- * unchanged; blocks is [n_seqs, tokens, tq_fork_block_bytes(bits)] bytes, 2-byte aligned (every block size is
- * even and a block starts with its fp16 norm; TQ_ERR_ALIGN otherwise).  Import fills the rows
+ * docs/papers/turbo4-resurrection.md:130-134), norm fp16 | rnorm fp16 | qs[64] nibbles (turbo4, 68 B = 4.25 bits
+ * per value: docs/papers/turbo4-resurrection.md:169,208, README.md:43; rnorm is the residual-norm slot that
+ * the fork's struct keeps from its 3-bit + QJL days, docs/turbo4-investigation.md:42-49: exported as 0, ignored
+ * on import; that it sits right after norm is this library's reading of the documents, which print the size and
+ * the nibble formula but not the field order), norm | qs[32] (turbo2, 34 B).  The norm is the corrected group
+ * norm in both formats, so codes and norms move unchanged; blocks is [n_seqs, tokens, tq_fork_block_bytes(bits)]
+ * bytes, 2-byte aligned (4-byte aligned for turbo4, whose rows move as 4-byte words; TQ_ERR_ALIGN otherwise).  Import fills the rows
  * past `tokens` of the last block like tq_store does.  The layout is known from the fork's
  * documents only (the reference tree holds no code for it). */
 int64_t tq_fork_block_bytes(int32_t bits);

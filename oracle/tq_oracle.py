@@ -728,12 +728,16 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
 #   turbo3: norm fp16 | qs[32] | signs[16]  (50 B), idx = low2 | hi1 << 2,
 #           low2 = (qs[j/4] >> ((j%4)*2)) & 3, hi1 = (signs[j/8] >> (j%8)) & 1
 #           (docs/papers/block-size-experiment.md:33-39, docs/papers/turbo4-resurrection.md:130-134)
-#   turbo4: norm fp16 | qs[64]  (66 B), idx = (qs[j/2] >> ((j%2)*4)) & 0xF (turbo4-resurrection.md:169)
+#   turbo4: norm fp16 | rnorm fp16 | qs[64]  (68 B = 4.25 bits per value: turbo4-resurrection.md:208 "qs[64],
+#           maintaining the 68-byte block size", README.md:43,94), idx = (qs[j/2] >> ((j%2)*4)) & 0xF
+#           (turbo4-resurrection.md:169).  rnorm is the residual-norm field the struct keeps from the 3-bit + QJL
+#           turbo4 (docs/turbo4-investigation.md:42-49); 4-bit PolarQuant does not use it: packed as 0, ignored
+#           when unpacked.  Its position (right after norm) is not printed anywhere in the reference tree.
 #   turbo2: norm fp16 | qs[32]  (34 B), idx = (qs[j/4] >> ((j%4)*2)) & 3   (the 2-bit half of turbo3)
 # --------------------------------------------------------------------------
 
 def fork_block_bytes(bits: int) -> int:
-    return {2: 34, 3: 50, 4: 66}[bits]
+    return {2: 34, 3: 50, 4: 68}[bits]
 
 
 def fork_blocks_pack(idx: np.ndarray, g: np.ndarray, bits: int) -> np.ndarray:
@@ -743,7 +747,7 @@ def fork_blocks_pack(idx: np.ndarray, g: np.ndarray, bits: int) -> np.ndarray:
     out = np.zeros((T, fork_block_bytes(bits)), dtype=np.uint8)
     out[:, 0:2] = np.asarray(g, dtype=np.float16).reshape(T, 1).view(np.uint8)
     if bits == 4:
-        out[:, 2:66] = idx[:, 0::2] | (idx[:, 1::2] << 4)
+        out[:, 4:68] = idx[:, 0::2] | (idx[:, 1::2] << 4)   # bytes 2..3: rnorm, unused, zero
         return out
     low = idx & 3
     out[:, 2:34] = low[:, 0::4] | (low[:, 1::4] << 2) | (low[:, 2::4] << 4) | (low[:, 3::4] << 6)
@@ -759,7 +763,7 @@ def fork_blocks_unpack(buf: np.ndarray, bits: int):
     g = np.ascontiguousarray(buf[:, 0:2]).view(np.float16).reshape(T)
     j = np.arange(128)
     if bits == 4:
-        idx = (buf[:, 2 + j // 2] >> ((j % 2) * 4)) & 0xF
+        idx = (buf[:, 4 + j // 2] >> ((j % 2) * 4)) & 0xF
         return idx.astype(np.uint8), g
     idx = (buf[:, 2 + j // 4] >> ((j % 4) * 2)) & 3
     if bits == 3:

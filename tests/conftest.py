@@ -4,6 +4,10 @@ import sys
 import numpy as np
 import pytest
 
+# Every DecodeAttention of the test suite fills its output rows with NaN before a call: a row that the launch's
+# in-kernel merge did not write fails the comparison instead of passing on the previous call's values.
+os.environ.setdefault("TQ_POISON_OUTPUT", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 for p in (ROOT, os.path.join(ROOT, "oracle")):
     if p not in sys.path:

@@ -69,7 +69,7 @@ int main() {
     EXPECT(tq_packed_bytes(3, -1, 1) < 0);
     EXPECT(tq_q8_0_bytes(1, 1) == 128 * 136);
     EXPECT(tq_q8_0_bytes(-1, 1) < 0);
-    EXPECT(tq_fork_block_bytes(3) == 50 && tq_fork_block_bytes(4) == 66 && tq_fork_block_bytes(2) == 34 && tq_fork_block_bytes(5) < 0);
+    EXPECT(tq_fork_block_bytes(3) == 50 && tq_fork_block_bytes(4) == 68 && tq_fork_block_bytes(2) == 34 && tq_fork_block_bytes(5) < 0);
 
     EXPECT(tq_store(nullptr, ok, 1, 1, TQ_F16, TQ_KIND_K, ok, nullptr) == TQ_ERR_ARG);
     EXPECT(tq_store_kv(nullptr, nullptr, ok, ok, 1, 1, TQ_F16, ok, ok, nullptr) == TQ_ERR_ARG);
@@ -91,6 +91,13 @@ int main() {
     EXPECT(tq_q8_0_unpack_v(nullptr, 1, 1, (int8_t *)ok, (float *)ok, nullptr) == TQ_ERR_ARG);
     EXPECT(tq_q8_0_append(nullptr, 1, 0, 1, 128, TQ_F16, TQ_KIND_K, ok, nullptr) == TQ_ERR_ARG);
     EXPECT(tq_q8_0_append(ok, 1, 127, 2, 128, TQ_F16, TQ_KIND_K, ok, nullptr) == TQ_ERR_ARG);   // past the capacity
+    // appends at a position in device memory: null position, misaligned position or overrun word, too many tokens
+    EXPECT(tq_q8_0_append_at(ok, 1, nullptr, 1, 128, TQ_F16, TQ_KIND_K, ok, nullptr, nullptr) == TQ_ERR_ARG);
+    EXPECT(tq_q8_0_append_at(ok, 1, (const int64_t *)odd, 1, 128, TQ_F16, TQ_KIND_K, ok, nullptr, nullptr) == TQ_ERR_ALIGN);
+    EXPECT(tq_q8_0_append_at(ok, 1, (const int64_t *)ok, 1, 128, TQ_F16, TQ_KIND_K, ok, (uint32_t *)odd, nullptr) == TQ_ERR_ALIGN);
+    EXPECT(tq_q8_0_append_at(ok, 1, (const int64_t *)ok, 129, 128, TQ_F16, TQ_KIND_K, ok, nullptr, nullptr) == TQ_ERR_ARG);
+    EXPECT(tq_append_at(nullptr, ok, 1, (const int64_t *)ok, 1, 128, TQ_F16, TQ_KIND_K, ok, nullptr, nullptr) == TQ_ERR_ARG);
+    EXPECT(tq_append_kv_at(nullptr, nullptr, ok, ok, 1, (const int64_t *)ok, 1, 128, TQ_F16, ok, ok, nullptr, nullptr) == TQ_ERR_ARG);
 
     tq_attn_params p;
     memset(&p, 0, sizeof p);

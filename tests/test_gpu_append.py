@@ -12,6 +12,7 @@ import pytest
 import tq_oracle as O
 import turboquant_plus_amd as tqa
 from turboquant_plus_amd import _lib as L
+from turboquant_plus_amd.turbo import OVERRUN_NEGATIVE, OVERRUN_NO_ROOM, overrun_bits
 from test_gpu_turbo import check_codes, np_
 
 pytestmark = pytest.mark.gpu
@@ -290,6 +291,9 @@ def test_fork_blocks_export_import(bits, kind):
     ridx = rng.integers(0, 1 << bits, size=(2 * 128, D)).astype(np.uint8)
     rg = np.abs(rng.standard_normal(2 * 128)).astype(np.float16)
     ext = O.fork_blocks_pack(ridx, rg, bits).reshape(2, 128, -1)
+    if bits == 4:
+        assert ext.shape[2] == 68 and (np_(blocks)[:, :, 2:4] == 0).all()   # 4.25 bits per value; rnorm exported as 0
+        ext[:, :, 2:4] = 0x5A                                                # and ignored on the way in
     i2, g2 = codec.unpack_codes(codec.import_fork_blocks(ext, kind=kind), 2, 128, kind=kind)
     assert np.array_equal(np_(i2).reshape(-1, D), ridx) and np.array_equal(np_(g2).reshape(-1).astype(np.float16), rg)
 
@@ -342,6 +346,15 @@ def test_fork_blocks_reject_an_odd_address():
     rc = lib.tq_import_fork_blocks(codec.handle.h, L.ptr(raw[1:]), 1, 128, L.KIND_K, L.ptr(packed), L.stream_ptr())
     assert rc == L.ERR_ALIGN
     assert (np_(raw) == 0).all()
+    # 4-bit blocks (68 bytes: norm, rnorm, sixteen 4-byte code words) move as 4-byte words
+    codec4 = tqa.TurboCodec(4, seed=42)
+    packed4 = codec4.store(np.random.default_rng(3).standard_normal((1, 128, D)).astype(np.float16))
+    raw4 = tt.zeros(128 * 68 + 4, dtype=tt.uint8, device="cuda")
+    rc = lib.tq_export_fork_blocks(codec4.handle.h, L.ptr(packed4), 1, 128, L.KIND_K, L.ptr(raw4[2:]), L.stream_ptr())
+    assert rc == L.ERR_ALIGN
+    rc = lib.tq_import_fork_blocks(codec4.handle.h, L.ptr(raw4[2:]), 1, 128, L.KIND_K, L.ptr(packed4), L.stream_ptr())
+    assert rc == L.ERR_ALIGN
+    assert (np_(raw4) == 0).all()
 
 
 # ---- q8_0-style buffers (boundary layers of a layer-adaptive policy) ---------------------------------------
@@ -612,15 +625,38 @@ def test_layer_appends_at_a_position_on_the_device(fmt):
     ak, av = layer.new_cache(n_seqs, cap)
     bk, bv = layer.new_cache(n_seqs, cap)
     pos_d = tt.zeros(1, dtype=tt.int64, device="cuda")
+    over = tt.zeros(1, dtype=tt.int32, device="cuda")     # the sticky word a refused position sets
     pos = 0
     for n_new in (100, 27, 1, 1, 130, 1):          # 0 -> 100 -> 127 -> 128 -> 129 -> 259 -> 260
         layer.append(k[:, pos:pos + n_new], v[:, pos:pos + n_new], ak, av, pos, cap)
         pos_d.fill_(pos)
-        layer.append(k[:, pos:pos + n_new], v[:, pos:pos + n_new], bk, bv, pos_d, cap)
+        layer.append(k[:, pos:pos + n_new], v[:, pos:pos + n_new], bk, bv, pos_d, cap, overrun=over)
         pos += n_new
         assert tt.equal(ak, bk) and tt.equal(av, bv), f"after {pos} tokens"
+    assert overrun_bits(over) == 0                  # every position so far had room
+    pos_d.fill_(cap - 2)                            # the last position with room for two tokens: accepted
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=over)
+    layer.append(k[:, :2], v[:, :2], ak, av, cap - 2, cap)
+    assert overrun_bits(over) == 0 and tt.equal(ak, bk) and tt.equal(av, bv)
+    # no room: nothing written, TQ_OK all the same, and the word says so and keeps saying so
     pos_d.fill_(cap - 1)
-    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap)                 # without a word: silent, as before
     assert tt.equal(ak, bk) and tt.equal(av, bv)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=over)
+    assert tt.equal(ak, bk) and tt.equal(av, bv) and overrun_bits(over) == OVERRUN_NO_ROOM
+    pos_d.fill_(0)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=over)   # a good append later does not clear it
+    layer.append(k[:, :2], v[:, :2], ak, av, 0, cap)
+    assert tt.equal(ak, bk) and tt.equal(av, bv) and overrun_bits(over) == OVERRUN_NO_ROOM
+    # a negative position, and a counter full of garbage whose sum with n_new would wrap an int64
+    pos_d.fill_(-5)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=over)
+    assert tt.equal(ak, bk) and tt.equal(av, bv) and overrun_bits(over) == OVERRUN_NO_ROOM | OVERRUN_NEGATIVE
+    over.zero_()
+    pos_d.fill_(2 ** 63 - 1)
+    layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=over)
+    assert tt.equal(ak, bk) and tt.equal(av, bv) and overrun_bits(over) == OVERRUN_NO_ROOM
+    with pytest.raises(ValueError):
+        layer.append(k[:, :2], v[:, :2], bk, bv, pos_d, cap, overrun=tt.zeros(1, dtype=tt.int64, device="cuda"))
     with pytest.raises(ValueError):
         layer.append(k[:, :2], v[:, :2], bk, bv, tt.zeros(1, dtype=tt.int32, device="cuda"), cap)

@@ -256,6 +256,33 @@ def test_decode_attention_many_groups_and_repeated_calls():
         assert np.array_equal(again, first)
 
 
+@pytest.mark.parametrize("n_splits,sparse", [(32, False), (64, False), (32, True)])
+def test_in_launch_merge_never_leaves_a_row_unwritten(n_splits, sparse):
+    """The split partials of a group are merged inside the launch by the workgroup that finds every flag of its group
+    raised.  Shape of the headline step in small: 32 splits = two workgroups of sixteen wavefronts per group (64: four).
+    1000 steps back to back on one workspace, the output rows filled with NaN before each: every step must equal the
+    first, which is checked against the oracle - a step whose merge found no taker would leave NaN, a merge that ran on
+    stale partials would differ.  The Sparse-V total travels by the same protocol and must be the first step's too."""
+    tt = L.torch()
+    B, Hq, Hkv, N = 4, 8, 2, 64 * n_splits
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=n_splits)
+    q = tt.from_numpy(np.random.default_rng(7).standard_normal((B, Hq, D)).astype(np.float16)).cuda()
+    tau = 1e-3 if sparse else 0.0
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau, poison_output=True)
+    first = attn(q, kp, vp).clone()
+    skip0 = attn.skip.clone()
+    ref, sk, _ = reference_attention(np_(q), kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau)
+    assert_close(np_(first), ref)
+    if sparse:
+        assert abs(attn.skip_rate() - sk) < 1e-3
+    bad = tt.zeros(1, dtype=tt.int64, device="cuda")
+    for step in range(1000):
+        out = attn(q, kp, vp)
+        bad += (~tt.eq(out, first)).sum() + (0 if not sparse else (~tt.eq(attn.skip, skip0)).sum())
+        if step % 100 == 99:                 # stop at the first failure, to the nearest hundred steps
+            assert int(bad.item()) == 0, f"a step among {step - 99}..{step} left a row unwritten or different"
+
+
 def test_decode_attention_q8_0_k_turbo2_v():
     """BASELINE config 4 shape family: K q8_0-style (not rotated), V turbo2."""
     B, Hq, Hkv, N = 1, 8, 2, 2048 + 64
@@ -413,7 +440,7 @@ def test_score_tile_edges(nk, nq):
     scale = np.linalg.norm(qs.astype(np.float64), axis=1).max() * np.linalg.norm(keys.astype(np.float64), axis=1).max()
     for dt, tol in ((tt.float32, 2e-3 * scale / np.sqrt(D) * 4), (tt.float16, 4e-3 * max(np.abs(ref).max(), 1.0))):
         # the logits sit in the middle of a larger buffer filled with a sentinel
-        for pad in (64,):  # the entry point asks for 16-byte aligned logits
+        for pad in (64, 1, 3):  # 16-byte aligned, and aligned to the element only (2 or 4, 6 or 12 bytes off)
             buf = tt.full((nq * nk + 2 * pad,), 1024.0, dtype=dt, device="cuda")
             out = buf[pad:pad + nq * nk].view(nq, nk)
             got = codec.score_tile(qs, packed, sbits, rn, nk, out_dtype=dt, out=out)

@@ -386,17 +386,22 @@ def test_score_tile_is_dequantised_inner_product():
 @pytest.mark.parametrize("bits", [2, 3, 4])
 def test_fork_block_layout_formulas(bits):
     """Per-128 block layout of the llama.cpp fork: the extraction formulas printed in
-    docs/papers/turbo4-resurrection.md:130-134,169 and the sizes of docs/papers/block-size-experiment.md:33-39,
-    applied element by element to what fork_blocks_pack wrote."""
+    docs/papers/turbo4-resurrection.md:130-134,169, applied element by element to what fork_blocks_pack wrote, and
+    the block sizes the reference prints: 50 B for turbo3 (3.125 bits per value, docs/papers/block-size-experiment.md:33-39),
+    68 B for turbo4 (docs/papers/turbo4-resurrection.md:208 "qs[64], maintaining the 68-byte block size"; 4.25 bits
+    per value, README.md:43,94), 34 B for turbo2 (2.125)."""
     rng = np.random.default_rng(bits)
     idx = rng.integers(0, 1 << bits, size=(5, 128)).astype(np.uint8)
     g = rng.standard_normal(5).astype(np.float16)
     buf = O.fork_blocks_pack(idx, g, bits)
-    assert buf.shape == (5, {2: 34, 3: 50, 4: 66}[bits])
+    assert buf.shape == (5, {2: 34, 3: 50, 4: 68}[bits])
+    assert O.fork_block_bytes(bits) * 8 / 128 == {2: 2.125, 3: 3.125, 4: 4.25}[bits]   # the figures the reference prints
     for t in range(5):
         row = buf[t]
         assert row[:2].view(np.float16)[0] == g[t]
-        qs = row[2:66] if bits == 4 else row[2:34]
+        if bits == 4:
+            assert row[2] == 0 and row[3] == 0          # the struct's unused rnorm field
+        qs = row[4:68] if bits == 4 else row[2:34]
         signs = row[34:50] if bits == 3 else None
         for j in range(128):
             if bits == 4:
@@ -408,3 +413,7 @@ def test_fork_block_layout_formulas(bits):
             assert got == idx[t, j]
     i2, g2 = O.fork_blocks_unpack(buf, bits)
     assert np.array_equal(i2, idx) and np.array_equal(g2.view(np.uint16), g.view(np.uint16))
+    if bits == 4:                                        # whatever a writer left in rnorm does not reach the codes
+        buf[:, 2:4] = 0xA5
+        i3, g3 = O.fork_blocks_unpack(buf, bits)
+        assert np.array_equal(i3, idx) and np.array_equal(g3.view(np.uint16), g.view(np.uint16))

@@ -61,9 +61,9 @@ PROTOTYPES = {
     "tq_store_kv_cache": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _P, _P, _P]),
     "tq_append": (_I, [_P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "tq_append_kv": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _P, _P]),
-    "tq_append_kv_at": (_I, [_P, _P, _P, _P, _L, _P, _L, _L, _I, _P, _P, _P]),
-    "tq_append_at": (_I, [_P, _P, _L, _P, _L, _L, _I, _I, _P, _P]),
-    "tq_q8_0_append_at": (_I, [_P, _L, _P, _L, _L, _I, _I, _P, _P]),
+    "tq_append_kv_at": (_I, [_P, _P, _P, _P, _L, _P, _L, _L, _I, _P, _P, _P, _P]),
+    "tq_append_at": (_I, [_P, _P, _L, _P, _L, _L, _I, _I, _P, _P, _P]),
+    "tq_q8_0_append_at": (_I, [_P, _L, _P, _L, _L, _I, _I, _P, _P, _P]),
     "tq_requantize": (_I, [_P, _P, _P, _L, _L, _I, _P, _P]),
     "tq_fork_block_bytes": (_L, [C.c_int32]),
     "tq_export_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),

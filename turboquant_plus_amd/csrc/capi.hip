@@ -80,7 +80,7 @@ int tq_check_launch(const char *what) {
 
 extern "C" {
 
-int tq_version(void) { return 100; }
+int tq_version(void) { return 101; }
 
 const char *tq_last_error(void) { return g_err; }
 
@@ -530,7 +530,7 @@ int tq_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
 }
 
 int tq_append_at(const tq_handle *h, const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
-                 int in_dtype, int kind, void *packed, void *stream) {
+                 int in_dtype, int kind, void *packed, uint32_t *overrun_dev, void *stream) {
     int rc = check_fast(h, "tq_append_at");
     if (rc) return rc;
     REQUIRE(n_seqs >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_append_at: bad argument");
@@ -541,11 +541,12 @@ int tq_append_at(const tq_handle *h, const void *x, int64_t n_seqs, const int64_
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_append_at: bad kind %d", kind);
     REQUIRE(aligned16(x) && aligned16(packed), TQ_ERR_ALIGN, "tq_append_at: x and packed must be 16-byte aligned");
     REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_append_at: pos_dev must be 8-byte aligned");
-    return tqk_append(h, x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev);
+    REQUIRE((reinterpret_cast<uintptr_t>(overrun_dev) & 3u) == 0, TQ_ERR_ALIGN, "tq_append_at: overrun_dev must be 4-byte aligned");
+    return tqk_append(h, x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev, overrun_dev);
 }
 
 int tq_q8_0_append_at(const void *x, int64_t n_seqs, const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype,
-                      int kind, void *packed, void *stream) {
+                      int kind, void *packed, uint32_t *overrun_dev, void *stream) {
     REQUIRE(n_seqs >= 0 && n_new >= 0 && capacity >= 0, TQ_ERR_ARG, "tq_q8_0_append_at: bad argument");
     REQUIRE(n_new <= capacity, TQ_ERR_ARG, "tq_q8_0_append_at: %lld tokens do not fit a capacity of %lld", (long long)n_new,
             (long long)capacity);
@@ -554,12 +555,13 @@ int tq_q8_0_append_at(const void *x, int64_t n_seqs, const int64_t *pos_dev, int
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "tq_q8_0_append_at: bad kind %d", kind);
     REQUIRE(aligned16(packed), TQ_ERR_ALIGN, "tq_q8_0_append_at: packed must be 16-byte aligned");
     REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_q8_0_append_at: pos_dev must be 8-byte aligned");
-    return tqk_q8_0_append(x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev);
+    REQUIRE((reinterpret_cast<uintptr_t>(overrun_dev) & 3u) == 0, TQ_ERR_ALIGN, "tq_q8_0_append_at: overrun_dev must be 4-byte aligned");
+    return tqk_q8_0_append(x, n_seqs, 0, n_new, capacity, in_dtype, kind, packed, (hipStream_t)stream, pos_dev, overrun_dev);
 }
 
 int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs,
                     const int64_t *pos_dev, int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v,
-                    void *stream) {
+                    uint32_t *overrun_dev, void *stream) {
     int rc = check_fast(hk, "tq_append_kv_at");
     rc = rc ? rc : check_fast(hv, "tq_append_kv_at");
     if (rc) return rc;
@@ -571,7 +573,9 @@ int tq_append_kv_at(const tq_handle *hk, const tq_handle *hv, const void *k, con
     REQUIRE(aligned16(k) && aligned16(v) && aligned16(packed_k) && aligned16(packed_v), TQ_ERR_ALIGN,
             "tq_append_kv_at: inputs and packed buffers must be 16-byte aligned");
     REQUIRE((reinterpret_cast<uintptr_t>(pos_dev) & 7u) == 0, TQ_ERR_ALIGN, "tq_append_kv_at: pos_dev must be 8-byte aligned");
-    return tqk_append_kv(hk, hv, k, v, n_seqs, 0, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream, pos_dev);
+    REQUIRE((reinterpret_cast<uintptr_t>(overrun_dev) & 3u) == 0, TQ_ERR_ALIGN, "tq_append_kv_at: overrun_dev must be 4-byte aligned");
+    return tqk_append_kv(hk, hv, k, v, n_seqs, 0, n_new, capacity, in_dtype, packed_k, packed_v, (hipStream_t)stream, pos_dev,
+                         overrun_dev);
 }
 
 int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *packed_src, int64_t n_seqs, int64_t tokens,
@@ -598,11 +602,15 @@ static int fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t
     REQUIRE(src && dst, TQ_ERR_ARG, "%s: null pointer", who);
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "%s: bad kind %d", who, kind);
     REQUIRE(aligned16(to_fork ? src : dst), TQ_ERR_ALIGN, "%s: the packed buffer must be 16-byte aligned", who);
-    REQUIRE(((uintptr_t)(to_fork ? dst : src) & 1u) == 0, TQ_ERR_ALIGN, "%s: the blocks must be 2-byte aligned (a block starts with an fp16 norm)", who);
+    // 4-bit blocks are 68 bytes (norm, rnorm, 16 code words): their rows are read and written as 4-byte words
+    const uintptr_t fork_align = h->bits == 4 ? 4u : 2u;
+    REQUIRE(((uintptr_t)(to_fork ? dst : src) & (fork_align - 1u)) == 0, TQ_ERR_ALIGN,
+            "%s: the blocks must be %d-byte aligned (a block starts with an fp16 norm%s)", who, (int)fork_align,
+            h->bits == 4 ? " and its 68-byte rows move as 4-byte words" : "");
     return tqk_fork_blocks(h, to_fork, src, n_seqs, tokens, kind, dst, (hipStream_t)stream);
 }
 
-int64_t tq_fork_block_bytes(int32_t bits) { return bits == 3 ? 50 : bits == 4 ? 66 : bits == 2 ? 34 : -1; }
+int64_t tq_fork_block_bytes(int32_t bits) { return bits == 3 ? 50 : bits == 4 ? 68 : bits == 2 ? 34 : -1; }
 
 int tq_export_fork_blocks(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *blocks,
                           void *stream) {
@@ -796,8 +804,10 @@ int tq_score_tile(const tq_handle *h, const void *q, int q_dtype, int64_t nq, co
     REQUIRE(out_dtype == TQ_F32 || out_dtype == TQ_F16, TQ_ERR_ARG, "tq_score_tile: logits must be fp32 or fp16");
     REQUIRE(workspace_bytes >= (nq + 31) / 32 * 32 * 256 * 2, TQ_ERR_ARG, "tq_score_tile: workspace %lld < %lld bytes",
             (long long)workspace_bytes, (long long)(nq * 256 * 2));
-    REQUIRE(aligned16(packed) && aligned16(workspace) && aligned16(logits), TQ_ERR_ALIGN,
-            "tq_score_tile: packed, workspace and logits must be 16-byte aligned");
+    REQUIRE(aligned16(packed) && aligned16(workspace), TQ_ERR_ALIGN, "tq_score_tile: packed and workspace must be 16-byte aligned");
+    // the logits leave as single-element buffer stores: a row slice of a larger matrix is fine
+    REQUIRE((reinterpret_cast<uintptr_t>(logits) & (out_dtype == TQ_F32 ? 3u : 1u)) == 0, TQ_ERR_ALIGN,
+            "tq_score_tile: logits must be aligned to their element type");
     if (nq == 0 || nk == 0) return TQ_OK;
     return tqk_score_tile(h, q, q_dtype, nq, packed, sign_bits, rnorms_f16, nk, logits, out_dtype, workspace,
                           workspace_bytes, (hipStream_t)stream);

@@ -79,10 +79,10 @@ int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_
 int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
               uint8_t *sign_bits, void *rnorms, hipStream_t s);
 int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
-               int kind, void *packed, hipStream_t s, const int64_t *pos_dev = nullptr);
+               int kind, void *packed, hipStream_t s, const int64_t *pos_dev = nullptr, uint32_t *overrun = nullptr);
 int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
                   int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s,
-                  const int64_t *pos_dev = nullptr);
+                  const int64_t *pos_dev = nullptr, uint32_t *overrun = nullptr);
 int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                    hipStream_t s);
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
@@ -97,7 +97,7 @@ int tqk_unpack_codes(const tq_handle *h, const void *packed, int64_t n_seqs, int
                      float *norms, hipStream_t s);
 int tqk_q8_0_store(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
 int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
-                    void *packed, hipStream_t s, const int64_t *pos_dev = nullptr);
+                    void *packed, hipStream_t s, const int64_t *pos_dev = nullptr, uint32_t *overrun = nullptr);
 int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, void *packed, hipStream_t s);
 int tqk_q8_0_unpack(const void *packed, int64_t n_seqs, int64_t tokens, int8_t *q, float *scales, int kind, hipStream_t s);
 

@@ -1372,14 +1372,24 @@ struct AppendArgs {
     int64_t pos, n_new, blocks_per_seq, first_block, n_touched;
     const int64_t *pos_dev;  // NULL, or where the position is read from when the launch runs (n_touched is then the
     int64_t capacity;        // largest number of blocks n_new tokens can touch, and some workgroups find nothing to do)
+    uint32_t *overrun;       // NULL, or a sticky word that a refused position sets (TQ_OVERRUN_* bits)
 };
+
+// A position read from device memory that is negative or leaves no room for n_new tokens (n_new <= capacity is
+// checked on the host, so the subtraction cannot wrap whatever the counter holds): nothing is written, and the
+// launch's first workgroup records why in the caller's word, if there is one.
+__device__ __forceinline__ bool append_position_ok(int64_t pos, int64_t n_new, int64_t capacity, uint32_t *overrun, bool reporter) {
+    const uint32_t why = pos < 0 ? (uint32_t)TQ_OVERRUN_NEGATIVE : pos > capacity - n_new ? (uint32_t)TQ_OVERRUN_NO_ROOM : 0u;
+    if (why && overrun && reporter && threadIdx.x == 0) atomicOr(overrun, why);
+    return why == 0u;
+}
 
 // Position from device memory (a captured launch replayed while the cache grows): fills in pos and first_block and
 // says whether workgroup `wg` has a block to rebuild.  Positions that do not fit the capacity write nothing.
 __device__ __forceinline__ bool resolve_append(AppendArgs &a, int64_t wg) {
     if (!a.pos_dev) return true;
     const int64_t pos = *a.pos_dev;
-    if (pos < 0 || pos + a.n_new > a.capacity) return false;
+    if (!append_position_ok(pos, a.n_new, a.capacity, a.overrun, wg == 0)) return false;
     a.pos = pos;
     a.first_block = pos / TQ_ROWS_PER_BLOCK;
     const int64_t touched = (pos + a.n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
@@ -2410,10 +2420,10 @@ __global__ __launch_bounds__(256) void k_q8_0_store_v_f16(const __half *x, uint8
 template <typename TI, int KIND>
 __global__ __launch_bounds__(256) void k_q8_0_append(const TI *x, uint8_t *packed, int64_t pos, int64_t n_new,
                                                      int64_t blocks_per_seq, int64_t first_block, int64_t n_touched,
-                                                     const int64_t *pos_dev, int64_t capacity) {
+                                                     const int64_t *pos_dev, int64_t capacity, uint32_t *overrun) {
     if (pos_dev) {  // the position is read when the launch runs (see resolve_append)
         pos = *pos_dev;
-        if (pos < 0 || pos + n_new > capacity) return;
+        if (!append_position_ok(pos, n_new, capacity, overrun, blockIdx.x == 0)) return;
         first_block = pos / TQ_ROWS_PER_BLOCK;
         if ((int64_t)(blockIdx.x % n_touched) >= (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - first_block + 1) return;
     }
@@ -2741,8 +2751,11 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
 
 // ---- interchange with the per-128 block layout of the llama.cpp fork --------------------------
 // One block per vector, token order: norm fp16 | qs | signs (3-bit: two low bits of every index
-// in qs, the third in signs; 4-bit: nibbles; 2-bit: qs only) - 50 / 66 / 34 bytes.
-__host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 66 : 34; }
+// in qs, the third in signs; 2-bit: qs only) - 50 / 34 bytes; 4-bit: norm fp16 | rnorm fp16 | qs[64] nibbles -
+// 68 bytes (4.25 bits per value).  rnorm is the residual-norm slot of the fork's earlier 3-bit + QJL turbo4,
+// which its 4-bit PolarQuant block keeps and does not use: written as 0, ignored when read.
+__host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 68 : 34; }
+__host__ __device__ constexpr int fork_codes_offset(int bits) { return bits == 4 ? 4 : 2; }
 
 // Sixteen lanes per row: lane li owns the codes of dims 8 li .. 8 li + 7, which are whole bytes of the fork's row in
 // every width (4-bit: four nibble bytes; 3-bit: two qs bytes and one signs byte; 2-bit: two qs bytes).
@@ -2768,8 +2781,8 @@ __global__ __launch_bounds__(256) void k_fork_export(const uint8_t *packed, uint
         uint8_t *row = out + (seq * tokens + tok) * FB;             // FB is even: the row is 2-byte aligned
         if (li == 0) *reinterpret_cast<uint16_t *>(row) = reinterpret_cast<const uint16_t *>(block_s + block_code_bytes(BITS))[t];
         if constexpr (BITS == 4) {
-            reinterpret_cast<uint16_t *>(row + 2)[2 * li] = (uint16_t)w;
-            reinterpret_cast<uint16_t *>(row + 2)[2 * li + 1] = (uint16_t)(w >> 16);
+            if (li == 1) *reinterpret_cast<uint16_t *>(row + 2) = 0;  // the unused rnorm slot
+            *reinterpret_cast<uint32_t *>(row + 4 + 4 * li) = w;       // 68-byte rows: the codes are 4-byte aligned
         } else if constexpr (BITS == 2) {
             reinterpret_cast<uint16_t *>(row + 2)[li] = (uint16_t)w;
         } else {
@@ -2806,8 +2819,7 @@ __global__ __launch_bounds__(256) void k_fork_import(const uint8_t *in, uint8_t 
             const uint8_t *row = in + (seq * tokens + tok) * FB;
             g = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(row)));
             if constexpr (BITS == 4) {
-                const uint32_t w = reinterpret_cast<const uint16_t *>(row + 2)[2 * li] |
-                                   ((uint32_t) reinterpret_cast<const uint16_t *>(row + 2)[2 * li + 1] << 16);
+                const uint32_t w = *reinterpret_cast<const uint32_t *>(row + 4 + 4 * li);
 #pragma unroll
                 for (int m = 0; m < 8; ++m) c[m] = (w >> (4 * m)) & 15u;
             } else {
@@ -2847,12 +2859,12 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
 }
 
 static AppendArgs make_append_args(const tq_handle *h, int64_t pos, const int64_t *pos_dev, int64_t n_new, int64_t capacity,
-                                   int kind) {
+                                   int kind, uint32_t *overrun = nullptr) {
     AppendArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
     a.kind = kind; a.norm_correction = h->norm_correction; a.zero_code = h->zero_code;
     a.pos = pos; a.n_new = n_new; a.blocks_per_seq = blocks_for(capacity);
-    a.pos_dev = pos_dev; a.capacity = capacity;
+    a.pos_dev = pos_dev; a.capacity = capacity; a.overrun = pos_dev ? overrun : nullptr;
     a.first_block = pos / TQ_ROWS_PER_BLOCK;
     a.n_touched = pos_dev ? (n_new + TQ_ROWS_PER_BLOCK - 2) / TQ_ROWS_PER_BLOCK + 1  // at the worst alignment
                           : (pos + n_new - 1) / TQ_ROWS_PER_BLOCK - a.first_block + 1;
@@ -2861,10 +2873,10 @@ static AppendArgs make_append_args(const tq_handle *h, int64_t pos, const int64_
 
 int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t pos,
                   int64_t n_new, int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s,
-                  const int64_t *pos_dev) {
+                  const int64_t *pos_dev, uint32_t *overrun) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
-    const AppendArgs ka = make_append_args(hk, pos, pos_dev, n_new, capacity, TQ_KIND_K);
-    const AppendArgs va = make_append_args(hv, pos, pos_dev, n_new, capacity, TQ_KIND_V);
+    const AppendArgs ka = make_append_args(hk, pos, pos_dev, n_new, capacity, TQ_KIND_K, overrun);
+    const AppendArgs va = make_append_args(hv, pos, pos_dev, n_new, capacity, TQ_KIND_V);  // the K half reports
     const unsigned grid = 2u * (unsigned)(n_seqs * ka.n_touched);
     const int kb = hk->bits, vb = hv->bits;
 #define TQ_APPEND_KV(KB, VB)                                                                                                   \
@@ -2877,17 +2889,17 @@ int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const
     else if (kb == 3 && vb == 2) { TQ_APPEND_KV(3, 2); }
     else if (kb == 4 && vb == 3) { TQ_APPEND_KV(4, 3); }
     else {  // other pairs: two launches
-        const int rc = tqk_append(hk, k, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_K, packed_k, s, pos_dev);
-        return rc ? rc : tqk_append(hv, v, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_V, packed_v, s, pos_dev);
+        const int rc = tqk_append(hk, k, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_K, packed_k, s, pos_dev, overrun);
+        return rc ? rc : tqk_append(hv, v, n_seqs, pos, n_new, capacity, in_dtype, TQ_KIND_V, packed_v, s, pos_dev, overrun);
     }
 #undef TQ_APPEND_KV
     return tq_check_launch("append_kv");
 }
 
 int tqk_append(const tq_handle *h, const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype,
-               int kind, void *packed, hipStream_t s, const int64_t *pos_dev) {
+               int kind, void *packed, hipStream_t s, const int64_t *pos_dev, uint32_t *overrun) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
-    const AppendArgs a = make_append_args(h, pos, pos_dev, n_new, capacity, kind);
+    const AppendArgs a = make_append_args(h, pos, pos_dev, n_new, capacity, kind, overrun);
     const unsigned grid = (unsigned)(n_seqs * a.n_touched);
 #define TQ_APPEND_BITS(B) \
     DISPATCH_T(in_dtype, TI, (k_append<B, TI><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, a)))
@@ -3070,7 +3082,7 @@ int tqk_q8_0_store_v(const void *x, int64_t n_seqs, int64_t tokens, int in_dtype
 }
 
 int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, int64_t capacity, int in_dtype, int kind,
-                    void *packed, hipStream_t s, const int64_t *pos_dev) {
+                    void *packed, hipStream_t s, const int64_t *pos_dev, uint32_t *overrun) {
     if (n_seqs == 0 || n_new == 0) return TQ_OK;
     const int64_t bps = blocks_for(capacity);
     const int64_t first = pos / TQ_ROWS_PER_BLOCK;
@@ -3079,10 +3091,10 @@ int tqk_q8_0_append(const void *x, int64_t n_seqs, int64_t pos, int64_t n_new, i
     const unsigned grid = (unsigned)(n_seqs * n_touched);
     if (kind == TQ_KIND_V) {
         DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_V><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
-                                                                                   bps, first, n_touched, pos_dev, capacity)));
+                                                                                   bps, first, n_touched, pos_dev, capacity, overrun)));
     } else {
         DISPATCH_T(in_dtype, TI, (k_q8_0_append<TI, TQ_KIND_K><<<grid, 256, 0, s>>>((const TI *)x, (uint8_t *)packed, pos, n_new,
-                                                                                   bps, first, n_touched, pos_dev, capacity)));
+                                                                                   bps, first, n_touched, pos_dev, capacity, overrun)));
     }
     return tq_check_launch("q8_0_append");
 }

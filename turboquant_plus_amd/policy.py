@@ -115,20 +115,21 @@ class LayerKV:
         return (tt.zeros(nbytes(self.k_codec), dtype=tt.uint8, device=dev),
                 tt.zeros(nbytes(self.v_codec), dtype=tt.uint8, device=dev))
 
-    def append(self, k, v, k_cache, v_cache, pos, capacity: int):
+    def append(self, k, v, k_cache, v_cache, pos, capacity: int, overrun=None):
         """The K and V tokens [n_seqs, n_new, 128] of a decode step at positions pos .. pos+n_new-1 (pos: an int, or an
-        int64 device tensor with one element read when the launches run)."""
+        int64 device tensor with one element read when the launches run; with such a position `overrun`, a zeroed int32
+        device tensor with one element, collects the OVERRUN_* bits of launches that refused the position)."""
         if self.k_codec is not None and self.v_codec is not None:
-            self.k_codec.append_kv(self.v_codec, k, v, k_cache, v_cache, pos, capacity)
+            self.k_codec.append_kv(self.v_codec, k, v, k_cache, v_cache, pos, capacity, overrun=overrun)
             return k_cache, v_cache
         if self.k_codec is None:
-            q8_0_append(k, k_cache, pos, capacity, kind="k")
+            q8_0_append(k, k_cache, pos, capacity, kind="k", overrun=overrun)
         else:
-            self.k_codec.append(k, k_cache, pos, capacity, kind="k")
+            self.k_codec.append(k, k_cache, pos, capacity, kind="k", overrun=overrun)
         if self.v_codec is None:
-            q8_0_append(v, v_cache, pos, capacity, kind="v")
+            q8_0_append(v, v_cache, pos, capacity, kind="v", overrun=overrun)
         else:
-            self.v_codec.append(v, v_cache, pos, capacity, kind="v")
+            self.v_codec.append(v, v_cache, pos, capacity, kind="v", overrun=overrun)
         return k_cache, v_cache
 
     def prefill(self, k, v, k_cache, v_cache, capacity: int):

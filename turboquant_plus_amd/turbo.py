@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import os
 
 import numpy as np
 
@@ -156,26 +157,30 @@ class TurboCodec:
                                     L.dtype_code(kd), L.ptr(pk), L.ptr(pv), L.stream_ptr()))
         return pk, pv
 
-    def append(self, x, packed, pos, capacity: int, kind: str = "k"):
+    def append(self, x, packed, pos, capacity: int, kind: str = "k", overrun=None):
         """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of
         `packed`, a buffer of packed_bytes(bits, n_seqs, capacity) bytes (tq_append).  pos: an int, or an int64
-        device tensor with one element that holds the position when the launch runs (tq_append_at)."""
+        device tensor with one element that holds the position when the launch runs (tq_append_at); with such a
+        position, `overrun` (a zeroed int32 device tensor with one element) collects OVERRUN_* bits when a launch
+        finds a position that it refuses, see overrun_bits()."""
         xd, n_seqs, n_new = self._as_seqs(x)
         need = packed_bytes(self.bits, n_seqs, capacity)
         if packed.numel() < need:
             raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
         if _position_on_device(pos):
             L.check(L.lib().tq_append_at(self.handle.h, L.ptr(xd), n_seqs, L.ptr(pos), n_new, capacity, L.dtype_code(xd),
-                                         L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+                                         L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), _overrun_ptr(overrun),
+                                         L.stream_ptr()))
             return packed
         L.check(L.lib().tq_append(self.handle.h, L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
                                   L.KIND_K if kind == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
         return packed
 
-    def append_kv(self, v_codec: "TurboCodec", k, v, packed_k, packed_v, pos, capacity: int):
+    def append_kv(self, v_codec: "TurboCodec", k, v, packed_k, packed_v, pos, capacity: int, overrun=None):
         """append() of the K tokens (this codec) and the V tokens (`v_codec`) of one decode step
         in one launch (tq_append_kv).  pos: an int, or an int64 device tensor with one element that holds the
-        position when the launch runs (tq_append_kv_at: a captured step replayed while the cache grows)."""
+        position when the launch runs (tq_append_kv_at: a captured step replayed while the cache grows; `overrun`
+        as in append())."""
         kd, n_seqs, n_new = self._as_seqs(k)
         vd, vs, vn = self._as_seqs(v)
         if (vs, vn) != (n_seqs, n_new) or vd.dtype != kd.dtype:
@@ -186,7 +191,8 @@ class TurboCodec:
                 raise ValueError(f"packed holds {buf.numel()} bytes, need {need}")
         if _position_on_device(pos):
             L.check(L.lib().tq_append_kv_at(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, L.ptr(pos), n_new,
-                                            capacity, L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
+                                            capacity, L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v),
+                                            _overrun_ptr(overrun), L.stream_ptr()))
             return packed_k, packed_v
         L.check(L.lib().tq_append_kv(self.handle.h, v_codec.handle.h, L.ptr(kd), L.ptr(vd), n_seqs, pos, n_new, capacity,
                                      L.dtype_code(kd), L.ptr(packed_k), L.ptr(packed_v), L.stream_ptr()))
@@ -205,7 +211,7 @@ class TurboCodec:
         return out
 
     def export_fork_blocks(self, packed, n_seqs: int, tokens: int, kind: str = "k"):
-        """-> uint8 [n_seqs, tokens, 50 | 66 | 34]: the llama.cpp fork's per-128 block layout."""
+        """-> uint8 [n_seqs, tokens, 50 | 68 | 34]: the llama.cpp fork's per-128 block layout."""
         tt = L.torch()
         fb = int(L.lib().tq_fork_block_bytes(self.bits))
         out = tt.empty((n_seqs, tokens, fb), dtype=tt.uint8, device=packed.device)
@@ -214,7 +220,7 @@ class TurboCodec:
         return out
 
     def import_fork_blocks(self, blocks, kind: str = "k"):
-        """Fork blocks [n_seqs, tokens, 50 | 66 | 34] -> packed buffer of this library."""
+        """Fork blocks [n_seqs, tokens, 50 | 68 | 34] -> packed buffer of this library."""
         tt = L.torch()
         dev = L.require_gpu()
         bd = blocks if isinstance(blocks, tt.Tensor) else tt.from_numpy(np.ascontiguousarray(blocks))
@@ -346,17 +352,37 @@ def _position_on_device(pos) -> bool:
     return True
 
 
-def q8_0_append(x, packed, pos, capacity: int, kind: str = "k"):
+OVERRUN_NEGATIVE, OVERRUN_NO_ROOM = 1, 2   # TQ_OVERRUN_* of include/tq.h
+
+
+def _overrun_ptr(overrun):
+    """NULL, or the address of the caller's sticky overrun word (int32 device tensor with one element)."""
+    if overrun is None:
+        return None
+    tt = L.torch()
+    if not isinstance(overrun, tt.Tensor) or overrun.dtype != tt.int32 or not overrun.is_cuda or overrun.numel() != 1:
+        raise ValueError("overrun must be an int32 device tensor with one element")
+    return L.ptr(overrun)
+
+
+def overrun_bits(overrun) -> int:
+    """Read the overrun word of the *_at appends (synchronises): 0, or OVERRUN_NEGATIVE | OVERRUN_NO_ROOM bits of
+    the launches that refused their position since the word was last cleared."""
+    return int(overrun.item())
+
+
+def q8_0_append(x, packed, pos, capacity: int, kind: str = "k", overrun=None):
     """Write the tokens x [n_seqs, n_new, 128] at positions pos .. pos+n_new-1 of a q8_0-style buffer laid
     out for `capacity` tokens per sequence (zero-initialised; tq_q8_0_append).  pos: an int, or an int64 device
-    tensor with one element read when the launch runs (tq_q8_0_append_at)."""
+    tensor with one element read when the launch runs (tq_q8_0_append_at; `overrun` as in TurboCodec.append)."""
     xd, n_seqs, n_new = TurboCodec._as_seqs(x)
     need = int(L.lib().tq_q8_0_bytes(n_seqs, capacity))
     if packed.numel() < need:
         raise ValueError(f"packed holds {packed.numel()} bytes, need {need}")
     if _position_on_device(pos):
         L.check(L.lib().tq_q8_0_append_at(L.ptr(xd), n_seqs, L.ptr(pos), n_new, capacity, L.dtype_code(xd),
-                                          L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
+                                          L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed),
+                                          _overrun_ptr(overrun), L.stream_ptr()))
         return packed
     L.check(L.lib().tq_q8_0_append(L.ptr(xd), n_seqs, pos, n_new, capacity, L.dtype_code(xd),
                                    L.KIND_K if _kind_name(kind) == "k" else L.KIND_V, L.ptr(packed), L.stream_ptr()))
@@ -388,10 +414,14 @@ class DecodeAttention:
 
     def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec | None, batch: int, n_q_heads: int, n_kv_heads: int,
                  tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0,
-                 capacity: int = 0, tokens_on_device=None):
+                 capacity: int = 0, tokens_on_device=None, poison_output: bool | None = None):
         """tokens_on_device: an int64 device tensor (one element) that holds the context length when a call runs;
         `tokens` is then the largest length it may take.  One captured launch (HIP graph) can so be replayed while
-        the cache grows; Sparse V is not available in this mode."""
+        the cache grows; Sparse V is not available in this mode.
+        poison_output (default: on when the environment holds TQ_POISON_OUTPUT=1): fill the output rows with NaN
+        before every call, so that a row the launch did not write - the split partials are merged inside the launch by
+        whichever workgroup of a group finishes last - shows as NaN instead of the previous call's values.  A debug
+        aid: one small fill kernel per call."""
         tt = L.torch()
         dev = L.require_gpu()
         self.k_codec, self.v_codec = k_codec, v_codec
@@ -415,10 +445,13 @@ class DecodeAttention:
         self.workspace = tt.empty(int(nbytes), dtype=tt.uint8, device=dev)
         self.skip = tt.zeros(2, dtype=tt.int64, device=dev)
         self.out = tt.empty((batch, n_q_heads, HEAD_DIM), dtype=tt.float32, device=dev)
+        self.poison_output = os.environ.get("TQ_POISON_OUTPUT", "0") == "1" if poison_output is None else bool(poison_output)
 
     def __call__(self, q, k_packed, v_packed, bias=None):
         """q [batch, n_q_heads, 128] in the original domain -> out fp32 [batch, n_q_heads, 128]."""
         qd = L.to_device(q)
+        if self.poison_output:
+            self.out.fill_(float("nan"))
         hk = self.k_codec.handle.h if self.k_codec is not None else None
         hv = self.v_codec.handle.h if self.v_codec is not None else None
         L.check(L.lib().tq_decode_attention(hk, hv, C.byref(self.params), L.ptr(qd),
