@@ -230,6 +230,12 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                     else if (b == 3) fl[c * 4 + v / 8] |= 1u << (3 * (v % 8) + 2);  // entry 3: the tail word
                 }
             rc = rc ? rc : upload(&h->s2flip, fl);
+            for (int i = 0; i < 16; ++i) h->s2flip_host[i] = fl[i];
+            for (int w = 0; w < 4; ++w) h->s1neg_host[w] = h->s2neg_host[w] = 0u;
+            for (int k = 0; k < 128; ++k) {
+                if (s1[k] < 0) h->s1neg_host[k >> 5] |= 1u << (k & 31);
+                if (s2[k] < 0) h->s2neg_host[k >> 5] |= 1u << (k & 31);
+            }
         }
         // sign-symmetric boundaries (in fp32) allow the thermometer quantiser
         const int nb = nc - 1, mid = nb / 2;
@@ -243,6 +249,7 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         st[0] = b32[mid];
         for (int j = 1; j <= mid; ++j) st[j] = b32[mid + j];
         rc = rc ? rc : upload(&h->symthr32, st);
+        for (int j = 0; j < 8; ++j) h->symthr_host[j] = j <= mid ? st[j] : 0.0f;
         // magnitude level by table: a bin of the value's top 12 bits holds at most one boundary, so
         // level = (boundaries below the bin) + (|value| > the bin's boundary)
         {
@@ -285,6 +292,7 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
                     if (m & bit) f[m] -= f[m ^ bit];
             std::vector<float> cf(f.begin(), f.end());
             rc = rc ? rc : upload(&h->sqcoef32, cf);
+            for (int j = 0; j < 8; ++j) h->sqcoef_host[j] = j < nl ? cf[j] : 0.0f;
         }
         if (cfg->projection) {
             // M = S R^T with R[k][m] = s2[k] H[k][m] s1[m] / sqrt(128); stored as [k*128+j] = M[j][k]

@@ -47,6 +47,11 @@ struct tq_handle {
                            // .y = fp32 bits of the one boundary inside the bin (+inf when there is none)
     int quant_lut_ok;      // every bin holds at most one boundary (else the table cannot decide a level)
     uint64_t quant_lut_hash;  // hash of the table's contents
+    // host copies of the small constants, passed to the fused K+V store by value (kernel arguments), so that its
+    // wavefronts need nothing from memory before their first input
+    uint32_t s1neg_host[4], s2neg_host[4];  // bit k of word k / 32: s1[k] < 0, s2[k] < 0
+    uint32_t s2flip_host[16];               // host copy of s2flip
+    float symthr_host[8], sqcoef_host[8];   // host copies of symthr32, sqcoef32 (2^(bits-1) entries used)
     int zero_code;         // codebook index of the value 0.0 (#boundaries below 0)
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };

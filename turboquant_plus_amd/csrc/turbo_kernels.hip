@@ -446,6 +446,39 @@ template <int BITS> __device__ __forceinline__ uint32_t fold_codes(uint32_t w) {
     }
 }
 
+#ifndef TQ_EXP
+#define TQ_EXP 0
+#endif
+#define TQ_EXP_PRIO (TQ_EXP & 3)
+// Measurement builds only (-DTQ_TIMELINE): per-wavefront timestamps (100 MHz wall clock) of the fused K+V store
+#ifdef TQ_TIMELINE
+__device__ unsigned long long g_tl[4096 * 16];
+#define TQ_TL(slot)                                                                                              \
+    do {                                                                                                         \
+        const unsigned tlw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);                                \
+        if ((threadIdx.x & 63) == 0 && tlw < 4096) g_tl[tlw * 16 + (slot)] = wall_clock64();                      \
+    } while (0)
+#define TQ_TL_VAL(slot, v)                                                                                       \
+    do {                                                                                                         \
+        const unsigned tlw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);                                \
+        if ((threadIdx.x & 63) == 0 && tlw < 4096) g_tl[tlw * 16 + (slot)] = (v);                                 \
+    } while (0)
+#else
+#define TQ_TL(slot) do {} while (0)
+#define TQ_TL_VAL(slot, v) do {} while (0)
+#endif
+
+// The compiler pads the distance between a matrix instruction and the first vector instruction that reads its result
+// with s_nop, but only along straight-line code: where a branch follows the matrix instructions, the path that takes the
+// branch arrives at the reader with no padding (observed: a wavefront that skipped a conditional block read the first
+// element of a 16x16x32 result too early).  Conditional blocks behind matrix instructions are therefore preceded by this
+// pause, pinned in place: 16 wait states, the longest such distance on this part.
+__device__ __forceinline__ void settle_matrix_results() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 7\n\ts_nop 7");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 struct StoreKArgs {
     const uint4 *afrag;      // [8 fragments f0*4+ks][64 lanes] 8 halves (+-1)
     const uint32_t *s2flip;  // [4 lane quarters][4]: sign-field positions of the dims with s2 = +1, per output dword
@@ -458,7 +491,50 @@ struct StoreKArgs {
     uint32_t blocks_per_seq, n_units;  // unit = 16 tokens
     FastDiv bps_div;                   // division by blocks_per_seq
     uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
+    // the same constants by value (REG kernels: nothing is fetched before the first input): bit k of s1neg = s1[k] < 0
+    uint32_t s1neg[4], flipw[16];
+    float thr[8], coef[8];
 };
+
+// ---- the +-1 operand fragments built in registers -------------------------------------------------
+// bit e of row hm of the 8 x 8 Hadamard sign pattern: parity(hm & e)
+__device__ __forceinline__ uint32_t h8_row(uint32_t hm) {
+    const uint64_t rows = 0x963C5AF066CCAA00ull;  // rows 0..7, one byte each
+    return (uint32_t)(rows >> (8u * hm)) & 0xFFu;
+}
+// eight sign bits (1 = negative) -> eight halves +-1.0
+__device__ __forceinline__ half8_t signs_to_half8(uint32_t bits) {
+    uint4 v;
+    v.x = 0x3C003C00u | ((bits << 15) & 0x8000u) | ((bits << 30) & 0x80000000u);
+    v.y = 0x3C003C00u | ((bits << 13) & 0x8000u) | ((bits << 28) & 0x80000000u);
+    v.z = 0x3C003C00u | ((bits << 11) & 0x8000u) | ((bits << 26) & 0x80000000u);
+    v.w = 0x3C003C00u | ((bits << 9) & 0x8000u) | ((bits << 24) & 0x80000000u);
+    return __builtin_bit_cast(half8_t, v);
+}
+// K rows (tq_handle::rfrag16k): fragment f0*4+ks, lane l, element e = s1[k] H[m][k], m = 32(l%16/4) + 4 f0 + l%4,
+// k = 32(l/16) + 8 ks + e.  m and k share the bits of e with 4 f0 + l%4 and the bits of l/16 with l%16/4.
+__device__ __forceinline__ void build_k_fragments(half8_t (&af)[8], const uint32_t (&s1neg)[4], int lane) {
+    const uint32_t r = lane & 15, kb = lane >> 4;
+    const uint32_t hi = (uint32_t)__builtin_popcount((r >> 2) & kb) & 1u ? 0xFFu : 0u;
+    const uint32_t w = kb == 0 ? s1neg[0] : kb == 1 ? s1neg[1] : kb == 2 ? s1neg[2] : s1neg[3];
+#pragma unroll
+    for (int f0 = 0; f0 < 2; ++f0) {
+        const uint32_t pat = h8_row(4u * f0 + (r & 3u)) ^ hi;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) af[f0 * 4 + ks] = signs_to_half8((pat ^ (w >> (8 * ks))) & 0xFFu);
+    }
+}
+// V rows (tq_handle::rfrag16v): fragment d0*4+ks, lane l, element e = s1[k] H[16 d0 + l%16][k], k = 32 ks + 8(l/16) + e
+__device__ __forceinline__ void build_v_fragments(half8_t (&bf)[8], const uint32_t (&s1neg)[4], int lane) {
+    const uint32_t n = lane & 15, kb = lane >> 4;
+    const uint32_t base = h8_row(n & 7u) ^ ((n >> 3) & kb & 1u ? 0xFFu : 0u);
+#pragma unroll
+    for (int d0 = 0; d0 < 2; ++d0) {
+        const uint32_t pat = base ^ (d0 && (kb >> 1) ? 0xFFu : 0u);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) bf[d0 * 4 + ks] = signs_to_half8((pat ^ (s1neg[ks] >> (8u * kb))) & 0xFFu);
+    }
+}
 
 // copy a handle's quantiser table (4096 x 8 B) into LDS with NT threads; every load is issued before the
 // first LDS write
@@ -518,7 +594,8 @@ constexpr int K_UNITS_AHEAD = 1;
 // first_ticket: the wavefront's first two tickets are first_ticket and first_ticket + 1 (the counter starts past
 // them), or DRAW_TICKET to draw them.  `stage` makes the workgroup's LDS copy of the constant operands (frag,
 // flips) readable; it runs after the first inputs have been requested.
-template <int BITS, bool RAGGED, bool DUP_LUT, typename Stage>
+// REG: the constants come from the argument block (fragments built in registers, frag and flips unused).
+template <int BITS, bool RAGGED, bool DUP_LUT, bool REG, typename Stage>
 __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const uint32_t *flips, uint32_t first_ticket, Stage &&stage) {
@@ -528,8 +605,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     float thr0[NT], coef[NT];
 #pragma unroll
     for (int k = 0; k < NT; ++k) {
-        thr0[k] = a.symthr[k];
-        coef[k] = a.sqcoef[k];
+        thr0[k] = REG ? a.thr[k] : a.symthr[k];
+        coef[k] = REG ? a.coef[k] : a.sqcoef[k];
     }
 
     const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
@@ -578,12 +655,44 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     }
     stage();
     half8_t af[8];
-#pragma unroll
-    for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
     uint32_t flip[4];
+    if constexpr (REG) {
+        build_k_fragments(af, a.s1neg, lane);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) flip[j] = flips[kc * 4 + j];
+        for (int j = 0; j < 4; ++j) flip[j] = kc == 0 ? a.flipw[j] : kc == 1 ? a.flipw[4 + j] : kc == 2 ? a.flipw[8 + j] : a.flipw[12 + j];
+    } else {
+#pragma unroll
+        for (int f = 0; f < 8; ++f) af[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) flip[j] = flips[kc * 4 + j];
+    }
 
+    [[maybe_unused]] unsigned tl_n = 0;
+    // The codes and the norm of a unit leave one unit later, right after the next unit's matrix instructions have been
+    // issued: loads and stores share one counter of outstanding operations, so a wait for input also waits for all
+    // but a few of the stores issued after that input was requested - stores issued at the end of a unit were waited
+    // for, with their full latency, at the top of the next one.
+    static_assert(DEPTH == 1, "the deferred stores assume one unit in flight");
+    uint32_t pend_g[BITS];
+    float pend_gn = 0.0f;
+    uint32_t pend_unit = 0;
+    bool pending = false;
+#pragma unroll
+    for (int j = 0; j < BITS; ++j) pend_g[j] = 0;
+    auto flush = [&] {
+        const uint32_t blk = pend_unit >> 3;
+        const int row = (int)(pend_unit & 7) * 16 + n16;
+        const uint32_t oseq = RAGGED ? a.bps_div.div(blk) : 0u;
+        const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + (blk - oseq * bps) : blk;
+        uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
+#if TQ_KNOCKOUT & 16
+        if (pend_g[0] == 0x12345678u && pend_g[BITS - 1] == 0x9abcdef0u)   // keeps the codes alive; not taken for real data
+#endif
+#pragma unroll
+        for (int j = 0; j < BITS; ++j)
+            stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kc * 4), pend_g[j]);
+        if (kc == 0) reinterpret_cast<__half *>(block + block_code_bytes(BITS))[row] = __float2half_rn(pend_gn);
+    };
 #pragma unroll 1
     for (bool more = true; more;) {
 #pragma unroll
@@ -593,6 +702,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
                 more = false;
                 break;
             }
+            if (tl_n == 1) TQ_TL(4);
+            ++tl_n;
             const uint32_t next = lo + step * take_ticket(counter, lane);
             uint4 (&xb)[4] = xq[r];
             if constexpr (RAGGED) {
@@ -623,6 +734,8 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
             ss = diag_here ? ss : 0.0f;
             cur[r] = next;
+            settle_matrix_results();
+            if (pending) flush();  // the previous unit's codes, behind this unit's wait for its input
             fetch(next, xb, xvalid[r]);
             ss += xor_lane<16>(ss);
             ss += xor_lane<32>(ss);
@@ -726,17 +839,6 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
                     g[j] = fold_codes<2>(nonzero ? w ^ flip[j] : (zero_word & 0xAAAAAAAAu));
                 }
             }
-            const uint32_t blk = unit >> 3;
-            const int row = (int)(unit & 7) * 16 + n16;
-            const uint32_t oseq = RAGGED ? a.bps_div.div(blk) : 0u;
-            const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + (blk - oseq * bps) : blk;
-            uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
-#if TQ_KNOCKOUT & 16
-            if (g[0] == 0x12345678u && g[BITS - 1] == 0x9abcdef0u)   // keeps the codes alive; not taken for real data
-#endif
-#pragma unroll
-            for (int j = 0; j < BITS; ++j) stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint32_t *>(block + j * 2048 + row * 16 + kc * 4), g[j]);
-
             float gn = norm;
             if (a.norm_correction) {
                 float cs = 32.0f * coef[0];
@@ -746,9 +848,20 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
                 cs += xor_lane<32>(cs);
                 gn = norm * __builtin_amdgcn_rsqf(cs);  // cs >= 128 min c^2 > 0
             }
-            if (kc == 0) reinterpret_cast<__half *>(block + block_code_bytes(BITS))[row] = __float2half_rn(gn);
+#pragma unroll
+            for (int j = 0; j < BITS; ++j) pend_g[j] = g[j];
+            pend_gn = gn;
+            pend_unit = unit;
+            pending = true;
+#if TQ_EXP & 64
+            flush();
+            pending = false;
+#endif
         }
     }
+    if (pending) flush();
+    TQ_TL(5);
+    TQ_TL_VAL(7, (unsigned long long)tl_n);
 }
 
 // ---- K2, fp16 input, V rows ---------------------------------------------------------------
@@ -900,6 +1013,8 @@ struct StoreVArgs {
     uint32_t blocks_per_seq, n_units;  // unit = 64-token tile (half a block)
     FastDiv bps_div;                   // division by blocks_per_seq
     uint32_t out_blocks_per_seq;       // blocks between two sequences in `packed` (RAGGED kernels; a cache laid out for more tokens)
+    uint32_t s1neg[4], s2neg[4];       // the constants by value (REG kernels): bit k = s1[k] < 0, s2[k] < 0
+    float thr[8], coef[8];
 };
 
 // Tiles lo, lo + step, .. below end through a ticket counter in LDS, as for the K units.  The first
@@ -908,10 +1023,15 @@ struct StoreVArgs {
 // constant operands (frag, s2: LDS) readable.
 // STREAM_IN: the input is read with the non-temporal hint (every 128-byte line is touched by two instructions of one
 // wavefront, back to back).  It gains 2 us in the fused K+V launch and loses 1 us in the V-only kernel (measured).
-template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, typename Stage>
+// REG: the constants come from the argument block (fragments built in registers, frag and s2 unused), the first tile is
+// requested before anything else and `stage` runs while it is in flight.
+// VDMA = 2: sub-tiles 1 and 0 of a tile travel through this wavefront's two 4 KB slots in LDS (`slots`; loads that write
+// LDS directly), requested together with the register loads of sub-tiles 3 and 2, so a whole tile (16 KB) is in flight
+// per wavefront instead of half of one, at no cost in registers.
+template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, bool REG, int VDMA = 0, typename Stage>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
-                                              const float *s2, uint32_t first_ticket, Stage &&stage) {
+                                              const float *s2, uint32_t first_ticket, Stage &&stage, uint4 *slots = nullptr) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
     const int tid = threadIdx.x, lane = tid & 63;
@@ -919,8 +1039,8 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     float thr0[NT], coef[NT];
 #pragma unroll
     for (int k = 0; k < NT; ++k) {
-        thr0[k] = a.symthr[k];
-        coef[k] = a.sqcoef[k];
+        thr0[k] = REG ? a.thr[k] : a.symthr[k];
+        coef[k] = REG ? a.coef[k] : a.sqcoef[k];
     }
     // an exact zero counts as positive only if the middle boundary is below zero
     const uint32_t zero_word = thr0[0] < 0.0f ? 0xFFFFFFFFu : 0u;
@@ -929,7 +1049,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // A operand of sub-tile u: row r = lane%16 is token 16(r/4) + 4u + r%4 of the tile, this lane
     // supplies inputs 32ks + 8kq .. +7.  The address is always valid (clamped); `valid` says
     // whether the row exists.
-    auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
+    auto row_ptr = [&](uint32_t unit, int u, bool &valid) -> const uint4 * {
         const bool beyond = unit > last_unit;  // past the share: every lane reads the tensor's first bytes (see the K units)
         unit = unit < last_unit ? unit : last_unit;
 #if TQ_KNOCKOUT & 32
@@ -937,19 +1057,38 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #endif
         const uint32_t blk = unit >> 1;
         const int tb = (int)(unit & 1) * 64 + 16 * (n16 >> 2) + 4 * u + (n16 & 3);
-        const uint4 *p;
         if constexpr (RAGGED) {
             const uint32_t seq = a.bps_div.div(blk), bis = blk - seq * bps;
             int64_t tok = (int64_t)bis * TQ_ROWS_PER_BLOCK + tb;
             valid = tok < a.tokens;
             tok = valid ? tok : a.tokens - 1;
-            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)seq * a.tokens + tok) * 128 + 8 * kq));
+            return reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)seq * a.tokens + tok) * 128 + 8 * kq));
         } else {
             valid = true;
-            p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq));
+            return reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq));
         }
+    };
+    auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
+        const uint4 *p = row_ptr(unit, u, valid);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
+    };
+    // the same sub-tile into LDS slot `sl` of this wavefront: instruction ks writes the lanes' 16-byte pieces to
+    // slots[(4 sl + ks) 64 + lane], which is where the lane reads its operand back
+    auto fetch_lds = [&](uint32_t unit, int u, int sl) {
+        bool valid;
+        const uint4 *p = row_ptr(unit, u, valid);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p + 4 * ks),
+                                             (__attribute__((address_space(3))) void *)(slots + (4 * sl + ks) * 64), 16, 0,
+                                             STREAM_IN ? 2 : 0);
+    };
+    auto read_lds = [&](uint32_t unit, int u, int sl, uint4 (&xb)[4], bool &valid) {
+        if constexpr (RAGGED) (void)row_ptr(unit, u, valid);
+        else valid = true;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) xb[ks] = slots[(4 * sl + ks) * 64 + lane];
     };
 
     uint4 xq[2][4];
@@ -959,21 +1098,92 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // chip ask for their first input at once, ahead of the constants, the burst takes several microseconds to serve and
     // the constants queue behind it (measured: no wavefront asking early 32.3 us, one per SIMD 32.9 us, two 33.1 us,
     // all 33.0 us for the 3-bit K+V launch; 4-bit alike within its run-to-run spread).
-    stage();
-    fetch(unit, 3, xq[0], xvalid[0]);
-    fetch(unit, 2, xq[1], xvalid[1]);
     half8_t bf[8];
-#pragma unroll
-    for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
     bool s2pos[4][2];
+    if constexpr (REG) {
+        // nothing has to come from memory before the first input: the constants are kernel arguments.  Only the
+        // first sub-tile is requested ahead of the barrier: with both in flight at once the chip-wide burst is twice
+        // as long and every wavefront's first data arrives later (measured: 33.2 against 32.2 us for the 3-bit launch)
+        fetch(unit, 3, xq[0], xvalid[0]);
+        TQ_TL(8);
+        build_v_fragments(bf, a.s1neg, lane);
 #pragma unroll
-    for (int dd = 0; dd < 4; ++dd)
+        for (int dd = 0; dd < 4; ++dd)
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = s2[64 * hf + 16 * dd + n16] > 0.0f;
+            for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = ((a.s2neg[2 * hf + (dd >> 1)] >> (16 * (dd & 1) + n16)) & 1u) == 0u;
+        TQ_TL(9);
+        stage();
+        TQ_TL(10);
+        if constexpr (VDMA == 2) {  // older than the load of sub-tile 2: when that one has arrived, so have these
+            fetch_lds(unit, 1, 0);
+            fetch_lds(unit, 0, 1);
+        }
+        fetch(unit, 2, xq[1], xvalid[1]);
+    } else {
+        stage();
+        fetch(unit, 3, xq[0], xvalid[0]);
+        fetch(unit, 2, xq[1], xvalid[1]);
+#pragma unroll
+        for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd)
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) s2pos[dd][hf] = s2[64 * hf + 16 * dd + n16] > 0.0f;
+    }
 
+    [[maybe_unused]] unsigned tl_n = 0;
+    TQ_TL(1);
+    // DEFER: codes and norms leave one sub-tile after they are complete, right behind the next sub-tile's matrix
+    // instructions (loads and stores share one counter of outstanding operations, so a wait for input also waits for all
+    // but a few of the stores issued after that input was requested; stores issued at the end of a sub-tile were waited
+    // for, with their full latency, at the top of the next one).  A sub-tile completes one dword of each of the lane's
+    // four rows (2-bit codes: every second sub-tile), which is finished - signs, zero tokens, fold - and parked in `park`;
+    // the last one of a tile crosses into the next tile (pend_unit) or is flushed after the loop.
+    constexpr bool DEFER = REG && !(TQ_EXP & 32);
+    uint32_t park[4] = {0, 0, 0, 0};
+    float park_norm = 0.0f;
+    uint32_t pend_unit = 0;
+    bool pending = false;
+    auto block_of = [&](uint32_t un) -> uint8_t * {
+        const uint32_t oseq = RAGGED ? a.bps_div.div(un >> 1) : 0u;
+        const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + ((un >> 1) - oseq * bps) : un >> 1;
+        return packed + (int64_t)oblk * block_bytes(BITS);
+    };
+    // the parked dword j of the four rows and the parked norms of sub-tile u, tile `un`
+    auto flush_park = [&](uint32_t un, int j, int u, bool with_codes) {
+        uint8_t *blockp = block_of(un);
+        const int hlf = (int)(un & 1);
+        if (with_codes) {
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                const int row = hlf * 64 + 16 * dd + n16;
+#if TQ_KNOCKOUT & 16
+                if (park[dd] == 0x12345678u)   // keeps the codes alive; practically never taken
+#endif
+                stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint32_t *>(blockp + j * 2048 + row * 16 + kq * 4), park[dd]);
+            }
+        }
+        __half *no = reinterpret_cast<__half *>(blockp + block_code_bytes(BITS)) + hlf * 64 + 16 * kq;
+        if (n16 < 4) no[4 * u + n16] = __float2half_rn(park_norm);
+    };
+    // does sub-tile u complete its dword?  (2-bit codes: two sub-tiles share a dword)
+    auto completes = [](int u) { return u == 0 || grp_word(BITS, 4 * (u - 1)) != grp_word(BITS, 4 * u); };
+    // the dword that sub-tile u's completed word makes storable (-1: none; 3-bit: the tail word only rides on the others)
+    auto storable = [&](int u) { const int j = grp_word(BITS, 4 * u); return !completes(u) || (BITS == 3 && j == 3) ? -1 : j; };
 #pragma unroll 1
     for (; unit < end;) {
-        const uint32_t next = lo + step * take_ticket(counter, lane);
+        if (tl_n == 1) TQ_TL(2);
+        ++tl_n;
+        // (with sub-tiles in LDS the ticket is drawn after the slots have been read: the compiler makes every LDS
+        // operation wait for all loads that write LDS, and at this point the whole tile is still in flight)
+        uint32_t next = 0;
+        if constexpr (VDMA == 0) next = lo + step * take_ticket(counter, lane);
+        if constexpr (REG) {
+            // A wavefront that takes another tile while its neighbours move on to the small K units must not be the one
+            // its SIMD serves last (the arbiter favours the oldest wavefront slots): it would carry a 64-token chunk to the
+            // end of the launch.  Later tiles run at raised issue priority, the K units at the default.
+            if (TQ_EXP_PRIO && ((TQ_EXP & 8) || unit != lo + step * first_ticket)) __builtin_amdgcn_s_setprio(TQ_EXP_PRIO);
+        }
         const uint32_t oseq = RAGGED ? a.bps_div.div(unit >> 1) : 0u;
         const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + ((unit >> 1) - oseq * bps) : unit >> 1;
         uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
@@ -1013,8 +1223,47 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
                                                               gram, 0, 0, 0);
 #endif
-            if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-            else fetch(next, 5 - q, xb, xvalid[q & 1]);
+            // (before this sub-tile's requests: the wait for a sub-tile's input lets only a few younger operations stay
+            // outstanding, and these stores are then a whole sub-tile old when the next wait comes)
+            if constexpr (DEFER) {
+                if (q == 0) {
+                    settle_matrix_results();
+                    if (pending) flush_park(pend_unit, 0, 0, true);  // the previous tile's last dword and norms
+                } else {
+                    flush_park(unit, storable(u + 1) < 0 ? 0 : storable(u + 1), u + 1, storable(u + 1) >= 0);
+                }
+            }
+            if constexpr (VDMA == 2) {
+                // vector memory operations complete in issue order, and the slots' loads were issued before the register
+                // load of sub-tile 2, whose data the matrix instructions of q = 1 have just used.  The slot address is
+                // tied to their result so that the reads cannot move up past them.
+                if (q == 1) {
+                    uint32_t dep = 0;
+                    asm volatile("" : "+v"(dep) : "v"(gram[0]));
+                    uint4 *keep = slots;
+                    slots += dep;
+                    read_lds(unit, 1, 0, xq[0], xvalid[0]);
+                    read_lds(unit, 0, 1, xq[1], xvalid[1]);
+                    slots = keep;
+                    next = lo + step * take_ticket(counter, lane);
+                } else if (q == 2) {
+                    // both slots have been read (their data feeds this sub-tile's and the next one's matrix instructions;
+                    // the wait below is for the second read): the next tile's sub-tiles 1 and 0 may land in them
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    fetch_lds(next, 1, 0);
+                    fetch_lds(next, 0, 1);
+                    fetch(next, 3, xb, xvalid[0]);
+                } else if (q == 3) {
+                    fetch(next, 2, xb, xvalid[1]);
+                }
+            } else {
+                if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
+                else fetch(next, 5 - q, xb, xvalid[q & 1]);
+            }
+#ifdef TQ_TIMELINE
+            if (q == 0 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(11);   // the first sub-tile's input has arrived
+            if (q == 1 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(12);
+#endif
 
             float nrm[4];
             float4_t inv;
@@ -1137,7 +1386,39 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             const int isel = n16 & 3;
             const float nsel = isel == 0 ? nrm[0] : isel == 1 ? nrm[1] : isel == 2 ? nrm[2] : nrm[3];
             const float gn = a.norm_correction ? nsel * __builtin_amdgcn_rsqf(cs) : nsel;
-            if (n16 < 4) norms_out[4 * u + n16] = __float2half_rn(gn);
+            if constexpr (DEFER) {
+                park_norm = gn;
+                if (completes(u)) {
+                    // finish the dword this sub-tile completed: appended sign bit = "negative before s2", the xor makes it
+                    // "positive after s2"; all-zero tokens (rare) get the sign field of an exact zero; then the fold
+                    const int j = grp_word(BITS, 4 * u);
+                    uint32_t zm = 0;
+                    if (__builtin_amdgcn_ballot_w64(zbits != 0) != 0) {
+#pragma unroll
+                        for (int t = 0; t < 16; ++t)
+                            zm |= (zbits >> t) & 1 ? (v_sign_mask(BITS, j, 0, 1u << t) | v_sign_mask(BITS, j, 1, 1u << t)) : 0u;
+                    }
+#pragma unroll
+                    for (int dd = 0; dd < 4; ++dd) {
+                        const uint32_t fm = (s2pos[dd][0] ? v_sign_mask(BITS, j, 0, 0xFFFFu) : 0u) | (s2pos[dd][1] ? v_sign_mask(BITS, j, 1, 0xFFFFu) : 0u);
+                        uint32_t ww = w[dd][j] ^ fm;
+                        ww = (ww & ~zm) | (zero_word & zm);
+                        w[dd][j] = fold_codes<BITS>(ww);
+                        if (storable(u) >= 0) {
+                            park[dd] = w[dd][j];
+                            if constexpr (BITS == 3) park[dd] = __builtin_amdgcn_perm(w[dd][3], w[dd][j], 0x04020100u + ((uint32_t)j << 24));
+                        }
+                    }
+                }
+            } else {
+                if (n16 < 4) norms_out[4 * u + n16] = __float2half_rn(gn);
+            }
+        }
+        if constexpr (DEFER) {
+            pend_unit = unit;
+            pending = true;
+            unit = next;
+            continue;
         }
 
         // sign fields: appended bit = "negative before s2"; xor makes it "positive after s2".  All-zero tokens
@@ -1174,6 +1455,12 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
         }
         unit = next;
     }
+    if constexpr (DEFER) {
+        if (pending) flush_park(pend_unit, 0, 0, true);
+    }
+    if constexpr (REG) __builtin_amdgcn_s_setprio(0);
+    TQ_TL(3);
+    TQ_TL_VAL(6, (unsigned long long)tl_n);
 }
 
 __device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g) { return (uint32_t)((uint64_t)n * b / g); }
@@ -1203,10 +1490,10 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
             if (t < 16) flip_s[t] = c3;
             __syncthreads();
         };
-        store_k_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s,
+        store_k_units<BITS, RAGGED, false, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s,
                                     flip_s, 0u, stage);
     } else {
-        store_k_units<BITS, RAGGED, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, a.afrag,
+        store_k_units<BITS, RAGGED, false, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, a.afrag,
                                     a.s2flip, 0u, [] {});
     }
 }
@@ -1228,7 +1515,7 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
         if (t < 128) s2_s[t] = c2;
         __syncthreads();
     };
-    store_v_units<BITS, RAGGED, false, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
+    store_v_units<BITS, RAGGED, false, false, false>(x, packed, a, blockIdx.x * 4 + wave, gridDim.x * 4, a.n_units, &counter[wave], qlut, frag_s, s2_s, 0u,
                                 stage);
 }
 
@@ -1236,38 +1523,46 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
 // contiguous share of both tensors: every wavefront takes V tiles until the workgroup's share
 // is gone, then K units; the fine-grained K units level what the coarse V tiles leave uneven,
 // and the launch and pipeline-fill time is paid once.
+// The leading scalar parameters are the ones a wavefront needs for its first request (they are candidates for the
+// hardware's preloading of kernel arguments into scalar registers, where the toolchain enables it); the two
+// argument blocks follow and are read in one batch while that request is in flight: left to the compiler, their cache
+// lines were fetched one after the other where first needed, up to three dependent misses of about a microsecond each
+// before a wavefront's first input request.
 template <int KB, int VB, bool RAGGED>
-__global__ __launch_bounds__(768) void k_store_kv(const __half *xk, uint8_t *pk, StoreKArgs ka, const __half *xv, uint8_t *pv,
-                                                  StoreVArgs va) {
+__global__ __launch_bounds__(768) void k_store_kv(const __half *xv, const __half *xk, uint32_t v_units, uint32_t k_units, uint8_t *pv,
+                                                  uint8_t *pk, StoreKArgs ka, StoreVArgs va) {
+    // The +-1 operand fragments, sign masks, boundaries and c^2 coefficients are built from the argument block in
+    // registers, so a wavefront's first memory request is its first input; only the 4-bit quantiser tables live in
+    // LDS, and they are fetched behind the first input and waited for by the barrier that also publishes the
+    // ticket counters.
     __shared__ uint32_t counter[2];
     __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 8192 : 2];  // every entry twice (load_quant_lut_dup)
     __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 8192 : 2];
-    __shared__ __attribute__((aligned(16))) uint4 frag_s[1024];  // V fragments, then K fragments
-    __shared__ float s2_s[128];
-    __shared__ uint32_t flip_s[16];
+    // two 4 KB slots per wavefront for the V sub-tiles that travel through LDS (96 KB; not beside the 4-bit tables)
+    constexpr int VDMA = (KB != 4 && VB != 4 && (TQ_EXP & 16)) ? 2 : 0;
+    __shared__ __attribute__((aligned(16))) uint4 vslots[VDMA ? 12 * 2 * 4 * 64 : 1];
     const int t = threadIdx.x;
-    const uint4 c0 = t < 512 ? va.bfrag[t] : ka.afrag[t - 512];
-    const uint4 c1 = ka.afrag[256 + (t & 255)];
-    const float c2 = va.s2[t & 127];
-    const uint32_t c3 = ka.s2flip[t & 15];
+    TQ_TL(0);
     if (t < 2) counter[t] = t == 0 ? 12u : 0u;  // V: the wavefronts' first tickets are their own numbers
     const bool share_lut = KB == 4 && VB == 4 && va.share_k_lut;  // equal tables: one copy serves both tensors
-    if constexpr (KB == 4) load_quant_lut_dup<768>(qlut_k, ka.quant_lut);
-    if constexpr (VB == 4) {
-        if (!share_lut) load_quant_lut_dup<768>(qlut_v, va.quant_lut);
-    }
     auto stage = [&] {
-        frag_s[t] = c0;
-        if (t < 256) frag_s[768 + t] = c1;
-        if (t < 128) s2_s[t] = c2;
-        if (t < 16) flip_s[t] = c3;
+#if (TQ_EXP & 4)
+        // one value from every 64-byte line of the two argument blocks: the loads are issued together
+        asm volatile("" ::"s"(va.s1neg[0]), "s"(va.thr[0]), "s"(va.coef[4]), "s"(va.tokens), "s"(ka.s1neg[0]), "s"(ka.flipw[8]),
+                     "s"(ka.thr[4]), "s"(ka.coef[7]), "s"(ka.tokens));
+#endif
+        if constexpr (KB == 4) load_quant_lut_dup<768>(qlut_k, ka.quant_lut);
+        if constexpr (VB == 4) {
+            if (!share_lut) load_quant_lut_dup<768>(qlut_v, va.quant_lut);
+        }
         __syncthreads();
     };
-    store_v_units<VB, RAGGED, true, true>(xv, pv, va, wg_share(va.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(va.n_units, blockIdx.x + 1, gridDim.x), &counter[0], share_lut ? qlut_k : qlut_v, frag_s, s2_s,
-                              (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6), stage);
-    store_k_units<KB, RAGGED, true>(xk, pk, ka, wg_share(ka.n_units, blockIdx.x, gridDim.x), 1,
-                              wg_share(ka.n_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, frag_s + 512, flip_s,
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6);
+    store_v_units<VB, RAGGED, true, true, true, VDMA>(xv, pv, va, wg_share(v_units, blockIdx.x, gridDim.x), 1,
+                              wg_share(v_units, blockIdx.x + 1, gridDim.x), &counter[0], share_lut ? qlut_k : qlut_v, nullptr, nullptr,
+                              wave, stage, vslots + (VDMA ? wave * (2 * 4 * 64) : 0u));
+    store_k_units<KB, RAGGED, true, true>(xk, pk, ka, wg_share(k_units, blockIdx.x, gridDim.x), 1,
+                              wg_share(k_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, nullptr, nullptr,
                               DRAW_TICKET, [] {});
 }
 
@@ -2518,6 +2813,10 @@ static bool store_fast_ok(const tq_handle *h, int in_dtype, int64_t n_blocks) {
            n_blocks < (1ll << 28);
 }
 
+#ifdef TQ_TIMELINE
+extern "C" int tq_dbg_read_timeline(void *host, long long bytes) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_tl), (size_t)bytes); }
+#endif
+
 static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, int64_t n_blocks) {
     StoreKArgs ka;
     ka.afrag = (const uint4 *)h->rfrag16k; ka.s2flip = h->s2flip; ka.symthr = h->symthr32; ka.sqcoef = h->sqcoef32;
@@ -2525,6 +2824,9 @@ static StoreKArgs make_k_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     ka.norm_correction = h->norm_correction; ka.tokens = tokens;
     ka.blocks_per_seq = (uint32_t)bps; ka.bps_div = make_fast_div((uint32_t)bps); ka.n_units = (uint32_t)(n_blocks * 8);
     ka.out_blocks_per_seq = (uint32_t)bps;
+    for (int i = 0; i < 4; ++i) ka.s1neg[i] = h->s1neg_host[i];
+    for (int i = 0; i < 16; ++i) ka.flipw[i] = h->s2flip_host[i];
+    for (int i = 0; i < 8; ++i) { ka.thr[i] = h->symthr_host[i]; ka.coef[i] = h->sqcoef_host[i]; }
     return ka;
 }
 
@@ -2535,6 +2837,8 @@ static StoreVArgs make_v_args(const tq_handle *h, int64_t tokens, int64_t bps, i
     va.norm_correction = h->norm_correction; va.tokens = tokens; va.share_k_lut = 0;
     va.blocks_per_seq = (uint32_t)bps; va.bps_div = make_fast_div((uint32_t)bps); va.n_units = (uint32_t)(n_blocks * 2);
     va.out_blocks_per_seq = (uint32_t)bps;
+    for (int i = 0; i < 4; ++i) { va.s1neg[i] = h->s1neg_host[i]; va.s2neg[i] = h->s2neg_host[i]; }
+    for (int i = 0; i < 8; ++i) { va.thr[i] = h->symthr_host[i]; va.coef[i] = h->sqcoef_host[i]; }
     return va;
 }
 
@@ -2600,8 +2904,8 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
             ka.n_units = 0;
             const unsigned grid = units12 < 256u ? units12 : 256u;
 #define TQ_ONE(B)                                                                                                                  \
-    if (ragged) k_store_kv<B, B, true><<<grid, 768, 0, s>>>((const __half *)x, (uint8_t *)packed, ka, (const __half *)x, (uint8_t *)packed, va); \
-    else k_store_kv<B, B, false><<<grid, 768, 0, s>>>((const __half *)x, (uint8_t *)packed, ka, (const __half *)x, (uint8_t *)packed, va)
+    if (ragged) k_store_kv<B, B, true><<<grid, 768, 0, s>>>((const __half *)x, (const __half *)x, va.n_units, ka.n_units, (uint8_t *)packed, (uint8_t *)packed, ka, va); \
+    else k_store_kv<B, B, false><<<grid, 768, 0, s>>>((const __half *)x, (const __half *)x, va.n_units, ka.n_units, (uint8_t *)packed, (uint8_t *)packed, ka, va)
             switch (h->bits) {
             case 2: TQ_ONE(2); break;
             case 3: TQ_ONE(3); break;
@@ -2935,10 +3239,10 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
     const unsigned wg = 768;
     const unsigned grid = (unsigned)((va.n_units + 11) / 12 < 256 ? (va.n_units + 11) / 12 : 256);
 #define TQ_KV(KB, VB)                                                                                                       \
-    if (ragged) k_store_kv<KB, VB, true><<<grid, wg, 0, s>>>((const __half *)k, (uint8_t *)packed_k, ka, (const __half *)v, \
-                                                              (uint8_t *)packed_v, va);                                      \
-    else k_store_kv<KB, VB, false><<<grid, wg, 0, s>>>((const __half *)k, (uint8_t *)packed_k, ka, (const __half *)v,        \
-                                                        (uint8_t *)packed_v, va)
+    if (ragged) k_store_kv<KB, VB, true><<<grid, wg, 0, s>>>((const __half *)v, (const __half *)k, va.n_units, ka.n_units,  \
+                                                              (uint8_t *)packed_v, (uint8_t *)packed_k, ka, va);             \
+    else k_store_kv<KB, VB, false><<<grid, wg, 0, s>>>((const __half *)v, (const __half *)k, va.n_units, ka.n_units,        \
+                                                        (uint8_t *)packed_v, (uint8_t *)packed_k, ka, va)
 #define TQ_KV_V(KB)                      \
     switch (hv->bits) {                  \
     case 2: TQ_KV(KB, 2); break;         \
