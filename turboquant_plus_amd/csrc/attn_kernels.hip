@@ -56,12 +56,9 @@ template <int BITS> __device__ __forceinline__ uint32_t pair_off(const uint32_t 
     return pair_lut_offset<BITS>(w, p);
 }
 
-// Measurement builds only (make EXTRA=-DTQ_PAIRTAB3=1): 3-bit codes decode through a pair table with one copy
+// TQ_PAIRTAB3 (tq_measure.h; measurement builds only): 3-bit codes decode through a pair table with one copy
 // per LDS bank (entry e of lane l at dword 64 e + l: no bank conflicts, two 4-byte reads per four values)
 // instead of the 4096-entry quad table (one 8-byte read per four values, about 1.6 conflicts per read).
-#ifndef TQ_PAIRTAB3
-#define TQ_PAIRTAB3 0
-#endif
 // bytes of the decode table of a codebook: quad entries for BITS <= 3, pair entries for 4
 __host__ __device__ constexpr int lut_bytes(int bits) {
     if (TQ_PAIRTAB3 && bits == 3) return 64 * 64 * 4;

@@ -2,6 +2,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -99,6 +100,16 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
         return TQ_ERR_ARG;
     }
     *out = nullptr;
+#ifdef TQ_MEASUREMENT_BUILD
+    // a library with a measurement switch compiled in computes wrong results on purpose: it serves nobody who did not ask
+    {
+        const char *ok = std::getenv("TQ_ALLOW_MEASUREMENT_BUILD");
+        if (!ok || std::strcmp(ok, "1") != 0) {
+            tq_set_error("tq_create: this library is a measurement build (TQ_MEASUREMENT_BUILD); set TQ_ALLOW_MEASUREMENT_BUILD=1 to use it");
+            return TQ_ERR_UNSUPPORTED;
+        }
+    }
+#endif
     if (cfg->d < 1 || cfg->d > TQ_MAX_D) {
         tq_set_error("tq_create: d must be in 1..%d (got %d)", TQ_MAX_D, cfg->d);
         return TQ_ERR_UNSUPPORTED;

@@ -3,6 +3,7 @@
 #pragma once
 #include "tq_internal.h"
 #include "tq_layout.h"
+#include "tq_measure.h"
 
 namespace tqd {
 
@@ -12,10 +13,7 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 // ---- streaming stores -----------------------------------------------------------
 // Output that a launch writes once and never reads back goes out with the non-temporal hint: the lines do not
 // wait in the L2 for the end-of-kernel write-back, so the writes overlap the rest of the launch.
-// TQ_STREAM_SITES (bit mask, measurement builds) switches the hint off per family of kernels.
-#ifndef TQ_STREAM_SITES
-#define TQ_STREAM_SITES 0xFFFF
-#endif
+// TQ_STREAM_SITES (bit mask, tq_measure.h: measurement builds only) switches the hint off per family of kernels.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 template <int SITE> __device__ __forceinline__ void stream_store(uint32_t *p, uint32_t v) {
     if constexpr ((TQ_STREAM_SITES & SITE) != 0) __builtin_nontemporal_store(v, p);

@@ -161,14 +161,11 @@ struct StoreArgs {
     int64_t blocks_per_seq;
 };
 
-// Measurement builds only (make KNOCKOUT=<bits>, default 0 = the product): TQ_KNOCKOUT removes one phase of the
-// fp16 store kernels so that its share of the launch time and of the vector instructions can be read off
-// (results are then meaningless).  1: quantiser compares (a value's code bits come from one xor of its raw
-// bits); 2: four-point butterfly over the input slices; 4: level counts and sum c^2; 8: the sum-of-squares
-// MFMAs (norm = 1); 16: the code stores; 32: the HBM reads (a wavefront re-reads the first units of its share).
-#ifndef TQ_KNOCKOUT
-#define TQ_KNOCKOUT 0
-#endif
+// TQ_KNOCKOUT (tq_measure.h; measurement builds only, 0 in the product) removes one phase of the fp16 store kernels so
+// that its share of the launch time and of the vector instructions can be read off (results are then meaningless).
+// 1: quantiser compares (a value's code bits come from one xor of its raw bits); 2: four-point butterfly over the input
+// slices; 4: level counts and sum c^2; 8: the sum-of-squares MFMAs (norm = 1); 16: the code stores; 32: the HBM reads
+// (a wavefront re-reads the first units of its share).
 // 16 bytes of input (read with the default cache policy: the four loads of a K unit touch every 128-byte line of
 // the unit four times, and with the non-temporal hint each touch went to memory: 20.7 -> 29.8 us for 262 144 K rows)
 __device__ __forceinline__ uint4 load_input16(const uint4 *p) { return *p; }
@@ -446,11 +443,8 @@ template <int BITS> __device__ __forceinline__ uint32_t fold_codes(uint32_t w) {
     }
 }
 
-#ifndef TQ_EXP
-#define TQ_EXP 0
-#endif
-#define TQ_EXP_PRIO (TQ_EXP & 3)
-// Measurement builds only (-DTQ_TIMELINE): per-wavefront timestamps (100 MHz wall clock) of the fused K+V store
+// TQ_TIMELINE (tq_measure.h; measurement builds only): per-wavefront timestamps (100 MHz wall clock) of the fused K+V
+// store; reading the clock costs about a microsecond per stamp, so deltas between neighbouring stamps are upper bounds
 #ifdef TQ_TIMELINE
 __device__ unsigned long long g_tl[4096 * 16];
 #define TQ_TL(slot)                                                                                              \
@@ -853,10 +847,6 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             pend_gn = gn;
             pend_unit = unit;
             pending = true;
-#if TQ_EXP & 64
-            flush();
-            pending = false;
-#endif
         }
     }
     if (pending) flush();
@@ -1025,13 +1015,10 @@ struct StoreVArgs {
 // wavefront, back to back).  It gains 2 us in the fused K+V launch and loses 1 us in the V-only kernel (measured).
 // REG: the constants come from the argument block (fragments built in registers, frag and s2 unused), the first tile is
 // requested before anything else and `stage` runs while it is in flight.
-// VDMA = 2: sub-tiles 1 and 0 of a tile travel through this wavefront's two 4 KB slots in LDS (`slots`; loads that write
-// LDS directly), requested together with the register loads of sub-tiles 3 and 2, so a whole tile (16 KB) is in flight
-// per wavefront instead of half of one, at no cost in registers.
-template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, bool REG, int VDMA = 0, typename Stage>
+template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, bool REG, typename Stage>
 __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
-                                              const float *s2, uint32_t first_ticket, Stage &&stage, uint4 *slots = nullptr) {
+                                              const float *s2, uint32_t first_ticket, Stage &&stage) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1073,24 +1060,6 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
     };
-    // the same sub-tile into LDS slot `sl` of this wavefront: instruction ks writes the lanes' 16-byte pieces to
-    // slots[(4 sl + ks) 64 + lane], which is where the lane reads its operand back
-    auto fetch_lds = [&](uint32_t unit, int u, int sl) {
-        bool valid;
-        const uint4 *p = row_ptr(unit, u, valid);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p + 4 * ks),
-                                             (__attribute__((address_space(3))) void *)(slots + (4 * sl + ks) * 64), 16, 0,
-                                             STREAM_IN ? 2 : 0);
-    };
-    auto read_lds = [&](uint32_t unit, int u, int sl, uint4 (&xb)[4], bool &valid) {
-        if constexpr (RAGGED) (void)row_ptr(unit, u, valid);
-        else valid = true;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = slots[(4 * sl + ks) * 64 + lane];
-    };
-
     uint4 xq[2][4];
     bool xvalid[2];
     uint32_t unit = lo + step * first_ticket;
@@ -1114,10 +1083,6 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
         TQ_TL(9);
         stage();
         TQ_TL(10);
-        if constexpr (VDMA == 2) {  // older than the load of sub-tile 2: when that one has arrived, so have these
-            fetch_lds(unit, 1, 0);
-            fetch_lds(unit, 0, 1);
-        }
         fetch(unit, 2, xq[1], xvalid[1]);
     } else {
         stage();
@@ -1139,7 +1104,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     // for, with their full latency, at the top of the next one).  A sub-tile completes one dword of each of the lane's
     // four rows (2-bit codes: every second sub-tile), which is finished - signs, zero tokens, fold - and parked in `park`;
     // the last one of a tile crosses into the next tile (pend_unit) or is flushed after the loop.
-    constexpr bool DEFER = REG && !(TQ_EXP & 32);
+    constexpr bool DEFER = REG;
     uint32_t park[4] = {0, 0, 0, 0};
     float park_norm = 0.0f;
     uint32_t pend_unit = 0;
@@ -1174,16 +1139,7 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     for (; unit < end;) {
         if (tl_n == 1) TQ_TL(2);
         ++tl_n;
-        // (with sub-tiles in LDS the ticket is drawn after the slots have been read: the compiler makes every LDS
-        // operation wait for all loads that write LDS, and at this point the whole tile is still in flight)
-        uint32_t next = 0;
-        if constexpr (VDMA == 0) next = lo + step * take_ticket(counter, lane);
-        if constexpr (REG) {
-            // A wavefront that takes another tile while its neighbours move on to the small K units must not be the one
-            // its SIMD serves last (the arbiter favours the oldest wavefront slots): it would carry a 64-token chunk to the
-            // end of the launch.  Later tiles run at raised issue priority, the K units at the default.
-            if (TQ_EXP_PRIO && ((TQ_EXP & 8) || unit != lo + step * first_ticket)) __builtin_amdgcn_s_setprio(TQ_EXP_PRIO);
-        }
+        const uint32_t next = lo + step * take_ticket(counter, lane);
         const uint32_t oseq = RAGGED ? a.bps_div.div(unit >> 1) : 0u;
         const uint32_t oblk = RAGGED ? oseq * a.out_blocks_per_seq + ((unit >> 1) - oseq * bps) : unit >> 1;
         uint8_t *block = packed + (int64_t)oblk * block_bytes(BITS);
@@ -1233,33 +1189,8 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                     flush_park(unit, storable(u + 1) < 0 ? 0 : storable(u + 1), u + 1, storable(u + 1) >= 0);
                 }
             }
-            if constexpr (VDMA == 2) {
-                // vector memory operations complete in issue order, and the slots' loads were issued before the register
-                // load of sub-tile 2, whose data the matrix instructions of q = 1 have just used.  The slot address is
-                // tied to their result so that the reads cannot move up past them.
-                if (q == 1) {
-                    uint32_t dep = 0;
-                    asm volatile("" : "+v"(dep) : "v"(gram[0]));
-                    uint4 *keep = slots;
-                    slots += dep;
-                    read_lds(unit, 1, 0, xq[0], xvalid[0]);
-                    read_lds(unit, 0, 1, xq[1], xvalid[1]);
-                    slots = keep;
-                    next = lo + step * take_ticket(counter, lane);
-                } else if (q == 2) {
-                    // both slots have been read (their data feeds this sub-tile's and the next one's matrix instructions;
-                    // the wait below is for the second read): the next tile's sub-tiles 1 and 0 may land in them
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    fetch_lds(next, 1, 0);
-                    fetch_lds(next, 0, 1);
-                    fetch(next, 3, xb, xvalid[0]);
-                } else if (q == 3) {
-                    fetch(next, 2, xb, xvalid[1]);
-                }
-            } else {
-                if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-                else fetch(next, 5 - q, xb, xvalid[q & 1]);
-            }
+            if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
+            else fetch(next, 5 - q, xb, xvalid[q & 1]);
 #ifdef TQ_TIMELINE
             if (q == 0 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(11);   // the first sub-tile's input has arrived
             if (q == 1 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(12);
@@ -1458,7 +1389,6 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
     if constexpr (DEFER) {
         if (pending) flush_park(pend_unit, 0, 0, true);
     }
-    if constexpr (REG) __builtin_amdgcn_s_setprio(0);
     TQ_TL(3);
     TQ_TL_VAL(6, (unsigned long long)tl_n);
 }
@@ -1523,11 +1453,11 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *pa
 // contiguous share of both tensors: every wavefront takes V tiles until the workgroup's share
 // is gone, then K units; the fine-grained K units level what the coarse V tiles leave uneven,
 // and the launch and pipeline-fill time is paid once.
-// The leading scalar parameters are the ones a wavefront needs for its first request (they are candidates for the
-// hardware's preloading of kernel arguments into scalar registers, where the toolchain enables it); the two
-// argument blocks follow and are read in one batch while that request is in flight: left to the compiler, their cache
-// lines were fetched one after the other where first needed, up to three dependent misses of about a microsecond each
-// before a wavefront's first input request.
+// The leading scalar parameters are what a wavefront needs for its first request; the two argument blocks follow.
+// (Measured and not kept: the hardware's preloading of the leading arguments into scalar registers, 33.3 against 32.4 us
+// for the 3-bit launch; reading one value of every cache line of the argument blocks in one batch at entry, 32.4 against
+// 31.9 us; raised issue priority for wavefronts that hold a V tile, which shortens the V phase of the slowest wavefronts
+// from 31 to 22 us and leaves the launch where it was.)
 template <int KB, int VB, bool RAGGED>
 __global__ __launch_bounds__(768) void k_store_kv(const __half *xv, const __half *xk, uint32_t v_units, uint32_t k_units, uint8_t *pv,
                                                   uint8_t *pk, StoreKArgs ka, StoreVArgs va) {
@@ -1538,19 +1468,11 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xv, const __half
     __shared__ uint32_t counter[2];
     __shared__ __attribute__((aligned(16))) uint2 qlut_k[KB == 4 ? 8192 : 2];  // every entry twice (load_quant_lut_dup)
     __shared__ __attribute__((aligned(16))) uint2 qlut_v[VB == 4 ? 8192 : 2];
-    // two 4 KB slots per wavefront for the V sub-tiles that travel through LDS (96 KB; not beside the 4-bit tables)
-    constexpr int VDMA = (KB != 4 && VB != 4 && (TQ_EXP & 16)) ? 2 : 0;
-    __shared__ __attribute__((aligned(16))) uint4 vslots[VDMA ? 12 * 2 * 4 * 64 : 1];
     const int t = threadIdx.x;
     TQ_TL(0);
     if (t < 2) counter[t] = t == 0 ? 12u : 0u;  // V: the wavefronts' first tickets are their own numbers
     const bool share_lut = KB == 4 && VB == 4 && va.share_k_lut;  // equal tables: one copy serves both tensors
     auto stage = [&] {
-#if (TQ_EXP & 4)
-        // one value from every 64-byte line of the two argument blocks: the loads are issued together
-        asm volatile("" ::"s"(va.s1neg[0]), "s"(va.thr[0]), "s"(va.coef[4]), "s"(va.tokens), "s"(ka.s1neg[0]), "s"(ka.flipw[8]),
-                     "s"(ka.thr[4]), "s"(ka.coef[7]), "s"(ka.tokens));
-#endif
         if constexpr (KB == 4) load_quant_lut_dup<768>(qlut_k, ka.quant_lut);
         if constexpr (VB == 4) {
             if (!share_lut) load_quant_lut_dup<768>(qlut_v, va.quant_lut);
@@ -1558,9 +1480,9 @@ __global__ __launch_bounds__(768) void k_store_kv(const __half *xv, const __half
         __syncthreads();
     };
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6);
-    store_v_units<VB, RAGGED, true, true, true, VDMA>(xv, pv, va, wg_share(v_units, blockIdx.x, gridDim.x), 1,
+    store_v_units<VB, RAGGED, true, true, true>(xv, pv, va, wg_share(v_units, blockIdx.x, gridDim.x), 1,
                               wg_share(v_units, blockIdx.x + 1, gridDim.x), &counter[0], share_lut ? qlut_k : qlut_v, nullptr, nullptr,
-                              wave, stage, vslots + (VDMA ? wave * (2 * 4 * 64) : 0u));
+                              wave, stage);
     store_k_units<KB, RAGGED, true, true>(xk, pk, ka, wg_share(k_units, blockIdx.x, gridDim.x), 1,
                               wg_share(k_units, blockIdx.x + 1, gridDim.x), &counter[1], qlut_k, nullptr, nullptr,
                               DRAW_TICKET, [] {});
