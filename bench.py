@@ -228,6 +228,34 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
         codec_k.load_kv(codec_v, kp_i, vp_i, heads, tokens, out_k=ok, out_v=ov)
     _, lev_ms = time_steps(torch, lstep, steps, warmup)
     load_algo = n_vec * (16 * bits + 2 + 256)
+    # fp32 rows (the reference's input type; config 1's path): the same K and V tensors as float32 through tq_store_kv,
+    # which runs the matrix-core kernels on two fp16 terms per value, one launch per tensor; and K alone
+    f32 = None
+    if bits == 3:
+        sets32 = [(k_.float(), v_.float(), kp_, vp_) for (k_, v_, kp_, vp_) in sets[:2]]
+
+        def fstep(i):
+            k_, v_, kp_, vp_ = sets32[i % 2]
+            codec_k.store_kv(codec_v, k_, v_, out_k=kp_, out_v=vp_)
+
+        def fkstep(i):
+            k_, _, kp_, _ = sets32[i % 2]
+            codec_k.store(k_, kind="k", out=kp_)
+        def fvstep(i):
+            _, v_, _, vp_ = sets32[i % 2]
+            codec_v.store(v_, kind="v", out=vp_)
+        _, fev_ms = time_steps(torch, fstep, steps, warmup)
+        _, fkev_ms = time_steps(torch, fkstep, steps, warmup)
+        _, fvev_ms = time_steps(torch, fvstep, steps, warmup)
+        f_algo = n_vec * (512 + 16 * bits + 2)
+        f32 = {"what": "K and V as float32 rows (512 B per vector in), two launches (k_store_k<float>, k_store_v<float>)",
+               "us_per_step": fev_ms * 1e3, "algorithmic_bytes_per_step": f_algo, "gbs": f_algo / (fev_ms * 1e-3) / 1e9,
+               "frac": f_algo / (fev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               "k_alone": {"us_per_launch": fkev_ms * 1e3, "gbs": f_algo / 2 / (fkev_ms * 1e-3) / 1e9,
+                           "frac": f_algo / 2 / (fkev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+               "v_alone": {"us_per_launch": fvev_ms * 1e3, "gbs": f_algo / 2 / (fvev_ms * 1e-3) / 1e9,
+                           "frac": f_algo / 2 / (fvev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}}
+        del sets32
     return {
         "workload": f"turbo{bits} store, K+V fp16 [8,32768,128], 4 K outlier channels x15, block 128",
         "ms_per_step": wall_ms, "event_ms_per_step": ev_ms, "kernel_us": launch_us,
@@ -238,6 +266,7 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
         "several_streams": None if two_us is None else {
             "streams": 4, "us_per_launch": two_us, "gbs": algo / (two_us * 1e-6) / 1e9, "frac": algo / (two_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
             "what": "the same launches issued round-robin on four streams, wall clock per launch; not the roofline figure"},
+        "fp32_rows": f32,
         "decompress": {"us_per_step": lev_ms * 1e3, "launches_per_step": 1, "io": "codes + fp16 norm in, fp16 out",
                        "gbs": load_algo / (lev_ms * 1e-3) / 1e9, "frac": load_algo / (lev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }

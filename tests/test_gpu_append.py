@@ -26,10 +26,13 @@ def blocks_of(buf, bits, n_seqs, capacity):
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("kind", ["k", "v"])
 def test_append_in_chunks_equals_store(bits, kind):
+    """float64 rows: tq_store serves them with the butterfly arithmetic that tq_append uses, so the bytes are equal
+    (fp16 and fp32 rows are stored through the matrix cores, whose codes agree with the append's outside the boundary
+    band: test_append_codes_match_oracle, test_prefill_into_a_cache_laid_out_for_more_tokens)."""
     tt = L.torch()
     codec = tqa.TurboCodec(bits, seed=7)
     n_seqs, capacity = 3, 512
-    x = np.random.default_rng(bits).standard_normal((n_seqs, 300, D)).astype(np.float32)
+    x = np.random.default_rng(bits).standard_normal((n_seqs, 300, D)).astype(np.float32).astype(np.float64)
     x[1, 5] = 0
     cache = tt.zeros(tqa.packed_bytes(bits, n_seqs, capacity), dtype=tt.uint8, device="cuda")
     pos = 0
@@ -55,8 +58,8 @@ def test_append_after_a_rewind_truncates(bits, kind, back_to, n_new):
     codec = tqa.TurboCodec(bits, seed=9)
     n_seqs, capacity = 2, 384
     rng = np.random.default_rng(bits * 100 + back_to)
-    x = rng.standard_normal((n_seqs, 230, D)).astype(np.float32)
-    y = rng.standard_normal((n_seqs, n_new, D)).astype(np.float32)
+    x = rng.standard_normal((n_seqs, 230, D)).astype(np.float32).astype(np.float64)   # float64 rows: see above
+    y = rng.standard_normal((n_seqs, n_new, D)).astype(np.float32).astype(np.float64)
     cache = tt.zeros(tqa.packed_bytes(bits, n_seqs, capacity), dtype=tt.uint8, device="cuda")
     codec.append(x, cache, 0, capacity, kind=kind)
     codec.append(y, cache, back_to, capacity, kind=kind)
@@ -469,13 +472,14 @@ def test_prefill_into_a_cache_laid_out_for_more_tokens(kb, vb, tokens):
         assert (idx_m[:, :tokens] != idx_t[:, :tokens]).mean() < 1e-4
 
 
-def test_prefill_falls_back_to_the_append_for_fp32_rows_and_checks_its_arguments():
+def test_prefill_falls_back_to_the_append_for_fp64_rows_and_checks_its_arguments():
+    """Rows the matrix-core store does not take (float64) reach a cache through the append from position 0."""
     tt = L.torch()
     n_seqs, tokens, capacity = 2, 150, 384
     kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
     rng = np.random.default_rng(8)
-    k = rng.standard_normal((n_seqs, tokens, D)).astype(np.float32)
-    v = rng.standard_normal((n_seqs, tokens, D)).astype(np.float32)
+    k = rng.standard_normal((n_seqs, tokens, D))
+    v = rng.standard_normal((n_seqs, tokens, D))
     ck, cv = (tt.zeros(tqa.packed_bytes(3, n_seqs, capacity), dtype=tt.uint8, device="cuda") for _ in range(2))
     ak, av = tt.zeros_like(ck), tt.zeros_like(cv)
     kc.store_kv(vc, k, v, out_k=ck, out_v=cv, capacity=capacity)

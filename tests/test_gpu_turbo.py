@@ -310,6 +310,63 @@ def test_config2_turbo4_store_full_size_properties():
             del x, xd, packed, idx, g, rec, org
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_store_fp32_rows_on_the_matrix_cores(bits, kind):
+    """fp32 rows go through the matrix-core store as two fp16 terms per value at a per-row power-of-two scale: codes and
+    norms against the float64 oracle at the same bar as fp16 rows, for rows whose norms span seven decades (what the
+    fp16 stored norm can hold), rows with x15 outlier channels, a row dominated by one element, a row of values below
+    fp16's range and zero rows; ragged token counts included."""
+    codec = tqa.TurboCodec(bits, seed=42)
+    rng = np.random.default_rng(100 * bits + (kind == "v"))
+    n_seqs, tokens = 3, 1000                      # 8 blocks per sequence, the last one ragged
+    x = rng.standard_normal((n_seqs, tokens, D)).astype(np.float32)
+    x *= np.exp(rng.uniform(-9, 7, (n_seqs, tokens, 1))).astype(np.float32)        # norms from 1e-3 to 1e4 (the stored norm is fp16)
+    x[0][:, rng.choice(D, size=4, replace=False)] *= 15.0
+    x[1, 5] = 0
+    x[1, 6, 3:] = 0                               # one non-zero element
+    x[2, 7] = rng.standard_normal(D).astype(np.float32) * 1e-3
+    x[2, 7, 0] = 3e4                              # one element that dwarfs the rest of its row
+    x[2, 8] = rng.standard_normal(D).astype(np.float32) * 1e-6   # a row whose elements are below fp16's normal range
+    packed = codec.store(x, kind=kind)
+    idx, g = codec.unpack_codes(packed, n_seqs, tokens, kind=kind)
+    idx, g = np_(idx).reshape(-1, D), np_(g).reshape(-1)
+    n_bad, n_ulp, idx_o, g_o = check_codes(codec, x.reshape(-1, D), idx, g)
+    print(f"fp32 rows, {bits} bits, {kind}: {n_bad} in-band index mismatches of {idx.size}, {n_ulp} norms one ulp apart")
+    # bytes: whole blocks against the oracle's layout of the codes just checked
+    xw = x[:, :896]
+    pw = codec.store(np.ascontiguousarray(xw), kind=kind)
+    iw, gw = codec.unpack_codes(pw, n_seqs, 896, kind=kind)
+    assert np.array_equal(np_(iw).reshape(-1, D), idx.reshape(n_seqs, tokens, D)[:, :896].reshape(-1, D))
+    assert np.array_equal(np_(pw), np.concatenate([O.layout_pack(np_(iw)[s_], np_(gw)[s_].astype(np.float16), bits, kind)
+                                                   for s_ in range(n_seqs)]))
+    # the same rows as fp16 (where they fit fp16's range): the same codes outside the boundary band
+    y = rng.standard_normal((2, 512, D)).astype(np.float16)
+    a, _ = codec.unpack_codes(codec.store(y, kind=kind), 2, 512, kind=kind)
+    b, _ = codec.unpack_codes(codec.store(y.astype(np.float32), kind=kind), 2, 512, kind=kind)
+    assert (np_(a) != np_(b)).sum() <= 2
+
+
+def test_store_kv_fp32_into_a_cache_layout():
+    """tq_store_kv / tq_store_kv_cache with fp32 rows run the matrix-core kernels (one launch per tensor): the bytes of
+    the single-tensor stores, also into caches laid out for a larger capacity (rest of the cache untouched)."""
+    tt = L.torch()
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(4, seed=542)
+    rng = np.random.default_rng(77)
+    k = rng.standard_normal((3, 300, D)).astype(np.float32)
+    v = rng.standard_normal((3, 300, D)).astype(np.float32)
+    pk, pv = kc.store_kv(vc, k, v)
+    assert tt.equal(pk, kc.store(k, kind="k")) and tt.equal(pv, vc.store(v, kind="v"))
+    cap = 1024
+    ck = tt.full((tqa.packed_bytes(3, 3, cap),), 0xA5, dtype=tt.uint8, device="cuda")
+    cv = tt.full((tqa.packed_bytes(4, 3, cap),), 0xA5, dtype=tt.uint8, device="cuda")
+    kc.store_kv(vc, k, v, out_k=ck, out_v=cv, capacity=cap)
+    for cache, ref, bits in ((ck, pk, 3), (cv, pv, 4)):
+        per_seq_cache, per_seq = tqa.packed_bytes(bits, 1, cap), tqa.packed_bytes(bits, 1, 300)
+        c, r = np_(cache).reshape(3, per_seq_cache), np_(ref).reshape(3, per_seq)
+        assert np.array_equal(c[:, :per_seq], r) and (c[:, per_seq:] == 0xA5).all()
+
+
 @pytest.mark.parametrize("bits", [4, 3])
 def test_config2_fused_store_full_size_bytes(bits):
     """The launch the benchmark times: tq_store_kv on config 2's tensors at full size (K with four outlier channels

@@ -473,6 +473,41 @@ __device__ __forceinline__ void settle_matrix_results() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// ---- fp32 rows on the fp16 matrix cores ---------------------------------------------------------
+// A row is scaled by a power of two to 512 <= ||x|| < 1024 (exact; every element then lies inside fp16's normal range or is
+// negligible against the row) and every scaled element is split into two fp16 terms, hi = rn(x), mid = rn(x - hi): hi +
+// mid equals x up to 2^-22 |x|.  The +-1 transform is applied to both terms into one accumulator, so the products are
+// exact and the rotated value differs from the fp32 butterfly's only by roundings of the same size (the codes are held
+// to the float64 oracle outside the 1e-6 boundary band, as for fp16 rows).  The norm comes from the fp32 values.
+typedef float float2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float row_pow2_scale(float norm) {
+    const uint32_t e = (__float_as_uint(norm) >> 23) & 0xFFu;  // biased exponent: norm = m 2^(e - 127), 1 <= m < 2
+    const uint32_t se = 263u - e;                              // 2^(9 - (e - 127)), biased
+    return (e == 0u || e == 255u) ? 1.0f : __uint_as_float((se > 254u ? 254u : se) << 23);
+}
+__device__ __forceinline__ float pow2_reciprocal(float p) { return __uint_as_float(0x7F000000u - __float_as_uint(p)); }  // p = 2^k, |k| < 127
+// eight consecutive fp32 inputs (two 16-byte pieces) times sc -> their hi and mid terms as MFMA operands
+__device__ __forceinline__ void split8(uint4 a, uint4 b, float sc, half8_t &hi, half8_t &mid) {
+    const float v[8] = {__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z), __uint_as_float(a.w),
+                        __uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float2_t xs = {v[2 * i] * sc, v[2 * i + 1] * sc};
+        const half2_t h = __builtin_convertvector(xs, half2_t);
+        const float2_t r = xs - __builtin_convertvector(h, float2_t);
+        const half2_t m = __builtin_convertvector(r, half2_t);
+        hi[2 * i] = h[0]; hi[2 * i + 1] = h[1];
+        mid[2 * i] = m[0]; mid[2 * i + 1] = m[1];
+    }
+}
+__device__ __forceinline__ float sumsq8(uint4 a, uint4 b, float acc) {
+    acc = fmaf(__uint_as_float(a.x), __uint_as_float(a.x), acc); acc = fmaf(__uint_as_float(a.y), __uint_as_float(a.y), acc);
+    acc = fmaf(__uint_as_float(a.z), __uint_as_float(a.z), acc); acc = fmaf(__uint_as_float(a.w), __uint_as_float(a.w), acc);
+    acc = fmaf(__uint_as_float(b.x), __uint_as_float(b.x), acc); acc = fmaf(__uint_as_float(b.y), __uint_as_float(b.y), acc);
+    acc = fmaf(__uint_as_float(b.z), __uint_as_float(b.z), acc); acc = fmaf(__uint_as_float(b.w), __uint_as_float(b.w), acc);
+    return acc;
+}
+
 struct StoreKArgs {
     const uint4 *afrag;      // [8 fragments f0*4+ks][64 lanes] 8 halves (+-1)
     const uint32_t *s2flip;  // [4 lane quarters][4]: sign-field positions of the dims with s2 = +1, per output dword
@@ -589,11 +624,14 @@ constexpr int K_UNITS_AHEAD = 1;
 // them), or DRAW_TICKET to draw them.  `stage` makes the workgroup's LDS copy of the constant operands (frag,
 // flips) readable; it runs after the first inputs have been requested.
 // REG: the constants come from the argument block (fragments built in registers, frag and flips unused).
-template <int BITS, bool RAGGED, bool DUP_LUT, bool REG, typename Stage>
-__device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
+// TI = float: fp32 rows, split into two fp16 terms (see row_pow2_scale).
+template <int BITS, bool RAGGED, bool DUP_LUT, bool REG, typename Stage, typename TI>
+__device__ __forceinline__ void store_k_units(const TI *x, uint8_t *packed, const StoreKArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const uint32_t *flips, uint32_t first_ticket, Stage &&stage) {
     constexpr int NT = 1 << (BITS - 1);
+    constexpr bool F32 = sizeof(TI) == 4;
+    constexpr int NX = F32 ? 8 : 4;  // 16-byte pieces of a lane's 32 inputs
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kc = lane >> 4;
     float thr0[NT], coef[NT];
@@ -604,10 +642,10 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     }
 
     const uint32_t bps = a.blocks_per_seq, last_unit = end ? end - 1 : 0;  // prefetches past the share re-read its last unit
-    // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B).
+    // This lane's 64 contiguous bytes of its token (inputs 32kc .. 32kc+31; slice ks = 16 B; twice that for fp32 rows).
     // The address is always valid: units past the end and rows past a sequence's last token
     // are clamped, and `valid` says whether the data is to be used.
-    auto fetch = [&](uint32_t unit, uint4 (&xb)[4], bool &valid) {
+    auto fetch = [&](uint32_t unit, uint4 (&xb)[NX], bool &valid) {
         // A prefetch past the share (its data is never used) reads the tensor's first bytes, every lane the same
         // ones: a clamped re-read of the last unit would go to memory again where rows are read with the
         // non-temporal hint, and a branch around the loads costs registers.
@@ -628,7 +666,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             p = reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)unit * 16 + n16) * 128 + 32 * kc));
         }
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = load_input16(p + ks);
+        for (int ks = 0; ks < NX; ++ks) xb[ks] = load_input16(p + ks);
     };
 
     // an exact zero counts as positive only if the middle boundary is below zero
@@ -639,7 +677,7 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
     // units of input in flight per wavefront: one ahead measures faster than two (262 144 rows of 3-bit K alone
     // 16.9 against 18.2 us, the fused K+V launch 34.4 against 36.0 us)
     constexpr int DEPTH = K_UNITS_AHEAD;
-    uint4 xq[DEPTH][4];
+    uint4 xq[DEPTH][NX];
     bool xvalid[DEPTH];
     uint32_t cur[DEPTH];
 #pragma unroll
@@ -699,47 +737,76 @@ __device__ __forceinline__ void store_k_units(const __half *x, uint8_t *packed, 
             if (tl_n == 1) TQ_TL(4);
             ++tl_n;
             const uint32_t next = lo + step * take_ticket(counter, lane);
-            uint4 (&xb)[4] = xq[r];
+            uint4 (&xb)[NX] = xq[r];
             if constexpr (RAGGED) {
                 if (!xvalid[r]) {
 #pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
+                    for (int ks = 0; ks < NX; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
                 }
             }
 
             float4_t q[2][4];
+            float ss, rowscale = 1.0f;  // rowscale: the power of two an fp32 row was multiplied by
+            if constexpr (F32) {
+                // norm first (the split needs the row's scale), from the fp32 values
+                float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
-            for (int f0 = 0; f0 < 2; ++f0)
+                for (int ks = 0; ks < 4; ks += 2) {
+                    s0 = sumsq8(xb[2 * ks], xb[2 * ks + 1], s0);
+                    s1 = sumsq8(xb[2 * ks + 2], xb[2 * ks + 3], s1);
+                }
+                ss = s0 + s1;
+                ss += xor_lane<16>(ss);
+                ss += xor_lane<32>(ss);
+                rowscale = row_pow2_scale(__builtin_amdgcn_sqrtf(ss));
+                half8_t hi[4], mid[4];
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
-                    q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], __builtin_bit_cast(half8_t, xb[ks]),
-                                                                       float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-            // ||x||^2 on the matrix cores as well: the diagonal of X X^T (the same registers serve as
-            // both operands); token n16's entry is element n16 % 4 of lane quarter n16 / 4
-            float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+                for (int ks = 0; ks < 4; ++ks) split8(xb[2 * ks], xb[2 * ks + 1], rowscale, hi[ks], mid[ks]);
+#pragma unroll
+                for (int f0 = 0; f0 < 2; ++f0)
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+                        q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], mid[ks], float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], hi[ks], q[f0][ks], 0, 0, 0);
+                    }
+                cur[r] = next;
+                settle_matrix_results();
+                if (pending) flush();  // the previous unit's codes, behind this unit's wait for its input
+                fetch(next, xb, xvalid[r]);
+            } else {
+#pragma unroll
+                for (int f0 = 0; f0 < 2; ++f0)
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks)
+                        q[f0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f0 * 4 + ks], __builtin_bit_cast(half8_t, xb[ks]),
+                                                                           float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                // ||x||^2 on the matrix cores as well: the diagonal of X X^T (the same registers serve as
+                // both operands); token n16's entry is element n16 % 4 of lane quarter n16 / 4
+                float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
 #if TQ_KNOCKOUT & 8
-            gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
+                gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
 #else
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-                gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
-                                                              gram, 0, 0, 0);
+                for (int ks = 0; ks < 4; ++ks)
+                    gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
+                                                                  gram, 0, 0, 0);
 #endif
-            float ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
-            ss = diag_here ? ss : 0.0f;
-            cur[r] = next;
-            settle_matrix_results();
-            if (pending) flush();  // the previous unit's codes, behind this unit's wait for its input
-            fetch(next, xb, xvalid[r]);
-            ss += xor_lane<16>(ss);
-            ss += xor_lane<32>(ss);
+                ss = diag_sel == 0 ? gram[0] : diag_sel == 1 ? gram[1] : diag_sel == 2 ? gram[2] : gram[3];
+                ss = diag_here ? ss : 0.0f;
+                cur[r] = next;
+                settle_matrix_results();
+                if (pending) flush();  // the previous unit's codes, behind this unit's wait for its input
+                fetch(next, xb, xvalid[r]);
+                ss += xor_lane<16>(ss);
+                ss += xor_lane<32>(ss);
+            }
             const float norm = __builtin_amdgcn_sqrtf(ss);  // 1 ulp: scales boundaries (1e-7 relative) and the stored fp16 norm
-            const float scale = norm > 0.0f ? norm * 11.313708498984761f : 1.0f;  // y' = sqrt(128) ||x|| y
+            const float scale = norm > 0.0f ? norm * rowscale * 11.313708498984761f : 1.0f;  // y' = sqrt(128) ||x|| y
             float thr[NT];
 #pragma unroll
             for (int k = 0; k < NT; ++k) thr[k] = thr0[k] * scale;
             // table path (4 bits): values are normalised instead of the boundaries being scaled
-            const float inv = norm > 0.0f ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;
+            const float inv = norm > 0.0f ? __builtin_amdgcn_rsqf(ss) * (0.08838834764831845f * pow2_reciprocal(rowscale)) : 1.0f;
 
             // butterfly over the input slices: fragment 2*fh + f0 holds dims 32kc + 8fh + 4f0 + i
             float4_t y[8];
@@ -1015,12 +1082,14 @@ struct StoreVArgs {
 // wavefront, back to back).  It gains 2 us in the fused K+V launch and loses 1 us in the V-only kernel (measured).
 // REG: the constants come from the argument block (fragments built in registers, frag and s2 unused), the first tile is
 // requested before anything else and `stage` runs while it is in flight.
-template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, bool REG, typename Stage>
-__device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
+template <int BITS, bool RAGGED, bool STREAM_IN, bool DUP_LUT, bool REG, typename Stage, typename TI>
+__device__ __forceinline__ void store_v_units(const TI *x, uint8_t *packed, const StoreVArgs &a, uint32_t lo, uint32_t step,
                                               uint32_t end, uint32_t *counter, const uint2 *qlut, const uint4 *frag,
                                               const float *s2, uint32_t first_ticket, Stage &&stage) {
     constexpr int NT = 1 << (BITS - 1);
     constexpr int NW = BITS == 3 ? 4 : BITS;  // dwords of a row group while it is built (3-bit: + the tail word)
+    constexpr bool F32 = sizeof(TI) == 4;     // fp32 rows: two fp16 terms per value (see row_pow2_scale)
+    constexpr int NX = F32 ? 8 : 4;           // 16-byte pieces of a lane's 32 inputs of one sub-tile
     const int tid = threadIdx.x, lane = tid & 63;
     const int n16 = lane & 15, kq = lane >> 4;
     float thr0[NT], coef[NT];
@@ -1055,13 +1124,24 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
             return reinterpret_cast<const uint4 *>(x + (beyond ? (int64_t)0 : ((int64_t)blk * TQ_ROWS_PER_BLOCK + tb) * 128 + 8 * kq));
         }
     };
-    auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[4], bool &valid) {
+    auto fetch = [&](uint32_t unit, int u, uint4 (&xb)[NX], bool &valid) {
         const uint4 *p = row_ptr(unit, u, valid);
+        if constexpr (F32) {  // inputs 32 ks + 8 kq .. + 7: 32 bytes at a 128-byte stride
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
+            for (int ks = 0; ks < 4; ++ks) {
+                xb[2 * ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 8 * ks) : p[8 * ks];
+                xb[2 * ks + 1] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 8 * ks + 1) : p[8 * ks + 1];
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) xb[ks] = STREAM_IN ? stream_load<STREAM_STORE_V_IN>(p + 4 * ks) : p[4 * ks];
+        }
     };
-    uint4 xq[2][4];
-    bool xvalid[2];
+    // sub-tiles of input in flight: two of fp16 rows, one of fp32 rows (which take twice the registers; two of them
+    // leave room for two wavefronts per SIMD only: 41 against 30 us for 262 144 rows)
+    constexpr int VD = F32 ? 1 : 2;
+    uint4 xq[VD][NX];
+    bool xvalid[VD];
     uint32_t unit = lo + step * first_ticket;
     // The first tile is requested behind the barrier that makes the constants readable: when the wavefronts of the
     // chip ask for their first input at once, ahead of the constants, the burst takes several microseconds to serve and
@@ -1083,11 +1163,11 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
         TQ_TL(9);
         stage();
         TQ_TL(10);
-        fetch(unit, 2, xq[1], xvalid[1]);
+        if constexpr (VD == 2) fetch(unit, 2, xq[1], xvalid[1]);
     } else {
         stage();
         fetch(unit, 3, xq[0], xvalid[0]);
-        fetch(unit, 2, xq[1], xvalid[1]);
+        if constexpr (VD == 2) fetch(unit, 2, xq[1], xvalid[1]);
 #pragma unroll
         for (int f = 0; f < 8; ++f) bf[f] = __builtin_bit_cast(half8_t, frag[f * 64 + lane]);
 #pragma unroll
@@ -1155,30 +1235,58 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int u = 3 - q;
-            uint4 (&xb)[4] = xq[q & 1];
+            const int xsel = VD == 2 ? (q & 1) : 0;
+            uint4 (&xb)[NX] = xq[xsel];
             if constexpr (RAGGED) {
-                if (!xvalid[q & 1]) {
+                if (!xvalid[xsel]) {
 #pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
+                    for (int ks = 0; ks < NX; ++ks) xb[ks] = make_uint4(0, 0, 0, 0);
                 }
             }
             float4_t qq[2][4];
-#pragma unroll
-            for (int d0 = 0; d0 < 2; ++d0)
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
-                    qq[d0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), bf[d0 * 4 + ks],
-                                                                        float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-            // ||x||^2: diagonal of X X^T; element i of this lane is row 4kq + i, column n16
+            // ||x||^2 of the four tokens whose values this lane ends up with, as gram[i] of the lane that holds it
+            // (row 4kq + i, column n16: the diagonal of X X^T)
             float4_t gram = float4_t{0.f, 0.f, 0.f, 0.f};
+            if constexpr (F32) {
+                // this lane's 32 inputs belong to token row n16: its squared norm over the four lanes that share it, from
+                // the fp32 values; then the two-term split at the row's scale
+                float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+                for (int ks = 0; ks < 4; ks += 2) {
+                    s0 = sumsq8(xb[2 * ks], xb[2 * ks + 1], s0);
+                    s1 = sumsq8(xb[2 * ks + 2], xb[2 * ks + 3], s1);
+                }
+                float ssr = s0 + s1;
+                ssr += xor_lane<16>(ssr);
+                ssr += xor_lane<32>(ssr);
+                gram[0] = gram[1] = gram[2] = gram[3] = ssr;  // picked where n16 == 4kq + i below
+                const float rs = row_pow2_scale(__builtin_amdgcn_sqrtf(ssr));
+                half8_t hi[4], mid[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) split8(xb[2 * ks], xb[2 * ks + 1], rs, hi[ks], mid[ks]);
+#pragma unroll
+                for (int d0 = 0; d0 < 2; ++d0)
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+                        qq[d0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mid[ks], bf[d0 * 4 + ks], float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        qq[d0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi[ks], bf[d0 * 4 + ks], qq[d0][ks], 0, 0, 0);
+                    }
+            } else {
+#pragma unroll
+                for (int d0 = 0; d0 < 2; ++d0)
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks)
+                        qq[d0][ks] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), bf[d0 * 4 + ks],
+                                                                            float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #if TQ_KNOCKOUT & 8
-            gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
+                gram[0] = gram[1] = gram[2] = gram[3] = 1.0f;
 #else
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-                gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
-                                                              gram, 0, 0, 0);
+                for (int ks = 0; ks < 4; ++ks)
+                    gram = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xb[ks]), __builtin_bit_cast(half8_t, xb[ks]),
+                                                                  gram, 0, 0, 0);
 #endif
+            }
             // (before this sub-tile's requests: the wait for a sub-tile's input lets only a few younger operations stay
             // outstanding, and these stores are then a whole sub-tile old when the next wait comes)
             if constexpr (DEFER) {
@@ -1189,8 +1297,13 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                     flush_park(unit, storable(u + 1) < 0 ? 0 : storable(u + 1), u + 1, storable(u + 1) >= 0);
                 }
             }
-            if (q < 2) fetch(unit, 1 - q, xb, xvalid[q & 1]);
-            else fetch(next, 5 - q, xb, xvalid[q & 1]);
+            if constexpr (VD == 2) {
+                if (q < 2) fetch(unit, 1 - q, xb, xvalid[xsel]);
+                else fetch(next, 5 - q, xb, xvalid[xsel]);
+            } else {
+                if (q < 3) fetch(unit, 2 - q, xb, xvalid[xsel]);
+                else fetch(next, 3, xb, xvalid[xsel]);
+            }
 #ifdef TQ_TIMELINE
             if (q == 0 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(11);   // the first sub-tile's input has arrived
             if (q == 1 && tl_n == 1 && gram[0] != 12345.678f) TQ_TL(12);
@@ -1204,11 +1317,12 @@ __device__ __forceinline__ void store_v_units(const __half *x, uint8_t *packed, 
                 const float ss = row16_sum(n16 == 4 * kq + i ? gram[i] : 0.0f);
                 nrm[i] = __builtin_amdgcn_sqrtf(ss);
                 const bool nz = ss > 0.0f;
+                const float rowscale = F32 ? row_pow2_scale(nrm[i]) : 1.0f;  // the power of two the token's fp32 row was multiplied by
                 if constexpr (BITS == 4) {
-                    inv[i] = nz ? __builtin_amdgcn_rsqf(ss) * 0.08838834764831845f : 1.0f;  // 1 / (||x|| sqrt(128))
+                    inv[i] = nz ? __builtin_amdgcn_rsqf(ss) * (0.08838834764831845f * pow2_reciprocal(rowscale)) : 1.0f;  // 1 / (||x|| sqrt(128))
                 } else {
                     inv[i] = 1.0f;
-                    const float scale = nz ? nrm[i] * 11.313708498984761f : 1.0f;
+                    const float scale = nz ? nrm[i] * rowscale * 11.313708498984761f : 1.0f;
 #pragma unroll
                     for (int k = 0; k < NT; ++k) thr_tok[i][k] = thr0[k] * scale;
                 }
@@ -1399,8 +1513,8 @@ __device__ __forceinline__ uint32_t wg_share(uint32_t n, uint32_t b, uint32_t g)
 // into LDS (thousands of wavefronts asking the L2 for the same 8 KB delayed the start by several microseconds).
 
 // single tensor: fixed strided share per wavefront (four workgroups of four wavefronts per CU for K, three for V)
-template <int BITS, bool RAGGED>
-__global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *packed, StoreKArgs a) {
+template <int BITS, bool RAGGED, typename TI = __half>
+__global__ __launch_bounds__(256, sizeof(TI) == 4 ? 3 : 4) void k_store_k(const TI *x, uint8_t *packed, StoreKArgs a) {
     // measured at 262 144 vectors: the LDS copy of the constants gains 1.6 us with 4-bit codes and 0.3 us with
     // 2-bit codes and loses 1.1 us with 3-bit codes, whose wavefronts then read them from memory themselves
     constexpr bool STAGED = BITS != 3;
@@ -1428,8 +1542,8 @@ __global__ __launch_bounds__(256, 4) void k_store_k(const __half *x, uint8_t *pa
     }
 }
 
-template <int BITS, bool RAGGED>
-__global__ __launch_bounds__(256, 3) void k_store_v(const __half *x, uint8_t *packed, StoreVArgs a) {
+template <int BITS, bool RAGGED, typename TI = __half>
+__global__ __launch_bounds__(256, 3) void k_store_v(const TI *x, uint8_t *packed, StoreVArgs a) {
     __shared__ uint32_t counter[4];
     __shared__ __attribute__((aligned(16))) uint2 qlut[BITS == 4 ? 4096 : 2];
     __shared__ __attribute__((aligned(16))) uint4 frag_s[512];
@@ -2731,8 +2845,8 @@ int tqk_rotate128(const tq_handle *h, const void *x, void *y, int64_t n, int in_
 // fp16 input with a sign-symmetric codebook: rotation on the matrix cores, codes packed in
 // registers.  The butterfly kernel serves every other case (fp32 / fp64 input, asymmetric codebooks).
 static bool store_fast_ok(const tq_handle *h, int in_dtype, int64_t n_blocks) {
-    return in_dtype == TQ_F16 && h->symmetric && h->bits >= 2 && h->bits <= 4 && (h->bits != 4 || h->quant_lut_ok) &&
-           n_blocks < (1ll << 28);
+    return (in_dtype == TQ_F16 || in_dtype == TQ_F32) && h->symmetric && h->bits >= 2 && h->bits <= 4 &&
+           (h->bits != 4 || h->quant_lut_ok) && n_blocks < (1ll << 28);
 }
 
 #ifdef TQ_TIMELINE
@@ -2775,6 +2889,52 @@ template <typename K> static unsigned resident_workgroups(K kernel) {
     return (unsigned)prop.multiProcessorCount * (unsigned)per_cu;
 }
 
+// single-tensor launches of the matrix-core store (fp16 or fp32 rows): as many workgroups of four wavefronts as are
+// resident at once (registers and LDS decide: 2 to 4 per CU)
+static int launch_store_k(const tq_handle *h, const void *x, int in_dtype, void *packed, const StoreKArgs &ka, bool ragged, hipStream_t s) {
+    const unsigned kneed = (unsigned)((ka.n_units + 3) / 4);
+#define TQ_STORE_K_T(B, T)                                                                              \
+    {                                                                                                   \
+        static const unsigned fit[2] = {resident_workgroups(k_store_k<B, false, T>), resident_workgroups(k_store_k<B, true, T>)}; \
+        const unsigned kgrid = kneed < fit[ragged] ? kneed : fit[ragged];                               \
+        if (ragged) k_store_k<B, true, T><<<kgrid, 256, 0, s>>>((const T *)x, (uint8_t *)packed, ka);     \
+        else k_store_k<B, false, T><<<kgrid, 256, 0, s>>>((const T *)x, (uint8_t *)packed, ka);           \
+    }
+#define TQ_STORE_K(B)                                \
+    if (in_dtype == TQ_F32) TQ_STORE_K_T(B, float)   \
+    else TQ_STORE_K_T(B, __half)
+    switch (h->bits) {
+    case 2: TQ_STORE_K(2); break;
+    case 3: TQ_STORE_K(3); break;
+    default: TQ_STORE_K(4); break;
+    }
+#undef TQ_STORE_K
+#undef TQ_STORE_K_T
+    return tq_check_launch("store_k");
+}
+
+static int launch_store_v(const tq_handle *h, const void *x, int in_dtype, void *packed, const StoreVArgs &va, bool ragged, hipStream_t s) {
+    const unsigned vneed = (unsigned)((va.n_units + 3) / 4);
+#define TQ_STORE_V_T(B, T)                                                                              \
+    {                                                                                                   \
+        static const unsigned fit[2] = {resident_workgroups(k_store_v<B, false, T>), resident_workgroups(k_store_v<B, true, T>)}; \
+        const unsigned vgrid = vneed < fit[ragged] ? vneed : fit[ragged];                               \
+        if (ragged) k_store_v<B, true, T><<<vgrid, 256, 0, s>>>((const T *)x, (uint8_t *)packed, va);     \
+        else k_store_v<B, false, T><<<vgrid, 256, 0, s>>>((const T *)x, (uint8_t *)packed, va);           \
+    }
+#define TQ_STORE_V(B)                                \
+    if (in_dtype == TQ_F32) TQ_STORE_V_T(B, float)   \
+    else TQ_STORE_V_T(B, __half)
+    switch (h->bits) {
+    case 2: TQ_STORE_V(2); break;
+    case 3: TQ_STORE_V(3); break;
+    default: TQ_STORE_V(4); break;
+    }
+#undef TQ_STORE_V
+#undef TQ_STORE_V_T
+    return tq_check_launch("store_v");
+}
+
 constexpr int64_t SINGLE_VIA_FUSED_BLOCKS = 512;  // 65 536 vectors
 int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens, int in_dtype, int kind, void *packed,
               uint8_t *sign_bits, void *rnorms, hipStream_t s) {
@@ -2814,7 +2974,7 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
     if (store_fast_ok(h, in_dtype, n_seqs * bps)) {
         const int64_t n_blocks = n_seqs * bps;
         const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK;
-        if (kind == TQ_KIND_V && n_blocks >= SINGLE_VIA_FUSED_BLOCKS) {
+        if (kind == TQ_KIND_V && n_blocks >= SINGLE_VIA_FUSED_BLOCKS && in_dtype == TQ_F16) {
             // A large V tensor: the K+V kernel with an empty K share (one workgroup of twelve wavefronts per CU drawing
             // tiles from a queue) is faster than k_store_v - 262 144 vectors: 20.9 against 21.9 us (3-bit), 22.4
             // against 23.3 us (4-bit), 18.2 against 19.1 us (2-bit).  K tensors are slower that way (17.7 against
@@ -2836,41 +2996,8 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 #undef TQ_ONE
             return tq_check_launch("store_v (through the K+V kernel)");
         }
-        if (kind == TQ_KIND_K) {
-            const StoreKArgs ka = make_k_args(h, tokens, bps, n_blocks);
-            // as many workgroups of four wavefronts as are resident at once (registers and LDS decide: 2 to 4 per CU)
-            const unsigned kneed = (unsigned)((ka.n_units + 3) / 4);
-#define TQ_STORE_K(B)                                                                                   \
-    {                                                                                                   \
-        static const unsigned fit[2] = {resident_workgroups(k_store_k<B, false>), resident_workgroups(k_store_k<B, true>)}; \
-        const unsigned kgrid = kneed < fit[ragged] ? kneed : fit[ragged];                               \
-        if (ragged) k_store_k<B, true><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);   \
-        else k_store_k<B, false><<<kgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, ka);         \
-    }
-            switch (h->bits) {
-            case 2: TQ_STORE_K(2); break;
-            case 3: TQ_STORE_K(3); break;
-            default: TQ_STORE_K(4); break;
-            }
-#undef TQ_STORE_K
-            return tq_check_launch("store_k");
-        }
-        const StoreVArgs va = make_v_args(h, tokens, bps, n_blocks);
-        const unsigned vneed = (unsigned)((va.n_units + 3) / 4);
-#define TQ_STORE_V(B)                                                                                   \
-    {                                                                                                   \
-        static const unsigned fit[2] = {resident_workgroups(k_store_v<B, false>), resident_workgroups(k_store_v<B, true>)}; \
-        const unsigned vgrid = vneed < fit[ragged] ? vneed : fit[ragged];                               \
-        if (ragged) k_store_v<B, true><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);   \
-        else k_store_v<B, false><<<vgrid, 256, 0, s>>>((const __half *)x, (uint8_t *)packed, va);         \
-    }
-        switch (h->bits) {
-        case 2: TQ_STORE_V(2); break;
-        case 3: TQ_STORE_V(3); break;
-        default: TQ_STORE_V(4); break;
-        }
-#undef TQ_STORE_V
-        return tq_check_launch("store_v");
+        if (kind == TQ_KIND_K) return launch_store_k(h, x, in_dtype, packed, make_k_args(h, tokens, bps, n_blocks), ragged, s);
+        return launch_store_v(h, x, in_dtype, packed, make_v_args(h, tokens, bps, n_blocks), ragged, s);
     }
     StoreArgs a;
     a.s1 = h->s1_32; a.s2 = h->s2_32; a.bounds = h->bounds32; a.cent = h->centroids32;
@@ -3157,6 +3284,10 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
     ka.out_blocks_per_seq = va.out_blocks_per_seq = (uint32_t)out_bps;
     va.share_k_lut = hk->bits == 4 && hv->bits == 4 && hk->quant_lut_hash == hv->quant_lut_hash;
     const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK || out_bps != bps;
+    if (in_dtype != TQ_F16) {  // fp32 rows: the single-tensor kernels, one launch per tensor
+        const int rc = launch_store_k(hk, k, in_dtype, packed_k, ka, ragged, s);
+        return rc ? rc : launch_store_v(hv, v, in_dtype, packed_v, va, ragged, s);
+    }
     // one workgroup of 12 wavefronts per CU
     const unsigned wg = 768;
     const unsigned grid = (unsigned)((va.n_units + 11) / 12 < 256 ? (va.n_units + 11) / 12 : 256);
