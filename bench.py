@@ -305,6 +305,37 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
     attn8 = tqa.DecodeAttention(kc, vc, B, 2 * Hq, Hkv, N)
     _, ev8_ms = time_steps(torch, lambda i: attn8(q64, sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
 
+    # Sparse V on this cache (turbo3 K and V: V is half of the bytes): the benchmark's queries and queries scaled x16
+    # (peaked attention), with the skip rate the kernel reports
+    sparse_v = {}
+    for name, qscale in (("bench_queries", 1.0), ("peaked_queries_x16", 16.0)):
+        qs_ = [(st[0].float() * qscale).to(torch.float16) for st in sets]
+        dn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N)
+        sp = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, sparse_v_tau=1e-6)
+        _, d_ms = time_steps(torch, lambda i: dn(qs_[i % n_sets], sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
+        _, s_ms = time_steps(torch, lambda i: sp(qs_[i % n_sets], sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
+        sparse_v[name] = {"dense_us_per_step": d_ms * 1e3, "sparse_v_us_per_step": s_ms * 1e3, "tau": 1e-6,
+                          "skip_rate": sp.skip_rate()}
+        del dn, sp
+
+    # small batches on the same kind of cache: few (batch, kv head) groups, so the context splits must fill the chip
+    small = {}
+    for name, b_, n_ in (("B1_ctx32768", 1, N), ("B4_ctx32768", 4, N), ("B256_ctx2048", 256, 2048)):
+        per_seq = tqa.packed_bytes(bits, Hkv, n_)
+        if b_ * per_seq <= sets[0][1].numel():
+            kp_, vp_ = sets[0][1][:b_ * per_seq], sets[0][2][:b_ * per_seq]     # any valid codes do for timing
+        else:
+            kp_ = sets[0][1].repeat(-(-b_ * per_seq // sets[0][1].numel()))[:b_ * per_seq]
+            vp_ = sets[0][2].repeat(-(-b_ * per_seq // sets[0][2].numel()))[:b_ * per_seq]
+        gq = torch.Generator(device="cuda").manual_seed(400 + b_)
+        qb = torch.randn((b_, Hq, D), generator=gq, device="cuda").to(torch.float16)
+        at = tqa.DecodeAttention(kc, vc, b_, Hq, Hkv, n_)
+        _, sm_ms = time_steps(torch, lambda i: at(qb, kp_, vp_), steps, warmup)
+        sm_algo = 2 * b_ * Hkv * n_ * 50
+        small[name] = {"us_per_step": sm_ms * 1e3, "n_splits": at.params.n_splits, "algorithmic_bytes_per_step": sm_algo,
+                       "gbs": sm_algo / (sm_ms * 1e-3) / 1e9, "frac": sm_algo / (sm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        del at, kp_, vp_
+
     # a whole serving step: append this step's K and V token of every sequence (the last position of the
     # cache is rewritten each time), then attention; launched one by one and replayed from one HIP graph
     g = torch.Generator(device="cuda").manual_seed(77)
@@ -339,6 +370,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         "gqa8": {"workload": "the same cache, 64 query heads on 8 KV heads (eight heads per pass over K/V)",
                  "us_per_step": ev8_ms * 1e3, "n_splits": attn8.params.n_splits,
                  "frac": algo / (ev8_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "sparse_v": sparse_v, "small_batches": small,
         "serving_step": {"workload": "tq_append_kv of one token per sequence + decode attention",
                          "us_per_step": serve_ms * 1e3, "us_per_step_hip_graph": graph_ms * 1e3 / n_sets},
     }
@@ -385,9 +417,15 @@ def asym_decode_leg(torch, tqa, steps, warmup):
         return below / float(B * Hq * N), rows_saved / float(B * Hkv * (N // 64))
     out = {}
     q_peaked = (q.float() * 16.0).to(torch.float16)  # a second input for Sparse V: logits 16 x as spread, few tiles matter
-    for name, tau, qq in (("dense", 0.0, q), ("sparse_v", 1e-6, q), ("sparse_v_peaked_queries", 1e-6, q_peaked)):
+    # the sharpening bias as per-head (position, value) lists: 64 entries per head instead of a dense fp32 row per head
+    sparse_bias = tqa.sparse_bias_from_dense(bias, max_entries=64)
+    for name, tau, qq, as_rows in (("dense", 0.0, q, False), ("dense_bias_as_rows", 0.0, q, True), ("sparse_v", 1e-6, q, False),
+                                   ("sparse_v_peaked_queries", 1e-6, q_peaked, False)):
         attn = tqa.DecodeAttention(None, vc, B, Hq, Hkv, N, sparse_v_tau=tau)
-        wall_ms, ev_ms = time_steps(torch, lambda i: attn(qq, kq, vp, bias=bias), steps, warmup)
+        if as_rows:
+            wall_ms, ev_ms = time_steps(torch, lambda i: attn(qq, kq, vp, bias=bias), steps, warmup)
+        else:
+            wall_ms, ev_ms = time_steps(torch, lambda i: attn(qq, kq, vp, sparse_bias=sparse_bias), steps, warmup)
         skip = attn.skip_rate() if tau else 0.0
         algo = B * Hkv * N * (136 + 34)               # dense bytes: the roofline figure of every variant
         us = ev_ms * 1e3
@@ -400,7 +438,8 @@ def asym_decode_leg(torch, tqa, steps, warmup):
             out[name]["v_rows_not_fetched"] = rows_saved
             out[name]["bytes_required"] = B * Hkv * N * (136 + (1.0 - rows_saved) * 34)
     out["workload"] = ("decode attention, K q8_0-style + V turbo2, B4 Hq32 Hkv8 ctx 131072, +6 bias on 64 key "
-                       "positions per head as an fp32 bias input (67 MB, not counted), Sparse V tau 1e-6; "
+                       "positions per head as 64 (position, value) entries per head (dense_bias_as_rows: the same bias as a dense "
+                       "fp32 row per head, 67 MB of input, not counted), Sparse V tau 1e-6; "
                        "sparse_v_peaked_queries: the same cache with the queries scaled x16; skip_rate = (query, position) "
                        "pairs whose weight the kernel dropped, v_rows_not_fetched = fraction of 64-token V rows it never "
                        "requested (whole tiles only), bytes_required = K + the V rows it did request")

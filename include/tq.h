@@ -284,6 +284,17 @@ typedef struct tq_attn_params {
                                            /* maximum, sizes the workspace and is the stride */
                                            /* of the bias rows): one captured launch replays */
                                            /* at a growing length.  skip_count must be NULL. */
+    int32_t bias_entries;                  /* sparse additive logit bias: entries per query   */
+                                           /* head, 0 = none (a bias that is zero but for a   */
+                                           /* few positions costs its list, not a dense row   */
+                                           /* per head); added to the dense bias if both come */
+    const int32_t *bias_pos;               /* [batch, n_q_heads, bias_entries] positions in   */
+                                           /* device memory, ascending within a head and each */
+                                           /* position at most once; a list shorter than      */
+                                           /* bias_entries is filled up with positions >=     */
+                                           /* tokens (INT32_MAX)                              */
+    const float *bias_val;                 /* [batch, n_q_heads, bias_entries] values, fp32,  */
+                                           /* natural-log units like the dense bias           */
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four

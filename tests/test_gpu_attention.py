@@ -192,6 +192,51 @@ def test_decode_attention_bias_and_sparse_v():
             np.testing.assert_allclose(out_s, out_d, rtol=0, atol=1e-4 * np.abs(ref_d).max())
 
 
+@pytest.mark.parametrize("G,n_splits,N,E", [(4, 4, 1000, 5), (4, 16, 4096, 64), (8, 8, 2111, 70), (1, 1, 64, 3), (6, 32, 2048, 130)])
+def test_decode_attention_sparse_bias(G, n_splits, N, E):
+    """A logit bias given as per-head (position, value) lists equals the same bias given as dense rows (to rounding: the
+    two forms run different instantiations of the kernel, and one adds the scaled bias with a fused multiply-add), and
+    both meet the oracle; lists of unequal length (padded), entries at a
+    tile's first and last position and at the context's last token, dense and sparse together, Sparse V on top."""
+    tt = L.torch()
+    B, Hkv = 2, 2
+    Hq = Hkv * G
+    k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=300 + G)
+    rng = np.random.default_rng(E)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    for b in range(B):
+        for h in range(Hq):
+            n_e = E if (b + h) % 3 else max(1, E // 2)                   # lists of unequal length
+            pos = rng.choice(N, size=min(n_e, N), replace=False)
+            bias[b, h, pos] = rng.uniform(2.0, 6.0, size=len(pos)).astype(np.float32)
+    bias[0, 0, [0, 63, min(64, N - 1), N - 1]] = [6.0, 5.0, 4.0, 3.0]     # tile edges and the last token
+    pos_d, val_d = tqa.sparse_bias_from_dense(bias)
+    assert pos_d.shape[2] >= 1 and int((val_d != 0).sum()) == int((bias != 0).sum())
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits)
+    dense = np_(attn(q, kp, vp, bias=tt.from_numpy(bias).cuda())).copy()
+    sparse = np_(attn(q, kp, vp, sparse_bias=(pos_d, val_d))).copy()
+    np.testing.assert_allclose(sparse, dense, rtol=0, atol=2e-6 * np.abs(dense).max())
+    ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, bias=bias)
+    assert_close(sparse, ref)
+    assert np.abs(sparse - np_(attn(q, kp, vp))).max() > 1e-3            # the bias is not a no-op
+    # half of the bias dense, half sparse: they add up
+    half = bias * (rng.random(bias.shape) < 0.5)
+    p2, v2 = tqa.sparse_bias_from_dense(bias - half)
+    both = np_(attn(q, kp, vp, bias=tt.from_numpy(half.astype(np.float32)).cuda(), sparse_bias=(p2, v2)))
+    assert_close(both, ref)
+    # with Sparse V: the same skipped pairs as with the dense form
+    tau = 1e-3
+    sv = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+    a1 = np_(sv(q, kp, vp, bias=tt.from_numpy(bias).cuda())).copy()
+    r1 = sv.skip_rate()
+    a2 = np_(sv(q, kp, vp, sparse_bias=(pos_d, val_d))).copy()
+    np.testing.assert_allclose(a2, a1, rtol=0, atol=2e-6 * np.abs(a1).max())
+    assert abs(sv.skip_rate() - r1) <= 1e-5
+    with pytest.raises(ValueError):
+        attn(q, kp, vp, sparse_bias=(pos_d.to(tt.int64), val_d))
+
+
 @pytest.mark.parametrize("N,misalign", [(1000, 0), (1001, 0), (999, 0), (1000, 1), (64, 0), (67, 1)])
 def test_decode_attention_dense_bias_every_position(N, misalign):
     """A bias that differs at every position, for context lengths that are and are not multiples of four and

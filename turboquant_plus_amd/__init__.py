@@ -11,10 +11,11 @@ from .turboquant import TurboQuant, TurboQuantMSE, CompressedVector
 from .kv_cache import KVCacheCompressor, CompressedKVCache
 from .outlier import OutlierTurboQuant, OutlierCompressedVector
 from .policy import LayerFormat, LayerKV, layer_formats, effective_bits
-from .turbo import (TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, q8_0_append, packed_bytes, PRODUCTION_CENTROIDS)
+from .turbo import (TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, q8_0_append, packed_bytes, PRODUCTION_CENTROIDS,
+                    sparse_bias_from_dense)
 
 __all__ = ["PolarQuant", "QJL", "TurboQuant", "TurboQuantMSE", "CompressedVector", "KVCacheCompressor",
            "OutlierTurboQuant", "OutlierCompressedVector",
            "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "q8_0_append", "packed_bytes",
-           "PRODUCTION_CENTROIDS", "LayerFormat", "LayerKV", "layer_formats",
+           "PRODUCTION_CENTROIDS", "sparse_bias_from_dense", "LayerFormat", "LayerKV", "layer_formats",
            "effective_bits"]

@@ -194,13 +194,16 @@ struct AttnArgs {
     const uint8_t *k, *v;
     const uint32_t *klut, *vlut;  // pair tables (half2 per pair code)
     const float *bias;            // [groups*4][tokens] natural-log units, or NULL
+    const int32_t *sbias_pos;     // sparse bias: [groups*q_group][sbias_n] positions, ascending within a head (entries that
+    const float *sbias_val;       // do not exist: any position >= tokens), and their values (natural-log units)
+    int sbias_n;                  // entries per head, 0 = no sparse bias
     float *part_o;                // [groups][workgroups per group][4][128]
     float *part_ml;               // [groups][workgroups per group][4][2]  (m in log2 units, l)
     unsigned long long *skip_slots;  // Sparse V: [workgroup] nonce tag | (query, position) pairs it skipped; 0 after the count
     // merge of the workgroups' partials by the last workgroup of a group to finish (see merge_group)
     float *out;                      // [groups * q_group][128]
     const float *vs1, *vs2;          // V rotation signs (NULL: V rows are stored unrotated)
-    unsigned long long *flags;       // [workgroup] nonce once the workgroup's partial is in memory, 0 after the merge
+    unsigned long long *flags;       // [group][workgroups per group]; word 0 of a group is its arrival counter (tag | count), 0 after the merge
     unsigned long long nonce;        // differs from call to call (and from whatever the workspace held before)
     int poll_slots;                       // Sparse V: the merging workgroups add the slots up themselves
     unsigned long long *pass_totals;      // Sparse V: [pass] skipped pairs of each four-head pass of this step
@@ -283,18 +286,20 @@ __device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, cons
 // block that this lane's dims of that dim half lie in
 template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 1]; };
 
+constexpr unsigned long long ARRIVAL_COUNT_MASK = 0xFFFFFFull;  // workgroups of a group (the tag of the call sits above)
 constexpr float Q8V_PRESCALE = 64.0f;  // keeps weight * scale products out of fp16's subnormals; 65504 / 64 > any scale
 
 // ---- merging the workgroups' partials inside the launch -------------------------------------
 // A group's partials are written by up to n_splits / wavefronts-per-workgroup workgroups that may run on
 // different dies, whose L2 caches are not coherent with each other for ordinary accesses.  Everything the
-// workgroups exchange therefore moves with device-scope atomic loads and stores (they go through to memory),
-// ordered by waiting for the stores to complete: a workgroup stores its partial, waits, raises its flag, waits,
-// and then reads the group's flags; the workgroup that finds every flag raised merges the group (two may, if
-// they finish together: both write the same values).  A flag holds the call's nonce, so what a fresh workspace
-// happens to contain is not mistaken for a raised flag, and the merging workgroup puts the flags back to zero,
-// so a replay of a captured launch (same nonce) starts clean.  No cache-wide write-back or invalidate is
-// involved, which is what made a merge behind device-scope fences cost more than the second launch it saved.
+// workgroups exchange therefore moves with device-scope atomic accesses (they go through to memory): a workgroup
+// stores its partial, waits for the stores to complete, and then increments the group's arrival counter with one
+// read-modify-write; the workgroup whose increment completes the count merges the group.  The counter carries a tag
+// of the call, so what a fresh workspace happens to contain is not mistaken for arrivals, and the merging workgroup
+// puts it back to zero, so a replay of a captured launch (same tag) starts clean.  No cache-wide write-back or
+// invalidate is involved, which is what made a merge behind device-scope fences cost more than the second launch it
+// saved.  (An earlier version raised a flag per workgroup and read the group's flags: two more trips to memory per
+// workgroup, and "somebody sees every flag" needed a store-to-load ordering argument where the counter needs none.)
 __device__ __forceinline__ void st_dev(float *p, float v) {
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -416,7 +421,9 @@ __device__ __forceinline__ unsigned long long block_sum(unsigned long long t, un
 // double the accumulators and the softmax state and run with at most 8 wavefronts too.
 __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { return vbits == 8 || hg == 2 ? 8 : 16; }
 
-template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG>
+// SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
+// registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
+template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS>
 __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_decode_attn(AttnArgs a) {
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
@@ -603,6 +610,42 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     float bias_next[HG][4];
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
+    // Sparse bias: a head's (position, value) list is walked by a cursor as the tiles go by.  The cursor starts at the
+    // head's first entry inside this split: the number of entries below the split's first token, counted with the
+    // whole wavefront (one entry per lane and round); the sixteen lanes that hold a head's logits move in step.
+    int sb_cur[HG], sb_pos[HG];
+    float sb_val[HG];
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) {
+        sb_cur[hg] = 0;
+        sb_pos[hg] = 0x7FFFFFFF;
+        sb_val[hg] = 0.0f;
+    }
+    // entry e of the list of this lane's head in set hg (addresses are formed where they are needed: the path is rare)
+    auto sb_entry = [&](int hg, int e) { return ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.sbias_n + e; };
+    if constexpr (SBIAS) {
+        const int first_tok = t_begin * 64;
+#pragma unroll
+        for (int hg = 0; hg < HG; ++hg) {
+            int below[4];
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const int32_t *prow = a.sbias_pos + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + h, a.q_group - 1)) * a.sbias_n;
+                int c = 0;
+                for (int e0 = 0; e0 < a.sbias_n; e0 += 64) {
+                    const int e = e0 + lane;
+                    const int pe = e < a.sbias_n ? prow[e] : 0x7FFFFFFF;
+                    c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(pe < first_tok));
+                }
+                below[h] = c;
+            }
+            sb_cur[hg] = j == 0 ? below[0] : j == 1 ? below[1] : j == 2 ? below[2] : below[3];
+            if (sb_cur[hg] < a.sbias_n) {
+                sb_pos[hg] = a.sbias_pos[sb_entry(hg, sb_cur[hg])];
+                sb_val[hg] = a.sbias_val[sb_entry(hg, sb_cur[hg])];
+            }
+        }
+    }
     unsigned nskip = 0;  // Sparse V: skipped (query, position) pairs of this wavefront (wave-uniform: counted from lane masks)
     bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
@@ -636,6 +679,25 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
 #pragma unroll
             for (int i = 0; i < 4; ++i) bias4[hg][i] = bias_next[hg][i] * LOG2E;
             load_bias(tile_n, hg, bias_next[hg]);
+        }
+        if constexpr (SBIAS) {
+            // entries of this tile (a handful per head and context: the loop body runs for few tiles)
+            const int tile_hi = tile * 64 + 64;
+#pragma unroll
+            for (int hg = 0; hg < HG; ++hg) {
+                while (__builtin_amdgcn_ballot_w64(sb_pos[hg] < tile_hi) != 0ull) {
+                    if (sb_pos[hg] < tile_hi) {
+                        const int d = sb_pos[hg] - tile * 64 - b4;  // an entry at an earlier position than the cursor expects is dropped
+                        const float add = sb_val[hg] * LOG2E;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) bias4[hg][i] += d == i ? add : 0.0f;
+                        ++sb_cur[hg];
+                        const bool more = sb_cur[hg] < a.sbias_n;
+                        sb_pos[hg] = more ? a.sbias_pos[sb_entry(hg, sb_cur[hg])] : 0x7FFFFFFF;
+                        sb_val[hg] = more ? a.sbias_val[sb_entry(hg, sb_cur[hg])] : 0.0f;
+                    }
+                }
+            }
         }
 
         // ---- QK ------------------------------------------------------------------
@@ -877,14 +939,33 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     wait_stores();  // this lane's part of the partial (and the skip slot) is in memory
     __syncthreads();
     if (n_parts > 1) {
+        // Arrival counter of the group: the call's tag in the upper 40 bits, the number of workgroups whose partial is
+        // in memory in the lower 24.  One read-modify-write per workgroup; a word that does not carry the tag (whatever a
+        // fresh workspace held, or the zero a finished call leaves) counts as zero arrivals.  Read-modify-writes on one
+        // word happen one after the other, so exactly one workgroup brings the count to n_parts: it merges, and every
+        // other partial was complete in memory before its owner's increment, hence before this one's.
+        __shared__ int i_am_last;
         if (tid == 0) {
-            st_dev(a.flags + blockIdx.x, a.nonce);
-            wait_stores();
+            unsigned long long *ctr = a.flags + (int64_t)group * n_parts;
+            const unsigned long long tag = a.nonce & ~ARRIVAL_COUNT_MASK;
+            unsigned long long seen = ld_dev(ctr), count;
+            for (;;) {
+                if ((seen & ~ARRIVAL_COUNT_MASK) == tag) {
+                    // the word is this call's (it stays so until the merge): a plain increment, no retry however many
+                    // workgroups arrive together
+                    count = (__hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & ARRIVAL_COUNT_MASK) + 1ull;
+                    break;
+                }
+                // first arrival of the call: install the tag with a count of one, unless somebody else just did
+                if (__hip_atomic_compare_exchange_strong(ctr, &seen, tag | 1ull, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                    count = 1ull;
+                    break;
+                }
+            }
+            i_am_last = (int)count == n_parts;
         }
-        __syncthreads();  // the flag is up before anybody reads the group's flags
-        int all_up = 1;
-        for (int p = tid; p < n_parts; p += (int)blockDim.x) all_up &= ld_dev(a.flags + (int64_t)group * n_parts + p) == a.nonce;
-        if (!__syncthreads_and(all_up)) return;
+        __syncthreads();
+        if (!i_am_last) return;
     }
     // Sparse V: every workgroup's slot carries its count (40 bits: at most 4 heads x 2^31 positions) under 24 bits
     // of the nonce.  A merging workgroup reads all slots of the launch now, so that the trip to memory overlaps
@@ -904,9 +985,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         }
     }
     merge_group<HG>(a, group, n_parts, tid, n_waves);
-    if (n_parts > 1) {
-        for (int p = tid; p < n_parts; p += (int)blockDim.x) st_dev(a.flags + (int64_t)group * n_parts + p, 0ull);
-    }
+    if (n_parts > 1 && tid == 0) st_dev(a.flags + (int64_t)group * n_parts, 0ull);  // a replay of a captured launch (same tag) starts from zero
     if constexpr (SPARSE) {
         if (a.poll_slots) {
             if (!__syncthreads_and(all_in)) return;
@@ -1029,6 +1108,13 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     const bool share = turbo_k && turbo_v && hk->bits == hv->bits &&
                        std::memcmp(hk->pair_lut_host, hv->pair_lut_host, sizeof(hk->pair_lut_host)) == 0;
     a.bias = bias;
+    a.sbias_n = p->bias_entries;
+    a.sbias_pos = p->bias_pos;
+    a.sbias_val = p->bias_val;
+    if (p->bias_entries < 0 || (p->bias_entries > 0 && (!p->bias_pos || !p->bias_val))) {
+        tq_set_error("tq_decode_attention: bias_entries %d needs bias_pos and bias_val", (int)p->bias_entries);
+        return TQ_ERR_ARG;
+    }
     a.part_o = part_o;
     a.part_ml = part_ml;
     a.skip_slots = reinterpret_cast<unsigned long long *>((char *)ws + w.skip_slots);
@@ -1087,8 +1173,10 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         a.nonce = next_nonce();
 #define TQ_ATTN_ONE(KF, KB, VB, SP, SH)                                            \
     {                                                                             \
-        if (hg == 2) k_decode_attn<KF, KB, VB, SP, SH, 2><<<grid, wg, merge_bytes, s>>>(a); \
-        else k_decode_attn<KF, KB, VB, SP, SH, 1><<<grid, wg, merge_bytes, s>>>(a);         \
+        if (hg == 2 && a.sbias_n) k_decode_attn<KF, KB, VB, SP, SH, 2, true><<<grid, wg, merge_bytes, s>>>(a);   \
+        else if (hg == 2) k_decode_attn<KF, KB, VB, SP, SH, 2, false><<<grid, wg, merge_bytes, s>>>(a);        \
+        else if (a.sbias_n) k_decode_attn<KF, KB, VB, SP, SH, 1, true><<<grid, wg, merge_bytes, s>>>(a);        \
+        else k_decode_attn<KF, KB, VB, SP, SH, 1, false><<<grid, wg, merge_bytes, s>>>(a);                      \
     }
 #define TQ_ATTN(KF, KB, VB)                         \
     if (sparse) TQ_ATTN_ONE(KF, KB, VB, true, false)  \

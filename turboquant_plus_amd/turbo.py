@@ -447,11 +447,28 @@ class DecodeAttention:
         self.out = tt.empty((batch, n_q_heads, HEAD_DIM), dtype=tt.float32, device=dev)
         self.poison_output = os.environ.get("TQ_POISON_OUTPUT", "0") == "1" if poison_output is None else bool(poison_output)
 
-    def __call__(self, q, k_packed, v_packed, bias=None):
-        """q [batch, n_q_heads, 128] in the original domain -> out fp32 [batch, n_q_heads, 128]."""
+    def __call__(self, q, k_packed, v_packed, bias=None, sparse_bias=None):
+        """q [batch, n_q_heads, 128] in the original domain -> out fp32 [batch, n_q_heads, 128].
+        bias: dense additive logit bias [batch, n_q_heads, tokens] fp32.  sparse_bias: (positions, values), int32 and fp32
+        device tensors [batch, n_q_heads, E]: a bias that is zero except at E positions per head, positions ascending
+        within a head and unique (sparse_bias_from_dense() builds the pair); both may be given and add up."""
         qd = L.to_device(q)
         if self.poison_output:
             self.out.fill_(float("nan"))
+        tt = L.torch()
+        if sparse_bias is not None:
+            pos, val = sparse_bias
+            want = (self.params.batch, self.params.n_q_heads)
+            if (pos.dtype != tt.int32 or val.dtype != tt.float32 or not pos.is_cuda or not val.is_cuda or pos.dim() != 3
+                    or tuple(pos.shape[:2]) != want or pos.shape != val.shape):
+                raise ValueError("sparse_bias must be (int32 positions, float32 values), device tensors [batch, n_q_heads, E]")
+            pos, val = pos.contiguous(), val.contiguous()
+            self.params.bias_entries = int(pos.shape[2])
+            self.params.bias_pos, self.params.bias_val = pos.data_ptr(), val.data_ptr()
+            self._sparse_bias = (pos, val)   # kept alive until the next call
+        else:
+            self.params.bias_entries = 0
+            self.params.bias_pos = self.params.bias_val = None
         hk = self.k_codec.handle.h if self.k_codec is not None else None
         hv = self.v_codec.handle.h if self.v_codec is not None else None
         L.check(L.lib().tq_decode_attention(hk, hv, C.byref(self.params), L.ptr(qd),
@@ -474,15 +491,37 @@ class DecodeAttention:
         return float(s[0]) / float(s[1]) if s[1] else 0.0
 
 
+def sparse_bias_from_dense(bias, max_entries: int | None = None):
+    """Dense logit bias [batch, n_q_heads, tokens] -> (positions int32, values fp32) [batch, n_q_heads, E] holding its
+    non-zero entries, positions ascending within a head and lists padded with position 2^31 - 1 (value 0).  E is the
+    largest count of non-zero entries over the heads (ValueError if that exceeds max_entries)."""
+    tt = L.torch()
+    bd = L.to_device(bias).to(tt.float32)
+    nz = bd != 0
+    e = int(nz.sum(dim=-1).max().item()) if bd.numel() else 0
+    if max_entries is not None and e > max_entries:
+        raise ValueError(f"a head has {e} non-zero bias entries, more than {max_entries}")
+    e = max(e, 1)
+    # a stable sort of "is zero" puts every head's non-zero positions first, in ascending order
+    order = tt.sort((~nz).to(tt.int8), dim=-1, stable=True).indices[..., :e]
+    val = tt.gather(bd, -1, order)
+    pos = tt.where(val != 0, order, tt.full_like(order, 2 ** 31 - 1)).to(tt.int32)
+    return pos.contiguous(), val.contiguous()
+
+
 def default_splits(n_groups: int, tokens: int) -> int:
     """Context splits per (batch, kv head): one wavefront per split, four
-    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each.
+    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each (2 when the groups are few).
     The kernel groups up to 16 splits (the largest power of two dividing the
     count) into one workgroup, so the count is rounded down to a multiple of 16,
     or to a power of two below 16."""
     tiles = max(1, (tokens + 63) // 64)
     want = max(1, (4 * 1024 + n_groups - 1) // n_groups)
     n = int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
+    if n_groups * max(n // 16, 1) < 256 and tiles >= 4:
+        # few groups (small batches): the chip is not full at four tiles per split; two tiles per split measured
+        # faster there (one sequence at 32K: 22.6 against 27.2 us), one tile per split no better
+        n = int(max(1, min(want, tiles // 2)))
     if n >= 16:
         return n // 16 * 16
     return 1 << (n.bit_length() - 1)
