@@ -12,7 +12,9 @@ A step is one pass of the hot path over one batch of synthetic input:
     batch 16, 32 query heads on 8 KV heads, context 32768.
 Further legs, each under its own key of the line: config 4 (q8_0-style K, turbo2 V, Sparse V), the config 5 score
 tile and QJL store, a boundary layer (q8_0-style K and V), the kernels that rework a packed cache (requantise, export
-to and import from the fork's blocks) and the measured peaks of this box (stream probes, fp16 MFMA loop).
+to and import from the fork's blocks) and the measured peaks of this box (stream probes, fp16 MFMA loop).  The store
+leg also times fp32 rows (two fp16 terms per value on the matrix cores), the config-3 decode leg a Sparse V variant and
+three small-batch shapes, config 4 its attention-sink bias as a sparse list and as dense rows.
 Inputs are resident in HBM before the timed region; every step cycles through
 several distinct buffer sets so that the 256 MB Infinity Cache cannot serve
 the reads.  Kernel durations come from HIP events recorded on the stream the
@@ -28,7 +30,9 @@ take less than 60 ms (e.g. --steps 20), the leg is therefore timed as several
 consecutive blocks of exactly `steps` steps and the median block is reported
 (`timed_blocks` in the JSON line says how many).
 
-Prints ONE JSON line.  `roofline` prices the store kernel against 8 TB/s with
+Prints ONE JSON line.  `value` is the algorithmic bytes of the turbo4 store over `ms_per_step`, the wall clock of the
+timed steps between two synchronisations; `roofline.achieved` is the same bytes over the kernel's own duration.
+`roofline` prices the store kernel against 8 TB/s with
 the algorithmic bytes per launch (322 B per vector for turbo4: 256 B fp16 in,
 64 B codes, 2 B norm); `cpu_baseline` is the NumPy oracle timed on this box's
 host cores over a stated sample of the same workload.
@@ -47,14 +51,32 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 D = 128
-# HBM bytes per launch as recorded in profiles/bench_all_legs_trace_hbm_sq.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
-# this file's run, each scaled by the reading of a 1 GiB device copy): recorded constants, not measured in this run;
-# the JSON line names the profile row next to each figure.
-TRAFFIC_BYTES = {"store4": 169.7e6, "store3": 161.1e6, "decode3": 424.2e6}
-_TRAFFIC_FILE = "profiles/bench_all_legs_trace_hbm_sq.txt"
-TRAFFIC_SOURCE = {"store4": _TRAFFIC_FILE + ", row k_store_kv<4, 4, false> of the HBM traffic table (recorded, not measured in this run)",
-                  "store3": _TRAFFIC_FILE + ", row k_store_kv<3, 3, false> of the HBM traffic table (recorded, not measured in this run)",
-                  "decode3": _TRAFFIC_FILE + ", row k_decode_attn<0, 3, 3, false, true, 1> of the HBM traffic table (recorded, not measured in this run)"}
+# HBM bytes per launch come from the table "HBM traffic per dispatch" of this profile (rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE of this file's run, each scaled by the reading of a 1 GiB device copy).  The table is read at run time;
+# a missing file or row gives "traffic": null.  The JSON line names the row next to each figure.
+TRAFFIC_FILE = "profiles/bench_all_legs_trace_hbm_sq.txt"
+TRAFFIC_ROWS = {"store4": "k_store_kv<4, 4, false>", "store3": "k_store_kv<3, 3, false>",
+                "decode3": "k_decode_attn<0, 3, 3, false, true, 1, false>"}
+
+
+def profile_traffic(key):
+    """(HBM bytes per launch, where the figure comes from) for one of TRAFFIC_ROWS, from the committed profile's
+    traffic table: columns kernel | FETCH KiB | read MB | WRITE KiB | write MB | traffic MB | ..."""
+    kernel = TRAFFIC_ROWS[key]
+    source = f"{TRAFFIC_FILE}, row {kernel} of the HBM traffic table (recorded by the profiler runs named there, not measured in this run)"
+    try:
+        in_table = False
+        for line in open(os.path.join(ROOT, TRAFFIC_FILE)):
+            if line.startswith("== "):
+                in_table = line.startswith("== HBM traffic per dispatch")
+            elif in_table and line.startswith(kernel):
+                cols = line[len(kernel):].split()
+                return float(cols[4]) * 1e6, source
+    except (OSError, ValueError, IndexError):
+        pass
+    return None, f"{TRAFFIC_FILE} has no row {kernel}"
+
+
 METRIC = "KV quantize GB/s + turbo3 decode-attn µs/step @32K ctx, % of HBM roofline"
 
 
@@ -272,7 +294,7 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
     }
 
 
-def decode_leg(torch, tqa, steps, warmup, n_sets=2):
+def decode_leg(torch, tqa, steps, warmup, n_sets=2, small_batches=True):
     B, Hq, Hkv, N, bits = 16, 32, 8, 32768, 3
     kc, vc = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
     sets = []
@@ -320,7 +342,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
 
     # small batches on the same kind of cache: few (batch, kv head) groups, so the context splits must fill the chip
     small = {}
-    for name, b_, n_ in (("B1_ctx32768", 1, N), ("B4_ctx32768", 4, N), ("B256_ctx2048", 256, 2048)):
+    for name, b_, n_ in (("B1_ctx32768", 1, N), ("B4_ctx32768", 4, N), ("B256_ctx2048", 256, 2048)) if small_batches else ():
         per_seq = tqa.packed_bytes(bits, Hkv, n_)
         if b_ * per_seq <= sets[0][1].numel():
             kp_, vp_ = sets[0][1][:b_ * per_seq], sets[0][2][:b_ * per_seq]     # any valid codes do for timing
@@ -363,7 +385,7 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2):
         "us_per_step": us, "wall_us_per_step": wall_ms * 1e3, "n_splits": attn.params.n_splits,
         "timed_blocks": info["timed_blocks"],
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES["decode3"], "traffic_source": TRAFFIC_SOURCE["decode3"],
+                     "traffic": profile_traffic("decode3")[0], "traffic_source": profile_traffic("decode3")[1],
                      "algorithmic_bytes_per_step": algo,
                      "kernel": "k_decode_attn<turbo3,turbo3> (one launch: the last workgroup of a group merges the partials)"},
         "buffer_sets": n_sets,
@@ -516,11 +538,14 @@ def cpu_baseline(bits):
     q = rng.standard_normal((4, D))
     idx, g, _ = O.turbo_encode(k, s1, s2, cent)
     vi, vg, _ = O.turbo_encode(v, s1, s2, cent)
-    t0 = time.perf_counter()
-    kr = O.turbo_decode_rotated(idx, g, cent)
-    vr = O.turbo_decode_rotated(vi, vg, cent)
-    O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
-    dta = time.perf_counter() - t0
+    atimes = []
+    for _ in range(n_samples):
+        t0 = time.perf_counter()
+        kr = O.turbo_decode_rotated(idx, g, cent)
+        vr = O.turbo_decode_rotated(vi, vg, cent)
+        O.decode_attention(O.rotate_fast(q, s1, s2, D), kr, vr, 1 / np.sqrt(D))
+        atimes.append(time.perf_counter() - t0)
+    dta = sorted(atimes)[n_samples // 2]
     return ({"value": algo / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
              "sample": f"NumPy oracle turbo{bits} encode+pack of {passes} x 2 x 32768 fp16 vectors (one head of K and one of V "
                        f"of config 2, {passes} passes = 3/4 of the layer), median of {n_samples} such samples "
@@ -528,7 +553,8 @@ def cpu_baseline(bits):
              "host_cpus": os.cpu_count()},
             {"value": dta * 128 * 1e6, "unit": "µs/step", "cores": blas_threads or 1, "kind": "port",
              "sample": f"NumPy oracle decompress->softmax->PV for 1 of 128 (batch, kv-head) groups at ctx 32768 "
-                       f"({dta * 1e3:.1f} ms), extrapolated x128", "host_cpus": os.cpu_count()})
+                       f"(median of {n_samples} samples: {dta * 1e3:.1f} ms; min {min(atimes) * 1e3:.1f}, max {max(atimes) * 1e3:.1f}), "
+                       f"extrapolated x128", "host_cpus": os.cpu_count()})
 
 
 def boundary_layer_leg(torch, tqa, steps, warmup):
@@ -605,6 +631,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--skip-small-batches", action="store_true",
+                    help="decode leg without its small-batch shapes (counter runs: they launch the same kernel instantiation "
+                         "as config 3, and a per-kernel mean would mix the shapes)")
     ap.add_argument("--legs", default="all",
                     help="comma-separated subset of store4,store3,decode,asym,tile,boundary,maintenance,peaks (profiling runs); "
                          "the JSON line then holds only those legs and is not the benchmark's line")
@@ -649,7 +678,7 @@ def main():
         if "store3" in legs:
             part["turbo3_store"] = store_leg(torch, tqa, 3, args.steps, args.warmup, several_streams=args.several_streams)
         if "decode" in legs:
-            part["decode_attn"] = decode_leg(torch, tqa, args.steps, args.warmup)
+            part["decode_attn"] = decode_leg(torch, tqa, args.steps, args.warmup, small_batches=not args.skip_small_batches)
         if "asym" in legs:
             part["asym_decode_q8k_turbo2v"] = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
         if "tile" in legs:
@@ -664,7 +693,7 @@ def main():
         return
     s4 = store_leg(torch, tqa, 4, args.steps, args.warmup, several_streams=args.several_streams)
     s3 = store_leg(torch, tqa, 3, args.steps, args.warmup, several_streams=args.several_streams)
-    dec = decode_leg(torch, tqa, args.steps, args.warmup)
+    dec = decode_leg(torch, tqa, args.steps, args.warmup, small_batches=not args.skip_small_batches)
     torch.cuda.empty_cache()
     asym = asym_decode_leg(torch, tqa, max(10, args.steps // 4), max(2, args.warmup // 4))
     torch.cuda.empty_cache()
@@ -682,13 +711,16 @@ def main():
     dec["cpu_baseline"] = cpu_attn
 
     line = {
-        "metric": METRIC, "value": s4["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        # value: whole-job throughput over the K timed steps between two synchronisations (wall clock: it contains the gaps
+        # between launches); roofline.achieved: the same bytes over the kernel's own duration (HIP events on the launch stream)
+        "metric": METRIC, "value": s4["algorithmic_bytes_per_launch"] / (s4["ms_per_step"] * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": s4["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": s4["workload"], "global_batch": 2 * 8 * 32768, "io": "fp16 in, 4-bit codes + fp16 norm out",
                    "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": s4["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s4["frac"],
-                     "traffic": TRAFFIC_BYTES["store4"], "traffic_source": TRAFFIC_SOURCE["store4"],
+                     "traffic": profile_traffic("store4")[0], "traffic_source": profile_traffic("store4")[1],
                      "kernel": "k_store_kv<4,4> (K and V of the layer, one launch per step)", "timed_blocks": s4["timed_blocks"],
                      "kernel_us": s4["kernel_us"],
                      "algorithmic_bytes_per_launch": s4["algorithmic_bytes_per_launch"]},
