@@ -303,11 +303,12 @@ def test_decode_attention_many_groups_and_repeated_calls():
 
 @pytest.mark.parametrize("n_splits,sparse", [(32, False), (64, False), (32, True)])
 def test_in_launch_merge_never_leaves_a_row_unwritten(n_splits, sparse):
-    """The split partials of a group are merged inside the launch by the workgroup that finds every flag of its group
-    raised.  Shape of the headline step in small: 32 splits = two workgroups of sixteen wavefronts per group (64: four).
+    """The split partials of a group are merged inside the launch by the workgroup whose increment completes the group's
+    arrival counter.  Shape of the headline step in small: 32 splits = two workgroups of sixteen wavefronts per group (64: four).
     1000 steps back to back on one workspace, the output rows filled with NaN before each: every step must equal the
     first, which is checked against the oracle - a step whose merge found no taker would leave NaN, a merge that ran on
-    stale partials would differ.  The Sparse-V total travels by the same protocol and must be the first step's too."""
+    stale partials would differ.  The Sparse-V total travels through tagged slots of the same workspace and must be the
+    first step's too."""
     tt = L.torch()
     B, Hq, Hkv, N = 4, 8, 2, 64 * n_splits
     k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=n_splits)
