@@ -263,6 +263,37 @@ def test_requantize_stored_cache(pair, kind):
     assert err(rec_s) < err(rec_d) < 1.6 * err(direct)
 
 
+@pytest.mark.parametrize("pair", [(3, 2), (4, 3), (4, 2)])
+def test_requantize_k_rows_whose_code_map_is_their_own(pair):
+    """K rows go through a code -> code table that holds for rows whose sum of squared centroids lies in an interval
+    around 1; other rows build their own table.  Rows drawn from a random subset of the levels (all outer levels, all
+    inner levels, one level only, ...) have sums between 0.2 and 5 and maps that differ from the common one - an outer
+    level that falls into an inner cell once the row is renormalised - and rows with norm zero take the same path.
+    Five blocks: the launch's workgroups serve eight at a time, so a ragged last set is covered too."""
+    sb, db = pair
+    src, dst = tqa.TurboCodec(sb, seed=42), tqa.TurboCodec(db, seed=42)
+    rng = np.random.default_rng(100 * sb + db)
+    tokens = 5 * 128
+    idx = np.zeros((tokens, D), dtype=np.uint8)
+    sums = np.zeros(tokens)
+    for r in range(tokens):
+        levels = np.flatnonzero(rng.random(1 << sb) < 0.4)
+        if levels.size == 0:
+            levels = np.array([rng.integers(1 << sb)])
+        idx[r] = rng.choice(levels, size=D)
+        sums[r] = np.sum(src.centroids[idx[r]] ** 2)
+    assert sums.min() < 0.5 and sums.max() > 3.0
+    g = rng.uniform(0.01, 30.0, tokens).astype(np.float16)
+    g[rng.integers(0, tokens, 7)] = 0
+    packed = L.torch().from_numpy(O.layout_pack(idx, g, sb, "k")).cuda()
+    out = _check_requant(src, dst, packed, 1, tokens, "k")
+    # the maps do differ: many rows do not get the codes a unit-sum row would
+    common = np.searchsorted(O.midpoints(dst.centroids), src.centroids, side="right")
+    i2, _ = O.layout_unpack(np_(out), db, "k")
+    live = g != 0
+    assert np.mean(np.any(i2[:tokens][live] != common[idx][live], axis=1)) > 0.2
+
+
 def test_requantize_rejects_widening():
     a, b = tqa.TurboCodec(2, seed=1), tqa.TurboCodec(3, seed=1)
     buf = L.torch().zeros(tqa.packed_bytes(2, 1, 128), dtype=L.torch().uint8, device="cuda")

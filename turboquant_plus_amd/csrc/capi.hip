@@ -152,6 +152,8 @@ int tq_create(tq_handle **out, const tq_config *cfg) {
     for (int k = 0; k + 1 < nc; ++k) bounds[k] = (cent[k] + cent[k + 1]) / 2.0;
     h->zero_code = 0;
     for (int k = 0; k + 1 < nc; ++k) h->zero_code += bounds[k] < 0.0 ? 1 : 0;
+    for (int k = 0; k < nc && k < 16; ++k) h->centroids_host[k] = cent[k];
+    for (int k = 0; k + 1 < nc && k < 15; ++k) h->bounds_host[k] = bounds[k];
     rc = rc ? rc : upload(&h->centroids64, cent);
     rc = rc ? rc : upload(&h->bounds64, bounds);
     std::vector<double> s1, s2;

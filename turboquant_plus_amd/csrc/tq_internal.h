@@ -52,6 +52,7 @@ struct tq_handle {
     uint32_t s1neg_host[4], s2neg_host[4];  // bit k of word k / 32: s1[k] < 0, s2[k] < 0
     uint32_t s2flip_host[16];               // host copy of s2flip
     float symthr_host[8], sqcoef_host[8];   // host copies of symthr32, sqcoef32 (2^(bits-1) entries used)
+    double centroids_host[16], bounds_host[15];  // host copies of the codebook and its midpoints (n_centroids <= 16)
     int zero_code;         // codebook index of the value 0.0 (#boundaries below 0)
     int symmetric;         // boundaries are sign-symmetric in fp32 (fast quantiser usable)
 };

@@ -3084,6 +3084,206 @@ __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t 
     pack_block<DB, 256>(codes, norms_s, dst + (int64_t)blockIdx.x * block_bytes(DB), a.kind);
 }
 
+// ---- K rows: a lane owns a token -----------------------------------------------------------------
+// A K row is one token's 128 codes, so one lane can requantise a row without exchanging anything.  The decision
+// value of a code is c_src[k] / sqrt(S), S = sum of c_src[code]^2 over the row (the stored norm cancels), so the
+// destination code depends on the source code and on S alone, and for S inside an interval around 1 that the host
+// works out from the two codebooks (RequantKArgs::s_lo, s_hi) the map k -> code is one fixed table T0.  Such rows -
+// all rows of a cache written by this library's store with its own codebooks - go through LDS tables indexed by
+// four 3-bit codes (a quad: 12 contiguous bits of the row) or two 4-bit codes (a byte): the table entry carries the
+// unit's share of S, its share of the destination's sum of squares, and the remapped codes.  A row whose S lies
+// outside the interval (hand-made codebooks, constant rows) or whose norm is zero builds its own table in float64
+// and remaps code by code.  Every source dword holds eight codes in both widths and its remapped codes are
+// contiguous in the destination (16 bits of a 2-bit row, 24 bits of a 3-bit row), so packing is a few shifts.
+struct RequantKArgs {
+    const double *cent_src, *cent_dst, *bounds_dst;  // float64 tables in device memory
+    unsigned long long t0;                          // 4 bits per source code: its destination code for S in (s_lo, s_hi)
+    float s_lo, s_hi;
+    uint32_t n_blocks;
+    float src_sq[16], dst_sq[16];                   // c_src[k]^2, c_dst[k]^2: by value, so that no table build waits for memory
+    uint32_t dst_fix[16];                           // c_dst[k]^2 / fix_unit, rounded: a row's 128 of them add up exactly in 32 bits
+    float fix_unit;
+};
+
+// one workgroup per CU: the tables are built once for the CU's share of the rows
+constexpr int RQK_THREADS = 1024, RQK_BLOCKS = RQK_THREADS / 128;
+template <int SB, int DB>
+__global__ __launch_bounds__(RQK_THREADS) void k_requantize_k(const uint8_t *src, uint8_t *dst, RequantKArgs a) {
+    constexpr int U = SB == 3 ? 4 : 2;   // codes per table unit
+    constexpr int NE = 1 << (SB * U);    // 4096 quads / 256 pairs
+    constexpr int NS = 1 << SB, ND = 1 << DB;
+    constexpr uint32_t SM = NS - 1;
+    // per unit: .x = sum of c_src^2 (fp32 bits); .y = the unit's destination codes in the top byte over the unit's sum of
+    // c_dst[T0]^2 in fixed point (24 bits, RequantKArgs::dst_fix per code, summed exactly in integers)
+    __shared__ uint2 unit_s[NE];
+    __shared__ uint2 pair_s[SB == 3 ? 64 : 1];
+    __shared__ uint2 one_s[NS];          // .x = c_src[k]^2, .y = T0[k] << 24 | fixed-point c_dst[T0[k]]^2
+    __shared__ float cdst2_s[ND];
+    const int tid = threadIdx.x, row = tid & 127;
+    // the first block's row is requested before the tables are built
+    uint32_t w[4 * SB];
+    float g = 0.0f;
+    auto fetch = [&](uint32_t blk) {
+        const uint8_t *sb = src + (int64_t)blk * block_bytes(SB);
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            const uint4 c = stream_load<STREAM_LOAD_OUT>(reinterpret_cast<const uint4 *>(sb + j * 2048 + row * 16));
+            w[4 * j] = c.x; w[4 * j + 1] = c.y; w[4 * j + 2] = c.z; w[4 * j + 3] = c.w;
+        }
+        g = __half2float(reinterpret_cast<const __half *>(sb + block_code_bytes(SB))[row]);
+    };
+    uint32_t blk = RQK_BLOCKS * blockIdx.x + (tid >> 7);
+    if (blk < a.n_blocks) fetch(blk);
+    if (tid < 64) {   // the argument arrays are indexed with constants only (they live in scalar registers)
+        float sq = 0.0f, dq = 0.0f;
+        uint32_t fx = 0;
+#pragma unroll
+        for (int k = 0; k < NS; ++k) sq = tid == k ? a.src_sq[k] : sq;
+#pragma unroll
+        for (int k = 0; k < ND; ++k) dq = tid == k ? a.dst_sq[k] : dq;
+        const uint32_t t = (uint32_t)((a.t0 >> (4 * (tid & 15))) & 15ull);
+#pragma unroll
+        for (int k = 0; k < ND; ++k) fx = t == (uint32_t)k ? a.dst_fix[k] : fx;
+        if (tid < NS) one_s[tid] = make_uint2(__float_as_uint(sq), (t << 24) | fx);
+        if (tid < ND) cdst2_s[tid] = dq;
+    }
+    __syncthreads();
+    // two entries joined: squares and fixed-point sums add, the second entry's codes go above the first's
+    auto join = [](uint2 e0, uint2 e1, int code_bits) {
+        const uint32_t codes = (e0.y >> 24) | ((e1.y >> 24) << code_bits);
+        return make_uint2(__float_as_uint(__uint_as_float(e0.x) + __uint_as_float(e1.x)),
+                          (codes << 24) | ((e0.y & 0xFFFFFFu) + (e1.y & 0xFFFFFFu)));
+    };
+    if constexpr (SB == 3) {
+        if (tid < 64) pair_s[tid] = join(one_s[tid & 7], one_s[tid >> 3], DB);
+        __syncthreads();
+        for (int e = tid; e < NE; e += RQK_THREADS) unit_s[e] = join(pair_s[e & 63], pair_s[e >> 6], 2 * DB);
+    } else if (tid < NE) {
+        unit_s[tid] = join(one_s[tid & 15], one_s[tid >> 4], DB);
+    }
+    __syncthreads();
+
+#pragma unroll 1
+    for (; blk < a.n_blocks;) {
+        // source word j of group q: eight codes, SB bits each (3-bit rows: 24 bits of a dword, or the group's tail)
+        auto src_word = [&](int q, int j) -> uint32_t {
+            if constexpr (SB == 4) return w[4 * j + q];
+            else return j < 3 ? (w[4 * j + q] & 0xFFFFFFu) : tail24(w, q);
+        };
+        uint32_t m[4][4];   // [group][source word]: the eight remapped codes, DB bits each
+        float s1 = 0.0f;
+        uint32_t fix = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t x = src_word(q, j);
+                uint32_t acc = 0;
+#pragma unroll
+                for (int u = 0; u < 8 / U; ++u) {
+                    const uint32_t e = (x >> (SB * U * u)) & (uint32_t)(NE - 1);
+                    const uint2 en = unit_s[e];
+                    s1 += __uint_as_float(en.x);
+                    fix = __umul24(en.y, 1u) + fix;   // the low 24 bits
+                    acc |= (en.y >> 24) << (DB * U * u);
+                }
+                m[q][j] = acc;
+            }
+        float recon = g * sqrtf(s1), s2 = (float)fix * a.fix_unit;
+        const bool table_ok = s1 > a.s_lo && s1 < a.s_hi && recon > 1e-10f;
+        if (__any(!table_ok)) {
+            if (!table_ok) {
+                // this row's own table, float64 as the reference's arithmetic: y = c_src[k] g / recon against the
+                // destination's midpoints, a value on a midpoint taking the higher code
+                const double rec = (double)g * sqrt((double)s1);
+                const double inv = rec > 1e-10 ? 1.0 / rec : 1.0;
+                recon = rec > 1e-10 ? (float)rec : 0.0f;
+                unsigned long long t = 0;
+                for (int k = 0; k < NS; ++k) {
+                    const double y = a.cent_src[k] * (double)g * inv;
+                    unsigned long long c = 0;
+                    for (int b = 0; b < ND - 1; ++b) c += a.bounds_dst[b] <= y ? 1ull : 0ull;
+                    t |= c << (4 * k);
+                }
+                s2 = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t x = src_word(q, j);
+                        uint32_t acc = 0;
+#pragma unroll 1
+                        for (int i = 0; i < 8; ++i) {
+                            const uint32_t c = (uint32_t)(t >> (4 * ((x >> (SB * i)) & SM))) & 15u;
+                            s2 += cdst2_s[c];
+                            acc |= c << (DB * i);
+                        }
+                        m[q][j] = acc;
+                    }
+            }
+        }
+        const float cn = sqrtf(s2);
+        const float gn = cn > 1e-10f ? recon / cn : recon;
+        uint8_t *db = dst + (int64_t)blk * block_bytes(DB);
+        blk += RQK_BLOCKS * gridDim.x;
+        if (blk < a.n_blocks) fetch(blk);   // the codes of this row are in m[][] by now
+        uint32_t d[4 * DB];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (DB == 2) {
+                d[q] = m[q][0] | (m[q][1] << 16);
+                d[4 + q] = m[q][2] | (m[q][3] << 16);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) d[4 * j + q] = m[q][j] | (((m[q][3] >> (8 * j)) & 0xFFu) << 24);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < DB; ++j)
+            stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint4 *>(db + j * 2048 + row * 16),
+                                             make_uint4(d[4 * j], d[4 * j + 1], d[4 * j + 2], d[4 * j + 3]));
+        reinterpret_cast<__half *>(db + block_code_bytes(DB))[row] = __float2half_rn(gn);
+    }
+}
+
+// T0 and the interval of S = sum of c_src[code]^2 for which every source code keeps its T0 destination: the decision
+// value of code k is c_src[k] / r with r = sqrt(S), and it meets the midpoint b at r = c_src[k] / b.  The interval is
+// what lies between the nearest such r below and above 1, shrunk by 1e-5 so that the fp32 sum decides safely.
+static bool requant_k_plan(const tq_handle *hs, const tq_handle *hd, RequantKArgs *a) {
+    const int ns = hs->n_centroids, nd = hd->n_centroids;
+    if (ns > 16 || nd > 16) return false;
+    double r_lo = 0.0, r_hi = 1e30;
+    a->t0 = 0;
+    for (int k = 0; k < ns; ++k) {
+        const double c = hs->centroids_host[k];
+        unsigned long long t = 0;
+        for (int b = 0; b + 1 < nd; ++b) {
+            const double bd = hd->bounds_host[b];
+            t += bd <= c ? 1ull : 0ull;
+            if (bd == 0.0 || c == 0.0 || (bd > 0.0) != (c > 0.0)) continue;
+            const double r = c / bd;
+            if (r <= 1.0 && r > r_lo) r_lo = r;
+            if (r >= 1.0 && r < r_hi) r_hi = r;
+        }
+        a->t0 |= t << (4 * k);
+    }
+    a->s_lo = (float)(r_lo * r_lo * (1.0 + 1e-5));
+    a->s_hi = (float)(r_hi * r_hi * (1.0 - 1e-5));
+    a->cent_src = hs->centroids64; a->cent_dst = hd->centroids64; a->bounds_dst = hd->bounds64;
+    for (int k = 0; k < 16; ++k) {
+        a->src_sq[k] = k < ns ? (float)(hs->centroids_host[k] * hs->centroids_host[k]) : 0.0f;
+        a->dst_sq[k] = k < nd ? (float)(hd->centroids_host[k] * hd->centroids_host[k]) : 0.0f;
+    }
+    // fixed point: the largest square just under 2^22, so that four of them fit the 24 bits of a table entry
+    double top = 0.0;
+    for (int k = 0; k < nd; ++k) top = fmax(top, hd->centroids_host[k] * hd->centroids_host[k]);
+    const double unit = top > 0.0 ? top / 4194300.0 : 1.0;
+    a->fix_unit = (float)unit;
+    for (int k = 0; k < 16; ++k)
+        a->dst_fix[k] = k < nd ? (uint32_t)llround(hd->centroids_host[k] * hd->centroids_host[k] / (double)a->fix_unit) : 0u;
+    return true;
+}
+
 int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                    hipStream_t s) {
     const unsigned grid = (unsigned)(n_seqs * blocks_for(tokens));
@@ -3091,6 +3291,18 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
     RequantArgs a;
     a.cent_src = hs->centroids32; a.cent_dst = hd->centroids32; a.bounds_dst = hd->bounds32; a.kind = kind;
     const int key = hs->bits * 10 + hd->bits;
+    RequantKArgs ka;
+    if (kind == TQ_KIND_K && (key == 32 || key == 43 || key == 42) && requant_k_plan(hs, hd, &ka)) {
+        ka.n_blocks = grid;
+        const unsigned sets = (grid + RQK_BLOCKS - 1) / RQK_BLOCKS;
+        const unsigned wgs = sets < 256u ? sets : 256u;
+        switch (key) {
+        case 32: k_requantize_k<3, 2><<<wgs, RQK_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        case 43: k_requantize_k<4, 3><<<wgs, RQK_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        default: k_requantize_k<4, 2><<<wgs, RQK_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        }
+        return tq_check_launch("requantize (K rows)");
+    }
     switch (key) {
     case 32: k_requantize<3, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
     case 43: k_requantize<4, 3><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
