@@ -361,6 +361,34 @@ def test_fork_blocks_and_requantize_at_config_2_size(bits, kind):
         assert np.allclose(np_(g2).reshape(-1)[rows], want_g, rtol=2e-3)
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_fork_blocks_at_the_least_alignment(bits, kind):
+    """Fork rows that start 2 bytes (4 for 68-byte rows) past a 16-byte boundary and sequences of 77 tokens, whose rows
+    start at every even residue: the K kernels move whole 16-byte pieces where the address allows and 2-byte pieces
+    around them, and must write nothing outside the rows."""
+    tt = L.torch()
+    codec = tqa.TurboCodec(bits, seed=42)
+    n_seqs, tokens, fb = 3, 77, O.fork_block_bytes(bits)
+    x = np.random.default_rng(40 + bits).standard_normal((n_seqs, tokens, D)).astype(np.float16)
+    packed = codec.store(x, kind=kind)
+    idx, g = codec.unpack_codes(packed, n_seqs, tokens, kind=kind)
+    want = O.fork_blocks_pack(np_(idx).reshape(-1, D), np_(g).reshape(-1).astype(np.float16), bits).reshape(-1)
+    off = 4 if bits == 4 else 2
+    raw = tt.full((off + want.size + 64,), 0xA5, dtype=tt.uint8, device="cuda")
+    lib = L.lib()
+    knd = L.KIND_K if kind == "k" else L.KIND_V
+    rc = lib.tq_export_fork_blocks(codec.handle.h, L.ptr(packed), n_seqs, tokens, knd, L.ptr(raw[off:]), L.stream_ptr())
+    assert rc == 0
+    got = np_(raw)
+    assert np.array_equal(got[off:off + want.size], want)
+    assert (got[:off] == 0xA5).all() and (got[off + want.size:] == 0xA5).all()
+    back = tt.full_like(packed, 0x3C)
+    rc = lib.tq_import_fork_blocks(codec.handle.h, L.ptr(raw[off:]), n_seqs, tokens, knd, L.ptr(back), L.stream_ptr())
+    assert rc == 0
+    assert tt.equal(back, packed)
+
+
 def test_fork_blocks_rejects_wrong_width():
     codec = tqa.TurboCodec(3, seed=42)
     with pytest.raises(ValueError):

@@ -3402,6 +3402,175 @@ __global__ __launch_bounds__(256) void k_fork_import(const uint8_t *in, uint8_t 
     pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), kind);
 }
 
+// ---- K rows of the fork layout: a lane owns a token ------------------------------------------------
+// The fork rows of one of this library's K blocks are 128 * FB contiguous bytes.  They move between memory and LDS
+// as 16-byte pieces (the stage keeps the address's low four bits, so a piece is aligned on both sides; what comes
+// before the first and after the last whole piece moves as 2-byte pieces, the alignment every fork buffer has), a
+// lane takes its token's row from the stage as 2- or 4-byte pieces, and the packed block is read or written as
+// 16-byte chunks contiguous over the lanes.  4- and 2-bit rows only change the order of their words; 3-bit rows
+// interleave the fork's two-bit fields and sign bits through byte-indexed tables.
+constexpr int FORK_K_THREADS = 256;   // two blocks per workgroup
+template <int FB>
+__device__ __forceinline__ void fork_stage_copy(uint8_t *stage, uint8_t *mem, int nbytes, bool to_mem, int t, int nt) {
+    const int mis = (int)(reinterpret_cast<uintptr_t>(mem) & 15);
+    uint8_t *lds = stage + mis;                              // same low address bits as the memory side
+    const int head = mis ? (16 - mis < nbytes ? 16 - mis : nbytes) : 0;
+    const int body = (nbytes - head) / 16, tail0 = head + 16 * body;
+    for (int e = t; e < body; e += nt) {
+        uint4 *m = reinterpret_cast<uint4 *>(mem + head) + e, *l = reinterpret_cast<uint4 *>(lds + head) + e;
+        if (to_mem) *m = *l;
+        else *l = *m;
+    }
+    const int edge = (head + (nbytes - tail0)) / 2;          // 2-byte pieces outside the whole 16-byte pieces
+    for (int e = t; e < edge; e += nt) {
+        const int off = 2 * e < head ? 2 * e : tail0 + (2 * e - head);
+        uint16_t *m = reinterpret_cast<uint16_t *>(mem + off), *l = reinterpret_cast<uint16_t *>(lds + off);
+        if (to_mem) *m = *l;
+        else *l = *m;
+    }
+}
+
+template <int BITS, bool TO_FORK>
+__global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed_in, uint8_t *packed_out, const uint8_t *fork_in,
+                                                            uint8_t *fork_out, int64_t tokens, int64_t blocks_per_seq,
+                                                            uint32_t zero_code, uint32_t n_blocks) {
+    constexpr int FB = fork_block_bytes(BITS);
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][TQ_ROWS_PER_BLOCK * FB + 16];
+    __shared__ uint16_t spread2_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of four 2-bit fields -> the fields at a stride of 3
+    __shared__ uint32_t spread1_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of eight sign bits -> bit 3m + 2
+    __shared__ uint16_t gather_s[BITS == 3 && TO_FORK ? 4096 : 1];    // four 3-bit codes -> their low bits (8) | their top bits << 8
+    const int tid = threadIdx.x, half = tid >> 7, row = tid & 127;
+    const uint32_t blk = 2 * blockIdx.x + half;
+    const bool live = blk < n_blocks;
+    const int64_t seq = live ? blk / blocks_per_seq : 0, bis = live ? blk % blocks_per_seq : 0;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK;
+    const int rows = !live ? 0 : tokens - tok0 < TQ_ROWS_PER_BLOCK ? (int)(tokens - tok0) : TQ_ROWS_PER_BLOCK;
+    uint8_t *fork_rows = const_cast<uint8_t *>(TO_FORK ? fork_out : fork_in) + (seq * tokens + tok0) * FB;
+    const int mis = (int)(reinterpret_cast<uintptr_t>(fork_rows) & 15);
+    uint8_t *mine = stage[half] + mis + row * FB;            // this lane's row in the stage
+
+    if constexpr (BITS == 3 && !TO_FORK) {
+        uint32_t a = 0, b = 0;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) a |= ((tid >> (2 * m)) & 3u) << (3 * m);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) b |= ((tid >> m) & 1u) << (3 * m + 2);
+        spread2_s[tid] = (uint16_t)a;
+        spread1_s[tid] = b;
+    }
+    if constexpr (BITS == 3 && TO_FORK) {
+        for (int e = tid; e < 4096; e += FORK_K_THREADS) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const uint32_t c = (e >> (3 * m)) & 7u;
+                lo |= (c & 3u) << (2 * m);
+                hi |= (c >> 2) << m;
+            }
+            gather_s[e] = (uint16_t)(lo | (hi << 8));
+        }
+    }
+    uint32_t w[4 * BITS];
+    uint16_t nrm = 0;
+    if constexpr (TO_FORK) {
+        if (live) {
+            const uint8_t *sb = packed_in + (int64_t)blk * block_bytes(BITS);
+#pragma unroll
+            for (int j = 0; j < BITS; ++j) {
+                const uint4 c = *reinterpret_cast<const uint4 *>(sb + j * 2048 + row * 16);
+                w[4 * j] = c.x; w[4 * j + 1] = c.y; w[4 * j + 2] = c.z; w[4 * j + 3] = c.w;
+            }
+            nrm = reinterpret_cast<const uint16_t *>(sb + block_code_bytes(BITS))[row];
+        }
+        __syncthreads();   // the table
+        if (row < rows) {
+            if constexpr (BITS == 4) {
+                uint32_t *d = reinterpret_cast<uint32_t *>(mine);   // 68-byte rows at a 4-byte aligned address
+                d[0] = nrm;                                         // norm, and 0 in the unused rnorm slot
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) d[1 + 4 * g + j] = w[4 * j + g];
+            } else if constexpr (BITS == 2) {
+                uint16_t *h = reinterpret_cast<uint16_t *>(mine);
+                h[0] = nrm;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        h[1 + 4 * g + 2 * j] = (uint16_t)w[4 * j + g];
+                        h[2 + 4 * g + 2 * j] = (uint16_t)(w[4 * j + g] >> 16);
+                    }
+            } else {
+                uint16_t *h = reinterpret_cast<uint16_t *>(mine);
+                h[0] = nrm;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    uint32_t sg = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t x = j < 3 ? (w[4 * j + g] & 0xFFFFFFu) : tail24(w, g);
+                        const uint32_t e0 = gather_s[x & 0xFFFu], e1 = gather_s[x >> 12];
+                        h[1 + 4 * g + j] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
+                        sg |= ((e0 >> 8) | ((e1 >> 8) << 4)) << (8 * j);
+                    }
+                    h[17 + 2 * g] = (uint16_t)sg;
+                    h[18 + 2 * g] = (uint16_t)(sg >> 16);
+                }
+            }
+        }
+        __syncthreads();
+        fork_stage_copy<FB>(stage[half], fork_rows, rows * FB, true, row, 128);
+    } else {
+        fork_stage_copy<FB>(stage[half], fork_rows, rows * FB, false, row, 128);
+        __syncthreads();
+        if (!live) return;
+        if (row < rows) {
+            if constexpr (BITS == 4) {
+                const uint32_t *d = reinterpret_cast<const uint32_t *>(mine);
+                nrm = (uint16_t)d[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) w[4 * j + g] = d[1 + 4 * g + j];
+            } else if constexpr (BITS == 2) {
+                const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
+                nrm = h[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) w[4 * j + g] = (uint32_t)h[1 + 4 * g + 2 * j] | ((uint32_t)h[2 + 4 * g + 2 * j] << 16);
+            } else {
+                const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
+                nrm = h[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t sg = (uint32_t)h[17 + 2 * g] | ((uint32_t)h[18 + 2 * g] << 16);
+                    uint32_t x[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t q = h[1 + 4 * g + j];
+                        x[j] = (uint32_t)spread2_s[q & 0xFFu] | ((uint32_t)spread2_s[q >> 8] << 12) | spread1_s[(sg >> (8 * j)) & 0xFFu];
+                    }
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) w[4 * j + g] = x[j] | (((x[3] >> (8 * j)) & 0xFFu) << 24);
+                }
+            }
+        } else {
+            // rows past the sequence's end: the code of 0.0 and norm 0, as the store kernels write them
+            const uint32_t pair = zero_code | (zero_code << BITS);
+            const uint32_t fill = BITS == 4 ? pair * 0x01010101u : BITS == 2 ? pair * 0x11111111u : pair * 0x041041u;
+#pragma unroll
+            for (int q = 0; q < 4 * BITS; ++q) w[q] = BITS == 3 ? fill | (((fill >> (8 * (q >> 2))) & 0xFFu) << 24) : fill;
+        }
+        uint8_t *db = packed_out + (int64_t)blk * block_bytes(BITS);
+#pragma unroll
+        for (int j = 0; j < BITS; ++j)
+            *reinterpret_cast<uint4 *>(db + j * 2048 + row * 16) = make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]);
+        reinterpret_cast<uint16_t *>(db + block_code_bytes(BITS))[row] = nrm;
+    }
+}
+
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                     hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
@@ -3410,8 +3579,13 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
     // index of 0.0: number of boundaries below it (a zero vector stores this code in every dim)
     uint32_t zero_code = (uint32_t)(h->n_centroids / 2);
     if (h->zero_code >= 0) zero_code = (uint32_t)h->zero_code;
+    const unsigned kgrid = (grid + 1) / 2;
 #define TQ_FORK(B)                                                                                                        \
-    if (to_fork) k_fork_export<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps);             \
+    if (kind == TQ_KIND_K && to_fork)                                                                                     \
+        k_fork_k<B, true><<<kgrid, FORK_K_THREADS, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
+    else if (kind == TQ_KIND_K)                                                                                           \
+        k_fork_k<B, false><<<kgrid, FORK_K_THREADS, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid); \
+    else if (to_fork) k_fork_export<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps);        \
     else k_fork_import<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps, zero_code)
     switch (h->bits) {
     case 2: TQ_FORK(2); break;
