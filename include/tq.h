@@ -295,6 +295,16 @@ typedef struct tq_attn_params {
                                            /* tokens (INT32_MAX)                              */
     const float *bias_val;                 /* [batch, n_q_heads, bias_entries] values, fp32,  */
                                            /* natural-log units like the dense bias           */
+    int32_t head_dim;                      /* 0 or 128: heads of 128 dims.  256: a head's     */
+                                           /* vector is two 128-value groups, each rotated,   */
+                                           /* quantised and normed by itself (the fork's      */
+                                           /* 128-value blocks, docs/getting-started.md:68):  */
+                                           /* K and V caches are those of 128-dim heads with  */
+                                           /* 2 * tokens rows, row 2 * token + half, written  */
+                                           /* by tq_store(_kv) / tq_append(_kv) from the      */
+                                           /* [tokens, 256] tensor taken as [2 * tokens, 128];*/
+                                           /* q and out are [batch, n_q_heads, 256].  Turbo K */
+                                           /* and V of one code width, dense, no bias         */
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four

@@ -85,6 +85,90 @@ def test_decode_attention_turbo3(N, n_splits):
     np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
 
 
+def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale):
+    """Oracle attention for heads of 256 dims on the GPU-stored codes: the caches hold 2 N rows of 128 per sequence,
+    row 2 t + half; a token's vector is its two rows side by side, each decoded and un-rotated by itself."""
+    G = Hq // Hkv
+    ki, kg = kc.unpack_codes(k_packed, B * Hkv, 2 * N, kind="k")
+    vi, vg = vc.unpack_codes(v_packed, B * Hkv, 2 * N, kind="v")
+    k_rot = O.turbo_decode_rotated(np_(ki), np_(kg).astype(np.float64), kc.centroids).reshape(B * Hkv, N, 2 * D)
+    v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids).reshape(B * Hkv, N, 2 * D)
+    q_rot = O.rotate_fast(q.astype(np.float64).reshape(B, Hq, 2, D), kc.signs1, kc.signs2, D).reshape(B, Hq, 2 * D)
+    out = np.zeros((B, Hq, 2 * D))
+    for b in range(B):
+        for h in range(Hkv):
+            g = b * Hkv + h
+            o, _, _ = O.decode_attention(q_rot[b, h * G:(h + 1) * G], k_rot[g], v_rot[g], scale)
+            o = O.rotate_fast(o.reshape(G, 2, D), vc.signs1, vc.signs2, D, transpose=True)
+            out[b, h * G:(h + 1) * G] = o.reshape(G, 2 * D)
+    return out
+
+
+@pytest.mark.parametrize("bits", [3, 4, 2])
+@pytest.mark.parametrize("N,n_splits,Hq", [(32, 1, 8), (64, 1, 8), (100, 1, 8), (1000, 3, 8), (4096 + 37, 8, 8), (2048, 16, 6),
+                                           (1536, 32, 16), (77, 2, 2)])
+def test_decode_attention_head_dim_256(bits, N, n_splits, Hq):
+    """Heads of 256 dims: two 128-value groups per vector, each with its own rotation, codes and norm; the caches are
+    those of 128-dim heads with two rows per token.  Groups of 4, 3, 8 (two passes) and 1 query heads per KV head,
+    ragged last tiles, one to 32 splits."""
+    B, Hkv = 2, 2
+    rng = np.random.default_rng(1000 * bits + N)
+    k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    k[:, :, 128:] *= 2.0                       # the halves have norms of their own
+    v[:, :, :128] *= 0.5
+    kc, vc = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
+    kp = kc.store(tqa.rows_of_256(k), kind="k")
+    vp = vc.store(tqa.rows_of_256(v), kind="v")
+    q = rng.standard_normal((B, Hq, 2 * D)).astype(np.float16)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256)
+    out = np_(attn(q, kp, vp))
+    assert out.shape == (B, Hq, 2 * D)
+    ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D))
+    assert_close(out, ref)
+
+
+def test_decode_attention_head_dim_256_grows_by_append():
+    """A 256-dim cache that grows in place: prefill and appends work on rows (two per token, positions and capacity
+    counted in rows), attention on tokens."""
+    B, Hq, Hkv, cap, N0 = 2, 8, 2, 512, 200
+    rng = np.random.default_rng(12)
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    k = rng.standard_normal((B * Hkv, N0 + 3, 2 * D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N0 + 3, 2 * D)).astype(np.float16)
+    tt = L.torch()
+    ck = tt.zeros(tqa.packed_bytes(3, B * Hkv, 2 * cap), dtype=tt.uint8, device="cuda")
+    cv = tt.zeros_like(ck)
+    kc.append_kv(vc, tqa.rows_of_256(k[:, :N0]), tqa.rows_of_256(v[:, :N0]), ck, cv, 0, 2 * cap)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N0, n_splits=4, capacity=cap, head_dim=256)
+    for step in range(3):
+        n = N0 + step
+        kc.append_kv(vc, tqa.rows_of_256(k[:, n:n + 1]), tqa.rows_of_256(v[:, n:n + 1]), ck, cv, 2 * n, 2 * cap)
+        attn.set_tokens(n + 1)
+        q = rng.standard_normal((B, Hq, 2 * D)).astype(np.float16)
+        out = np_(attn(q, ck, cv)).copy()
+        kp = kc.store(tqa.rows_of_256(np.ascontiguousarray(k[:, :n + 1])), kind="k")
+        vp = vc.store(tqa.rows_of_256(np.ascontiguousarray(v[:, :n + 1])), kind="v")
+        want = np_(tqa.DecodeAttention(kc, vc, B, Hq, Hkv, n + 1, n_splits=4, head_dim=256)(q, kp, vp))
+        np.testing.assert_allclose(out, want, rtol=0, atol=2e-3 * np.abs(want).max())
+
+
+def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
+    B, Hq, Hkv, N = 1, 4, 1, 128
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    tt = L.torch()
+    buf = tt.zeros(tqa.packed_bytes(3, B * Hkv, 2 * N), dtype=tt.uint8, device="cuda")
+    q = tt.zeros((B, Hq, 256), dtype=tt.float16, device="cuda")
+    with pytest.raises(NotImplementedError):
+        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256, sparse_v_tau=1e-3)(q, buf, buf)
+    with pytest.raises(NotImplementedError):
+        tqa.DecodeAttention(kc, tqa.TurboCodec(2, seed=542), B, Hq, Hkv, N, head_dim=256)(q, buf, buf)
+    with pytest.raises(NotImplementedError):
+        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf, bias=tt.zeros((B, Hq, N), device="cuda"))
+    with pytest.raises(ValueError):
+        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=64)
+
+
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("n_splits", [16, 3])
 def test_decode_attention_with_unequal_codebooks_of_one_width(bits, n_splits):

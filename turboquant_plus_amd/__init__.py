@@ -12,10 +12,10 @@ from .kv_cache import KVCacheCompressor, CompressedKVCache
 from .outlier import OutlierTurboQuant, OutlierCompressedVector
 from .policy import LayerFormat, LayerKV, layer_formats, effective_bits
 from .turbo import (TurboCodec, DecodeAttention, q8_0_store, q8_0_unpack, q8_0_append, packed_bytes, PRODUCTION_CENTROIDS,
-                    sparse_bias_from_dense)
+                    sparse_bias_from_dense, rows_of_256)
 
 __all__ = ["PolarQuant", "QJL", "TurboQuant", "TurboQuantMSE", "CompressedVector", "KVCacheCompressor",
            "OutlierTurboQuant", "OutlierCompressedVector",
            "CompressedKVCache", "TurboCodec", "DecodeAttention", "q8_0_store", "q8_0_unpack", "q8_0_append", "packed_bytes",
-           "PRODUCTION_CENTROIDS", "sparse_bias_from_dense", "LayerFormat", "LayerKV", "layer_formats",
+           "PRODUCTION_CENTROIDS", "sparse_bias_from_dense", "rows_of_256", "LayerFormat", "LayerKV", "layer_formats",
            "effective_bits"]

@@ -34,7 +34,8 @@ class TQAttnParams(C.Structure):
     _fields_ = [("batch", C.c_int32), ("n_q_heads", C.c_int32), ("n_kv_heads", C.c_int32), ("tokens", C.c_int64),
                 ("capacity", C.c_int64), ("n_splits", C.c_int32), ("k_format", C.c_int32), ("v_format", C.c_int32),
                 ("scale", C.c_float), ("sparse_v_tau", C.c_float), ("tokens_dev", C.c_void_p),
-                ("bias_entries", C.c_int32), ("bias_pos", C.c_void_p), ("bias_val", C.c_void_p)]
+                ("bias_entries", C.c_int32), ("bias_pos", C.c_void_p), ("bias_val", C.c_void_p),
+                ("head_dim", C.c_int32)]
 
 
 _P, _I, _L, _D = C.c_void_p, C.c_int, C.c_int64, C.c_double

@@ -214,6 +214,7 @@ struct AttnArgs {
     const int64_t *tokens_dev;  // NULL, or where the step's context length is read from (<= tokens, which then is the maximum)
     int n_groups, n_splits, tiles_per_split, n_tiles;
     int q_group, head_off;  // query heads per KV head; first of the (up to) four heads this launch works on
+    int d256;               // heads of 256 dims: a token is two 128-value rows (2 token + half) of the K and V caches
     float tau;
 };
 
@@ -230,6 +231,37 @@ __device__ __forceinline__ void qk_turbo(std::integer_sequence<int, G...>, const
          const half4_t kv = quad_values<BITS>(kw, lut, G);
 #pragma unroll
          for (int hg = 0; hg < HG; ++hg) acc[hg][G & 3] = mfma4_bcast<(G & 15)>(qa[hg][G >> 4], kv, acc[hg][G & 3]);
+     }()),
+     ...);
+}
+
+// Heads of 256 dims: the lower half of the wavefront holds the rows of the tile's 32 tokens' first 128 dims, the
+// upper half the rows of their second 128 dims, and each half takes its half of the query from its own blocks
+// (A broadcast inside a half-wavefront, block G % 8; a lane keeps four dim groups)
+template <int BITS, int... G>
+__device__ __forceinline__ void qk_turbo_d256(std::integer_sequence<int, G...>, const uint32_t (&kw)[4 * BITS],
+                                              const char *lut, const half4_t (&qa4)[4], float4_t (&acc)[4]) {
+    (([&] {
+         const half4_t kv = quad_values<BITS>(kw, lut, G);
+         acc[G & 3] = mfma4_bcast8<(G & 7)>(qa4[G >> 3], kv, acc[G & 3]);
+     }()),
+     ...);
+}
+
+// ... and V rows whose 64 "tokens" are (token, half) pairs: quad T holds the rows of tokens 2T, 2T+1 in the order
+// (2T, 0), (2T, 1), (2T+1, 0), (2T+1, 1).  The weights of tokens 4b..4b+3 sit in block b, so quad T takes them from
+// block T / 2, with zeros in the places of the other half: one look-up feeds the output's two halves.
+template <int BITS, int... T>
+__device__ __forceinline__ void pv_all_d256(std::integer_sequence<int, T...>, const uint32_t (&vw)[4 * BITS], const char *lut,
+                                            const half4_t (&pv_even)[2], const half4_t (&pv_odd)[2], float4_t (&acc_o)[2][2][2]) {
+    (([&] {
+         const half4_t v0 = quad_values<BITS>(vw, lut, 2 * T), v1 = quad_values<BITS>(vw, lut, 2 * T + 1);
+#pragma unroll
+         for (int dh = 0; dh < 2; ++dh) {
+             const half4_t w = (T & 1) ? pv_odd[dh] : pv_even[dh];
+             acc_o[dh][0][T & 1] = mfma4_bcast<(T >> 1)>(w, v0, acc_o[dh][0][T & 1]);
+             acc_o[dh][1][T & 1] = mfma4_bcast<(T >> 1)>(w, v1, acc_o[dh][1][T & 1]);
+         }
      }()),
      ...);
 }
@@ -284,7 +316,8 @@ __device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, cons
 // per-tile side data of the V rows: turbo = the fp16 norms of this lane's four tokens; q8_0-style = the fp16 scales
 // [2 * dim half + swapped]: of this lane's four tokens (0) and of the four tokens of lane ^ 32 (1), for the 32-dim
 // block that this lane's dims of that dim half lie in
-template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 1]; };
+// heads of 256 dims: the eight fp16 norms of the rows of this lane's four tokens (v[0], v[1])
+template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 2]; };
 
 constexpr unsigned long long ARRIVAL_COUNT_MASK = 0xFFFFFFull;  // workgroups of a group (the tag of the call sits above)
 constexpr float Q8V_PRESCALE = 64.0f;  // keeps weight * scale products out of fp16's subnormals; 65504 / 64 > any scale
@@ -325,8 +358,11 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
     const float *ml0 = a.part_ml + (int64_t)group * n_parts * ML;
     const float *po0 = a.part_o + (int64_t)group * n_parts * PO;
     for (int head = wave; head < NH; head += n_waves) {
-        if (a.head_off + head >= a.q_group) continue;  // a repeated head of a group with fewer than four left
-        const int64_t r_out = (int64_t)group * a.q_group + a.head_off + head;
+        // heads of 256 dims (HG = 2): partial row 4 dh + i is dims 128 dh .. 128 dh + 127 of head i
+        const int hq = a.d256 ? (head & 3) : head;
+        if (a.head_off + hq >= a.q_group) continue;  // a repeated head of a group with fewer than four left
+        const int64_t r_out = a.d256 ? 2 * ((int64_t)group * a.q_group + a.head_off + hq) + (head >> 2)
+                                     : (int64_t)group * a.q_group + a.head_off + head;
         float M = -INFINITY, L = 0.0f, o0 = 0.0f, o1 = 0.0f;
         if (n_parts <= 4) {
             float2 ml[4], v[4];
@@ -423,8 +459,13 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 
 // SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
 // registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
-template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS>
+// D256: heads of 256 dims (turbo K and V, dense, no bias).  A token is rows 2 token and 2 token + 1 of caches that are
+// otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
+// then the output's two halves of one set of four heads: one softmax, two accumulator sets.
+template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
 __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_decode_attn(AttnArgs a) {
+    static_assert(!D256 || (HG == 2 && KFMT == KFMT_TURBO && VBITS != 8 && !SPARSE && !SBIAS), "256-dim heads: turbo K and V, dense");
+    constexpr int HQ = D256 ? 1 : HG;   // sets of four heads whose logits and softmax state the wavefront keeps
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
     constexpr int VBLOCK = VBITS == 8 ? TQ_ROWS_PER_BLOCK * 136 : TQ_ROWS_PER_BLOCK * (16 * VBITS + 2);
@@ -452,13 +493,17 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     if (a.tokens_dev) {
         const int64_t t = *a.tokens_dev;
         tokens_now = __builtin_amdgcn_readfirstlane((int)(t < 0 ? 0 : (t < a.tokens ? t : a.tokens)));
-        n_tiles = (tokens_now + 63) >> 6;
+        n_tiles = ((D256 ? 2 : 1) * tokens_now + 63) >> 6;
         tiles_per_split = (n_tiles + a.n_splits - 1) / a.n_splits;
     }
+    const int rows_now = (D256 ? 2 : 1) * tokens_now;   // rows of the caches that hold the context
     const int t_begin = split * tiles_per_split;
     const int t_end = min(t_begin + tiles_per_split, n_tiles);
     const int b4 = lane & ~3;  // 4 * block index
     const int j = lane & 3;    // query head of the logits this lane holds; sub-row for V
+    // K row of the tile that this lane owns, and the tile row of element i of its logits (e4 + es * i)
+    const int krow = D256 ? 2 * (lane & 31) + (lane >> 5) : lane;
+    const int e4 = D256 ? 2 * (b4 & 31) : b4, es = D256 ? 2 : 1;
 
     const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
     const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
@@ -478,7 +523,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     // K: this lane's token's fp16 norm (turbo) or its four fp16 block scales (q8_0-style)
     auto load_knorm = [&](int tile) -> uint2 {
         const uint8_t *kb = kbase + (int64_t)(tile >> 1) * KBLOCK;
-        const int r = (tile & 1) * 64 + lane;
+        const int r = (tile & 1) * 64 + krow;
         if constexpr (KFMT == KFMT_TURBO)
             return make_uint2(reinterpret_cast<const uint16_t *>(kb + TQ_ROWS_PER_BLOCK * 16 * KBITS)[r], 0u);
         else
@@ -494,8 +539,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             for (int e = 0; e < 4; ++e)
                 r.v[e] = *reinterpret_cast<const uint2 *>(side + 2 * ((((tile & 1) * 4 + 2 * (e >> 1) + bh) * 64) +
                                                                       (e & 1 ? b4 ^ 32 : b4)));
+        } else if constexpr (D256) {
+            const uint4 n8 = *reinterpret_cast<const uint4 *>(side + 2 * ((tile & 1) * 64 + e4));
+            r.v[0] = make_uint2(n8.x, n8.y);
+            r.v[1] = make_uint2(n8.z, n8.w);
         } else {
             r.v[0] = *reinterpret_cast<const uint2 *>(side + 2 * ((tile & 1) * 64 + b4));
+            r.v[1] = make_uint2(0u, 0u);
         }
         return r;
     };
@@ -507,7 +557,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     if (tile < t_end) {
         const int row0 = (tile & 1) * 64 + lane;
         const uint8_t *kb = kbase + (int64_t)(tile >> 1) * KBLOCK;
-        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, row0, kw);
+        if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, (tile & 1) * 64 + krow, kw);
         else load_row<8>(kb, row0, kw);
         kn = load_knorm(tile);
         load_row<VBITS>(vbase + (int64_t)(tile >> 1) * VBLOCK, row0, vw);
@@ -533,7 +583,8 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     for (int h = wave; h < 4 * HG; h += n_waves) {
         _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + h * 128;
         // heads past the group's last one repeat it (their results are not written)
-        const int64_t e = ((int64_t)group * a.q_group + min(a.head_off + h, a.q_group - 1)) * 128 + 2 * lane;
+        const int64_t e = D256 ? ((int64_t)group * a.q_group + min(a.head_off + (h & 3), a.q_group - 1)) * 256 + 128 * (h >> 2) + 2 * lane
+                               : ((int64_t)group * a.q_group + min(a.head_off + h, a.q_group - 1)) * 128 + 2 * lane;
         float x0, x1;
         if (a.q_dtype == TQ_F16) {
             const __half *qp = reinterpret_cast<const __half *>(a.q);
@@ -569,11 +620,17 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     }
     __syncthreads();
     half4_t qa[HG][2];
+    half4_t qa4[4];   // 256-dim heads: dim groups b, b + 8, b + 16, b + 24 of this half-wavefront's half of the query
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) {
         const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + (4 * hg + j) * 128);
         qa[hg][0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
         qa[hg][1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
+    }
+    if constexpr (D256) {
+        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + (4 * (lane >> 5) + j) * 128);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) qa4[k] = __builtin_bit_cast(half4_t, qp[((lane >> 2) & 7) + 8 * k]);
     }
     __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
     if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
@@ -670,8 +727,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         const int tile_next = tile + 1;
         const int tile_n = min(tile_next, t_end - 1);
         const int row_n = tile_next < t_end ? (tile_n & 1) * 64 + lane : 0;  // past the split: every lane the same row
+        const int krow_n = tile_next < t_end ? (tile_n & 1) * 64 + krow : 0;
         const VSide<VBITS> gvu_next = load_vnorm(tile_n);
-        const int n_valid = tokens_now - tile * 64;   // >= 64 except in the sequence's last tile
+        const int n_valid = rows_now - tile * 64;   // >= 64 except in the sequence's last tile
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
         float bias4[HG][4];
 #pragma unroll
@@ -708,7 +766,16 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         for (int hg = 0; hg < HG; ++hg)
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[hg][c] = float4_t{0.f, 0.f, 0.f, 0.f};
-        if constexpr (KFMT == KFMT_TURBO) {
+        if constexpr (D256) {
+            // each half-wavefront: its half of the query against its rows; a token's two halves meet across lane ^ 32
+            qk_turbo_d256<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa4, acc[0]);
+            const float gk_own = __half2float(__ushort_as_half((unsigned short)kn.x));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float part = ((acc[0][0][i] + acc[0][1][i]) + (acc[0][2][i] + acc[0][3][i])) * gk_own;
+                sc[0][i] = part + xor_lane<32>(part);
+            }
+        } else if constexpr (KFMT == KFMT_TURBO) {
             qk_turbo<KBITS, HG>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa, acc);
             const float gk_own = __half2float(__ushort_as_half((unsigned short)kn.x));
 #pragma unroll
@@ -729,7 +796,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         }
         {   // kw is dead now: fetch the next tile's K row into it
             const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
-            if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, row_n, kw);
+            if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, krow_n, kw);
             else load_row<8>(kbn, row_n, kw);
             kn = load_knorm(tile_n);
         }
@@ -745,7 +812,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             }
         }
 #pragma unroll
-        for (int hg = 0; hg < HG; ++hg) {
+        for (int hg = 0; hg < HQ; ++hg) {
             quad_transpose(sc[hg], lane);
             float s[4];
 #pragma unroll
@@ -753,7 +820,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             if (n_valid < 64) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (b4 + i >= n_valid) s[i] = -INFINITY;
+                    if (e4 + es * i >= n_valid) s[i] = -INFINITY;
             }
             const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
             const float m_new = fmaxf(m_run[hg], mx);
@@ -764,11 +831,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
                 // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
                 const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
 #pragma unroll
+                for (int ho = (D256 ? 0 : hg); ho < (D256 ? 2 : hg + 1); ++ho)   // 256-dim heads: both halves of the output
+#pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    acc_o[hg][c >> 1][c & 1][0] *= c0;
-                    acc_o[hg][c >> 1][c & 1][1] *= c1;
-                    acc_o[hg][c >> 1][c & 1][2] *= c2;
-                    acc_o[hg][c >> 1][c & 1][3] *= c3;
+                    acc_o[ho][c >> 1][c & 1][0] *= c0;
+                    acc_o[ho][c >> 1][c & 1][1] *= c1;
+                    acc_o[ho][c >> 1][c & 1][2] *= c2;
+                    acc_o[ho][c >> 1][c & 1][3] *= c3;
                 }
                 m_run[hg] = m_new;
             }
@@ -832,6 +901,22 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
                 }
             }
             pv_all_q8<HG>(std::make_integer_sequence<int, 16>{}, vw, a_lo, a_hi, acc_o);
+        } else if constexpr (D256) {
+            // norms of rows 8b..8b+7 = (token 4b + i, half h) at 2 i + h
+            const uint32_t nw[4] = {gvu.v[0].x, gvu.v[0].y, gvu.v[1].x, gvu.v[1].y};
+            half4_t pv_even[2], pv_odd[2];
+#pragma unroll
+            for (int dh = 0; dh < 2; ++dh) {
+                float g[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) g[i] = __half2float(__ushort_as_half((unsigned short)(dh ? nw[i] >> 16 : nw[i] & 0xffff)));
+                const _Float16 z = (_Float16)0.0f;
+                const _Float16 w0 = (_Float16)(p[0][0] * g[0]), w1 = (_Float16)(p[0][1] * g[1]);
+                const _Float16 w2 = (_Float16)(p[0][2] * g[2]), w3 = (_Float16)(p[0][3] * g[3]);
+                pv_even[dh] = dh ? half4_t{z, w0, z, w1} : half4_t{w0, z, w1, z};
+                pv_odd[dh] = dh ? half4_t{z, w2, z, w3} : half4_t{w2, z, w3, z};
+            }
+            pv_all_d256<VBITS>(std::make_integer_sequence<int, 16>{}, vw, vlut_b, pv_even, pv_odd, acc_o);
         } else {
             const float g0 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x & 0xffff)));
             const float g1 = __half2float(__ushort_as_half((unsigned short)(gvu.v[0].x >> 16)));
@@ -866,6 +951,12 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     float l_tot[HG];
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) l_tot[hg] = sum_over_blocks(l_run[hg]);
+    if constexpr (D256) {
+        // both half-wavefronts added the same 32 weights; the second accumulator set shares the softmax state
+        l_tot[0] *= 0.5f;
+        l_tot[1] = l_tot[0];
+        m_run[1] = m_run[0];
+    }
     if (n_waves == 1) {
 #pragma unroll
         for (int hg = 0; hg < HG; ++hg) {
@@ -1047,7 +1138,8 @@ struct AttnPlan {
 };
 AttnPlan attn_plan(const tq_attn_params *p) {
     AttnPlan pl;
-    pl.hg = p->n_q_heads / p->n_kv_heads > 4 ? 2 : 1;
+    // 256-dim heads run as two accumulator sets (the output's halves) of one set of four heads
+    pl.hg = p->head_dim == 256 || p->n_q_heads / p->n_kv_heads > 4 ? 2 : 1;
     pl.wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
     while (p->n_splits % pl.wpw) pl.wpw >>= 1;
     pl.n_parts = p->n_splits / pl.wpw;
@@ -1082,6 +1174,17 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     }
     const int64_t rows = (int64_t)p->batch * p->n_q_heads;
     const int groups = p->batch * p->n_kv_heads;
+    const bool d256 = p->head_dim == 256;
+    if (p->head_dim != 0 && p->head_dim != 128 && p->head_dim != 256) {
+        tq_set_error("tq_decode_attention: head_dim %d (128 or 256)", (int)p->head_dim);
+        return TQ_ERR_UNSUPPORTED;
+    }
+    if (d256 && (p->k_format != TQ_KFMT_TURBO || p->v_format != TQ_KFMT_TURBO || !hk || !hv || hk->bits != hv->bits ||
+                 p->sparse_v_tau > 0.0f || bias || p->bias_entries)) {
+        tq_set_error("tq_decode_attention: head_dim 256 takes turbo K and V of one code width, dense, without bias");
+        return TQ_ERR_UNSUPPORTED;
+    }
+    const int64_t cache_rows = (d256 ? 2 : 1) * p->tokens;   // a 256-dim token is two rows of the caches
     float *part_o = reinterpret_cast<float *>((char *)ws + w.part_o);
     float *part_ml = reinterpret_cast<float *>((char *)ws + w.part_ml);
     const bool turbo_k = p->k_format == TQ_KFMT_TURBO;
@@ -1118,7 +1221,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.part_o = part_o;
     a.part_ml = part_ml;
     a.skip_slots = reinterpret_cast<unsigned long long *>((char *)ws + w.skip_slots);
-    if (p->tokens >= ((int64_t)1 << 31)) {
+    if (cache_rows >= ((int64_t)1 << 31)) {
         tq_set_error("tq_decode_attention: tokens %lld beyond 2^31 - 1", (long long)p->tokens);
         return TQ_ERR_UNSUPPORTED;
     }
@@ -1128,10 +1231,11 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: the Sparse-V count is not kept for a context length read from memory (tokens_dev)");
         return TQ_ERR_UNSUPPORTED;
     }
-    a.blocks_per_seq = ((p->capacity > 0 ? p->capacity : p->tokens) + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
+    a.blocks_per_seq = ((d256 ? 2 : 1) * (p->capacity > 0 ? p->capacity : p->tokens) + TQ_ROWS_PER_BLOCK - 1) / TQ_ROWS_PER_BLOCK;
     a.n_groups = groups;
     a.n_splits = p->n_splits;
-    a.n_tiles = (int)((p->tokens + 63) / 64);
+    a.n_tiles = (int)((cache_rows + 63) / 64);
+    a.d256 = d256 ? 1 : 0;
     a.tiles_per_split = (a.n_tiles + p->n_splits - 1) / p->n_splits;
     a.tau = p->sparse_v_tau;
     const bool sparse = p->sparse_v_tau > 0.0f;
@@ -1154,7 +1258,8 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     // ceil(G / 8) passes over the same K/V; a last pass with fewer heads than it has rows repeats the group's
     // last head and does not write the repeats.
     a.q_group = p->n_q_heads / p->n_kv_heads;
-    if ((a.q_group + 4 * hg - 1) / (4 * hg) > MAX_PASSES) {
+    const int heads_per_pass = d256 ? 4 : 4 * hg;
+    if ((a.q_group + heads_per_pass - 1) / heads_per_pass > MAX_PASSES) {
         tq_set_error("tq_decode_attention: %d query heads per KV head (at most %d)", a.q_group, 4 * MAX_PASSES);
         return TQ_ERR_UNSUPPORTED;
     }
@@ -1168,9 +1273,21 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     a.total_pairs = total_pairs;
     (void)n_parts;
     (void)kb;
-    for (a.head_off = 0; a.head_off < a.q_group; a.head_off += 4 * hg) {
-        a.pass = a.head_off / (4 * hg);
+    for (a.head_off = 0; a.head_off < a.q_group; a.head_off += heads_per_pass) {
+        a.pass = a.head_off / heads_per_pass;
         a.nonce = next_nonce();
+        if (d256) {
+#define TQ_ATTN_256(B)                                                                                                  \
+    if (share) k_decode_attn<KFMT_TURBO, B, B, false, true, 2, false, true><<<grid, wg, merge_bytes, s>>>(a);           \
+    else k_decode_attn<KFMT_TURBO, B, B, false, false, 2, false, true><<<grid, wg, merge_bytes, s>>>(a)
+            if (kb == 3) { TQ_ATTN_256(3); }
+            else if (kb == 4) { TQ_ATTN_256(4); }
+            else { TQ_ATTN_256(2); }
+#undef TQ_ATTN_256
+            rc = tq_check_launch("decode_attn (256-dim heads)");
+            if (rc) return rc;
+            continue;
+        }
 #define TQ_ATTN_ONE(KF, KB, VB, SP, SH)                                            \
     {                                                                             \
         if (hg == 2 && a.sbias_n) k_decode_attn<KF, KB, VB, SP, SH, 2, true><<<grid, wg, merge_bytes, s>>>(a);   \

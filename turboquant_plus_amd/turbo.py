@@ -414,24 +414,31 @@ class DecodeAttention:
 
     def __init__(self, k_codec: TurboCodec | None, v_codec: TurboCodec | None, batch: int, n_q_heads: int, n_kv_heads: int,
                  tokens: int, *, n_splits: int | None = None, scale: float | None = None, sparse_v_tau: float = 0.0,
-                 capacity: int = 0, tokens_on_device=None, poison_output: bool | None = None):
+                 capacity: int = 0, tokens_on_device=None, poison_output: bool | None = None, head_dim: int = HEAD_DIM):
         """tokens_on_device: an int64 device tensor (one element) that holds the context length when a call runs;
         `tokens` is then the largest length it may take.  One captured launch (HIP graph) can so be replayed while
         the cache grows; Sparse V is not available in this mode.
         poison_output (default: on when the environment holds TQ_POISON_OUTPUT=1): fill the output rows with NaN
         before every call, so that a row the launch did not write - the split partials are merged inside the launch by
         whichever workgroup of a group finishes last - shows as NaN instead of the previous call's values.  A debug
-        aid: one small fill kernel per call."""
+        aid: one small fill kernel per call.
+        head_dim: 128, or 256 - a head's vector as two 128-value groups, each rotated, quantised and normed by itself
+        (the fork's 128-value blocks, docs/getting-started.md:68).  The caches are then those of 128-dim heads with
+        two rows per token: rows_of_256(x) gives the [n, 2 * tokens, 128] view that store / append / load take, and
+        `tokens`, `capacity`, `pos` of those calls count rows (2 * tokens).  Turbo K and V of one width, dense."""
         tt = L.torch()
         dev = L.require_gpu()
         self.k_codec, self.v_codec = k_codec, v_codec
+        if head_dim not in (HEAD_DIM, 2 * HEAD_DIM):
+            raise ValueError(f"head_dim {head_dim}: the packed-cache kernels take 128 or 256")
+        self.head_dim = head_dim
         if n_splits is None:
-            n_splits = default_splits(batch * n_kv_heads, tokens)
+            n_splits = default_splits(batch * n_kv_heads, tokens * (head_dim // HEAD_DIM))
         self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
                                      capacity=capacity, n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
                                      v_format=L.KFMT_TURBO if v_codec is not None else L.KFMT_Q8_0,
-                                     scale=(1.0 / math.sqrt(HEAD_DIM)) if scale is None else scale,
-                                     sparse_v_tau=sparse_v_tau)
+                                     scale=(1.0 / math.sqrt(head_dim)) if scale is None else scale,
+                                     sparse_v_tau=sparse_v_tau, head_dim=head_dim)
         self.tokens_on_device = tokens_on_device   # kept alive with the object
         if tokens_on_device is not None:
             if tokens_on_device.dtype != tt.int64 or not tokens_on_device.is_cuda or tokens_on_device.numel() != 1:
@@ -444,7 +451,7 @@ class DecodeAttention:
             L.check(L.ERR_ARG)
         self.workspace = tt.empty(int(nbytes), dtype=tt.uint8, device=dev)
         self.skip = tt.zeros(2, dtype=tt.int64, device=dev)
-        self.out = tt.empty((batch, n_q_heads, HEAD_DIM), dtype=tt.float32, device=dev)
+        self.out = tt.empty((batch, n_q_heads, head_dim), dtype=tt.float32, device=dev)
         self.poison_output = os.environ.get("TQ_POISON_OUTPUT", "0") == "1" if poison_output is None else bool(poison_output)
 
     def __call__(self, q, k_packed, v_packed, bias=None, sparse_bias=None):
@@ -489,6 +496,17 @@ class DecodeAttention:
     def skip_rate(self) -> float:
         s = self.skip.cpu().numpy()
         return float(s[0]) / float(s[1]) if s[1] else 0.0
+
+
+def rows_of_256(x):
+    """[n, tokens, 256] -> the [n, 2 * tokens, 128] view of the same memory: row 2 * token + half holds dims
+    128 * half .. 128 * half + 127 of the token, the unit that the store, append and load calls work on for heads of
+    256 dims (no copy; x must be contiguous)."""
+    if x.shape[-1] != 2 * HEAD_DIM:
+        raise ValueError(f"last dimension {x.shape[-1]}, expected {2 * HEAD_DIM}")
+    if hasattr(x, "is_contiguous") and not x.is_contiguous():
+        raise ValueError("rows_of_256 needs a contiguous tensor")
+    return x.reshape(*x.shape[:-2], 2 * x.shape[-2], HEAD_DIM)
 
 
 def sparse_bias_from_dense(bias, max_entries: int | None = None):
