@@ -327,6 +327,12 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2, small_batches=True):
     attn8 = tqa.DecodeAttention(kc, vc, B, 2 * Hq, Hkv, N)
     _, ev8_ms = time_steps(torch, lambda i: attn8(q64, sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
 
+    # heads of 256 dims: the same buffers read as 16 384 tokens of two rows each (the same bytes per step)
+    g2 = torch.Generator(device="cuda").manual_seed(302)
+    q256 = torch.randn((B, Hq, 2 * D), generator=g2, device="cuda").to(torch.float16)
+    attn256 = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N // 2, head_dim=256)
+    _, ev256_ms = time_steps(torch, lambda i: attn256(q256, sets[i % n_sets][1], sets[i % n_sets][2]), steps, warmup)
+
     # Sparse V on this cache (turbo3 K and V: V is half of the bytes): the benchmark's queries and queries scaled x16
     # (peaked attention), with the skip rate the kernel reports
     sparse_v = {}
@@ -392,6 +398,9 @@ def decode_leg(torch, tqa, steps, warmup, n_sets=2, small_batches=True):
         "gqa8": {"workload": "the same cache, 64 query heads on 8 KV heads (eight heads per pass over K/V)",
                  "us_per_step": ev8_ms * 1e3, "n_splits": attn8.params.n_splits,
                  "frac": algo / (ev8_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "head_dim_256": {"workload": "the same buffers as 16384 tokens of 256 dims (two 128-value rows per token), 32 query heads on 8 KV heads",
+                         "us_per_step": ev256_ms * 1e3, "n_splits": attn256.params.n_splits,
+                         "frac": algo / (ev256_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "sparse_v": sparse_v, "small_batches": small,
         "serving_step": {"workload": "tq_append_kv of one token per sequence + decode attention",
                          "us_per_step": serve_ms * 1e3, "us_per_step_hip_graph": graph_ms * 1e3 / n_sets},

@@ -85,15 +85,20 @@ def test_decode_attention_turbo3(N, n_splits):
     np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
 
 
-def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale):
+def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None):
     """Oracle attention for heads of 256 dims on the GPU-stored codes: the caches hold 2 N rows of 128 per sequence,
     row 2 t + half; a token's vector is its two rows side by side, each decoded and un-rotated by itself."""
     G = Hq // Hkv
-    ki, kg = kc.unpack_codes(k_packed, B * Hkv, 2 * N, kind="k")
+    if k_q8 is None:
+        ki, kg = kc.unpack_codes(k_packed, B * Hkv, 2 * N, kind="k")
+        k_rot = O.turbo_decode_rotated(np_(ki), np_(kg).astype(np.float64), kc.centroids).reshape(B * Hkv, N, 2 * D)
+        q_rot = O.rotate_fast(q.astype(np.float64).reshape(B, Hq, 2, D), kc.signs1, kc.signs2, D).reshape(B, Hq, 2 * D)
+    else:
+        qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, 2 * N)
+        k_rot = O.q8_0_dequantize(np_(qq), np_(ss)).reshape(B * Hkv, N, 2 * D)
+        q_rot = q.astype(np.float64)
     vi, vg = vc.unpack_codes(v_packed, B * Hkv, 2 * N, kind="v")
-    k_rot = O.turbo_decode_rotated(np_(ki), np_(kg).astype(np.float64), kc.centroids).reshape(B * Hkv, N, 2 * D)
     v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids).reshape(B * Hkv, N, 2 * D)
-    q_rot = O.rotate_fast(q.astype(np.float64).reshape(B, Hq, 2, D), kc.signs1, kc.signs2, D).reshape(B, Hq, 2 * D)
     out = np.zeros((B, Hq, 2 * D))
     for b in range(B):
         for h in range(Hkv):
@@ -125,6 +130,29 @@ def test_decode_attention_head_dim_256(bits, N, n_splits, Hq):
     out = np_(attn(q, kp, vp))
     assert out.shape == (B, Hq, 2 * D)
     ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D))
+    assert_close(out, ref)
+
+
+@pytest.mark.parametrize("kbits,vbits", [(8, 4), (8, 3), (8, 2), (4, 2), (3, 2), (4, 3)])
+@pytest.mark.parametrize("N,n_splits", [(100, 1), (2048 + 31, 8)])
+def test_decode_attention_head_dim_256_mixed_formats(kbits, vbits, N, n_splits):
+    """256-dim heads with q8_0-style K rows (the fork's recommended "-ctk q8_0 -ctv turboN") and with K wider than V."""
+    B, Hq, Hkv = 2, 8, 2
+    rng = np.random.default_rng(100 * kbits + vbits + N)
+    k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    k[:, :, :7] *= 4.0
+    vc = tqa.TurboCodec(vbits, seed=542)
+    vp = vc.store(tqa.rows_of_256(v), kind="v")
+    q = rng.standard_normal((B, Hq, 2 * D)).astype(np.float16)
+    if kbits == 8:
+        kc, kp = None, tqa.q8_0_store(tqa.rows_of_256(k))[0]
+    else:
+        kc = tqa.TurboCodec(kbits, seed=42)
+        kp = kc.store(tqa.rows_of_256(k), kind="k")
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256)
+    out = np_(attn(q, kp, vp))
+    ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D), k_q8=kp if kbits == 8 else None)
     assert_close(out, ref)
 
 
@@ -162,7 +190,7 @@ def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
     with pytest.raises(NotImplementedError):
         tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256, sparse_v_tau=1e-3)(q, buf, buf)
     with pytest.raises(NotImplementedError):
-        tqa.DecodeAttention(kc, tqa.TurboCodec(2, seed=542), B, Hq, Hkv, N, head_dim=256)(q, buf, buf)
+        tqa.DecodeAttention(tqa.TurboCodec(2, seed=42), vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf)   # K narrower than V
     with pytest.raises(NotImplementedError):
         tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf, bias=tt.zeros((B, Hq, N), device="cuda"))
     with pytest.raises(ValueError):

@@ -248,6 +248,16 @@ __device__ __forceinline__ void qk_turbo_d256(std::integer_sequence<int, G...>, 
      ...);
 }
 
+template <int... G>
+__device__ __forceinline__ void qk_q8_d256(std::integer_sequence<int, G...>, const uint32_t (&kw)[32], const half4_t (&qa4)[4],
+                                           float4_t (&acc)[4]) {
+    (([&] {
+         const half4_t kv = int8x4_to_half_0213(kw[G]);
+         acc[G >> 3] = mfma4_bcast8<(G & 7)>(qa4[G >> 3], kv, acc[G >> 3]);
+     }()),
+     ...);
+}
+
 // ... and V rows whose 64 "tokens" are (token, half) pairs: quad T holds the rows of tokens 2T, 2T+1 in the order
 // (2T, 0), (2T, 1), (2T+1, 0), (2T+1, 1).  The weights of tokens 4b..4b+3 sit in block b, so quad T takes them from
 // block T / 2, with zeros in the places of the other half: one look-up feeds the output's two halves.
@@ -459,12 +469,12 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 
 // SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
 // registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
-// D256: heads of 256 dims (turbo K and V, dense, no bias).  A token is rows 2 token and 2 token + 1 of caches that are
+// D256: heads of 256 dims (turbo or q8_0-style K, turbo V, dense, no bias).  A token is rows 2 token and 2 token + 1 of caches that are
 // otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
 // then the output's two halves of one set of four heads: one softmax, two accumulator sets.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
 __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_decode_attn(AttnArgs a) {
-    static_assert(!D256 || (HG == 2 && KFMT == KFMT_TURBO && VBITS != 8 && !SPARSE && !SBIAS), "256-dim heads: turbo K and V, dense");
+    static_assert(!D256 || (HG == 2 && VBITS != 8 && !SPARSE && !SBIAS), "256-dim heads: turbo V, dense");
     constexpr int HQ = D256 ? 1 : HG;   // sets of four heads whose logits and softmax state the wavefront keeps
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
@@ -558,7 +568,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         const int row0 = (tile & 1) * 64 + lane;
         const uint8_t *kb = kbase + (int64_t)(tile >> 1) * KBLOCK;
         if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kb, (tile & 1) * 64 + krow, kw);
-        else load_row<8>(kb, row0, kw);
+        else load_row<8>(kb, (tile & 1) * 64 + krow, kw);
         kn = load_knorm(tile);
         load_row<VBITS>(vbase + (int64_t)(tile >> 1) * VBLOCK, row0, vw);
         gvu = load_vnorm(tile);
@@ -768,11 +778,20 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             for (int c = 0; c < 4; ++c) acc[hg][c] = float4_t{0.f, 0.f, 0.f, 0.f};
         if constexpr (D256) {
             // each half-wavefront: its half of the query against its rows; a token's two halves meet across lane ^ 32
-            qk_turbo_d256<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa4, acc[0]);
-            const float gk_own = __half2float(__ushort_as_half((unsigned short)kn.x));
+            float d[4];
+            if constexpr (KFMT == KFMT_TURBO) {
+                qk_turbo_d256<KBITS>(std::make_integer_sequence<int, 32>{}, kw, klut_b, qa4, acc[0]);
+                d[0] = d[1] = d[2] = d[3] = __half2float(__ushort_as_half((unsigned short)kn.x));
+            } else {
+                qk_q8_d256(std::make_integer_sequence<int, 32>{}, kw, qa4, acc[0]);
+                d[0] = __half2float(__ushort_as_half((unsigned short)(kn.x & 0xffff))) * a.scale_log2e;
+                d[1] = __half2float(__ushort_as_half((unsigned short)(kn.x >> 16))) * a.scale_log2e;
+                d[2] = __half2float(__ushort_as_half((unsigned short)(kn.y & 0xffff))) * a.scale_log2e;
+                d[3] = __half2float(__ushort_as_half((unsigned short)(kn.y >> 16))) * a.scale_log2e;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float part = ((acc[0][0][i] + acc[0][1][i]) + (acc[0][2][i] + acc[0][3][i])) * gk_own;
+                const float part = (acc[0][0][i] * d[0] + acc[0][1][i] * d[1]) + (acc[0][2][i] * d[2] + acc[0][3][i] * d[3]);
                 sc[0][i] = part + xor_lane<32>(part);
             }
         } else if constexpr (KFMT == KFMT_TURBO) {
@@ -797,7 +816,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
         {   // kw is dead now: fetch the next tile's K row into it
             const uint8_t *kbn = kbase + (int64_t)(tile_n >> 1) * KBLOCK;
             if constexpr (KFMT == KFMT_TURBO) load_row<KBITS>(kbn, krow_n, kw);
-            else load_row<8>(kbn, row_n, kw);
+            else load_row<8>(kbn, krow_n, kw);
             kn = load_knorm(tile_n);
         }
         // -> lane (b, j): head j (of each set), tokens 4b..4b+3; then the online softmax in base 2
@@ -1179,9 +1198,8 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: head_dim %d (128 or 256)", (int)p->head_dim);
         return TQ_ERR_UNSUPPORTED;
     }
-    if (d256 && (p->k_format != TQ_KFMT_TURBO || p->v_format != TQ_KFMT_TURBO || !hk || !hv || hk->bits != hv->bits ||
-                 p->sparse_v_tau > 0.0f || bias || p->bias_entries)) {
-        tq_set_error("tq_decode_attention: head_dim 256 takes turbo K and V of one code width, dense, without bias");
+    if (d256 && (p->v_format != TQ_KFMT_TURBO || !hv || p->sparse_v_tau > 0.0f || bias || p->bias_entries)) {
+        tq_set_error("tq_decode_attention: head_dim 256 takes turbo V rows, dense, without bias");
         return TQ_ERR_UNSUPPORTED;
     }
     const int64_t cache_rows = (d256 ? 2 : 1) * p->tokens;   // a 256-dim token is two rows of the caches
@@ -1280,10 +1298,22 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
 #define TQ_ATTN_256(B)                                                                                                  \
     if (share) k_decode_attn<KFMT_TURBO, B, B, false, true, 2, false, true><<<grid, wg, merge_bytes, s>>>(a);           \
     else k_decode_attn<KFMT_TURBO, B, B, false, false, 2, false, true><<<grid, wg, merge_bytes, s>>>(a)
-            if (kb == 3) { TQ_ATTN_256(3); }
-            else if (kb == 4) { TQ_ATTN_256(4); }
-            else { TQ_ATTN_256(2); }
+#define TQ_ATTN_256X(KF, KB, VB) k_decode_attn<KF, KB, VB, false, false, 2, false, true><<<grid, wg, merge_bytes, s>>>(a)
+            if (turbo_k && kb == vb && kb == 3) { TQ_ATTN_256(3); }
+            else if (turbo_k && kb == vb && kb == 4) { TQ_ATTN_256(4); }
+            else if (turbo_k && kb == vb && kb == 2) { TQ_ATTN_256(2); }
+            else if (turbo_k && kb == 4 && vb == 2) { TQ_ATTN_256X(KFMT_TURBO, 4, 2); }
+            else if (turbo_k && kb == 3 && vb == 2) { TQ_ATTN_256X(KFMT_TURBO, 3, 2); }
+            else if (turbo_k && kb == 4 && vb == 3) { TQ_ATTN_256X(KFMT_TURBO, 4, 3); }
+            else if (!turbo_k && vb == 2) { TQ_ATTN_256X(KFMT_Q8, 3, 2); }
+            else if (!turbo_k && vb == 3) { TQ_ATTN_256X(KFMT_Q8, 3, 3); }
+            else if (!turbo_k && vb == 4) { TQ_ATTN_256X(KFMT_Q8, 3, 4); }
+            else {
+                tq_set_error("tq_decode_attention: head_dim 256 with K %d bits, V %d bits is not built", kb, vb);
+                return TQ_ERR_UNSUPPORTED;
+            }
 #undef TQ_ATTN_256
+#undef TQ_ATTN_256X
             rc = tq_check_launch("decode_attn (256-dim heads)");
             if (rc) return rc;
             continue;
