@@ -270,7 +270,7 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
         _, fkev_ms = time_steps(torch, fkstep, steps, warmup)
         _, fvev_ms = time_steps(torch, fvstep, steps, warmup)
         f_algo = n_vec * (512 + 16 * bits + 2)
-        f32 = {"what": "K and V as float32 rows (512 B per vector in), two launches (k_store_k<float>, k_store_v<float>)",
+        f32 = {"what": "K and V as float32 rows (512 B per vector in), one launch (k_store_kv<float>); k_alone / v_alone: the single-tensor kernels",
                "us_per_step": fev_ms * 1e3, "algorithmic_bytes_per_step": f_algo, "gbs": f_algo / (fev_ms * 1e-3) / 1e9,
                "frac": f_algo / (fev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                "k_alone": {"us_per_launch": fkev_ms * 1e3, "gbs": f_algo / 2 / (fkev_ms * 1e-3) / 1e9,

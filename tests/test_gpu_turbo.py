@@ -367,6 +367,30 @@ def test_store_kv_fp32_into_a_cache_layout():
         assert np.array_equal(c[:, :per_seq], r) and (c[:, per_seq:] == 0xA5).all()
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("shape", [(3, 300), (8, 8192)])
+def test_store_kv_fp32_one_launch(bits, shape):
+    """K and V of one code width as fp32 rows go out in one launch (the fused K+V kernel on two fp16 terms per value):
+    the bytes of the single-tensor fp32 stores, plain and into caches laid out for a larger capacity."""
+    tt = L.torch()
+    n, tokens = shape
+    kc, vc = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
+    rng = np.random.default_rng(bits + tokens)
+    k = (rng.standard_normal((n, tokens, D)) * rng.uniform(0.01, 50.0, (n, tokens, 1))).astype(np.float32)
+    v = rng.standard_normal((n, tokens, D)).astype(np.float32)
+    kd, vd = tt.from_numpy(k).cuda(), tt.from_numpy(v).cuda()
+    pk, pv = kc.store_kv(vc, kd, vd)
+    assert tt.equal(pk, kc.store(kd, kind="k")) and tt.equal(pv, vc.store(vd, kind="v"))
+    cap = tokens + 200
+    ck = tt.full((tqa.packed_bytes(bits, n, cap),), 0xA5, dtype=tt.uint8, device="cuda")
+    cv = tt.full_like(ck, 0xA5)
+    kc.store_kv(vc, kd, vd, out_k=ck, out_v=cv, capacity=cap)
+    per_seq_cache, per_seq = tqa.packed_bytes(bits, 1, cap), tqa.packed_bytes(bits, 1, tokens)
+    for cache, ref in ((ck, pk), (cv, pv)):
+        c, r = np_(cache).reshape(n, per_seq_cache), np_(ref).reshape(n, per_seq)
+        assert np.array_equal(c[:, :per_seq], r) and (c[:, per_seq:] == 0xA5).all()
+
+
 @pytest.mark.parametrize("bits", [4, 3])
 def test_config2_fused_store_full_size_bytes(bits):
     """The launch the benchmark times: tq_store_kv on config 2's tensors at full size (K with four outlier channels

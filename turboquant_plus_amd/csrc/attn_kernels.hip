@@ -843,7 +843,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             }
             const float mx = max_over_blocks(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
             const float m_new = fmaxf(m_run[hg], mx);
-            {
+            // After the first tiles the running maximum rarely moves, and a correction factor of exactly 1 changes
+            // nothing: the rescaling is skipped when no lane's maximum moved (a wave-uniform branch; same results).
+            if (__builtin_amdgcn_ballot_w64(m_new != m_run[hg]) != 0ull) {
                 // 0 on the first tile, 1 when the maximum stays (also while every position so far is masked with -inf)
                 const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run[hg] - m_new);
                 l_run[hg] *= corr;

@@ -1572,8 +1572,8 @@ __global__ __launch_bounds__(256, 3) void k_store_v(const TI *x, uint8_t *packed
 // for the 3-bit launch; reading one value of every cache line of the argument blocks in one batch at entry, 32.4 against
 // 31.9 us; raised issue priority for wavefronts that hold a V tile, which shortens the V phase of the slowest wavefronts
 // from 31 to 22 us and leaves the launch where it was.)
-template <int KB, int VB, bool RAGGED>
-__global__ __launch_bounds__(768) void k_store_kv(const __half *xv, const __half *xk, uint32_t v_units, uint32_t k_units, uint8_t *pv,
+template <int KB, int VB, bool RAGGED, typename TI = __half>
+__global__ __launch_bounds__(768) void k_store_kv(const TI *xv, const TI *xk, uint32_t v_units, uint32_t k_units, uint8_t *pv,
                                                   uint8_t *pk, StoreKArgs ka, StoreVArgs va) {
     // The +-1 operand fragments, sign masks, boundaries and c^2 coefficients are built from the argument block in
     // registers, so a wavefront's first memory request is its first input; only the 4-bit quantiser tables live in
@@ -3670,13 +3670,28 @@ int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const 
     ka.out_blocks_per_seq = va.out_blocks_per_seq = (uint32_t)out_bps;
     va.share_k_lut = hk->bits == 4 && hv->bits == 4 && hk->quant_lut_hash == hv->quant_lut_hash;
     const bool ragged = tokens != bps * TQ_ROWS_PER_BLOCK || out_bps != bps;
-    if (in_dtype != TQ_F16) {  // fp32 rows: the single-tensor kernels, one launch per tensor
-        const int rc = launch_store_k(hk, k, in_dtype, packed_k, ka, ragged, s);
-        return rc ? rc : launch_store_v(hv, v, in_dtype, packed_v, va, ragged, s);
-    }
     // one workgroup of 12 wavefronts per CU
     const unsigned wg = 768;
     const unsigned grid = (unsigned)((va.n_units + 11) / 12 < 256 ? (va.n_units + 11) / 12 : 256);
+    if (in_dtype != TQ_F16) {  // fp32 rows
+        if (hk->bits == hv->bits) {
+#define TQ_KV32(B)                                                                                                            \
+    if (ragged) k_store_kv<B, B, true, float><<<grid, wg, 0, s>>>((const float *)v, (const float *)k, va.n_units, ka.n_units, \
+                                                                   (uint8_t *)packed_v, (uint8_t *)packed_k, ka, va);           \
+    else k_store_kv<B, B, false, float><<<grid, wg, 0, s>>>((const float *)v, (const float *)k, va.n_units, ka.n_units,       \
+                                                             (uint8_t *)packed_v, (uint8_t *)packed_k, ka, va)
+            switch (hk->bits) {
+            case 2: TQ_KV32(2); break;
+            case 3: TQ_KV32(3); break;
+            default: TQ_KV32(4); break;
+            }
+#undef TQ_KV32
+            return tq_check_launch("store_kv (fp32 rows)");
+        }
+        // K and V of different widths: the single-tensor kernels, one launch per tensor
+        const int rc = launch_store_k(hk, k, in_dtype, packed_k, ka, ragged, s);
+        return rc ? rc : launch_store_v(hv, v, in_dtype, packed_v, va, ragged, s);
+    }
 #define TQ_KV(KB, VB)                                                                                                       \
     if (ragged) k_store_kv<KB, VB, true><<<grid, wg, 0, s>>>((const __half *)v, (const __half *)k, va.n_units, ka.n_units,  \
                                                               (uint8_t *)packed_v, (uint8_t *)packed_k, ka, va);             \
