@@ -361,71 +361,95 @@ __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)
 // Log-sum-exp merge of a group's n_parts partials, transpose of the V rotation, output rows; one wavefront per
 // query head (the partials come straight from memory: every load of a head is issued before the first is used
 // when there are at most four).
+// The partials [p_lo, p_hi) of one head of a group, merged by one wavefront: running maximum M (log2 units), weight
+// sum L and this lane's two output dims, all relative to M.  Up to 16 partials have every load requested before the
+// first is used, so the merge costs one trip to memory (in batches of four, sixteen partials took four trips at the
+// very end of the launch).
+struct MergedPart {
+    float M, L, o0, o1;
+};
+__device__ __forceinline__ MergedPart merge_range(const float *ml0, const float *po0, int ML, int PO, int head, int p_lo, int p_hi,
+                                                  int lane) {
+    MergedPart r{-INFINITY, 0.0f, 0.0f, 0.0f};
+    const int n = p_hi - p_lo;
+    auto merge_few = [&](auto np_tag) {
+        constexpr int NP = decltype(np_tag)::value;
+        float2 ml[NP], v[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int pc = p_lo + (p < n ? p : 0);
+            ml[p] = ld_dev2(ml0 + pc * ML + head * 2);
+            v[p] = ld_dev2(po0 + (int64_t)pc * PO + head * 128 + 2 * lane);
+            if (p >= n) ml[p].y = 0.0f;
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+            if (ml[p].y > 0.0f) r.M = fmaxf(r.M, ml[p].x);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const float w = ml[p].y > 0.0f ? exp2f(ml[p].x - r.M) : 0.0f;
+            r.L = fmaf(ml[p].y, w, r.L);
+            r.o0 = fmaf(v[p].x, w, r.o0);
+            r.o1 = fmaf(v[p].y, w, r.o1);
+        }
+    };
+    if (n <= 0) return r;
+    if (n <= 4) {
+        merge_few(std::integral_constant<int, 4>{});
+    } else if (n <= 16) {
+        merge_few(std::integral_constant<int, 16>{});
+    } else {
+        for (int p0 = p_lo; p0 < p_hi; p0 += 64) {  // lane <-> partial: maximum, then weights
+            const int p = p0 + lane;
+            float m = -INFINITY;
+            if (p < p_hi) {
+                const float2 e = ld_dev2(ml0 + p * ML + head * 2);
+                if (e.y > 0.0f) m = e.x;
+            }
+            for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+            r.M = fmaxf(r.M, m);
+        }
+        for (int p0 = p_lo; p0 < p_hi; p0 += 64) {
+            const int p = p0 + lane;
+            float w = 0.0f, l = 0.0f;
+            if (p < p_hi) {
+                const float2 e = ld_dev2(ml0 + p * ML + head * 2);
+                l = e.y;
+                w = l > 0.0f ? exp2f(e.x - r.M) : 0.0f;
+            }
+            float lw = l * w;
+            for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
+            r.L += lw;
+            const int cnt = min(64, p_hi - p0);
+#pragma unroll 4
+            for (int t = 0; t < cnt; ++t) {
+                const float wt = __shfl(w, t);
+                const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * PO + head * 128 + 2 * lane);
+                r.o0 = fmaf(v.x, wt, r.o0);
+                r.o1 = fmaf(v.y, wt, r.o1);
+            }
+        }
+    }
+    return r;
+}
+
+// The group's partials -> output rows (log-sum-exp merge, then the V rotation's transpose).  A workgroup with at least
+// twice as many wavefronts as the pass has heads gives every head several wavefronts, each merging a share of the
+// partials, and joins their results through `lds` (free LDS of 132 floats per wavefront; unused otherwise): the merge
+// runs at the very end of the launch, so its trips to memory are the launch's tail.
 template <int HG>
-__device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_parts, int tid, int n_waves) {
+__device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_parts, int tid, int n_waves, float *lds) {
     constexpr int NH = 4 * HG, ML = 2 * NH, PO = 128 * NH;  // heads, (m, l) floats and output floats of one partial
     const int lane = tid & 63, wave = tid >> 6;
     const float *ml0 = a.part_ml + (int64_t)group * n_parts * ML;
     const float *po0 = a.part_o + (int64_t)group * n_parts * PO;
-    for (int head = wave; head < NH; head += n_waves) {
+    auto finish = [&](int head, MergedPart r) {
         // heads of 256 dims (HG = 2): partial row 4 dh + i is dims 128 dh .. 128 dh + 127 of head i
         const int hq = a.d256 ? (head & 3) : head;
-        if (a.head_off + hq >= a.q_group) continue;  // a repeated head of a group with fewer than four left
         const int64_t r_out = a.d256 ? 2 * ((int64_t)group * a.q_group + a.head_off + hq) + (head >> 2)
                                      : (int64_t)group * a.q_group + a.head_off + head;
-        float M = -INFINITY, L = 0.0f, o0 = 0.0f, o1 = 0.0f;
-        if (n_parts <= 4) {
-            float2 ml[4], v[4];
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const int pc = p < n_parts ? p : 0;
-                ml[p] = ld_dev2(ml0 + pc * ML + head * 2);
-                v[p] = ld_dev2(po0 + (int64_t)pc * PO + head * 128 + 2 * lane);
-                if (p >= n_parts) ml[p].y = 0.0f;
-            }
-#pragma unroll
-            for (int p = 0; p < 4; ++p)
-                if (ml[p].y > 0.0f) M = fmaxf(M, ml[p].x);
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const float w = ml[p].y > 0.0f ? exp2f(ml[p].x - M) : 0.0f;
-                L = fmaf(ml[p].y, w, L);
-                o0 = fmaf(v[p].x, w, o0);
-                o1 = fmaf(v[p].y, w, o1);
-            }
-        } else {
-            for (int p0 = 0; p0 < n_parts; p0 += 64) {  // lane <-> partial: maximum, then weights
-                const int p = p0 + lane;
-                float m = -INFINITY;
-                if (p < n_parts) {
-                    const float2 e = ld_dev2(ml0 + p * ML + head * 2);
-                    if (e.y > 0.0f) m = e.x;
-                }
-                for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-                M = fmaxf(M, m);
-            }
-            for (int p0 = 0; p0 < n_parts; p0 += 64) {
-                const int p = p0 + lane;
-                float w = 0.0f, l = 0.0f;
-                if (p < n_parts) {
-                    const float2 e = ld_dev2(ml0 + p * ML + head * 2);
-                    l = e.y;
-                    w = l > 0.0f ? exp2f(e.x - M) : 0.0f;
-                }
-                float lw = l * w;
-                for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
-                L += lw;
-                const int cnt = min(64, n_parts - p0);
-#pragma unroll 4
-                for (int t = 0; t < cnt; ++t) {
-                    const float wt = __shfl(w, t);
-                    const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * PO + head * 128 + 2 * lane);
-                    o0 = fmaf(v.x, wt, o0);
-                    o1 = fmaf(v.y, wt, o1);
-                }
-            }
-        }
-        const float invL = L > 0.0f ? 1.0f / L : 0.0f;
+        const float invL = r.L > 0.0f ? 1.0f / r.L : 0.0f;
+        float o0 = r.o0, o1 = r.o1;
         float2 res;
         if (!a.vs1) {  // V rows were stored unrotated
             res = make_float2(o0 * invL, o1 * invL);
@@ -438,8 +462,47 @@ __device__ __forceinline__ void merge_group(const AttnArgs &a, int group, int n_
             res = make_float2(o0 * (s1v.x * RSQRT128), o1 * (s1v.y * RSQRT128));
         }
         *reinterpret_cast<float2 *>(a.out + r_out * 128 + 2 * lane) = res;
+    };
+    // a repeated head of a group with fewer than four left is not written
+    auto head_exists = [&](int head) { return a.head_off + (a.d256 ? (head & 3) : head) < a.q_group; };
+    const int n_sub = lds && n_waves >= 2 * NH && n_parts > 4 ? n_waves / NH : 1;
+    if (n_sub == 1) {
+        for (int head = wave; head < NH; head += n_waves)
+            if (head_exists(head)) finish(head, merge_range(ml0, po0, ML, PO, head, 0, n_parts, lane));
+        return;
+    }
+    const int head = wave % NH, sub = wave / NH;
+    const int per = (n_parts + n_sub - 1) / n_sub;
+    const bool mine = sub < n_sub && head_exists(head);
+    MergedPart r{-INFINITY, 0.0f, 0.0f, 0.0f};
+    if (mine) r = merge_range(ml0, po0, ML, PO, head, min(sub * per, n_parts), min(sub * per + per, n_parts), lane);
+    float *slot = lds + (head * n_sub + (sub < n_sub ? sub : 0)) * 132;
+    if (mine) {
+        *reinterpret_cast<float2 *>(slot + 2 * lane) = make_float2(r.o0, r.o1);
+        if (lane == 0) {
+            slot[128] = r.M;
+            slot[129] = r.L;
+        }
+    }
+    __syncthreads();
+    if (mine && sub == 0) {
+        const float *s0 = lds + head * n_sub * 132;
+        float M = -INFINITY;
+        for (int k = 0; k < n_sub; ++k)
+            if (s0[k * 132 + 129] > 0.0f) M = fmaxf(M, s0[k * 132 + 128]);
+        MergedPart t{M, 0.0f, 0.0f, 0.0f};
+        for (int k = 0; k < n_sub; ++k) {
+            const float l = s0[k * 132 + 129];
+            const float w = l > 0.0f ? exp2f(s0[k * 132 + 128] - M) : 0.0f;
+            const float2 o = *reinterpret_cast<const float2 *>(s0 + k * 132 + 2 * lane);
+            t.L = fmaf(l, w, t.L);
+            t.o0 = fmaf(o.x, w, t.o0);
+            t.o1 = fmaf(o.y, w, t.o1);
+        }
+        finish(head, t);
     }
 }
+
 
 // sum over the workgroup of one 64-bit value per thread (every thread gets the total); red: one shared word
 __device__ __forceinline__ unsigned long long block_sum(unsigned long long t, unsigned long long *red, int tid) {
@@ -473,7 +536,9 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 // otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
 // then the output's two halves of one set of four heads: one softmax, two accumulator sets.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
-__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KFMT == KFMT_TURBO ? 4 : 1) void k_decode_attn(AttnArgs a) {
+    // (256-dim heads on turbo K rows: four wavefronts per SIMD = two workgroups of eight per CU, i.e. at most 128 registers - the
+    // variant sits at 119-136 without the bound, and one register over 128 halves its occupancy)
     static_assert(!D256 || (HG == 2 && VBITS != 8 && !SPARSE && !SBIAS), "256-dim heads: turbo V, dense");
     constexpr int HQ = D256 ? 1 : HG;   // sets of four heads whose logits and softmax state the wavefront keeps
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
@@ -482,10 +547,11 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     constexpr int KLUT_BYTES = KFMT == KFMT_TURBO ? lut_bytes(KBITS) : 0;
     static_assert(!SHARE || (KFMT == KFMT_TURBO && KBITS == VBITS), "a shared table needs equal code widths");
     // static LDS (its address is a compile-time constant, so table positions fold into the LDS
-    // instructions): [K table][V table unless shared with K].  Before the tables are built the
-    // first 1 KB stages the group's four rotated queries.
+    // instructions): [K table][V table unless shared with K], and 1 KB per set of four heads that stages the
+    // group's rotated queries (a region of its own: the tables are built while the queries are still on their way)
     constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
-    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 1024 * HG ? LUT_TOTAL : 1024 * HG];
+    __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 16 ? LUT_TOTAL : 16];
+    __shared__ __attribute__((aligned(16))) char q_stage[1024 * HG];
     __shared__ uint32_t lead;  // tiles finished by the wavefront that is furthest ahead
     __shared__ uint32_t skipped;  // Sparse V: (query, position) pairs skipped by this workgroup
     char *klut_s = smem;
@@ -590,12 +656,10 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     // dim groups g = b and g = b + 16 (4 dims each); MFMA g reads it from block g % 16.
     // The group's four queries are rotated by the first wavefronts (one 128-point butterfly per
     // head, two values per lane), scaled and parked as fp16 in 1 KB of LDS for everybody.
-    for (int h = wave; h < 4 * HG; h += n_waves) {
-        _Float16 *qw = reinterpret_cast<_Float16 *>(smem) + h * 128;
+    auto load_q = [&](int h, float &x0, float &x1) {
         // heads past the group's last one repeat it (their results are not written)
         const int64_t e = D256 ? ((int64_t)group * a.q_group + min(a.head_off + (h & 3), a.q_group - 1)) * 256 + 128 * (h >> 2) + 2 * lane
                                : ((int64_t)group * a.q_group + min(a.head_off + h, a.q_group - 1)) * 128 + 2 * lane;
-        float x0, x1;
         if (a.q_dtype == TQ_F16) {
             const __half *qp = reinterpret_cast<const __half *>(a.q);
             x0 = __half2float(qp[e]);
@@ -609,6 +673,17 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             x0 = (float)qp[e];
             x1 = (float)qp[e + 1];
         }
+    };
+    // this wavefront's first head is requested now and rotated after the tables are built (the tables need only the
+    // pair entries requested above, and nobody reads them before the barrier below)
+    float xq0 = 0.0f, xq1 = 0.0f;
+    if (wave < 4 * HG) load_q(wave, xq0, xq1);
+    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
+    if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
+    for (int h = wave; h < 4 * HG; h += n_waves) {
+        _Float16 *qw = reinterpret_cast<_Float16 *>(q_stage) + h * 128;
+        float x0 = xq0, x1 = xq1;
+        if (h != wave) load_q(h, x0, x1);
         if (a.ks1) {
             x0 *= a.ks1[2 * lane];
             x1 *= a.ks1[2 * lane + 1];
@@ -633,19 +708,15 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
     half4_t qa4[4];   // 256-dim heads: dim groups b, b + 8, b + 16, b + 24 of this half-wavefront's half of the query
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) {
-        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + (4 * hg + j) * 128);
+        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(q_stage) + (4 * hg + j) * 128);
         qa[hg][0] = __builtin_bit_cast(half4_t, qp[lane >> 2]);
         qa[hg][1] = __builtin_bit_cast(half4_t, qp[(lane >> 2) + 16]);
     }
     if constexpr (D256) {
-        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(smem) + (4 * (lane >> 5) + j) * 128);
+        const uint2 *qp = reinterpret_cast<const uint2 *>(reinterpret_cast<const _Float16 *>(q_stage) + (4 * (lane >> 5) + j) * 128);
 #pragma unroll
         for (int k = 0; k < 4; ++k) qa4[k] = __builtin_bit_cast(half4_t, qp[((lane >> 2) & 7) + 8 * k]);
     }
-    __syncthreads();  // every wavefront has its queries in registers: the staging area becomes table space
-    if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
-    if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
-    __syncthreads();
     // out[head i][dim 64*hf + lane] partial sums; two chains per dim half for MFMA issue overlap
     float4_t acc_o[HG][2][2];
     float m_run[HG], l_run[HG];
@@ -1096,7 +1167,11 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG)) void k_dec
             }
         }
     }
-    merge_group<HG>(a, group, n_parts, tid, n_waves);
+    {
+        // the wavefronts' merge space is free again (every partial of this workgroup is in memory)
+        extern __shared__ float merge_s[];
+        merge_group<HG>(a, group, n_parts, tid, n_waves, n_waves > 1 ? merge_s : nullptr);
+    }
     if (n_parts > 1 && tid == 0) st_dev(a.flags + (int64_t)group * n_parts, 0ull);  // a replay of a captured launch (same tag) starts from zero
     if constexpr (SPARSE) {
         if (a.poll_slots) {
@@ -1163,6 +1238,10 @@ AttnPlan attn_plan(const tq_attn_params *p) {
     pl.hg = p->head_dim == 256 || p->n_q_heads / p->n_kv_heads > 4 ? 2 : 1;
     pl.wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
     while (p->n_splits % pl.wpw) pl.wpw >>= 1;
+    // few groups (small batches): smaller workgroups, so that every CU gets one (a tile costs a wavefront the same
+    // issue time however many share the SIMD)
+    const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
+    while (pl.wpw > 4 && groups * (p->n_splits / pl.wpw) < 256) pl.wpw >>= 1;
     pl.n_parts = p->n_splits / pl.wpw;
     return pl;
 }
