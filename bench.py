@@ -631,6 +631,21 @@ def cache_maintenance_leg(torch, tqa, steps, warmup):
     torch.cuda.synchronize()
     if not torch.equal(back3, packed3):
         raise RuntimeError("export followed by import changed the packed cache")
+    # the same three on the V tensor: a token's codes are spread over the 64 rows of its tile, so these kernels stage a
+    # block in LDS and work with sixteen lanes per token
+    v = synth_kv(torch, heads, tokens, 901, outliers=0)
+    packed3v = c3.store(v, kind="v")
+    vt = {}
+    for name, fn, nbytes in (
+            ("requantize_3to2", lambda i: L.check(lib.tq_requantize(c3.handle.h, c2.handle.h, L.ptr(packed3v), heads, tokens, L.KIND_V, L.ptr(out2), L.stream_ptr())), n3 + n2),
+            ("export_fork_blocks", lambda i: L.check(lib.tq_export_fork_blocks(c3.handle.h, L.ptr(packed3v), heads, tokens, L.KIND_V, L.ptr(blocks), L.stream_ptr())), n3 + heads * tokens * fb),
+            ("import_fork_blocks", lambda i: L.check(lib.tq_import_fork_blocks(c3.handle.h, L.ptr(blocks), heads, tokens, L.KIND_V, L.ptr(back3), L.stream_ptr())), n3 + heads * tokens * fb)):
+        _, ms = time_steps(torch, fn, steps, warmup)
+        vt[name] = {"us_per_call": ms * 1e3, "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    torch.cuda.synchronize()
+    if not torch.equal(back3, packed3v):
+        raise RuntimeError("export followed by import changed the packed V cache")
+    out["v_tensor"] = vt
     return out
 
 

@@ -264,9 +264,11 @@ def test_requantize_stored_cache(pair, kind):
 
 
 @pytest.mark.parametrize("pair", [(3, 2), (4, 3), (4, 2)])
-def test_requantize_k_rows_whose_code_map_is_their_own(pair):
-    """K rows go through a code -> code table that holds for rows whose sum of squared centroids lies in an interval
-    around 1; other rows build their own table.  Rows drawn from a random subset of the levels (all outer levels, all
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_requantize_rows_whose_code_map_is_their_own(pair, kind):
+    """Rows go through a code -> code table that holds for rows whose sum of squared centroids lies in an interval
+    around 1; other rows build their own table (K: the row's lane; V: the token's lane, and every lane of the tile
+    re-maps its two codes of that token).  Rows drawn from a random subset of the levels (all outer levels, all
     inner levels, one level only, ...) have sums between 0.2 and 5 and maps that differ from the common one - an outer
     level that falls into an inner cell once the row is renormalised - and rows with norm zero take the same path.
     Five blocks: the launch's workgroups serve eight at a time, so a ragged last set is covered too."""
@@ -285,11 +287,11 @@ def test_requantize_k_rows_whose_code_map_is_their_own(pair):
     assert sums.min() < 0.5 and sums.max() > 3.0
     g = rng.uniform(0.01, 30.0, tokens).astype(np.float16)
     g[rng.integers(0, tokens, 7)] = 0
-    packed = L.torch().from_numpy(O.layout_pack(idx, g, sb, "k")).cuda()
-    out = _check_requant(src, dst, packed, 1, tokens, "k")
+    packed = L.torch().from_numpy(O.layout_pack(idx, g, sb, kind)).cuda()
+    out = _check_requant(src, dst, packed, 1, tokens, kind)
     # the maps do differ: many rows do not get the codes a unit-sum row would
     common = np.searchsorted(O.midpoints(dst.centroids), src.centroids, side="right")
-    i2, _ = O.layout_unpack(np_(out), db, "k")
+    i2, _ = O.layout_unpack(np_(out), db, kind)
     live = g != 0
     assert np.mean(np.any(i2[:tokens][live] != common[idx][live], axis=1)) > 0.2
 

@@ -3022,6 +3022,14 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 struct RequantArgs {
     const float *cent_src, *cent_dst, *bounds_dst;
     int kind;
+    // The destination code of a source code depends on the row's S = sum of c_src[code]^2 alone, and for S inside
+    // (s_lo, s_hi) it is the fixed table t0 (4 bits per source code; requant_plan): such rows take their sums and codes
+    // from a table over pairs of codes; has_plan = 0 (more than 16 levels) leaves every row to the per-value code.
+    int has_plan;
+    unsigned long long t0;
+    float s_lo, s_hi, fix_unit;
+    float src_sq[16];        // c_src[k]^2
+    uint32_t dst_fix[16];    // c_dst[k]^2 / fix_unit, rounded: a row's 128 of them add up exactly in 32 bits
 };
 
 template <int SB, int DB>
@@ -3032,6 +3040,8 @@ __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t 
     __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
     __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
     __shared__ float csrc_s[1 << SB], cdst_s[1 << DB];
+    constexpr int NPAIR = 1 << (2 * SB);
+    __shared__ uint2 pair_s[NPAIR];   // per pair of source codes: .x = sum of c_src^2 (fp32 bits), .y = its two t0 codes << 24 | fixed-point sum of c_dst[t0]^2
     const int tid = threadIdx.x, lane = tid & 63;
     const int li = lane & 15, grp = tid >> 4;
     {
@@ -3040,6 +3050,24 @@ __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t 
     }
     if (tid < (1 << SB)) csrc_s[tid] = a.cent_src[tid];
     if (tid < (1 << DB)) cdst_s[tid] = a.cent_dst[tid];
+    if (a.has_plan && tid < NPAIR) {
+        // the argument arrays are indexed with constants only (they live in scalar registers)
+        const int k0 = tid & ((1 << SB) - 1), k1 = tid >> SB;
+        float q0 = 0.0f, q1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < (1 << SB); ++k) {
+            q0 = k0 == k ? a.src_sq[k] : q0;
+            q1 = k1 == k ? a.src_sq[k] : q1;
+        }
+        const uint32_t t0 = (uint32_t)((a.t0 >> (4 * k0)) & 15ull), t1 = (uint32_t)((a.t0 >> (4 * k1)) & 15ull);
+        uint32_t f0 = 0, f1 = 0;
+#pragma unroll
+        for (int k = 0; k < (1 << DB); ++k) {
+            f0 = t0 == (uint32_t)k ? a.dst_fix[k] : f0;
+            f1 = t1 == (uint32_t)k ? a.dst_fix[k] : f1;
+        }
+        pair_s[tid] = make_uint2(__float_as_uint(q0 + q1), ((t0 | (t1 << DB)) << 24) | (f0 + f1));
+    }
     float bnd[NB];
 #pragma unroll
     for (int k = 0; k < NB; ++k) bnd[k] = a.bounds_dst[k];
@@ -3049,6 +3077,35 @@ __global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t 
         const int t = it * 16 + grp;
         const uint32_t c8 = load_codes8<SB>(block_s, a.kind, t, li);
         const float g = block_norm(block_s, SB, t);
+        if (a.has_plan) {
+            // the row's sums and, if its S lies in the plan's interval, its codes: four table reads per lane
+            float s1 = 0.0f;
+            uint32_t fix = 0, codes8 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint2 en = pair_s[(c8 >> (2 * SB * i)) & (uint32_t)(NPAIR - 1)];
+                s1 += __uint_as_float(en.x);
+                fix += en.y & 0xFFFFFFu;
+                codes8 |= (en.y >> 24) << (2 * DB * i);
+            }
+            s1 = row16_sum(s1);
+            fix = row16_sum(fix);
+            const float recon_p = g * sqrtf(s1);
+            if (s1 > a.s_lo && s1 < a.s_hi && recon_p > 1e-10f) {   // the same for the row's sixteen lanes
+                uint32_t b0 = 0, b1 = 0;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    b0 |= ((codes8 >> (DB * m)) & ((1u << DB) - 1u)) << (8 * m);
+                    b1 |= ((codes8 >> (DB * (m + 4))) & ((1u << DB) - 1u)) << (8 * m);
+                }
+                *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(b0, b1);
+                if (li == 0) {
+                    const float cn = sqrtf((float)fix * a.fix_unit);
+                    norms_s[t] = cn > 1e-10f ? recon_p / cn : recon_p;
+                }
+                continue;
+            }
+        }
         float v[8];
         float ss = 0.0f;
 #pragma unroll
@@ -3103,6 +3160,9 @@ struct RequantKArgs {
     float src_sq[16], dst_sq[16];                   // c_src[k]^2, c_dst[k]^2: by value, so that no table build waits for memory
     uint32_t dst_fix[16];                           // c_dst[k]^2 / fix_unit, rounded: a row's 128 of them add up exactly in 32 bits
     float fix_unit;
+    uint32_t src_fix[16];                           // the same for c_src[k]^2 / src_unit (V rows: sums across lanes in integers)
+    float src_unit;
+    int zero_dst;                                   // destination code of the value 0.0 (rows with norm 0)
 };
 
 // one workgroup per CU: the tables are built once for the CU's share of the rows
@@ -3246,10 +3306,228 @@ __global__ __launch_bounds__(RQK_THREADS) void k_requantize_k(const uint8_t *src
     }
 }
 
+// ---- V rows: a wavefront owns a 64-token tile ----------------------------------------------------
+// Lane l holds packed row l of the tile: dims l and l + 64 of the tile's 64 tokens (word j of group q = tokens
+// 16 q + 4 j .. + 3, first the four codes of dim l, then those of dim l + 64).  The codes are remapped through the
+// same T0 table as K rows; a token's sums run over the 64 lanes, so every lane looks up the squares of its two codes
+// per token (a table over pairs of codes: two tokens per read, fixed point, exact integer adds) and a six-stage
+// exchange (lane ^ 1, 2, 4, 8 by DPP, 16 and 32 by the half-swap instructions) adds them up so that lane t ends
+// with token t's two sums.  Tokens with norm 0 get the code of 0.0 and norm 0; a token whose S lies outside the
+// plan's interval is redone on its own: its lane builds the token's table in float64, every lane re-maps its two
+// codes of that token, and the token's destination sum is added up again.
+template <int M> __device__ __forceinline__ uint32_t combine_lanes(uint32_t a, uint32_t b, int lane) {
+    if constexpr (M == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+        return r[0] + r[1];
+    } else if constexpr (M == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+        return r[0] + r[1];
+    } else {
+        const bool up = lane & M;
+        const uint32_t give = up ? a : b;           // what the partner keeps
+        return (up ? b : a) + xor_lane<M>(give);
+    }
+}
+
+constexpr int RQV_THREADS = 1024;   // sixteen tiles (eight blocks) per workgroup and turn: the tables are built once per CU
+template <int SB, int DB>
+__global__ __launch_bounds__(RQV_THREADS) void k_requantize_v(const uint8_t *src, uint8_t *dst, RequantKArgs a) {
+    constexpr int U = SB == 3 ? 4 : 2;   // codes per remap unit
+    constexpr int NE = 1 << (SB * U);
+    constexpr int NS = 1 << SB, ND = 1 << DB;
+    constexpr int NPAIR = 1 << (2 * SB);
+    constexpr uint32_t SM = NS - 1, DM = ND - 1;
+    __shared__ uint8_t remap_s[NE];       // a unit's destination codes, DB bits each
+    __shared__ uint8_t pair_remap_s[SB == 3 ? 64 : 1];
+    __shared__ uint4 pairfix_s[NPAIR];    // codes (lo, hi): c_src^2 of lo, of hi, c_dst[T0]^2 of lo, of hi (fixed point)
+    __shared__ uint32_t dstfix_s[ND];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t w[4 * SB];
+    uint16_t gbits = 0;
+    auto fetch = [&](uint32_t tile) {
+        const uint8_t *sb = src + (int64_t)(tile >> 1) * block_bytes(SB);
+        const int row = (int)(tile & 1) * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            const uint4 c = stream_load<STREAM_LOAD_OUT>(reinterpret_cast<const uint4 *>(sb + j * 2048 + row * 16));
+            w[4 * j] = c.x; w[4 * j + 1] = c.y; w[4 * j + 2] = c.z; w[4 * j + 3] = c.w;
+        }
+        gbits = reinterpret_cast<const uint16_t *>(sb + block_code_bytes(SB))[row];   // lane <-> token for the norms
+    };
+    const uint32_t n_tiles = 2 * a.n_blocks;
+    uint32_t tile = 16 * blockIdx.x + wave;
+    if (tile < n_tiles) fetch(tile);
+    // tables (argument arrays are indexed with constants only: they live in scalar registers)
+    auto pick = [](const auto &arr, uint32_t k, int n) {
+        auto v = arr[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i)
+            if (i < n) v = k == (uint32_t)i ? arr[i] : v;
+        return v;
+    };
+    if (tid < NPAIR) {
+        const uint32_t k0 = tid & SM, k1 = (uint32_t)tid >> SB;
+        const uint32_t t0 = (uint32_t)((a.t0 >> (4 * k0)) & 15ull), t1 = (uint32_t)((a.t0 >> (4 * k1)) & 15ull);
+        pairfix_s[tid] = make_uint4(pick(a.src_fix, k0, NS), pick(a.src_fix, k1, NS), pick(a.dst_fix, t0, ND), pick(a.dst_fix, t1, ND));
+        if constexpr (SB == 3) pair_remap_s[tid] = (uint8_t)(t0 | (t1 << DB));
+        else remap_s[tid] = (uint8_t)(t0 | (t1 << DB));
+    }
+    if (tid < ND) dstfix_s[tid] = pick(a.dst_fix, (uint32_t)tid, ND);
+    __syncthreads();
+    if constexpr (SB == 3) {
+        for (int e = tid; e < NE; e += RQV_THREADS) remap_s[e] = (uint8_t)(pair_remap_s[e & 63] | (pair_remap_s[e >> 6] << (2 * DB)));
+        __syncthreads();
+    }
+
+#pragma unroll 1
+    for (; tile < n_tiles;) {
+        // source word j of group q: eight codes, SB bits each = tokens 16 q + 4 j .. + 3 of dim l, then of dim l + 64
+        auto src_word = [&](int q, int j) -> uint32_t {
+            if constexpr (SB == 4) return w[4 * j + q];
+            else return j < 3 ? (w[4 * j + q] & 0xFFFFFFu) : tail24(w, q);
+        };
+        uint32_t m[4][4];
+        // sums: the leaves are token pairs (t, t + 1), whose codes are one pair entry per dim half; lane ^ 1 joins them
+        uint32_t f1_tree[7], f2_tree[7];   // results of finished subtrees by level (a binary counter over the 32 leaves)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t x = src_word(q, j);
+                uint32_t acc = 0;
+#pragma unroll
+                for (int u = 0; u < 8 / U; ++u) acc |= (uint32_t)remap_s[(x >> (SB * U * u)) & (uint32_t)(NE - 1)] << (DB * U * u);
+                m[q][j] = acc;
+                // tokens 16 q + 4 j + (0, 1) and + (2, 3): pair i of the first dim half, pair 2 + i of the second
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const uint4 e0 = pairfix_s[(x >> (2 * SB * i)) & (uint32_t)(NPAIR - 1)];
+                    const uint4 e1 = pairfix_s[(x >> (2 * SB * (2 + i))) & (uint32_t)(NPAIR - 1)];
+                    uint32_t v1 = combine_lanes<1>(e0.x + e1.x, e0.y + e1.y, lane);
+                    uint32_t v2 = combine_lanes<1>(e0.z + e1.z, e0.w + e1.w, lane);
+                    // leaf number (token pair) 8 q + 2 j + i: carry it up the tree
+                    const int leaf = 8 * q + 2 * j + i;
+#pragma unroll
+                    for (int lv = 1; lv < 6; ++lv) {
+                        if (((leaf >> (lv - 1)) & 1) == 0) {
+                            f1_tree[lv] = v1;
+                            f2_tree[lv] = v2;
+                            break;
+                        }
+                        if (lv == 1) { v1 = combine_lanes<2>(f1_tree[1], v1, lane); v2 = combine_lanes<2>(f2_tree[1], v2, lane); }
+                        if (lv == 2) { v1 = combine_lanes<4>(f1_tree[2], v1, lane); v2 = combine_lanes<4>(f2_tree[2], v2, lane); }
+                        if (lv == 3) { v1 = combine_lanes<8>(f1_tree[3], v1, lane); v2 = combine_lanes<8>(f2_tree[3], v2, lane); }
+                        if (lv == 4) { v1 = combine_lanes<16>(f1_tree[4], v1, lane); v2 = combine_lanes<16>(f2_tree[4], v2, lane); }
+                        if (lv == 5) {
+                            f1_tree[6] = combine_lanes<32>(f1_tree[5], v1, lane);
+                            f2_tree[6] = combine_lanes<32>(f2_tree[5], v2, lane);
+                        }
+                    }
+                }
+            }
+        // lane t: token t of the tile
+        const float g = __half2float(__ushort_as_half(gbits));
+        const float s1 = (float)f1_tree[6] * a.src_unit;
+        float s2 = (float)f2_tree[6] * a.fix_unit;
+        float recon = g * sqrtf(s1);
+        const bool zero_tok = !(recon > 1e-10f);
+        const bool redo = !zero_tok && !(s1 > a.s_lo && s1 < a.s_hi);
+        // tokens with norm 0: the code of 0.0 in every dim, norm 0
+        const unsigned long long zmask = __builtin_amdgcn_ballot_w64(zero_tok);
+        if (zmask) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t zb = (uint32_t)(zmask >> (16 * q + 4 * j)) & 15u;   // wave-uniform
+                    if (zb) {
+                        uint32_t fm = 0;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if ((zb >> i) & 1u) fm |= (DM << (DB * i)) | (DM << (DB * (4 + i)));
+                        uint32_t zz = 0;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) zz |= (uint32_t)a.zero_dst << (DB * i);
+                        m[q][j] = (m[q][j] & ~fm) | (zz & fm);
+                    }
+                }
+        }
+        // tokens outside the interval, one at a time
+        unsigned long long rmask = __builtin_amdgcn_ballot_w64(redo);
+        while (rmask) {
+            const int t = __builtin_ctzll(rmask);
+            rmask &= rmask - 1;
+            // token t's own table (its lane's values count; every lane runs the arithmetic)
+            const double rec = (double)g * sqrt((double)s1);
+            const double inv = rec > 1e-10 ? 1.0 / rec : 1.0;
+            unsigned long long tab = 0;
+            for (int k = 0; k < NS; ++k) {
+                const double y = a.cent_src[k] * (double)g * inv;
+                unsigned long long c = 0;
+                for (int b = 0; b < ND - 1; ++b) c += a.bounds_dst[b] <= y ? 1ull : 0ull;
+                tab |= c << (4 * k);
+            }
+            const uint32_t tab_lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)tab, t);
+            const uint32_t tab_hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(tab >> 32), t);
+            const unsigned long long tt = ((unsigned long long)tab_hi << 32) | tab_lo;
+            // this lane's two codes of token t: word (t >> 4, (t >> 2) & 3), slots t & 3 and 4 + (t & 3)
+            uint32_t x = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if ((t >> 4) == q && ((t >> 2) & 3) == j) x = src_word(q, j);
+            const uint32_t c0 = (x >> (SB * (t & 3))) & SM, c1 = (x >> (SB * (4 + (t & 3)))) & SM;
+            const uint32_t n0 = (uint32_t)(tt >> (4 * c0)) & 15u, n1 = (uint32_t)(tt >> (4 * c1)) & 15u;
+            const uint32_t fm = (DM << (DB * (t & 3))) | (DM << (DB * (4 + (t & 3))));
+            const uint32_t nv = (n0 << (DB * (t & 3))) | (n1 << (DB * (4 + (t & 3))));
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if ((t >> 4) == q && ((t >> 2) & 3) == j) m[q][j] = (m[q][j] & ~fm) | nv;
+            // the token's destination sum, over all lanes
+            uint32_t part = dstfix_s[n0] + dstfix_s[n1];
+            part += xor_lane<1>(part);
+            part += xor_lane<2>(part);
+            part += xor_lane<4>(part);
+            part += xor_lane<8>(part);
+            part += xor_lane<16>(part);
+            part += xor_lane<32>(part);
+            if (lane == t) s2 = (float)part * a.fix_unit;
+        }
+        const float cn = sqrtf(s2);
+        float gn = cn > 1e-10f ? recon / cn : recon;
+        if (zero_tok) gn = 0.0f;
+        const uint32_t out_tile = tile;
+        tile += 16 * gridDim.x;
+        // the source words are in m[][] by now
+        const int row = (int)(out_tile & 1) * 64 + lane;
+        uint8_t *db = dst + (int64_t)(out_tile >> 1) * block_bytes(DB);
+        uint32_t d[4 * DB];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (DB == 2) {
+                d[q] = m[q][0] | (m[q][1] << 16);
+                d[4 + q] = m[q][2] | (m[q][3] << 16);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) d[4 * j + q] = m[q][j] | (((m[q][3] >> (8 * j)) & 0xFFu) << 24);
+            }
+        }
+        if (tile < n_tiles) fetch(tile);
+#pragma unroll
+        for (int j = 0; j < DB; ++j)
+            stream_store<STREAM_STORE_CODES>(reinterpret_cast<uint4 *>(db + j * 2048 + row * 16),
+                                             make_uint4(d[4 * j], d[4 * j + 1], d[4 * j + 2], d[4 * j + 3]));
+        reinterpret_cast<__half *>(db + block_code_bytes(DB))[row] = __float2half_rn(gn);
+    }
+}
+
 // T0 and the interval of S = sum of c_src[code]^2 for which every source code keeps its T0 destination: the decision
 // value of code k is c_src[k] / r with r = sqrt(S), and it meets the midpoint b at r = c_src[k] / b.  The interval is
 // what lies between the nearest such r below and above 1, shrunk by 1e-5 so that the fp32 sum decides safely.
-static bool requant_k_plan(const tq_handle *hs, const tq_handle *hd, RequantKArgs *a) {
+static bool requant_plan(const tq_handle *hs, const tq_handle *hd, RequantKArgs *a) {
     const int ns = hs->n_centroids, nd = hd->n_centroids;
     if (ns > 16 || nd > 16) return false;
     double r_lo = 0.0, r_hi = 1e30;
@@ -3281,6 +3559,13 @@ static bool requant_k_plan(const tq_handle *hs, const tq_handle *hd, RequantKArg
     a->fix_unit = (float)unit;
     for (int k = 0; k < 16; ++k)
         a->dst_fix[k] = k < nd ? (uint32_t)llround(hd->centroids_host[k] * hd->centroids_host[k] / (double)a->fix_unit) : 0u;
+    double stop = 0.0;
+    for (int k = 0; k < ns; ++k) stop = fmax(stop, hs->centroids_host[k] * hs->centroids_host[k]);
+    a->src_unit = (float)(stop > 0.0 ? stop / 4194300.0 : 1.0);
+    for (int k = 0; k < 16; ++k)
+        a->src_fix[k] = k < ns ? (uint32_t)llround(hs->centroids_host[k] * hs->centroids_host[k] / (double)a->src_unit) : 0u;
+    a->zero_dst = 0;
+    for (int b = 0; b + 1 < nd; ++b) a->zero_dst += hd->bounds_host[b] <= 0.0 ? 1 : 0;
     return true;
 }
 
@@ -3292,7 +3577,16 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
     a.cent_src = hs->centroids32; a.cent_dst = hd->centroids32; a.bounds_dst = hd->bounds32; a.kind = kind;
     const int key = hs->bits * 10 + hd->bits;
     RequantKArgs ka;
-    if (kind == TQ_KIND_K && (key == 32 || key == 43 || key == 42) && requant_k_plan(hs, hd, &ka)) {
+    const bool planned = (key == 32 || key == 43 || key == 42) && requant_plan(hs, hd, &ka);
+    a.has_plan = planned ? 1 : 0;
+    if (planned) {
+        a.t0 = ka.t0; a.s_lo = ka.s_lo; a.s_hi = ka.s_hi; a.fix_unit = ka.fix_unit;
+        for (int k = 0; k < 16; ++k) {
+            a.src_sq[k] = ka.src_sq[k];
+            a.dst_fix[k] = ka.dst_fix[k];
+        }
+    }
+    if (kind == TQ_KIND_K && planned) {
         ka.n_blocks = grid;
         const unsigned sets = (grid + RQK_BLOCKS - 1) / RQK_BLOCKS;
         const unsigned wgs = sets < 256u ? sets : 256u;
@@ -3302,6 +3596,17 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
         default: k_requantize_k<4, 2><<<wgs, RQK_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
         }
         return tq_check_launch("requantize (K rows)");
+    }
+    if (kind == TQ_KIND_V && planned) {
+        ka.n_blocks = grid;
+        const unsigned sets = (grid + 7) / 8;
+        const unsigned wgs = sets < 256u ? sets : 256u;
+        switch (key) {
+        case 32: k_requantize_v<3, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        case 43: k_requantize_v<4, 3><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        default: k_requantize_v<4, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+        }
+        return tq_check_launch("requantize (V rows)");
     }
     switch (key) {
     case 32: k_requantize<3, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
