@@ -55,8 +55,8 @@ D = 128
 # WRITE_SIZE of this file's run, each scaled by the reading of a 1 GiB device copy).  The table is read at run time;
 # a missing file or row gives "traffic": null.  The JSON line names the row next to each figure.
 TRAFFIC_FILE = "profiles/bench_all_legs_trace_hbm_sq.txt"
-TRAFFIC_ROWS = {"store4": "k_store_kv<4, 4, false>", "store3": "k_store_kv<3, 3, false>",
-                "decode3": "k_decode_attn<0, 3, 3, false, true, 1, false>"}
+TRAFFIC_ROWS = {"store4": "k_store_kv<4, 4, false, __half>", "store3": "k_store_kv<3, 3, false, __half>",
+                "decode3": "k_decode_attn<0, 3, 3, false, true, 1, false, false>"}
 
 
 def profile_traffic(key):
