@@ -71,7 +71,8 @@ def make_kv(B, Hkv, N, seed, kbits=3, vbits=3):
     return k, v, kc, vc, kc.store(k, kind="k"), vc.store(v, kind="v")
 
 
-@pytest.mark.parametrize("N,n_splits", [(64, 1), (128, 1), (100, 1), (1000, 3), (2048, 4), (4096 + 37, 8), (8192, 64)])
+@pytest.mark.parametrize("N,n_splits", [(64, 1), (128, 1), (100, 1), (1000, 3), (2048, 4), (4096 + 37, 8), (8192, 64),
+                                        (8192, 128), (16384, 256)])   # the last two: 32 and 64 partials per group
 def test_decode_attention_turbo3(N, n_splits):
     B, Hq, Hkv = 2, 8, 2
     k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=N)

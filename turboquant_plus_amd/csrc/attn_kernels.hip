@@ -421,12 +421,22 @@ __device__ __forceinline__ MergedPart merge_range(const float *ml0, const float 
             for (int o = 32; o > 0; o >>= 1) lw += __shfl_xor(lw, o);
             r.L += lw;
             const int cnt = min(64, p_hi - p0);
-#pragma unroll 4
-            for (int t = 0; t < cnt; ++t) {
-                const float wt = __shfl(w, t);
-                const float2 v = ld_dev2(po0 + (int64_t)(p0 + t) * PO + head * 128 + 2 * lane);
-                r.o0 = fmaf(v.x, wt, r.o0);
-                r.o1 = fmaf(v.y, wt, r.o1);
+            // eight partials per trip to memory (a lane exchange cannot sit in a loop that the compiler unrolls with
+            // a remainder, so the batches are written out: past the count the last partial is read again with weight 0)
+            for (int t0 = 0; t0 < cnt; t0 += 8) {
+                float2 v[8];
+                float wt[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int t = min(t0 + k, cnt - 1);
+                    v[k] = ld_dev2(po0 + (int64_t)(p0 + t) * PO + head * 128 + 2 * lane);
+                    wt[k] = t0 + k < cnt ? __shfl(w, t) : 0.0f;
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    r.o0 = fmaf(v[k].x, wt[k], r.o0);
+                    r.o1 = fmaf(v[k].y, wt[k], r.o1);
+                }
             }
         }
     }
@@ -923,13 +933,15 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
                 // accumulator register i belongs to head i; the factor of head i lives in lanes with lane%4 == i
                 const float c0 = dpp<0x00>(corr), c1 = dpp<0x55>(corr), c2 = dpp<0xAA>(corr), c3 = dpp<0xFF>(corr);
 #pragma unroll
-                for (int ho = (D256 ? 0 : hg); ho < (D256 ? 2 : hg + 1); ++ho)   // 256-dim heads: both halves of the output
+                for (int ho = 0; ho < HG; ++ho) {
+                    if (!D256 && ho != hg) continue;   // 256-dim heads: both halves of the output share the softmax
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    acc_o[ho][c >> 1][c & 1][0] *= c0;
-                    acc_o[ho][c >> 1][c & 1][1] *= c1;
-                    acc_o[ho][c >> 1][c & 1][2] *= c2;
-                    acc_o[ho][c >> 1][c & 1][3] *= c3;
+                    for (int c = 0; c < 4; ++c) {
+                        acc_o[ho][c >> 1][c & 1][0] *= c0;
+                        acc_o[ho][c >> 1][c & 1][1] *= c1;
+                        acc_o[ho][c >> 1][c & 1][2] *= c2;
+                        acc_o[ho][c >> 1][c & 1][3] *= c3;
+                    }
                 }
                 m_run[hg] = m_new;
             }
