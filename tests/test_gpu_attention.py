@@ -86,6 +86,33 @@ def test_decode_attention_turbo3(N, n_splits):
     np.testing.assert_allclose(out, out1, rtol=0, atol=1e-3 * np.abs(ref).max())
 
 
+@pytest.mark.parametrize("B,N,n_splits,Hq,sparse", [(256, 256, 2, 32, False), (64, 1024, 8, 32, False), (512, 128, 1, 32, False),
+                                                     (256, 200, 2, 16, True), (256, 256, 4, 64, False)])
+def test_decode_attention_many_short_sequences(B, N, n_splits, Hq, sparse):
+    """Short contexts: a group has fewer splits than a workgroup has wavefronts, so several (batch, kv head) groups
+    share a workgroup and its decode tables (8, 2 and 16 groups per workgroup here; 2 with eight heads per pass),
+    each group merged by its own wavefronts.  Checked on a sample of the groups."""
+    Hkv = 8
+    tt = L.torch()
+    g = tt.Generator(device="cuda").manual_seed(B + N)
+    k = tt.randn((B * Hkv, N, D), generator=g, device="cuda").to(tt.float16)
+    v = tt.randn((B * Hkv, N, D), generator=g, device="cuda").to(tt.float16)
+    q = tt.randn((B, Hq, D), generator=g, device="cuda").to(tt.float16)
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    kp, vp = kc.store(k, kind="k"), vc.store(v, kind="v")
+    tau = 1e-3 if sparse else 0.0
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=tau)
+    out = np_(attn(q, kp, vp))
+    # oracle on a few sequences (all their kv heads), from the stored codes
+    per = tqa.packed_bytes(3, Hkv, N)
+    for b in (0, 1, B // 2 + 1, B - 1):
+        ref, sk, _ = reference_attention(np_(q[b:b + 1]), kc, vc, kp[b * per:(b + 1) * per], vp[b * per:(b + 1) * per], 1, Hq, Hkv, N,
+                                         1 / np.sqrt(D), n_splits=n_splits, tau=tau)
+        assert_close(out[b:b + 1], ref)
+    # and every row was written
+    assert np.isfinite(out).all()
+
+
 def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None):
     """Oracle attention for heads of 256 dims on the GPU-stored codes: the caches hold 2 N rows of 128 per sequence,
     row 2 t + half; a token's vector is its two rows side by side, each decoded and un-rotated by itself."""

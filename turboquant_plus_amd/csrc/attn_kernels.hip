@@ -215,6 +215,10 @@ struct AttnArgs {
     int n_groups, n_splits, tiles_per_split, n_tiles;
     int q_group, head_off;  // query heads per KV head; first of the (up to) four heads this launch works on
     int d256;               // heads of 256 dims: a token is two 128-value rows (2 token + half) of the K and V caches
+    int gpw;                // (batch, kv head) groups per workgroup: 1, or wavefronts per workgroup / n_splits when a group's
+                            // splits are fewer than a workgroup's wavefronts (short contexts: the groups share the decode tables)
+    int gw_shift;           // gpw > 1: log2(n_splits), a power of two then
+    int wgs_per_group;      // gpw == 1: n_splits / wavefronts per workgroup
     float tau;
 };
 
@@ -561,7 +565,6 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     // group's rotated queries (a region of its own: the tables are built while the queries are still on their way)
     constexpr int LUT_TOTAL = KLUT_BYTES + (SHARE ? 0 : lut_bytes(VBITS));
     __shared__ __attribute__((aligned(16))) char smem[LUT_TOTAL > 16 ? LUT_TOTAL : 16];
-    __shared__ __attribute__((aligned(16))) char q_stage[1024 * HG];
     __shared__ uint32_t lead;  // tiles finished by the wavefront that is furthest ahead
     __shared__ uint32_t skipped;  // Sparse V: (query, position) pairs skipped by this workgroup
     char *klut_s = smem;
@@ -570,9 +573,23 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     const int tid = threadIdx.x, lane = tid & 63;
     // workgroup-uniform values in scalar registers: tile loop, block addresses and bounds become scalar work
     const int n_waves = (int)(blockDim.x >> 6), wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wgs_per_group = a.n_splits / n_waves;
-    const int group = (int)(blockIdx.x / wgs_per_group), part = (int)(blockIdx.x % wgs_per_group);
-    const int split = part * n_waves + wave;  // index of this wavefront's partial
+    // Wavefronts of this workgroup that work on one group: all of them, or - short contexts, a.gpw groups per
+    // workgroup - as many as the group has splits; wave_g numbers them, tid_g their threads.
+    // (shifts and masks prepared by the host: an integer division here is a few dozen instructions in front of the
+    // first row request, which showed as half a microsecond per launch)
+    const int gw = a.gpw > 1 ? a.n_splits : n_waves;
+    const int wave_g = a.gpw > 1 ? (wave & (gw - 1)) : wave, wave0 = wave - wave_g;
+    const int gidx = a.gpw > 1 ? (wave >> a.gw_shift) : 0;   // this wavefront's group among the workgroup's
+    const int tid_g = tid - 64 * wave0;
+    const int wgs_per_group = a.wgs_per_group;
+    const int group = __builtin_amdgcn_readfirstlane(a.gpw > 1 ? (int)blockIdx.x * a.gpw + gidx : (int)(blockIdx.x / wgs_per_group));
+    const int part = a.gpw > 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(blockIdx.x % wgs_per_group));
+    const int split = part * n_waves + wave_g;  // index of this wavefront's partial
+    // dynamic LDS: the wavefronts' merge space (end of the split), then 1 KB per group and set of four heads that
+    // stages the rotated queries
+    extern __shared__ float merge_s[];
+    char *q_stage = reinterpret_cast<char *>(merge_s) + (n_waves > 1 ? (size_t)n_waves * HG * MERGE_FLOATS * sizeof(float) : 0) +
+                    (size_t)gidx * (1024 * HG);
     // The context length: a kernel argument, or read from memory when the caller replays one captured launch at
     // changing lengths (the split geometry then follows the length; a.tokens stays the bias rows' stride).
     int tokens_now = (int)a.tokens, n_tiles = a.n_tiles, tiles_per_split = a.tiles_per_split;
@@ -687,13 +704,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     // this wavefront's first head is requested now and rotated after the tables are built (the tables need only the
     // pair entries requested above, and nobody reads them before the barrier below)
     float xq0 = 0.0f, xq1 = 0.0f;
-    if (wave < 4 * HG) load_q(wave, xq0, xq1);
+    if (wave_g < 4 * HG) load_q(wave_g, xq0, xq1);
     if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
     if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
-    for (int h = wave; h < 4 * HG; h += n_waves) {
+    for (int h = wave_g; h < 4 * HG; h += gw) {
         _Float16 *qw = reinterpret_cast<_Float16 *>(q_stage) + h * 128;
         float x0 = xq0, x1 = xq1;
-        if (h != wave) load_q(h, x0, x1);
+        if (h != wave_g) load_q(h, x0, x1);
         if (a.ks1) {
             x0 *= a.ks1[2 * lane];
             x1 *= a.ks1[2 * lane + 1];
@@ -1061,7 +1078,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
         l_tot[1] = l_tot[0];
         m_run[1] = m_run[0];
     }
-    if (n_waves == 1) {
+    if (gw == 1) {
 #pragma unroll
         for (int hg = 0; hg < HG; ++hg) {
 #pragma unroll
@@ -1075,8 +1092,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
             }
         }
     } else {
-        // per wavefront and set of four heads: out[4][128], then m[4], l[4]
-        extern __shared__ float merge_s[];
+        // per wavefront and set of four heads: out[4][128], then m[4], l[4]; a group's wavefronts are wave0 .. wave0 + gw - 1
         constexpr int MS = MERGE_FLOATS * HG;
         float *mine = merge_s + wave * MS;
 #pragma unroll
@@ -1091,8 +1107,10 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
         for (int hg = 0; hg < HG; ++hg) {
             // head j's maximum over the wavefronts that saw an unmasked position
             M[hg] = -INFINITY;
-            for (int w = 0; w < n_waves; ++w)
-                if (merge_s[w * MS + hg * MERGE_FLOATS + 516 + j] > 0.0f) M[hg] = fmaxf(M[hg], merge_s[w * MS + hg * MERGE_FLOATS + 512 + j]);
+            const float *ml_g = merge_s + wave0 * MS + hg * MERGE_FLOATS;   // the group's first wavefront
+#pragma unroll 8
+            for (int w = 0; w < gw; ++w)
+                if (ml_g[w * MS + 516 + j] > 0.0f) M[hg] = fmaxf(M[hg], ml_g[w * MS + 512 + j]);
             const float f = l_tot[hg] > 0.0f ? __builtin_amdgcn_exp2f(m_run[hg] - M[hg]) : 0.0f;
             const float f4[4] = {dpp<0x00>(f), dpp<0x55>(f), dpp<0xAA>(f), dpp<0xFF>(f)};
 #pragma unroll
@@ -1102,19 +1120,23 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
                     mine[hg * MERGE_FLOATS + i * 128 + 64 * hf + lane] = (acc_o[hg][hf][0][i] + acc_o[hg][hf][1][i]) * f4[i];
         }
         __syncthreads();
-        for (int e = tid; e < 512 * HG; e += 64 * n_waves) {
+        for (int e = tid_g; e < 512 * HG; e += 64 * gw) {
             const int src = (e >> 9) * MERGE_FLOATS + (e & 511);  // partial element e = head e / 128, dim e % 128
             float sum = 0.0f;
-            for (int w = 0; w < n_waves; ++w) sum += merge_s[w * MS + src];
+            const float *col = merge_s + wave0 * MS + src;
+#pragma unroll 8
+            for (int w = 0; w < gw; ++w) sum += col[w * MS];
             st_dev(po + e, sum);
         }
-        if (tid < 4) {  // lanes 0..3 of wavefront 0 hold heads 0..3 of each set
+        if (tid_g < 4) {  // lanes 0..3 of the group's first wavefront hold heads 0..3 of each set
 #pragma unroll
             for (int hg = 0; hg < HG; ++hg) {
                 float L = 0.0f;
-                for (int w = 0; w < n_waves; ++w) {
-                    const float lw = merge_s[w * MS + hg * MERGE_FLOATS + 516 + j];
-                    if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(merge_s[w * MS + hg * MERGE_FLOATS + 512 + j] - M[hg]), L);
+                const float *ml_g = merge_s + wave0 * MS + hg * MERGE_FLOATS;
+#pragma unroll 8
+                for (int w = 0; w < gw; ++w) {
+                    const float lw = ml_g[w * MS + 516 + j];
+                    if (lw > 0.0f) L = fmaf(lw, __builtin_amdgcn_exp2f(ml_g[w * MS + 512 + j] - M[hg]), L);
                 }
                 st_dev(pml + 2 * (4 * hg + j), M[hg]);
                 st_dev(pml + 2 * (4 * hg + j) + 1, L);
@@ -1179,11 +1201,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
             }
         }
     }
-    {
-        // the wavefronts' merge space is free again (every partial of this workgroup is in memory)
-        extern __shared__ float merge_s[];
-        merge_group<HG>(a, group, n_parts, tid, n_waves, n_waves > 1 ? merge_s : nullptr);
-    }
+    // the wavefronts' merge space is free again (every partial of this workgroup is in memory); with several groups
+    // per workgroup every group's wavefronts finish their own group (one partial: no exchange between them)
+    merge_group<HG>(a, group, n_parts, tid_g, gw, n_waves > 1 && a.gpw <= 1 ? merge_s : nullptr);
     if (n_parts > 1 && tid == 0) st_dev(a.flags + (int64_t)group * n_parts, 0ull);  // a replay of a captured launch (same tag) starts from zero
     if constexpr (SPARSE) {
         if (a.poll_slots) {
@@ -1242,7 +1262,7 @@ struct WsLayout {
 // heads), wavefronts per workgroup (the largest power of two up to the variant's limit that divides the split
 // count) and workgroups = partials per group.
 struct AttnPlan {
-    int hg, wpw, n_parts;
+    int hg, wpw, n_parts, gpw;
 };
 AttnPlan attn_plan(const tq_attn_params *p) {
     AttnPlan pl;
@@ -1253,6 +1273,20 @@ AttnPlan attn_plan(const tq_attn_params *p) {
     // few groups (small batches): smaller workgroups, so that every CU gets one (a tile costs a wavefront the same
     // issue time however many share the SIMD)
     const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
+    // short contexts: a group has fewer splits than a workgroup has room for wavefronts.  Several groups then share a
+    // workgroup (and its decode tables), provided that still makes a workgroup per CU
+    const int wmax = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
+    pl.gpw = 1;
+    if (p->n_splits < wmax && wmax % p->n_splits == 0) {
+        int g = wmax / p->n_splits;
+        while (g > 1 && (groups % g != 0 || groups / g < 256)) g >>= 1;
+        if (g > 1) {
+            pl.gpw = g;
+            pl.wpw = g * p->n_splits;
+            pl.n_parts = 1;
+            return pl;
+        }
+    }
     while (pl.wpw > 4 && groups * (p->n_splits / pl.wpw) < 256) pl.wpw >>= 1;
     pl.n_parts = p->n_splits / pl.wpw;
     return pl;
@@ -1358,10 +1392,15 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     // that divides the split count
     const AttnPlan pl = attn_plan(p);
     const int wpw = pl.wpw, hg = pl.hg;
-    const unsigned grid = (unsigned)((int64_t)groups * pl.n_parts);
+    const unsigned grid = (unsigned)((int64_t)groups * pl.n_parts / pl.gpw);
     const unsigned wg = 64u * (unsigned)wpw;
     const int n_parts = pl.n_parts;  // partials per group: the wavefronts of a workgroup merge theirs in LDS
-    const size_t merge_bytes = wpw > 1 ? (size_t)wpw * hg * MERGE_FLOATS * sizeof(float) : 0;
+    // dynamic LDS: the wavefronts' merge space, then the staged queries of the workgroup's groups
+    const size_t merge_bytes = (wpw > 1 ? (size_t)wpw * hg * MERGE_FLOATS * sizeof(float) : 0) + (size_t)pl.gpw * 1024 * hg;
+    a.gpw = pl.gpw;
+    a.gw_shift = 0;
+    while ((1 << a.gw_shift) < p->n_splits) ++a.gw_shift;
+    a.wgs_per_group = pl.gpw > 1 ? 1 : p->n_splits / wpw;
     const int vb = turbo_v ? hv->bits : 8;
     const int kb = turbo_k ? hk->bits : 8;
     // The kernels work on four query heads of a KV head at a time (the 4-row MFMA block), or on eight (two sets
