@@ -306,7 +306,8 @@ typedef struct tq_attn_params {
                                            /* q and out are [batch, n_q_heads, 256].  V turbo */
                                            /* (K turbo of the same width, of 4|2, 3|2, 4|3    */
                                            /* bits, or q8_0-style rows written the same way   */
-                                           /* by tq_q8_0_store), dense, no bias               */
+                                           /* by tq_q8_0_store); Sparse V tests tiles of 32   */
+                                           /* tokens; bias rows and lists count tokens        */
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four

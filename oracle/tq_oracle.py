@@ -812,7 +812,7 @@ def softmax_rows(s):
 
 
 def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
-                     logit_bias=None):
+                     logit_bias=None, tile=64):
     """One (batch, kv-head) group.
 
     q_rot [G,128] queries already rotated by the K rotation; k_rot / v_rot
@@ -821,7 +821,8 @@ def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
     transpose once), the fraction of (query, position) pairs whose V row was
     skipped, and the fraction with final softmax weight < tau.
 
-    Splits are runs of ceil(ceil(N/64) / n_splits) tiles of 64 positions.
+    Splits are runs of ceil(ceil(N/tile) / n_splits) tiles of `tile` positions (64; 32 for
+    heads of 256 dims, whose tokens take two rows of a 64-row tile).
     Sparse V: within split s the running maximum is the maximum over the
     positions of that split seen so far in tiles of 64; a position's V row is
     skipped for query g when exp(s_i - m_running) < tau.  Softmax statistics
@@ -835,9 +836,9 @@ def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
     p_final = softmax_rows(s)
     if sparse_v_tau <= 0.0:
         return p_final @ v_rot, 0.0, 0.0
-    n_tiles = -(-N // 64)
+    n_tiles = -(-N // tile)
     tiles_per_split = -(-n_tiles // n_splits)
-    bounds = np.minimum(np.arange(n_splits + 1) * tiles_per_split * 64, N)
+    bounds = np.minimum(np.arange(n_splits + 1) * tiles_per_split * tile, N)
     num = np.zeros((G, v_rot.shape[1]))
     den = np.zeros(G)
     m_all = np.full(G, -np.inf)
@@ -848,8 +849,8 @@ def decode_attention(q_rot, k_rot, v_rot, scale, n_splits=1, sparse_v_tau=0.0,
         m = np.full(G, -np.inf)
         acc = np.zeros((G, v_rot.shape[1]))
         l = np.zeros(G)
-        for c in range(a, b, 64):
-            sc = s[:, c:min(c + 64, b)]
+        for c in range(a, b, tile):
+            sc = s[:, c:min(c + tile, b)]
             m_new = np.maximum(m, sc.max(axis=1))
             corr = np.exp(m - m_new)
             w = np.exp(sc - m_new[:, None])

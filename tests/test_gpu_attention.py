@@ -113,7 +113,7 @@ def test_decode_attention_many_short_sequences(B, N, n_splits, Hq, sparse):
     assert np.isfinite(out).all()
 
 
-def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None):
+def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None, n_splits=1, tau=0.0, bias=None):
     """Oracle attention for heads of 256 dims on the GPU-stored codes: the caches hold 2 N rows of 128 per sequence,
     row 2 t + half; a token's vector is its two rows side by side, each decoded and un-rotated by itself."""
     G = Hq // Hkv
@@ -128,13 +128,17 @@ def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale,
     vi, vg = vc.unpack_codes(v_packed, B * Hkv, 2 * N, kind="v")
     v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids).reshape(B * Hkv, N, 2 * D)
     out = np.zeros((B, Hq, 2 * D))
+    skipped = 0.0
     for b in range(B):
         for h in range(Hkv):
             g = b * Hkv + h
-            o, _, _ = O.decode_attention(q_rot[b, h * G:(h + 1) * G], k_rot[g], v_rot[g], scale)
+            bb = None if bias is None else bias[b, h * G:(h + 1) * G]
+            o, sk, _ = O.decode_attention(q_rot[b, h * G:(h + 1) * G], k_rot[g], v_rot[g], scale, n_splits=n_splits,
+                                          sparse_v_tau=tau, logit_bias=bb, tile=32)
             o = O.rotate_fast(o.reshape(G, 2, D), vc.signs1, vc.signs2, D, transpose=True)
             out[b, h * G:(h + 1) * G] = o.reshape(G, 2 * D)
-    return out
+            skipped += sk
+    return (out, skipped / (B * Hkv)) if tau > 0 else out
 
 
 @pytest.mark.parametrize("bits", [3, 4, 2])
@@ -209,6 +213,40 @@ def test_decode_attention_head_dim_256_grows_by_append():
         np.testing.assert_allclose(out, want, rtol=0, atol=2e-3 * np.abs(want).max())
 
 
+@pytest.mark.parametrize("N,n_splits", [(100, 1), (2048 + 31, 8), (4096, 32)])
+def test_decode_attention_head_dim_256_sparse_v_and_bias(N, n_splits):
+    """256-dim heads with Sparse V (the skip test runs on tiles of 32 tokens: a token is two rows of a 64-row tile),
+    a dense logit bias, a sparse one, and both."""
+    B, Hq, Hkv = 2, 8, 2
+    rng = np.random.default_rng(N)
+    k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+    kp, vp = kc.store(tqa.rows_of_256(k), kind="k"), vc.store(tqa.rows_of_256(v), kind="v")
+    q = (2.0 * rng.standard_normal((B, Hq, 2 * D))).astype(np.float16)
+    scale = 1 / np.sqrt(2 * D)
+    tau = 1e-3
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256, sparse_v_tau=tau)
+    out = np_(attn(q, kp, vp)).copy()
+    ref, sk = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, scale, n_splits=n_splits, tau=tau)
+    assert_close(out, ref)
+    assert abs(attn.skip_rate() - sk) < 2e-3 and sk > 0.05
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    bias[:, :, : min(4, N)] = 3.0
+    bias[:, 1::2, N - 1] = -2.0
+    bias[0, 0, N // 2] = 5.0
+    dense = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256)
+    ref_b = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, scale, bias=bias.astype(np.float64))
+    bd = L.torch().from_numpy(bias).cuda()
+    assert_close(np_(dense(q, kp, vp, bias=bd)), ref_b)
+    assert_close(np_(dense(q, kp, vp, sparse_bias=tqa.sparse_bias_from_dense(bd))), ref_b)
+    half = bd.clone()
+    half[:, :, N // 2:] = 0
+    assert_close(np_(dense(q, kp, vp, bias=half, sparse_bias=tqa.sparse_bias_from_dense(bd - half))), ref_b)
+    out_sb, sk_b = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, scale, n_splits=n_splits, tau=tau, bias=bias.astype(np.float64))
+    assert_close(np_(attn(q, kp, vp, sparse_bias=tqa.sparse_bias_from_dense(bd))), out_sb)
+
+
 def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
     B, Hq, Hkv, N = 1, 4, 1, 128
     kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
@@ -216,11 +254,9 @@ def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
     buf = tt.zeros(tqa.packed_bytes(3, B * Hkv, 2 * N), dtype=tt.uint8, device="cuda")
     q = tt.zeros((B, Hq, 256), dtype=tt.float16, device="cuda")
     with pytest.raises(NotImplementedError):
-        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256, sparse_v_tau=1e-3)(q, buf, buf)
-    with pytest.raises(NotImplementedError):
         tqa.DecodeAttention(tqa.TurboCodec(2, seed=42), vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf)   # K narrower than V
     with pytest.raises(NotImplementedError):
-        tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf, bias=tt.zeros((B, Hq, N), device="cuda"))
+        tqa.DecodeAttention(kc, None, B, Hq, Hkv, N, head_dim=256)(q, buf, buf)                          # q8_0-style V rows
     with pytest.raises(ValueError):
         tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=64)
 

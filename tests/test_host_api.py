@@ -44,13 +44,20 @@ def test_size_entry_points_need_no_gpu():
     assert lib.tq_q8_0_bytes(1, 128) == 128 * 136
     p = L.TQAttnParams(batch=16, n_q_heads=32, n_kv_heads=8, tokens=32768, n_splits=16,
                        k_format=L.KFMT_TURBO, scale=0.088, sparse_v_tau=0.0)
-    # one partial (four heads x (128 outputs + maximum + sum)) per workgroup, and the 16 splits of a group are one workgroup
+    # one partial (four heads x (128 outputs + maximum + sum)) per workgroup; the 16 splits of a group go to two
+    # workgroups of eight wavefronts (128 workgroups of sixteen would leave half of the CUs without one)
     one_per_group = 16 * 8 * 4 * 130 * 4
-    assert one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 2 * one_per_group
+    assert 2 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 3 * one_per_group
+    p.batch = 64                                           # 512 groups: sixteen splits are one workgroup
+    assert 4 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 5 * one_per_group
     p.n_q_heads = 16                                       # groups of 2: two of the four head rows per pass idle
-    assert one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 2 * one_per_group
+    assert 4 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 5 * one_per_group
+    p.batch = 16
     p.n_q_heads, p.n_splits = 64, 32                       # groups of 8: eight heads per pass, eight wavefronts per workgroup
     assert 4 * 2 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 4 * 2 * one_per_group + 65536
+    p.n_q_heads, p.n_splits, p.head_dim = 32, 32, 256      # heads of 256 dims: two accumulator sets, like eight heads per pass
+    assert 4 * 2 * one_per_group <= lib.tq_attn_workspace_bytes(C.byref(p)) < 4 * 2 * one_per_group + 65536
+    p.head_dim = 0
     p.n_splits = 16
     p.n_q_heads = 20                                       # not a multiple of the KV head count
     assert lib.tq_attn_workspace_bytes(C.byref(p)) == -1

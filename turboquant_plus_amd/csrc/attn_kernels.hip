@@ -546,14 +546,14 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 
 // SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
 // registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
-// D256: heads of 256 dims (turbo or q8_0-style K, turbo V, dense, no bias).  A token is rows 2 token and 2 token + 1 of caches that are
+// D256: heads of 256 dims (turbo or q8_0-style K, turbo V).  A token is rows 2 token and 2 token + 1 of caches that are
 // otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
 // then the output's two halves of one set of four heads: one softmax, two accumulator sets.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
 __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KFMT == KFMT_TURBO ? 4 : 1) void k_decode_attn(AttnArgs a) {
     // (256-dim heads on turbo K rows: four wavefronts per SIMD = two workgroups of eight per CU, i.e. at most 128 registers - the
     // variant sits at 119-136 without the bound, and one register over 128 halves its occupancy)
-    static_assert(!D256 || (HG == 2 && VBITS != 8 && !SPARSE && !SBIAS), "256-dim heads: turbo V, dense");
+    static_assert(!D256 || (HG == 2 && VBITS != 8), "256-dim heads: turbo V rows");
     constexpr int HQ = D256 ? 1 : HG;   // sets of four heads whose logits and softmax state the wavefront keeps
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
@@ -607,6 +607,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     // K row of the tile that this lane owns, and the tile row of element i of its logits (e4 + es * i)
     const int krow = D256 ? 2 * (lane & 31) + (lane >> 5) : lane;
     const int e4 = D256 ? 2 * (b4 & 31) : b4, es = D256 ? 2 : 1;
+    // tokens per tile, and the first of this lane's four tokens inside the tile
+    constexpr int TT = D256 ? 32 : 64;
+    const int t4 = D256 ? (b4 & 31) : b4;
 
     const uint8_t *kbase = a.k + (int64_t)group * a.blocks_per_seq * KBLOCK;
     const uint8_t *vbase = a.v + (int64_t)group * a.blocks_per_seq * VBLOCK;
@@ -761,7 +764,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
 #pragma unroll
         for (int i = 0; i < 4; ++i) bv[i] = 0.0f;
         if (!a.bias) return;
-        const int tk = t * 64 + b4;  // the launcher checks tokens < 2^31
+        const int tk = t * TT + t4;  // the launcher checks tokens < 2^31
         const float *row = a.bias + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.tokens;
         if (bias_vec && tk + 3 < tokens_now) {
             const float4 v = *reinterpret_cast<const float4 *>(row + tk);
@@ -774,7 +777,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     };
     float bias_next[HG][4];
 #pragma unroll
-    for (int hg = 0; hg < HG; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
+    for (int hg = 0; hg < HQ; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
     // Sparse bias: a head's (position, value) list is walked by a cursor as the tiles go by.  The cursor starts at the
     // head's first entry inside this split: the number of entries below the split's first token, counted with the
     // whole wavefront (one entry per lane and round); the sixteen lanes that hold a head's logits move in step.
@@ -789,9 +792,9 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     // entry e of the list of this lane's head in set hg (addresses are formed where they are needed: the path is rare)
     auto sb_entry = [&](int hg, int e) { return ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.sbias_n + e; };
     if constexpr (SBIAS) {
-        const int first_tok = t_begin * 64;
+        const int first_tok = t_begin * TT;
 #pragma unroll
-        for (int hg = 0; hg < HG; ++hg) {
+        for (int hg = 0; hg < HQ; ++hg) {
             int below[4];
 #pragma unroll
             for (int h = 0; h < 4; ++h) {
@@ -841,19 +844,19 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
         // the bias of this tile was requested a tile ago, like the rows; now the next tile's
         float bias4[HG][4];
 #pragma unroll
-        for (int hg = 0; hg < HG; ++hg) {
+        for (int hg = 0; hg < HQ; ++hg) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) bias4[hg][i] = bias_next[hg][i] * LOG2E;
             load_bias(tile_n, hg, bias_next[hg]);
         }
         if constexpr (SBIAS) {
             // entries of this tile (a handful per head and context: the loop body runs for few tiles)
-            const int tile_hi = tile * 64 + 64;
+            const int tile_hi = tile * TT + TT;
 #pragma unroll
-            for (int hg = 0; hg < HG; ++hg) {
+            for (int hg = 0; hg < HQ; ++hg) {
                 while (__builtin_amdgcn_ballot_w64(sb_pos[hg] < tile_hi) != 0ull) {
                     if (sb_pos[hg] < tile_hi) {
-                        const int d = sb_pos[hg] - tile * 64 - b4;  // an entry at an earlier position than the cursor expects is dropped
+                        const int d = sb_pos[hg] - tile * TT - t4;  // an entry at an earlier position than the cursor expects is dropped
                         const float add = sb_val[hg] * LOG2E;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) bias4[hg][i] += d == i ? add : 0.0f;
@@ -925,7 +928,7 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
         if constexpr (SPARSE) {
             if (n_valid < 64) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) token_ok[i] = __builtin_amdgcn_ballot_w64(b4 + i < n_valid);
+                for (int i = 0; i < 4; ++i) token_ok[i] = __builtin_amdgcn_ballot_w64(e4 + es * i < n_valid);
             }
         }
 #pragma unroll
@@ -970,7 +973,8 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
                 if constexpr (SPARSE) {
                     const bool keep = p[hg][i] >= a.tau;
                     const unsigned long long keep_m = __builtin_amdgcn_ballot_w64(keep);
-                    const unsigned long long in_range = token_ok[i] & head_ok[hg];
+                    // 256-dim heads: both half-wavefronts hold the same 32 tokens; the lower one counts
+                    const unsigned long long in_range = token_ok[i] & head_ok[hg] & (D256 ? 0xFFFFFFFFull : ~0ull);
                     nskip += (unsigned)__builtin_popcountll(in_range & ~keep_m);
                     if (!keep) p[hg][i] = 0.0f;
                     any_keep |= keep_m & in_range;
@@ -1325,8 +1329,8 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: head_dim %d (128 or 256)", (int)p->head_dim);
         return TQ_ERR_UNSUPPORTED;
     }
-    if (d256 && (p->v_format != TQ_KFMT_TURBO || !hv || p->sparse_v_tau > 0.0f || bias || p->bias_entries)) {
-        tq_set_error("tq_decode_attention: head_dim 256 takes turbo V rows, dense, without bias");
+    if (d256 && (p->v_format != TQ_KFMT_TURBO || !hv)) {
+        tq_set_error("tq_decode_attention: head_dim 256 takes turbo V rows");
         return TQ_ERR_UNSUPPORTED;
     }
     const int64_t cache_rows = (d256 ? 2 : 1) * p->tokens;   // a 256-dim token is two rows of the caches
@@ -1427,10 +1431,17 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         a.pass = a.head_off / heads_per_pass;
         a.nonce = next_nonce();
         if (d256) {
-#define TQ_ATTN_256(B)                                                                                                  \
-    if (share) k_decode_attn<KFMT_TURBO, B, B, false, true, 2, false, true><<<grid, wg, merge_bytes, s>>>(a);           \
-    else k_decode_attn<KFMT_TURBO, B, B, false, false, 2, false, true><<<grid, wg, merge_bytes, s>>>(a)
-#define TQ_ATTN_256X(KF, KB, VB) k_decode_attn<KF, KB, VB, false, false, 2, false, true><<<grid, wg, merge_bytes, s>>>(a)
+#define TQ_ATTN_256_ONE(KF, KB, VB, SH)                                                                              \
+    {                                                                                                                 \
+        if (sparse && a.sbias_n) k_decode_attn<KF, KB, VB, true, SH, 2, true, true><<<grid, wg, merge_bytes, s>>>(a);  \
+        else if (sparse) k_decode_attn<KF, KB, VB, true, SH, 2, false, true><<<grid, wg, merge_bytes, s>>>(a);         \
+        else if (a.sbias_n) k_decode_attn<KF, KB, VB, false, SH, 2, true, true><<<grid, wg, merge_bytes, s>>>(a);      \
+        else k_decode_attn<KF, KB, VB, false, SH, 2, false, true><<<grid, wg, merge_bytes, s>>>(a);                   \
+    }
+#define TQ_ATTN_256(B)                                   \
+    if (share) TQ_ATTN_256_ONE(KFMT_TURBO, B, B, true)   \
+    else TQ_ATTN_256_ONE(KFMT_TURBO, B, B, false)
+#define TQ_ATTN_256X(KF, KB, VB) TQ_ATTN_256_ONE(KF, KB, VB, false)
             if (turbo_k && kb == vb && kb == 3) { TQ_ATTN_256(3); }
             else if (turbo_k && kb == vb && kb == 4) { TQ_ATTN_256(4); }
             else if (turbo_k && kb == vb && kb == 2) { TQ_ATTN_256(2); }
@@ -1446,10 +1457,8 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
             }
 #undef TQ_ATTN_256
 #undef TQ_ATTN_256X
-            rc = tq_check_launch("decode_attn (256-dim heads)");
-            if (rc) return rc;
-            continue;
-        }
+#undef TQ_ATTN_256_ONE
+        } else {
 #define TQ_ATTN_ONE(KF, KB, VB, SP, SH)                                            \
     {                                                                             \
         if (hg == 2 && a.sbias_n) k_decode_attn<KF, KB, VB, SP, SH, 2, true><<<grid, wg, merge_bytes, s>>>(a);   \
@@ -1486,6 +1495,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: unsupported K/V format pair (k bits %d, v bits %d)", kb, vb);
         return TQ_ERR_UNSUPPORTED;
     }
+        }
 #undef TQ_ATTN
 #undef TQ_ATTN_SAME
 #undef TQ_ATTN_ONE
