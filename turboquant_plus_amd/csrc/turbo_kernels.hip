@@ -3627,86 +3627,6 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
 __host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 68 : 34; }
 __host__ __device__ constexpr int fork_codes_offset(int bits) { return bits == 4 ? 4 : 2; }
 
-// Sixteen lanes per row: lane li owns the codes of dims 8 li .. 8 li + 7, which are whole bytes of the fork's row in
-// every width (4-bit: four nibble bytes; 3-bit: two qs bytes and one signs byte; 2-bit: two qs bytes).
-template <int BITS>
-__global__ __launch_bounds__(256) void k_fork_export(const uint8_t *packed, uint8_t *out, int kind, int64_t tokens,
-                                                     int64_t blocks_per_seq) {
-    constexpr int FB = fork_block_bytes(BITS);
-    constexpr int SRC_BYTES = block_bytes(BITS);
-    __shared__ __attribute__((aligned(16))) uint8_t block_s[SRC_BYTES];  // the block, copied with 16-byte loads
-    const int tid = threadIdx.x, li = tid & 15, grp = tid >> 4;
-    const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
-    {
-        const uint4 *sb = reinterpret_cast<const uint4 *>(packed + blk * SRC_BYTES);
-        for (int e = tid; e < SRC_BYTES / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = sb[e];
-    }
-    __syncthreads();
-#pragma unroll 1
-    for (int it = 0; it < 8; ++it) {
-        const int t = it * 16 + grp;
-        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
-        if (tok >= tokens) continue;
-        const uint32_t w = load_codes8<BITS>(block_s, kind, t, li);  // code m at bit m BITS
-        uint8_t *row = out + (seq * tokens + tok) * FB;             // FB is even: the row is 2-byte aligned
-        if (li == 0) *reinterpret_cast<uint16_t *>(row) = reinterpret_cast<const uint16_t *>(block_s + block_code_bytes(BITS))[t];
-        if constexpr (BITS == 4) {
-            if (li == 1) *reinterpret_cast<uint16_t *>(row + 2) = 0;  // the unused rnorm slot
-            *reinterpret_cast<uint32_t *>(row + 4 + 4 * li) = w;       // 68-byte rows: the codes are 4-byte aligned
-        } else if constexpr (BITS == 2) {
-            reinterpret_cast<uint16_t *>(row + 2)[li] = (uint16_t)w;
-        } else {
-            uint32_t qs = 0, sg = 0;
-#pragma unroll
-            for (int m = 0; m < 8; ++m) {
-                const uint32_t c = (w >> (3 * m)) & 7u;
-                qs |= (c & 3u) << (2 * m);
-                sg |= (c >> 2) << m;
-            }
-            reinterpret_cast<uint16_t *>(row + 2)[li] = (uint16_t)qs;
-            row[34 + li] = (uint8_t)sg;
-        }
-    }
-}
-
-template <int BITS>
-__global__ __launch_bounds__(256) void k_fork_import(const uint8_t *in, uint8_t *packed, int kind, int64_t tokens,
-                                                     int64_t blocks_per_seq, uint32_t zero_code) {
-    constexpr int FB = fork_block_bytes(BITS);
-    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
-    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
-    const int tid = threadIdx.x, li = tid & 15, grp = tid >> 4;
-    const int64_t blk = blockIdx.x, seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
-#pragma unroll 1
-    for (int it = 0; it < 8; ++it) {
-        const int t = it * 16 + grp;
-        const int64_t tok = bis * TQ_ROWS_PER_BLOCK + t;
-        uint32_t c[8];
-        float g = 0.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) c[m] = zero_code;  // rows past the end: what the store kernels write there
-        if (tok < tokens) {
-            const uint8_t *row = in + (seq * tokens + tok) * FB;
-            g = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(row)));
-            if constexpr (BITS == 4) {
-                const uint32_t w = *reinterpret_cast<const uint32_t *>(row + 4 + 4 * li);
-#pragma unroll
-                for (int m = 0; m < 8; ++m) c[m] = (w >> (4 * m)) & 15u;
-            } else {
-                const uint32_t qs = reinterpret_cast<const uint16_t *>(row + 2)[li];
-                const uint32_t sg = BITS == 3 ? row[34 + li] : 0u;
-#pragma unroll
-                for (int m = 0; m < 8; ++m) c[m] = ((qs >> (2 * m)) & 3u) | (((sg >> m) & 1u) << 2);
-            }
-        }
-        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) =
-            make_uint2(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
-        if (li == 0) norms_s[t] = g;
-    }
-    __syncthreads();
-    pack_block<BITS, 256>(codes, norms_s, packed + blk * block_bytes(BITS), kind);
-}
-
 // ---- K rows of the fork layout: a lane owns a token ------------------------------------------------
 // The fork rows of one of this library's K blocks are 128 * FB contiguous bytes.  They move between memory and LDS
 // as 16-byte pieces (the stage keeps the address's low four bits, so a piece is aligned on both sides; what comes
@@ -3876,6 +3796,236 @@ __global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed
     }
 }
 
+// ---- V rows of the fork layout: a wavefront owns a 64-token tile ------------------------------------
+// A V tile holds its 64 tokens dim-major (lane l of the wavefront = packed row l = dims l and l + 64), the fork's rows
+// are token-major, so the tile is transposed on the way - in units of four codes (a 16-bit piece: four tokens of one
+// dim on the V side, four dims of one token on the token side) through 32 LDS rows of 64 pieces: every lane writes
+// its 32 pieces, one per row, then reads two rows' worth of 8-byte groups and keeps one code of each piece.  Rows
+// are 136 bytes apart, so that lanes reading different rows hit different banks.  The token side then is what the
+// K kernel has: a lane owns a token, takes or puts its fork row in the wavefront's stage, and the stage moves
+// between LDS and memory in 16-byte pieces.
+constexpr int FORK_V_WAVES = 8, FORK_X_ROW = 136;
+
+// a row's sixteen words of eight codes (word j of group q) <-> its packed dwords
+template <int BITS> __device__ __forceinline__ void words_from_packed(const uint32_t (&w)[4 * BITS], uint32_t (&cw)[4][4]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (BITS == 4) cw[q][j] = w[4 * j + q];
+            else if constexpr (BITS == 2) cw[q][j] = (w[4 * (j >> 1) + q] >> (16 * (j & 1))) & 0xFFFFu;
+            else cw[q][j] = j < 3 ? (w[4 * j + q] & 0xFFFFFFu) : tail24(w, q);
+        }
+}
+template <int BITS> __device__ __forceinline__ void packed_from_words(const uint32_t (&cw)[4][4], uint32_t (&w)[4 * BITS]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[4 * j + q] = cw[q][j];
+        } else if constexpr (BITS == 2) {
+            w[q] = cw[q][0] | (cw[q][1] << 16);
+            w[4 + q] = cw[q][2] | (cw[q][3] << 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) w[4 * j + q] = cw[q][j] | (((cw[q][3] >> (8 * j)) & 0xFFu) << 24);
+        }
+    }
+}
+// code number `slot` of each of the four 16-bit pieces of an 8-byte group, as four codes side by side
+template <int BITS> __device__ __forceinline__ uint32_t pick_codes(uint2 d, int off_lo, int off_hi) {
+    const uint32_t a = __builtin_amdgcn_ubfe(d.x, off_lo, BITS) | (__builtin_amdgcn_ubfe(d.x, off_hi, BITS) << BITS);
+    const uint32_t b = __builtin_amdgcn_ubfe(d.y, off_lo, BITS) | (__builtin_amdgcn_ubfe(d.y, off_hi, BITS) << BITS);
+    return a | (b << (2 * BITS));
+}
+
+template <int BITS, bool TO_FORK>
+__global__ __launch_bounds__(64 * FORK_V_WAVES) void k_fork_v(const uint8_t *packed_in, uint8_t *packed_out, const uint8_t *fork_in,
+                                                              uint8_t *fork_out, int64_t tokens, int64_t blocks_per_seq,
+                                                              uint32_t zero_code, uint32_t n_blocks) {
+    constexpr int FB = fork_block_bytes(BITS);
+    constexpr uint32_t QM = (1u << (4 * BITS)) - 1u;   // four codes
+    __shared__ __attribute__((aligned(16))) uint8_t stage_s[FORK_V_WAVES][64 * FB + 16];
+    __shared__ __attribute__((aligned(8))) uint8_t xs_s[FORK_V_WAVES][32 * FORK_X_ROW];
+    __shared__ uint16_t spread2_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of four 2-bit fields -> the fields at a stride of 3
+    __shared__ uint32_t spread1_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of eight sign bits -> bit 3m + 2
+    __shared__ uint16_t gather_s[BITS == 3 && TO_FORK ? 4096 : 1];    // four 3-bit codes -> their low bits (8) | their top bits << 8
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if constexpr (BITS == 3 && !TO_FORK) {
+        if (tid < 256) {
+            uint32_t a = 0, b = 0;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) a |= ((tid >> (2 * m)) & 3u) << (3 * m);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) b |= ((tid >> m) & 1u) << (3 * m + 2);
+            spread2_s[tid] = (uint16_t)a;
+            spread1_s[tid] = b;
+        }
+    }
+    if constexpr (BITS == 3 && TO_FORK) {
+        for (int e = tid; e < 4096; e += 64 * FORK_V_WAVES) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const uint32_t c = (e >> (3 * m)) & 7u;
+                lo |= (c & 3u) << (2 * m);
+                hi |= (c >> 2) << m;
+            }
+            gather_s[e] = (uint16_t)(lo | (hi << 8));
+        }
+    }
+    const uint32_t tile = FORK_V_WAVES * blockIdx.x + wave;
+    const bool live = tile < 2 * n_blocks;
+    const uint32_t blk = live ? tile >> 1 : 0;
+    const int half = (int)(tile & 1);
+    const int64_t seq = blk / blocks_per_seq, bis = blk % blocks_per_seq;
+    const int64_t tok0 = bis * TQ_ROWS_PER_BLOCK + half * 64;
+    const int rows = !live || tokens <= tok0 ? 0 : tokens - tok0 < 64 ? (int)(tokens - tok0) : 64;
+    uint8_t *fork_rows = const_cast<uint8_t *>(TO_FORK ? fork_out : fork_in) + (seq * tokens + tok0) * FB;
+    const int mis = (int)(reinterpret_cast<uintptr_t>(fork_rows) & 15);
+    uint8_t *stage = stage_s[wave], *xs = xs_s[wave];
+    uint8_t *mine = stage + mis + lane * FB;       // this lane's token's row in the stage
+    const int off_lo = BITS * (lane & 3), off_hi = 16 + off_lo;
+    uint32_t vw[4][4], kw[4][4];                  // V row (lane = packed row) and token row (lane = token), as words of eight codes
+    uint32_t w[4 * BITS];
+    uint16_t nrm = 0;
+    __syncthreads();   // the tables
+    if (!live) return;
+
+    if constexpr (TO_FORK) {
+        const uint8_t *sb = packed_in + (int64_t)blk * block_bytes(BITS);
+        const int prow = half * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < BITS; ++j) {
+            const uint4 c = *reinterpret_cast<const uint4 *>(sb + j * 2048 + prow * 16);
+            w[4 * j] = c.x; w[4 * j + 1] = c.y; w[4 * j + 2] = c.z; w[4 * j + 3] = c.w;
+        }
+        nrm = reinterpret_cast<const uint16_t *>(sb + block_code_bytes(BITS))[prow];   // lane <-> token for the norms
+        words_from_packed<BITS>(w, vw);
+        // word (q, j): tokens 16 q + 4 j .. + 3 of dim l, then of dim l + 64 -> rows 2 (4 q + j) and + 1, column l
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint16_t *>(xs + (2 * (4 * q + j)) * FORK_X_ROW + 2 * lane) = (uint16_t)(vw[q][j] & QM);
+                *reinterpret_cast<uint16_t *>(xs + (2 * (4 * q + j) + 1) * FORK_X_ROW + 2 * lane) = (uint16_t)(vw[q][j] >> (4 * BITS));
+            }
+        __builtin_amdgcn_wave_barrier();
+        // token lane >> 2's group of four tokens, this token's place in it lane & 3: dims 32 q + 8 j .. + 7 sit in
+        // row 2 T + (q >> 1), columns 32 (q & 1) + 8 j .. + 7
+        const uint8_t *r0 = xs + (2 * (lane >> 2)) * FORK_X_ROW, *r1 = r0 + FORK_X_ROW;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint8_t *g = (q >> 1 ? r1 : r0) + 2 * (32 * (q & 1) + 8 * j);
+                kw[q][j] = pick_codes<BITS>(*reinterpret_cast<const uint2 *>(g), off_lo, off_hi) |
+                           (pick_codes<BITS>(*reinterpret_cast<const uint2 *>(g + 8), off_lo, off_hi) << (4 * BITS));
+            }
+        if (lane < rows) {
+            if constexpr (BITS == 4) {
+                uint32_t *d = reinterpret_cast<uint32_t *>(mine);   // 68-byte rows at a 4-byte aligned address
+                d[0] = nrm;                                         // norm, and 0 in the unused rnorm slot
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) d[1 + 4 * g + j] = kw[g][j];
+            } else if constexpr (BITS == 2) {
+                uint16_t *h = reinterpret_cast<uint16_t *>(mine);
+                h[0] = nrm;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) h[1 + 4 * g + j] = (uint16_t)kw[g][j];
+            } else {
+                uint16_t *h = reinterpret_cast<uint16_t *>(mine);
+                h[0] = nrm;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    uint32_t sg = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t e0 = gather_s[kw[g][j] & 0xFFFu], e1 = gather_s[kw[g][j] >> 12];
+                        h[1 + 4 * g + j] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
+                        sg |= ((e0 >> 8) | ((e1 >> 8) << 4)) << (8 * j);
+                    }
+                    h[17 + 2 * g] = (uint16_t)sg;
+                    h[18 + 2 * g] = (uint16_t)(sg >> 16);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        fork_stage_copy<FB>(stage, fork_rows, rows * FB, true, lane, 64);
+    } else {
+        fork_stage_copy<FB>(stage, fork_rows, rows * FB, false, lane, 64);
+        __builtin_amdgcn_wave_barrier();
+        if (lane < rows) {
+            if constexpr (BITS == 4) {
+                const uint32_t *d = reinterpret_cast<const uint32_t *>(mine);
+                nrm = (uint16_t)d[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) kw[g][j] = d[1 + 4 * g + j];
+            } else if constexpr (BITS == 2) {
+                const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
+                nrm = h[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) kw[g][j] = h[1 + 4 * g + j];
+            } else {
+                const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
+                nrm = h[0];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t sg = (uint32_t)h[17 + 2 * g] | ((uint32_t)h[18 + 2 * g] << 16);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t q = h[1 + 4 * g + j];
+                        kw[g][j] = (uint32_t)spread2_s[q & 0xFFu] | ((uint32_t)spread2_s[q >> 8] << 12) | spread1_s[(sg >> (8 * j)) & 0xFFu];
+                    }
+                }
+            }
+        } else {
+            // tokens past the sequence's end: the code of 0.0 and norm 0, as the store kernels write them
+            uint32_t fill = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) fill |= zero_code << (BITS * i);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) kw[g][j] = fill;
+        }
+        // word (q, j) of a token: dims 32 q + 8 j .. + 3 and .. + 4 .. + 7 -> rows 8 q + 2 j and + 1, column = token
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint16_t *>(xs + (8 * q + 2 * j) * FORK_X_ROW + 2 * lane) = (uint16_t)(kw[q][j] & QM);
+                *reinterpret_cast<uint16_t *>(xs + (8 * q + 2 * j + 1) * FORK_X_ROW + 2 * lane) = (uint16_t)(kw[q][j] >> (4 * BITS));
+            }
+        __builtin_amdgcn_wave_barrier();
+        // packed row l = dims l and l + 64: rows l >> 2 and 16 + (l >> 2), place l & 3 in a piece; word (q, j) = tokens 16 q + 4 j .. + 3
+        const uint8_t *r0 = xs + (lane >> 2) * FORK_X_ROW, *r1 = r0 + 16 * FORK_X_ROW;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = 2 * (16 * q + 4 * j);
+                vw[q][j] = pick_codes<BITS>(*reinterpret_cast<const uint2 *>(r0 + col), off_lo, off_hi) |
+                           (pick_codes<BITS>(*reinterpret_cast<const uint2 *>(r1 + col), off_lo, off_hi) << (4 * BITS));
+            }
+        packed_from_words<BITS>(vw, w);
+        uint8_t *db = packed_out + (int64_t)blk * block_bytes(BITS);
+        const int prow = half * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < BITS; ++j)
+            *reinterpret_cast<uint4 *>(db + j * 2048 + prow * 16) = make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]);
+        reinterpret_cast<uint16_t *>(db + block_code_bytes(BITS))[prow] = nrm;
+    }
+}
+
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                     hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
@@ -3884,14 +4034,16 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
     // index of 0.0: number of boundaries below it (a zero vector stores this code in every dim)
     uint32_t zero_code = (uint32_t)(h->n_centroids / 2);
     if (h->zero_code >= 0) zero_code = (uint32_t)h->zero_code;
-    const unsigned kgrid = (grid + 1) / 2;
+    const unsigned kgrid = (grid + 1) / 2, vgrid = (2 * grid + FORK_V_WAVES - 1) / FORK_V_WAVES;
 #define TQ_FORK(B)                                                                                                        \
     if (kind == TQ_KIND_K && to_fork)                                                                                     \
         k_fork_k<B, true><<<kgrid, FORK_K_THREADS, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
     else if (kind == TQ_KIND_K)                                                                                           \
         k_fork_k<B, false><<<kgrid, FORK_K_THREADS, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid); \
-    else if (to_fork) k_fork_export<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps);        \
-    else k_fork_import<B><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, kind, tokens, bps, zero_code)
+    else if (to_fork)                                                                                                     \
+        k_fork_v<B, true><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
+    else                                                                                                                  \
+        k_fork_v<B, false><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid)
     switch (h->bits) {
     case 2: TQ_FORK(2); break;
     case 3: TQ_FORK(3); break;
