@@ -3017,130 +3017,7 @@ int tqk_store(const tq_handle *h, const void *x, int64_t n_seqs, int64_t tokens,
 
 // ---- temporal decay: re-quantise packed rows to a narrower codebook ------------------------
 // Per row in the rotated domain: values = c_src[idx] * g, renormalise, nearest centroid of the
-// destination codebook, corrected norm for the new codes.  One workgroup per block: unpack into
-// the LDS stage, 16 lanes per row, pack with the destination width.
-struct RequantArgs {
-    const float *cent_src, *cent_dst, *bounds_dst;
-    int kind;
-    // The destination code of a source code depends on the row's S = sum of c_src[code]^2 alone, and for S inside
-    // (s_lo, s_hi) it is the fixed table t0 (4 bits per source code; requant_plan): such rows take their sums and codes
-    // from a table over pairs of codes; has_plan = 0 (more than 16 levels) leaves every row to the per-value code.
-    int has_plan;
-    unsigned long long t0;
-    float s_lo, s_hi, fix_unit;
-    float src_sq[16];        // c_src[k]^2
-    uint32_t dst_fix[16];    // c_dst[k]^2 / fix_unit, rounded: a row's 128 of them add up exactly in 32 bits
-};
-
-template <int SB, int DB>
-__global__ __launch_bounds__(256) void k_requantize(const uint8_t *src, uint8_t *dst, RequantArgs a) {
-    constexpr int NB = (1 << DB) - 1;
-    constexpr int SRC_BYTES = block_bytes(SB);
-    __shared__ __attribute__((aligned(16))) uint8_t block_s[SRC_BYTES];  // the source block, copied with 16-byte loads
-    __shared__ __attribute__((aligned(16))) uint8_t codes[TQ_ROWS_PER_BLOCK * CODE_STRIDE];
-    __shared__ float norms_s[TQ_ROWS_PER_BLOCK];
-    __shared__ float csrc_s[1 << SB], cdst_s[1 << DB];
-    constexpr int NPAIR = 1 << (2 * SB);
-    __shared__ uint2 pair_s[NPAIR];   // per pair of source codes: .x = sum of c_src^2 (fp32 bits), .y = its two t0 codes << 24 | fixed-point sum of c_dst[t0]^2
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int li = lane & 15, grp = tid >> 4;
-    {
-        const uint4 *sb = reinterpret_cast<const uint4 *>(src + (int64_t)blockIdx.x * SRC_BYTES);
-        for (int e = tid; e < SRC_BYTES / 16; e += 256) reinterpret_cast<uint4 *>(block_s)[e] = sb[e];
-    }
-    if (tid < (1 << SB)) csrc_s[tid] = a.cent_src[tid];
-    if (tid < (1 << DB)) cdst_s[tid] = a.cent_dst[tid];
-    if (a.has_plan && tid < NPAIR) {
-        // the argument arrays are indexed with constants only (they live in scalar registers)
-        const int k0 = tid & ((1 << SB) - 1), k1 = tid >> SB;
-        float q0 = 0.0f, q1 = 0.0f;
-#pragma unroll
-        for (int k = 0; k < (1 << SB); ++k) {
-            q0 = k0 == k ? a.src_sq[k] : q0;
-            q1 = k1 == k ? a.src_sq[k] : q1;
-        }
-        const uint32_t t0 = (uint32_t)((a.t0 >> (4 * k0)) & 15ull), t1 = (uint32_t)((a.t0 >> (4 * k1)) & 15ull);
-        uint32_t f0 = 0, f1 = 0;
-#pragma unroll
-        for (int k = 0; k < (1 << DB); ++k) {
-            f0 = t0 == (uint32_t)k ? a.dst_fix[k] : f0;
-            f1 = t1 == (uint32_t)k ? a.dst_fix[k] : f1;
-        }
-        pair_s[tid] = make_uint2(__float_as_uint(q0 + q1), ((t0 | (t1 << DB)) << 24) | (f0 + f1));
-    }
-    float bnd[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) bnd[k] = a.bounds_dst[k];
-    __syncthreads();
-#pragma unroll 1
-    for (int it = 0; it < 8; ++it) {
-        const int t = it * 16 + grp;
-        const uint32_t c8 = load_codes8<SB>(block_s, a.kind, t, li);
-        const float g = block_norm(block_s, SB, t);
-        if (a.has_plan) {
-            // the row's sums and, if its S lies in the plan's interval, its codes: four table reads per lane
-            float s1 = 0.0f;
-            uint32_t fix = 0, codes8 = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint2 en = pair_s[(c8 >> (2 * SB * i)) & (uint32_t)(NPAIR - 1)];
-                s1 += __uint_as_float(en.x);
-                fix += en.y & 0xFFFFFFu;
-                codes8 |= (en.y >> 24) << (2 * DB * i);
-            }
-            s1 = row16_sum(s1);
-            fix = row16_sum(fix);
-            const float recon_p = g * sqrtf(s1);
-            if (s1 > a.s_lo && s1 < a.s_hi && recon_p > 1e-10f) {   // the same for the row's sixteen lanes
-                uint32_t b0 = 0, b1 = 0;
-#pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    b0 |= ((codes8 >> (DB * m)) & ((1u << DB) - 1u)) << (8 * m);
-                    b1 |= ((codes8 >> (DB * (m + 4))) & ((1u << DB) - 1u)) << (8 * m);
-                }
-                *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(b0, b1);
-                if (li == 0) {
-                    const float cn = sqrtf((float)fix * a.fix_unit);
-                    norms_s[t] = cn > 1e-10f ? recon_p / cn : recon_p;
-                }
-                continue;
-            }
-        }
-        float v[8];
-        float ss = 0.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            v[m] = csrc_s[(c8 >> (m * SB)) & ((1u << SB) - 1u)] * g;
-            ss = fmaf(v[m], v[m], ss);
-        }
-        ss = row16_sum(ss);
-        float recon = sqrtf(ss);
-        const float inv = recon > 1e-10f ? 1.0f / recon : 1.0f;
-        if (!(recon > 1e-10f)) recon = 0.0f;
-        uint32_t w0 = 0, w1 = 0;
-        float cs = 0.0f;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            const float yv = v[m] * inv;
-            uint32_t c = 0;
-#pragma unroll
-            for (int k = 0; k < NB; ++k) c += (bnd[k] <= yv) ? 1u : 0u;  // a value on a midpoint takes the higher index
-            const float cd = cdst_s[c];
-            cs = fmaf(cd, cd, cs);
-            if (m < 4) w0 |= c << (8 * m);
-            else w1 |= c << (8 * (m - 4));
-        }
-        cs = row16_sum(cs);
-        *reinterpret_cast<uint2 *>(&codes[t * CODE_STRIDE + 8 * li]) = make_uint2(w0, w1);
-        if (li == 0) {
-            const float cn = sqrtf(cs);
-            norms_s[t] = cn > 1e-10f ? recon / cn : recon;
-        }
-    }
-    __syncthreads();
-    pack_block<DB, 256>(codes, norms_s, dst + (int64_t)blockIdx.x * block_bytes(DB), a.kind);
-}
-
+// destination codebook, corrected norm for the new codes.  K rows and V rows have a kernel each.
 // ---- K rows: a lane owns a token -----------------------------------------------------------------
 // A K row is one token's 128 codes, so one lane can requantise a row without exchanging anything.  The decision
 // value of a code is c_src[k] / sqrt(S), S = sum of c_src[code]^2 over the row (the stored norm cancels), so the
@@ -3573,21 +3450,14 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
                    hipStream_t s) {
     const unsigned grid = (unsigned)(n_seqs * blocks_for(tokens));
     if (grid == 0) return TQ_OK;
-    RequantArgs a;
-    a.cent_src = hs->centroids32; a.cent_dst = hd->centroids32; a.bounds_dst = hd->bounds32; a.kind = kind;
     const int key = hs->bits * 10 + hd->bits;
     RequantKArgs ka;
-    const bool planned = (key == 32 || key == 43 || key == 42) && requant_plan(hs, hd, &ka);
-    a.has_plan = planned ? 1 : 0;
-    if (planned) {
-        a.t0 = ka.t0; a.s_lo = ka.s_lo; a.s_hi = ka.s_hi; a.fix_unit = ka.fix_unit;
-        for (int k = 0; k < 16; ++k) {
-            a.src_sq[k] = ka.src_sq[k];
-            a.dst_fix[k] = ka.dst_fix[k];
-        }
+    if ((key != 32 && key != 43 && key != 42) || !requant_plan(hs, hd, &ka)) {
+        tq_set_error("tq_requantize: supported width pairs are 3->2, 4->3, 4->2 (got %d->%d)", hs->bits, hd->bits);
+        return TQ_ERR_UNSUPPORTED;
     }
-    if (kind == TQ_KIND_K && planned) {
-        ka.n_blocks = grid;
+    ka.n_blocks = grid;
+    if (kind == TQ_KIND_K) {
         const unsigned sets = (grid + RQK_BLOCKS - 1) / RQK_BLOCKS;
         const unsigned wgs = sets < 256u ? sets : 256u;
         switch (key) {
@@ -3597,26 +3467,14 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
         }
         return tq_check_launch("requantize (K rows)");
     }
-    if (kind == TQ_KIND_V && planned) {
-        ka.n_blocks = grid;
-        const unsigned sets = (grid + 7) / 8;
-        const unsigned wgs = sets < 256u ? sets : 256u;
-        switch (key) {
-        case 32: k_requantize_v<3, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
-        case 43: k_requantize_v<4, 3><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
-        default: k_requantize_v<4, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
-        }
-        return tq_check_launch("requantize (V rows)");
-    }
+    const unsigned sets = (grid + 7) / 8;
+    const unsigned wgs = sets < 256u ? sets : 256u;
     switch (key) {
-    case 32: k_requantize<3, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
-    case 43: k_requantize<4, 3><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
-    case 42: k_requantize<4, 2><<<grid, 256, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, a); break;
-    default:
-        tq_set_error("tq_requantize: supported width pairs are 3->2, 4->3, 4->2 (got %d->%d)", hs->bits, hd->bits);
-        return TQ_ERR_UNSUPPORTED;
+    case 32: k_requantize_v<3, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+    case 43: k_requantize_v<4, 3><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
+    default: k_requantize_v<4, 2><<<wgs, RQV_THREADS, 0, s>>>((const uint8_t *)src, (uint8_t *)dst, ka); break;
     }
-    return tq_check_launch("requantize");
+    return tq_check_launch("requantize (V rows)");
 }
 
 // ---- interchange with the per-128 block layout of the llama.cpp fork --------------------------
