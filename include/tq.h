@@ -205,6 +205,21 @@ int tq_export_fork_blocks(const tq_handle *h, const void *packed, int64_t n_seqs
 int tq_import_fork_blocks(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind,
                           void *packed, void *stream);
 
+/* The same interchange for caches written by the fork's earlier builds, whose 2- and 3-bit storage blocks hold
+ * block_values = 32 values (QK_TURBO3 = QK_TURBO2 = 32; 64 was measured too), docs/papers/block-size-experiment.md:27-39,270:
+ * a vector is 128 / block_values blocks of norm fp16 | qs | signs over its own values, one after the other, the
+ * extraction formulas above applied inside a block - 14 B (3.5 bits per value) and 26 B (3.25) per 3-bit block,
+ * 10 B and 18 B per 2-bit block.  Rotation and norm correction work on the 128-value group whatever the block
+ * size, so every block of a vector carries the same norm: export writes it into each, import reads the first.
+ * tq_fork_row_bytes: bytes of one vector, (128 / block_values) * (2 + block_values * bits / 8); -1 for a pair the fork
+ * does not have (4-bit rows exist with 128 values per block only).  block_values = 128 is the layout of the entry
+ * points above.  blocks is [n_seqs, tokens, tq_fork_row_bytes(bits, block_values)] bytes, 2-byte aligned. */
+int64_t tq_fork_row_bytes(int32_t bits, int32_t block_values);
+int tq_export_fork_blocks_sized(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind,
+                                int32_t block_values, void *blocks, void *stream);
+int tq_import_fork_blocks_sized(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind,
+                                int32_t block_values, void *packed, void *stream);
+
 /* Inverse of tq_store (KVCacheCompressor.decompress, kv_cache.py:143-165, MSE-only
  * format): out [n_seqs, tokens, 128] in the rotated domain (norm * centroid) or the
  * original domain (transpose rotation applied). */

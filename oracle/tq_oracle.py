@@ -734,41 +734,72 @@ def layout_unpack(buf: np.ndarray, bits: int, kind: str):
 #           turbo4 (docs/turbo4-investigation.md:42-49); 4-bit PolarQuant does not use it: packed as 0, ignored
 #           when unpacked.  Its position (right after norm) is not printed anywhere in the reference tree.
 #   turbo2: norm fp16 | qs[32]  (34 B), idx = (qs[j/4] >> ((j%4)*2)) & 3   (the 2-bit half of turbo3)
+#   Storage blocks of 32 or 64 values (the fork's QK_TURBO3 / QK_TURBO2 before they became 128,
+#   docs/papers/block-size-experiment.md:27-39,270): a vector is 128 / block_values blocks, each norm | qs | signs
+#   over its own values with the formulas above taken inside the block (turbo3: 14 B per 32, 26 B per 64; turbo2:
+#   10 B, 18 B), and every block of a vector carries the same group norm (block-size-experiment.md:13,45-55).
 # --------------------------------------------------------------------------
 
-def fork_block_bytes(bits: int) -> int:
-    return {2: 34, 3: 50, 4: 68}[bits]
+def fork_block_bytes(bits: int, block_values: int = 128) -> int:
+    """Bytes of ONE storage block (of block_values values)."""
+    if bits == 4:
+        if block_values != 128:
+            raise ValueError("turbo4 blocks hold 128 values")
+        return 68
+    if bits not in (2, 3) or block_values not in (32, 64, 128):
+        raise ValueError("no such fork block")
+    return 2 + block_values // 4 + (block_values // 8 if bits == 3 else 0)
 
 
-def fork_blocks_pack(idx: np.ndarray, g: np.ndarray, bits: int) -> np.ndarray:
-    """idx [T,128], g [T] fp16 -> uint8 [T, fork_block_bytes(bits)], token order."""
+def fork_row_bytes(bits: int, block_values: int = 128) -> int:
+    """Bytes of one 128-value vector: its 128 / block_values storage blocks."""
+    return (128 // block_values) * fork_block_bytes(bits, block_values)
+
+
+def fork_blocks_pack(idx: np.ndarray, g: np.ndarray, bits: int, block_values: int = 128) -> np.ndarray:
+    """idx [T,128], g [T] fp16 -> uint8 [T, fork_row_bytes(bits, block_values)], token order."""
     idx = np.asarray(idx).astype(np.uint8)
     T = idx.shape[0]
-    out = np.zeros((T, fork_block_bytes(bits)), dtype=np.uint8)
-    out[:, 0:2] = np.asarray(g, dtype=np.float16).reshape(T, 1).view(np.uint8)
+    gb = np.asarray(g, dtype=np.float16).reshape(T, 1).view(np.uint8)
     if bits == 4:
+        out = np.zeros((T, fork_block_bytes(4, block_values)), dtype=np.uint8)
+        out[:, 0:2] = gb
         out[:, 4:68] = idx[:, 0::2] | (idx[:, 1::2] << 4)   # bytes 2..3: rnorm, unused, zero
         return out
-    low = idx & 3
-    out[:, 2:34] = low[:, 0::4] | (low[:, 1::4] << 2) | (low[:, 2::4] << 4) | (low[:, 3::4] << 6)
-    if bits == 3:
-        hi = (idx >> 2) & 1
-        out[:, 34:50] = np.packbits(hi, axis=1, bitorder="little")
-    return out
+    bv, bb = block_values, fork_block_bytes(bits, block_values)
+    out = np.zeros((T, 128 // bv, bb), dtype=np.uint8)
+    for s in range(128 // bv):                              # one storage block after the other
+        part = idx[:, s * bv:(s + 1) * bv]
+        low = part & 3
+        out[:, s, 0:2] = gb
+        out[:, s, 2:2 + bv // 4] = low[:, 0::4] | (low[:, 1::4] << 2) | (low[:, 2::4] << 4) | (low[:, 3::4] << 6)
+        if bits == 3:
+            out[:, s, 2 + bv // 4:] = np.packbits((part >> 2) & 1, axis=1, bitorder="little")
+    return out.reshape(T, -1)
 
 
-def fork_blocks_unpack(buf: np.ndarray, bits: int):
-    buf = np.asarray(buf, dtype=np.uint8).reshape(-1, fork_block_bytes(bits))
-    T = buf.shape[0]
-    g = np.ascontiguousarray(buf[:, 0:2]).view(np.float16).reshape(T)
-    j = np.arange(128)
+def fork_blocks_unpack(buf: np.ndarray, bits: int, block_values: int = 128):
+    """-> idx [T,128], g [T] fp16 (the first block's norm; the blocks of a vector all carry the same one)."""
     if bits == 4:
+        buf = np.asarray(buf, dtype=np.uint8).reshape(-1, fork_block_bytes(4, block_values))
+        T = buf.shape[0]
+        g = np.ascontiguousarray(buf[:, 0:2]).view(np.float16).reshape(T)
+        j = np.arange(128)
         idx = (buf[:, 4 + j // 2] >> ((j % 2) * 4)) & 0xF
         return idx.astype(np.uint8), g
-    idx = (buf[:, 2 + j // 4] >> ((j % 4) * 2)) & 3
-    if bits == 3:
-        idx = idx | (((buf[:, 34 + j // 8] >> (j % 8)) & 1) << 2)
-    return idx.astype(np.uint8), g
+    bv, bb = block_values, fork_block_bytes(bits, block_values)
+    buf = np.asarray(buf, dtype=np.uint8).reshape(-1, 128 // bv, bb)
+    T = buf.shape[0]
+    g = np.ascontiguousarray(buf[:, 0, 0:2]).view(np.float16).reshape(T)
+    j = np.arange(bv)
+    idx = np.zeros((T, 128), dtype=np.uint8)
+    for s in range(128 // bv):
+        blk = buf[:, s]
+        part = (blk[:, 2 + j // 4] >> ((j % 4) * 2)) & 3
+        if bits == 3:
+            part = part | (((blk[:, 2 + bv // 4 + j // 8] >> (j % 8)) & 1) << 2)
+        idx[:, s * bv:(s + 1) * bv] = part
+    return idx, g
 
 
 # --------------------------------------------------------------------------

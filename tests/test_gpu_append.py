@@ -391,6 +391,73 @@ def test_fork_blocks_at_the_least_alignment(bits, kind):
     assert tt.equal(back, packed)
 
 
+@pytest.mark.parametrize("bits", [2, 3])
+@pytest.mark.parametrize("kind", ["k", "v"])
+@pytest.mark.parametrize("block_values", [32, 64])
+def test_fork_blocks_of_32_and_64_values(bits, kind, block_values):
+    """Caches of the fork's earlier builds (storage blocks of 32 values, 64 measured too;
+    docs/papers/block-size-experiment.md:27-39): the export equals the oracle's packing block by block with the group's
+    norm in every block, the import gives the packed buffer back byte for byte (ragged last block included) and reads
+    the first block's norm; rows at the least alignment write nothing outside themselves."""
+    tt = L.torch()
+    codec = tqa.TurboCodec(bits, seed=42, centroids=tqa.PRODUCTION_CENTROIDS[bits])
+    n_seqs, tokens = 3, 205
+    x = np.random.default_rng(7 * bits + block_values).standard_normal((n_seqs, tokens, D)).astype(np.float16)
+    x[1, 17] = 0
+    packed = codec.store(x, kind=kind)
+    idx, g = codec.unpack_codes(packed, n_seqs, tokens, kind=kind)
+    idx, g = np_(idx).reshape(-1, D), np_(g).reshape(-1).astype(np.float16)
+    rb = O.fork_row_bytes(bits, block_values)
+    assert L.lib().tq_fork_row_bytes(bits, block_values) == rb
+    blocks = codec.export_fork_blocks(packed, n_seqs, tokens, kind=kind, block_values=block_values)
+    assert tuple(blocks.shape) == (n_seqs, tokens, rb)
+    want = O.fork_blocks_pack(idx, g, bits, block_values)
+    assert np.array_equal(np_(blocks).reshape(-1, rb), want)
+    assert tt.equal(codec.import_fork_blocks(blocks, kind=kind, block_values=block_values), packed)
+    # blocks written elsewhere: random codes; the later blocks of a vector carry another norm, which nobody reads
+    rng = np.random.default_rng(block_values)
+    ridx = rng.integers(0, 1 << bits, size=(2 * 128, D)).astype(np.uint8)
+    rg = np.abs(rng.standard_normal(2 * 128)).astype(np.float16)
+    ext = O.fork_blocks_pack(ridx, rg, bits, block_values).reshape(2 * 128, 128 // block_values, -1)
+    ext[:, 1:, 0:2] = 0x3C
+    i2, g2 = codec.unpack_codes(codec.import_fork_blocks(ext.reshape(2, 128, rb), kind=kind, block_values=block_values),
+                                2, 128, kind=kind)
+    assert np.array_equal(np_(i2).reshape(-1, D), ridx) and np.array_equal(np_(g2).reshape(-1).astype(np.float16), rg)
+    # 2 bytes past a 16-byte boundary, 77 tokens per sequence
+    tokens = 77
+    packed = codec.store(x[:, :tokens], kind=kind)
+    idx, g = codec.unpack_codes(packed, n_seqs, tokens, kind=kind)
+    want = O.fork_blocks_pack(np_(idx).reshape(-1, D), np_(g).reshape(-1).astype(np.float16), bits, block_values).reshape(-1)
+    raw = tt.full((2 + want.size + 64,), 0xA5, dtype=tt.uint8, device="cuda")
+    lib = L.lib()
+    knd = L.KIND_K if kind == "k" else L.KIND_V
+    rc = lib.tq_export_fork_blocks_sized(codec.handle.h, L.ptr(packed), n_seqs, tokens, knd, block_values, L.ptr(raw[2:]),
+                                         L.stream_ptr())
+    assert rc == 0
+    got = np_(raw)
+    assert np.array_equal(got[2:2 + want.size], want)
+    assert (got[:2] == 0xA5).all() and (got[2 + want.size:] == 0xA5).all()
+    back = tt.full_like(packed, 0x3C)
+    rc = lib.tq_import_fork_blocks_sized(codec.handle.h, L.ptr(raw[2:]), n_seqs, tokens, knd, block_values, L.ptr(back),
+                                         L.stream_ptr())
+    assert rc == 0
+    assert tt.equal(back, packed)
+
+
+def test_fork_blocks_refuse_a_block_size_the_fork_lacks():
+    tt = L.torch()
+    c4, c3 = tqa.TurboCodec(4, seed=42), tqa.TurboCodec(3, seed=42)
+    p4 = c4.store(np.ones((1, 128, D), dtype=np.float16))
+    with pytest.raises(ValueError, match="no 4-bit layout with 32 values"):
+        c4.export_fork_blocks(p4, 1, 128, block_values=32)
+    with pytest.raises(ValueError, match="no 3-bit layout with 16 values"):
+        c3.import_fork_blocks(np.zeros((1, 128, 50), dtype=np.uint8), block_values=16)
+    out = tt.zeros(128 * 68, dtype=tt.uint8, device="cuda")
+    rc = L.lib().tq_export_fork_blocks_sized(c4.handle.h, L.ptr(p4), 1, 128, L.KIND_K, 64, L.ptr(out), L.stream_ptr())
+    assert rc == L.ERR_UNSUPPORTED and "not a layout of the fork" in L.last_error()
+    assert not np_(out).any()
+
+
 def test_fork_blocks_rejects_wrong_width():
     codec = tqa.TurboCodec(3, seed=42)
     with pytest.raises(ValueError):

@@ -42,6 +42,11 @@ def test_size_entry_points_need_no_gpu():
     assert lib.tq_packed_bytes(3, 2, 130) == 2 * 2 * 6400  # ragged: two blocks per sequence
     assert lib.tq_packed_bytes(5, 1, 128) == -1
     assert lib.tq_q8_0_bytes(1, 128) == 128 * 136
+    # the fork's storage blocks: 128 / block_values blocks of 2 + block_values * bits / 8 bytes per vector
+    assert [lib.tq_fork_row_bytes(3, bv) for bv in (32, 64, 128)] == [4 * 14, 2 * 26, 50]
+    assert [lib.tq_fork_row_bytes(2, bv) for bv in (32, 64, 128)] == [4 * 10, 2 * 18, 34]
+    assert lib.tq_fork_row_bytes(4, 128) == 68 == lib.tq_fork_block_bytes(4)
+    assert lib.tq_fork_row_bytes(4, 32) == -1 and lib.tq_fork_row_bytes(3, 16) == -1 and lib.tq_fork_row_bytes(5, 128) == -1
     p = L.TQAttnParams(batch=16, n_q_heads=32, n_kv_heads=8, tokens=32768, n_splits=16,
                        k_format=L.KFMT_TURBO, scale=0.088, sparse_v_tau=0.0)
     # one partial (four heads x (128 outputs + maximum + sum)) per workgroup; the 16 splits of a group go to two

@@ -417,3 +417,44 @@ def test_fork_block_layout_formulas(bits):
         buf[:, 2:4] = 0xA5
         i3, g3 = O.fork_blocks_unpack(buf, bits)
         assert np.array_equal(i3, idx) and np.array_equal(g3.view(np.uint16), g.view(np.uint16))
+
+
+@pytest.mark.parametrize("bits", [2, 3])
+@pytest.mark.parametrize("block_values", [32, 64, 128])
+def test_fork_storage_block_sizes(bits, block_values):
+    """The fork's earlier storage blocks of 32 (and 64) values, docs/papers/block-size-experiment.md:33-39: "norm(2B) +
+    qs(8B) + signs(4B) = 14B per 32" (3.50 bits per value, 4.57x), 26 B per 64 (3.25, 4.92x), 50 B per 128 (3.125,
+    5.12x); four blocks of a 128-value group "receive the same corrected norm value" (:13).  The extraction formulas
+    are applied by hand inside every block of what fork_blocks_pack wrote."""
+    bb = O.fork_block_bytes(bits, block_values)
+    if bits == 3:
+        assert bb == {32: 14, 64: 26, 128: 50}[block_values]
+        assert bb * 8 / block_values == {32: 3.5, 64: 3.25, 128: 3.125}[block_values]
+        assert round(16 / (bb * 8 / block_values), 2) == {32: 4.57, 64: 4.92, 128: 5.12}[block_values]
+    else:
+        assert bb == {32: 10, 64: 18, 128: 34}[block_values]
+    n_blocks = 128 // block_values
+    assert O.fork_row_bytes(bits, block_values) == n_blocks * bb
+    rng = np.random.default_rng(10 * bits + block_values)
+    idx = rng.integers(0, 1 << bits, size=(4, 128)).astype(np.uint8)
+    g = np.abs(rng.standard_normal(4)).astype(np.float16)
+    buf = O.fork_blocks_pack(idx, g, bits, block_values)
+    assert buf.shape == (4, n_blocks * bb)
+    for t in range(4):
+        for b in range(n_blocks):
+            blk = buf[t, b * bb:(b + 1) * bb]
+            assert blk[:2].view(np.float16)[0] == g[t]                     # the group's norm in every block
+            qs = blk[2:2 + block_values // 4]
+            signs = blk[2 + block_values // 4:]
+            assert len(signs) == (block_values // 8 if bits == 3 else 0)
+            for j in range(block_values):
+                got = (qs[j // 4] >> ((j % 4) * 2)) & 3
+                if bits == 3 and signs[j // 8] & (1 << (j % 8)):
+                    got |= 4
+                assert got == idx[t, b * block_values + j]
+    i2, g2 = O.fork_blocks_unpack(buf, bits, block_values)
+    assert np.array_equal(i2, idx) and np.array_equal(g2.view(np.uint16), g.view(np.uint16))
+    if block_values == 128:                                                # the default is the per-128 layout
+        assert np.array_equal(buf, O.fork_blocks_pack(idx, g, bits))
+    with pytest.raises(ValueError):
+        O.fork_block_bytes(4, 32)                                          # turbo4 blocks hold 128 values

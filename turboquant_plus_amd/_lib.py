@@ -70,6 +70,9 @@ PROTOTYPES = {
     "tq_fork_block_bytes": (_L, [C.c_int32]),
     "tq_export_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
     "tq_import_fork_blocks": (_I, [_P, _P, _L, _L, _I, _P, _P]),
+    "tq_fork_row_bytes": (_L, [C.c_int32, C.c_int32]),
+    "tq_export_fork_blocks_sized": (_I, [_P, _P, _L, _L, _I, C.c_int32, _P, _P]),
+    "tq_import_fork_blocks_sized": (_I, [_P, _P, _L, _L, _I, C.c_int32, _P, _P]),
     "tq_load": (_I, [_P, _P, _L, _L, _I, _P, _I, _I, _P]),
     "tq_load_kv": (_I, [_P, _P, _P, _P, _L, _L, _P, _P, _P]),
     "tq_unpack_codes": (_I, [_P, _P, _L, _L, _I, _P, _P, _P]),

@@ -614,11 +614,23 @@ int tq_requantize(const tq_handle *src_h, const tq_handle *dst_h, const void *pa
     return tqk_requantize(src_h, dst_h, packed_src, n_seqs, tokens, kind, packed_dst, (hipStream_t)stream);
 }
 
+// bytes of one 128-value vector in the fork's layout: 128 / block_values storage blocks of norm | qs | signs
+int64_t tq_fork_row_bytes(int32_t bits, int32_t block_values) {
+    if (bits == 4) return block_values == 128 ? 68 : -1;
+    if ((bits != 2 && bits != 3) || (block_values != 32 && block_values != 64 && block_values != 128)) return -1;
+    return (128 / block_values) * (2 + block_values * bits / 8);
+}
+
+int64_t tq_fork_block_bytes(int32_t bits) { return tq_fork_row_bytes(bits, 128); }
+
 static int fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
-                       void *stream, const char *who) {
+                       int block_values, void *stream, const char *who) {
     int rc = check_fast(h, who);
     if (rc) return rc;
     REQUIRE(n_seqs >= 0 && tokens >= 0, TQ_ERR_ARG, "%s: bad argument", who);
+    REQUIRE(tq_fork_row_bytes(h->bits, block_values) > 0, TQ_ERR_UNSUPPORTED,
+            "%s: %d-bit rows in storage blocks of %d values are not a layout of the fork (2- and 3-bit: 32, 64 or 128 values "
+            "per block; 4-bit: 128)", who, h->bits, block_values);
     if (n_seqs == 0 || tokens == 0) return TQ_OK;
     REQUIRE(src && dst, TQ_ERR_ARG, "%s: null pointer", who);
     REQUIRE(kind == TQ_KIND_K || kind == TQ_KIND_V, TQ_ERR_ARG, "%s: bad kind %d", who, kind);
@@ -628,19 +640,27 @@ static int fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t
     REQUIRE(((uintptr_t)(to_fork ? dst : src) & (fork_align - 1u)) == 0, TQ_ERR_ALIGN,
             "%s: the blocks must be %d-byte aligned (a block starts with an fp16 norm%s)", who, (int)fork_align,
             h->bits == 4 ? " and its 68-byte rows move as 4-byte words" : "");
-    return tqk_fork_blocks(h, to_fork, src, n_seqs, tokens, kind, dst, (hipStream_t)stream);
+    return tqk_fork_blocks(h, to_fork, src, n_seqs, tokens, kind, dst, block_values, (hipStream_t)stream);
 }
-
-int64_t tq_fork_block_bytes(int32_t bits) { return bits == 3 ? 50 : bits == 4 ? 68 : bits == 2 ? 34 : -1; }
 
 int tq_export_fork_blocks(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *blocks,
                           void *stream) {
-    return fork_blocks(h, 1, packed, n_seqs, tokens, kind, blocks, stream, "tq_export_fork_blocks");
+    return fork_blocks(h, 1, packed, n_seqs, tokens, kind, blocks, 128, stream, "tq_export_fork_blocks");
 }
 
 int tq_import_fork_blocks(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind, void *packed,
                           void *stream) {
-    return fork_blocks(h, 0, blocks, n_seqs, tokens, kind, packed, stream, "tq_import_fork_blocks");
+    return fork_blocks(h, 0, blocks, n_seqs, tokens, kind, packed, 128, stream, "tq_import_fork_blocks");
+}
+
+int tq_export_fork_blocks_sized(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind,
+                                int32_t block_values, void *blocks, void *stream) {
+    return fork_blocks(h, 1, packed, n_seqs, tokens, kind, blocks, block_values, stream, "tq_export_fork_blocks_sized");
+}
+
+int tq_import_fork_blocks_sized(const tq_handle *h, const void *blocks, int64_t n_seqs, int64_t tokens, int kind,
+                                int32_t block_values, void *packed, void *stream) {
+    return fork_blocks(h, 0, blocks, n_seqs, tokens, kind, packed, block_values, stream, "tq_import_fork_blocks_sized");
 }
 
 int tq_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,

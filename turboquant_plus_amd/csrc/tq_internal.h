@@ -92,7 +92,7 @@ int tqk_append_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const
 int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
                    hipStream_t s);
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
-                    hipStream_t s);
+                    int block_values, hipStream_t s);
 int tqk_store_kv(const tq_handle *hk, const tq_handle *hv, const void *k, const void *v, int64_t n_seqs, int64_t tokens,
                  int64_t capacity, int in_dtype, void *packed_k, void *packed_v, hipStream_t s);
 int tqk_load(const tq_handle *h, const void *packed, int64_t n_seqs, int64_t tokens, int kind, void *out,

@@ -3482,8 +3482,23 @@ int tqk_requantize(const tq_handle *hs, const tq_handle *hd, const void *src, in
 // in qs, the third in signs; 2-bit: qs only) - 50 / 34 bytes; 4-bit: norm fp16 | rnorm fp16 | qs[64] nibbles -
 // 68 bytes (4.25 bits per value).  rnorm is the residual-norm slot of the fork's earlier 3-bit + QJL turbo4,
 // which its 4-bit PolarQuant block keeps and does not use: written as 0, ignored when read.
-__host__ __device__ constexpr int fork_block_bytes(int bits) { return bits == 3 ? 50 : bits == 4 ? 68 : 34; }
-__host__ __device__ constexpr int fork_codes_offset(int bits) { return bits == 4 ? 4 : 2; }
+// The fork's earlier builds stored 2- and 3-bit rows in blocks of 32 values (QK_TURBO3 = QK_TURBO2 = 32; 64 was tried
+// as well, docs/papers/block-size-experiment.md:27-39,270): a vector is then SUB = 4 or 2 blocks of norm | qs | signs
+// over its own 32 or 64 values, one after the other, every block with the same (group) norm - 14 / 26 bytes per 3-bit
+// block, 10 / 18 per 2-bit block.  The extraction formulas are those of the 128-value block applied inside a block.
+// ForkRow gives the 16-bit positions of a vector's fields: a group g of 32 values has four pieces of qs (eight values
+// each) and, for 3-bit rows, two pieces of signs (sixteen values each).
+template <int BITS, int SUB> struct ForkRow {
+    static constexpr int PER = 4 / SUB;                                       // groups of 32 values per storage block
+    static constexpr int SH = 1 + 4 * PER + (BITS == 3 ? 2 * PER : 0);        // 16-bit pieces per storage block
+    static constexpr int BYTES = BITS == 4 ? 68 : 2 * SUB * SH;               // one vector
+    __host__ __device__ static constexpr int norm(int s) { return s * SH; }
+    __host__ __device__ static constexpr int qs(int g, int j) { return (g / PER) * SH + 1 + 4 * (g % PER) + j; }
+    __host__ __device__ static constexpr int sg(int g, int k) { return (g / PER) * SH + 1 + 4 * PER + 2 * (g % PER) + k; }
+};
+static_assert(ForkRow<3, 1>::BYTES == 50 && ForkRow<3, 2>::BYTES == 2 * 26 && ForkRow<3, 4>::BYTES == 4 * 14, "3-bit fork blocks");
+static_assert(ForkRow<2, 1>::BYTES == 34 && ForkRow<2, 2>::BYTES == 2 * 18 && ForkRow<2, 4>::BYTES == 4 * 10, "2-bit fork blocks");
+static_assert(ForkRow<3, 1>::qs(3, 3) == 16 && ForkRow<3, 1>::sg(0, 0) == 17 && ForkRow<3, 1>::sg(3, 1) == 24, "per-128 block");
 
 // ---- K rows of the fork layout: a lane owns a token ------------------------------------------------
 // The fork rows of one of this library's K blocks are 128 * FB contiguous bytes.  They move between memory and LDS
@@ -3513,11 +3528,12 @@ __device__ __forceinline__ void fork_stage_copy(uint8_t *stage, uint8_t *mem, in
     }
 }
 
-template <int BITS, bool TO_FORK>
+template <int BITS, bool TO_FORK, int SUB>
 __global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed_in, uint8_t *packed_out, const uint8_t *fork_in,
                                                             uint8_t *fork_out, int64_t tokens, int64_t blocks_per_seq,
                                                             uint32_t zero_code, uint32_t n_blocks) {
-    constexpr int FB = fork_block_bytes(BITS);
+    using R = ForkRow<BITS, SUB>;
+    constexpr int FB = R::BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][TQ_ROWS_PER_BLOCK * FB + 16];
     __shared__ uint16_t spread2_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of four 2-bit fields -> the fields at a stride of 3
     __shared__ uint32_t spread1_s[BITS == 3 && !TO_FORK ? 256 : 1];   // byte of eight sign bits -> bit 3m + 2
@@ -3576,17 +3592,19 @@ __global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed
                     for (int j = 0; j < 4; ++j) d[1 + 4 * g + j] = w[4 * j + g];
             } else if constexpr (BITS == 2) {
                 uint16_t *h = reinterpret_cast<uint16_t *>(mine);
-                h[0] = nrm;
+#pragma unroll
+                for (int sb = 0; sb < SUB; ++sb) h[R::norm(sb)] = nrm;   // every storage block carries the group's norm
 #pragma unroll
                 for (int g = 0; g < 4; ++g)
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        h[1 + 4 * g + 2 * j] = (uint16_t)w[4 * j + g];
-                        h[2 + 4 * g + 2 * j] = (uint16_t)(w[4 * j + g] >> 16);
+                        h[R::qs(g, 2 * j)] = (uint16_t)w[4 * j + g];
+                        h[R::qs(g, 2 * j + 1)] = (uint16_t)(w[4 * j + g] >> 16);
                     }
             } else {
                 uint16_t *h = reinterpret_cast<uint16_t *>(mine);
-                h[0] = nrm;
+#pragma unroll
+                for (int sb = 0; sb < SUB; ++sb) h[R::norm(sb)] = nrm;   // every storage block carries the group's norm
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     uint32_t sg = 0;
@@ -3594,11 +3612,11 @@ __global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t x = j < 3 ? (w[4 * j + g] & 0xFFFFFFu) : tail24(w, g);
                         const uint32_t e0 = gather_s[x & 0xFFFu], e1 = gather_s[x >> 12];
-                        h[1 + 4 * g + j] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
+                        h[R::qs(g, j)] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
                         sg |= ((e0 >> 8) | ((e1 >> 8) << 4)) << (8 * j);
                     }
-                    h[17 + 2 * g] = (uint16_t)sg;
-                    h[18 + 2 * g] = (uint16_t)(sg >> 16);
+                    h[R::sg(g, 0)] = (uint16_t)sg;
+                    h[R::sg(g, 1)] = (uint16_t)(sg >> 16);
                 }
             }
         }
@@ -3622,17 +3640,17 @@ __global__ __launch_bounds__(FORK_K_THREADS) void k_fork_k(const uint8_t *packed
 #pragma unroll
                 for (int g = 0; g < 4; ++g)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) w[4 * j + g] = (uint32_t)h[1 + 4 * g + 2 * j] | ((uint32_t)h[2 + 4 * g + 2 * j] << 16);
+                    for (int j = 0; j < 2; ++j) w[4 * j + g] = (uint32_t)h[R::qs(g, 2 * j)] | ((uint32_t)h[R::qs(g, 2 * j + 1)] << 16);
             } else {
                 const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
                 nrm = h[0];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const uint32_t sg = (uint32_t)h[17 + 2 * g] | ((uint32_t)h[18 + 2 * g] << 16);
+                    const uint32_t sg = (uint32_t)h[R::sg(g, 0)] | ((uint32_t)h[R::sg(g, 1)] << 16);
                     uint32_t x[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const uint32_t q = h[1 + 4 * g + j];
+                        const uint32_t q = h[R::qs(g, j)];
                         x[j] = (uint32_t)spread2_s[q & 0xFFu] | ((uint32_t)spread2_s[q >> 8] << 12) | spread1_s[(sg >> (8 * j)) & 0xFFu];
                     }
 #pragma unroll
@@ -3697,11 +3715,12 @@ template <int BITS> __device__ __forceinline__ uint32_t pick_codes(uint2 d, int 
     return a | (b << (2 * BITS));
 }
 
-template <int BITS, bool TO_FORK>
+template <int BITS, bool TO_FORK, int SUB>
 __global__ __launch_bounds__(64 * FORK_V_WAVES) void k_fork_v(const uint8_t *packed_in, uint8_t *packed_out, const uint8_t *fork_in,
                                                               uint8_t *fork_out, int64_t tokens, int64_t blocks_per_seq,
                                                               uint32_t zero_code, uint32_t n_blocks) {
-    constexpr int FB = fork_block_bytes(BITS);
+    using R = ForkRow<BITS, SUB>;
+    constexpr int FB = R::BYTES;
     constexpr uint32_t QM = (1u << (4 * BITS)) - 1u;   // four codes
     __shared__ __attribute__((aligned(16))) uint8_t stage_s[FORK_V_WAVES][64 * FB + 16];
     __shared__ __attribute__((aligned(8))) uint8_t xs_s[FORK_V_WAVES][32 * FORK_X_ROW];
@@ -3790,25 +3809,27 @@ __global__ __launch_bounds__(64 * FORK_V_WAVES) void k_fork_v(const uint8_t *pac
                     for (int j = 0; j < 4; ++j) d[1 + 4 * g + j] = kw[g][j];
             } else if constexpr (BITS == 2) {
                 uint16_t *h = reinterpret_cast<uint16_t *>(mine);
-                h[0] = nrm;
+#pragma unroll
+                for (int sb = 0; sb < SUB; ++sb) h[R::norm(sb)] = nrm;   // every storage block carries the group's norm
 #pragma unroll
                 for (int g = 0; g < 4; ++g)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) h[1 + 4 * g + j] = (uint16_t)kw[g][j];
+                    for (int j = 0; j < 4; ++j) h[R::qs(g, j)] = (uint16_t)kw[g][j];
             } else {
                 uint16_t *h = reinterpret_cast<uint16_t *>(mine);
-                h[0] = nrm;
+#pragma unroll
+                for (int sb = 0; sb < SUB; ++sb) h[R::norm(sb)] = nrm;   // every storage block carries the group's norm
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     uint32_t sg = 0;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t e0 = gather_s[kw[g][j] & 0xFFFu], e1 = gather_s[kw[g][j] >> 12];
-                        h[1 + 4 * g + j] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
+                        h[R::qs(g, j)] = (uint16_t)((e0 & 0xFFu) | ((e1 & 0xFFu) << 8));
                         sg |= ((e0 >> 8) | ((e1 >> 8) << 4)) << (8 * j);
                     }
-                    h[17 + 2 * g] = (uint16_t)sg;
-                    h[18 + 2 * g] = (uint16_t)(sg >> 16);
+                    h[R::sg(g, 0)] = (uint16_t)sg;
+                    h[R::sg(g, 1)] = (uint16_t)(sg >> 16);
                 }
             }
         }
@@ -3831,16 +3852,16 @@ __global__ __launch_bounds__(64 * FORK_V_WAVES) void k_fork_v(const uint8_t *pac
 #pragma unroll
                 for (int g = 0; g < 4; ++g)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) kw[g][j] = h[1 + 4 * g + j];
+                    for (int j = 0; j < 4; ++j) kw[g][j] = h[R::qs(g, j)];
             } else {
                 const uint16_t *h = reinterpret_cast<const uint16_t *>(mine);
                 nrm = h[0];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const uint32_t sg = (uint32_t)h[17 + 2 * g] | ((uint32_t)h[18 + 2 * g] << 16);
+                    const uint32_t sg = (uint32_t)h[R::sg(g, 0)] | ((uint32_t)h[R::sg(g, 1)] << 16);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const uint32_t q = h[1 + 4 * g + j];
+                        const uint32_t q = h[R::qs(g, j)];
                         kw[g][j] = (uint32_t)spread2_s[q & 0xFFu] | ((uint32_t)spread2_s[q >> 8] << 12) | spread1_s[(sg >> (8 * j)) & 0xFFu];
                     }
                 }
@@ -3885,7 +3906,7 @@ __global__ __launch_bounds__(64 * FORK_V_WAVES) void k_fork_v(const uint8_t *pac
 }
 
 int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_seqs, int64_t tokens, int kind, void *dst,
-                    hipStream_t s) {
+                    int block_values, hipStream_t s) {
     const int64_t bps = blocks_for(tokens);
     const unsigned grid = (unsigned)(n_seqs * bps);
     if (grid == 0) return TQ_OK;
@@ -3893,20 +3914,28 @@ int tqk_fork_blocks(const tq_handle *h, int to_fork, const void *src, int64_t n_
     uint32_t zero_code = (uint32_t)(h->n_centroids / 2);
     if (h->zero_code >= 0) zero_code = (uint32_t)h->zero_code;
     const unsigned kgrid = (grid + 1) / 2, vgrid = (2 * grid + FORK_V_WAVES - 1) / FORK_V_WAVES;
-#define TQ_FORK(B)                                                                                                        \
+#define TQ_FORK(B, SUB)                                                                                                   \
     if (kind == TQ_KIND_K && to_fork)                                                                                     \
-        k_fork_k<B, true><<<kgrid, FORK_K_THREADS, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
+        k_fork_k<B, true, SUB><<<kgrid, FORK_K_THREADS, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
     else if (kind == TQ_KIND_K)                                                                                           \
-        k_fork_k<B, false><<<kgrid, FORK_K_THREADS, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid); \
+        k_fork_k<B, false, SUB><<<kgrid, FORK_K_THREADS, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid); \
     else if (to_fork)                                                                                                     \
-        k_fork_v<B, true><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
+        k_fork_v<B, true, SUB><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>((const uint8_t *)src, nullptr, nullptr, (uint8_t *)dst, tokens, bps, zero_code, grid); \
     else                                                                                                                  \
-        k_fork_v<B, false><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid)
-    switch (h->bits) {
-    case 2: TQ_FORK(2); break;
-    case 3: TQ_FORK(3); break;
-    case 4: TQ_FORK(4); break;
-    default: tq_set_error("fork blocks: bits must be 2, 3 or 4 (got %d)", h->bits); return TQ_ERR_UNSUPPORTED;
+        k_fork_v<B, false, SUB><<<vgrid, 64 * FORK_V_WAVES, 0, s>>>(nullptr, (uint8_t *)dst, (const uint8_t *)src, nullptr, tokens, bps, zero_code, grid)
+    const int sub = block_values == 128 ? 1 : block_values == 64 ? 2 : block_values == 32 ? 4 : 0;
+    switch (h->bits * 8 + sub) {
+    case 2 * 8 + 1: TQ_FORK(2, 1); break;
+    case 2 * 8 + 2: TQ_FORK(2, 2); break;
+    case 2 * 8 + 4: TQ_FORK(2, 4); break;
+    case 3 * 8 + 1: TQ_FORK(3, 1); break;
+    case 3 * 8 + 2: TQ_FORK(3, 2); break;
+    case 3 * 8 + 4: TQ_FORK(3, 4); break;
+    case 4 * 8 + 1: TQ_FORK(4, 1); break;
+    default:
+        tq_set_error("fork blocks: %d-bit rows in storage blocks of %d values are not a layout of the fork (2- and 3-bit: "
+                     "32, 64 or 128 values per block; 4-bit: 128)", h->bits, block_values);
+        return TQ_ERR_UNSUPPORTED;
     }
 #undef TQ_FORK
     return tq_check_launch("fork_blocks");

@@ -210,27 +210,36 @@ class TurboCodec:
                                       L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
         return out
 
-    def export_fork_blocks(self, packed, n_seqs: int, tokens: int, kind: str = "k"):
-        """-> uint8 [n_seqs, tokens, 50 | 68 | 34]: the llama.cpp fork's per-128 block layout."""
+    def export_fork_blocks(self, packed, n_seqs: int, tokens: int, kind: str = "k", block_values: int = 128):
+        """-> uint8 [n_seqs, tokens, row bytes]: the llama.cpp fork's block layout, 50 | 68 | 34 bytes per vector with
+        the fork's present 128-value storage blocks; block_values = 32 or 64 gives the layout of its earlier builds
+        (2- and 3-bit rows: four blocks of 14 | 10 bytes, two of 26 | 18; docs/papers/block-size-experiment.md:27-39)."""
         tt = L.torch()
-        fb = int(L.lib().tq_fork_block_bytes(self.bits))
+        fb = int(L.lib().tq_fork_row_bytes(self.bits, block_values))
+        if fb < 0:
+            raise ValueError(f"the fork has no {self.bits}-bit layout with {block_values} values per storage block")
         out = tt.empty((n_seqs, tokens, fb), dtype=tt.uint8, device=packed.device)
-        L.check(L.lib().tq_export_fork_blocks(self.handle.h, L.ptr(packed), n_seqs, tokens,
-                                              L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        L.check(L.lib().tq_export_fork_blocks_sized(self.handle.h, L.ptr(packed), n_seqs, tokens,
+                                                    L.KIND_K if kind == "k" else L.KIND_V, block_values, L.ptr(out),
+                                                    L.stream_ptr()))
         return out
 
-    def import_fork_blocks(self, blocks, kind: str = "k"):
-        """Fork blocks [n_seqs, tokens, 50 | 68 | 34] -> packed buffer of this library."""
+    def import_fork_blocks(self, blocks, kind: str = "k", block_values: int = 128):
+        """Fork blocks [n_seqs, tokens, row bytes of this width and block size] -> packed buffer of this library."""
         tt = L.torch()
         dev = L.require_gpu()
         bd = blocks if isinstance(blocks, tt.Tensor) else tt.from_numpy(np.ascontiguousarray(blocks))
-        if bd.dtype != tt.uint8 or bd.dim() != 3 or bd.shape[2] != int(L.lib().tq_fork_block_bytes(self.bits)):
-            raise ValueError("blocks must be uint8 [n_seqs, tokens, block bytes of this width]")
+        fb = int(L.lib().tq_fork_row_bytes(self.bits, block_values))
+        if fb < 0:
+            raise ValueError(f"the fork has no {self.bits}-bit layout with {block_values} values per storage block")
+        if bd.dtype != tt.uint8 or bd.dim() != 3 or bd.shape[2] != fb:
+            raise ValueError("blocks must be uint8 [n_seqs, tokens, row bytes of this width and block size]")
         bd = bd.to(dev)
         n_seqs, tokens = int(bd.shape[0]), int(bd.shape[1])
         out = tt.empty(packed_bytes(self.bits, n_seqs, tokens), dtype=tt.uint8, device=bd.device)
-        L.check(L.lib().tq_import_fork_blocks(self.handle.h, L.ptr(bd.contiguous()), n_seqs, tokens,
-                                              L.KIND_K if kind == "k" else L.KIND_V, L.ptr(out), L.stream_ptr()))
+        L.check(L.lib().tq_import_fork_blocks_sized(self.handle.h, L.ptr(bd.contiguous()), n_seqs, tokens,
+                                                    L.KIND_K if kind == "k" else L.KIND_V, block_values, L.ptr(out),
+                                                    L.stream_ptr()))
         return out
 
     def store_qjl(self, x):
