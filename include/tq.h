@@ -318,11 +318,12 @@ typedef struct tq_attn_params {
                                            /* 2 * tokens rows, row 2 * token + half, written  */
                                            /* by tq_store(_kv) / tq_append(_kv) from the      */
                                            /* [tokens, 256] tensor taken as [2 * tokens, 128];*/
-                                           /* q and out are [batch, n_q_heads, 256].  V turbo */
-                                           /* (K turbo of the same width, of 4|2, 3|2, 4|3    */
-                                           /* bits, or q8_0-style rows written the same way   */
-                                           /* by tq_q8_0_store); Sparse V tests tiles of 32   */
-                                           /* tokens; bias rows and lists count tokens        */
+                                           /* q and out are [batch, n_q_heads, 256].  K and V */
+                                           /* turbo of one width or of 4|2, 3|2, 4|3 bits, or */
+                                           /* q8_0-style rows on either side (written the     */
+                                           /* same way by tq_q8_0_store / tq_q8_0_store_v);   */
+                                           /* Sparse V tests tiles of 32 tokens; bias rows    */
+                                           /* and lists count tokens                          */
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four

@@ -113,7 +113,8 @@ def test_decode_attention_many_short_sequences(B, N, n_splits, Hq, sparse):
     assert np.isfinite(out).all()
 
 
-def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None, n_splits=1, tau=0.0, bias=None):
+def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale, k_q8=None, n_splits=1, tau=0.0, bias=None,
+                            v_q8=None):
     """Oracle attention for heads of 256 dims on the GPU-stored codes: the caches hold 2 N rows of 128 per sequence,
     row 2 t + half; a token's vector is its two rows side by side, each decoded and un-rotated by itself."""
     G = Hq // Hkv
@@ -125,8 +126,12 @@ def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale,
         qq, ss = tqa.q8_0_unpack(k_q8, B * Hkv, 2 * N)
         k_rot = O.q8_0_dequantize(np_(qq), np_(ss)).reshape(B * Hkv, N, 2 * D)
         q_rot = q.astype(np.float64)
-    vi, vg = vc.unpack_codes(v_packed, B * Hkv, 2 * N, kind="v")
-    v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids).reshape(B * Hkv, N, 2 * D)
+    if v_q8 is None:
+        vi, vg = vc.unpack_codes(v_packed, B * Hkv, 2 * N, kind="v")
+        v_rot = O.turbo_decode_rotated(np_(vi), np_(vg).astype(np.float64), vc.centroids).reshape(B * Hkv, N, 2 * D)
+    else:                                      # q8_0-style V rows: stored unrotated
+        qq, ss = tqa.q8_0_unpack(v_q8, B * Hkv, 2 * N, kind="v")
+        v_rot = O.q8_0_dequantize(np_(qq), np_(ss)).reshape(B * Hkv, N, 2 * D)
     out = np.zeros((B, Hq, 2 * D))
     skipped = 0.0
     for b in range(B):
@@ -135,7 +140,8 @@ def reference_attention_256(q, kc, vc, k_packed, v_packed, B, Hq, Hkv, N, scale,
             bb = None if bias is None else bias[b, h * G:(h + 1) * G]
             o, sk, _ = O.decode_attention(q_rot[b, h * G:(h + 1) * G], k_rot[g], v_rot[g], scale, n_splits=n_splits,
                                           sparse_v_tau=tau, logit_bias=bb, tile=32)
-            o = O.rotate_fast(o.reshape(G, 2, D), vc.signs1, vc.signs2, D, transpose=True)
+            if v_q8 is None:
+                o = O.rotate_fast(o.reshape(G, 2, D), vc.signs1, vc.signs2, D, transpose=True)
             out[b, h * G:(h + 1) * G] = o.reshape(G, 2 * D)
             skipped += sk
     return (out, skipped / (B * Hkv)) if tau > 0 else out
@@ -165,17 +171,23 @@ def test_decode_attention_head_dim_256(bits, N, n_splits, Hq):
     assert_close(out, ref)
 
 
-@pytest.mark.parametrize("kbits,vbits", [(8, 4), (8, 3), (8, 2), (4, 2), (3, 2), (4, 3)])
+@pytest.mark.parametrize("kbits,vbits", [(8, 4), (8, 3), (8, 2), (4, 2), (3, 2), (4, 3), (8, 8), (4, 8), (3, 8), (2, 8)])
 @pytest.mark.parametrize("N,n_splits", [(100, 1), (2048 + 31, 8)])
 def test_decode_attention_head_dim_256_mixed_formats(kbits, vbits, N, n_splits):
-    """256-dim heads with q8_0-style K rows (the fork's recommended "-ctk q8_0 -ctv turboN") and with K wider than V."""
+    """256-dim heads with q8_0-style K rows (the fork's recommended "-ctk q8_0 -ctv turboN"), with K wider than V, and
+    with q8_0-style V rows (the boundary layers of the fork's Boundary V policy)."""
     B, Hq, Hkv = 2, 8, 2
     rng = np.random.default_rng(100 * kbits + vbits + N)
     k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
     v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
     k[:, :, :7] *= 4.0
-    vc = tqa.TurboCodec(vbits, seed=542)
-    vp = vc.store(tqa.rows_of_256(v), kind="v")
+    if vbits == 8:
+        v[:, :, 128:] *= 3.0                   # the halves' 32-value groups have scales of their own
+        v[:, 5::7, 40:72] *= 0.25
+        vc, vp = None, tqa.q8_0_store(tqa.rows_of_256(v), kind="v")[0]
+    else:
+        vc = tqa.TurboCodec(vbits, seed=542)
+        vp = vc.store(tqa.rows_of_256(v), kind="v")
     q = rng.standard_normal((B, Hq, 2 * D)).astype(np.float16)
     if kbits == 8:
         kc, kp = None, tqa.q8_0_store(tqa.rows_of_256(k))[0]
@@ -184,7 +196,8 @@ def test_decode_attention_head_dim_256_mixed_formats(kbits, vbits, N, n_splits):
         kp = kc.store(tqa.rows_of_256(k), kind="k")
     attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256)
     out = np_(attn(q, kp, vp))
-    ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D), k_q8=kp if kbits == 8 else None)
+    ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D), k_q8=kp if kbits == 8 else None,
+                                  v_q8=vp if vbits == 8 else None)
     assert_close(out, ref)
 
 
@@ -247,6 +260,40 @@ def test_decode_attention_head_dim_256_sparse_v_and_bias(N, n_splits):
     assert_close(np_(attn(q, kp, vp, sparse_bias=tqa.sparse_bias_from_dense(bd))), out_sb)
 
 
+@pytest.mark.parametrize("kbits", [8, 3])
+def test_decode_attention_head_dim_256_q8_v_rows_sparse_v_and_bias(kbits):
+    """256-dim heads on q8_0-style V rows with Sparse V, a dense and a sparse logit bias, and a group of three query
+    heads per KV head (a pass with an idle head row)."""
+    B, Hq, Hkv, N, n_splits = 2, 6, 2, 2048 + 31, 8
+    rng = np.random.default_rng(77 + kbits)
+    k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+    v[:, :, 128:] *= 2.0
+    if kbits == 8:
+        kc, kp = None, tqa.q8_0_store(tqa.rows_of_256(k))[0]
+    else:
+        kc = tqa.TurboCodec(kbits, seed=42)
+        kp = kc.store(tqa.rows_of_256(k), kind="k")
+    vp = tqa.q8_0_store(tqa.rows_of_256(v), kind="v")[0]
+    q = (2.0 * rng.standard_normal((B, Hq, 2 * D))).astype(np.float16)
+    scale, tau = 1 / np.sqrt(2 * D), 1e-3
+    kq = kp if kbits == 8 else None
+    attn = tqa.DecodeAttention(kc, None, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256, sparse_v_tau=tau)
+    out = np_(attn(q, kp, vp)).copy()
+    ref, sk = reference_attention_256(q, kc, None, kp, vp, B, Hq, Hkv, N, scale, k_q8=kq, v_q8=vp, n_splits=n_splits, tau=tau)
+    assert_close(out, ref)
+    assert abs(attn.skip_rate() - sk) < 2e-3 and sk > 0.05
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    bias[:, :, :4] = 3.0
+    bias[:, 1::2, N - 1] = -2.0
+    bias[0, 0, N // 2] = 5.0
+    bd = L.torch().from_numpy(bias).cuda()
+    dense = tqa.DecodeAttention(kc, None, B, Hq, Hkv, N, n_splits=n_splits, head_dim=256)
+    ref_b = reference_attention_256(q, kc, None, kp, vp, B, Hq, Hkv, N, scale, k_q8=kq, v_q8=vp, bias=bias.astype(np.float64))
+    assert_close(np_(dense(q, kp, vp, bias=bd)), ref_b)
+    assert_close(np_(dense(q, kp, vp, sparse_bias=tqa.sparse_bias_from_dense(bd))), ref_b)
+
+
 def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
     B, Hq, Hkv, N = 1, 4, 1, 128
     kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
@@ -255,8 +302,6 @@ def test_decode_attention_head_dim_256_refuses_what_it_does_not_take():
     q = tt.zeros((B, Hq, 256), dtype=tt.float16, device="cuda")
     with pytest.raises(NotImplementedError):
         tqa.DecodeAttention(tqa.TurboCodec(2, seed=42), vc, B, Hq, Hkv, N, head_dim=256)(q, buf, buf)   # K narrower than V
-    with pytest.raises(NotImplementedError):
-        tqa.DecodeAttention(kc, None, B, Hq, Hkv, N, head_dim=256)(q, buf, buf)                          # q8_0-style V rows
     with pytest.raises(ValueError):
         tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, head_dim=64)
 

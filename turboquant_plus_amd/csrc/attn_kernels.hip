@@ -327,10 +327,30 @@ __device__ __forceinline__ void pv_all_q8(std::integer_sequence<int, T...>, cons
      ...);
 }
 
+// q8_0-style V rows under heads of 256 dims: dword 16*hf + T = rows 4T..4T+3 = (token 2T, half 0), (2T, 1), (2T+1, 0),
+// (2T+1, 1) of dim half hf, handed over in the order 0, 2, 1, 3.  a8[dh][hf][T & 1]: the weights of tokens 2T, 2T+1
+// times the scales of their rows of half dh (for this half-wavefront's 32-dim block of dim half hf) in the places of
+// that half's rows, zeros in the others; both half-wavefronts hold the same 32 tokens, so token pair T is served by
+// block T / 2 of either half with its own scales.
+template <int... T>
+__device__ __forceinline__ void pv_all_q8_d256(std::integer_sequence<int, T...>, const uint32_t (&vw)[32],
+                                               const half4_t (&a8)[2][2][2], float4_t (&acc_o)[2][2][2]) {
+    (([&] {
+         const half4_t v0 = int8x4_to_half_0213(vw[T]), v1 = int8x4_to_half_0213(vw[16 + T]);
+#pragma unroll
+         for (int dh = 0; dh < 2; ++dh) {
+             acc_o[dh][0][T & 1] = mfma4_bcast8<(T >> 1)>(a8[dh][0][T & 1], v0, acc_o[dh][0][T & 1]);
+             acc_o[dh][1][T & 1] = mfma4_bcast8<(T >> 1)>(a8[dh][1][T & 1], v1, acc_o[dh][1][T & 1]);
+         }
+     }()),
+     ...);
+}
+
 // per-tile side data of the V rows: turbo = the fp16 norms of this lane's four tokens; q8_0-style = the fp16 scales
 // [2 * dim half + swapped]: of this lane's four tokens (0) and of the four tokens of lane ^ 32 (1), for the 32-dim
 // block that this lane's dims of that dim half lie in
-// heads of 256 dims: the eight fp16 norms of the rows of this lane's four tokens (v[0], v[1])
+// heads of 256 dims: the eight fp16 norms of the rows of this lane's four tokens (v[0], v[1]); q8_0-style: the eight
+// scales of those rows for the 32-dim block of this lane's dims of dim half hf (v[2 hf], v[2 hf + 1])
 template <int VBITS> struct VSide { uint2 v[VBITS == 8 ? 4 : 2]; };
 
 constexpr unsigned long long ARRIVAL_COUNT_MASK = 0xFFFFFFull;  // workgroups of a group (the tag of the call sits above)
@@ -546,14 +566,14 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 
 // SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
 // registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
-// D256: heads of 256 dims (turbo or q8_0-style K, turbo V).  A token is rows 2 token and 2 token + 1 of caches that are
+// D256: heads of 256 dims.  A token is rows 2 token and 2 token + 1 of caches that are
 // otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
 // then the output's two halves of one set of four heads: one softmax, two accumulator sets.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
-__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KFMT == KFMT_TURBO ? 4 : 1) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KFMT == KFMT_TURBO && VBITS != 8 ? 4 : 1) void k_decode_attn(AttnArgs a) {
     // (256-dim heads on turbo K rows: four wavefronts per SIMD = two workgroups of eight per CU, i.e. at most 128 registers - the
     // variant sits at 119-136 without the bound, and one register over 128 halves its occupancy)
-    static_assert(!D256 || (HG == 2 && VBITS != 8), "256-dim heads: turbo V rows");
+    static_assert(!D256 || HG == 2, "256-dim heads: two accumulator sets, the output's halves");
     constexpr int HQ = D256 ? 1 : HG;   // sets of four heads whose logits and softmax state the wavefront keeps
     constexpr int KROW_DW = KFMT == KFMT_TURBO ? 4 * KBITS : 32;
     constexpr int KBLOCK = KFMT == KFMT_TURBO ? TQ_ROWS_PER_BLOCK * (16 * KBITS + 2) : TQ_ROWS_PER_BLOCK * 136;
@@ -639,7 +659,15 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
     auto load_vnorm = [&](int tile) -> VSide<VBITS> {
         VSide<VBITS> r;
         const uint8_t *side = vbase + (int64_t)(tile >> 1) * VBLOCK + TQ_ROWS_PER_BLOCK * 16 * VBITS;
-        if constexpr (VBITS == 8) {
+        if constexpr (VBITS == 8 && D256) {
+            const int bh = lane >> 5;
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {   // rows e4 .. e4 + 7 of the tile: this lane's four tokens, both halves
+                const uint4 s8 = *reinterpret_cast<const uint4 *>(side + 2 * ((((tile & 1) * 4 + 2 * hf + bh) * 64) + e4));
+                r.v[2 * hf] = make_uint2(s8.x, s8.y);
+                r.v[2 * hf + 1] = make_uint2(s8.z, s8.w);
+            }
+        } else if constexpr (VBITS == 8) {
             const int bh = lane >> 5;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -995,7 +1023,26 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KF
 
         // ---- PV ------------------------------------------------------------------------
         // weights (times the stored V norm) as fp16: this lane is token group T = lane/4, head lane%4
-        if constexpr (VBITS == 8) {
+        if constexpr (VBITS == 8 && D256) {
+            half4_t a8[2][2][2];
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                // scales of rows 8b..8b+7 = (token 4b + i, half h) at 2 i + h
+                const uint32_t sw[4] = {gvu.v[2 * hf].x, gvu.v[2 * hf].y, gvu.v[2 * hf + 1].x, gvu.v[2 * hf + 1].y};
+#pragma unroll
+                for (int dh = 0; dh < 2; ++dh) {
+                    _Float16 w[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        w[i] = (_Float16)(p[0][i] * (__half2float(__ushort_as_half((unsigned short)(dh ? sw[i] >> 16 : sw[i] & 0xffff))) *
+                                                     Q8V_PRESCALE));
+                    const _Float16 z = (_Float16)0.0f;
+                    a8[dh][hf][0] = dh ? half4_t{z, z, w[0], w[1]} : half4_t{w[0], w[1], z, z};
+                    a8[dh][hf][1] = dh ? half4_t{z, z, w[2], w[3]} : half4_t{w[2], w[3], z, z};
+                }
+            }
+            pv_all_q8_d256(std::make_integer_sequence<int, 16>{}, vw, a8, acc_o);
+        } else if constexpr (VBITS == 8) {
             // The dims of block b lie in 32-dim block b / 8 (+ 2 for the upper dim half), so the weights carry that
             // block's scale and are broadcast inside each half of the wavefront: token group T is served by block
             // T % 8 of both halves, which therefore also needs the weights of the lane 32 away.
@@ -1329,10 +1376,6 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
         tq_set_error("tq_decode_attention: head_dim %d (128 or 256)", (int)p->head_dim);
         return TQ_ERR_UNSUPPORTED;
     }
-    if (d256 && (p->v_format != TQ_KFMT_TURBO || !hv)) {
-        tq_set_error("tq_decode_attention: head_dim 256 takes turbo V rows");
-        return TQ_ERR_UNSUPPORTED;
-    }
     const int64_t cache_rows = (d256 ? 2 : 1) * p->tokens;   // a 256-dim token is two rows of the caches
     float *part_o = reinterpret_cast<float *>((char *)ws + w.part_o);
     float *part_ml = reinterpret_cast<float *>((char *)ws + w.part_ml);
@@ -1451,6 +1494,10 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
             else if (!turbo_k && vb == 2) { TQ_ATTN_256X(KFMT_Q8, 3, 2); }
             else if (!turbo_k && vb == 3) { TQ_ATTN_256X(KFMT_Q8, 3, 3); }
             else if (!turbo_k && vb == 4) { TQ_ATTN_256X(KFMT_Q8, 3, 4); }
+            else if (!turbo_k && vb == 8) { TQ_ATTN_256X(KFMT_Q8, 3, 8); }
+            else if (turbo_k && kb == 2 && vb == 8) { TQ_ATTN_256X(KFMT_TURBO, 2, 8); }
+            else if (turbo_k && kb == 3 && vb == 8) { TQ_ATTN_256X(KFMT_TURBO, 3, 8); }
+            else if (turbo_k && kb == 4 && vb == 8) { TQ_ATTN_256X(KFMT_TURBO, 4, 8); }
             else {
                 tq_set_error("tq_decode_attention: head_dim 256 with K %d bits, V %d bits is not built", kb, vb);
                 return TQ_ERR_UNSUPPORTED;

@@ -434,7 +434,8 @@ class DecodeAttention:
         head_dim: 128, or 256 - a head's vector as two 128-value groups, each rotated, quantised and normed by itself
         (the fork's 128-value blocks, docs/getting-started.md:68).  The caches are then those of 128-dim heads with
         two rows per token: rows_of_256(x) gives the [n, 2 * tokens, 128] view that store / append / load take, and
-        `tokens`, `capacity`, `pos` of those calls count rows (2 * tokens).  Turbo K and V of one width, dense."""
+        `tokens`, `capacity`, `pos` of those calls count rows (2 * tokens).  Turbo K at least as wide as turbo V, or
+        q8_0-style rows on either side."""
         tt = L.torch()
         dev = L.require_gpu()
         self.k_codec, self.v_codec = k_codec, v_codec
