@@ -538,18 +538,17 @@ def sparse_bias_from_dense(bias, max_entries: int | None = None):
 
 
 def default_splits(n_groups: int, tokens: int) -> int:
-    """Context splits per (batch, kv head): one wavefront per split, four
-    wavefronts per SIMD on 256 CUs x 4 SIMDs, at least 4 tiles of 64 tokens each (2 when the groups are few).
-    The kernel groups up to 16 splits (the largest power of two dividing the
-    count) into one workgroup, so the count is rounded down to a multiple of 16,
-    or to a power of two below 16."""
+    """Context splits per (batch, kv head): one wavefront per split.  A large step (eight or more 64-token tiles
+    per wavefront at four wavefronts per SIMD on 256 CUs x 4 SIMDs) gets those 4096 wavefronts; a smaller one is
+    bound by what a workgroup does once (tables, queries, the merge of its wavefronts' partials) and measured faster
+    on 2048 wavefronts, i.e. one workgroup of eight per CU (four sequences at 32K: 25.7 against 27.1 us; one at 128K:
+    27.6 against 30.2 us), down to two tiles per split (one sequence at 32K: 15.5 us; one tile per split 18.6 us).
+    The kernel groups up to 16 splits (the largest power of two dividing the count) into one workgroup, so the count
+    is rounded down to a multiple of 16, or to a power of two below 16."""
     tiles = max(1, (tokens + 63) // 64)
-    want = max(1, (4 * 1024 + n_groups - 1) // n_groups)
-    n = int(max(1, min(want, tiles // 4 if tiles >= 4 else 1)))
-    if n_groups * max(n // 16, 1) < 256 and tiles >= 4:
-        # few groups (small batches): the chip is not full at four tiles per split; two tiles per split measured
-        # faster there (one sequence at 32K: 22.6 against 27.2 us), one tile per split no better
-        n = int(max(1, min(want, tiles // 2)))
+    waves = 4096 if n_groups * tiles >= 8 * 4096 else 2048
+    want = max(1, (waves + n_groups - 1) // n_groups)
+    n = int(max(1, min(want, tiles // 2 if tiles >= 2 else 1)))
     if n >= 16:
         return n // 16 * 16
     return 1 << (n.bit_length() - 1)
