@@ -278,6 +278,19 @@ def store_leg(torch, tqa, bits, steps, warmup, n_sets=4, several_streams=False):
                "v_alone": {"us_per_launch": fvev_ms * 1e3, "gbs": f_algo / 2 / (fvev_ms * 1e-3) / 1e9,
                            "frac": f_algo / 2 / (fvev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}}
         del sets32
+        # float64 rows (the reference's own dtype): the butterfly kernel k_store, one launch per tensor; K alone
+        k64 = sets[0][0].double()
+        kp64 = sets[0][2]
+
+        def dstep(i):
+            codec_k.store(k64, kind="k", out=kp64)
+        _, dev_ms = time_steps(torch, dstep, max(steps // 2, 1), warmup)
+        d_algo = n_vec // 2 * (1024 + 16 * bits + 2)
+        f32["f64_rows_k_alone"] = {"what": "the K tensor as float64 rows (1024 B per vector in) through the butterfly kernel (k_store<double>)",
+                                   "us_per_launch": dev_ms * 1e3, "algorithmic_bytes_per_launch": d_algo,
+                                   "gbs": d_algo / (dev_ms * 1e-3) / 1e9, "frac": d_algo / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        codec_k.store(sets[0][0], kind="k", out=kp64)      # the set's packed K as the fp16 rows give it
+        del k64
     return {
         "workload": f"turbo{bits} store, K+V fp16 [8,32768,128], 4 K outlier channels x15, block 128",
         "ms_per_step": wall_ms, "event_ms_per_step": ev_ms, "kernel_us": launch_us,
