@@ -327,8 +327,12 @@ typedef struct tq_attn_params {
 } tq_attn_params;
 
 /* Bytes of workspace tq_decode_attention needs: one partial (2 KB; 4 KB when a KV head serves more than four
- * query heads) per workgroup, plus flags and Sparse-V slots.  The workspace may hold anything on entry; calls
- * that share one workspace must not overlap in time. */
+ * query heads) per workgroup, plus flags and Sparse-V slots; it does not depend on bias_entries / bias_pos /
+ * bias_val, which may change from call to call (a call with a bias list may run smaller workgroups: the size covers
+ * either).  The workspace may hold anything on entry; calls that share one workspace must not overlap in time.
+ * n_splits: any count >= 1; workgroups take the largest power of two up to 16 that divides it (8 for q8_0-style V
+ * rows, for 256-dim heads and for more than four query heads per KV head - there 12 when 12 divides it and K and V
+ * are turbo rows, which is the best shape for large steps: 256 workgroups of twelve). */
 int64_t tq_attn_workspace_bytes(const tq_attn_params *p);
 
 /* softmax(scale * q k^T) v over packed K/V (tests/test_kv_cache.py:73-89,128-131

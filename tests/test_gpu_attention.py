@@ -767,6 +767,51 @@ def test_decode_attention_every_format_pair(kfmt, vfmt):
             assert abs(attn.skip_rate() - skip_o) <= 0.02 * max(skip_o, 1e-3) + 1e-4
 
 
+@pytest.mark.parametrize("bits,n_splits,Hq", [(3, 12, 64), (4, 24, 64), (2, 12, 40), (3, 36, 48)])
+def test_decode_attention_eight_heads_in_workgroups_of_twelve(bits, n_splits, Hq):
+    """Eight heads per pass on turbo K and V rows with a split count that is a multiple of 12 and enough groups to
+    fill the chip: workgroups of twelve wavefronts (three per SIMD).  Dense, Sparse V, a dense bias; a call with a
+    bias list on the same object runs workgroups of eight or four (more partials per group, in the workspace sized at
+    construction).  Checked on a sample of the sequences."""
+    B, Hkv, N = 32, 8, 1500
+    tt = L.torch()
+    g = tt.Generator(device="cuda").manual_seed(bits * 100 + n_splits)
+    k = tt.randn((B * Hkv, N, D), generator=g, device="cuda").to(tt.float16)
+    v = tt.randn((B * Hkv, N, D), generator=g, device="cuda").to(tt.float16)
+    # (2-bit rows with queries 1.5 times as long sit at 1.2 times the fp16 bar with every workgroup shape: the rows'
+    # few large centroids times a peaked softmax)
+    q = ((1.5 if bits > 2 else 1.0) * tt.randn((B, Hq, D), generator=g, device="cuda")).to(tt.float16)
+    kc, vc = tqa.TurboCodec(bits, seed=42), tqa.TurboCodec(bits, seed=542)
+    kp, vp = kc.store(k, kind="k"), vc.store(v, kind="v")
+    bias = tt.zeros((B, Hq, N), dtype=tt.float32, device="cuda")
+    bias[:, :, :4] = 2.0
+    bias[:, 1::2, N - 1] = -1.5
+    per = tqa.packed_bytes(bits, Hkv, N)
+    sample = (0, 7, B - 1)
+
+    def check(out, tau, bias_np, skip=None):
+        for b in sample:
+            bb = None if bias_np is None else bias_np[b:b + 1]
+            ref, sk, _ = reference_attention(np_(q[b:b + 1]), kc, vc, kp[b * per:(b + 1) * per], vp[b * per:(b + 1) * per], 1, Hq, Hkv,
+                                             N, 1 / np.sqrt(D), n_splits=n_splits, tau=tau, bias=bb)
+            assert_close(out[b:b + 1], ref)
+        assert np.isfinite(out).all()
+
+    dense = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, poison_output=True)
+    check(np_(dense(q, kp, vp)).copy(), 0.0, None)
+    bias_np = np_(bias).astype(np.float64)
+    check(np_(dense(q, kp, vp, bias=bias)).copy(), 0.0, bias_np)
+    check(np_(dense(q, kp, vp, sparse_bias=tqa.sparse_bias_from_dense(bias))).copy(), 0.0, bias_np)
+    check(np_(dense(q, kp, vp)).copy(), 0.0, None)                       # and back to the wide workgroups
+    sparse = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, sparse_v_tau=1e-3, poison_output=True)
+    check(np_(sparse(q, kp, vp)).copy(), 1e-3, None)
+    assert 0.0 < sparse.skip_rate() < 1.0
+    # the default split count of such a shape is a multiple of 12 when the step is large enough
+    assert tqa.turbo.default_splits(128, 32768, eight_heads=True) == 24
+    assert tqa.turbo.default_splits(128, 32768, eight_heads=True, turbo_rows=False) == 16
+    assert tqa.turbo.default_splits(64, 32768, eight_heads=True) == 32
+
+
 @pytest.mark.parametrize("kfmt,vfmt", [("turbo3", "turbo3"), ("turbo4", "turbo2"), ("q8_0", "turbo2"), ("q8_0", "q8_0"), ("turbo3", "q8_0"),
                                        ("turbo2", "turbo4")])
 def test_decode_attention_eight_heads_per_kv_head(kfmt, vfmt):

@@ -562,7 +562,12 @@ __device__ __forceinline__ unsigned long long block_sum(unsigned long long t, un
 // which leaves each more than the 128 registers of a 16-wavefront workgroup.
 // Two sets of four query heads per pass (HG = 2: GQA groups of more than four heads read K/V once per eight heads)
 // double the accumulators and the softmax state and run with at most 8 wavefronts too.
-__host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { return vbits == 8 || hg == 2 ? 8 : 16; }
+// Wavefronts per workgroup that a variant is compiled for (its register budget follows: 16 -> 128, 12 -> 168, 8 -> 256).
+// wide12: eight heads per pass on turbo K and V rows of 128-dim heads without a bias list - 145-165 registers, so twelve
+// wavefronts (three per SIMD) fit where two workgroups of eight do not.
+__host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg, bool wide12 = false) {
+    return vbits == 8 ? 8 : hg == 2 ? (wide12 ? 12 : 8) : 16;
+}
 
 // SBIAS: the call carries a sparse logit bias (a.sbias_n > 0).  A template parameter and not a branch: the cursor
 // registers and the per-tile test cost the eight-head variant 4 us per step when they were compiled in unconditionally.
@@ -570,7 +575,8 @@ __host__ __device__ constexpr int max_waves_per_workgroup(int vbits, int hg) { r
 // otherwise those of 128-dim heads with twice the tokens; a 64-row tile is 32 tokens.  The two sets of HG = 2 are
 // then the output's two halves of one set of four heads: one softmax, two accumulator sets.
 template <int KFMT, int KBITS, int VBITS, bool SPARSE, bool SHARE, int HG, bool SBIAS, bool D256 = false>
-__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG), D256 && KFMT == KFMT_TURBO && VBITS != 8 ? 4 : 1) void k_decode_attn(AttnArgs a) {
+__global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFMT_TURBO && !D256 && !SBIAS),
+                             D256 && KFMT == KFMT_TURBO && VBITS != 8 ? 4 : 1) void k_decode_attn(AttnArgs a) {
     // (256-dim heads on turbo K rows: four wavefronts per SIMD = two workgroups of eight per CU, i.e. at most 128 registers - the
     // variant sits at 119-136 without the bound, and one register over 128 halves its occupancy)
     static_assert(!D256 || HG == 2, "256-dim heads: two accumulator sets, the output's halves");
@@ -1315,18 +1321,21 @@ struct WsLayout {
 struct AttnPlan {
     int hg, wpw, n_parts, gpw;
 };
-AttnPlan attn_plan(const tq_attn_params *p) {
+AttnPlan attn_plan(const tq_attn_params *p, bool bias_list) {
     AttnPlan pl;
     // 256-dim heads run as two accumulator sets (the output's halves) of one set of four heads
     pl.hg = p->head_dim == 256 || p->n_q_heads / p->n_kv_heads > 4 ? 2 : 1;
-    pl.wpw = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
+    const bool turbo_k = p->k_format == TQ_KFMT_TURBO, turbo_v = p->v_format == TQ_KFMT_TURBO;
+    const bool wide12 = turbo_k && p->head_dim != 256 && !bias_list;
+    pl.wpw = max_waves_per_workgroup(turbo_v ? 0 : 8, pl.hg, wide12);
+    if (pl.wpw == 12 && p->n_splits % 12 != 0) pl.wpw = 8;
     while (p->n_splits % pl.wpw) pl.wpw >>= 1;
     // few groups (small batches): smaller workgroups, so that every CU gets one (a tile costs a wavefront the same
     // issue time however many share the SIMD)
     const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
     // short contexts: a group has fewer splits than a workgroup has room for wavefronts.  Several groups then share a
     // workgroup (and its decode tables), provided that still makes a workgroup per CU
-    const int wmax = max_waves_per_workgroup(p->v_format == TQ_KFMT_TURBO ? 0 : 8, pl.hg);
+    const int wmax = max_waves_per_workgroup(turbo_v ? 0 : 8, pl.hg);   // groups share a workgroup in powers of two
     pl.gpw = 1;
     if (p->n_splits < wmax && wmax % p->n_splits == 0) {
         int g = wmax / p->n_splits;
@@ -1338,14 +1347,15 @@ AttnPlan attn_plan(const tq_attn_params *p) {
             return pl;
         }
     }
-    while (pl.wpw > 4 && groups * (p->n_splits / pl.wpw) < 256) pl.wpw >>= 1;
+    while (pl.wpw > 4 && pl.wpw % 2 == 0 && groups * (p->n_splits / pl.wpw) < 256) pl.wpw >>= 1;
     pl.n_parts = p->n_splits / pl.wpw;
     return pl;
 }
 WsLayout ws_layout(const tq_attn_params *p) {
     const int64_t groups = (int64_t)p->batch * p->n_kv_heads;
-    const AttnPlan pl = attn_plan(p);
-    const int64_t parts = groups * pl.n_parts;
+    // a call with a bias list may run smaller workgroups (more partials per group) than one without: room for either
+    const AttnPlan pl = attn_plan(p, false), pl_list = attn_plan(p, true);
+    const int64_t parts = groups * (pl.n_parts > pl_list.n_parts ? pl.n_parts : pl_list.n_parts);
     WsLayout w;
     w.part_o = 0;
     w.part_ml = w.part_o + align256(parts * 4 * pl.hg * 128 * 4);
@@ -1437,7 +1447,7 @@ int tqk_decode_attention(const tq_handle *hk, const tq_handle *hv, const tq_attn
     }
     // wavefronts per workgroup: the largest power of two up to 16 (8 for int8 V rows and for eight heads per pass)
     // that divides the split count
-    const AttnPlan pl = attn_plan(p);
+    const AttnPlan pl = attn_plan(p, p->bias_entries > 0);
     const int wpw = pl.wpw, hg = pl.hg;
     const unsigned grid = (unsigned)((int64_t)groups * pl.n_parts / pl.gpw);
     const unsigned wg = 64u * (unsigned)wpw;

@@ -443,7 +443,9 @@ class DecodeAttention:
             raise ValueError(f"head_dim {head_dim}: the packed-cache kernels take 128 or 256")
         self.head_dim = head_dim
         if n_splits is None:
-            n_splits = default_splits(batch * n_kv_heads, tokens * (head_dim // HEAD_DIM))
+            n_splits = default_splits(batch * n_kv_heads, tokens * (head_dim // HEAD_DIM),
+                                      eight_heads=head_dim == HEAD_DIM and n_q_heads // max(n_kv_heads, 1) > 4,
+                                      turbo_rows=k_codec is not None and v_codec is not None)
         self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
                                      capacity=capacity, n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
                                      v_format=L.KFMT_TURBO if v_codec is not None else L.KFMT_Q8_0,
@@ -537,16 +539,29 @@ def sparse_bias_from_dense(bias, max_entries: int | None = None):
     return pos.contiguous(), val.contiguous()
 
 
-def default_splits(n_groups: int, tokens: int) -> int:
+def default_splits(n_groups: int, tokens: int, eight_heads: bool = False, turbo_rows: bool = True) -> int:
     """Context splits per (batch, kv head): one wavefront per split.  A large step (eight or more 64-token tiles
     per wavefront at four wavefronts per SIMD on 256 CUs x 4 SIMDs) gets those 4096 wavefronts; a smaller one is
     bound by what a workgroup does once (tables, queries, the merge of its wavefronts' partials) and measured faster
     on 2048 wavefronts, i.e. one workgroup of eight per CU (four sequences at 32K: 25.7 against 27.1 us; one at 128K:
     27.6 against 30.2 us), down to two tiles per split (one sequence at 32K: 15.5 us; one tile per split 18.6 us).
     The kernel groups up to 16 splits (the largest power of two dividing the count) into one workgroup, so the count
-    is rounded down to a multiple of 16, or to a power of two below 16."""
+    is rounded down to a multiple of 16, or to a power of two below 16.
+    eight_heads: more than four query heads per KV head (128-dim heads).  That variant's registers leave room for one
+    workgroup per CU, so one round of 256 workgroups is the aim: twelve wavefronts each (a split count that is a
+    multiple of 12; turbo K and V rows) when a wavefront then still has twenty tiles, eight otherwise (16 sequences x 8
+    KV heads at 32K, 64 query heads: 94.6 us with 24 splits, 97.9 with 16, 104.8 with 32; 8 sequences: 51.5 us with 32
+    splits, 52.0 with 48, 64.6 with 64)."""
     tiles = max(1, (tokens + 63) // 64)
-    waves = 4096 if n_groups * tiles >= 8 * 4096 else 2048
+    total = n_groups * tiles
+    if eight_heads:
+        if turbo_rows and total >= 20 * 3072 and 3072 // n_groups >= 12:
+            n = min(3072 // n_groups, tiles // 2) // 12 * 12
+            if n >= 12:
+                return n
+        waves = 2048
+    else:
+        waves = 4096 if total >= 8 * 4096 else 2048
     want = max(1, (waves + n_groups - 1) // n_groups)
     n = int(max(1, min(want, tiles // 2 if tiles >= 2 else 1)))
     if n >= 16:
