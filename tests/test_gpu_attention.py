@@ -458,6 +458,59 @@ def test_decode_attention_sparse_bias(G, n_splits, N, E):
         attn(q, kp, vp, sparse_bias=(pos_d.to(tt.int64), val_d))
 
 
+@pytest.mark.parametrize("where", ["front", "back", "spread", "mixed"])
+@pytest.mark.parametrize("G,n_splits,head_dim", [(4, 8, 128), (8, 3, 128), (4, 16, 256)])
+def test_decode_attention_sparse_bias_long_lists(where, G, n_splits, head_dim):
+    """Lists of hundreds of positions per head - runs of consecutive positions at the front or the back of the context
+    (a window of recent tokens), every fourth position, and heads with lists of very different lengths: the walk takes
+    a head's list sixteen entries at a time, several windows inside one tile and windows that straddle tiles and
+    splits.  Equal to the same bias as dense rows, and to the oracle."""
+    tt = L.torch()
+    B, Hkv, N = 2, 2, 1500
+    Hq = Hkv * G
+    rng = np.random.default_rng(len(where) + G + head_dim)
+    bias = np.zeros((B, Hq, N), dtype=np.float32)
+    vals = lambda n: rng.uniform(-3.0, 3.0, size=n).astype(np.float32) + 0.01
+    for b in range(B):
+        for h in range(Hq):
+            if where == "front":
+                n_e = 520 if h % 2 else 33
+                bias[b, h, :n_e] = vals(n_e)
+            elif where == "back":
+                n_e = 300 + 17 * h
+                bias[b, h, N - n_e:] = vals(n_e)
+            elif where == "spread":
+                sel = np.arange(h % 4, N, 4)
+                bias[b, h, sel] = vals(len(sel))
+            else:
+                if h % 3 == 0:
+                    bias[b, h, 5] = 4.0                                   # one entry
+                elif h % 3 == 1:
+                    bias[b, h, :] = vals(N)                               # every position
+                else:
+                    sel = rng.choice(N, size=160, replace=False)
+                    bias[b, h, sel] = vals(160)
+    pos_d, val_d = tqa.sparse_bias_from_dense(bias)
+    bd = tt.from_numpy(bias).cuda()
+    if head_dim == 256:
+        k = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+        v = rng.standard_normal((B * Hkv, N, 2 * D)).astype(np.float16)
+        kc, vc = tqa.TurboCodec(3, seed=42), tqa.TurboCodec(3, seed=542)
+        kp, vp = kc.store(tqa.rows_of_256(k), kind="k"), vc.store(tqa.rows_of_256(v), kind="v")
+        q = rng.standard_normal((B, Hq, 2 * D)).astype(np.float16)
+        ref = reference_attention_256(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(2 * D), bias=bias.astype(np.float64))
+    else:
+        k, v, kc, vc, kp, vp = make_kv(B, Hkv, N, seed=77 + G)
+        q = rng.standard_normal((B, Hq, D)).astype(np.float16)
+        ref, _, _ = reference_attention(q, kc, vc, kp, vp, B, Hq, Hkv, N, 1 / np.sqrt(D), n_splits=n_splits, bias=bias)
+    attn = tqa.DecodeAttention(kc, vc, B, Hq, Hkv, N, n_splits=n_splits, head_dim=head_dim, poison_output=True)
+    dense = np_(attn(q, kp, vp, bias=bd)).copy()
+    sparse = np_(attn(q, kp, vp, sparse_bias=(pos_d, val_d))).copy()
+    # (the two forms add the scaled bias in different instantiations, one with a fused multiply-add: an ulp of a logit, 1e-5 of an output)
+    np.testing.assert_allclose(sparse, dense, rtol=0, atol=5e-5 * np.abs(dense).max())
+    assert_close(sparse, ref)
+
+
 @pytest.mark.parametrize("N,misalign", [(1000, 0), (1001, 0), (999, 0), (1000, 1), (64, 0), (67, 1)])
 def test_decode_attention_dense_bias_every_position(N, misalign):
     """A bias that differs at every position, for context lengths that are and are not multiples of four and

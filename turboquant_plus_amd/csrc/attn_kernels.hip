@@ -812,19 +812,28 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
     float bias_next[HG][4];
 #pragma unroll
     for (int hg = 0; hg < HQ; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
-    // Sparse bias: a head's (position, value) list is walked by a cursor as the tiles go by.  The cursor starts at the
-    // head's first entry inside this split: the number of entries below the split's first token, counted with the
-    // whole wavefront (one entry per lane and round); the sixteen lanes that hold a head's logits move in step.
-    int sb_cur[HG], sb_pos[HG];
+    // Sparse bias: a head's (position, value) list is walked as the tiles go by, sixteen entries at a time: lane (b, j)
+    // holds entry sb_win + b of head j's list (b = lane / 4: the sixteen lanes that hold a head's logits hold a window
+    // of its list), so a window is one load per lane, and a tile that has entries adds the window's sixteen to the
+    // lanes that own their positions (an entry per dependent trip to memory made a list of 512 positions at the front
+    // of the context double the step).  The window starts at the head's first entry inside this split: the number
+    // of entries below the split's first token, counted with the whole wavefront (one entry per lane and round).
+    int sb_win[HG], sb_pos[HG];
     float sb_val[HG];
 #pragma unroll
     for (int hg = 0; hg < HG; ++hg) {
-        sb_cur[hg] = 0;
+        sb_win[hg] = 0;
         sb_pos[hg] = 0x7FFFFFFF;
         sb_val[hg] = 0.0f;
     }
     // entry e of the list of this lane's head in set hg (addresses are formed where they are needed: the path is rare)
     auto sb_entry = [&](int hg, int e) { return ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.sbias_n + e; };
+    auto sb_load = [&](int hg) {   // this lane's entry of the window
+        const int e = sb_win[hg] + (lane >> 2);
+        const bool in = e < a.sbias_n;
+        sb_pos[hg] = in ? a.sbias_pos[sb_entry(hg, in ? e : 0)] : 0x7FFFFFFF;
+        sb_val[hg] = in ? a.sbias_val[sb_entry(hg, in ? e : 0)] : 0.0f;
+    };
     if constexpr (SBIAS) {
         const int first_tok = t_begin * TT;
 #pragma unroll
@@ -841,11 +850,8 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
                 }
                 below[h] = c;
             }
-            sb_cur[hg] = j == 0 ? below[0] : j == 1 ? below[1] : j == 2 ? below[2] : below[3];
-            if (sb_cur[hg] < a.sbias_n) {
-                sb_pos[hg] = a.sbias_pos[sb_entry(hg, sb_cur[hg])];
-                sb_val[hg] = a.sbias_val[sb_entry(hg, sb_cur[hg])];
-            }
+            sb_win[hg] = j == 0 ? below[0] : j == 1 ? below[1] : j == 2 ? below[2] : below[3];
+            sb_load(hg);
         }
     }
     unsigned nskip = 0;  // Sparse V: skipped (query, position) pairs of this wavefront (wave-uniform: counted from lane masks)
@@ -884,21 +890,40 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
             load_bias(tile_n, hg, bias_next[hg]);
         }
         if constexpr (SBIAS) {
-            // entries of this tile (a handful per head and context: the loop body runs for few tiles)
-            const int tile_hi = tile * TT + TT;
+            // entries of this tile: positions ascend, so a window is done with once its last position lies below the
+            // tile's end; a head then takes its next sixteen entries (wave-uniform loop, heads advance on their own)
+            const int tile_lo = tile * TT, tile_hi = tile_lo + TT;
 #pragma unroll
             for (int hg = 0; hg < HQ; ++hg) {
-                while (__builtin_amdgcn_ballot_w64(sb_pos[hg] < tile_hi) != 0ull) {
-                    if (sb_pos[hg] < tile_hi) {
-                        const int d = sb_pos[hg] - tile * TT - t4;  // an entry at an earlier position than the cursor expects is dropped
-                        const float add = sb_val[hg] * LOG2E;
+                bool fresh = true;   // this head's window has not been added to this tile yet
+                while (true) {
+                    const bool mine = fresh && sb_pos[hg] >= tile_lo && sb_pos[hg] < tile_hi;
+                    // window slots (lane / 4) that hold an entry of this tile for any of the four heads
+                    unsigned long long slots = __builtin_amdgcn_ballot_w64(mine);
+                    slots = (slots | (slots >> 1) | (slots >> 2) | (slots >> 3)) & 0x1111111111111111ull;
+                    auto add_slot = [&](int e4) {   // e4 = 4 * slot
+                        const int pe = __shfl(sb_pos[hg], e4 + j);
+                        const float ve = __shfl(sb_val[hg], e4 + j) * LOG2E;
+                        const int d = pe - tile_lo - t4;   // positions outside this lane's four tokens (or this tile) match no i
+                        if (fresh) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) bias4[hg][i] += d == i ? add : 0.0f;
-                        ++sb_cur[hg];
-                        const bool more = sb_cur[hg] < a.sbias_n;
-                        sb_pos[hg] = more ? a.sbias_pos[sb_entry(hg, sb_cur[hg])] : 0x7FFFFFFF;
-                        sb_val[hg] = more ? a.sbias_val[sb_entry(hg, sb_cur[hg])] : 0.0f;
+                            for (int i = 0; i < 4; ++i) bias4[hg][i] += d == i ? ve : 0.0f;
+                        }
+                    };
+#pragma unroll 1
+                    while (slots) {   // (unrolled over all sixteen slots this was faster for runs of positions and cost registers)
+                        add_slot(__builtin_ctzll(slots));
+                        slots &= slots - 1;
                     }
+                    fresh = false;
+                    // the whole window lies before the tile's end (padding never does): the head's last lanes hold its last entry
+                    const bool advance = __shfl(sb_pos[hg], 60 + j) < tile_hi;
+                    if (__builtin_amdgcn_ballot_w64(advance) == 0ull) break;
+                    if (advance) {
+                        sb_win[hg] += 16;
+                        fresh = true;
+                    }
+                    if (advance) sb_load(hg);
                 }
             }
         }
