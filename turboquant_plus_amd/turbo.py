@@ -445,7 +445,8 @@ class DecodeAttention:
         if n_splits is None:
             n_splits = default_splits(batch * n_kv_heads, tokens * (head_dim // HEAD_DIM),
                                       eight_heads=head_dim == HEAD_DIM and n_q_heads // max(n_kv_heads, 1) > 4,
-                                      turbo_rows=k_codec is not None and v_codec is not None)
+                                      turbo_rows=k_codec is not None and v_codec is not None,
+                                      one_workgroup_per_cu=v_codec is None or (head_dim != HEAD_DIM and k_codec is None))
         self.params = L.TQAttnParams(batch=batch, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, tokens=tokens,
                                      capacity=capacity, n_splits=n_splits, k_format=L.KFMT_TURBO if k_codec is not None else L.KFMT_Q8_0,
                                      v_format=L.KFMT_TURBO if v_codec is not None else L.KFMT_Q8_0,
@@ -539,7 +540,8 @@ def sparse_bias_from_dense(bias, max_entries: int | None = None):
     return pos.contiguous(), val.contiguous()
 
 
-def default_splits(n_groups: int, tokens: int, eight_heads: bool = False, turbo_rows: bool = True) -> int:
+def default_splits(n_groups: int, tokens: int, eight_heads: bool = False, turbo_rows: bool = True,
+                   one_workgroup_per_cu: bool = False) -> int:
     """Context splits per (batch, kv head): one wavefront per split.  A large step (eight or more 64-token tiles
     per wavefront at four wavefronts per SIMD on 256 CUs x 4 SIMDs) gets those 4096 wavefronts; a smaller one is
     bound by what a workgroup does once (tables, queries, the merge of its wavefronts' partials) and measured faster
@@ -551,7 +553,11 @@ def default_splits(n_groups: int, tokens: int, eight_heads: bool = False, turbo_
     workgroup per CU, so one round of 256 workgroups is the aim: twelve wavefronts each (a split count that is a
     multiple of 12; turbo K and V rows) when a wavefront then still has twenty tiles, eight otherwise (16 sequences x 8
     KV heads at 32K, 64 query heads: 94.6 us with 24 splits, 97.9 with 16, 104.8 with 32; 8 sequences: 51.5 us with 32
-    splits, 52.0 with 48, 64.6 with 64)."""
+    splits, 52.0 with 48, 64.6 with 64).
+    one_workgroup_per_cu: the other variants whose workgroups of eight wavefronts fit a CU once (q8_0-style V rows; 256-dim
+    heads with q8_0-style rows on either side): 2048 wavefronts, one round of workgroups (16 x 8 groups at 32K, turbo3 K
+    with q8_0-style V: 120.5 us with 16 splits against 124.9 with 32; 256-dim heads, q8_0-style K with turbo3 V: 123.2
+    against 130.1; with Sparse V the same or more)."""
     tiles = max(1, (tokens + 63) // 64)
     total = n_groups * tiles
     if eight_heads:
@@ -559,6 +565,8 @@ def default_splits(n_groups: int, tokens: int, eight_heads: bool = False, turbo_
             n = min(3072 // n_groups, tiles // 2) // 12 * 12
             if n >= 12:
                 return n
+        waves = 2048
+    elif one_workgroup_per_cu:
         waves = 2048
     else:
         waves = 4096 if total >= 8 * 4096 else 2048
