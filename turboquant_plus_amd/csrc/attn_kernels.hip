@@ -742,6 +742,52 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
     // pair entries requested above, and nobody reads them before the barrier below)
     float xq0 = 0.0f, xq1 = 0.0f;
     if (wave_g < 4 * HG) load_q(wave_g, xq0, xq1);
+    // (placed here, in front of the table build and the query rotation, so that its two dependent trips to memory - the
+    // count of entries below the split, then the first window - pass while those run: behind them it delayed every
+    // wavefront's first tile)
+    // Sparse bias: a head's (position, value) list is walked as the tiles go by, sixteen entries at a time: lane (b, j)
+    // holds entry sb_win + b of head j's list (b = lane / 4: the sixteen lanes that hold a head's logits hold a window
+    // of its list), so a window is one load per lane, and a tile that has entries adds the window's sixteen to the
+    // lanes that own their positions (an entry per dependent trip to memory made a list of 512 positions at the front
+    // of the context double the step).  The window starts at the head's first entry inside this split: the number
+    // of entries below the split's first token, counted with the whole wavefront (one entry per lane and round).
+    int sb_win[HG], sb_pos[HG], sb_last[HG];   // sb_last: the window's last position (a cross-lane read per tile otherwise)
+    float sb_val[HG];
+#pragma unroll
+    for (int hg = 0; hg < HG; ++hg) {
+        sb_win[hg] = 0;
+        sb_pos[hg] = sb_last[hg] = 0x7FFFFFFF;
+        sb_val[hg] = 0.0f;
+    }
+    // entry e of the list of this lane's head in set hg (addresses are formed where they are needed: the path is rare)
+    auto sb_entry = [&](int hg, int e) { return ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.sbias_n + e; };
+    auto sb_load = [&](int hg) {   // this lane's entry of the window
+        const int e = sb_win[hg] + (lane >> 2);
+        const bool in = e < a.sbias_n;
+        sb_pos[hg] = in ? a.sbias_pos[sb_entry(hg, in ? e : 0)] : 0x7FFFFFFF;
+        sb_val[hg] = in ? a.sbias_val[sb_entry(hg, in ? e : 0)] : 0.0f;
+        sb_last[hg] = __shfl(sb_pos[hg], 60 + j);   // the head's last lanes hold the window's last entry
+    };
+    if constexpr (SBIAS) {
+        const int first_tok = t_begin * TT;
+#pragma unroll
+        for (int hg = 0; hg < HQ; ++hg) {
+            int below[4];
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const int32_t *prow = a.sbias_pos + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + h, a.q_group - 1)) * a.sbias_n;
+                int c = 0;
+                for (int e0 = 0; e0 < a.sbias_n; e0 += 64) {
+                    const int e = e0 + lane;
+                    const int pe = e < a.sbias_n ? prow[e] : 0x7FFFFFFF;
+                    c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(pe < first_tok));
+                }
+                below[h] = c;
+            }
+            sb_win[hg] = j == 0 ? below[0] : j == 1 ? below[1] : j == 2 ? below[2] : below[3];
+            sb_load(hg);
+        }
+    }
     if constexpr (KFMT == KFMT_TURBO) build_lut<KBITS>(klut_s, a.klut, kpair, tid, n_waves);
     if constexpr (!SHARE && VBITS != 8) build_lut<VBITS>(vlut_s, a.vlut, vpair, tid, n_waves);
     for (int h = wave_g; h < 4 * HG; h += gw) {
@@ -812,48 +858,6 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
     float bias_next[HG][4];
 #pragma unroll
     for (int hg = 0; hg < HQ; ++hg) load_bias(min(t_begin, max(t_end - 1, 0)), hg, bias_next[hg]);
-    // Sparse bias: a head's (position, value) list is walked as the tiles go by, sixteen entries at a time: lane (b, j)
-    // holds entry sb_win + b of head j's list (b = lane / 4: the sixteen lanes that hold a head's logits hold a window
-    // of its list), so a window is one load per lane, and a tile that has entries adds the window's sixteen to the
-    // lanes that own their positions (an entry per dependent trip to memory made a list of 512 positions at the front
-    // of the context double the step).  The window starts at the head's first entry inside this split: the number
-    // of entries below the split's first token, counted with the whole wavefront (one entry per lane and round).
-    int sb_win[HG], sb_pos[HG];
-    float sb_val[HG];
-#pragma unroll
-    for (int hg = 0; hg < HG; ++hg) {
-        sb_win[hg] = 0;
-        sb_pos[hg] = 0x7FFFFFFF;
-        sb_val[hg] = 0.0f;
-    }
-    // entry e of the list of this lane's head in set hg (addresses are formed where they are needed: the path is rare)
-    auto sb_entry = [&](int hg, int e) { return ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + j, a.q_group - 1)) * a.sbias_n + e; };
-    auto sb_load = [&](int hg) {   // this lane's entry of the window
-        const int e = sb_win[hg] + (lane >> 2);
-        const bool in = e < a.sbias_n;
-        sb_pos[hg] = in ? a.sbias_pos[sb_entry(hg, in ? e : 0)] : 0x7FFFFFFF;
-        sb_val[hg] = in ? a.sbias_val[sb_entry(hg, in ? e : 0)] : 0.0f;
-    };
-    if constexpr (SBIAS) {
-        const int first_tok = t_begin * TT;
-#pragma unroll
-        for (int hg = 0; hg < HQ; ++hg) {
-            int below[4];
-#pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                const int32_t *prow = a.sbias_pos + ((int64_t)group * a.q_group + min(a.head_off + 4 * hg + h, a.q_group - 1)) * a.sbias_n;
-                int c = 0;
-                for (int e0 = 0; e0 < a.sbias_n; e0 += 64) {
-                    const int e = e0 + lane;
-                    const int pe = e < a.sbias_n ? prow[e] : 0x7FFFFFFF;
-                    c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(pe < first_tok));
-                }
-                below[h] = c;
-            }
-            sb_win[hg] = j == 0 ? below[0] : j == 1 ? below[1] : j == 2 ? below[2] : below[3];
-            sb_load(hg);
-        }
-    }
     unsigned nskip = 0;  // Sparse V: skipped (query, position) pairs of this wavefront (wave-uniform: counted from lane masks)
     bool v_ahead = true;  // Sparse V: this tile's V row was requested while the previous tile was processed
 
@@ -916,14 +920,13 @@ __global__ __launch_bounds__(64 * max_waves_per_workgroup(VBITS, HG, KFMT == KFM
                         slots &= slots - 1;
                     }
                     fresh = false;
-                    // the whole window lies before the tile's end (padding never does): the head's last lanes hold its last entry
-                    const bool advance = __shfl(sb_pos[hg], 60 + j) < tile_hi;
+                    const bool advance = sb_last[hg] < tile_hi;   // the whole window lies before the tile's end (padding never does)
                     if (__builtin_amdgcn_ballot_w64(advance) == 0ull) break;
                     if (advance) {
                         sb_win[hg] += 16;
                         fresh = true;
                     }
-                    if (advance) sb_load(hg);
+                    sb_load(hg);   // by every lane (the load ends in a cross-lane read); heads that stay reload what they hold
                 }
             }
         }
